@@ -1,0 +1,453 @@
+"""CPU oracle for the Huginn/Raven recurrent-core decode path.  TEST INFRASTRUCTURE ONLY.
+
+This file restates, with plain PyTorch CPU ops, the arithmetic of the reference's
+inference model (recpre/raven_modeling_minimal.py, "RMM" below).  It is the checker the
+HIP kernels are compared with; nothing in the shipped package may import it.  Only
+tests/, __graft_entry__.smoke() and the cpu_baseline leg of bench.py use it.
+
+Every function names the reference lines it follows.  Rounding points are the ones a
+dtype-cast reference model has (no autocast): each nn.Linear output, each elementwise
+result and each norm output is stored in the model dtype; reductions, softmax and
+RoPE run in fp32.
+
+How each function is pinned (tests/test_oracle_pins.py), without running the reference:
+  rmsnorm            closed forms (constant rows, one-hot rows), F.rms_norm cross-check,
+                     fp64 brute force, rounding-order test                       -> pinned
+  rope_table/apply   complex multiplication form, pos=0 identity, norm preservation,
+                     relative-position property, spot values                     -> pinned
+  DictCache          brute-force list model, step enumeration, seen-token law,
+                     cache-size known answers from the reference notebooks       -> pinned
+  attention          eager softmax(QK^T/sqrt d)V in fp64, T=1 and q=0 special cases,
+                     torch SDPA library cross-check                               -> pinned
+  linear/adapter     fp64 matmul, split-concat identity, swapped-order negative   -> pinned
+  gated_mlp          fp64 restatement, gate-half negative test                    -> pinned
+  block/iterate/forward/greedy   composition laws (r=0, cache vs no-cache,
+                     prefill-then-decode vs token-by-token)                       -> pinned
+  initialize_state   bounds, std, scale=0, generator determinism                  -> pinned
+The reference holds no golden vectors for this path (it has no test suite); the only
+exact numbers it publishes are three KV-cache sizes, used as known-answer tests.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+
+
+# --------------------------------------------------------------------------------------
+# shape / config  (recpre/raven_config_minimal.py:12-91)
+# --------------------------------------------------------------------------------------
+@dataclass
+class RavenShape:
+    n_embd: int = 5280
+    n_heads: int = 55
+    intermediate_size: int = 17920
+    vocab_size: int = 65536
+    n_layers_in_prelude: int = 2
+    n_layers_in_recurrent_block: int = 4
+    n_layers_in_coda: int = 2
+    mean_recurrence: int = 32
+    block_size: int = 4096
+    rope_base: float = 50000.0
+    norm_eps: float = 1e-6
+    qk_bias: bool = True
+
+    @property
+    def head_dim(self) -> int:
+        return self.n_embd // self.n_heads
+
+    @property
+    def emb_scale(self) -> float:  # RMM:27-33, 50-52
+        return math.sqrt(self.n_embd)
+
+    @property
+    def init_std(self) -> float:  # raven_config_minimal.py:86
+        return math.sqrt(2.0 / (5.0 * self.n_embd))
+
+    @staticmethod
+    def nebel() -> "RavenShape":
+        return RavenShape()
+
+    @staticmethod
+    def tiny() -> "RavenShape":
+        return RavenShape(
+            n_embd=256, n_heads=4, intermediate_size=704, vocab_size=1024,
+            n_layers_in_prelude=1, n_layers_in_recurrent_block=2, n_layers_in_coda=1,
+            mean_recurrence=4,
+        )
+
+
+def block_keys(prefix: str, qk_bias: bool = True) -> list[str]:
+    """State-dict names of one SandwichBlock, in module registration order (RMM:515-523, 440-452, 497-503)."""
+    keys = [f"{prefix}.norm_1.weight", f"{prefix}.attn.Wqkv.weight"]
+    if qk_bias:
+        keys.append(f"{prefix}.attn.qk_bias")
+    keys += [
+        f"{prefix}.attn.proj.weight", f"{prefix}.norm_2.weight",
+        f"{prefix}.mlp.fc.weight", f"{prefix}.mlp.proj.weight",
+        f"{prefix}.norm_3.weight", f"{prefix}.norm_4.weight",
+    ]
+    return keys
+
+
+def state_dict_layout(s: RavenShape) -> list[tuple[str, tuple[int, ...]]]:
+    """(name, shape) of every tensor of the interchange format, in registration order (RMM:551-577)."""
+    h, hd, nh, inter = s.n_embd, s.head_dim, s.n_heads, s.intermediate_size
+
+    def blk(prefix):
+        shapes = {
+            "norm_1.weight": (h,), "norm_2.weight": (h,), "norm_3.weight": (h,), "norm_4.weight": (h,),
+            "attn.Wqkv.weight": (3 * h, h), "attn.qk_bias": (2, 1, nh, hd), "attn.proj.weight": (h, h),
+            "mlp.fc.weight": (2 * inter, h), "mlp.proj.weight": (h, inter),
+        }
+        return [(k, shapes[k[len(prefix) + 1:]]) for k in block_keys(prefix, s.qk_bias)]
+
+    out = [("transformer.wte.weight", (s.vocab_size, h))]
+    for i in range(s.n_layers_in_prelude):
+        out += blk(f"transformer.prelude.{i}")
+    out.append(("transformer.adapter.weight", (h, 2 * h)))
+    for i in range(s.n_layers_in_recurrent_block):
+        out += blk(f"transformer.core_block.{i}")
+    for i in range(s.n_layers_in_coda):
+        out += blk(f"transformer.coda.{i}")
+    out.append(("transformer.ln_f.weight", (h,)))
+    return out
+
+
+def make_weights(s: RavenShape, seed: int = 0, dtype=torch.float32, only_core: bool = False) -> dict[str, torch.Tensor]:
+    """Seeded synthetic weights: matrices, embedding and qk_bias ~ N(0, 0.02); norm weights ~ N(1, 0.02).
+
+    One CPU generator, one draw per tensor in state-dict order, drawn in fp32 and then cast, so any
+    host reproduces the same values.  lm_head is tied to wte (RMM:574-575).  `only_core` restricts the
+    draw to the adapter and core blocks (what one recurrence iteration touches); that subset uses its
+    own stream and does not equal the same tensors of the full draw.
+    """
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    w: dict[str, torch.Tensor] = {}
+    for name, shape in state_dict_layout(s):
+        if only_core and not (name.startswith("transformer.core_block") or name.startswith("transformer.adapter")):
+            continue
+        mean = 1.0 if (name.endswith("weight") and len(shape) == 1) else 0.0
+        t = torch.empty(shape, dtype=torch.float32).normal_(mean, 0.02, generator=g)
+        w[name] = t.to(dtype)
+    if not only_core:
+        w["lm_head.weight"] = w["transformer.wte.weight"]
+        w["freqs_cis"] = rope_table(s.head_dim, s.block_size, s.rope_base)
+    return w
+
+
+# --------------------------------------------------------------------------------------
+# elementary ops
+# --------------------------------------------------------------------------------------
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """RMM:137-142.  Normalise in fp32, cast to x's dtype, THEN scale by the weight in that dtype."""
+    x32 = x.float()
+    inv = torch.rsqrt(x32.pow(2).mean(dim=-1, keepdim=True) + eps)
+    return (x32 * inv).to(x.dtype) * weight
+
+
+def rope_table(head_dim: int, n_pos: int, base: float) -> torch.Tensor:
+    """RMM:2076-2081 with condense_ratio 1.  fp32 table [1, n_pos, 1, head_dim/2, 2] of (cos, sin)."""
+    expo = torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim
+    inv_freq = 1.0 / (base ** expo)
+    ang = torch.outer(torch.arange(n_pos, dtype=torch.float32), inv_freq).float()
+    return torch.stack([ang.cos()[None, :, None, :], ang.sin()[None, :, None, :]], dim=4)
+
+
+def apply_rope(q: torch.Tensor, k: torch.Tensor, freqs: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """RMM:2087-2098.  q,k [B,S,nh,hd]; freqs [1,S,1,hd/2,2].  Adjacent element pairs are rotated in fp32."""
+    def rot(t):
+        p = t.float().unflatten(-1, (-1, 2))
+        c, s_ = freqs[..., 0], freqs[..., 1]
+        out = torch.stack([p[..., 0] * c - p[..., 1] * s_, p[..., 1] * c + p[..., 0] * s_], dim=-1)
+        return out.flatten(3).to(t.dtype)
+    return rot(q), rot(k)
+
+
+def remap_step(step_idx: int, strategy: str) -> int:
+    """Cache-sharing remap of the step slot, RMM:169-182 (hard-codes 2 prelude and 4 core blocks)."""
+    if "compress-" in strategy and step_idx > 1:
+        if "compress-s" in strategy:
+            n = int(strategy.split("compress-")[1][1:])
+            return (step_idx - 2) % n + 2
+        if "compress-anchor" in strategy:
+            return step_idx if step_idx - 2 < 32 else 34 + (step_idx - 34) % 4
+        n = int(strategy.split("compress-")[1][1:])
+        return (step_idx - 2) // n + 2
+    return step_idx
+
+
+class DictCache:
+    """Brute-force model of HuginnDynamicCache (RMM:148-308): cache[step][position] -> [B, nh, hd] tensor."""
+
+    def __init__(self, lookup_strategy: str = "full"):
+        self._seen_tokens = 0
+        self.key_cache: dict[int, dict[int, torch.Tensor]] = {}
+        self.value_cache: dict[int, dict[int, torch.Tensor]] = {}
+        self.lookup_strategy = lookup_strategy
+
+    def update(self, k: torch.Tensor, v: torch.Tensor, step_idx, lookup_strategy: Optional[str] = None):
+        """k, v: [B, nh, S, hd].  Returns the stacked K, V of that step, [B, nh, T, hd] (RMM:160-204)."""
+        step = remap_step(int(step_idx), self.lookup_strategy)
+        lookup = self.lookup_strategy if lookup_strategy is None else lookup_strategy
+        n_new = k.shape[-2]
+        kc = self.key_cache.setdefault(step, {})
+        vc = self.value_cache.setdefault(step, {})
+        if step == 0:                                   # RMM:188-189
+            self._seen_tokens += n_new
+        first = self._seen_tokens - n_new
+        for i in range(n_new):
+            if "compress-" not in self.lookup_strategy:  # RMM:192-193
+                assert step < 0 or (first + i) not in kc, "overwrite of a cached position"
+            kc[first + i] = k[..., i, :]
+            vc[first + i] = v[..., i, :]
+        if len(kc) == self._seen_tokens or self.lookup_strategy == "full":
+            return torch.stack(list(kc.values()), dim=-2), torch.stack(list(vc.values()), dim=-2)
+        return self._lookup_partial(step, lookup)
+
+    def _lookup_partial(self, step: int, lookup: str):
+        """Fallbacks when some positions were never computed at this step (RMM:206-273)."""
+        ks, vs = [], []
+        for pos in range(self._seen_tokens):
+            if lookup.startswith("latest-m4") or lookup.startswith("always-last-m4"):
+                if step >= 2:
+                    pool = range(step + 1) if lookup.startswith("latest-m4") else list(self.key_cache)
+                    have = [s for s in pool if pos in self.key_cache.get(s, {})]
+                    src = max(s for s in have if s >= 2 and s % 4 == step % 4)
+                else:
+                    src = step if pos in self.key_cache[step] else 0
+            elif lookup.startswith("available-m4"):
+                if pos in self.key_cache[step]:
+                    src = step
+                else:
+                    have = [s for s in range(step + 1) if pos in self.key_cache.get(s, {})]
+                    src = max(s for s in have if s >= 2 and s % 4 == step % 4)
+            elif lookup.startswith("skip"):
+                if pos not in self.key_cache[step]:
+                    continue
+                src = step
+            else:
+                raise ValueError(f"Unknown lookup strategy: {lookup}")
+            ks.append(self.key_cache[src][pos])
+            vs.append(self.value_cache[src][pos])
+        return torch.stack(ks, dim=-2), torch.stack(vs, dim=-2)
+
+    def reset(self):  # RMM:275-279
+        self._seen_tokens = 0
+        self.key_cache.clear()
+        self.value_cache.clear()
+
+    def clear_last_k_entries(self, k: int = 0):  # RMM:281-293
+        assert self._seen_tokens >= k
+        self._seen_tokens -= k
+        keep = self._seen_tokens
+        self.key_cache = {s: {p: t for p, t in c.items() if p < keep} for s, c in self.key_cache.items()}
+        self.value_cache = {s: {p: t for p, t in c.items() if p < keep} for s, c in self.value_cache.items()}
+
+    def get_seq_length(self, step_idx: int = 0) -> int:  # RMM:295-296
+        return self._seen_tokens
+
+    def get_memory_usage(self) -> float:  # RMM:298-308: key bytes, doubled, in MiB
+        n = sum(t.nelement() * t.element_size() for c in self.key_cache.values() for t in c.values())
+        return n * 2 / (1024 * 1024)
+
+
+def sdpa(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    """The three mask cases of RMM:484-491, written out as an explicit fp32 softmax.
+
+    q [B,nh,Sq,hd], k/v [B,nh,Sk,hd].  Sq == Sk: causal.  1 < Sq < Sk: causal aligned to the
+    lower-right corner (query i sees keys 0 .. Sk-Sq+i).  Sq == 1: no mask.  Scale 1/sqrt(hd).
+    """
+    sq, sk = q.shape[-2], k.shape[-2]
+    scores = (q.float() @ k.float().transpose(-1, -2)) / math.sqrt(q.shape[-1])
+    if sq > 1:
+        qi = torch.arange(sq)[:, None]
+        kj = torch.arange(sk)[None, :]
+        scores = scores.masked_fill(kj > qi + (sk - sq), float("-inf"))
+    return (torch.softmax(scores, dim=-1) @ v.float()).to(q.dtype)
+
+
+def attention(x, w, prefix, freqs, step_idx, cache, s: RavenShape):
+    """CausalSelfAttention.forward, RMM:454-493.  x [B,S,h] is the already-normalised input."""
+    b, sq, h = x.shape
+    nh, hd = s.n_heads, s.head_dim
+    qkv = F.linear(x, w[f"{prefix}.attn.Wqkv.weight"])
+    q, k, v = (t.view(b, sq, nh, hd) for t in qkv.split([h, h, h], dim=2))
+    if s.qk_bias:
+        bias = w[f"{prefix}.attn.qk_bias"]
+        q, k = (q + bias[0:1]).to(q.dtype), (k + bias[1:2]).to(q.dtype)
+    q, k = apply_rope(q, k, freqs)
+    q, k, v = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
+    if cache is not None:
+        k, v = cache.update(k, v, step_idx)
+    y = sdpa(q, k, v)
+    y = y.transpose(1, 2).reshape(b, sq, h)
+    return F.linear(y, w[f"{prefix}.attn.proj.weight"])
+
+
+def gated_mlp(x, w, prefix):
+    """GatedMLP.forward, RMM:505-509.  The gate is the FIRST half of fc's output."""
+    gate, up = F.linear(x, w[f"{prefix}.mlp.fc.weight"]).chunk(2, dim=-1)
+    return F.linear(F.silu(gate) * up, w[f"{prefix}.mlp.proj.weight"])
+
+
+def sandwich_block(x, w, prefix, freqs, step_idx, cache, s: RavenShape):
+    """SandwichBlock.forward, RMM:525-536."""
+    eps = s.norm_eps
+    a = attention(rmsnorm(x, w[f"{prefix}.norm_1.weight"], eps), w, prefix, freqs, step_idx, cache, s)
+    x = rmsnorm(a + x, w[f"{prefix}.norm_2.weight"], eps)
+    m = gated_mlp(rmsnorm(x, w[f"{prefix}.norm_3.weight"], eps), w, prefix)
+    return rmsnorm(m + x, w[f"{prefix}.norm_4.weight"], eps)
+
+
+def core_block_forward(x, embeds, w, freqs, cache, block_idx: int, s: RavenShape):
+    """RMM:764-781 with test_time_noise == 0.  Adapter input order is (state, embedded input)."""
+    x = F.linear(torch.cat([x, embeds], dim=-1), w["transformer.adapter.weight"])
+    for j in range(s.n_layers_in_recurrent_block):
+        block_idx += 1
+        x = sandwich_block(x, w, f"transformer.core_block.{j}", freqs, block_idx, cache, s)
+    return x, block_idx
+
+
+def initialize_state(embeds: torch.Tensor, s: RavenShape, scale: float = 1.0,
+                     generator: Optional[torch.Generator] = None) -> torch.Tensor:
+    """RMM:804-813.  randn draw (discarded), truncated normal +-3 std, then times sqrt(n_embd)."""
+    x = torch.empty_like(embeds).normal_(generator=generator)
+    std = s.init_std * scale
+    if std > 0:
+        torch.nn.init.trunc_normal_(x, mean=0.0, std=std, a=-3 * std, b=3 * std, generator=generator)
+        x = x * s.emb_scale
+    else:
+        x.zero_()
+    return x
+
+
+def split_num_steps(num_steps, s: RavenShape) -> tuple[int, int]:
+    """RMM:739-744 and the eval branch of the sampler, RMM:799-802."""
+    if num_steps is None:
+        return s.mean_recurrence, 0
+    if isinstance(num_steps, torch.Tensor) and num_steps.dim() == 0:  # a 0-d tensor counts as an int
+        return int(num_steps), 0
+    if hasattr(num_steps, "__len__") and len(num_steps) > 1:
+        return int(num_steps[0]), int(num_steps[1])
+    return int(num_steps), 0
+
+
+def iterate_forward(embeds, input_states, w, freqs, block_idx: int, cache, num_steps, s: RavenShape,
+                    init_scale: float = 1.0, generator=None):
+    """RMM:726-762 (inference: the no-grad and grad loops do the same arithmetic)."""
+    x = initialize_state(embeds, s, init_scale, generator) if input_states is None else input_states.clone()
+    n0, n1 = split_num_steps(num_steps, s)
+    for _ in range(n0 + n1):
+        x, block_idx = core_block_forward(x, embeds, w, freqs, cache, block_idx, s)
+    return rmsnorm(x, w["transformer.ln_f.weight"], s.norm_eps), block_idx
+
+
+def pick_freqs(table: torch.Tensor, n_tokens: int, position_ids=None, cache_position=None):
+    """Position selection shared by forward / iterate_one_step / predict_from_latents (RMM:660-665)."""
+    if position_ids is None and cache_position is None:
+        return table[:, :n_tokens]
+    if position_ids is not None:
+        return table.index_select(1, position_ids.squeeze())
+    return table[:, cache_position]
+
+
+@dataclass
+class OracleOutput:
+    logits: torch.Tensor
+    latent_states: torch.Tensor
+    past_key_values: Optional[DictCache] = None
+    hidden_states: Optional[torch.Tensor] = None
+
+
+def forward(w, s: RavenShape, input_ids=None, input_embeds=None, input_states=None, position_ids=None,
+            num_steps=None, past_key_values=None, use_cache=False, cache_position=None, init_scale=1.0,
+            generator=None) -> OracleOutput:
+    """RavenForCausalLM.forward, RMM:638-724 (labels / stats branches left out; attention_mask is ignored there)."""
+    n_tok = input_ids.shape[1] if input_ids is not None else input_embeds.shape[1]
+    freqs = pick_freqs(w["freqs_cis"], n_tok, position_ids, cache_position)
+    if input_embeds is None:
+        input_embeds = F.embedding(input_ids, w["transformer.wte.weight"])
+    input_embeds = input_embeds * s.emb_scale
+    if use_cache and past_key_values is None:
+        past_key_values = DictCache()
+    cache = past_key_values
+    block_idx = -1
+    for i in range(s.n_layers_in_prelude):
+        block_idx += 1
+        input_embeds = sandwich_block(input_embeds, w, f"transformer.prelude.{i}", freqs, block_idx, cache, s)
+    x, block_idx = iterate_forward(input_embeds, input_states, w, freqs, block_idx, cache, num_steps, s,
+                                   init_scale, generator)
+    latents = x.clone()
+    block_idx = 0
+    for i in range(s.n_layers_in_coda):
+        block_idx -= 1
+        x = sandwich_block(x, w, f"transformer.coda.{i}", freqs, block_idx, cache, s)
+    x = rmsnorm(x, w["transformer.ln_f.weight"], s.norm_eps)
+    logits = F.linear(x, w["lm_head.weight"]).float()
+    return OracleOutput(logits=logits, latent_states=latents, past_key_values=cache, hidden_states=x)
+
+
+def greedy_generate(w, s: RavenShape, input_ids: torch.Tensor, max_new_tokens: int, num_steps=None,
+                    state_fn=None, stop_tokens=(), record: Optional[dict] = None) -> torch.Tensor:
+    """The greedy branch of generate_minimal (RMM:1165-1232, argmax at RMM:1988-1989).
+
+    `state_fn(call_index, embeds_shape)` supplies the latent state injected into each forward (the
+    reference draws it from the global RNG on every call, RMM:738; parity runs inject it instead).
+    `record`, if given, receives per-token top-2 logit margins and the cache object.
+    """
+    cache = DictCache()
+    ids = input_ids.clone()
+    alive = torch.ones(ids.shape[0], dtype=torch.bool)
+    margins = []
+    for call in range(max_new_tokens):
+        seen = cache.get_seq_length()
+        pos = torch.arange(seen, ids.shape[1])
+        step_ids = ids[:, pos]
+        states = None if state_fn is None else state_fn(call, (ids.shape[0], step_ids.shape[1], s.n_embd))
+        out = forward(w, s, input_ids=step_ids, input_states=states, num_steps=num_steps,
+                      past_key_values=cache, use_cache=True, cache_position=pos,
+                      init_scale=0.0 if state_fn is None else 1.0)
+        last = out.logits[:, -1, :].float()
+        top2 = last.topk(2, dim=-1).values
+        margins.append((top2[:, 0] - top2[:, 1]).tolist())
+        nxt = last.argmax(dim=-1, keepdim=True)
+        ids = torch.cat([ids, nxt], dim=-1)
+        for b in range(ids.shape[0]):
+            if alive[b] and int(nxt[b, 0]) in stop_tokens:
+                alive[b] = False
+        if not alive.any():
+            break
+    if record is not None:
+        record["margins"] = margins
+        record["cache"] = cache
+    return ids
+
+
+# --------------------------------------------------------------------------------------
+# closed-form accounting used as known-answer tests and by the roofline arithmetic
+# --------------------------------------------------------------------------------------
+def n_cache_slots(s: RavenShape, num_steps: Optional[int] = None) -> int:
+    r = s.mean_recurrence if num_steps is None else num_steps
+    return s.n_layers_in_prelude + s.n_layers_in_recurrent_block * r + s.n_layers_in_coda
+
+
+def step_indices(s: RavenShape, num_steps: Optional[int] = None) -> list[int]:
+    """Order in which one forward touches the cache slots (RMM:677-681, 774-779, 697-700)."""
+    r = s.mean_recurrence if num_steps is None else num_steps
+    idx = list(range(s.n_layers_in_prelude + s.n_layers_in_recurrent_block * r))
+    return idx + [-(i + 1) for i in range(s.n_layers_in_coda)]
+
+
+def core_iteration_bytes(s: RavenShape, batch: int, t_cached: int, elt: int = 2) -> dict:
+    """Algorithmic HBM bytes of one recurrence iteration at decode: weights once, KV read, KV write."""
+    h, inter, nb = s.n_embd, s.intermediate_size, s.n_layers_in_recurrent_block
+    per_block = (3 * h * h + h * h + 2 * inter * h + h * inter + 4 * h + (2 * h if s.qk_bias else 0)) * elt
+    weights = nb * per_block + 2 * h * h * elt
+    kv_read = batch * nb * 2 * h * t_cached * elt
+    kv_write = batch * nb * 2 * h * elt
+    return {"weights": weights, "kv_read": kv_read, "kv_write": kv_write, "total": weights + kv_read + kv_write}

@@ -1,0 +1,392 @@
+"""Pins for the CPU oracle: each check is something the mathematics or a library routine fixes
+independently of the oracle's own formulas, chosen so that a dropped term, a wrong sign or index,
+or a swapped operand fails at least one of them.  The reference holds no golden vectors for this
+path; its only exact published numbers (three KV-cache sizes, examples/inference_demo.ipynb:252,
+373, 491) are used as known-answer tests at the bottom."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import raven_oracle as O
+
+torch.manual_seed(1234)
+EPS = 1e-6
+
+
+# ----------------------------------------------------------------------------- RMSNorm
+def test_rmsnorm_constant_row_closed_form():
+    n, c = 5280, 3.0
+    w = torch.linspace(0.5, 1.5, n)
+    y = O.rmsnorm(torch.full((2, n), c), w, EPS)
+    assert torch.allclose(y, w * c / math.sqrt(c * c + EPS), rtol=1e-6, atol=0)
+
+
+def test_rmsnorm_one_hot_row_closed_form():
+    n, c, j = 96, -2.5, 17
+    x = torch.zeros(1, n)
+    x[0, j] = c
+    w = torch.rand(n) + 0.5
+    y = O.rmsnorm(x, w, EPS)
+    assert y[0, j].item() == pytest.approx(w[j].item() * c / math.sqrt(c * c / n + EPS), rel=1e-6)
+    assert y[0].abs().sum().item() == pytest.approx(abs(y[0, j].item()), rel=1e-6)
+
+
+def test_rmsnorm_brute_force_fp64_and_library():
+    x = torch.randn(5, 16)
+    w = torch.randn(16)
+    want = torch.empty(5, 16, dtype=torch.float64)
+    for i in range(5):
+        ms = sum(float(v) ** 2 for v in x[i]) / 16
+        for j in range(16):
+            want[i, j] = float(x[i, j]) / math.sqrt(ms + EPS) * float(w[j])
+    assert torch.allclose(O.rmsnorm(x, w, EPS).double(), want, rtol=1e-5, atol=1e-6)
+    lib = F.rms_norm(x, (16,), eps=EPS) * w
+    assert torch.allclose(O.rmsnorm(x, w, EPS), lib, rtol=1e-5, atol=1e-6)
+
+
+def test_rmsnorm_scale_invariance_and_eps_placement():
+    x = torch.randn(3, 256)
+    w = torch.ones(256)
+    assert torch.allclose(O.rmsnorm(x, w, EPS), O.rmsnorm(1000.0 * x, w, EPS), rtol=1e-4, atol=1e-5)
+    # eps is added to the MEAN of squares (not the sum, not outside the sqrt): tiny inputs expose it
+    tiny = torch.full((1, 4), 1e-3)
+    assert O.rmsnorm(tiny, torch.ones(4), 1e-6)[0, 0].item() == pytest.approx(1e-3 / math.sqrt(2e-6), rel=1e-5)
+
+
+def test_rmsnorm_rounds_before_weight_in_bf16():
+    x = torch.randn(64, 5280).bfloat16()
+    w = (1 + 0.02 * torch.randn(5280)).bfloat16()
+    got = O.rmsnorm(x, w, EPS)
+    x32 = x.float()
+    normed = x32 * torch.rsqrt((x32 * x32).mean(-1, keepdim=True) + EPS)
+    two_roundings = (normed.bfloat16().float() * w.float()).bfloat16()
+    one_rounding = (normed * w.float()).bfloat16()
+    assert got.dtype == torch.bfloat16
+    assert torch.equal(got, two_roundings)
+    assert not torch.equal(two_roundings, one_rounding)  # the distinction is observable
+
+
+# ----------------------------------------------------------------------------- RoPE
+def test_rope_table_spot_values_and_shape():
+    t = O.rope_table(96, 4096, 50000.0)
+    assert t.shape == (1, 4096, 1, 48, 2) and t.dtype == torch.float32
+    for pos, i in [(0, 0), (1, 0), (7, 5), (1023, 47), (4095, 13)]:
+        ang = np.float32(pos) * np.float32(1.0 / (50000.0 ** (2 * i / 96)))
+        assert t[0, pos, 0, i, 0].item() == pytest.approx(math.cos(ang), abs=2e-4)
+        assert t[0, pos, 0, i, 1].item() == pytest.approx(math.sin(ang), abs=2e-4)
+    assert torch.equal(t[0, 0, 0, :, 0], torch.ones(48)) and torch.equal(t[0, 0, 0, :, 1], torch.zeros(48))
+
+
+def test_rope_equals_complex_multiplication():
+    b, s, nh, hd = 2, 5, 3, 8
+    q, k = torch.randn(b, s, nh, hd), torch.randn(b, s, nh, hd)
+    tab = O.rope_table(hd, 16, 50000.0)[:, 3:3 + s]
+    rq, rk = O.apply_rope(q, k, tab)
+    ang = torch.outer(torch.arange(3, 3 + s).float(), 1.0 / (50000.0 ** (torch.arange(0, hd, 2).float() / hd)))
+    cis = torch.polar(torch.ones_like(ang), ang)[None, :, None, :]
+    for got, src in ((rq, q), (rk, k)):
+        want = torch.view_as_real(torch.view_as_complex(src.reshape(b, s, nh, hd // 2, 2)) * cis).flatten(3)
+        assert torch.allclose(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_rope_identity_norm_and_relative_position():
+    hd = 96
+    tab = O.rope_table(hd, 64, 50000.0)
+    q, k = torch.randn(1, 1, 2, hd), torch.randn(1, 1, 2, hd)
+    q0, k0 = O.apply_rope(q, k, tab[:, 0:1])
+    assert torch.equal(q0, q) and torch.equal(k0, k)
+    qm, _ = O.apply_rope(q, k, tab[:, 9:10])
+    pn = lambda t: t.unflatten(-1, (-1, 2)).norm(dim=-1)
+    assert torch.allclose(pn(qm), pn(q), rtol=1e-5, atol=1e-6)
+    dots = []
+    for m, n in ((9, 4), (25, 20), (45, 40)):
+        a, _ = O.apply_rope(q, q, tab[:, m:m + 1])
+        _, c = O.apply_rope(k, k, tab[:, n:n + 1])
+        dots.append((a * c).sum().item())
+    assert dots[0] == pytest.approx(dots[1], rel=1e-4, abs=1e-4) and dots[1] == pytest.approx(dots[2], rel=1e-4, abs=1e-4)
+    # sign convention: rotating (1, 0) by +angle gives (cos, +sin)
+    e = torch.zeros(1, 1, 1, hd)
+    e[..., 0] = 1.0
+    r, _ = O.apply_rope(e, e, tab[:, 5:6])
+    assert r[0, 0, 0, 0].item() == pytest.approx(math.cos(5.0), abs=1e-5)
+    assert r[0, 0, 0, 1].item() == pytest.approx(math.sin(5.0), abs=1e-5)
+
+
+# ----------------------------------------------------------------------------- attention
+def _eager64(q, k, v, mask=None):
+    s = (q.double() @ k.double().transpose(-1, -2)) / math.sqrt(q.shape[-1])
+    if mask is not None:
+        s = s.masked_fill(~mask, float("-inf"))
+    return torch.softmax(s, -1) @ v.double()
+
+
+def test_sdpa_decode_special_cases():
+    q, k, v = torch.randn(2, 3, 1, 16), torch.randn(2, 3, 7, 16), torch.randn(2, 3, 7, 16)
+    assert torch.allclose(O.sdpa(q, k, v).double(), _eager64(q, k, v), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(O.sdpa(q, k[..., :1, :], v[..., :1, :]), v[..., :1, :], rtol=1e-6, atol=1e-7)
+    assert torch.allclose(O.sdpa(torch.zeros_like(q), k, v), v.mean(-2, keepdim=True), rtol=1e-5, atol=1e-6)
+
+
+def test_sdpa_mask_cases_match_library():
+    q, k, v = torch.randn(1, 2, 5, 8), torch.randn(1, 2, 5, 8), torch.randn(1, 2, 5, 8)
+    assert torch.allclose(O.sdpa(q, k, v), F.scaled_dot_product_attention(q, k, v, is_causal=True), rtol=1e-5, atol=1e-6)
+    k2, v2 = torch.randn(1, 2, 9, 8), torch.randn(1, 2, 9, 8)
+    mask = torch.ones(5, 9, dtype=torch.bool).tril(diagonal=4)       # lower-right aligned causal
+    assert torch.allclose(O.sdpa(q, k2, v2).double(), _eager64(q, k2, v2, mask), rtol=1e-5, atol=1e-6)
+    lib = F.scaled_dot_product_attention(q, k2, v2, attn_mask=mask)
+    assert torch.allclose(O.sdpa(q, k2, v2), lib, rtol=1e-5, atol=1e-6)
+    q1 = q[..., :1, :]
+    assert torch.allclose(O.sdpa(q1, k2, v2), F.scaled_dot_product_attention(q1, k2, v2), rtol=1e-5, atol=1e-6)
+
+
+# ----------------------------------------------------------------------------- linear pieces
+def _tiny(dtype=torch.float32, seed=0):
+    s = O.RavenShape.tiny()
+    return s, O.make_weights(s, seed=seed, dtype=dtype)
+
+
+def test_adapter_operand_order_and_split_identity():
+    s, w = _tiny()
+    h = s.n_embd
+    state, emb = torch.randn(1, 1, h), torch.randn(1, 1, h)
+    wa = w["transformer.adapter.weight"]
+    want = (state.double() @ wa[:, :h].double().T) + (emb.double() @ wa[:, h:].double().T)
+    blocks_off = dict(w)
+    got = F.linear(torch.cat([state, emb], -1), wa)
+    assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-6)
+    swapped = F.linear(torch.cat([emb, state], -1), wa)
+    assert not torch.allclose(got, swapped, rtol=1e-3, atol=1e-4)
+    # the oracle's core step applies exactly that adapter before its blocks
+    s0 = O.RavenShape(**{**s.__dict__, "n_layers_in_recurrent_block": 0})
+    x, idx = O.core_block_forward(state, emb, blocks_off, None, None, 0, s0)
+    assert torch.equal(x, got) and idx == 0
+
+
+def test_gated_mlp_fp64_and_gate_half():
+    s, w = _tiny()
+    p = "transformer.core_block.0"
+    x = torch.randn(2, 3, s.n_embd)
+    fc, pr = w[f"{p}.mlp.fc.weight"].double(), w[f"{p}.mlp.proj.weight"].double()
+    z = x.double() @ fc.T
+    a, b = z[..., : s.intermediate_size], z[..., s.intermediate_size:]
+    want = ((a / (1 + torch.exp(-a))) * b) @ pr.T
+    got = O.gated_mlp(x, w, p).double()
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-7)
+    wrong = ((b / (1 + torch.exp(-b))) * a) @ pr.T
+    assert not torch.allclose(got, wrong, rtol=1e-2, atol=1e-5)
+
+
+def test_attention_projection_split_bias_and_cache_contents():
+    s, w = _tiny()
+    p = "transformer.prelude.0"
+    h, nh, hd = s.n_embd, s.n_heads, s.head_dim
+    x = torch.randn(2, 3, h)
+    freqs = w["freqs_cis"][:, 4:7]
+    cache = O.DictCache()
+    cache._seen_tokens = 4  # pretend four tokens were seen; step 0 adds 3 more
+    out = O.attention(x, w, p, freqs, 0, cache, s)
+    qkv = x.double() @ w[f"{p}.attn.Wqkv.weight"].double().T
+    q, k, v = qkv[..., :h], qkv[..., h:2 * h], qkv[..., 2 * h:]
+    bias = w[f"{p}.attn.qk_bias"].double()
+    k = (k.view(2, 3, nh, hd) + bias[1])
+    ang = torch.outer(torch.arange(4, 7).double(), 1.0 / (50000.0 ** (torch.arange(0, hd, 2).double() / hd)))
+    cis = torch.polar(torch.ones_like(ang), ang)[None, :, None, :]
+    k_rot = torch.view_as_real(torch.view_as_complex(k.reshape(2, 3, nh, hd // 2, 2).contiguous()) * cis).flatten(3)
+    assert sorted(cache.key_cache[0]) == [4, 5, 6] and cache.get_seq_length() == 7
+    for i, pos in enumerate((4, 5, 6)):
+        assert torch.allclose(cache.key_cache[0][pos].double(), k_rot[:, i], rtol=1e-4, atol=1e-5)  # post-bias, post-RoPE
+        assert torch.allclose(cache.value_cache[0][pos].double(), v.view(2, 3, nh, hd)[:, i], rtol=1e-4, atol=1e-5)  # no bias on v
+    assert out.shape == (2, 3, h)
+
+
+def test_sandwich_block_is_the_stated_composition():
+    s, w = _tiny()
+    p = "transformer.core_block.1"
+    x = torch.randn(1, 4, s.n_embd)
+    freqs = w["freqs_cis"][:, :4]
+    got = O.sandwich_block(x, w, p, freqs, 3, None, s)
+    n = lambda t, k: O.rmsnorm(t, w[f"{p}.norm_{k}.weight"], s.norm_eps)
+    a = O.attention(n(x, 1), w, p, freqs, 3, None, s)
+    x2 = n(a + x, 2)
+    want = n(O.gated_mlp(n(x2, 3), w, p) + x2, 4)
+    assert torch.equal(got, want)
+    # a residual taken from the wrong place (pre-norm style) gives something else
+    wrong = n(O.gated_mlp(n(x2, 3), w, p) + x, 4)
+    assert not torch.allclose(got, wrong, rtol=1e-3, atol=1e-4)
+
+
+# ----------------------------------------------------------------------------- recurrence and forward
+def test_num_steps_forms_and_zero_steps():
+    s, w = _tiny()
+    emb = torch.randn(1, 2, s.n_embd)
+    st = torch.randn(1, 2, s.n_embd)
+    fr = w["freqs_cis"][:, :2]
+    y0, idx0 = O.iterate_forward(emb, st, w, fr, 0, None, 0, s)
+    assert torch.equal(y0, O.rmsnorm(st, w["transformer.ln_f.weight"], s.norm_eps)) and idx0 == 0
+    a, ia = O.iterate_forward(emb, st, w, fr, 0, None, 3, s)
+    b, ib = O.iterate_forward(emb, st, w, fr, 0, None, torch.tensor(3), s)
+    c, ic = O.iterate_forward(emb, st, w, fr, 0, None, (2, 1), s)
+    d, idd = O.iterate_forward(emb, st, w, fr, 0, None, None, O.RavenShape(**{**s.__dict__, "mean_recurrence": 3}))
+    assert torch.equal(a, b) and torch.equal(a, c) and torch.equal(a, d)
+    assert ia == ib == ic == idd == 3 * s.n_layers_in_recurrent_block
+
+
+def test_step_index_enumeration():
+    assert O.step_indices(O.RavenShape.nebel()) == list(range(130)) + [-1, -2]
+    assert O.step_indices(O.RavenShape.tiny()) == list(range(9)) + [-1]
+    assert O.n_cache_slots(O.RavenShape.nebel()) == 132
+    s, w = _tiny()
+    cache = O.DictCache()
+    O.forward(w, s, input_ids=torch.randint(0, s.vocab_size, (1, 3)), input_states=torch.zeros(1, 3, s.n_embd),
+              past_key_values=cache, use_cache=True)
+    assert list(cache.key_cache) == O.step_indices(s)
+    assert all(sorted(c) == [0, 1, 2] for c in cache.key_cache.values())
+    assert cache.get_seq_length() == 3
+
+
+def test_cache_and_no_cache_agree_and_prefill_then_decode():
+    s, w = _tiny()
+    ids = torch.randint(0, s.vocab_size, (2, 6))
+    states = 0.6 * torch.randn(2, 6, s.n_embd)
+    full = O.forward(w, s, input_ids=ids, input_states=states).logits
+    # prefill 4, then two single-token decode steps through the cache
+    cache = O.DictCache()
+    a = O.forward(w, s, input_ids=ids[:, :4], input_states=states[:, :4], past_key_values=cache, use_cache=True,
+                  cache_position=torch.arange(0, 4)).logits
+    b = O.forward(w, s, input_ids=ids[:, 4:5], input_states=states[:, 4:5], past_key_values=cache, use_cache=True,
+                  cache_position=torch.arange(4, 5)).logits
+    c = O.forward(w, s, input_ids=ids[:, 5:6], input_states=states[:, 5:6], past_key_values=cache, use_cache=True,
+                  cache_position=torch.arange(5, 6)).logits
+    got = torch.cat([a, b, c], dim=1)
+    assert torch.allclose(got, full, rtol=1e-4, atol=1e-5)
+    # two-token chunk against a longer cache exercises the lower-right-aligned causal case
+    cache2 = O.DictCache()
+    O.forward(w, s, input_ids=ids[:, :4], input_states=states[:, :4], past_key_values=cache2, use_cache=True,
+              cache_position=torch.arange(0, 4))
+    d = O.forward(w, s, input_ids=ids[:, 4:6], input_states=states[:, 4:6], past_key_values=cache2, use_cache=True,
+                  cache_position=torch.arange(4, 6)).logits
+    assert torch.allclose(d, full[:, 4:6], rtol=1e-4, atol=1e-5)
+
+
+def test_forward_head_is_tied_scaled_and_double_normed():
+    s, w = _tiny()
+    ids = torch.randint(0, s.vocab_size, (1, 2))
+    st = torch.randn(1, 2, s.n_embd)
+    out = O.forward(w, s, input_ids=ids, input_states=st, num_steps=0)
+    # with zero recurrences the latent is ln_f(state), and the logits follow from the coda alone
+    lat = O.rmsnorm(st, w["transformer.ln_f.weight"], s.norm_eps)
+    assert torch.equal(out.latent_states, lat)
+    x = O.sandwich_block(lat, w, "transformer.coda.0", w["freqs_cis"][:, :2], -1, None, s)
+    x = O.rmsnorm(x, w["transformer.ln_f.weight"], s.norm_eps)
+    assert torch.allclose(out.logits, x @ w["transformer.wte.weight"].T, rtol=1e-5, atol=1e-6)
+    assert out.logits.dtype == torch.float32
+    # embedding scale sqrt(n_embd): feeding pre-scaled embeddings by hand must not change anything
+    emb = F.embedding(ids, w["transformer.wte.weight"])
+    out2 = O.forward(w, s, input_embeds=emb, input_states=st, num_steps=1)
+    out3 = O.forward(w, s, input_ids=ids, input_states=st, num_steps=1)
+    assert torch.equal(out2.logits, out3.logits)
+    pre = O.sandwich_block(emb * 16.0, w, "transformer.prelude.0", w["freqs_cis"][:, :2], 0, None, s)
+    x1, _ = O.core_block_forward(st, pre, w, w["freqs_cis"][:, :2], None, 0, s)
+    assert torch.equal(out3.latent_states, O.rmsnorm(x1, w["transformer.ln_f.weight"], s.norm_eps))
+
+
+def test_initialize_state_distribution():
+    s = O.RavenShape.nebel()
+    g = torch.Generator().manual_seed(7)
+    x = O.initialize_state(torch.empty(4, 8, s.n_embd), s, 1.0, g)
+    bound = 3 * s.init_std * s.emb_scale
+    assert x.abs().max().item() <= bound * (1 + 1e-6)
+    assert x.std().item() == pytest.approx(math.sqrt(2 / 5) * 0.9866, rel=2e-2)  # std of a +-3 sigma truncated normal
+    assert torch.equal(x, O.initialize_state(torch.empty(4, 8, s.n_embd), s, 1.0, torch.Generator().manual_seed(7)))
+    assert O.initialize_state(torch.empty(1, 2, 16), s, 0.0).abs().sum().item() == 0.0
+
+
+def test_greedy_is_argmax_of_last_position_and_deterministic():
+    s, w = _tiny()
+    prompt = torch.randint(0, s.vocab_size, (1, 8), generator=torch.Generator().manual_seed(3))
+    rec = {}
+    ids = O.greedy_generate(w, s, prompt, 5, record=rec)
+    assert ids.shape == (1, 13) and torch.equal(ids[:, :8], prompt)
+    ids2 = O.greedy_generate(w, s, prompt, 5)
+    assert torch.equal(ids, ids2)
+    # first new token equals argmax of a cache-less full forward with a zero state
+    logits = O.forward(w, s, input_ids=prompt, input_states=torch.zeros(1, 8, s.n_embd)).logits
+    assert int(ids[0, 8]) == int(logits[0, -1].argmax())
+    assert rec["cache"].get_seq_length() == 12  # the last generated token was never fed back
+    assert len(rec["margins"]) == 5
+
+
+# ----------------------------------------------------------------------------- cache model
+def test_dict_cache_against_list_model():
+    rng = torch.Generator().manual_seed(5)
+    cache = O.DictCache()
+    log: dict[int, list] = {}
+    seen = 0
+    for n_new in (3, 1, 1, 2):
+        for step in (0, 1, 2, 5, -1):
+            k = torch.randn(2, 3, n_new, 4, generator=rng)
+            v = torch.randn(2, 3, n_new, 4, generator=rng)
+            if step == 0:
+                seen += n_new
+            log.setdefault(step, []).append((k, v))
+            gk, gv = cache.update(k, v, torch.tensor(step))
+            assert torch.equal(gk, torch.cat([a for a, _ in log[step]], dim=-2))
+            assert torch.equal(gv, torch.cat([b for _, b in log[step]], dim=-2))
+            assert cache.get_seq_length() == seen
+    assert seen == 7 and sorted(cache.key_cache[5]) == list(range(7))
+    cache.clear_last_k_entries(2)
+    assert cache.get_seq_length() == 5 and all(sorted(c) == list(range(5)) for c in cache.key_cache.values())
+    with pytest.raises(AssertionError):
+        cache.update(torch.zeros(2, 3, 1, 4), torch.zeros(2, 3, 1, 4), 1)  # step 1 before step 0: position 4 exists
+    cache.reset()
+    assert cache.get_seq_length() == 0 and not cache.key_cache
+
+
+def test_step_remap_strategies():
+    assert [O.remap_step(i, "full") for i in (0, 1, 2, 129, -1)] == [0, 1, 2, 129, -1]
+    assert [O.remap_step(i, "latest-m4-compress-s4") for i in (0, 1, 2, 5, 6, 9, 129, -1, -2)] == [0, 1, 2, 5, 2, 5, 5, -1, -2]
+    assert [O.remap_step(i, "compress-s16") for i in (2, 17, 18, 33, 34)] == [2, 17, 2, 17, 2]
+    assert [O.remap_step(i, "compress-r4") for i in (2, 5, 6, 129)] == [2, 2, 3, 33]
+    assert [O.remap_step(i, "compress-anchor") for i in (2, 33, 34, 37, 38, 41, 129)] == [2, 33, 34, 37, 34, 37, 37]
+
+
+def test_published_cache_sizes():
+    """examples/inference_demo.ipynb:252, 373, 491 of the reference."""
+    s = O.RavenShape.nebel()
+    entry = torch.zeros(1, s.n_heads, s.head_dim, dtype=torch.bfloat16)
+    c = O.DictCache()
+    for step in O.step_indices(s):
+        c.key_cache[step] = {p: entry for p in range(366)}
+    assert c.get_memory_usage() == 973.0810546875
+    c16 = O.DictCache("latest-m4-compress-s16")
+    for step in sorted({O.remap_step(i, c16.lookup_strategy) for i in O.step_indices(s)}):
+        c16.key_cache[step] = {p: entry for p in range(366)}
+    assert len(c16.key_cache) == 20 and c16.get_memory_usage() == 147.4365234375
+    assert 132 * 55 * 1024 * 96 * 2 * 2 / 2**20 == 2722.5
+
+
+def test_core_iteration_byte_count_matches_survey():
+    s = O.RavenShape.nebel()
+    b1 = O.core_iteration_bytes(s, 1, 1024)
+    assert b1["weights"] == 3_274_698_240 and b1["kv_read"] == 86_507_520 and b1["kv_write"] == 84_480
+    assert O.core_iteration_bytes(s, 32, 1024)["total"] == 3_274_698_240 + 32 * (86_507_520 + 84_480)
+
+
+def test_make_weights_layout_and_determinism():
+    s = O.RavenShape.tiny()
+    w = O.make_weights(s, seed=0)
+    names = [n for n, _ in O.state_dict_layout(s)]
+    assert names[0] == "transformer.wte.weight" and names[-1] == "transformer.ln_f.weight"
+    assert "transformer.prelude.0.attn.qk_bias" in names and "transformer.adapter.weight" in names
+    assert w["lm_head.weight"] is w["transformer.wte.weight"]
+    assert w["transformer.core_block.1.mlp.fc.weight"].shape == (2 * 704, 256)
+    assert w["transformer.prelude.0.attn.qk_bias"].shape == (2, 1, 4, 64)
+    w2 = O.make_weights(s, seed=0)
+    assert all(torch.equal(w[k], w2[k]) for k in w)
+    assert abs(w["transformer.ln_f.weight"].mean().item() - 1.0) < 0.01
+    n_params = sum(math.prod(sh) for _, sh in O.state_dict_layout(O.RavenShape.nebel()))
+    assert n_params == 3_564_976_800 + 0  # tied head counted once
