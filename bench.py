@@ -1,0 +1,255 @@
+#!/usr/bin/env python3
+"""Benchmark of the recurrent-core decode path on one MI355X.
+
+A step is one decoded token at the nebel-raven-3.5b shape in bf16: embedding, 2 prelude blocks,
+r = 32 recurrences of (adapter + 4 SandwichBlocks), 2 coda blocks, ln_f, LM head over 65536 and the
+greedy argmax, with the KV cache of a 512-token prompt already resident (random-init weights, random
+token ids).  Prints ONE JSON line:
+  value            decoded tokens/s (whole job, one GPU, batch `--batch`, default 1)
+  roofline         the dominant kernel (fc GEMV with the SwiGLU epilogue, 47 % of a token's bytes):
+                   algorithmic bytes per launch / its mean duration (HIP events on the launch stream)
+  core_iteration   one recurrence iteration (the unit the 70 %-of-HBM target is stated on)
+  cpu_baseline     the CPU oracle on this box's host cores, on a bounded sample, scaled to tokens/s
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=48)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--recurrence", type=int, default=32)
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-iters", type=int, default=3)
+    ap.add_argument("--also-batch", type=int, default=32, help="second batch size reported under 'also' (0 = skip)")
+    return ap.parse_args()
+
+
+def event_time_ms(fn, reps, warm=3):
+    import torch
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+def fill_synthetic(model, seed=0):
+    """Random-init weights N(0, 0.02) (norm weights N(1, 0.02)) drawn on the GPU: synthetic data."""
+    import torch
+    torch.manual_seed(seed)
+    with torch.no_grad():
+        for name, p in model.state_dict().items():
+            if name == "freqs_cis" or (name == "lm_head.weight" and model.config.tie_embeddings):
+                continue
+            p.normal_(1.0 if p.dim() == 1 else 0.0, 0.02)
+
+
+def decode_tokens_per_s(pkg, model, batch, prompt_len, steps, warmup, r, use_graph):
+    """Prefills a random prompt, then times `steps` greedy decode steps (state re-drawn per token)."""
+    import torch
+    cfg = model.config
+    g = torch.Generator().manual_seed(1)
+    prompt = torch.randint(0, cfg.vocab_size, (batch, prompt_len), generator=g).cuda()
+    total = prompt_len + warmup + steps + 1
+    cache = pkg.HuginnDynamicCache(max_length=total)
+    t0 = time.perf_counter()
+    out = model(input_ids=prompt, past_key_values=cache, use_cache=True, cache_position=torch.arange(prompt_len).cuda(), num_steps=r)
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    tok = out.logits[:, -1].argmax(-1)
+    runner = pkg.DecodeRunner(model, cache, batch, r, greedy=True, use_graph=use_graph)
+    for _ in range(warmup):
+        _, nxt, _ = runner.step(tok, None, 1.0)
+        tok = nxt.clone()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        _, nxt, _ = runner.step(tok, None, 1.0)
+        tok = nxt.clone()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    return batch * steps / dt, dt / steps * 1e3, prefill_s, cache
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the decode path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import __graft_entry__ as entry
+    from oracle import raven_oracle as O
+
+    pkg = entry.import_package()
+    pkg.hip.load()
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    shape = O.RavenShape.nebel()
+    cfg = pkg.RavenConfig()
+    r = args.recurrence
+    model = pkg.RavenForCausalLM(cfg, device=dev, dtype=torch.bfloat16)
+    fill_synthetic(model, 0)
+    use_graph = not args.no_graph
+
+    tok_s, ms_step, prefill_s, cache = decode_tokens_per_s(pkg, model, args.batch, args.prompt, args.steps, args.warmup, r, use_graph)
+    mean_t = args.prompt + args.warmup + args.steps / 2.0
+    blocks_bytes = O.core_iteration_bytes(shape, args.batch, int(mean_t))
+    per_block_w = (blocks_bytes["weights"] - 2 * shape.n_embd * shape.n_embd * 2) // 4
+    token_bytes = (r * blocks_bytes["total"] + 4 * (per_block_w + (blocks_bytes["kv_read"] + blocks_bytes["kv_write"]) // 4)
+                   + shape.vocab_size * shape.n_embd * 2)
+    del cache
+    torch.cuda.empty_cache()
+
+    # ---- one recurrence iteration at T = 1024 (the unit of the roofline target) ----
+    B = args.batch
+    h, nh, hd, T = cfg.n_embd, cfg.n_heads, cfg.head_dim, 1024
+    nat = model._natives()
+    kc = torch.randn(4, B, nh, T + 1, hd, device=dev, dtype=torch.bfloat16)
+    vc = torch.randn(4, B, nh, T + 1, hd, device=dev, dtype=torch.bfloat16)
+    kv = pkg.hip.make_cache(kc, vc)
+    ws = pkg.hip.block_workspace(nat["dims"], B, dev)
+    state = torch.randn(B, h, device=dev, dtype=torch.bfloat16)
+    emb = torch.randn(B, h, device=dev, dtype=torch.bfloat16)
+    outb = torch.empty_like(state)
+    adapter_w = model.transformer.adapter.weight
+
+    def one_iter():
+        pkg.hip.core_iteration(nat["dims"], adapter_w, nat["core"], state, emb, outb, nat["freqs"], kv, 0, B, 1, T, ws)
+
+    iter_eager_ms = event_time_ms(one_iter, 20)
+    one_iter()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(8):
+            one_iter()
+    iter_graph_ms = event_time_ms(graph.replay, 10) / 8
+    it_bytes = O.core_iteration_bytes(shape, B, T)["total"]
+    iter_ms = min(iter_eager_ms, iter_graph_ms)
+
+    # ---- dominant kernel: fc GEMV + SwiGLU ----
+    fc_w = model.transformer.core_block[0].mlp.fc.weight
+    xin = torch.randn(B, h, device=dev, dtype=torch.bfloat16)
+    gout = torch.empty(B, cfg.intermediate_size, device=dev, dtype=torch.bfloat16)
+    lib = pkg.hip.load()
+
+    def fc_launch():
+        lib.raven_gemm_swiglu(xin.data_ptr(), fc_w.data_ptr(), gout.data_ptr(), B, cfg.intermediate_size, h, pkg.hip.BF16,
+                              torch.cuda.current_stream().cuda_stream)
+
+    fc_ms = event_time_ms(fc_launch, 200, warm=10)
+    fc_bytes = fc_w.numel() * 2 + B * h * 2 + B * cfg.intermediate_size * 2
+    fc_gbs = fc_bytes / (fc_ms * 1e-3) / 1e9
+
+    # ---- device copy bandwidth, for context next to the published peak ----
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    copy_ms = event_time_ms(lambda: dst.copy_(src), 10)
+    copy_gbs = 2 * src.numel() / (copy_ms * 1e-3) / 1e9
+    del src, dst, kc, vc
+
+    also = None
+    if args.also_batch and args.also_batch != args.batch:
+        torch.cuda.empty_cache()
+        steps2 = max(8, args.steps // 4)
+        t2, ms2, _, c2 = decode_tokens_per_s(pkg, model, args.also_batch, args.prompt, steps2, 2, r, use_graph)
+        also = {"batch": args.also_batch, "tokens_per_s": round(t2, 2), "ms_per_step": round(ms2, 3), "steps": steps2}
+        del c2
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(O, shape, model, args.cpu_iters, r)
+
+    line = {
+        "metric": "decode tokens/s at r=32, raven-3.5b shape bf16 bs=1/32; % HBM roofline",
+        "value": round(tok_s, 3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"full-token greedy decode, nebel-raven-3.5b shape, r={r}, bs={args.batch}, "
+                               f"{args.prompt}-token random prompt, {args.steps} timed tokens (BASELINE configs[3])",
+                   "batch": args.batch, "recurrence": r, "prompt": args.prompt, "hip_graph": use_graph},
+        "recurrence_steps_per_s": round(tok_s * r / args.batch, 2),
+        "token_roofline": {"bytes_per_token": int(token_bytes), "achieved_GBs": round(token_bytes * (tok_s / args.batch) / 1e9, 1),
+                           "frac": round(token_bytes * (tok_s / args.batch) / 1e9 / HBM_PEAK_GBS, 4)},
+        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<bf16,SwiGLU> (mlp.fc 35840x5280)" if B <= 4 else "mfma_kernel<SwiGLU> (mlp.fc 35840x5280)",
+                     "achieved": round(fc_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(fc_gbs / HBM_PEAK_GBS, 4),
+                     "bytes_per_launch": int(fc_bytes), "avg_us": round(fc_ms * 1e3, 2), "traffic": None},
+        "core_iteration": {"T": T, "batch": B, "bytes": int(it_bytes), "ms_eager": round(iter_eager_ms, 4),
+                           "ms_graph": round(iter_graph_ms, 4), "achieved_GBs": round(it_bytes / (iter_ms * 1e-3) / 1e9, 1),
+                           "frac": round(it_bytes / (iter_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+        "device_copy_GBs": round(copy_gbs, 1),
+        "prefill_s": round(prefill_s, 3),
+        "also": also,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+def cpu_baseline(O, shape, model, n_iters, r):
+    """The CPU oracle (a port of the reference's CPU path) on the host cores: a few recurrence
+    iterations plus one LM-head product at the nebel shape, bs=1, 512 cached positions, scaled to
+    tokens/s as 1 / ((r + 1) * t_iteration + t_head) -- the 4 prelude/coda blocks cost one iteration."""
+    import torch
+    T = 512
+    w = {}
+    for name, p in model.state_dict().items():
+        if name.startswith("transformer.core_block") or name.startswith("transformer.adapter") or name == "transformer.wte.weight":
+            w[name] = p.detach().cpu()
+    table = O.rope_table(shape.head_dim, shape.block_size, shape.rope_base).to(torch.bfloat16)
+    g = torch.Generator().manual_seed(0)
+    cache = O.DictCache()
+    cache._seen_tokens = T
+    kv = torch.randn(2, 1, shape.n_heads, T, shape.head_dim, generator=g).to(torch.bfloat16)
+    x = O.initialize_state(torch.empty(1, 1, shape.n_embd), shape, 1.0, g).to(torch.bfloat16)
+    emb = torch.randn(1, 1, shape.n_embd, generator=g).to(torch.bfloat16)
+    n_threads = torch.get_num_threads()
+    times = []
+    for it in range(n_iters + 1):  # first pass is warm-up
+        for j in range(4):
+            cache.key_cache[2 + j] = {p: kv[0, :, :, p] for p in range(T - 1)}
+            cache.value_cache[2 + j] = {p: kv[1, :, :, p] for p in range(T - 1)}
+        t0 = time.perf_counter()
+        O.core_block_forward(x, emb, w, table[:, T - 1:T], cache, 1, shape)
+        times.append(time.perf_counter() - t0)
+    t_iter = sum(times[1:]) / max(1, len(times) - 1)
+    t0 = time.perf_counter()
+    torch.nn.functional.linear(x, w["transformer.wte.weight"]).float()
+    t_head = time.perf_counter() - t0
+    tok_s = 1.0 / ((r + 1) * t_iter + t_head)
+    return {"value": round(tok_s, 5), "unit": "tokens/s", "cores": n_threads, "kind": "port",
+            "sample": f"{n_iters} recurrence iterations (mean {t_iter * 1e3:.1f} ms) + 1 LM head ({t_head * 1e3:.1f} ms) at nebel shape, "
+                      f"bs=1, {T} cached positions, torch CPU bf16, {n_threads} threads of {os.cpu_count()} cpus; "
+                      f"scaled to a token as ({r}+1) iterations + head"}
+
+
+if __name__ == "__main__":
+    main()

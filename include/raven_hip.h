@@ -1,0 +1,155 @@
+/*
+ * raven_hip.h -- C ABI of libraven_hip.so: hand-written gfx950 (MI355X) kernels for the
+ * recurrent-core decode path of the Huginn/Raven model.
+ *
+ * The reference (seal-rg/recurrent-pretraining) is pure Python and has no FFI; each entry point
+ * below names the lines of recpre/raven_modeling_minimal.py ("RMM") whose arithmetic it replaces.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the name ends in _host; buffers are caller-owned;
+ *     nothing here allocates, frees or synchronises; work is enqueued on `stream` (a hipStream_t).
+ *   - tensors are dense row-major. "T" is the model dtype: RAVEN_F32 or RAVEN_BF16.
+ *   - token rows: activations are [M, h] with M = B*S rows; row m belongs to sequence b = m / S and
+ *     has position pos0 + (m % S).  Decode is S = 1; a prefill chunk is S > 1.
+ *   - `pos_dev` (nullable): when given, kernels read pos0 from this device int32 instead of the
+ *     by-value argument, so a captured HIP graph can be replayed as the sequence grows; the by-value
+ *     `pos0` then only sizes grids and must be >= the largest value *pos_dev will take.
+ *   - return value: 0 ok; < 0 invalid argument (see raven_last_error()); > 0 a hipError_t.
+ *   - workspaces must be 256-byte aligned.  The attention workspace must be zero-filled once before
+ *     its first use (it holds arrival counters that every call leaves at zero again).
+ *   - calls that share a workspace must be ordered on one stream.
+ */
+#ifndef RAVEN_HIP_H
+#define RAVEN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { RAVEN_F32 = 0, RAVEN_BF16 = 1 };
+
+/* Shape of one SandwichBlock (recpre/raven_config_minimal.py:12-91). */
+typedef struct raven_dims {
+    int32_t n_embd;       /* h                                   */
+    int32_t n_heads;      /* nh, with h == nh * head_dim          */
+    int32_t head_dim;     /* hd, even, hd * sizeof(T) <= 256      */
+    int32_t intermediate; /* I: fc is [2I, h], mlp.proj is [h, I] */
+    float   eps;          /* RMSNorm epsilon                      */
+    int32_t dtype;        /* RAVEN_F32 | RAVEN_BF16               */
+} raven_dims;
+
+/* Weights of one SandwichBlock, state-dict names in comments (RMM:515-523). */
+typedef struct raven_block_weights {
+    const void* norm_1;   /* [h]      norm_1.weight          */
+    const void* norm_2;   /* [h]      norm_2.weight          */
+    const void* norm_3;   /* [h]      norm_3.weight          */
+    const void* norm_4;   /* [h]      norm_4.weight          */
+    const void* wqkv;     /* [3h, h]  attn.Wqkv.weight       */
+    const void* qk_bias;  /* [2,nh,hd] attn.qk_bias or NULL  */
+    const void* proj;     /* [h, h]   attn.proj.weight       */
+    const void* fc;       /* [2I, h]  mlp.fc.weight          */
+    const void* mlp_proj; /* [h, I]   mlp.proj.weight        */
+} raven_block_weights;
+
+/* Step-indexed KV cache, the HuginnStaticCache layout (RMM:344-349): K and V are
+ * [n_slots, batch, nh, t_max, hd] of T.  Slot s of the reference's step index is s for s >= 0 and
+ * n_slots + s for the coda's negative indices (RMM:375-380 index from the end the same way). */
+typedef struct raven_kv_cache {
+    void*   k;
+    void*   v;
+    int32_t n_slots;
+    int32_t batch;
+    int32_t t_max;
+} raven_kv_cache;
+
+/* Library identity: version, the gfx arch the kernels were compiled for, last error text. */
+int         raven_version(void);
+const char* raven_arch(void);
+const char* raven_last_error(void);
+
+/* RMSNorm with the reference's two roundings, optionally preceded by a residual add and followed by
+ * a second norm.  RMM:137-142 (norm), RMM:534-535 (the adds feeding norm_2 / norm_4).
+ *   s  = residual ? T(x + residual) : x          -> stored to sum_out when non-NULL
+ *   y  = T(s32 * rsqrt(mean(s32^2) + eps)) * weight          (y may be NULL when only y2 is wanted)
+ *   y2 = T(y32 * rsqrt(mean(y32^2) + eps)) * weight2         (only when weight2 and y2 are given)
+ * x, residual, y, sum_out, y2: [rows, dim] of T; weights [dim] of T. dim * sizeof(T) % 16 == 0. */
+int raven_rmsnorm_residual(const void* x, const void* residual, const void* weight, void* y,
+                           void* sum_out, const void* weight2, void* y2,
+                           int64_t rows, int32_t dim, float eps, int32_t dtype, void* stream);
+
+/* Y[M,N] = X[M,K] W[N,K]^T for skinny M (any M >= 1; the weight matrix is streamed once per 32
+ * (bf16) or 8 (f32) rows).  Replaces the nn.Linear calls of attn.proj (RMM:493), mlp.proj (RMM:509)
+ * and lm_head (RMM:711).  fp32 accumulate, result rounded to T; then, if residual != NULL,
+ * Y = T(Y + residual) (RMM:534-535); if out_f32 != 0 the rounded result is stored as float
+ * (the `.float()` of RMM:711).  K * sizeof(T) % 16 == 0. */
+int raven_gemm(const void* x, const void* w, const void* residual, void* y,
+               int32_t M, int32_t N, int32_t K, int32_t dtype, int32_t out_f32, void* stream);
+
+/* Adapter Linear(2h -> h) over concat(state, embeds) without materialising the concat
+ * (RMM:776: torch.cat([x, input_embeds], -1) then nn.Linear).  w is [N, K0 + K1]; x0 [M, K0] pairs
+ * with w[:, :K0] and x1 [M, K1] with w[:, K0:]. */
+int raven_adapter_gemm_concat(const void* x0, const void* x1, const void* w, void* y,
+                              int32_t M, int32_t N, int32_t K0, int32_t K1, int32_t dtype, void* stream);
+
+/* GatedMLP first half with the activation in the epilogue (RMM:507-508):
+ *   z = X fc^T, gate = T(z[:, :I]), up = T(z[:, I:]), out[M, I] = T(T(silu(gate)) * up). */
+int raven_gemm_swiglu(const void* x, const void* fc, void* out,
+                      int32_t M, int32_t I, int32_t K, int32_t dtype, void* stream);
+
+/* Split fused qkv rows, add q/k bias, rotate q and k, append k and v to the cache slot
+ * (RMM:463-479 and HuginnStaticCache.update's index_copy_, RMM:375-380).
+ *   qkv [M, 3h] of T; freqs [n_pos, hd/2, 2] float (cos, sin) -- rows picked by position;
+ *   q_out [M, h] of T receives the rotated queries. */
+int raven_qkv_bias_rope_cache_append(const void* qkv, const void* qk_bias, const float* freqs,
+                                     void* q_out, const raven_kv_cache* cache, int32_t slot,
+                                     int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
+                                     int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream);
+
+/* softmax(q K^T / sqrt(hd)) V over the cached positions of one slot, for each of the M = B*S rows
+ * (RMM:481-491).  Row m attends to positions 0 .. pos0 + (m % S) inclusive: for S == 1 this is the
+ * unmasked decode case, for S > 1 the lower-right-aligned causal case.  The new keys/values must
+ * already be in the cache.  q [M, h]; y [M, h] in the layout y.transpose(1,2).reshape(B,S,h) has. */
+size_t raven_decode_attention_workspace_bytes(int32_t M, int32_t n_heads, int32_t head_dim);
+int    raven_decode_attention(const void* q, void* y, const raven_kv_cache* cache, int32_t slot,
+                              int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
+                              int32_t n_heads, int32_t head_dim, int32_t dtype,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
+/* Token embedding times sqrt(h) (RMM:667-671): out[m] = T(wte[ids[m]] * scale); ids are int64. */
+int raven_embed(const void* wte, const int64_t* ids, void* out, int32_t M, int32_t dim,
+                int64_t vocab, float scale, int32_t dtype, void* stream);
+
+/* Greedy selection (RMM:1988-1989): out[m] = index of the first maximum of logits[m, :]. */
+int raven_argmax(const float* logits, int64_t* out, int32_t M, int64_t vocab, void* stream);
+
+/* *pos += delta, on the stream: advances the device-side position a replayed graph reads. */
+int raven_advance_pos(int32_t* pos_dev, int32_t delta, void* stream);
+
+/* One SandwichBlock (RMM:525-536) on M = B*S token rows: x_in -> x_out, both [M, h] (may alias).
+ * `slot` is the cache slot this block appends to and reads.  ln_f (nullable) applies one more
+ * RMSNorm to the block output (the ln_f after the last recurrence, RMM:762, and after the coda,
+ * RMM:701); in that case x_out receives the normed values. */
+size_t raven_block_workspace_bytes(const raven_dims* dims, int32_t M);
+int    raven_sandwich_block(const raven_dims* dims, const raven_block_weights* w, const void* ln_f,
+                            const void* x_in, void* x_out, const float* freqs,
+                            const raven_kv_cache* cache, int32_t slot,
+                            int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* One recurrence iteration (core_block_forward, RMM:764-781): adapter over (state, embeds), then
+ * n_blocks SandwichBlocks using cache slots first_slot .. first_slot + n_blocks - 1.
+ * state_in / embeds / state_out: [M, h]; state_out may alias state_in.  ln_f as above. */
+int raven_core_iteration(const raven_dims* dims, const void* adapter_w,
+                         const raven_block_weights* blocks, int32_t n_blocks, const void* ln_f,
+                         const void* state_in, const void* embeds, void* state_out,
+                         const float* freqs, const raven_kv_cache* cache, int32_t first_slot,
+                         int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RAVEN_HIP_H */

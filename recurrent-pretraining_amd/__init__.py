@@ -1,0 +1,22 @@
+"""MI355X-native recurrent-core decode path of the Huginn/Raven model.
+
+The directory name carries a hyphen, so the package is imported under the name
+`recurrent_pretraining_amd` through `__graft_entry__.import_package()` (or any importlib call that
+registers this directory under that name).
+"""
+
+from . import hip  # noqa: F401
+from .cache import HuginnDynamicCache, remap_step  # noqa: F401
+from .config import RavenConfig  # noqa: F401
+from .modeling import (  # noqa: F401
+    CausalLMOutputRecurrentLatents,
+    DecodeRunner,
+    GenerationSettings,
+    RavenForCausalLM,
+    precompute_freqs_cis,
+)
+
+__all__ = [
+    "hip", "HuginnDynamicCache", "remap_step", "RavenConfig", "RavenForCausalLM", "DecodeRunner",
+    "CausalLMOutputRecurrentLatents", "GenerationSettings", "precompute_freqs_cis",
+]

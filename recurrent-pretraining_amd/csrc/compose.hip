@@ -1,0 +1,135 @@
+// Composed entry points: one SandwichBlock and one recurrence iteration, as sequences of the
+// kernels in this library on one stream.  Follows SandwichBlock.forward and core_block_forward of
+// the reference (recpre/raven_modeling_minimal.py:525-536, 764-781):
+//   a  = proj(attention(norm_1(x)));  x2 = norm_2(a + x);  out = norm_4(mlp(norm_3(x2)) + x2)
+// The residual adds ride in the epilogue of the proj / mlp.proj GEMMs, norm_2 and norm_3 are one
+// launch, and inside an iteration norm_4 of one block and norm_1 of the next are one launch.
+
+#include "raven_common.h"
+
+namespace raven {
+
+struct BlockScratch {
+    char *n1, *qkv, *q, *ya, *x1, *x2, *n3, *g, *x3, *xa;
+    void* attn_ws;
+    size_t attn_ws_bytes;
+};
+
+static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
+    const size_t es = raven_host::elt_size(d->dtype);
+    const size_t row = raven_host::align_up((size_t)M * d->n_embd * es);
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        char* p = base ? base + off : nullptr;
+        off += raven_host::align_up(bytes);
+        return p;
+    };
+    BlockScratch s;
+    s.n1 = take(row);
+    s.qkv = take(3 * row);
+    s.q = take(row);
+    s.ya = take(row);
+    s.x1 = take(row);
+    s.x2 = take(row);
+    s.n3 = take(row);
+    s.g = take((size_t)M * d->intermediate * es);
+    s.x3 = take(row);
+    s.xa = take(row);
+    s.attn_ws_bytes = raven_decode_attention_workspace_bytes(M, d->n_heads, d->head_dim);
+    s.attn_ws = take(s.attn_ws_bytes);
+    if (out) *out = s;
+    return off;
+}
+
+static int check_dims(const char* who, const raven_dims* d) {
+    RAVEN_REQUIRE(d != nullptr, "%s: null dims", who);
+    RAVEN_REQUIRE(d->dtype == RAVEN_F32 || d->dtype == RAVEN_BF16, "%s: unknown dtype %d", who, d->dtype);
+    RAVEN_REQUIRE(d->n_embd > 0 && d->n_heads > 0 && d->head_dim > 0 && d->intermediate > 0, "%s: non-positive dimension", who);
+    RAVEN_REQUIRE(d->n_embd == d->n_heads * d->head_dim, "%s: n_embd %d != n_heads %d * head_dim %d", who, d->n_embd, d->n_heads, d->head_dim);
+    return 0;
+}
+
+static int check_block_weights(const char* who, const raven_block_weights* w) {
+    RAVEN_REQUIRE(w && w->norm_1 && w->norm_2 && w->norm_3 && w->norm_4 && w->wqkv && w->proj && w->fc && w->mlp_proj,
+                  "%s: null block weight", who);
+    return 0;
+}
+
+// One block.  n1_ready: scratch.n1 already holds norm_1(x_in).  tail_w / tail_out: a second norm
+// applied to the block output (next block's norm_1, or ln_f); y_out may be null when only the tail
+// result is wanted.
+static int run_block(const raven_dims* d, const raven_block_weights* w, const BlockScratch& s, bool n1_ready,
+                     const void* x_in, void* y_out, const void* tail_w, void* tail_out, const float* freqs,
+                     const raven_kv_cache* cache, int slot, int B, int S, int pos0, const int32_t* pos_dev, void* stream) {
+    const int M = B * S, h = d->n_embd, I = d->intermediate, dt = d->dtype;
+    int rc;
+    if (!n1_ready)
+        if ((rc = raven_rmsnorm_residual(x_in, nullptr, w->norm_1, s.n1, nullptr, nullptr, nullptr, M, h, d->eps, dt, stream))) return rc;
+    if ((rc = raven_gemm(s.n1, w->wqkv, nullptr, s.qkv, M, 3 * h, h, dt, 0, stream))) return rc;
+    if ((rc = raven_qkv_bias_rope_cache_append(s.qkv, w->qk_bias, freqs, s.q, cache, slot, B, S, pos0, pos_dev, d->n_heads,
+                                               d->head_dim, dt, stream))) return rc;
+    if ((rc = raven_decode_attention(s.q, s.ya, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, s.attn_ws,
+                                     s.attn_ws_bytes, stream))) return rc;
+    if ((rc = raven_gemm(s.ya, w->proj, x_in, s.x1, M, h, h, dt, 0, stream))) return rc;
+    if ((rc = raven_rmsnorm_residual(s.x1, nullptr, w->norm_2, s.x2, nullptr, w->norm_3, s.n3, M, h, d->eps, dt, stream))) return rc;
+    if ((rc = raven_gemm_swiglu(s.n3, w->fc, s.g, M, I, h, dt, stream))) return rc;
+    if ((rc = raven_gemm(s.g, w->mlp_proj, s.x2, s.x3, M, h, I, dt, 0, stream))) return rc;
+    return raven_rmsnorm_residual(s.x3, nullptr, w->norm_4, y_out, nullptr, tail_w, tail_out, M, h, d->eps, dt, stream);
+}
+
+}  // namespace raven
+
+extern "C" size_t raven_block_workspace_bytes(const raven_dims* dims, int32_t M) {
+    if (!dims || M <= 0) return 0;
+    return raven::carve(dims, M, nullptr, nullptr);
+}
+
+extern "C" int raven_sandwich_block(const raven_dims* dims, const raven_block_weights* w, const void* ln_f, const void* x_in,
+                                    void* x_out, const float* freqs, const raven_kv_cache* cache, int32_t slot, int32_t B,
+                                    int32_t S, int32_t pos0, const int32_t* pos_dev, void* workspace, size_t workspace_bytes,
+                                    void* stream) {
+    using namespace raven;
+    if (int rc = check_dims("sandwich_block", dims)) return rc;
+    if (int rc = check_block_weights("sandwich_block", w)) return rc;
+    RAVEN_REQUIRE(x_in && x_out && freqs, "sandwich_block: null pointer");
+    RAVEN_REQUIRE(B > 0 && S > 0, "sandwich_block: bad B=%d S=%d", B, S);
+    const size_t need = carve(dims, B * S, nullptr, nullptr);
+    RAVEN_REQUIRE(workspace && workspace_bytes >= need, "sandwich_block: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    RAVEN_REQUIRE(((uintptr_t)workspace & 255) == 0, "sandwich_block: workspace must be 256-byte aligned");
+    BlockScratch s;
+    carve(dims, B * S, static_cast<char*>(workspace), &s);
+    if (ln_f) return run_block(dims, w, s, false, x_in, nullptr, ln_f, x_out, freqs, cache, slot, B, S, pos0, pos_dev, stream);
+    return run_block(dims, w, s, false, x_in, x_out, nullptr, nullptr, freqs, cache, slot, B, S, pos0, pos_dev, stream);
+}
+
+extern "C" int raven_core_iteration(const raven_dims* dims, const void* adapter_w, const raven_block_weights* blocks,
+                                    int32_t n_blocks, const void* ln_f, const void* state_in, const void* embeds,
+                                    void* state_out, const float* freqs, const raven_kv_cache* cache, int32_t first_slot,
+                                    int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+    using namespace raven;
+    if (int rc = check_dims("core_iteration", dims)) return rc;
+    RAVEN_REQUIRE(adapter_w && state_in && embeds && state_out && freqs, "core_iteration: null pointer");
+    RAVEN_REQUIRE(n_blocks >= 1 && blocks, "core_iteration: needs at least one block");
+    RAVEN_REQUIRE(B > 0 && S > 0, "core_iteration: bad B=%d S=%d", B, S);
+    for (int j = 0; j < n_blocks; ++j)
+        if (int rc = check_block_weights("core_iteration", &blocks[j])) return rc;
+    const int M = B * S, h = dims->n_embd;
+    const size_t need = carve(dims, M, nullptr, nullptr);
+    RAVEN_REQUIRE(workspace && workspace_bytes >= need, "core_iteration: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    RAVEN_REQUIRE(((uintptr_t)workspace & 255) == 0, "core_iteration: workspace must be 256-byte aligned");
+    BlockScratch s;
+    carve(dims, M, static_cast<char*>(workspace), &s);
+
+    int rc;
+    if ((rc = raven_adapter_gemm_concat(state_in, embeds, adapter_w, s.xa, M, h, h, h, dims->dtype, stream))) return rc;
+    for (int j = 0; j < n_blocks; ++j) {
+        const bool last = j == n_blocks - 1;
+        void* y_out = last ? (ln_f ? nullptr : state_out) : s.xa;
+        const void* tail_w = last ? ln_f : blocks[j + 1].norm_1;
+        void* tail_out = last ? (ln_f ? state_out : nullptr) : s.n1;
+        if ((rc = run_block(dims, &blocks[j], s, j > 0, s.xa, y_out, tail_w, tail_out, freqs, cache, first_slot + j, B, S, pos0,
+                            pos_dev, stream))) return rc;
+    }
+    return 0;
+}

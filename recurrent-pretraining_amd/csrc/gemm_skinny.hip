@@ -1,0 +1,403 @@
+// Skinny GEMMs of the decode path: Y[M,N] = X[M,K] W[N,K]^T with M = a handful of token rows and
+// W a weight matrix that is streamed from HBM exactly once per call (per 32 rows of X).
+//
+// Two kernels:
+//   gemv_kernel  (any T, up to 8 rows of X per pass)  -- X lives in LDS, every wave owns whole rows
+//                of W, reads them with 16-byte lane-contiguous loads and accumulates with
+//                v_dot2_f32_bf16 / fp32 FMA; a DPP wave reduction finishes each row.
+//   mfma_kernel  (bf16, up to 32 rows of X per pass)   -- 16-row tiles of W are the A operand of
+//                v_mfma_f32_16x16x32_bf16, X is the B operand; the four waves of a workgroup split
+//                K and reduce through LDS.
+// Epilogues (all round the fp32 accumulator to T first, as an nn.Linear output would be stored):
+//   plain (+ residual add in T, + optional float store)   RMM:493, 509, 711, 534-535
+//   SwiGLU: T(T(silu(gate)) * up), gate row j, up row j+I  RMM:507-508
+// The adapter's concat (RMM:776) is folded in by giving X as two pointers that cover K0 and K1.
+
+#include "raven_common.h"
+
+namespace raven {
+
+enum { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
+
+struct GemmArgs {
+    const void* w;         // [N_total, K]
+    const void* x0;        // [M, k0]
+    const void* x1;        // [M, k1] or null
+    const void* residual;  // [M, N] or null
+    void* y;               // [M, N] (T, or float when out_f32)
+    int M, N, K, k0, k1;   // N = number of output columns (I for SwiGLU)
+    int out_f32;
+    int units_per_wave;    // gemv: row pairs per wave
+};
+
+template <typename T>
+__device__ __forceinline__ void store_out(const GemmArgs& a, int m, int n, float acc) {
+    float r = round_to<T>(acc);
+    if (a.residual) r = round_to<T>(r + to_f32(static_cast<const T*>(a.residual)[(int64_t)m * a.N + n]));
+    if (a.out_f32)
+        static_cast<float*>(a.y)[(int64_t)m * a.N + n] = r;
+    else
+        static_cast<T*>(a.y)[(int64_t)m * a.N + n] = from_f32<T>(r);
+}
+
+template <typename T>
+__device__ __forceinline__ float swiglu(float gate_acc, float up_acc) {
+    const float g = round_to<T>(gate_acc), u = round_to<T>(up_acc);
+    return round_to<T>(round_to<T>(silu_f32(g)) * u);
+}
+
+// ------------------------------------------------------------------------------------------------
+// gemv_kernel: 256 threads; dynamic LDS holds X as [MB][K] of T.
+// ------------------------------------------------------------------------------------------------
+template <typename T, int MB, int EPI>
+__global__ __launch_bounds__(256) void gemv_kernel(GemmArgs a) {
+    constexpr int E = Chunk<T>::N;
+    constexpr int U = 4;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* xs = reinterpret_cast<T*>(smem_raw);
+
+    const int K = a.K, n_chunks = K / E, c0 = a.k0 / E;
+    // stage X: row m of LDS = concat(x0[m], x1[m]); rows >= M are zero
+    for (int i = threadIdx.x; i < MB * n_chunks; i += 256) {
+        const int m = i / n_chunks, c = i - m * n_chunks;
+        Chunk<T> v = zero_chunk<T>();
+        if (m < a.M) {
+            v = (c < c0) ? load_chunk(static_cast<const T*>(a.x0) + (int64_t)m * a.k0 + c * E)
+                         : load_chunk(static_cast<const T*>(a.x1) + (int64_t)m * a.k1 + (c - c0) * E);
+        }
+        store_chunk(xs + (int64_t)m * K + c * E, v);
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const int gwave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int n_units = (EPI == EPI_SWIGLU) ? a.N : (a.N + 1) / 2;
+    const T* W = static_cast<const T*>(a.w);
+
+    for (int u = 0; u < a.units_per_wave; ++u) {
+        const int unit = gwave * a.units_per_wave + u;
+        if (unit >= n_units) break;
+        int r0, r1;
+        bool r1_ok = true;
+        if (EPI == EPI_SWIGLU) {
+            r0 = unit;
+            r1 = unit + a.N;
+        } else {
+            r0 = 2 * unit;
+            r1 = r0 + 1;
+            if (r1 >= a.N) { r1 = r0; r1_ok = false; }
+        }
+        const T* w0 = W + (int64_t)r0 * K;
+        const T* w1 = W + (int64_t)r1 * K;
+        float acc0[MB], acc1[MB];
+#pragma unroll
+        for (int m = 0; m < MB; ++m) acc0[m] = acc1[m] = 0.f;
+
+        for (int c = lane; c < n_chunks; c += 64 * U) {
+            Chunk<T> a0[U], a1[U];
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                const int cc = c + 64 * j;
+                if (cc < n_chunks) {
+                    a0[j] = load_chunk(w0 + cc * E);
+                    a1[j] = load_chunk(w1 + cc * E);
+                } else {
+                    a0[j] = zero_chunk<T>();
+                    a1[j] = zero_chunk<T>();
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                const int cc = min(c + 64 * j, n_chunks - 1);
+#pragma unroll
+                for (int m = 0; m < MB; ++m) {
+                    const Chunk<T> xv = load_chunk(xs + (int64_t)m * K + cc * E);
+                    acc0[m] = dot_chunk(a0[j], xv, acc0[m]);
+                    acc1[m] = dot_chunk(a1[j], xv, acc1[m]);
+                }
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            acc0[m] = wave_sum(acc0[m]);
+            acc1[m] = wave_sum(acc1[m]);
+        }
+        if (lane == 0) {
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                if (m < a.M) {
+                    if (EPI == EPI_SWIGLU) {
+                        static_cast<T*>(a.y)[(int64_t)m * a.N + unit] = from_f32<T>(swiglu<T>(acc0[m], acc1[m]));
+                    } else {
+                        store_out<T>(a, m, r0, acc0[m]);
+                        if (r1_ok) store_out<T>(a, m, r1, acc1[m]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// mfma_kernel: bf16, 256 threads = 4 waves that split K; MT = ceil(M/16) batch tiles; NT weight
+// tiles of 16 rows per workgroup.  D = A * B with A = W tile [16 n x 32 k], B = X^T [32 k x 16 m]:
+// lane l supplies A[n = l%16][k = 8*(l/16) ..+8] and B[k = 8*(l/16) ..+8][m = l%16] and receives
+// D[n = 4*(l/16) + v][m = l%16], v = 0..3.
+// ------------------------------------------------------------------------------------------------
+template <int MT, int NT, int EPI>
+__global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
+    __shared__ float red[3][NT * MT][64][4];  // partial accumulators of waves 1..3
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int ln = lane & 15, kq = lane >> 4;
+    const int K = a.K;
+    const int n_steps = K / 32;
+    const int s_begin = (int)((int64_t)n_steps * wave / 4), s_end = (int)((int64_t)n_steps * (wave + 1) / 4);
+    const int n_tiles = (EPI == EPI_SWIGLU) ? a.N / 16 : (a.N / 16 + NT - 1) / NT;  // units
+    const int unit = blockIdx.x;
+    if (unit >= n_tiles) return;
+
+    const bf16* W = static_cast<const bf16*>(a.w);
+    const bf16* wrow[NT];
+    bool tile_ok[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        int row;
+        if (EPI == EPI_SWIGLU) {
+            row = unit * 16 + ln + t * a.N;  // t = 0 gate tile, t = 1 up tile
+            tile_ok[t] = true;
+        } else {
+            const int tile = unit * NT + t;
+            tile_ok[t] = tile * 16 < a.N;
+            row = (tile_ok[t] ? tile : unit * NT) * 16 + ln;
+        }
+        wrow[t] = W + (int64_t)row * K + kq * 8;
+    }
+    // X row pointers: batch row m = mt*16 + ln, clamped (columns of D past M are never stored)
+    const bf16* xrow[MT];
+    int xk0[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = min(mt * 16 + ln, a.M - 1);
+        xrow[mt] = static_cast<const bf16*>(a.x0) + (int64_t)m * a.k0 + kq * 8;
+        xk0[mt] = m;
+    }
+    const bf16* x1 = static_cast<const bf16*>(a.x1);
+
+    f32x4 acc[NT][MT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    constexpr int U = 4;
+    for (int s = s_begin; s < s_end; s += U) {
+        bf16x8 av[U][NT], bv[U][MT];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int k = min(s + j, s_end - 1) * 32;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) av[j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + k);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const bf16* p = (k < a.k0) ? xrow[mt] + k : x1 + (int64_t)xk0[mt] * a.k1 + kq * 8 + (k - a.k0);
+                bv[j][mt] = *reinterpret_cast<const bf16x8*>(p);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            if (s + j < s_end) {
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[j][t], bv[j][mt], acc[t][mt], 0, 0, 0);
+            }
+        }
+    }
+
+    // cross-wave reduction over the K split
+    if (wave > 0) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) red[wave - 1][t * MT + mt][lane][v] = acc[t][mt][v];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                acc[t][mt][v] += red[0][t * MT + mt][lane][v] + red[1][t * MT + mt][lane][v] + red[2][t * MT + mt][lane][v];
+
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + ln;
+        if (m >= a.M) continue;
+        if (EPI == EPI_SWIGLU) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int n = unit * 16 + kq * 4 + v;
+                static_cast<bf16*>(a.y)[(int64_t)m * a.N + n] = from_f32<bf16>(swiglu<bf16>(acc[0][mt][v], acc[NT - 1][mt][v]));
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                if (!tile_ok[t]) continue;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) store_out<bf16>(a, m, (unit * NT + t) * 16 + kq * 4 + v, acc[t][mt][v]);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host dispatch
+// ------------------------------------------------------------------------------------------------
+static int n_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t p;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;
+        if (cus <= 0) cus = 256;
+    }
+    return cus;
+}
+
+template <typename T, int MB, int EPI>
+static int launch_gemv(GemmArgs a, hipStream_t s) {
+    const size_t lds = (size_t)MB * a.K * sizeof(T);
+    RAVEN_REQUIRE(lds <= 160 * 1024, "gemm: %d rows x K=%d does not fit the 160 KB LDS", MB, a.K);
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemv_kernel<T, MB, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) {
+            raven_host::set_error("gemm: hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+            return (int)e;
+        }
+        attr_set = true;
+    }
+    const int n_units = (EPI == EPI_SWIGLU) ? a.N : (a.N + 1) / 2;
+    // as few units per wave as keeps every workgroup resident at once (about 4 per CU)
+    const int max_wgs = n_cus() * 4;
+    int upw = 1;
+    while ((n_units + 4 * upw - 1) / (4 * upw) > max_wgs) ++upw;
+    a.units_per_wave = upw;
+    const int wgs = (n_units + 4 * upw - 1) / (4 * upw);
+    gemv_kernel<T, MB, EPI><<<dim3(wgs), dim3(256), lds, s>>>(a);
+    return raven_host::check_launch("gemv");
+}
+
+template <typename T, int EPI>
+static int dispatch_gemv(GemmArgs a, hipStream_t s) {
+    if (a.M <= 1) return launch_gemv<T, 1, EPI>(a, s);
+    if (a.M <= 2) return launch_gemv<T, 2, EPI>(a, s);
+    if (a.M <= 4) return launch_gemv<T, 4, EPI>(a, s);
+    return launch_gemv<T, 8, EPI>(a, s);
+}
+
+template <int EPI>
+static int dispatch_mfma(GemmArgs a, hipStream_t s) {
+    const int n_tiles16 = a.N / 16;
+    if (EPI == EPI_SWIGLU) {
+        if (a.M <= 16)
+            mfma_kernel<1, 2, EPI><<<dim3(n_tiles16), dim3(256), 0, s>>>(a);
+        else
+            mfma_kernel<2, 2, EPI><<<dim3(n_tiles16), dim3(256), 0, s>>>(a);
+    } else {
+        // two tiles per workgroup once that still leaves every CU several workgroups
+        const bool two = n_tiles16 / 2 >= 2 * n_cus();
+        const int units = two ? (n_tiles16 + 1) / 2 : n_tiles16;
+        if (a.M <= 16) {
+            if (two) mfma_kernel<1, 2, EPI><<<dim3(units), dim3(256), 0, s>>>(a);
+            else     mfma_kernel<1, 1, EPI><<<dim3(units), dim3(256), 0, s>>>(a);
+        } else {
+            if (two) mfma_kernel<2, 2, EPI><<<dim3(units), dim3(256), 0, s>>>(a);
+            else     mfma_kernel<2, 1, EPI><<<dim3(units), dim3(256), 0, s>>>(a);
+        }
+    }
+    return raven_host::check_launch("mfma gemm");
+}
+
+// Runs one GEMM over all M rows, in passes of at most 32 (MFMA) or 8 / 4 (vector) rows.
+template <int EPI>
+static int run_gemm(GemmArgs a, int dtype, hipStream_t s) {
+    const size_t es = raven_host::elt_size(dtype);
+    const bool mfma_ok = dtype == RAVEN_BF16 && a.K % 32 == 0 && a.k0 % 32 == 0 && a.N % 16 == 0;
+    const int M = a.M;
+    const size_t out_es = a.out_f32 ? 4 : es;
+    for (int m0 = 0; m0 < M;) {
+        const int left = M - m0;
+        int pass;
+        const bool use_mfma = mfma_ok && left > 4;
+        if (use_mfma) pass = left < 32 ? left : 32;
+        else if (dtype == RAVEN_BF16) pass = left < 4 ? left : 4;
+        else pass = left < 8 ? left : 8;
+        GemmArgs p = a;
+        p.M = pass;
+        p.x0 = static_cast<const char*>(a.x0) + (size_t)m0 * a.k0 * es;
+        if (a.x1) p.x1 = static_cast<const char*>(a.x1) + (size_t)m0 * a.k1 * es;
+        if (a.residual) p.residual = static_cast<const char*>(a.residual) + (size_t)m0 * a.N * es;
+        p.y = static_cast<char*>(a.y) + (size_t)m0 * a.N * out_es;
+        int rc;
+        if (use_mfma) rc = dispatch_mfma<EPI>(p, s);
+        else if (dtype == RAVEN_BF16) rc = dispatch_gemv<bf16, EPI>(p, s);
+        else rc = dispatch_gemv<float, EPI>(p, s);
+        if (rc != 0) return rc;
+        m0 += pass;
+    }
+    return 0;
+}
+
+static int check_common(const char* who, int M, int N, int K, int dtype) {
+    RAVEN_REQUIRE(dtype == RAVEN_F32 || dtype == RAVEN_BF16, "%s: unknown dtype %d", who, dtype);
+    RAVEN_REQUIRE(M >= 0 && N > 0 && K > 0, "%s: bad shape M=%d N=%d K=%d", who, M, N, K);
+    const int elts = 16 / (int)raven_host::elt_size(dtype);
+    RAVEN_REQUIRE(K % elts == 0, "%s: K=%d must be a multiple of %d", who, K, elts);
+    return 0;
+}
+
+}  // namespace raven
+
+extern "C" int raven_gemm(const void* x, const void* w, const void* residual, void* y, int32_t M, int32_t N, int32_t K,
+                          int32_t dtype, int32_t out_f32, void* stream) {
+    using namespace raven;
+    if (int rc = check_common("gemm", M, N, K, dtype)) return rc;
+    RAVEN_REQUIRE(x && w && y, "gemm: null pointer");
+    if (M == 0) return 0;
+    GemmArgs a{};
+    a.w = w; a.x0 = x; a.x1 = nullptr; a.residual = residual; a.y = y;
+    a.M = M; a.N = N; a.K = K; a.k0 = K; a.k1 = 0; a.out_f32 = out_f32;
+    return run_gemm<EPI_PLAIN>(a, dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int raven_adapter_gemm_concat(const void* x0, const void* x1, const void* w, void* y, int32_t M, int32_t N,
+                                         int32_t K0, int32_t K1, int32_t dtype, void* stream) {
+    using namespace raven;
+    if (int rc = check_common("adapter", M, N, K0 + K1, dtype)) return rc;
+    RAVEN_REQUIRE(x0 && x1 && w && y, "adapter: null pointer");
+    const int elts = 16 / (int)raven_host::elt_size(dtype);
+    RAVEN_REQUIRE(K0 > 0 && K1 > 0 && K0 % elts == 0 && K1 % elts == 0, "adapter: K0=%d, K1=%d must be positive multiples of %d", K0, K1, elts);
+    if (M == 0) return 0;
+    GemmArgs a{};
+    a.w = w; a.x0 = x0; a.x1 = x1; a.residual = nullptr; a.y = y;
+    a.M = M; a.N = N; a.K = K0 + K1; a.k0 = K0; a.k1 = K1; a.out_f32 = 0;
+    return run_gemm<EPI_PLAIN>(a, dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int raven_gemm_swiglu(const void* x, const void* fc, void* out, int32_t M, int32_t I, int32_t K, int32_t dtype,
+                                 void* stream) {
+    using namespace raven;
+    if (int rc = check_common("gemm_swiglu", M, I, K, dtype)) return rc;
+    RAVEN_REQUIRE(x && fc && out, "gemm_swiglu: null pointer");
+    if (M == 0) return 0;
+    GemmArgs a{};
+    a.w = fc; a.x0 = x; a.x1 = nullptr; a.residual = nullptr; a.y = out;
+    a.M = M; a.N = I; a.K = K; a.k0 = K; a.k1 = 0; a.out_f32 = 0;
+    return run_gemm<EPI_SWIGLU>(a, dtype, static_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,115 @@
+// Fused (residual add +) RMSNorm (+ second RMSNorm) for [rows, dim] activations.
+// One 256-thread workgroup per row; the row stays in registers between the add, the two
+// reductions and the stores, so HBM sees each element once on the way in and once per output.
+// Arithmetic follows RMSNorm.forward of the reference (recpre/raven_modeling_minimal.py:137-142):
+// normalise in fp32, round to T, then multiply by the weight in T (a second rounding).
+
+#include "raven_common.h"
+
+namespace raven {
+
+constexpr int kNormThreads = 256;
+constexpr int kNormMaxChunks = 4;  // per thread: dim <= 256 * 4 * (16 / sizeof(T)) elements
+
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+    v = wave_sum(v);
+    const int wave = threadIdx.x >> 6;
+    __syncthreads();  // protects `red` against the previous use
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+}
+
+template <typename T>
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
+    const T* __restrict__ x, const T* __restrict__ residual, const T* __restrict__ weight, T* __restrict__ y,
+    T* __restrict__ sum_out, const T* __restrict__ weight2, T* __restrict__ y2, int dim, float eps) {
+    constexpr int E = Chunk<T>::N;
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;
+    const int n_chunks = dim / E;
+    const T* xr = x + row * dim;
+    const T* rr = residual ? residual + row * dim : nullptr;
+
+    float v[kNormMaxChunks][E];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kNormMaxChunks; ++i) {
+        const int c = threadIdx.x + i * kNormThreads;
+        if (c < n_chunks) {
+            Chunk<T> cx = load_chunk(xr + c * E);
+            if (rr) {
+                Chunk<T> cr = load_chunk(rr + c * E);
+#pragma unroll
+                for (int e = 0; e < E; ++e) cx.v[e] = from_f32<T>(to_f32(cx.v[e]) + to_f32(cr.v[e]));
+                if (sum_out) store_chunk(sum_out + row * dim + c * E, cx);
+            }
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                v[i][e] = to_f32(cx.v[e]);
+                ss = __builtin_fmaf(v[i][e], v[i][e], ss);
+            }
+        }
+    }
+    float inv = rsqrtf(block_sum_256(ss, red) / (float)dim + eps);
+
+    float ss2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < kNormMaxChunks; ++i) {
+        const int c = threadIdx.x + i * kNormThreads;
+        if (c < n_chunks) {
+            Chunk<T> cw = load_chunk(weight + c * E);
+            Chunk<T> co;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                co.v[e] = from_f32<T>(round_to<T>(v[i][e] * inv) * to_f32(cw.v[e]));
+                v[i][e] = to_f32(co.v[e]);
+                ss2 = __builtin_fmaf(v[i][e], v[i][e], ss2);
+            }
+            if (y) store_chunk(y + row * dim + c * E, co);
+        }
+    }
+    if (weight2 == nullptr) return;
+
+    inv = rsqrtf(block_sum_256(ss2, red) / (float)dim + eps);
+#pragma unroll
+    for (int i = 0; i < kNormMaxChunks; ++i) {
+        const int c = threadIdx.x + i * kNormThreads;
+        if (c < n_chunks) {
+            Chunk<T> cw = load_chunk(weight2 + c * E);
+            Chunk<T> co;
+#pragma unroll
+            for (int e = 0; e < E; ++e) co.v[e] = from_f32<T>(round_to<T>(v[i][e] * inv) * to_f32(cw.v[e]));
+            store_chunk(y2 + row * dim + c * E, co);
+        }
+    }
+}
+
+}  // namespace raven
+
+extern "C" int raven_rmsnorm_residual(const void* x, const void* residual, const void* weight, void* y,
+                                      void* sum_out, const void* weight2, void* y2, int64_t rows, int32_t dim,
+                                      float eps, int32_t dtype, void* stream) {
+    using namespace raven;
+    RAVEN_REQUIRE(dtype == RAVEN_F32 || dtype == RAVEN_BF16, "rmsnorm: unknown dtype %d", dtype);
+    RAVEN_REQUIRE(x && weight && (y || y2), "rmsnorm: null x / weight / output");
+    RAVEN_REQUIRE((weight2 == nullptr) == (y2 == nullptr), "rmsnorm: weight2 and y2 must be given together");
+    RAVEN_REQUIRE(sum_out == nullptr || residual != nullptr, "rmsnorm: sum_out needs a residual");
+    const int elts = 16 / (int)raven_host::elt_size(dtype);
+    RAVEN_REQUIRE(dim > 0 && dim % elts == 0, "rmsnorm: dim %d is not a multiple of %d", dim, elts);
+    RAVEN_REQUIRE(dim / elts <= kNormThreads * kNormMaxChunks, "rmsnorm: dim %d too large (max %d)", dim,
+                  kNormThreads * kNormMaxChunks * elts);
+    RAVEN_REQUIRE(rows >= 0 && rows < (1ll << 31), "rmsnorm: bad row count %lld", (long long)rows);
+    if (rows == 0) return 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == RAVEN_BF16) {
+        rmsnorm_kernel<bf16><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(
+            (const bf16*)x, (const bf16*)residual, (const bf16*)weight, (bf16*)y, (bf16*)sum_out, (const bf16*)weight2,
+            (bf16*)y2, dim, eps);
+    } else {
+        rmsnorm_kernel<float><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(
+            (const float*)x, (const float*)residual, (const float*)weight, (float*)y, (float*)sum_out,
+            (const float*)weight2, (float*)y2, dim, eps);
+    }
+    return raven_host::check_launch("rmsnorm");
+}

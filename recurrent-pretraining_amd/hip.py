@@ -1,0 +1,261 @@
+"""ctypes binding of libraven_hip.so (the C ABI declared in include/raven_hip.h).
+
+PyTorch is used only for device memory and streams: tensors cross the boundary as raw device
+pointers plus sizes, and every launch goes to torch's current HIP stream.  There is no fallback:
+if the library is missing or a call fails, an exception is raised.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional
+
+import torch
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libraven_hip.so")
+
+F32, BF16 = 0, 1
+_DTYPES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class RavenHipError(RuntimeError):
+    pass
+
+
+class Dims(C.Structure):
+    _fields_ = [("n_embd", C.c_int32), ("n_heads", C.c_int32), ("head_dim", C.c_int32),
+                ("intermediate", C.c_int32), ("eps", C.c_float), ("dtype", C.c_int32)]
+
+
+class BlockWeights(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in
+                ("norm_1", "norm_2", "norm_3", "norm_4", "wqkv", "qk_bias", "proj", "fc", "mlp_proj")]
+
+
+class KVCache(C.Structure):
+    _fields_ = [("k", C.c_void_p), ("v", C.c_void_p), ("n_slots", C.c_int32), ("batch", C.c_int32),
+                ("t_max", C.c_int32)]
+
+
+# name -> (restype, argtypes); kept in one table so the export test can walk it
+_VP, _I32, _I64, _F, _SZ = C.c_void_p, C.c_int32, C.c_int64, C.c_float, C.c_size_t
+SIGNATURES = {
+    "raven_version": (C.c_int, []),
+    "raven_arch": (C.c_char_p, []),
+    "raven_last_error": (C.c_char_p, []),
+    "raven_rmsnorm_residual": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I32, _F, _I32, _VP]),
+    "raven_gemm": (C.c_int, [_VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _VP]),
+    "raven_adapter_gemm_concat": (C.c_int, [_VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _VP]),
+    "raven_gemm_swiglu": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I32, _I32, _VP]),
+    "raven_qkv_bias_rope_cache_append": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32,
+                                                   _VP, _I32, _I32, _I32, _VP]),
+    "raven_decode_attention_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
+    "raven_decode_attention": (C.c_int, [_VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _I32, _I32, _I32,
+                                         _VP, _SZ, _VP]),
+    "raven_embed": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I64, _F, _I32, _VP]),
+    "raven_argmax": (C.c_int, [_VP, _VP, _I32, _I64, _VP]),
+    "raven_advance_pos": (C.c_int, [_VP, _I32, _VP]),
+    "raven_block_workspace_bytes": (_SZ, [C.POINTER(Dims), _I32]),
+    "raven_sandwich_block": (C.c_int, [C.POINTER(Dims), C.POINTER(BlockWeights), _VP, _VP, _VP, _VP,
+                                       C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _VP, _SZ, _VP]),
+    "raven_core_iteration": (C.c_int, [C.POINTER(Dims), _VP, C.POINTER(BlockWeights), _I32, _VP, _VP, _VP, _VP, _VP,
+                                       C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _VP, _SZ, _VP]),
+}
+
+_lib: Optional[C.CDLL] = None
+
+
+def load() -> C.CDLL:
+    """Loads the library (once).  Raises when it has not been built: there is no other code path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RavenHipError(
+                f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as e; e.build()'` "
+                "(hipcc, gfx950).  This package has no CPU or PyTorch fallback.")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().raven_last_error().decode("utf-8", "replace")
+        raise RavenHipError(f"{what} failed (code {rc}): {msg}")
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DTYPES[dt]
+    except KeyError:
+        raise RavenHipError(f"unsupported dtype {dt}: the kernels take float32 and bfloat16") from None
+
+
+def _ptr(t: Optional[torch.Tensor], name: str, dtype: Optional[torch.dtype] = None) -> Optional[int]:
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise RavenHipError(f"{name} must live on the GPU (got {t.device}); there is no CPU path")
+    if not t.is_contiguous():
+        raise RavenHipError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise RavenHipError(f"{name} has dtype {t.dtype}, expected {dtype}")
+    return t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def make_dims(n_embd: int, n_heads: int, intermediate: int, eps: float, dtype: torch.dtype) -> Dims:
+    return Dims(n_embd, n_heads, n_embd // n_heads, intermediate, eps, dtype_code(dtype))
+
+
+def make_cache(k: torch.Tensor, v: torch.Tensor) -> KVCache:
+    """k, v: [n_slots, batch, nh, t_max, hd], contiguous, on the GPU."""
+    if k.shape != v.shape or k.dim() != 5:
+        raise RavenHipError("cache tensors must be [n_slots, batch, nh, t_max, hd] and of equal shape")
+    return KVCache(_ptr(k, "cache.k"), _ptr(v, "cache.v", k.dtype), k.shape[0], k.shape[1], k.shape[3])
+
+
+def make_block_weights(norm_1, norm_2, norm_3, norm_4, wqkv, qk_bias, proj, fc, mlp_proj) -> BlockWeights:
+    dt = wqkv.dtype
+    return BlockWeights(_ptr(norm_1, "norm_1", dt), _ptr(norm_2, "norm_2", dt), _ptr(norm_3, "norm_3", dt),
+                        _ptr(norm_4, "norm_4", dt), _ptr(wqkv, "wqkv", dt), _ptr(qk_bias, "qk_bias", dt),
+                        _ptr(proj, "proj", dt), _ptr(fc, "fc", dt), _ptr(mlp_proj, "mlp_proj", dt))
+
+
+# ---------------------------------------------------------------------------------------------
+# per-kernel wrappers (used by the tests and by the host model)
+# ---------------------------------------------------------------------------------------------
+def rmsnorm_residual(x, weight, eps, residual=None, weight2=None, want_sum=False, want_y=True):
+    """Returns (y, sum, y2); entries not asked for are None.  x: [..., dim]."""
+    dt = x.dtype
+    dim = x.shape[-1]
+    rows = x.numel() // dim
+    y = torch.empty_like(x) if want_y else None
+    s = torch.empty_like(x) if (want_sum and residual is not None) else None
+    y2 = torch.empty_like(x) if weight2 is not None else None
+    rc = load().raven_rmsnorm_residual(_ptr(x, "x"), _ptr(residual, "residual", dt), _ptr(weight, "weight", dt),
+                                       _ptr(y, "y"), _ptr(s, "sum"), _ptr(weight2, "weight2", dt), _ptr(y2, "y2"),
+                                       rows, dim, eps, dtype_code(dt), _stream())
+    _check(rc, "raven_rmsnorm_residual")
+    return y, s, y2
+
+
+def gemm(x, w, residual=None, out_f32=False):
+    """x [M, K], w [N, K] -> [M, N]."""
+    dt = x.dtype
+    M, K = x.shape
+    N = w.shape[0]
+    assert w.shape[1] == K
+    y = torch.empty(M, N, device=x.device, dtype=torch.float32 if out_f32 else dt)
+    rc = load().raven_gemm(_ptr(x, "x"), _ptr(w, "w", dt), _ptr(residual, "residual", dt), _ptr(y, "y"),
+                           M, N, K, dtype_code(dt), int(out_f32), _stream())
+    _check(rc, "raven_gemm")
+    return y
+
+
+def adapter_gemm_concat(x0, x1, w):
+    dt = x0.dtype
+    M, K0 = x0.shape
+    K1 = x1.shape[1]
+    N = w.shape[0]
+    assert w.shape[1] == K0 + K1 and x1.shape[0] == M
+    y = torch.empty(M, N, device=x0.device, dtype=dt)
+    rc = load().raven_adapter_gemm_concat(_ptr(x0, "x0"), _ptr(x1, "x1", dt), _ptr(w, "w", dt), _ptr(y, "y"),
+                                          M, N, K0, K1, dtype_code(dt), _stream())
+    _check(rc, "raven_adapter_gemm_concat")
+    return y
+
+
+def gemm_swiglu(x, fc):
+    dt = x.dtype
+    M, K = x.shape
+    inter = fc.shape[0] // 2
+    assert fc.shape[1] == K
+    y = torch.empty(M, inter, device=x.device, dtype=dt)
+    rc = load().raven_gemm_swiglu(_ptr(x, "x"), _ptr(fc, "fc", dt), _ptr(y, "out"), M, inter, K, dtype_code(dt), _stream())
+    _check(rc, "raven_gemm_swiglu")
+    return y
+
+
+def qkv_bias_rope_cache_append(qkv, qk_bias, freqs, cache: KVCache, slot, B, S, pos0, n_heads, head_dim, pos_dev=None):
+    dt = qkv.dtype
+    q = torch.empty(B * S, n_heads * head_dim, device=qkv.device, dtype=dt)
+    rc = load().raven_qkv_bias_rope_cache_append(
+        _ptr(qkv, "qkv"), _ptr(qk_bias, "qk_bias", dt), _ptr(freqs, "freqs", torch.float32), _ptr(q, "q"),
+        C.byref(cache), slot, B, S, pos0, _ptr(pos_dev, "pos_dev", torch.int32), n_heads, head_dim, dtype_code(dt), _stream())
+    _check(rc, "raven_qkv_bias_rope_cache_append")
+    return q
+
+
+def attention_workspace(M, n_heads, head_dim, device) -> torch.Tensor:
+    n = load().raven_decode_attention_workspace_bytes(M, n_heads, head_dim)
+    return torch.zeros(max(n, 256), dtype=torch.uint8, device=device)
+
+
+def decode_attention(q, cache: KVCache, slot, B, S, pos0, n_heads, head_dim, workspace, pos_dev=None):
+    y = torch.empty_like(q)
+    rc = load().raven_decode_attention(
+        _ptr(q, "q"), _ptr(y, "y"), C.byref(cache), slot, B, S, pos0, _ptr(pos_dev, "pos_dev", torch.int32),
+        n_heads, head_dim, dtype_code(q.dtype), _ptr(workspace, "workspace", torch.uint8), workspace.numel(), _stream())
+    _check(rc, "raven_decode_attention")
+    return y
+
+
+def embed(wte, ids, scale, out=None):
+    M = ids.numel()
+    dim = wte.shape[1]
+    if out is None:
+        out = torch.empty(M, dim, device=wte.device, dtype=wte.dtype)
+    rc = load().raven_embed(_ptr(wte, "wte"), _ptr(ids, "ids", torch.int64), _ptr(out, "out", wte.dtype), M, dim,
+                            wte.shape[0], scale, dtype_code(wte.dtype), _stream())
+    _check(rc, "raven_embed")
+    return out
+
+
+def argmax(logits, out=None):
+    M, V = logits.shape
+    if out is None:
+        out = torch.empty(M, device=logits.device, dtype=torch.int64)
+    rc = load().raven_argmax(_ptr(logits, "logits", torch.float32), _ptr(out, "out", torch.int64), M, V, _stream())
+    _check(rc, "raven_argmax")
+    return out
+
+
+def advance_pos(pos_dev, delta=1):
+    _check(load().raven_advance_pos(_ptr(pos_dev, "pos_dev", torch.int32), delta, _stream()), "raven_advance_pos")
+
+
+def block_workspace(dims: Dims, M: int, device) -> torch.Tensor:
+    n = load().raven_block_workspace_bytes(C.byref(dims), M)
+    return torch.zeros(max(n, 256), dtype=torch.uint8, device=device)
+
+
+def sandwich_block(dims: Dims, w: BlockWeights, x_in, x_out, freqs, cache: KVCache, slot, B, S, pos0, workspace,
+                   ln_f=None, pos_dev=None):
+    rc = load().raven_sandwich_block(
+        C.byref(dims), C.byref(w), _ptr(ln_f, "ln_f", x_in.dtype), _ptr(x_in, "x_in"), _ptr(x_out, "x_out", x_in.dtype),
+        _ptr(freqs, "freqs", torch.float32), C.byref(cache), slot, B, S, pos0, _ptr(pos_dev, "pos_dev", torch.int32),
+        _ptr(workspace, "workspace", torch.uint8), workspace.numel(), _stream())
+    _check(rc, "raven_sandwich_block")
+    return x_out
+
+
+def core_iteration(dims: Dims, adapter_w, blocks, state_in, embeds, state_out, freqs, cache: KVCache, first_slot,
+                   B, S, pos0, workspace, ln_f=None, pos_dev=None):
+    """blocks: a ctypes array (BlockWeights * n)."""
+    rc = load().raven_core_iteration(
+        C.byref(dims), _ptr(adapter_w, "adapter_w", state_in.dtype), blocks, len(blocks), _ptr(ln_f, "ln_f", state_in.dtype),
+        _ptr(state_in, "state_in"), _ptr(embeds, "embeds", state_in.dtype), _ptr(state_out, "state_out", state_in.dtype),
+        _ptr(freqs, "freqs", torch.float32), C.byref(cache), first_slot, B, S, pos0,
+        _ptr(pos_dev, "pos_dev", torch.int32), _ptr(workspace, "workspace", torch.uint8), workspace.numel(), _stream())
+    _check(rc, "raven_core_iteration")
+    return state_out

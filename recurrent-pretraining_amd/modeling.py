@@ -1,0 +1,749 @@
+"""Host side of the MI355X recurrent-core decode path: a model class with the surface of the
+reference's RavenForCausalLM (recpre/raven_modeling_minimal.py, "RMM": forward 638-724,
+iterate_forward 726-762, core_block_forward 764-781, iterate_one_step 841-868, predict_from_latents
+870-900, embed_inputs 902-934, generate_minimal 1165-1232) whose arithmetic runs in the HIP kernels
+of libraven_hip.so.  torch.nn modules are used only as named parameter containers, so a reference
+state dict loads with `load_state_dict` unchanged.
+
+What differs from the reference on purpose:
+  * token rows are processed as [B*S, h]; K/V live in one contiguous step-indexed buffer;
+  * positions must be contiguous and, when a cache is given, continue the cache
+    (position == cache index); anything else raises NotImplementedError;
+  * `attention_mask` is accepted and ignored, as in the reference (RMM:676);
+  * only inference: no autograd, no labels-driven backward (a loss value is still returned).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import math
+from dataclasses import dataclass
+from typing import Any, Callable, Optional, Union
+
+import torch
+
+from . import hip
+from .cache import HuginnDynamicCache, remap_step
+from .config import RavenConfig
+
+
+@dataclass
+class CausalLMOutputRecurrentLatents:  # RMM:113-123
+    loss: Optional[torch.Tensor] = None
+    log_ppl: Optional[torch.Tensor] = None
+    logits: Optional[torch.Tensor] = None
+    past_key_values: Optional[HuginnDynamicCache] = None
+    latent_states: Optional[torch.Tensor] = None
+    hidden_states: Optional[torch.Tensor] = None
+    attention_maps: Optional[dict] = None
+    stats: Optional[dict] = None
+
+    def __getitem__(self, k):
+        return getattr(self, k)
+
+
+@dataclass
+class GenerationSettings:
+    """The fields of transformers.GenerationConfig that the generate loops read."""
+    max_length: int = 4096
+    max_new_tokens: Optional[int] = None
+    do_sample: bool = False
+    temperature: Optional[float] = None
+    top_k: Optional[int] = None
+    top_p: Optional[float] = None
+    min_p: Optional[float] = None
+    repetition_penalty: Optional[float] = None
+    eos_token_id: Any = None
+    return_dict_in_generate: bool = False
+
+
+@dataclass
+class GenerateOutput:
+    sequences: torch.Tensor
+    past_key_values: Optional[HuginnDynamicCache] = None
+    scores: Optional[dict] = None
+
+
+# ------------------------------------------------------------------------------------------------
+# parameter containers with the reference's module/parameter names (RMM:129-145, 439-452, 496-503, 512-523)
+# ------------------------------------------------------------------------------------------------
+class RMSNorm(torch.nn.Module):
+    def __init__(self, dim: int, eps: float):
+        super().__init__()
+        self.eps = eps
+        self.weight = torch.nn.Parameter(torch.ones(dim), requires_grad=False)
+
+
+def _linear(n_in: int, n_out: int) -> torch.nn.Linear:
+    lin = torch.nn.Linear(n_in, n_out, bias=False)
+    lin.weight.requires_grad_(False)
+    return lin
+
+
+class CausalSelfAttention(torch.nn.Module):
+    def __init__(self, cfg: RavenConfig):
+        super().__init__()
+        self.Wqkv = _linear(cfg.n_embd, 3 * cfg.n_embd)
+        if cfg.qk_bias:
+            self.qk_bias = torch.nn.Parameter(torch.zeros(2, 1, cfg.n_heads, cfg.head_dim), requires_grad=False)
+        self.proj = _linear(cfg.n_embd, cfg.n_embd)
+
+
+class GatedMLP(torch.nn.Module):
+    def __init__(self, cfg: RavenConfig):
+        super().__init__()
+        self.fc = _linear(cfg.n_embd, 2 * cfg.intermediate_size)
+        self.proj = _linear(cfg.intermediate_size, cfg.n_embd)
+
+
+class SandwichBlock(torch.nn.Module):
+    def __init__(self, cfg: RavenConfig, layer_id: int):
+        super().__init__()
+        self.norm_1 = RMSNorm(cfg.n_embd, cfg.norm_eps)
+        self.attn = CausalSelfAttention(cfg)
+        self.norm_2 = RMSNorm(cfg.n_embd, cfg.norm_eps)
+        self.mlp = GatedMLP(cfg)
+        self.norm_3 = RMSNorm(cfg.n_embd, cfg.norm_eps)
+        self.norm_4 = RMSNorm(cfg.n_embd, cfg.norm_eps)
+        self.layer_id = layer_id
+
+    def native(self) -> hip.BlockWeights:
+        a, m = self.attn, self.mlp
+        bias = a.qk_bias if hasattr(a, "qk_bias") else None
+        return hip.make_block_weights(self.norm_1.weight, self.norm_2.weight, self.norm_3.weight, self.norm_4.weight,
+                                      a.Wqkv.weight, bias, a.proj.weight, m.fc.weight, m.proj.weight)
+
+
+def precompute_freqs_cis(dim: int, end: int, theta: float) -> torch.Tensor:
+    """(cos, sin) table [1, end, 1, dim/2, 2] in fp32 (RMM:2076-2081)."""
+    inv = 1.0 / (theta ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim))
+    ang = torch.outer(torch.arange(end, dtype=torch.float32), inv).float()
+    return torch.stack([ang.cos()[None, :, None, :], ang.sin()[None, :, None, :]], dim=4)
+
+
+def _as_int(v) -> int:
+    return int(v.item()) if isinstance(v, torch.Tensor) else int(v)
+
+
+class RavenForCausalLM(torch.nn.Module):
+    config_class = RavenConfig
+
+    def __init__(self, config: RavenConfig, device: Union[str, torch.device] = "cuda", dtype: Optional[torch.dtype] = None):
+        super().__init__()
+        self.config = config
+        dtype = dtype if dtype is not None else getattr(torch, config.torch_dtype)
+        with torch.device(device):
+            prelude = torch.nn.ModuleList(SandwichBlock(config, i) for i in range(config.n_layers_in_prelude))
+            adapter = _linear(2 * config.n_embd, config.n_embd)
+            core = torch.nn.ModuleList(SandwichBlock(config, i + config.n_layers_in_prelude)
+                                       for i in range(config.n_layers_in_recurrent_block))
+            o = config.n_layers_in_prelude + config.n_layers_in_recurrent_block * config.mean_recurrence
+            coda = torch.nn.ModuleList(SandwichBlock(config, i + o) for i in range(config.n_layers_in_coda))
+            wte = torch.nn.Embedding(config.padded_vocab_size, config.n_embd)
+            wte.weight.requires_grad_(False)
+            self.transformer = torch.nn.ModuleDict(dict(wte=wte, prelude=prelude, adapter=adapter, core_block=core,
+                                                        coda=coda, ln_f=RMSNorm(config.n_embd, config.norm_eps)))
+            self.lm_head = _linear(config.n_embd, config.padded_vocab_size)
+            if config.tie_embeddings:
+                self.lm_head.weight = self.transformer.wte.weight
+            self.register_buffer("freqs_cis", precompute_freqs_cis(config.head_dim, config.block_size, config.rope_base),
+                                 persistent=True)
+        self.to(dtype)  # casts the RoPE table too, as nn.Module.to does for the reference (RMM:577)
+        self.generation_config = GenerationSettings()
+        self._native_key = None
+        self._native: dict = {}
+        self._scratch: dict = {}
+        self.eval()
+
+    # ---- small helpers -------------------------------------------------------------------------
+    @property
+    def emb_scale(self) -> float:  # RMM:50-52
+        return self.config.init_values["embed_scale"]
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self.transformer.wte.weight.dtype
+
+    @property
+    def device(self) -> torch.device:
+        return self.transformer.wte.weight.device
+
+    def get_input_embeddings(self):
+        return self.transformer.wte
+
+    def get_output_embeddings(self):
+        return self.lm_head
+
+    def synthetic_weight_order(self) -> list:
+        """Tensor names in the order the synthetic draw visits them: embedding, prelude blocks, adapter,
+        core blocks, coda blocks, ln_f; inside a block norm_1, Wqkv, qk_bias, proj, norm_2, fc, mlp.proj,
+        norm_3, norm_4."""
+        cfg = self.config
+        per_block = ["norm_1.weight", "attn.Wqkv.weight"] + (["attn.qk_bias"] if cfg.qk_bias else []) + [
+            "attn.proj.weight", "norm_2.weight", "mlp.fc.weight", "mlp.proj.weight", "norm_3.weight", "norm_4.weight"]
+        names = ["transformer.wte.weight"]
+        for group, n in (("prelude", cfg.n_layers_in_prelude), ("adapter", 0), ("core_block", cfg.n_layers_in_recurrent_block),
+                         ("coda", cfg.n_layers_in_coda)):
+            if group == "adapter":
+                names.append("transformer.adapter.weight")
+            names += [f"transformer.{group}.{i}.{k}" for i in range(n) for k in per_block]
+        names.append("transformer.ln_f.weight")
+        if not cfg.tie_embeddings:
+            names.append("lm_head.weight")
+        return names
+
+    @torch.no_grad()
+    def init_weights(self, seed: int = 0, std: float = 0.02) -> None:
+        """Synthetic weights: every tensor ~ N(0, std) (norm weights ~ N(1, std)), drawn on the CPU in
+        synthetic_weight_order() from one seeded generator and cast, so that any host reproduces them."""
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        sd = self.state_dict()
+        for name in self.synthetic_weight_order():
+            p = sd[name]
+            mean = 1.0 if (name.endswith("weight") and p.dim() == 1) else 0.0
+            p.copy_(torch.empty(p.shape, dtype=torch.float32).normal_(mean, std, generator=g).to(p.dtype))
+
+    def _natives(self) -> dict:
+        """ctypes views of the weights; rebuilt when a parameter's storage has moved."""
+        key = (self.transformer.wte.weight.data_ptr(), self.transformer.adapter.weight.data_ptr(),
+               self.freqs_cis.data_ptr(), self.transformer.ln_f.weight.data_ptr(), self.dtype)
+        if key != self._native_key:
+            cfg, t = self.config, self.transformer
+            core = (hip.BlockWeights * len(t.core_block))(*[b.native() for b in t.core_block])
+            self._native = {
+                "dims": hip.make_dims(cfg.n_embd, cfg.n_heads, cfg.intermediate_size, cfg.norm_eps, self.dtype),
+                "prelude": [b.native() for b in t.prelude],
+                "core": core,
+                "coda": [b.native() for b in t.coda],
+                "freqs": self.freqs_cis.float().reshape(cfg.block_size, cfg.head_dim // 2, 2).contiguous(),
+            }
+            self._native_key = key
+            self._scratch.clear()
+        return self._native
+
+    def _workspace(self, M: int) -> torch.Tensor:
+        ws = self._scratch.get(("ws", M))
+        if ws is None:
+            ws = hip.block_workspace(self._natives()["dims"], M, self.device)
+            self._scratch[("ws", M)] = ws
+        return ws
+
+    def _scratch_cache(self, B: int, S: int) -> HuginnDynamicCache:
+        """A one-slot cache for forwards without past_key_values: every block appends its S new
+        keys to it and attends causally, which is what the reference does with no cache."""
+        key = ("nocache", B)
+        c = self._scratch.get(key)
+        cfg = self.config
+        if c is None or c.t_max < S:
+            c = HuginnDynamicCache()
+            c.ensure(1, 0, B, cfg.n_heads, cfg.head_dim, S, self.dtype, self.device)
+            self._scratch[key] = c
+        return c
+
+    def _positions(self, n_tokens: int, position_ids, cache_position) -> int:
+        """First RoPE position of this call (RMM:660-665); positions must be contiguous."""
+        src = position_ids if position_ids is not None else cache_position
+        if src is None:
+            return 0
+        pos = src.reshape(-1)[-n_tokens:].tolist() if src.numel() >= n_tokens else src.reshape(-1).tolist()
+        if len(pos) != n_tokens or any(pos[i] != pos[0] + i for i in range(n_tokens)):
+            raise NotImplementedError("positions must be one contiguous range shared by the batch")
+        if pos[0] + n_tokens > self.config.block_size:
+            raise ValueError(f"positions up to {pos[0] + n_tokens - 1} exceed block_size {self.config.block_size}")
+        return int(pos[0])
+
+    def _split_steps(self, num_steps) -> int:
+        """Total recurrences (RMM:739-744; eval sampler RMM:799-802)."""
+        if num_steps is None:
+            return self.config.mean_recurrence
+        if isinstance(num_steps, torch.Tensor) and num_steps.dim() == 0:
+            return int(num_steps)
+        if hasattr(num_steps, "__len__") and len(num_steps) > 1:
+            return int(num_steps[0]) + int(num_steps[1])
+        return int(num_steps)
+
+    # ---- pieces of the forward --------------------------------------------------------------------
+    def _run_block(self, which: str, i: int, step_idx: int, x: torch.Tensor, cache: HuginnDynamicCache, private: bool,
+                   B: int, S: int, pos0: int, ln_f: bool = False) -> torch.Tensor:
+        nat = self._natives()
+        slot = 0 if private else cache.note_append(step_idx, S, pos0)
+        out = torch.empty_like(x)
+        hip.sandwich_block(nat["dims"], nat[which][i], x, out, nat["freqs"], cache.native(), slot, B, S, pos0,
+                           self._workspace(B * S), ln_f=self.transformer.ln_f.weight if ln_f else None)
+        return out
+
+    def _run_core(self, x: torch.Tensor, embeds: torch.Tensor, first_step: int, cache: HuginnDynamicCache, private: bool,
+                  B: int, S: int, pos0: int, ln_f: bool) -> torch.Tensor:
+        """One core_block_forward (RMM:764-781) on [B*S, h] rows."""
+        nat, t = self._natives(), self.transformer
+        n_core = len(t.core_block)
+        slots = [0 if private else cache.note_append(first_step + j, S, pos0) for j in range(n_core)]
+        out = torch.empty_like(x)
+        ws = self._workspace(B * S)
+        lnw = t.ln_f.weight if ln_f else None
+        if not private and n_core > 0 and all(slots[j] == slots[0] + j for j in range(n_core)):
+            hip.core_iteration(nat["dims"], t.adapter.weight, nat["core"], x, embeds, out, nat["freqs"], cache.native(),
+                               slots[0], B, S, pos0, ws, ln_f=lnw)
+            return out
+        cur = hip.adapter_gemm_concat(x, embeds, t.adapter.weight)
+        for j in range(n_core):
+            last = j == n_core - 1
+            nxt = out if last else torch.empty_like(x)
+            hip.sandwich_block(nat["dims"], nat["core"][j], cur, nxt, nat["freqs"], cache.native(), slots[j], B, S, pos0, ws,
+                               ln_f=lnw if last else None)
+            cur = nxt
+        if n_core == 0:
+            out = cur if lnw is None else hip.rmsnorm_residual(cur, lnw, self.config.norm_eps)[0]
+        return out
+
+    @torch.no_grad()
+    def initialize_state(self, input_embeds: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+        """RMM:804-813, with torch's generator of the tensor's device."""
+        x = torch.randn_like(input_embeds)
+        std = self.config.init_values["std"] * scale
+        if std > 0:
+            torch.nn.init.trunc_normal_(x, mean=0.0, std=std, a=-3 * std, b=3 * std)
+            if self.emb_scale != 1:
+                x = x * self.emb_scale
+        else:
+            x.zero_()
+        return x
+
+    def _prepare_cache(self, past_key_values, use_cache: bool, B: int, S: int, r: int):
+        """Returns (cache, private, cache_pos0) and reserves storage for this call's steps."""
+        cfg = self.config
+        if use_cache and past_key_values is None:
+            past_key_values = HuginnDynamicCache()
+        if past_key_values is None:
+            return self._scratch_cache(B, S), True, 0
+        if not isinstance(past_key_values, HuginnDynamicCache):
+            raise TypeError("past_key_values must be this package's HuginnDynamicCache")
+        cache = past_key_values
+        pos0 = cache._seen_tokens
+        n_pos = cfg.n_layers_in_prelude + cfg.n_layers_in_recurrent_block * r
+        n_pos = max((remap_step(s, cache.lookup_strategy) for s in range(n_pos)), default=-1) + 1
+        cache.ensure(max(n_pos, 1), cfg.n_layers_in_coda, B, cfg.n_heads, cfg.head_dim, pos0 + S, self.dtype, self.device)
+        return cache, False, pos0
+
+    # ---- reference surface -----------------------------------------------------------------------
+    @torch.no_grad()
+    def forward(
+        self,
+        input_ids: Optional[torch.Tensor] = None,
+        input_embeds: Optional[torch.Tensor] = None,
+        input_states: Optional[torch.Tensor] = None,
+        attention_mask: Optional[torch.Tensor] = None,
+        position_ids: Optional[torch.Tensor] = None,
+        labels: Optional[torch.Tensor] = None,
+        num_steps=None,
+        past_key_values: Optional[HuginnDynamicCache] = None,
+        output_details: dict = {"return_logits": True, "return_latents": True, "return_head": False, "return_stats": False},
+        use_cache: bool = False,
+        cache_position: Optional[torch.Tensor] = None,
+        init_scale: float = 1.0,
+        **kwargs,
+    ) -> CausalLMOutputRecurrentLatents:
+        cfg, t = self.config, self.transformer
+        src = input_ids if input_embeds is None else input_embeds
+        B, S = src.shape[0], src.shape[1]
+        M, h = B * S, cfg.n_embd
+        rope_pos0 = self._positions(S, position_ids, cache_position)
+        r = self._split_steps(num_steps)
+        cache, private, pos0 = self._prepare_cache(past_key_values, use_cache, B, S, r)
+        if rope_pos0 != pos0 and not (private and position_ids is None and cache_position is None):
+            raise NotImplementedError(f"positions start at {rope_pos0} but the cache holds {pos0} tokens")
+        if not private:
+            cache._seen_tokens += S  # what the step-0 update does in the reference (RMM:188-189)
+
+        if input_embeds is None:
+            x = hip.embed(t.wte.weight, input_ids.reshape(-1).to(torch.int64).contiguous(), self.emb_scale)
+        else:
+            x = (input_embeds.to(self.dtype) * self.emb_scale).reshape(M, h).contiguous()
+
+        block_idx = -1
+        for i in range(len(t.prelude)):
+            block_idx += 1
+            x = self._run_block("prelude", i, block_idx, x, cache, private, B, S, pos0)
+        embeds = x
+
+        if input_states is None:
+            state = self.initialize_state(embeds, init_scale)
+        else:
+            state = input_states.to(self.dtype).reshape(M, h).clone()
+        x = self._iterate(state, embeds, block_idx, cache, private, B, S, pos0, r)
+        latents = x.view(B, S, h).clone()
+
+        n_coda = len(t.coda)
+        for i in range(n_coda):
+            x = self._run_block("coda", i, -(i + 1), x, cache, private, B, S, pos0, ln_f=(i == n_coda - 1))
+        if n_coda == 0:
+            x = hip.rmsnorm_residual(x, t.ln_f.weight, cfg.norm_eps)[0]
+
+        logits = hip.gemm(x, self.lm_head.weight, out_f32=True).view(B, S, -1)
+        if labels is not None:
+            loss = torch.nn.functional.cross_entropy(logits.view(-1, logits.shape[-1]), labels.view(-1), ignore_index=-100)
+            log_ppl = loss.clone()
+        else:
+            loss, log_ppl = torch.as_tensor(0.0), torch.as_tensor(0.0)
+        return CausalLMOutputRecurrentLatents(
+            loss=loss, log_ppl=log_ppl,
+            logits=logits if output_details.get("return_logits", True) else None,
+            past_key_values=None if private else cache,
+            hidden_states=x.view(B, S, h) if output_details.get("return_head", False) else None,
+            latent_states=latents if output_details.get("return_latents", True) else None,
+        )
+
+    def _iterate(self, state, embeds, block_idx: int, cache, private, B, S, pos0, r: int) -> torch.Tensor:
+        """The r-loop of iterate_forward plus its closing ln_f (RMM:751-762)."""
+        n_core = len(self.transformer.core_block)
+        x = state
+        for it in range(r):
+            x = self._run_core(x, embeds, block_idx + 1 + it * n_core, cache, private, B, S, pos0, ln_f=(it == r - 1))
+        if r == 0:
+            x = hip.rmsnorm_residual(x, self.transformer.ln_f.weight, self.config.norm_eps)[0]
+        return x
+
+    @torch.no_grad()
+    def iterate_forward(self, input_embeds, input_states, freqs_cis=None, block_idx=None, mask=None, past_key_values=None,
+                        num_steps=None, init_scale: float = 1.0):
+        """RMM:726-762.  `freqs_cis` is not needed (positions follow from the cache) and is ignored.
+        Returns (ln_f(x), n_no_grad, n_grad, None, block_idx)."""
+        B, S, h = input_embeds.shape
+        r = self._split_steps(num_steps)
+        b0 = _as_int(block_idx) if block_idx is not None else len(self.transformer.prelude) - 1
+        cache, private, pos0 = self._cache_for_piece(past_key_values, B, S, b0 + 1 + r * len(self.transformer.core_block))
+        embeds = input_embeds.to(self.dtype).reshape(B * S, h).contiguous()
+        state = (self.initialize_state(embeds, init_scale) if input_states is None
+                 else input_states.to(self.dtype).reshape(B * S, h).clone())
+        x = self._iterate(state, embeds, b0, cache, private, B, S, pos0, r)
+        out_idx = torch.tensor(b0 + r * len(self.transformer.core_block), dtype=torch.long)
+        return x.view(B, S, h), r, 0, None, out_idx
+
+    def _cache_for_piece(self, past_key_values, B: int, S: int, n_pos_steps: int):
+        """Cache handling for the per-piece entry points, which run after step 0 has already
+        advanced the token count: the new tokens sit at _seen_tokens - S (RMM:194)."""
+        cfg = self.config
+        if past_key_values is None:
+            return self._scratch_cache(B, S), True, 0
+        cache = past_key_values
+        pos0 = cache._seen_tokens - S
+        if pos0 < 0:
+            raise ValueError("the cache has seen fewer tokens than this call brings: run embed_inputs first")
+        n_pos = max((remap_step(s, cache.lookup_strategy) for s in range(n_pos_steps)), default=-1) + 1
+        cache.ensure(max(n_pos, 1), cfg.n_layers_in_coda, B, cfg.n_heads, cfg.head_dim, pos0 + S, self.dtype, self.device)
+        return cache, False, pos0
+
+    @torch.no_grad()
+    def core_block_forward(self, x, input_embeds, freqs_cis=None, mask=None, past_key_values=None, block_idx=0,
+                           current_step=0):
+        """RMM:764-781: one recurrence; returns (x, block_idx + n_core)."""
+        B, S, h = x.shape
+        b0 = _as_int(block_idx)
+        n_core = len(self.transformer.core_block)
+        cache, private, pos0 = self._cache_for_piece(past_key_values, B, S, b0 + 1 + n_core)
+        out = self._run_core(x.to(self.dtype).reshape(B * S, h).contiguous(),
+                             input_embeds.to(self.dtype).reshape(B * S, h).contiguous(), b0 + 1, cache, private, B, S, pos0,
+                             ln_f=False)
+        return out.view(B, S, h), torch.tensor(b0 + n_core, dtype=torch.long)
+
+    @torch.no_grad()
+    def iterate_one_step(self, input_embeds, input_states, position_ids=None, cache_position=None,
+                         block_idx=torch.tensor(0, dtype=torch.long), attention_mask=None, past_key_values=None,
+                         current_step: int = 0):
+        """RMM:841-868."""
+        x, block_idx = self.core_block_forward(input_states, input_embeds, None, attention_mask, past_key_values, block_idx,
+                                               current_step)
+        return x, block_idx, current_step + 1
+
+    @torch.no_grad()
+    def predict_from_latents(self, latents, attention_mask=None, position_ids=None, cache_position=None,
+                             past_key_values=None):
+        """RMM:870-900: ln_f, coda, ln_f, head."""
+        cfg, t = self.config, self.transformer
+        B, S, h = latents.shape
+        cache, private, pos0 = self._cache_for_piece(past_key_values, B, S, 1)
+        x = hip.rmsnorm_residual(latents.to(self.dtype).reshape(B * S, h).contiguous(), t.ln_f.weight, cfg.norm_eps)[0]
+        n_coda = len(t.coda)
+        for i in range(n_coda):
+            x = self._run_block("coda", i, -(i + 1), x, cache, private, B, S, pos0, ln_f=(i == n_coda - 1))
+        if n_coda == 0:
+            x = hip.rmsnorm_residual(x, t.ln_f.weight, cfg.norm_eps)[0]
+        logits = hip.gemm(x, self.lm_head.weight, out_f32=True).view(B, S, -1)
+        return CausalLMOutputRecurrentLatents(loss=torch.as_tensor(0.0), log_ppl=torch.as_tensor(0.0), logits=logits,
+                                              past_key_values=past_key_values, latent_states=x.view(B, S, h))
+
+    @torch.no_grad()
+    def embed_inputs(self, input_ids, attention_mask=None, position_ids=None, past_key_values=None, use_cache=False,
+                     cache_position=None, **kwargs):
+        """RMM:902-934: embedding times sqrt(h), then the prelude; returns (embeds, block_idx)."""
+        cfg, t = self.config, self.transformer
+        B, S = input_ids.shape
+        rope_pos0 = self._positions(S, position_ids, cache_position)
+        cache, private, pos0 = self._prepare_cache(past_key_values, use_cache, B, S, 0)
+        if rope_pos0 != pos0 and not (private and position_ids is None and cache_position is None):
+            raise NotImplementedError(f"positions start at {rope_pos0} but the cache holds {pos0} tokens")
+        if not private:
+            cache._seen_tokens += S
+        x = hip.embed(t.wte.weight, input_ids.reshape(-1).to(torch.int64).contiguous(), self.emb_scale)
+        block_idx = -1
+        for i in range(len(t.prelude)):
+            block_idx += 1
+            x = self._run_block("prelude", i, block_idx, x, cache, private, B, S, pos0)
+        return x.view(B, S, cfg.n_embd), torch.tensor(block_idx, dtype=torch.long)
+
+    # ---- generation --------------------------------------------------------------------------------
+    def prepare_inputs_for_generation(self, input_ids, past_key_values=None, attention_mask=None, inputs_embeds=None,
+                                      cache_position=None, cache_lookup_strategy: str = "full", **kwargs):
+        """RMM:1066-1110, without the HF cache swapping: feeds the tokens the cache has not seen."""
+        model_inputs = {}
+        seen = past_key_values.get_seq_length() if past_key_values is not None else 0
+        if cache_position is None:
+            cache_position = torch.arange(seen, input_ids.shape[1], device=input_ids.device)
+        model_inputs["cache_position"] = cache_position
+        model_inputs["past_key_values"] = past_key_values if kwargs.get("use_cache", True) else None
+        model_inputs["input_ids"] = input_ids[:, cache_position].contiguous()
+        for key, value in kwargs.items():
+            if key not in model_inputs:
+                model_inputs[key] = value
+        return model_inputs
+
+    def _get_stops(self, generation_config, model_kwargs=None) -> set:
+        stops = {65504, 65505, 65508}  # begin_text, end_text, end_turn (RMM:1929-1931)
+        eos = getattr(generation_config, "eos_token_id", None)
+        if eos is not None:
+            try:
+                stops.update(eos)
+            except TypeError:
+                stops.add(eos)
+        return stops
+
+    def _sample_next_token(self, next_token_logits: torch.Tensor, input_ids, generation_config) -> torch.Tensor:
+        """RMM:1944-1989.  Greedy selection runs in the HIP argmax kernel."""
+        gc = generation_config
+        if not getattr(gc, "do_sample", False):
+            return hip.argmax(next_token_logits.float().contiguous()).unsqueeze(-1)
+        logits = next_token_logits.to(torch.float32)
+        if gc.temperature:
+            logits = logits / gc.temperature
+        probs = torch.softmax(logits, dim=-1)
+        if gc.top_k:
+            kth = torch.topk(probs, gc.top_k, dim=-1).values[:, -1:]
+            probs = torch.where(probs < kth, torch.zeros_like(probs), probs)
+        if gc.top_p:
+            sp, si = torch.sort(probs, descending=True, dim=-1)
+            remove = torch.cumsum(sp, dim=-1) > gc.top_p
+            remove[:, 0] = False
+            mask = torch.zeros_like(probs, dtype=torch.bool).scatter(1, si, remove)
+            probs = torch.where(mask, torch.zeros_like(probs), probs)
+        if gc.min_p:
+            probs = torch.where(probs < gc.min_p * probs.max(dim=-1, keepdim=True).values, torch.zeros_like(probs), probs)
+        probs = probs / probs.sum(dim=-1, keepdim=True).clamp(min=1e-10)
+        return torch.multinomial(probs, num_samples=1)
+
+    @torch.no_grad()
+    def generate(self, input_ids: torch.Tensor, generation_config=None, **kwargs):
+        """Dispatcher of RMM:1112-1127.  The adaptive-compute, speculative and diffusion-style loops
+        of the reference are not part of this package; everything else goes to generate_minimal."""
+        for k in ("criterion", "exit_threshold", "exit_evaluator", "draft_steps", "lookahead_for_draft",
+                  "verification_threshold", "headway", "state_noise_mixing", "inner_recurrence", "freeze_strategy"):
+            if k in kwargs:
+                raise NotImplementedError(f"generate(..., {k}=...) selects a sampler this package does not provide")
+        return self.generate_minimal(input_ids, generation_config, **kwargs)
+
+    @torch.no_grad()
+    def generate_minimal(self, input_ids: torch.Tensor, generation_config=None, tokenizer=None, streamer=None,
+                         continuous_compute: bool = False, init_scale: float = 1.0, cache_lookup_strategy: str = "full",
+                         input_states_fn: Optional[Callable] = None, stop_tokens: Optional[set] = None,
+                         use_graph: bool = True, **model_kwargs):
+        """RMM:1165-1232.  Prefill through forward(), then one token per step through the decode
+        runner (all kernels of a token on one stream, optionally replayed as a HIP graph).
+
+        input_states_fn(call_index, (B, S, h)) -> latent state to inject into that forward (an
+        extension for reproducible runs: the reference re-draws the state from the device RNG on
+        every call, RMM:738).  stop_tokens overrides the reference's fixed stop set."""
+        gc = generation_config if generation_config is not None else self.generation_config
+        B, prompt_len = input_ids.shape
+        if "max_new_tokens" in model_kwargs and model_kwargs["max_new_tokens"] is not None:
+            max_new = model_kwargs["max_new_tokens"]
+            if "max_length" in model_kwargs:
+                max_new = min(max_new, model_kwargs["max_length"] - prompt_len)
+        elif getattr(gc, "max_new_tokens", None):
+            max_new = gc.max_new_tokens
+        else:
+            max_new = model_kwargs.get("max_length", gc.max_length) - prompt_len
+        num_steps = model_kwargs.get("num_steps", None)
+        stops = self._get_stops(gc) if stop_tokens is None else set(stop_tokens)
+        input_ids = input_ids.to(self.device)
+        if max_new <= 0:
+            return input_ids
+        total = min(prompt_len + max_new, self.config.block_size)
+        cache = model_kwargs.get("past_key_values") or HuginnDynamicCache(cache_lookup_strategy, max_length=total)
+
+        def state_for(call: int, S: int, embeds_like=None):
+            if input_states_fn is not None:
+                return input_states_fn(call, (B, S, self.config.n_embd)).to(self.device, self.dtype)
+            return None
+
+        # prefill
+        seen = cache.get_seq_length()
+        pos = torch.arange(seen, prompt_len, device=self.device)
+        out = self.forward(input_ids=input_ids[:, seen:], input_states=state_for(0, prompt_len - seen), num_steps=num_steps,
+                           past_key_values=cache, use_cache=True, cache_position=pos, init_scale=init_scale)
+        next_tok = self._sample_next_token(out.logits[:, -1, :], input_ids, gc)
+        carried = out.latent_states[:, -1:, :] if continuous_compute else None
+        tokens = [next_tok]
+        alive = torch.ones(B, dtype=torch.bool)
+        if streamer:
+            streamer.put(next_tok.cpu())
+
+        def update_alive(tok) -> bool:
+            if stops:
+                for b, v in enumerate(tok.view(-1).tolist()):
+                    if alive[b] and v in stops:
+                        alive[b] = False
+            return bool(alive.any())
+
+        runner = None
+        call = 1
+        while len(tokens) < max_new and update_alive(tokens[-1]) and cache.get_seq_length() + 1 <= total:
+            if runner is None:
+                runner = DecodeRunner(self, cache, B, self._split_steps(num_steps), greedy=not getattr(gc, "do_sample", False),
+                                      use_graph=use_graph)
+            state = carried if continuous_compute else state_for(call, 1)
+            logits, nxt, latents = runner.step(tokens[-1].view(-1), state, init_scale)
+            if getattr(gc, "do_sample", False):
+                nxt = self._sample_next_token(logits, input_ids, gc).view(-1)
+            tokens.append(nxt.view(B, 1).clone())
+            if continuous_compute:
+                carried = latents.view(B, 1, -1).clone()
+            if streamer:
+                streamer.put(tokens[-1].cpu())
+            call += 1
+        if streamer:
+            streamer.end()
+        sequences = torch.cat([input_ids] + tokens, dim=-1)
+        if getattr(gc, "return_dict_in_generate", False):
+            return GenerateOutput(sequences=sequences, past_key_values=cache, scores={})
+        return sequences
+
+
+class DecodeRunner:
+    """One decode step (S = 1) with every buffer preallocated: embedding, prelude, r recurrences,
+    coda, ln_f, LM head and greedy argmax are enqueued back to back on the current stream.  The
+    position is read by the kernels from a device counter, so the identical launch sequence serves
+    every token and can be replayed as one HIP graph."""
+
+    def __init__(self, model: RavenForCausalLM, cache: HuginnDynamicCache, batch: int, num_steps: int, greedy: bool = True,
+                 use_graph: bool = True):
+        cfg = model.config
+        self.model, self.cache, self.B, self.r, self.greedy = model, cache, batch, num_steps, greedy
+        dev, dt, h = model.device, model.dtype, cfg.n_embd
+        n_pos = cfg.n_layers_in_prelude + cfg.n_layers_in_recurrent_block * num_steps
+        n_pos = max((remap_step(s, cache.lookup_strategy) for s in range(n_pos)), default=-1) + 1
+        need_t = cache.max_length if cache.max_length is not None else cache.get_seq_length() + 1
+        cache.ensure(max(n_pos, 1), cfg.n_layers_in_coda, batch, cfg.n_heads, cfg.head_dim, need_t, dt, dev)
+        self.ids = torch.zeros(batch, dtype=torch.int64, device=dev)
+        self.pos = torch.zeros(1, dtype=torch.int32, device=dev)
+        self.state = torch.zeros(batch, h, dtype=dt, device=dev)
+        self.embeds = torch.empty(batch, h, dtype=dt, device=dev)
+        self.x = torch.empty(batch, h, dtype=dt, device=dev)
+        self.y = torch.empty(batch, h, dtype=dt, device=dev)
+        self.latents = torch.empty(batch, h, dtype=dt, device=dev)
+        self.logits = torch.empty(batch, cfg.padded_vocab_size, dtype=torch.float32, device=dev)
+        self.next_ids = torch.zeros(batch, dtype=torch.int64, device=dev)
+        self.ws = hip.block_workspace(model._natives()["dims"], batch, dev)
+        self.use_graph = use_graph
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self._graph_t_max = None
+        self._warm = False
+
+    def _slots(self):
+        """(prelude slots, first core slot per recurrence or per-block slots, coda slots) for one token."""
+        cfg, c = self.model.config, self.cache
+        n_pre, n_core, n_coda = cfg.n_layers_in_prelude, cfg.n_layers_in_recurrent_block, cfg.n_layers_in_coda
+        pre = [c._slot(remap_step(i, c.lookup_strategy)) for i in range(n_pre)]
+        core = [[c._slot(remap_step(n_pre + it * n_core + j, c.lookup_strategy)) for j in range(n_core)] for it in range(self.r)]
+        coda = [c._slot(-(i + 1)) for i in range(n_coda)]
+        return pre, core, coda
+
+    def _enqueue(self):
+        """Launches one token's kernels; reads the position from self.pos."""
+        m, t = self.model, self.model.transformer
+        nat, cfg, B = m._natives(), m.config, self.B
+        kv = self.cache.native()
+        hint = self.cache.t_max - 1  # sizes grids; the kernels take the true position from the device
+        pre, core, coda = self._slots()
+        hip.embed(t.wte.weight, self.ids, m.emb_scale, out=self.embeds)
+        cur = self.embeds
+        for i, slot in enumerate(pre):
+            hip.sandwich_block(nat["dims"], nat["prelude"][i], cur, self.embeds, nat["freqs"], kv, slot, B, 1, hint, self.ws,
+                               pos_dev=self.pos)
+        x = self.state
+        n_core = len(t.core_block)
+        for it, slots in enumerate(core):
+            lnw = t.ln_f.weight if it == self.r - 1 else None
+            if n_core > 0 and all(slots[j] == slots[0] + j for j in range(n_core)):
+                hip.core_iteration(nat["dims"], t.adapter.weight, nat["core"], x, self.embeds, self.x, nat["freqs"], kv, slots[0],
+                                   B, 1, hint, self.ws, ln_f=lnw, pos_dev=self.pos)
+            else:
+                hip_x = hip.adapter_gemm_concat(x, self.embeds, t.adapter.weight)
+                for j in range(n_core):
+                    last = j == n_core - 1
+                    hip.sandwich_block(nat["dims"], nat["core"][j], hip_x, self.x if last else hip_x, nat["freqs"], kv, slots[j],
+                                       B, 1, hint, self.ws, ln_f=lnw if last else None, pos_dev=self.pos)
+            x = self.x
+        if self.r == 0:
+            hip.load().raven_rmsnorm_residual(x.data_ptr(), None, t.ln_f.weight.data_ptr(), self.x.data_ptr(), None, None, None,
+                                              B, cfg.n_embd, cfg.norm_eps, hip.dtype_code(m.dtype), hip._stream())
+            x = self.x
+        self.latents.copy_(x)
+        n_coda = len(coda)
+        for i, slot in enumerate(coda):
+            hip.sandwich_block(nat["dims"], nat["coda"][i], x, self.y, nat["freqs"], kv, slot, B, 1, hint, self.ws,
+                               ln_f=t.ln_f.weight if i == n_coda - 1 else None, pos_dev=self.pos)
+            x = self.y
+        if n_coda == 0:
+            hip.load().raven_rmsnorm_residual(x.data_ptr(), None, t.ln_f.weight.data_ptr(), self.y.data_ptr(), None, None, None,
+                                              B, cfg.n_embd, cfg.norm_eps, hip.dtype_code(m.dtype), hip._stream())
+            x = self.y
+        rc = hip.load().raven_gemm(x.data_ptr(), m.lm_head.weight.data_ptr(), None, self.logits.data_ptr(), B,
+                                   cfg.padded_vocab_size, cfg.n_embd, hip.dtype_code(m.dtype), 1, hip._stream())
+        hip._check(rc, "raven_gemm")
+        hip.argmax(self.logits, out=self.next_ids)
+        hip.advance_pos(self.pos, 1)
+
+    def step(self, ids: torch.Tensor, state: Optional[torch.Tensor], init_scale: float = 1.0):
+        """Feeds one token per sequence; returns (logits [B,V] f32, next ids [B], latents [B,h]).
+        The returned tensors are the runner's own buffers: copy what must outlive the next step."""
+        m, c = self.model, self.cache
+        pos0 = c._seen_tokens
+        if pos0 + 1 > c.t_max:
+            c.ensure(1, 0, self.B, m.config.n_heads, m.config.head_dim, pos0 + 1, m.dtype, m.device)  # grows; pointers move
+            self.graph = None
+        self.ids.copy_(ids.view(-1))
+        self.pos.fill_(pos0)
+        if state is None:
+            if init_scale > 0:
+                self.state.copy_(m.initialize_state(self.embeds, init_scale))
+            else:
+                self.state.zero_()
+        else:
+            self.state.copy_(state.reshape(self.B, -1))
+        if self.use_graph and self._warm:
+            if self.graph is None or self._graph_t_max != c.t_max:
+                self.graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(self.graph):
+                    self._enqueue()
+                self._graph_t_max = c.t_max
+                self.pos.fill_(pos0)  # capture does not execute; make sure the counter is what this step needs
+            self.graph.replay()
+        else:
+            self._enqueue()
+            self._warm = True
+        # bookkeeping the reference does inside cache.update (RMM:188-196)
+        cfg = m.config
+        c._seen_tokens += 1
+        n_steps = cfg.n_layers_in_prelude + cfg.n_layers_in_recurrent_block * self.r
+        for s in list(range(n_steps)) + [-(i + 1) for i in range(cfg.n_layers_in_coda)]:
+            c.note_append(s, 1, pos0)
+        return self.logits, self.next_ids, self.latents

@@ -1,0 +1,248 @@
+"""GPU parity tests, kernel by kernel, through the C ABI (pkg.hip wrappers are thin ctypes calls)
+against the CPU oracle on identical seeded inputs.
+
+Tolerances: bf16 results must satisfy max-abs <= 2e-2 and rel-L2 <= 1e-2 against the oracle
+(the bar the build's target states for per-kernel outputs); fp32 results 1e-4 / 1e-5; integer
+outputs (argmax ids, cache positions) bit-exact."""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import raven_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+BF16_MAXABS, BF16_RELL2 = 2e-2, 1e-2
+F32_MAXABS, F32_RELL2 = 1e-4, 1e-5
+
+
+def close(got: torch.Tensor, want: torch.Tensor, what: str = ""):
+    got, want = got.detach().float().cpu(), want.detach().float().cpu()
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: non-finite values"
+    bf = want.dtype == torch.bfloat16 or True
+    max_abs = (got - want).abs().max().item()
+    rel = ((got - want).norm() / want.norm().clamp_min(1e-30)).item()
+    return max_abs, rel
+
+
+def check(got, want, dtype, what=""):
+    max_abs, rel = close(got, want, what)
+    lim_a, lim_r = (BF16_MAXABS, BF16_RELL2) if dtype == torch.bfloat16 else (F32_MAXABS, F32_RELL2)
+    scale = max(1.0, want.detach().float().abs().max().item())
+    assert max_abs <= lim_a * scale and rel <= lim_r, f"{what}: max-abs {max_abs:.3e} (scale {scale:.2f}), rel-L2 {rel:.3e}"
+
+
+def rnd(shape, dtype, seed, std=1.0, mean=0.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * std + mean).to(dtype)
+
+
+# ----------------------------------------------------------------------------- RMSNorm (config 2)
+@pytest.mark.parametrize("rows", [1, 32, 4096])
+def test_rmsnorm_residual_bf16_5280(pkg, rows):
+    dt, n = torch.bfloat16, 5280
+    x, res = rnd((rows, n), dt, 1), rnd((rows, n), dt, 2)
+    w = rnd((n,), dt, 3, 0.02, 1.0)
+    y, s, _ = pkg.hip.rmsnorm_residual(x.cuda(), w.cuda(), 1e-6, residual=res.cuda(), want_sum=True)
+    want_sum = x + res
+    assert torch.equal(s.cpu(), want_sum), "residual sum must be bit-exact (one bf16 add)"
+    check(y, O.rmsnorm(want_sum, w, 1e-6), dt, f"rmsnorm+residual rows={rows}")
+    # against an fp32-accumulate torch statement of the same op
+    ref32 = (F.rms_norm(want_sum.float(), (n,), eps=1e-6).to(dt).float() * w.float())
+    check(y, ref32, dt, "rmsnorm vs F.rms_norm")
+    # without a residual, and the fraction of bit-identical outputs should be overwhelming
+    y2, _, _ = pkg.hip.rmsnorm_residual(x.cuda(), w.cuda(), 1e-6)
+    want = O.rmsnorm(x, w, 1e-6)
+    check(y2, want, dt, "rmsnorm")
+    assert (y2.cpu() == want).float().mean().item() > 0.999
+
+
+def test_rmsnorm_double_and_fp32_and_ragged_dims(pkg):
+    for dt, n, rows in ((torch.float32, 256, 7), (torch.bfloat16, 5280, 3), (torch.bfloat16, 8, 2), (torch.float32, 4, 1),
+                        (torch.bfloat16, 8192, 2)):
+        x = rnd((rows, n), dt, 5)
+        w1, w2 = rnd((n,), dt, 6, 0.02, 1.0), rnd((n,), dt, 7, 0.02, 1.0)
+        y, _, y2 = pkg.hip.rmsnorm_residual(x.cuda(), w1.cuda(), 1e-6, weight2=w2.cuda())
+        want1 = O.rmsnorm(x, w1, 1e-6)
+        check(y, want1, dt, f"norm {dt} {n}")
+        check(y2, O.rmsnorm(want1, w2, 1e-6), dt, f"double norm {dt} {n}")
+    # closed form: constant rows
+    xc = torch.full((2, 5280), 3.0, dtype=torch.bfloat16)
+    y, _, _ = pkg.hip.rmsnorm_residual(xc.cuda(), torch.ones(5280, dtype=torch.bfloat16).cuda(), 1e-6)
+    assert torch.equal(y.cpu(), torch.ones(2, 5280, dtype=torch.bfloat16))
+    # empty input and bad sizes
+    e, _, _ = pkg.hip.rmsnorm_residual(torch.empty(0, 256, device="cuda"), torch.ones(256, device="cuda"), 1e-6)
+    assert e.shape == (0, 256)
+    with pytest.raises(pkg.hip.RavenHipError):
+        pkg.hip.rmsnorm_residual(torch.zeros(1, 6, device="cuda"), torch.ones(6, device="cuda"), 1e-6)
+
+
+# ----------------------------------------------------------------------------- skinny GEMMs
+def lin(x, w):
+    return F.linear(x.float(), w.float())
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 16, 17, 32, 33, 70])
+def test_gemm_bf16_all_row_counts(pkg, M):
+    dt, N, K = torch.bfloat16, 528, 1056
+    x, w = rnd((M, K), dt, 10 + M), rnd((N, K), dt, 20, 0.05)
+    res = rnd((M, N), dt, 30)
+    y = pkg.hip.gemm(x.cuda(), w.cuda())
+    check(y, lin(x, w).to(dt), dt, f"gemm M={M}")
+    yr = pkg.hip.gemm(x.cuda(), w.cuda(), residual=res.cuda())
+    check(yr, (lin(x, w).to(dt) + res), dt, f"gemm+residual M={M}")
+    yf = pkg.hip.gemm(x.cuda(), w.cuda(), out_f32=True)
+    assert yf.dtype == torch.float32
+    assert torch.equal(yf.cpu(), y.float().cpu()), "float store must be the upcast of the rounded result"
+
+
+@pytest.mark.parametrize("M", [1, 4, 8, 32])
+@pytest.mark.parametrize("N,K", [(5280, 5280), (15840, 5280), (5280, 17920)])
+def test_gemm_bf16_nebel_shapes(pkg, M, N, K):
+    dt = torch.bfloat16
+    x, w = rnd((M, K), dt, 40 + M), rnd((N, K), dt, 41, 0.02)
+    y = pkg.hip.gemm(x.cuda(), w.cuda())
+    check(y, lin(x, w).to(dt), dt, f"gemm {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 9, 40])
+def test_gemm_fp32_tiny_shapes(pkg, M):
+    dt = torch.float32
+    for N, K in ((768, 256), (256, 256), (256, 704), (1024, 256), (6, 4)):
+        x, w = rnd((M, K), dt, 50), rnd((N, K), dt, 51, 0.1)
+        check(pkg.hip.gemm(x.cuda(), w.cuda()), lin(x, w), dt, f"fp32 gemm {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("dt,M,h", [(torch.bfloat16, 1, 5280), (torch.bfloat16, 32, 5280), (torch.bfloat16, 6, 64),
+                                    (torch.float32, 1, 256), (torch.float32, 12, 256)])
+def test_adapter_concat(pkg, dt, M, h):
+    x0, x1 = rnd((M, h), dt, 60), rnd((M, h), dt, 61)
+    w = rnd((h, 2 * h), dt, 62, 0.02)
+    y = pkg.hip.adapter_gemm_concat(x0.cuda(), x1.cuda(), w.cuda())
+    want = lin(torch.cat([x0, x1], -1), w).to(dt)
+    check(y, want, dt, "adapter (state, embeds)")
+    swapped = lin(torch.cat([x1, x0], -1), w).to(dt)
+    assert close(y, swapped)[1] > 0.1, "operand order must matter"
+
+
+@pytest.mark.parametrize("dt,M,I,K", [(torch.bfloat16, 1, 17920, 5280), (torch.bfloat16, 32, 17920, 5280),
+                                      (torch.bfloat16, 8, 17920, 5280), (torch.bfloat16, 3, 176, 64),
+                                      (torch.float32, 1, 704, 256), (torch.float32, 20, 704, 256)])
+def test_gemm_swiglu(pkg, dt, M, I, K):
+    x, fc = rnd((M, K), dt, 70), rnd((2 * I, K), dt, 71, 0.03)
+    y = pkg.hip.gemm_swiglu(x.cuda(), fc.cuda())
+    z = lin(x, fc).to(dt)
+    gate, up = z[:, :I], z[:, I:]
+    want = F.silu(gate) * up
+    check(y, want, dt, "swiglu")
+    wrong = F.silu(up) * gate
+    assert close(y, wrong)[1] > 0.1, "the gate must be the first half"
+
+
+# ----------------------------------------------------------------------------- RoPE + cache append
+def make_cache(pkg, n_slots, B, nh, t_max, hd, dt, fill_seed=None):
+    if fill_seed is None:
+        k = torch.zeros(n_slots, B, nh, t_max, hd, dtype=dt)
+        v = torch.zeros_like(k)
+    else:
+        k, v = rnd((n_slots, B, nh, t_max, hd), dt, fill_seed), rnd((n_slots, B, nh, t_max, hd), dt, fill_seed + 1)
+    kd, vd = k.cuda(), v.cuda()
+    return k, v, kd, vd, pkg.hip.make_cache(kd, vd)
+
+
+@pytest.mark.parametrize("dt,nh,hd,B,S,pos0", [(torch.bfloat16, 55, 96, 1, 1, 1023), (torch.bfloat16, 55, 96, 4, 3, 7),
+                                               (torch.float32, 4, 64, 2, 5, 0), (torch.bfloat16, 2, 128, 1, 2, 3)])
+def test_qkv_bias_rope_cache_append(pkg, dt, nh, hd, B, S, pos0):
+    h, t_max, slot = nh * hd, 1024, 2
+    qkv = rnd((B * S, 3 * h), dt, 80)
+    bias = rnd((2, 1, nh, hd), dt, 81, 0.5)
+    table = O.rope_table(hd, t_max, 50000.0).to(dt)  # the table as a dtype-cast module holds it
+    freqs = table.float().reshape(t_max, hd // 2, 2).contiguous()
+    k0, v0, kd, vd, cache = make_cache(pkg, 4, B, nh, t_max, hd, dt, fill_seed=82)
+    q = pkg.hip.qkv_bias_rope_cache_append(qkv.cuda(), bias.cuda(), freqs.cuda(), cache, slot, B, S, pos0, nh, hd)
+    # oracle: the same lines of the attention function
+    qq, kk, vv = (t.view(B, S, nh, hd) for t in qkv.view(B, S, 3 * h).split([h, h, h], dim=2))
+    qq, kk = (qq + bias[0:1]).to(dt), (kk + bias[1:2]).to(dt)
+    rq, rk = O.apply_rope(qq, kk, table[:, pos0:pos0 + S])
+    check(q.view(B, S, nh, hd), rq, dt, "rotated q")
+    got_k = kd[slot, :, :, pos0:pos0 + S].cpu()
+    got_v = vd[slot, :, :, pos0:pos0 + S].cpu()
+    check(got_k, rk.transpose(1, 2), dt, "cached k")
+    assert torch.equal(got_v, vv.transpose(1, 2)), "v is copied unchanged"
+    assert (q.view(B, S, nh, hd).cpu() == rq).float().mean() > 0.995
+    # nothing outside the written window changed: indexing is bit-exact
+    kd2, vd2 = kd.cpu(), vd.cpu()
+    kd2[slot, :, :, pos0:pos0 + S] = k0[slot, :, :, pos0:pos0 + S]
+    vd2[slot, :, :, pos0:pos0 + S] = v0[slot, :, :, pos0:pos0 + S]
+    assert torch.equal(kd2, k0) and torch.equal(vd2, v0)
+    # negative slot indexes from the end; device-side position overrides the by-value one
+    pos_dev = torch.tensor([pos0], dtype=torch.int32, device="cuda")
+    pkg.hip.qkv_bias_rope_cache_append(qkv.cuda(), bias.cuda(), freqs.cuda(), cache, -1, B, S, t_max - S, nh, hd, pos_dev=pos_dev)
+    assert torch.equal(kd[3, :, :, pos0:pos0 + S].cpu(), got_k)
+    with pytest.raises(pkg.hip.RavenHipError):
+        pkg.hip.qkv_bias_rope_cache_append(qkv.cuda(), bias.cuda(), freqs.cuda(), cache, 4, B, S, pos0, nh, hd)
+    with pytest.raises(pkg.hip.RavenHipError):
+        pkg.hip.qkv_bias_rope_cache_append(qkv.cuda(), bias.cuda(), freqs.cuda(), cache, 0, B, S, t_max, nh, hd)
+
+
+# ----------------------------------------------------------------------------- decode attention
+@pytest.mark.parametrize("dt,nh,hd,B,S,pos0", [
+    (torch.bfloat16, 55, 96, 1, 1, 1023),   # config 3, bs=1: 1024 cached positions
+    (torch.bfloat16, 55, 96, 32, 1, 1023),  # config 3, bs=32 (no split)
+    (torch.bfloat16, 55, 96, 1, 1, 0),      # a single key: output equals v
+    (torch.bfloat16, 55, 96, 2, 1, 70),
+    (torch.bfloat16, 55, 96, 1, 6, 200),    # chunk of 6 queries, lower-right causal
+    (torch.float32, 4, 64, 1, 1, 11),
+    (torch.float32, 4, 64, 2, 8, 0),        # prefill from an empty cache: plain causal
+    (torch.bfloat16, 3, 128, 1, 1, 300),
+])
+def test_decode_attention(pkg, dt, nh, hd, B, S, pos0):
+    t_max = 1024
+    k, v, kd, vd, cache = make_cache(pkg, 2, B, nh, t_max, hd, dt, fill_seed=90)
+    q = rnd((B * S, nh * hd), dt, 92)
+    ws = pkg.hip.attention_workspace(B * S, nh, hd, "cuda")
+    y = pkg.hip.decode_attention(q.cuda(), cache, 1, B, S, pos0, nh, hd, ws)
+    T = pos0 + S
+    qq = q.view(B, S, nh, hd).transpose(1, 2)
+    want = O.sdpa(qq, k[1, :, :, :T], v[1, :, :, :T]).transpose(1, 2).reshape(B * S, nh * hd)
+    check(y, want, dt, f"attention B={B} S={S} T={T}")
+    lib = F.scaled_dot_product_attention(qq.float(), k[1, :, :, :T].float(), v[1, :, :, :T].float(),
+                                         attn_mask=None if S == 1 else torch.ones(S, T, dtype=torch.bool).tril(T - S))
+    check(y, lib.transpose(1, 2).reshape(B * S, nh * hd), dt, "attention vs torch SDPA")
+    if T == 1:
+        check(y.view(B, nh, hd), v[1, :, :, 0], dt, "T=1 returns v")
+    # second call reuses the workspace (arrival counters must have been left at zero), device position
+    pos_dev = torch.tensor([pos0], dtype=torch.int32, device="cuda")
+    y2 = pkg.hip.decode_attention(q.cuda(), cache, 1, B, S, t_max - S, nh, hd, ws, pos_dev=pos_dev)
+    check(y2, want, dt, "attention, device-side position")
+    assert int(ws[: B * S * nh * 4].view(torch.int32).abs().sum()) == 0
+
+
+def test_decode_attention_zero_query_gives_mean(pkg):
+    dt, nh, hd, T = torch.bfloat16, 55, 96, 513
+    k, v, kd, vd, cache = make_cache(pkg, 1, 1, nh, 1024, hd, dt, fill_seed=95)
+    ws = pkg.hip.attention_workspace(1, nh, hd, "cuda")
+    y = pkg.hip.decode_attention(torch.zeros(1, nh * hd, dtype=dt, device="cuda"), cache, 0, 1, 1, T - 1, nh, hd, ws)
+    check(y.view(nh, hd), v[0, 0, :, :T].float().mean(1), dt, "q=0 -> mean of V")
+
+
+# ----------------------------------------------------------------------------- embed / argmax
+def test_embed_and_argmax(pkg):
+    for dt in (torch.bfloat16, torch.float32):
+        wte = rnd((1000, 256), dt, 100, 0.02)
+        ids = torch.tensor([0, 999, 17, 17, 500])
+        got = pkg.hip.embed(wte.cuda(), ids.cuda(), 16.0)
+        assert torch.equal(got.cpu(), F.embedding(ids, wte) * 16.0)
+        got = pkg.hip.embed(wte.cuda(), ids.cuda(), math.sqrt(5280))
+        assert torch.equal(got.cpu(), F.embedding(ids, wte) * math.sqrt(5280))
+    logits = rnd((5, 65536), torch.float32, 101)
+    logits[1, 7] = logits[1, 60000] = 99.0      # tie: the first index wins
+    logits[2, 65535] = 100.0
+    logits[3] = -float("inf")
+    assert torch.equal(pkg.hip.argmax(logits.cuda()).cpu(), logits.argmax(-1))
+    small = rnd((3, 1024), torch.float32, 102)
+    assert torch.equal(pkg.hip.argmax(small.cuda()).cpu(), small.argmax(-1))

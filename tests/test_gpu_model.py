@@ -1,0 +1,236 @@
+"""GPU parity tests of the composed path: SandwichBlock, one recurrence iteration, the full forward and
+greedy decode, against the CPU oracle on identical seeded weights and injected latent states.
+
+Tolerances as in test_gpu_kernels.py (bf16: max-abs <= 2e-2 * max(1, |ref|_max), rel-L2 <= 1e-2);
+token ids and cache indexing bit-exact; fp32 greedy streams identical over 64 tokens."""
+
+import ctypes
+
+import pytest
+import torch
+
+from oracle import raven_oracle as O
+from test_gpu_kernels import check, close, rnd
+
+pytestmark = pytest.mark.gpu
+
+
+def build_model(pkg, shape_cfg, w, dtype):
+    model = pkg.RavenForCausalLM(shape_cfg, device="cuda:0", dtype=dtype)
+    model.load_state_dict(w, strict=True)
+    return model
+
+
+@pytest.fixture(scope="module")
+def tiny32(pkg):
+    s = O.RavenShape.tiny()
+    w = O.make_weights(s, seed=0, dtype=torch.float32)
+    return s, w, build_model(pkg, pkg.RavenConfig.tiny(), w, torch.float32)
+
+
+@pytest.fixture(scope="module")
+def tiny16(pkg):
+    s = O.RavenShape.tiny()
+    w = O.make_weights(s, seed=0, dtype=torch.bfloat16)
+    w["freqs_cis"] = w["freqs_cis"].to(torch.bfloat16)  # a dtype-cast module rounds its RoPE table too
+    return s, w, build_model(pkg, pkg.RavenConfig.tiny(), w, torch.bfloat16)
+
+
+def test_init_weights_equals_oracle_draw(pkg, tiny32):
+    s, w, _ = tiny32
+    m = pkg.RavenForCausalLM(pkg.RavenConfig.tiny(), device="cuda:0", dtype=torch.float32)
+    m.init_weights(seed=0)
+    sd = m.state_dict()
+    assert set(sd) == set(w)
+    for k in w:
+        assert torch.equal(sd[k].cpu(), w[k]), k
+    assert m.lm_head.weight.data_ptr() == m.transformer.wte.weight.data_ptr()
+
+
+@pytest.mark.parametrize("B,S", [(1, 8), (2, 5), (1, 1), (3, 40)])
+def test_forward_tiny_fp32_matches_oracle(tiny32, B, S):
+    s, w, model = tiny32
+    g = torch.Generator().manual_seed(B * 100 + S)
+    ids = torch.randint(0, s.vocab_size, (B, S), generator=g)
+    states = O.initialize_state(torch.empty(B, S, s.n_embd), s, 1.0, g)
+    want = O.forward(w, s, input_ids=ids, input_states=states)
+    got = model(input_ids=ids.cuda(), input_states=states.cuda())
+    check(got.logits, want.logits, torch.float32, "logits")
+    check(got.latent_states, want.latent_states, torch.float32, "latents")
+    assert got.logits.dtype == torch.float32 and got.logits.shape == (B, S, s.vocab_size)
+    assert torch.equal(got.logits.argmax(-1).cpu(), want.logits.argmax(-1))
+    for r in (0, 1, 3):
+        a = model(input_ids=ids.cuda(), input_states=states.cuda(), num_steps=r).logits
+        check(a, O.forward(w, s, input_ids=ids, input_states=states, num_steps=r).logits, torch.float32, f"r={r}")
+
+
+def test_forward_with_cache_prefill_then_decode_and_cache_contents(pkg, tiny32):
+    s, w, model = tiny32
+    g = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, s.vocab_size, (2, 7), generator=g)
+    states = O.initialize_state(torch.empty(2, 7, s.n_embd), s, 1.0, g)
+    ref_cache, cache = O.DictCache(), pkg.HuginnDynamicCache()
+    for lo, hi in ((0, 4), (4, 6), (6, 7)):  # prefill 4, a 2-token chunk (lower-right causal), one decode token
+        pos = torch.arange(lo, hi)
+        want = O.forward(w, s, input_ids=ids[:, lo:hi], input_states=states[:, lo:hi], past_key_values=ref_cache,
+                         use_cache=True, cache_position=pos)
+        got = model(input_ids=ids[:, lo:hi].cuda(), input_states=states[:, lo:hi].cuda(), past_key_values=cache,
+                    use_cache=True, cache_position=pos.cuda())
+        check(got.logits, want.logits, torch.float32, f"logits {lo}:{hi}")
+        assert got.past_key_values is cache and cache.get_seq_length() == ref_cache.get_seq_length() == hi
+    # indexing is bit-exact: same step keys in the same order, same positions under each
+    assert list(cache.key_cache) == list(ref_cache.key_cache) == O.step_indices(s)
+    for step in ref_cache.key_cache:
+        assert list(cache.key_cache[step].keys()) == sorted(ref_cache.key_cache[step]) == list(range(7))
+        for p in (0, 3, 4, 6):
+            check(cache.key_cache[step][p], ref_cache.key_cache[step][p], torch.float32, f"K[{step}][{p}]")
+            check(cache.value_cache[step][p], ref_cache.value_cache[step][p], torch.float32, f"V[{step}][{p}]")
+    assert cache.get_memory_usage() == ref_cache.get_memory_usage()
+    # the whole sequence in one no-cache call gives the same last logits
+    full = model(input_ids=ids.cuda(), input_states=states.cuda()).logits
+    check(full[:, -1], got.logits[:, -1], torch.float32, "cache vs no cache")
+    # roll back two tokens and redo them: same result, no overwrite assertion
+    cache.clear_last_k_entries(2)
+    ref_cache.clear_last_k_entries(2)
+    again = model(input_ids=ids[:, 5:7].cuda(), input_states=states[:, 5:7].cuda(), past_key_values=cache, use_cache=True,
+                  cache_position=torch.arange(5, 7).cuda())
+    check(again.logits[:, -1], got.logits[:, -1], torch.float32, "after clear_last_k_entries")
+    with pytest.raises(NotImplementedError):
+        model(input_ids=ids[:, :2].cuda(), past_key_values=cache, use_cache=True, cache_position=torch.arange(0, 2).cuda())
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_greedy_64_tokens_identical_fp32(tiny32, use_graph):
+    """Config 1: 8-token prompt, 64 greedy tokens, r=4, a CPU-drawn latent state injected into every forward."""
+    s, w, model = tiny32
+    prompt = torch.randint(0, s.vocab_size, (1, 8), generator=torch.Generator().manual_seed(0))
+
+    def state_fn(call, shape):
+        return O.initialize_state(torch.empty(shape), s, 1.0, torch.Generator().manual_seed(1000 + call))
+
+    rec = {}
+    want = O.greedy_generate(w, s, prompt, 64, state_fn=state_fn, record=rec)
+    got = model.generate(prompt.cuda(), max_new_tokens=64, input_states_fn=state_fn, stop_tokens=set(), use_graph=use_graph)
+    margin = min(m[0] for m in rec["margins"])
+    assert torch.equal(got.cpu(), want), f"token streams differ (smallest oracle top-2 margin {margin:.3e})"
+    assert got.shape == (1, 72)
+
+
+def test_greedy_batch_and_zero_state_and_stop(tiny32):
+    s, w, model = tiny32
+    prompt = torch.randint(0, s.vocab_size, (3, 5), generator=torch.Generator().manual_seed(9))
+    want = O.greedy_generate(w, s, prompt, 12)
+    got = model.generate(prompt.cuda(), max_new_tokens=12, init_scale=0.0, stop_tokens=set())
+    assert torch.equal(got.cpu(), want)
+    stop = int(want[0, 7])  # stop as soon as sequence 0 emits its 3rd token; the others keep going until all stopped
+    want_s = O.greedy_generate(w, s, prompt[:1], 12, stop_tokens={stop})
+    got_s = model.generate(prompt[:1].cuda(), max_new_tokens=12, init_scale=0.0, stop_tokens={stop})
+    assert torch.equal(got_s.cpu(), want_s) and got_s.shape[1] < 17
+
+
+def test_forward_tiny_bf16_matches_oracle(tiny16):
+    s, w, model = tiny16
+    g = torch.Generator().manual_seed(3)
+    ids = torch.randint(0, s.vocab_size, (2, 6), generator=g)
+    states = O.initialize_state(torch.empty(2, 6, s.n_embd), s, 1.0, g).to(torch.bfloat16)
+    want = O.forward(w, s, input_ids=ids, input_states=states)
+    got = model(input_ids=ids.cuda(), input_states=states.cuda())
+    check(got.latent_states, want.latent_states, torch.bfloat16, "bf16 latents")
+    check(got.logits, want.logits, torch.bfloat16, "bf16 logits")
+
+
+def test_piecewise_surface_equals_forward(tiny32):
+    """embed_inputs -> iterate_one_step x r -> predict_from_latents reproduces forward (RMM:841-934)."""
+    s, w, model = tiny32
+    g = torch.Generator().manual_seed(21)
+    ids = torch.randint(0, s.vocab_size, (2, 4), generator=g).cuda()
+    states = O.initialize_state(torch.empty(2, 4, s.n_embd), s, 1.0, g).cuda()
+    ref = model(input_ids=ids, input_states=states)
+    emb, block_idx = model.embed_inputs(ids)
+    assert int(block_idx) == 0
+    x, step = states, 0
+    for _ in range(s.mean_recurrence):
+        x, block_idx, step = model.iterate_one_step(emb, x, block_idx=block_idx, current_step=step)
+    assert int(block_idx) == 8 and step == 4
+    out = model.predict_from_latents(x)
+    check(out.logits, ref.logits, torch.float32, "piecewise logits")
+    y, n0, n1, _, bi = model.iterate_forward(emb, states, block_idx=torch.tensor(0), num_steps=4)
+    check(y, ref.latent_states, torch.float32, "iterate_forward latents")
+    assert (n0, n1, int(bi)) == (4, 0, 8)
+    # the same pieces through a cache, one decode token after a prefill
+    cache = model(input_ids=ids, input_states=states, use_cache=True).past_key_values
+    tok = torch.randint(0, s.vocab_size, (2, 1), generator=g).cuda()
+    st1 = O.initialize_state(torch.empty(2, 1, s.n_embd), s, 1.0, g).cuda()
+    emb1, bi = model.embed_inputs(tok, past_key_values=cache, use_cache=True, cache_position=torch.tensor([4]).cuda())
+    x = st1
+    for _ in range(s.mean_recurrence):
+        x, bi, _ = model.iterate_one_step(emb1, x, block_idx=bi, past_key_values=cache)
+    got = model.predict_from_latents(x, past_key_values=cache).logits
+    cache2 = model(input_ids=ids, input_states=states, use_cache=True).past_key_values
+    want = model(input_ids=tok, input_states=st1, past_key_values=cache2, use_cache=True, cache_position=torch.tensor([4]).cuda()).logits
+    check(got, want, torch.float32, "piecewise decode logits")
+
+
+# ----------------------------------------------------------------------------- nebel shape (config 3)
+@pytest.fixture(scope="module")
+def nebel_core(pkg):
+    s = O.RavenShape.nebel()
+    w = O.make_weights(s, seed=0, dtype=torch.bfloat16, only_core=True)
+    dev = {k: v.cuda() for k, v in w.items()}
+    return s, w, dev
+
+
+def _block_weights(pkg, dev, prefix):
+    return pkg.hip.make_block_weights(
+        dev[f"{prefix}.norm_1.weight"], dev[f"{prefix}.norm_2.weight"], dev[f"{prefix}.norm_3.weight"], dev[f"{prefix}.norm_4.weight"],
+        dev[f"{prefix}.attn.Wqkv.weight"], dev[f"{prefix}.attn.qk_bias"], dev[f"{prefix}.attn.proj.weight"],
+        dev[f"{prefix}.mlp.fc.weight"], dev[f"{prefix}.mlp.proj.weight"])
+
+
+@pytest.mark.parametrize("B", [1, 32])
+def test_core_iteration_nebel_bf16_config3(pkg, nebel_core, B):
+    """One recurrence iteration at decode, 1024 cached positions per step slot filled with N(0,1)."""
+    s, w, dev = nebel_core
+    dt, h, nh, hd, T = torch.bfloat16, s.n_embd, s.n_heads, s.head_dim, 1024
+    t_max = T + 1
+    kc, vc = rnd((4, B, nh, t_max, hd), dt, 200 + B), rnd((4, B, nh, t_max, hd), dt, 300 + B)
+    kd, vd = kc.cuda(), vc.cuda()
+    cache = pkg.hip.make_cache(kd, vd)
+    g = torch.Generator().manual_seed(B)
+    state = O.initialize_state(torch.empty(B, 1, h), s, 1.0, g).to(dt)
+    embeds = (torch.randn(B, 1, h, generator=g)).to(dt)
+    table = O.rope_table(hd, s.block_size, s.rope_base).to(dt)
+    freqs = table.float().reshape(s.block_size, hd // 2, 2).contiguous().cuda()
+    # oracle: a dict cache holding the same 1024 positions for core steps 2..5
+    ref_cache = O.DictCache()
+    ref_cache._seen_tokens = T + 1
+    for j in range(4):
+        ref_cache.key_cache[2 + j] = {p: kc[j, :, :, p] for p in range(T)}
+        ref_cache.value_cache[2 + j] = {p: vc[j, :, :, p] for p in range(T)}
+    ww = dict(w)
+    want, idx = O.core_block_forward(state, embeds, ww, table[:, T:T + 1], ref_cache, 1, s)
+    assert idx == 5
+    dims = pkg.hip.make_dims(h, nh, s.intermediate_size, s.norm_eps, dt)
+    blocks = (pkg.hip.BlockWeights * 4)(*[_block_weights(pkg, dev, f"transformer.core_block.{j}") for j in range(4)])
+    ws = pkg.hip.block_workspace(dims, B, "cuda")
+    out = torch.empty(B, h, dtype=dt, device="cuda")
+    pkg.hip.core_iteration(dims, dev["transformer.adapter.weight"], blocks, state.view(B, h).cuda(), embeds.view(B, h).cuda(), out,
+                           freqs, cache, 0, B, 1, T, ws)
+    check(out, want.view(B, h), dt, f"core iteration B={B}")
+    for j in range(4):  # the new key/value rows landed at position T of each slot
+        check(kd[j, :, :, T], ref_cache.key_cache[2 + j][T], dt, f"appended K slot {j}")
+        check(vd[j, :, :, T], ref_cache.value_cache[2 + j][T], dt, f"appended V slot {j}")
+    assert torch.equal(kd[:, :, :, :T].cpu(), kc[:, :, :, :T]), "cached positions must be untouched"
+    # a single SandwichBlock with the closing ln_f folded in
+    x_in = rnd((B, h), dt, 77)
+    lnw = rnd((h,), dt, 78, 0.02, 1.0)
+    kd2, vd2 = kc.cuda(), vc.cuda()
+    cache2 = pkg.hip.make_cache(kd2, vd2)
+    got = pkg.hip.sandwich_block(dims, blocks[1], x_in.cuda(), torch.empty(B, h, dtype=dt, device="cuda"), freqs, cache2, 1, B, 1, T, ws,
+                                 ln_f=lnw.cuda())
+    rc = O.DictCache()
+    rc._seen_tokens = T + 1
+    rc.key_cache[3] = {p: kc[1, :, :, p] for p in range(T)}
+    rc.value_cache[3] = {p: vc[1, :, :, p] for p in range(T)}
+    wb = O.sandwich_block(x_in.view(B, 1, h), ww, "transformer.core_block.1", table[:, T:T + 1], 3, rc, s)
+    check(got, O.rmsnorm(wb, lnw, s.norm_eps).view(B, h), dt, "block + ln_f")

@@ -1,0 +1,136 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the header declares, and the
+host logic (config, cache bookkeeping, step remaps) agrees with the oracle's brute-force model.
+No kernel is launched here."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from oracle import raven_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "raven_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(raven_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    assert os.path.exists(pkg.hip.LIB_PATH), "libraven_hip.so has not been built"
+    lib = ctypes.CDLL(pkg.hip.LIB_PATH)
+    names = _declared_functions()
+    assert len(names) >= 16
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in raven_hip.h but not exported"
+    assert sorted(pkg.hip.SIGNATURES) == names, "the ctypes table and the header disagree"
+
+
+def test_library_identity_and_argument_errors(pkg):
+    lib = pkg.hip.load()
+    assert lib.raven_version() >= 1 and lib.raven_arch() == b"gfx950"
+    # argument validation happens before any launch, so it can be exercised without a GPU
+    rc = lib.raven_rmsnorm_residual(None, None, None, None, None, None, None, 1, 5280, 1e-6, 1, None)
+    assert rc < 0 and b"null" in lib.raven_last_error()
+    rc = lib.raven_gemm(1, 1, None, 1, 1, 16, 7, 1, 0, None)
+    assert rc < 0 and b"multiple" in lib.raven_last_error()
+    rc = lib.raven_rmsnorm_residual(1, None, 1, 1, None, None, None, 1, 5280, 1e-6, 7, None)
+    assert rc < 0 and b"dtype" in lib.raven_last_error()
+    assert lib.raven_decode_attention_workspace_bytes(1, 55, 96) > 0
+    dims = pkg.hip.make_dims(5280, 55, 17920, 1e-6, torch.bfloat16)
+    n1 = lib.raven_block_workspace_bytes(ctypes.byref(dims), 1)
+    n32 = lib.raven_block_workspace_bytes(ctypes.byref(dims), 32)
+    assert 0 < n1 < n32 and n1 % 256 == 0
+
+
+def test_wrappers_refuse_cpu_tensors(pkg):
+    x = torch.zeros(1, 16)
+    with pytest.raises(pkg.hip.RavenHipError, match="GPU"):
+        pkg.hip.rmsnorm_residual(x, torch.ones(16), 1e-6)
+
+
+def test_config_matches_reference_defaults_and_oracle(pkg):
+    cfg = pkg.RavenConfig()
+    s = O.RavenShape.nebel()
+    assert (cfg.n_embd, cfg.n_heads, cfg.head_dim, cfg.intermediate_size, cfg.vocab_size) == (5280, 55, 96, 17920, 65536)
+    assert cfg.effective_expected_depth == 132 and cfg.mean_recurrence == 32
+    assert cfg.init_values["std"] == pytest.approx(s.init_std) and cfg.init_values["embed_scale"] == pytest.approx(s.emb_scale)
+    t = pkg.RavenConfig.tiny()
+    assert (t.n_embd, t.head_dim, t.n_layers_in_recurrent_block, t.mean_recurrence) == (256, 64, 2, 4)
+    assert pkg.RavenConfig(**cfg.to_dict()).to_dict() == cfg.to_dict()
+    with pytest.raises(ValueError):
+        pkg.RavenConfig(n_embd=100, n_heads=3)
+
+
+def test_remap_agrees_with_oracle(pkg):
+    for strat in ("full", "latest-m4-compress-s4", "compress-s16", "compress-r4", "compress-anchor"):
+        for step in list(range(0, 132)) + [-1, -2]:
+            assert pkg.remap_step(step, strat) == O.remap_step(step, strat)
+
+
+def test_rope_table_matches_oracle(pkg):
+    assert torch.equal(pkg.precompute_freqs_cis(96, 512, 50000.0), O.rope_table(96, 512, 50000.0))
+
+
+def test_cache_update_against_dict_model_on_cpu(pkg):
+    """The contiguous cache driven through the reference's update() interface returns bit-identical
+    K/V and the same bookkeeping as the brute-force dict model."""
+    rng = torch.Generator().manual_seed(11)
+    mine, ref = pkg.HuginnDynamicCache(), O.DictCache()
+    for n_new in (5, 1, 1, 3):
+        for step in (0, 1, 2, 3, -1, -2):
+            k = torch.randn(2, 3, n_new, 8, generator=rng)
+            v = torch.randn(2, 3, n_new, 8, generator=rng)
+            gk, gv = mine.update(k, v, torch.tensor(step))
+            wk, wv = ref.update(k, v, torch.tensor(step))
+            assert torch.equal(gk, wk) and torch.equal(gv, wv)
+            assert mine.get_seq_length() == ref.get_seq_length()
+    assert list(mine.key_cache) == list(ref.key_cache)  # same step keys, same first-touch order
+    for step in ref.key_cache:
+        assert sorted(mine.key_cache[step].keys()) == sorted(ref.key_cache[step])
+        for pos, t in ref.key_cache[step].items():
+            assert torch.equal(mine.key_cache[step][pos], t)
+            assert torch.equal(mine.value_cache[step][pos], ref.value_cache[step][pos])
+    assert mine.get_memory_usage() == ref.get_memory_usage()
+    mine.clear_last_k_entries(4)
+    ref.clear_last_k_entries(4)
+    assert mine.get_seq_length() == ref.get_seq_length() == 6
+    assert all(len(mine.key_cache[s]) == len(ref.key_cache[s]) for s in ref.key_cache)
+    with pytest.raises(AssertionError):
+        mine.update(torch.zeros(2, 3, 1, 8), torch.zeros(2, 3, 1, 8), 2)  # overwrite of position 5 at a non-coda step
+    mine.reset()
+    assert mine.get_seq_length() == 0 and len(mine.key_cache) == 0
+
+
+def test_cache_growth_keeps_contents_and_slot_order(pkg):
+    c = pkg.HuginnDynamicCache()
+    k = torch.arange(2 * 2 * 300 * 4, dtype=torch.float32).view(2, 2, 300, 4)
+    c.update(k, -k, 0)
+    c.update(k + 1, -k - 1, -1)
+    assert c.t_max == 512
+    c.update(k[:, :, :250], k[:, :, :250], 0)      # 550 tokens: storage doubles
+    c.update(k[:, :, :250] + 1, k[:, :, :250], -1)
+    c.update(k[:, :, :1], k[:, :, :1], 7)          # a new, higher step: slots are appended
+    assert c.t_max == 1024 and c.get_seq_length() == 550
+    assert torch.equal(c.key_cache[0][299], k[:, :, 299]) and torch.equal(c.key_cache[-1][0], k[:, :, 0] + 1)
+    assert torch.equal(c.key_cache[0][300], k[:, :, 0]) and torch.equal(c.value_cache[-1][549], k[:, :, 249])
+    fixed = pkg.HuginnDynamicCache(max_length=8)
+    fixed.update(torch.zeros(1, 1, 8, 4), torch.zeros(1, 1, 8, 4), 0)
+    with pytest.raises(ValueError, match="max_length"):
+        fixed.update(torch.zeros(1, 1, 1, 4), torch.zeros(1, 1, 1, 4), 0)
+
+
+def test_cache_size_known_answers(pkg):
+    """The reference notebooks' cache sizes (examples/inference_demo.ipynb:252, 373) from the
+    contiguous cache's own accounting."""
+    s = O.RavenShape.nebel()
+    for strat, want in (("full", 973.0810546875), ("latest-m4-compress-s16", 147.4365234375)):
+        c = pkg.HuginnDynamicCache(strat)
+        c._k = torch.empty(1, 1, s.n_heads, 1, s.head_dim, dtype=torch.bfloat16)  # shape carrier only
+        for step in O.step_indices(s):
+            c.note_append(step, 366, 0)
+        assert c.get_memory_usage() == want
