@@ -15,9 +15,7 @@
  *     by-value argument, so a captured HIP graph can be replayed as the sequence grows; the by-value
  *     `pos0` then only sizes grids and must be >= the largest value *pos_dev will take.
  *   - return value: 0 ok; < 0 invalid argument (see raven_last_error()); > 0 a hipError_t.
- *   - workspaces must be 256-byte aligned.  The attention workspace must be zero-filled once before
- *     its first use (it holds arrival counters that every call leaves at zero again).
- *   - calls that share a workspace must be ordered on one stream.
+ *   - workspaces must be 256-byte aligned; calls that share a workspace must be ordered on one stream.
  */
 #ifndef RAVEN_HIP_H
 #define RAVEN_HIP_H
@@ -112,11 +110,17 @@ int raven_qkv_bias_rope_cache_append(const void* qkv, const void* qk_bias, const
  * (RMM:481-491).  Row m attends to positions 0 .. pos0 + (m % S) inclusive: for S == 1 this is the
  * unmasked decode case, for S > 1 the lower-right-aligned causal case.  The new keys/values must
  * already be in the cache.  q [M, h]; y [M, h] in the layout y.transpose(1,2).reshape(B,S,h) has. */
-size_t raven_decode_attention_workspace_bytes(int32_t M, int32_t n_heads, int32_t head_dim);
-int    raven_decode_attention(const void* q, void* y, const raven_kv_cache* cache, int32_t slot,
-                              int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
-                              int32_t n_heads, int32_t head_dim, int32_t dtype,
-                              void* workspace, size_t workspace_bytes, void* stream);
+int raven_decode_attention(const void* q, void* y, const raven_kv_cache* cache, int32_t slot,
+                           int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
+                           int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream);
+
+/* Decode step (S == 1) of RMM:463-491 in one launch: takes the fused qkv GEMM output [B, 3h], adds
+ * the q/k bias, rotates q and k for position pos0, writes the new k and v rows into the cache slot
+ * and returns softmax(q K^T / sqrt(hd)) V over positions 0 .. pos0 in y [B, h]. */
+int raven_qkv_attention_decode(const void* qkv, const void* qk_bias, const float* freqs, void* y,
+                               const raven_kv_cache* cache, int32_t slot, int32_t B, int32_t pos0,
+                               const int32_t* pos_dev, int32_t n_heads, int32_t head_dim,
+                               int32_t dtype, void* stream);
 
 /* Token embedding times sqrt(h) (RMM:667-671): out[m] = T(wte[ids[m]] * scale); ids are int64. */
 int raven_embed(const void* wte, const int64_t* ids, void* out, int32_t M, int32_t dim,

@@ -143,6 +143,25 @@ def make_weights(s: RavenShape, seed: int = 0, dtype=torch.float32, only_core: b
 # --------------------------------------------------------------------------------------
 # elementary ops
 # --------------------------------------------------------------------------------------
+LINEAR_MODE = "native"
+
+
+def set_linear_mode(mode: str) -> None:
+    """'native': nn.Linear semantics in the tensor's own dtype, what the reference executes.
+    'f32': upcast both operands, multiply in fp32, round once to the input dtype -- the same
+    mathematics with another accumulation order; the distance between the two modes is the
+    accumulation-order sensitivity that composed bf16 results are judged against."""
+    global LINEAR_MODE
+    assert mode in ("native", "f32")
+    LINEAR_MODE = mode
+
+
+def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    if LINEAR_MODE == "f32" and x.dtype != torch.float32:
+        return F.linear(x.float(), w.float()).to(x.dtype)
+    return F.linear(x, w)
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """RMM:137-142.  Normalise in fp32, cast to x's dtype, THEN scale by the weight in that dtype."""
     x32 = x.float()
@@ -275,7 +294,7 @@ def attention(x, w, prefix, freqs, step_idx, cache, s: RavenShape):
     """CausalSelfAttention.forward, RMM:454-493.  x [B,S,h] is the already-normalised input."""
     b, sq, h = x.shape
     nh, hd = s.n_heads, s.head_dim
-    qkv = F.linear(x, w[f"{prefix}.attn.Wqkv.weight"])
+    qkv = linear(x, w[f"{prefix}.attn.Wqkv.weight"])
     q, k, v = (t.view(b, sq, nh, hd) for t in qkv.split([h, h, h], dim=2))
     if s.qk_bias:
         bias = w[f"{prefix}.attn.qk_bias"]
@@ -286,13 +305,13 @@ def attention(x, w, prefix, freqs, step_idx, cache, s: RavenShape):
         k, v = cache.update(k, v, step_idx)
     y = sdpa(q, k, v)
     y = y.transpose(1, 2).reshape(b, sq, h)
-    return F.linear(y, w[f"{prefix}.attn.proj.weight"])
+    return linear(y, w[f"{prefix}.attn.proj.weight"])
 
 
 def gated_mlp(x, w, prefix):
     """GatedMLP.forward, RMM:505-509.  The gate is the FIRST half of fc's output."""
-    gate, up = F.linear(x, w[f"{prefix}.mlp.fc.weight"]).chunk(2, dim=-1)
-    return F.linear(F.silu(gate) * up, w[f"{prefix}.mlp.proj.weight"])
+    gate, up = linear(x, w[f"{prefix}.mlp.fc.weight"]).chunk(2, dim=-1)
+    return linear(F.silu(gate) * up, w[f"{prefix}.mlp.proj.weight"])
 
 
 def sandwich_block(x, w, prefix, freqs, step_idx, cache, s: RavenShape):
@@ -306,7 +325,7 @@ def sandwich_block(x, w, prefix, freqs, step_idx, cache, s: RavenShape):
 
 def core_block_forward(x, embeds, w, freqs, cache, block_idx: int, s: RavenShape):
     """RMM:764-781 with test_time_noise == 0.  Adapter input order is (state, embedded input)."""
-    x = F.linear(torch.cat([x, embeds], dim=-1), w["transformer.adapter.weight"])
+    x = linear(torch.cat([x, embeds], dim=-1), w["transformer.adapter.weight"])
     for j in range(s.n_layers_in_recurrent_block):
         block_idx += 1
         x = sandwich_block(x, w, f"transformer.core_block.{j}", freqs, block_idx, cache, s)
@@ -388,7 +407,7 @@ def forward(w, s: RavenShape, input_ids=None, input_embeds=None, input_states=No
         block_idx -= 1
         x = sandwich_block(x, w, f"transformer.coda.{i}", freqs, block_idx, cache, s)
     x = rmsnorm(x, w["transformer.ln_f.weight"], s.norm_eps)
-    logits = F.linear(x, w["lm_head.weight"]).float()
+    logits = linear(x, w["lm_head.weight"]).float()
     return OracleOutput(logits=logits, latent_states=latents, past_key_values=cache, hidden_states=x)
 
 

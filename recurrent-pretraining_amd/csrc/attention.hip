@@ -4,13 +4,13 @@
 // K, V = [n_slots, batch, n_heads, t_max, head_dim]; one head's positions are contiguous, so a
 // workgroup streams [positions x head_dim] with 16-byte lane-contiguous loads.
 //
-// Attention kernel: grid (splits, heads, token rows).  A position occupies one row of 16 lanes
+// Attention kernel: grid (heads, token rows).  A position occupies one row of 16 lanes
 // (head_dim * sizeof(T) / 16 of them active, 12 for head_dim 96 in bf16); a wave covers 4 positions
-// per load instruction and the 4 waves of a workgroup interleave, so each iteration of a
-// workgroup reads 16 consecutive positions of K and of V.  Scores are reduced with DPP row
-// operations; every 16-lane row runs its own online softmax and the rows are merged through LDS.
-// With more than one split the partial (max, sum, unnormalised output) triples go to a workspace and
-// the last workgroup to arrive for a (row, head) merges them (arrival counter + __threadfence).
+// per load instruction and the waves of a workgroup interleave, so each load step of a workgroup
+// reads 16 or 64 consecutive positions of K and of V.  Scores are reduced with DPP row operations;
+// every 16-lane row runs its own online softmax (one max update per 4 positions) and the rows are
+// merged through LDS.  Nothing is exchanged between workgroups: a split over positions with a
+// device-scope fence per workgroup measured 10x slower than one 16-wave workgroup per head.
 
 #include <math.h>
 
@@ -68,25 +68,49 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
-constexpr int kAttnMaxSplits = 32;
 constexpr int kAttnMaxHd = 128;
+constexpr int kAttnU = 4;  // positions per 16-lane row and loop iteration
 
+// bias + RoPE of one 16-byte chunk of a q or k head row (sec 0 = q, 1 = k); d = first column of the chunk
 template <typename T>
-__global__ __launch_bounds__(256) void decode_attention_kernel(
-    const T* __restrict__ q, T* __restrict__ y, CacheView cv, int S, int pos0, const int* __restrict__ pos_dev,
-    int n_splits, float scale_log2, int* __restrict__ counters, float* __restrict__ ws_ml, float* __restrict__ ws_o) {
+__device__ __forceinline__ Chunk<T> bias_rope_chunk(Chunk<T> x, const T* __restrict__ qk_bias, int sec, int h, int col,
+                                                    const float* __restrict__ freqs, int pos, int hd, int d) {
     constexpr int E = Chunk<T>::N;
-    __shared__ float sm_m[16], sm_l[16];
-    __shared__ float sm_o[16][kAttnMaxHd];
-    __shared__ int sm_ticket;
+    if (qk_bias) {
+        const Chunk<T> bch = load_chunk(qk_bias + sec * h + col);
+#pragma unroll
+        for (int e = 0; e < E; ++e) x.v[e] = from_f32<T>(to_f32(x.v[e]) + to_f32(bch.v[e]));
+    }
+    const float* f = freqs + ((int64_t)pos * (hd / 2) + d / 2) * 2;
+#pragma unroll
+    for (int e = 0; e < E; e += 2) {
+        const float cs = f[e], sn = f[e + 1];
+        const float x0 = to_f32(x.v[e]), x1 = to_f32(x.v[e + 1]);
+        x.v[e] = from_f32<T>(x0 * cs - x1 * sn);
+        x.v[e + 1] = from_f32<T>(x1 * cs + x0 * sn);
+    }
+    return x;
+}
 
-    const int split = blockIdx.x, head = blockIdx.y, m = blockIdx.z;
+// One workgroup per (head, token row): no split over positions, so nothing crosses workgroups.
+// WAVES = 16 when there are few (head, row) pairs (a CU then keeps 16 waves of loads in flight for its
+// head), 4 otherwise.  FUSED (decode, S == 1): q, and the new position's k and v, come straight from the
+// fused qkv GEMM output -- bias and RoPE are applied here, the new k/v row is written to the cache by
+// this workgroup and used from registers.
+template <typename T, int WAVES, bool FUSED>
+__global__ __launch_bounds__(WAVES * 64) void decode_attention_kernel(
+    const T* __restrict__ q_or_qkv, const T* __restrict__ qk_bias, const float* __restrict__ freqs, T* __restrict__ y,
+    CacheView cv, int S, int pos0, const int* __restrict__ pos_dev, float scale_log2) {
+    constexpr int E = Chunk<T>::N;
+    constexpr int G = WAVES * 4;  // 16-lane rows in the workgroup
+    __shared__ float sm_m[G], sm_l[G];
+    __shared__ float sm_o[G][kAttnMaxHd];
+
+    const int head = blockIdx.x, m = blockIdx.y;
     const int hd = cv.hd, h = cv.nh * hd;
     const int b = m / S, s = m - b * S;
-    int len = (pos_dev ? *pos_dev : pos0) + s + 1;
-    len = min(len, cv.t_max);
-    const int per = (len + n_splits - 1) / n_splits;
-    const int start = split * per, end = min(len, start + per);
+    const int pos = (pos_dev ? *pos_dev : pos0) + s;  // position of this row's own token
+    const int len = min(pos + 1, cv.t_max);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane >> 4, ci = lane & 15;
@@ -98,21 +122,36 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
     const T* Kb = static_cast<const T*>(cv.k) + head_off + ci * E;
     const T* Vb = static_cast<const T*>(cv.v) + head_off + ci * E;
 
-    Chunk<T> qc = zero_chunk<T>();
-    if (active) qc = load_chunk(q + (int64_t)m * h + head * hd + ci * E);
+    Chunk<T> qc = zero_chunk<T>(), knew = zero_chunk<T>(), vnew = zero_chunk<T>();
+    if (active) {
+        const int col = head * hd + ci * E;
+        if (FUSED) {
+            const T* row = q_or_qkv + (int64_t)m * 3 * h;
+            qc = bias_rope_chunk<T>(load_chunk(row + col), qk_bias, 0, h, col, freqs, pos, hd, ci * E);
+            knew = bias_rope_chunk<T>(load_chunk(row + h + col), qk_bias, 1, h, col, freqs, pos, hd, ci * E);
+            vnew = load_chunk(row + 2 * h + col);
+            if (group == 0 && pos < cv.t_max) {
+                store_chunk(static_cast<T*>(cv.k) + head_off + (int64_t)pos * hd + ci * E, knew);
+                store_chunk(static_cast<T*>(cv.v) + head_off + (int64_t)pos * hd + ci * E, vnew);
+            }
+        } else {
+            qc = load_chunk(q_or_qkv + (int64_t)m * h + col);
+        }
+    }
 
     float m_run = -INFINITY, l_run = 0.f, o[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) o[e] = 0.f;
 
-    constexpr int U = 2;
-    for (int base = start; base < end; base += 16 * U) {  // trip count is uniform over the workgroup
-        const int p0 = base + group;
-        Chunk<T> kc[U], vc[U];
+    for (int base = 0; base < len; base += G * kAttnU) {  // trip count is uniform over the workgroup
+        Chunk<T> kc[kAttnU], vc[kAttnU];
 #pragma unroll
-        for (int j = 0; j < U; ++j) {
-            const int p = p0 + 16 * j;
-            if (active && p < end) {
+        for (int j = 0; j < kAttnU; ++j) {
+            const int p = base + j * G + group;
+            if (FUSED && p == pos) {
+                kc[j] = knew;
+                vc[j] = vnew;
+            } else if (active && p < len) {
                 kc[j] = load_chunk(Kb + (int64_t)p * hd);
                 vc[j] = load_chunk(Vb + (int64_t)p * hd);
             } else {
@@ -120,23 +159,34 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
                 vc[j] = zero_chunk<T>();
             }
         }
+        float sc[kAttnU], m_new = m_run;
 #pragma unroll
-        for (int j = 0; j < U; ++j) {
-            const int p = p0 + 16 * j;
-            float sc = row16_sum(dot_chunk(qc, kc[j], 0.f)) * scale_log2;
-            if (p < end) {
-                const float m_new = fmaxf(m_run, sc);
-                const float corr = exp2f(m_run - m_new);
-                const float pe = exp2f(sc - m_new);
-                l_run = l_run * corr + pe;
-#pragma unroll
-                for (int e = 0; e < E; ++e) o[e] = o[e] * corr + pe * to_f32(vc[j].v[e]);
-                m_run = m_new;
-            }
+        for (int j = 0; j < kAttnU; ++j) {
+            const int p = base + j * G + group;
+            sc[j] = row16_sum(dot_chunk(qc, kc[j], 0.f)) * scale_log2;
+            if (p >= len) sc[j] = -INFINITY;
+            m_new = fmaxf(m_new, sc[j]);
         }
+        if (m_new == -INFINITY) continue;  // this row has not seen a valid position yet
+        const float corr = exp2f(m_run - m_new);
+        float pe[kAttnU], psum = 0.f;
+#pragma unroll
+        for (int j = 0; j < kAttnU; ++j) {
+            pe[j] = exp2f(sc[j] - m_new);
+            psum += pe[j];
+        }
+        l_run = l_run * corr + psum;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float acc = o[e] * corr;
+#pragma unroll
+            for (int j = 0; j < kAttnU; ++j) acc = __builtin_fmaf(pe[j], to_f32(vc[j].v[e]), acc);
+            o[e] = acc;
+        }
+        m_run = m_new;
     }
 
-    // merge the 16 row groups of the workgroup
+    // merge the G rows of the workgroup
     if (ci == 0) {
         sm_m[group] = m_run;
         sm_l[group] = l_run;
@@ -147,56 +197,18 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
     }
     __syncthreads();
     const int t = threadIdx.x;
-    float M = -INFINITY, L = 0.f, O = 0.f;
     if (t < hd) {
-#pragma unroll
-        for (int g = 0; g < 16; ++g) M = fmaxf(M, sm_m[g]);
-#pragma unroll
-        for (int g = 0; g < 16; ++g) {
+        float M = -INFINITY, L = 0.f, O = 0.f;
+#pragma unroll 8
+        for (int g = 0; g < G; ++g) M = fmaxf(M, sm_m[g]);
+#pragma unroll 8
+        for (int g = 0; g < G; ++g) {
             const float wgt = (sm_m[g] == -INFINITY) ? 0.f : exp2f(sm_m[g] - M);
             L += sm_l[g] * wgt;
             O += sm_o[g][t] * wgt;
         }
+        y[(int64_t)m * h + head * hd + t] = from_f32<T>(O / L);
     }
-    if (n_splits == 1) {
-        if (t < hd) y[(int64_t)m * h + head * hd + t] = from_f32<T>(O / L);
-        return;
-    }
-
-    const int64_t mh = (int64_t)m * cv.nh + head;
-    if (t < hd) {
-        ws_o[(mh * n_splits + split) * hd + t] = O;
-        if (t == 0) {
-            ws_ml[(mh * n_splits + split) * 2] = M;
-            ws_ml[(mh * n_splits + split) * 2 + 1] = L;
-        }
-    }
-    __threadfence();
-    __syncthreads();
-    if (t == 0) sm_ticket = atomicAdd(&counters[mh], 1);
-    __syncthreads();
-    if (sm_ticket != n_splits - 1) return;
-    __threadfence();
-    if (t == 0) counters[mh] = 0;  // leave the counter ready for the next call
-    if (t < hd) {
-        float Mg = -INFINITY;
-        for (int sp = 0; sp < n_splits; ++sp) Mg = fmaxf(Mg, ws_ml[(mh * n_splits + sp) * 2]);
-        float Lg = 0.f, Og = 0.f;
-        for (int sp = 0; sp < n_splits; ++sp) {
-            const float ms = ws_ml[(mh * n_splits + sp) * 2];
-            const float wgt = (ms == -INFINITY) ? 0.f : exp2f(ms - Mg);
-            Lg += ws_ml[(mh * n_splits + sp) * 2 + 1] * wgt;
-            Og += ws_o[(mh * n_splits + sp) * hd + t] * wgt;
-        }
-        y[(int64_t)m * h + head * hd + t] = from_f32<T>(Og / Lg);
-    }
-}
-
-static int max_splits_for(int M, int nh) {
-    int ns = (1024 + nh * M - 1) / (nh * M);
-    if (ns < 1) ns = 1;
-    if (ns > kAttnMaxSplits) ns = kAttnMaxSplits;
-    return ns;
 }
 
 static int make_view(const char* who, const raven_kv_cache* cache, int slot, int B, int nh, int hd, CacheView* cv) {
@@ -247,50 +259,52 @@ extern "C" int raven_qkv_bias_rope_cache_append(const void* qkv, const void* qk_
     return raven_host::check_launch("qkv_append");
 }
 
-extern "C" size_t raven_decode_attention_workspace_bytes(int32_t M, int32_t n_heads, int32_t head_dim) {
+template <typename T>
+static void launch_attention(bool fused, const void* q, const void* bias, const float* freqs, void* y, const raven::CacheView& cv,
+                             int S, int M, int pos0, const int32_t* pos_dev, float scale_log2, hipStream_t s) {
     using namespace raven;
-    if (M <= 0 || n_heads <= 0 || head_dim <= 0) return 0;
-    const size_t ns = (size_t)max_splits_for(M, n_heads);
-    const size_t mh = (size_t)M * n_heads;
-    return raven_host::align_up(mh * 4) + raven_host::align_up(mh * ns * 2 * 4) + raven_host::align_up(mh * ns * head_dim * 4);
+    const dim3 grid(cv.nh, M);
+    const bool wide = (int64_t)cv.nh * M < 1024;
+    if (fused) {
+        if (wide) decode_attention_kernel<T, 16, true><<<grid, dim3(1024), 0, s>>>((const T*)q, (const T*)bias, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2);
+        else      decode_attention_kernel<T, 4, true><<<grid, dim3(256), 0, s>>>((const T*)q, (const T*)bias, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2);
+    } else {
+        if (wide) decode_attention_kernel<T, 16, false><<<grid, dim3(1024), 0, s>>>((const T*)q, nullptr, nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2);
+        else      decode_attention_kernel<T, 4, false><<<grid, dim3(256), 0, s>>>((const T*)q, nullptr, nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2);
+    }
+}
+
+static int attention_common(const char* who, bool fused, const void* q, const void* bias, const float* freqs, void* y,
+                            const raven_kv_cache* cache, int slot, int B, int S, int pos0, const int32_t* pos_dev, int n_heads,
+                            int head_dim, int dtype, void* stream) {
+    using namespace raven;
+    if (int rc = check_heads(who, n_heads, head_dim, dtype)) return rc;
+    RAVEN_REQUIRE(q && y, "%s: null pointer", who);
+    RAVEN_REQUIRE(!fused || freqs, "%s: null RoPE table", who);
+    RAVEN_REQUIRE(B > 0 && S > 0 && pos0 >= 0, "%s: bad B=%d S=%d pos0=%d", who, B, S, pos0);
+    CacheView cv;
+    if (int rc = make_view(who, cache, slot, B, n_heads, head_dim, &cv)) return rc;
+    RAVEN_REQUIRE(pos0 + S <= cv.t_max, "%s: positions up to %d exceed the cache length %d", who, pos0 + S - 1, cv.t_max);
+    const int M = B * S;
+    RAVEN_REQUIRE(M <= 65535, "%s: too many token rows (%d)", who, M);
+    const float scale_log2 = (float)(1.0 / sqrt((double)head_dim) * 1.4426950408889634);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == RAVEN_BF16) launch_attention<bf16>(fused, q, bias, freqs, y, cv, S, M, pos0, pos_dev, scale_log2, s);
+    else launch_attention<float>(fused, q, bias, freqs, y, cv, S, M, pos0, pos_dev, scale_log2, s);
+    return raven_host::check_launch(who);
 }
 
 extern "C" int raven_decode_attention(const void* q, void* y, const raven_kv_cache* cache, int32_t slot, int32_t B,
                                       int32_t S, int32_t pos0, const int32_t* pos_dev, int32_t n_heads, int32_t head_dim,
-                                      int32_t dtype, void* workspace, size_t workspace_bytes, void* stream) {
-    using namespace raven;
-    if (int rc = check_heads("decode_attention", n_heads, head_dim, dtype)) return rc;
-    RAVEN_REQUIRE(q && y, "decode_attention: null pointer");
-    RAVEN_REQUIRE(B > 0 && S > 0 && pos0 >= 0, "decode_attention: bad B=%d S=%d pos0=%d", B, S, pos0);
-    CacheView cv;
-    if (int rc = make_view("decode_attention", cache, slot, B, n_heads, head_dim, &cv)) return rc;
-    RAVEN_REQUIRE(pos0 + S <= cv.t_max, "decode_attention: positions up to %d exceed the cache length %d", pos0 + S - 1, cv.t_max);
-    const int M = B * S;
-    RAVEN_REQUIRE(M <= 65535, "decode_attention: too many token rows (%d)", M);
-    int ns = max_splits_for(M, n_heads);
-    const int by_len = (pos0 + S + 63) / 64;  // at least 64 positions per split
-    if (ns > by_len) ns = by_len;
-    if (ns < 1) ns = 1;
-    const size_t mh = (size_t)M * n_heads;
-    int* counters = nullptr;
-    float *ws_ml = nullptr, *ws_o = nullptr;
-    if (ns > 1) {
-        const size_t need = raven_decode_attention_workspace_bytes(M, n_heads, head_dim);
-        RAVEN_REQUIRE(workspace && workspace_bytes >= need, "decode_attention: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-        RAVEN_REQUIRE(((uintptr_t)workspace & 255) == 0, "decode_attention: workspace must be 256-byte aligned");
-        char* p = static_cast<char*>(workspace);
-        counters = reinterpret_cast<int*>(p);
-        p += raven_host::align_up(mh * 4);
-        ws_ml = reinterpret_cast<float*>(p);
-        p += raven_host::align_up(mh * (size_t)max_splits_for(M, n_heads) * 2 * 4);
-        ws_o = reinterpret_cast<float*>(p);
-    }
-    const float scale_log2 = (float)(1.0 / sqrt((double)head_dim) * 1.4426950408889634);
-    dim3 grid(ns, n_heads, M);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == RAVEN_BF16)
-        decode_attention_kernel<bf16><<<grid, dim3(256), 0, s>>>((const bf16*)q, (bf16*)y, cv, S, pos0, pos_dev, ns, scale_log2, counters, ws_ml, ws_o);
-    else
-        decode_attention_kernel<float><<<grid, dim3(256), 0, s>>>((const float*)q, (float*)y, cv, S, pos0, pos_dev, ns, scale_log2, counters, ws_ml, ws_o);
-    return raven_host::check_launch("decode_attention");
+                                      int32_t dtype, void* stream) {
+    return attention_common("decode_attention", false, q, nullptr, nullptr, y, cache, slot, B, S, pos0, pos_dev, n_heads, head_dim,
+                            dtype, stream);
+}
+
+extern "C" int raven_qkv_attention_decode(const void* qkv, const void* qk_bias, const float* freqs, void* y,
+                                          const raven_kv_cache* cache, int32_t slot, int32_t B, int32_t pos0,
+                                          const int32_t* pos_dev, int32_t n_heads, int32_t head_dim, int32_t dtype,
+                                          void* stream) {
+    return attention_common("qkv_attention_decode", true, qkv, qk_bias, freqs, y, cache, slot, B, 1, pos0, pos_dev, n_heads,
+                            head_dim, dtype, stream);
 }

@@ -11,8 +11,6 @@ namespace raven {
 
 struct BlockScratch {
     char *n1, *qkv, *q, *ya, *x1, *x2, *n3, *g, *x3, *xa;
-    void* attn_ws;
-    size_t attn_ws_bytes;
 };
 
 static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
@@ -35,8 +33,6 @@ static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
     s.g = take((size_t)M * d->intermediate * es);
     s.x3 = take(row);
     s.xa = take(row);
-    s.attn_ws_bytes = raven_decode_attention_workspace_bytes(M, d->n_heads, d->head_dim);
-    s.attn_ws = take(s.attn_ws_bytes);
     if (out) *out = s;
     return off;
 }
@@ -66,10 +62,14 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
     if (!n1_ready)
         if ((rc = raven_rmsnorm_residual(x_in, nullptr, w->norm_1, s.n1, nullptr, nullptr, nullptr, M, h, d->eps, dt, stream))) return rc;
     if ((rc = raven_gemm(s.n1, w->wqkv, nullptr, s.qkv, M, 3 * h, h, dt, 0, stream))) return rc;
-    if ((rc = raven_qkv_bias_rope_cache_append(s.qkv, w->qk_bias, freqs, s.q, cache, slot, B, S, pos0, pos_dev, d->n_heads,
-                                               d->head_dim, dt, stream))) return rc;
-    if ((rc = raven_decode_attention(s.q, s.ya, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, s.attn_ws,
-                                     s.attn_ws_bytes, stream))) return rc;
+    if (S == 1) {  // decode: bias, RoPE, cache append and attention in one launch
+        if ((rc = raven_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, cache, slot, B, pos0, pos_dev, d->n_heads,
+                                             d->head_dim, dt, stream))) return rc;
+    } else {       // a chunk of S tokens: every row's keys must be in the cache before any row attends
+        if ((rc = raven_qkv_bias_rope_cache_append(s.qkv, w->qk_bias, freqs, s.q, cache, slot, B, S, pos0, pos_dev, d->n_heads,
+                                                   d->head_dim, dt, stream))) return rc;
+        if ((rc = raven_decode_attention(s.q, s.ya, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, stream))) return rc;
+    }
     if ((rc = raven_gemm(s.ya, w->proj, x_in, s.x1, M, h, h, dt, 0, stream))) return rc;
     if ((rc = raven_rmsnorm_residual(s.x1, nullptr, w->norm_2, s.x2, nullptr, w->norm_3, s.n3, M, h, d->eps, dt, stream))) return rc;
     if ((rc = raven_gemm_swiglu(s.n3, w->fc, s.g, M, I, h, dt, stream))) return rc;

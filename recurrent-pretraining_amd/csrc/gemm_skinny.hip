@@ -368,8 +368,8 @@ extern "C" int raven_gemm(const void* x, const void* w, const void* residual, vo
                           int32_t dtype, int32_t out_f32, void* stream) {
     using namespace raven;
     if (int rc = check_common("gemm", M, N, K, dtype)) return rc;
-    RAVEN_REQUIRE(x && w && y, "gemm: null pointer");
     if (M == 0) return 0;
+    RAVEN_REQUIRE(x && w && y, "gemm: null pointer");
     GemmArgs a{};
     a.w = w; a.x0 = x; a.x1 = nullptr; a.residual = residual; a.y = y;
     a.M = M; a.N = N; a.K = K; a.k0 = K; a.k1 = 0; a.out_f32 = out_f32;
@@ -380,6 +380,7 @@ extern "C" int raven_adapter_gemm_concat(const void* x0, const void* x1, const v
                                          int32_t K0, int32_t K1, int32_t dtype, void* stream) {
     using namespace raven;
     if (int rc = check_common("adapter", M, N, K0 + K1, dtype)) return rc;
+    if (M == 0) return 0;
     RAVEN_REQUIRE(x0 && x1 && w && y, "adapter: null pointer");
     const int elts = 16 / (int)raven_host::elt_size(dtype);
     RAVEN_REQUIRE(K0 > 0 && K1 > 0 && K0 % elts == 0 && K1 % elts == 0, "adapter: K0=%d, K1=%d must be positive multiples of %d", K0, K1, elts);
@@ -394,8 +395,8 @@ extern "C" int raven_gemm_swiglu(const void* x, const void* fc, void* out, int32
                                  void* stream) {
     using namespace raven;
     if (int rc = check_common("gemm_swiglu", M, I, K, dtype)) return rc;
-    RAVEN_REQUIRE(x && fc && out, "gemm_swiglu: null pointer");
     if (M == 0) return 0;
+    RAVEN_REQUIRE(x && fc && out, "gemm_swiglu: null pointer");
     GemmArgs a{};
     a.w = fc; a.x0 = x; a.x1 = nullptr; a.residual = nullptr; a.y = out;
     a.M = M; a.N = I; a.K = K; a.k0 = K; a.k1 = 0; a.out_f32 = 0;

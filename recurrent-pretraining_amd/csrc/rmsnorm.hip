@@ -92,6 +92,7 @@ extern "C" int raven_rmsnorm_residual(const void* x, const void* residual, const
                                       float eps, int32_t dtype, void* stream) {
     using namespace raven;
     RAVEN_REQUIRE(dtype == RAVEN_F32 || dtype == RAVEN_BF16, "rmsnorm: unknown dtype %d", dtype);
+    if (rows == 0) return 0;  // an empty tensor has no storage to point at
     RAVEN_REQUIRE(x && weight && (y || y2), "rmsnorm: null x / weight / output");
     RAVEN_REQUIRE((weight2 == nullptr) == (y2 == nullptr), "rmsnorm: weight2 and y2 must be given together");
     RAVEN_REQUIRE(sum_out == nullptr || residual != nullptr, "rmsnorm: sum_out needs a residual");
@@ -99,8 +100,7 @@ extern "C" int raven_rmsnorm_residual(const void* x, const void* residual, const
     RAVEN_REQUIRE(dim > 0 && dim % elts == 0, "rmsnorm: dim %d is not a multiple of %d", dim, elts);
     RAVEN_REQUIRE(dim / elts <= kNormThreads * kNormMaxChunks, "rmsnorm: dim %d too large (max %d)", dim,
                   kNormThreads * kNormMaxChunks * elts);
-    RAVEN_REQUIRE(rows >= 0 && rows < (1ll << 31), "rmsnorm: bad row count %lld", (long long)rows);
-    if (rows == 0) return 0;
+    RAVEN_REQUIRE(rows > 0 && rows < (1ll << 31), "rmsnorm: bad row count %lld", (long long)rows);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == RAVEN_BF16) {
         rmsnorm_kernel<bf16><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(

@@ -51,9 +51,9 @@ SIGNATURES = {
     "raven_gemm_swiglu": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I32, _I32, _VP]),
     "raven_qkv_bias_rope_cache_append": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32,
                                                    _VP, _I32, _I32, _I32, _VP]),
-    "raven_decode_attention_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
-    "raven_decode_attention": (C.c_int, [_VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _I32, _I32, _I32,
-                                         _VP, _SZ, _VP]),
+    "raven_decode_attention": (C.c_int, [_VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _I32, _I32, _I32, _VP]),
+    "raven_qkv_attention_decode": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _VP, _I32, _I32,
+                                             _I32, _VP]),
     "raven_embed": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I64, _F, _I32, _VP]),
     "raven_argmax": (C.c_int, [_VP, _VP, _I32, _I64, _VP]),
     "raven_advance_pos": (C.c_int, [_VP, _I32, _VP]),
@@ -196,17 +196,23 @@ def qkv_bias_rope_cache_append(qkv, qk_bias, freqs, cache: KVCache, slot, B, S, 
     return q
 
 
-def attention_workspace(M, n_heads, head_dim, device) -> torch.Tensor:
-    n = load().raven_decode_attention_workspace_bytes(M, n_heads, head_dim)
-    return torch.zeros(max(n, 256), dtype=torch.uint8, device=device)
-
-
-def decode_attention(q, cache: KVCache, slot, B, S, pos0, n_heads, head_dim, workspace, pos_dev=None):
+def decode_attention(q, cache: KVCache, slot, B, S, pos0, n_heads, head_dim, pos_dev=None):
     y = torch.empty_like(q)
     rc = load().raven_decode_attention(
         _ptr(q, "q"), _ptr(y, "y"), C.byref(cache), slot, B, S, pos0, _ptr(pos_dev, "pos_dev", torch.int32),
-        n_heads, head_dim, dtype_code(q.dtype), _ptr(workspace, "workspace", torch.uint8), workspace.numel(), _stream())
+        n_heads, head_dim, dtype_code(q.dtype), _stream())
     _check(rc, "raven_decode_attention")
+    return y
+
+
+def qkv_attention_decode(qkv, qk_bias, freqs, cache: KVCache, slot, B, pos0, n_heads, head_dim, pos_dev=None):
+    """Decode step: fused qkv rows [B, 3h] -> attention output [B, h]; appends k, v at pos0."""
+    dt = qkv.dtype
+    y = torch.empty(B, n_heads * head_dim, device=qkv.device, dtype=dt)
+    rc = load().raven_qkv_attention_decode(
+        _ptr(qkv, "qkv"), _ptr(qk_bias, "qk_bias", dt), _ptr(freqs, "freqs", torch.float32), _ptr(y, "y"), C.byref(cache),
+        slot, B, pos0, _ptr(pos_dev, "pos_dev", torch.int32), n_heads, head_dim, dtype_code(dt), _stream())
+    _check(rc, "raven_qkv_attention_decode")
     return y
 
 

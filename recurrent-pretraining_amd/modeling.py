@@ -116,8 +116,9 @@ class SandwichBlock(torch.nn.Module):
 
 def precompute_freqs_cis(dim: int, end: int, theta: float) -> torch.Tensor:
     """(cos, sin) table [1, end, 1, dim/2, 2] in fp32 (RMM:2076-2081)."""
-    inv = 1.0 / (theta ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim))
-    ang = torch.outer(torch.arange(end, dtype=torch.float32), inv).float()
+    # always evaluated on the CPU, so the table does not depend on where the model lives
+    inv = 1.0 / (theta ** (torch.arange(0, dim, 2, dtype=torch.float32, device="cpu") / dim))
+    ang = torch.outer(torch.arange(end, dtype=torch.float32, device="cpu"), inv).float()
     return torch.stack([ang.cos()[None, :, None, :], ang.sin()[None, :, None, :]], dim=4)
 
 
@@ -146,8 +147,8 @@ class RavenForCausalLM(torch.nn.Module):
             self.lm_head = _linear(config.n_embd, config.padded_vocab_size)
             if config.tie_embeddings:
                 self.lm_head.weight = self.transformer.wte.weight
-            self.register_buffer("freqs_cis", precompute_freqs_cis(config.head_dim, config.block_size, config.rope_base),
-                                 persistent=True)
+            table = precompute_freqs_cis(config.head_dim, config.block_size, config.rope_base)
+            self.register_buffer("freqs_cis", table.to(device), persistent=True)
         self.to(dtype)  # casts the RoPE table too, as nn.Module.to does for the reference (RMM:577)
         self.generation_config = GenerationSettings()
         self._native_key = None
