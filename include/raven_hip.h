@@ -68,6 +68,11 @@ int         raven_version(void);
 const char* raven_arch(void);
 const char* raven_last_error(void);
 
+/* Launch-shape overrides for experiments (grid sizing and load hints of the skinny-GEMM kernels);
+ * results never depend on them.  Keys: gemv_units_per_wave, gemv_interleave, gemv_nontemporal,
+ * gemv_wgs_per_cu.  Not needed in normal use: the defaults are the tuned values. */
+int raven_set_tuning(const char* key, int32_t value);
+
 /* RMSNorm with the reference's two roundings, optionally preceded by a residual add and followed by
  * a second norm.  RMM:137-142 (norm), RMM:534-535 (the adds feeding norm_2 / norm_4).
  *   s  = residual ? T(x + residual) : x          -> stored to sum_out when non-NULL
@@ -96,6 +101,19 @@ int raven_adapter_gemm_concat(const void* x0, const void* x1, const void* w, voi
  *   z = X fc^T, gate = T(z[:, :I]), up = T(z[:, I:]), out[M, I] = T(T(silu(gate)) * up). */
 int raven_gemm_swiglu(const void* x, const void* fc, void* out,
                       int32_t M, int32_t I, int32_t K, int32_t dtype, void* stream);
+
+/* Decode fast path for ONE token row, one launch:
+ *     x  = norm_a ? T(rmsnorm(x0) * norm_a) : x0      -> stored to xa_out when non-NULL
+ *     x  = norm_b ? T(rmsnorm(x)  * norm_b) : x
+ *     z  = concat(x, x1) W^T                          (x1 / K1 optional: the adapter's second operand)
+ *     y  = swiglu ? T(T(silu(T(z[:N]))) * T(z[N:]))   : T(z) [+ residual, in T] [stored as float]
+ * i.e. the RMSNorms of RMM:525-536 folded into the nn.Linear that consumes them (norm_4 of the
+ * previous block and norm_1 before Wqkv, norm_2 and norm_3 before mlp.fc), with the epilogues of
+ * raven_gemm / raven_gemm_swiglu.  x0 [K0], x1 [K1], norm_a / norm_b / xa_out [K0], w [N or 2N, K0+K1],
+ * residual / y [N].  xa_out must not alias x0.  (K0 + K1) * sizeof(T) <= 36 KiB. */
+int raven_gemv_fused(const void* x0, const void* x1, const void* norm_a, const void* norm_b, void* xa_out,
+                     const void* w, const void* residual, void* y, int32_t N, int32_t K0, int32_t K1,
+                     float eps, int32_t swiglu, int32_t out_f32, int32_t dtype, void* stream);
 
 /* Split fused qkv rows, add q/k bias, rotate q and k, append k and v to the cache slot
  * (RMM:463-479 and HuginnStaticCache.update's index_copy_, RMM:375-380).

@@ -2,15 +2,25 @@
 // kernels in this library on one stream.  Follows SandwichBlock.forward and core_block_forward of
 // the reference (recpre/raven_modeling_minimal.py:525-536, 764-781):
 //   a  = proj(attention(norm_1(x)));  x2 = norm_2(a + x);  out = norm_4(mlp(norm_3(x2)) + x2)
-// The residual adds ride in the epilogue of the proj / mlp.proj GEMMs, norm_2 and norm_3 are one
-// launch, and inside an iteration norm_4 of one block and norm_1 of the next are one launch.
+//
+// Two schedules:
+//   one token row (decode, bs = 1): 5 launches per block -- every RMSNorm rides in the prologue of the
+//     GEMV that consumes it (norm_4 of the previous block + norm_1 before Wqkv, norm_2 + norm_3 before
+//     mlp.fc), the residual adds ride in the proj / mlp.proj epilogues, bias + RoPE + cache append ride in
+//     the attention kernel; one closing norm_4 (+ ln_f) launch per call.
+//   several rows: the residual adds still ride in the GEMM epilogues, norm_2 + norm_3 are one launch, and
+//     inside an iteration norm_4 of one block and norm_1 of the next are one launch.
 
 #include "raven_common.h"
+
+extern "C" int raven_gemv_fused(const void* x0, const void* x1, const void* norm_a, const void* norm_b, void* xa_out,
+                                const void* w, const void* residual, void* y, int32_t N, int32_t K0, int32_t K1, float eps,
+                                int32_t swiglu, int32_t out_f32, int32_t dtype, void* stream);
 
 namespace raven {
 
 struct BlockScratch {
-    char *n1, *qkv, *q, *ya, *x1, *x2, *n3, *g, *x3, *xa;
+    char *n1, *qkv, *q, *ya, *x1, *x2, *n3, *g, *x3, *xa, *xr;
 };
 
 static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
@@ -33,6 +43,7 @@ static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
     s.g = take((size_t)M * d->intermediate * es);
     s.x3 = take(row);
     s.xa = take(row);
+    s.xr = take(row);
     if (out) *out = s;
     return off;
 }
@@ -51,7 +62,14 @@ static int check_block_weights(const char* who, const raven_block_weights* w) {
     return 0;
 }
 
-// One block.  n1_ready: scratch.n1 already holds norm_1(x_in).  tail_w / tail_out: a second norm
+// the one-row kernel keeps a quarter of K per wave in registers: 9 chunks of 16 bytes per lane at most
+static bool one_row_fits(const raven_dims* d) {
+    const int elts = 16 / (int)raven_host::elt_size(d->dtype);
+    const int longest = d->intermediate > 2 * d->n_embd ? d->intermediate : 2 * d->n_embd;
+    return ((longest / elts + 3) / 4 + 1 + 63) / 64 <= 9;
+}
+
+// Several rows.  n1_ready: scratch.n1 already holds norm_1(x_in).  tail_w / tail_out: a second norm
 // applied to the block output (next block's norm_1, or ln_f); y_out may be null when only the tail
 // result is wanted.
 static int run_block(const raven_dims* d, const raven_block_weights* w, const BlockScratch& s, bool n1_ready,
@@ -77,6 +95,33 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
     return raven_rmsnorm_residual(s.x3, nullptr, w->norm_4, y_out, nullptr, tail_w, tail_out, M, h, d->eps, dt, stream);
 }
 
+// One row.  x_raw is the block input before `pre_norm` (the previous block's norm_4, or null when x_raw is
+// the input itself).  Leaves the block output BEFORE its norm_4 in scratch.x3.
+static int run_block_one_row(const raven_dims* d, const raven_block_weights* w, const BlockScratch& s, const void* x_raw,
+                             const void* pre_norm, const float* freqs, const raven_kv_cache* cache, int slot, int pos0,
+                             const int32_t* pos_dev, void* stream) {
+    const int h = d->n_embd, I = d->intermediate, dt = d->dtype;
+    const float eps = d->eps;
+    int rc;
+    const void* x_res = x_raw;  // the residual the attention output is added to (RMM:534)
+    if (pre_norm) {
+        if ((rc = raven_gemv_fused(x_raw, nullptr, pre_norm, w->norm_1, s.xr, w->wqkv, nullptr, s.qkv, 3 * h, h, 0, eps, 0, 0, dt, stream))) return rc;
+        x_res = s.xr;
+    } else {
+        if ((rc = raven_gemv_fused(x_raw, nullptr, w->norm_1, nullptr, nullptr, w->wqkv, nullptr, s.qkv, 3 * h, h, 0, eps, 0, 0, dt, stream))) return rc;
+    }
+    if ((rc = raven_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, cache, slot, 1, pos0, pos_dev, d->n_heads, d->head_dim, dt, stream))) return rc;
+    if ((rc = raven_gemv_fused(s.ya, nullptr, nullptr, nullptr, nullptr, w->proj, x_res, s.x1, h, h, 0, eps, 0, 0, dt, stream))) return rc;
+    if ((rc = raven_gemv_fused(s.x1, nullptr, w->norm_2, w->norm_3, s.x2, w->fc, nullptr, s.g, I, h, 0, eps, 1, 0, dt, stream))) return rc;
+    return raven_gemv_fused(s.g, nullptr, nullptr, nullptr, nullptr, w->mlp_proj, s.x2, s.x3, h, I, 0, eps, 0, 0, dt, stream);
+}
+
+// closing norm_4 (+ ln_f) of the one-row schedule
+static int close_one_row(const raven_dims* d, const BlockScratch& s, const void* norm_4, const void* ln_f, void* out, void* stream) {
+    if (ln_f) return raven_rmsnorm_residual(s.x3, nullptr, norm_4, nullptr, nullptr, ln_f, out, 1, d->n_embd, d->eps, d->dtype, stream);
+    return raven_rmsnorm_residual(s.x3, nullptr, norm_4, out, nullptr, nullptr, nullptr, 1, d->n_embd, d->eps, d->dtype, stream);
+}
+
 }  // namespace raven
 
 extern "C" size_t raven_block_workspace_bytes(const raven_dims* dims, int32_t M) {
@@ -98,6 +143,10 @@ extern "C" int raven_sandwich_block(const raven_dims* dims, const raven_block_we
     RAVEN_REQUIRE(((uintptr_t)workspace & 255) == 0, "sandwich_block: workspace must be 256-byte aligned");
     BlockScratch s;
     carve(dims, B * S, static_cast<char*>(workspace), &s);
+    if (B * S == 1 && one_row_fits(dims)) {
+        if (int rc = run_block_one_row(dims, w, s, x_in, nullptr, freqs, cache, slot, pos0, pos_dev, stream)) return rc;
+        return close_one_row(dims, s, w->norm_4, ln_f, x_out, stream);
+    }
     if (ln_f) return run_block(dims, w, s, false, x_in, nullptr, ln_f, x_out, freqs, cache, slot, B, S, pos0, pos_dev, stream);
     return run_block(dims, w, s, false, x_in, x_out, nullptr, nullptr, freqs, cache, slot, B, S, pos0, pos_dev, stream);
 }
@@ -122,6 +171,16 @@ extern "C" int raven_core_iteration(const raven_dims* dims, const void* adapter_
     carve(dims, M, static_cast<char*>(workspace), &s);
 
     int rc;
+    if (M == 1 && one_row_fits(dims)) {
+        if ((rc = raven_gemv_fused(state_in, embeds, nullptr, nullptr, nullptr, adapter_w, nullptr, s.xa, h, h, h, dims->eps, 0, 0,
+                                   dims->dtype, stream))) return rc;
+        for (int j = 0; j < n_blocks; ++j) {
+            const void* x_raw = j == 0 ? (const void*)s.xa : (const void*)s.x3;
+            const void* pre = j == 0 ? nullptr : blocks[j - 1].norm_4;
+            if ((rc = run_block_one_row(dims, &blocks[j], s, x_raw, pre, freqs, cache, first_slot + j, pos0, pos_dev, stream))) return rc;
+        }
+        return close_one_row(dims, s, blocks[n_blocks - 1].norm_4, ln_f, state_out, stream);
+    }
     if ((rc = raven_adapter_gemm_concat(state_in, embeds, adapter_w, s.xa, M, h, h, h, dims->dtype, stream))) return rc;
     for (int j = 0; j < n_blocks; ++j) {
         const bool last = j == n_blocks - 1;

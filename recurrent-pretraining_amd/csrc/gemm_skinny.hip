@@ -13,7 +13,13 @@
 //   SwiGLU: T(T(silu(gate)) * up), gate row j, up row j+I  RMM:507-508
 // The adapter's concat (RMM:776) is folded in by giving X as two pointers that cover K0 and K1.
 
+#include <string>
+
 #include "raven_common.h"
+
+extern "C" int raven_gemv_fused(const void* x0, const void* x1, const void* norm_a, const void* norm_b, void* xa_out,
+                                const void* w, const void* residual, void* y, int32_t N, int32_t K0, int32_t K1, float eps,
+                                int32_t swiglu, int32_t out_f32, int32_t dtype, void* stream);
 
 namespace raven {
 
@@ -28,7 +34,27 @@ struct GemmArgs {
     int M, N, K, k0, k1;   // N = number of output columns (I for SwiGLU)
     int out_f32;
     int units_per_wave;    // gemv: row pairs per wave
+    int interleave;        // gemv: unit = u * total_waves + wave (1) or wave * units_per_wave + u (0)
 };
+
+// Launch-shape knobs (raven_set_tuning); 0 = automatic.
+struct Tuning {
+    int gemv_units_per_wave = 0;
+    int gemv_interleave = 1;
+    int gemv_nontemporal = 1;
+    int gemv_wgs_per_cu = 4;
+};
+static Tuning g_tuning;
+
+// weight rows are read exactly once: stream them past the caches
+template <bool NT, typename T>
+__device__ __forceinline__ Chunk<T> load_weight(const T* p) {
+    if (!NT) return load_chunk(p);
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    Chunk<T> c;
+    *reinterpret_cast<u32x4*>(&c) = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return c;
+}
 
 template <typename T>
 __device__ __forceinline__ void store_out(const GemmArgs& a, int m, int n, float acc) {
@@ -49,7 +75,7 @@ __device__ __forceinline__ float swiglu(float gate_acc, float up_acc) {
 // ------------------------------------------------------------------------------------------------
 // gemv_kernel: 256 threads; dynamic LDS holds X as [MB][K] of T.
 // ------------------------------------------------------------------------------------------------
-template <typename T, int MB, int EPI>
+template <typename T, int MB, int EPI, bool NT>
 __global__ __launch_bounds__(256) void gemv_kernel(GemmArgs a) {
     constexpr int E = Chunk<T>::N;
     constexpr int U = 4;
@@ -71,11 +97,13 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemmArgs a) {
 
     const int lane = threadIdx.x & 63;
     const int gwave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int total_waves = gridDim.x * 4;
     const int n_units = (EPI == EPI_SWIGLU) ? a.N : (a.N + 1) / 2;
     const T* W = static_cast<const T*>(a.w);
 
     for (int u = 0; u < a.units_per_wave; ++u) {
-        const int unit = gwave * a.units_per_wave + u;
+        // interleaved: at any moment the waves of the whole grid read neighbouring rows
+        const int unit = a.interleave ? u * total_waves + gwave : gwave * a.units_per_wave + u;
         if (unit >= n_units) break;
         int r0, r1;
         bool r1_ok = true;
@@ -99,8 +127,8 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemmArgs a) {
             for (int j = 0; j < U; ++j) {
                 const int cc = c + 64 * j;
                 if (cc < n_chunks) {
-                    a0[j] = load_chunk(w0 + cc * E);
-                    a1[j] = load_chunk(w1 + cc * E);
+                    a0[j] = load_weight<NT>(w0 + cc * E);
+                    a1[j] = load_weight<NT>(w1 + cc * E);
                 } else {
                     a0[j] = zero_chunk<T>();
                     a1[j] = zero_chunk<T>();
@@ -269,13 +297,13 @@ static int n_cus() {
     return cus;
 }
 
-template <typename T, int MB, int EPI>
-static int launch_gemv(GemmArgs a, hipStream_t s) {
+template <typename T, int MB, int EPI, bool NT>
+static int launch_gemv_nt(GemmArgs a, hipStream_t s) {
     const size_t lds = (size_t)MB * a.K * sizeof(T);
     RAVEN_REQUIRE(lds <= 160 * 1024, "gemm: %d rows x K=%d does not fit the 160 KB LDS", MB, a.K);
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemv_kernel<T, MB, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t e = hipFuncSetAttribute((const void*)gemv_kernel<T, MB, EPI, NT>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) {
             raven_host::set_error("gemm: hipFuncSetAttribute failed: %s", hipGetErrorString(e));
             return (int)e;
@@ -283,14 +311,23 @@ static int launch_gemv(GemmArgs a, hipStream_t s) {
         attr_set = true;
     }
     const int n_units = (EPI == EPI_SWIGLU) ? a.N : (a.N + 1) / 2;
-    // as few units per wave as keeps every workgroup resident at once (about 4 per CU)
-    const int max_wgs = n_cus() * 4;
-    int upw = 1;
-    while ((n_units + 4 * upw - 1) / (4 * upw) > max_wgs) ++upw;
+    // as few units per wave as keeps every workgroup resident at once
+    const int max_wgs = n_cus() * (g_tuning.gemv_wgs_per_cu > 0 ? g_tuning.gemv_wgs_per_cu : 4);
+    int upw = g_tuning.gemv_units_per_wave;
+    if (upw <= 0) {
+        upw = 1;
+        while ((n_units + 4 * upw - 1) / (4 * upw) > max_wgs) ++upw;
+    }
     a.units_per_wave = upw;
+    a.interleave = g_tuning.gemv_interleave;
     const int wgs = (n_units + 4 * upw - 1) / (4 * upw);
-    gemv_kernel<T, MB, EPI><<<dim3(wgs), dim3(256), lds, s>>>(a);
+    gemv_kernel<T, MB, EPI, NT><<<dim3(wgs), dim3(256), lds, s>>>(a);
     return raven_host::check_launch("gemv");
+}
+
+template <typename T, int MB, int EPI>
+static int launch_gemv(GemmArgs a, hipStream_t s) {
+    return g_tuning.gemv_nontemporal ? launch_gemv_nt<T, MB, EPI, true>(a, s) : launch_gemv_nt<T, MB, EPI, false>(a, s);
 }
 
 template <typename T, int EPI>
@@ -334,6 +371,15 @@ static int run_gemm(GemmArgs a, int dtype, hipStream_t s) {
     for (int m0 = 0; m0 < M;) {
         const int left = M - m0;
         int pass;
+        const int elts = 16 / (int)es;
+        if (left == 1 && ((a.K / elts + 3) / 4 + 1 + 63) / 64 <= 9) {  // a single row: the K-split one-row kernel
+            const char* x0 = static_cast<const char*>(a.x0) + (size_t)m0 * a.k0 * es;
+            const char* x1 = a.x1 ? static_cast<const char*>(a.x1) + (size_t)m0 * a.k1 * es : nullptr;
+            const char* res = a.residual ? static_cast<const char*>(a.residual) + (size_t)m0 * a.N * es : nullptr;
+            char* y = static_cast<char*>(a.y) + (size_t)m0 * a.N * out_es;
+            return raven_gemv_fused(x0, x1, nullptr, nullptr, nullptr, a.w, res, y, a.N, a.k0, a.k1, 0.f, EPI == EPI_SWIGLU, a.out_f32,
+                                    dtype, s);
+        }
         const bool use_mfma = mfma_ok && left > 4;
         if (use_mfma) pass = left < 32 ? left : 32;
         else if (dtype == RAVEN_BF16) pass = left < 4 ? left : 4;
@@ -363,6 +409,18 @@ static int check_common(const char* who, int M, int N, int K, int dtype) {
 }
 
 }  // namespace raven
+
+extern "C" int raven_set_tuning(const char* key, int32_t value) {
+    using namespace raven;
+    RAVEN_REQUIRE(key != nullptr, "set_tuning: null key");
+    const std::string k(key);
+    if (k == "gemv_units_per_wave") g_tuning.gemv_units_per_wave = value;
+    else if (k == "gemv_interleave") g_tuning.gemv_interleave = value;
+    else if (k == "gemv_nontemporal") g_tuning.gemv_nontemporal = value;
+    else if (k == "gemv_wgs_per_cu") g_tuning.gemv_wgs_per_cu = value;
+    else RAVEN_REQUIRE(false, "set_tuning: unknown key %s", key);
+    return 0;
+}
 
 extern "C" int raven_gemm(const void* x, const void* w, const void* residual, void* y, int32_t M, int32_t N, int32_t K,
                           int32_t dtype, int32_t out_f32, void* stream) {

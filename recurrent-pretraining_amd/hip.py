@@ -45,10 +45,12 @@ SIGNATURES = {
     "raven_version": (C.c_int, []),
     "raven_arch": (C.c_char_p, []),
     "raven_last_error": (C.c_char_p, []),
+    "raven_set_tuning": (C.c_int, [C.c_char_p, _I32]),
     "raven_rmsnorm_residual": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _I32, _F, _I32, _VP]),
     "raven_gemm": (C.c_int, [_VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _VP]),
     "raven_adapter_gemm_concat": (C.c_int, [_VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _VP]),
     "raven_gemm_swiglu": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I32, _I32, _VP]),
+    "raven_gemv_fused": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _F, _I32, _I32, _I32, _VP]),
     "raven_qkv_bias_rope_cache_append": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32,
                                                    _VP, _I32, _I32, _I32, _VP]),
     "raven_decode_attention": (C.c_int, [_VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _I32, _I32, _I32, _VP]),
@@ -88,6 +90,10 @@ def _check(rc: int, what: str) -> None:
     if rc != 0:
         msg = load().raven_last_error().decode("utf-8", "replace")
         raise RavenHipError(f"{what} failed (code {rc}): {msg}")
+
+
+def set_tuning(key: str, value: int) -> None:
+    _check(load().raven_set_tuning(key.encode(), int(value)), "raven_set_tuning")
 
 
 def dtype_code(dt: torch.dtype) -> int:
@@ -184,6 +190,22 @@ def gemm_swiglu(x, fc):
     rc = load().raven_gemm_swiglu(_ptr(x, "x"), _ptr(fc, "fc", dt), _ptr(y, "out"), M, inter, K, dtype_code(dt), _stream())
     _check(rc, "raven_gemm_swiglu")
     return y
+
+
+def gemv_fused(x0, w, x1=None, norm_a=None, norm_b=None, want_xa=False, residual=None, swiglu=False, out_f32=False, eps=1e-6):
+    """One token row: (norms on x0) -> concat(x0, x1) W^T -> epilogue.  Returns (y, norm_a(x0) or None)."""
+    dt = x0.dtype
+    K0 = x0.numel()
+    K1 = 0 if x1 is None else x1.numel()
+    N = w.shape[0] // 2 if swiglu else w.shape[0]
+    assert w.shape[1] == K0 + K1
+    y = torch.empty(N, device=x0.device, dtype=torch.float32 if out_f32 else dt)
+    xa = torch.empty_like(x0) if want_xa else None
+    rc = load().raven_gemv_fused(_ptr(x0, "x0"), _ptr(x1, "x1", dt), _ptr(norm_a, "norm_a", dt), _ptr(norm_b, "norm_b", dt),
+                                 _ptr(xa, "xa_out"), _ptr(w, "w", dt), _ptr(residual, "residual", dt), _ptr(y, "y"), N, K0, K1,
+                                 eps, int(swiglu), int(out_f32), dtype_code(dt), _stream())
+    _check(rc, "raven_gemv_fused")
+    return y, xa
 
 
 def qkv_bias_rope_cache_append(qkv, qk_bias, freqs, cache: KVCache, slot, B, S, pos0, n_heads, head_dim, pos_dev=None):

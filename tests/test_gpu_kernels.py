@@ -143,6 +143,43 @@ def test_gemm_swiglu(pkg, dt, M, I, K):
     assert close(y, wrong)[1] > 0.1, "the gate must be the first half"
 
 
+@pytest.mark.parametrize("dt,h,I", [(torch.bfloat16, 5280, 17920), (torch.float32, 256, 704), (torch.bfloat16, 64, 176)])
+def test_gemv_fused_one_row(pkg, dt, h, I):
+    """The one-row kernel with its norm prologues and epilogues, against the oracle's separate ops."""
+    x = rnd((h,), dt, 120)
+    wa, wb = rnd((h,), dt, 121, 0.02, 1.0), rnd((h,), dt, 122, 0.02, 1.0)
+    res = rnd((h,), dt, 123)
+    wqkv, fc, mlp = rnd((3 * h, h), dt, 124, 0.02), rnd((2 * I, h), dt, 125, 0.03), rnd((h, I), dt, 126, 0.02)
+    ada, x1 = rnd((h, 2 * h), dt, 127, 0.02), rnd((h,), dt, 128)
+    xa_want = O.rmsnorm(x[None], wa, 1e-6)
+    xb_want = O.rmsnorm(xa_want, wb, 1e-6)
+    dev = lambda t: t.cuda()
+    # norm_4 -> norm_1 -> Wqkv, with the first norm written out
+    y, xa = pkg.hip.gemv_fused(dev(x), dev(wqkv), norm_a=dev(wa), norm_b=dev(wb), want_xa=True)
+    check(xa[None], xa_want, dt, "norm_a output")
+    check(y[None], lin(xb_want, wqkv).to(dt), dt, "double norm + qkv")
+    # single norm, no store
+    y, _ = pkg.hip.gemv_fused(dev(x), dev(wqkv), norm_a=dev(wa))
+    check(y[None], lin(xa_want, wqkv).to(dt), dt, "norm + qkv")
+    # norm_2 -> norm_3 -> fc with SwiGLU
+    y, xa = pkg.hip.gemv_fused(dev(x), dev(fc), norm_a=dev(wa), norm_b=dev(wb), want_xa=True, swiglu=True)
+    z = lin(xb_want, fc).to(dt)
+    check(y[None], F.silu(z[:, :I]) * z[:, I:], dt, "double norm + fc + swiglu")
+    # long K with residual (mlp.proj) and the adapter's two operands
+    g = rnd((I,), dt, 129)
+    y, _ = pkg.hip.gemv_fused(dev(g), dev(mlp), residual=dev(res))
+    check(y[None], lin(g[None], mlp).to(dt) + res, dt, "mlp.proj + residual")
+    y, _ = pkg.hip.gemv_fused(dev(x), dev(ada), x1=dev(x1))
+    check(y[None], lin(torch.cat([x, x1])[None], ada).to(dt), dt, "adapter")
+    y, _ = pkg.hip.gemv_fused(dev(x), dev(ada), x1=dev(x1), norm_a=dev(wa))
+    check(y[None], lin(torch.cat([xa_want[0], x1])[None], ada).to(dt), dt, "norm on the first operand only")
+    yf, _ = pkg.hip.gemv_fused(dev(x), dev(wqkv), out_f32=True)
+    y, _ = pkg.hip.gemv_fused(dev(x), dev(wqkv))
+    assert yf.dtype == torch.float32 and torch.equal(yf, y.float())
+    with pytest.raises(pkg.hip.RavenHipError):
+        pkg.hip.gemv_fused(dev(x), dev(wqkv), norm_b=dev(wb))  # norm_b without norm_a
+
+
 # ----------------------------------------------------------------------------- RoPE + cache append
 def make_cache(pkg, n_slots, B, nh, t_max, hd, dt, fill_seed=None):
     if fill_seed is None:
