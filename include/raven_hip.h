@@ -70,7 +70,7 @@ const char* raven_last_error(void);
 
 /* Launch-shape overrides for experiments (grid sizing and load hints of the skinny-GEMM kernels);
  * results never depend on them.  Keys: gemv_units_per_wave, gemv_interleave, gemv_nontemporal,
- * gemv_wgs_per_cu.  Not needed in normal use: the defaults are the tuned values. */
+ * gemv_wgs_per_cu, gemv1_pairs_norm, gemv1_pairs_plain.  Not needed in normal use: the defaults are the tuned values. */
 int raven_set_tuning(const char* key, int32_t value);
 
 /* RMSNorm with the reference's two roundings, optionally preceded by a residual add and followed by

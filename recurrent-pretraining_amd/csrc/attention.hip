@@ -69,7 +69,6 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(
 
 // ------------------------------------------------------------------------------------------------
 constexpr int kAttnMaxHd = 128;
-constexpr int kAttnU = 4;  // positions per 16-lane row and loop iteration
 
 // bias + RoPE of one 16-byte chunk of a q or k head row (sec 0 = q, 1 = k); d = first column of the chunk
 template <typename T>
@@ -103,6 +102,8 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attention_kernel(
     CacheView cv, int S, int pos0, const int* __restrict__ pos_dev, float scale_log2) {
     constexpr int E = Chunk<T>::N;
     constexpr int G = WAVES * 4;  // 16-lane rows in the workgroup
+    // positions per row and loop iteration: a lone 16-wave workgroup per CU needs every load it can keep in flight
+    constexpr int kAttnU = WAVES == 16 ? 6 : 4;
     __shared__ float sm_m[G], sm_l[G];
     __shared__ float sm_o[G][kAttnMaxHd];
 

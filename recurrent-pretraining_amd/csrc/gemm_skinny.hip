@@ -23,6 +23,8 @@ extern "C" int raven_gemv_fused(const void* x0, const void* x1, const void* norm
 
 namespace raven {
 
+int set_gemv1_tuning(const char* key, int value);
+
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
 
 struct GemmArgs {
@@ -418,7 +420,7 @@ extern "C" int raven_set_tuning(const char* key, int32_t value) {
     else if (k == "gemv_interleave") g_tuning.gemv_interleave = value;
     else if (k == "gemv_nontemporal") g_tuning.gemv_nontemporal = value;
     else if (k == "gemv_wgs_per_cu") g_tuning.gemv_wgs_per_cu = value;
-    else RAVEN_REQUIRE(false, "set_tuning: unknown key %s", key);
+    else RAVEN_REQUIRE(set_gemv1_tuning(key, value) == 0, "set_tuning: unknown key %s", key);
     return 0;
 }
 

@@ -14,6 +14,8 @@
 //
 // C = weight chunks per lane, per row: ceil(ceil(K / E / 4) / 64) rounded up to 3, 6 or 9.
 
+#include <string>
+
 #include "raven_common.h"
 
 namespace raven {
@@ -30,6 +32,7 @@ struct Gemv1Args {
     int N, K, k0;
     int out_f32;
     float eps;
+    int pairs_per_wg;      // weight-row pairs each workgroup walks through
 };
 
 template <bool NT, typename T>
@@ -50,40 +53,53 @@ __device__ __forceinline__ float wg_sum(float v, float* red) {
     return red[0] + red[1] + red[2] + red[3];
 }
 
-template <typename T, int C, bool SWIGLU, bool NORM>
+constexpr int kMaxPairsPerWg = 16;
+
+// MULTI: the workgroup walks several row pairs and double-buffers their weights in registers
+template <typename T, int C, bool SWIGLU, bool NORM, bool MULTI>
 __global__ __launch_bounds__(256) void gemv1_kernel(Gemv1Args a) {
     constexpr int E = Chunk<T>::N;
     __shared__ float red[4];
-    __shared__ float part[4][2];
+    __shared__ float part[kMaxPairsPerWg][4][2];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n_chunks = a.K / E, c0 = a.k0 / E;
     const int cb = (int)((int64_t)n_chunks * wave / 4), ce = (int)((int64_t)n_chunks * (wave + 1) / 4);
-    const int unit = blockIdx.x;
-    int r0, r1;
-    bool r1_ok = true;
-    if (SWIGLU) {
-        r0 = unit;
-        r1 = unit + a.N;
-    } else {
-        r0 = 2 * unit;
-        r1 = r0 + 1;
-        if (r1 >= a.N) { r1 = r0; r1_ok = false; }
-    }
-    const T* w0 = static_cast<const T*>(a.w) + (int64_t)r0 * a.K;
-    const T* w1 = static_cast<const T*>(a.w) + (int64_t)r1 * a.K;
+    const int n_units = SWIGLU ? a.N : (a.N + 1) / 2;
+    const int ppw = MULTI ? a.pairs_per_wg : 1;
+    const T* W = static_cast<const T*>(a.w);
     const T* x0 = static_cast<const T*>(a.x0);
     const T* x1 = static_cast<const T*>(a.x1);
 
-    // x first (older loads return first), then every weight chunk of this lane
-    Chunk<T> xc[C], na[NORM ? C : 1], nb[NORM ? C : 1], wa[C], wb[C];
-    bool ok[C], in0[C];
+    // pair p of this workgroup; consecutive workgroups take consecutive pairs, so the grid as a whole
+    // walks the matrix front to back
+    auto unit_of = [&](int p) { return p * (int)gridDim.x + (int)blockIdx.x; };
+    auto load_pair = [&](int unit, Chunk<T>* wa, Chunk<T>* wb) {
+        const int r0 = SWIGLU ? unit : 2 * unit;
+        const int r1 = SWIGLU ? unit + a.N : min(r0 + 1, a.N - 1);
+        const T* w0 = W + (int64_t)r0 * a.K;
+        const T* w1 = W + (int64_t)r1 * a.K;
+#pragma unroll
+        for (int j = 0; j < C; ++j) {
+            const int c = cb + lane + 64 * j;
+            if (c < ce && unit < n_units) {
+                wa[j] = ld_weight<true>(w0 + c * E);
+                wb[j] = ld_weight<true>(w1 + c * E);
+            } else {
+                wa[j] = zero_chunk<T>();
+                wb[j] = zero_chunk<T>();
+            }
+        }
+    };
+
+    // x first (older loads return first), then the first pair's weights
+    Chunk<T> xc[C], na[NORM ? C : 1], nb[NORM ? C : 1];
+    bool in0[C];
 #pragma unroll
     for (int j = 0; j < C; ++j) {
         const int c = cb + lane + 64 * j;
-        ok[j] = c < ce;
-        in0[j] = ok[j] && c < c0;
+        in0[j] = c < ce && c < c0;
         xc[j] = zero_chunk<T>();
-        if (ok[j]) xc[j] = (c < c0) ? load_chunk(x0 + c * E) : load_chunk(x1 + (c - c0) * E);
+        if (c < ce) xc[j] = (c < c0) ? load_chunk(x0 + c * E) : load_chunk(x1 + (c - c0) * E);
     }
     if (NORM && a.norm_a) {
 #pragma unroll
@@ -95,17 +111,8 @@ __global__ __launch_bounds__(256) void gemv1_kernel(Gemv1Args a) {
         for (int j = 0; j < C; ++j)
             if (in0[j]) nb[NORM ? j : 0] = load_chunk(static_cast<const T*>(a.norm_b) + (cb + lane + 64 * j) * E);
     }
-#pragma unroll
-    for (int j = 0; j < C; ++j) {
-        const int c = cb + lane + 64 * j;
-        if (ok[j]) {
-            wa[j] = ld_weight<true>(w0 + c * E);
-            wb[j] = ld_weight<true>(w1 + c * E);
-        } else {
-            wa[j] = zero_chunk<T>();
-            wb[j] = zero_chunk<T>();
-        }
-    }
+    Chunk<T> wa0[C], wb0[C], wa1[MULTI ? C : 1], wb1[MULTI ? C : 1];
+    load_pair(unit_of(0), wa0, wb0);
 
     // RMSNorm prologue(s) over x0 (recpre/raven_modeling_minimal.py:137-142): fp32 statistics,
     // round to T, multiply by the weight in T
@@ -143,26 +150,46 @@ __global__ __launch_bounds__(256) void gemv1_kernel(Gemv1Args a) {
             }
     }
 
-    float acc0 = 0.f, acc1 = 0.f;
+    auto finish_pair = [&](int p, const Chunk<T>* wa, const Chunk<T>* wb) {
+        float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
-    for (int j = 0; j < C; ++j) {
-        acc0 = dot_chunk(wa[j], xc[j], acc0);
-        acc1 = dot_chunk(wb[j], xc[j], acc1);
-    }
-    acc0 = wave_sum(acc0);
-    acc1 = wave_sum(acc1);
-    if (lane == 0) {
-        part[wave][0] = acc0;
-        part[wave][1] = acc1;
+        for (int j = 0; j < C; ++j) {
+            acc0 = dot_chunk(wa[j], xc[j], acc0);
+            acc1 = dot_chunk(wb[j], xc[j], acc1);
+        }
+        acc0 = wave_sum(acc0);
+        acc1 = wave_sum(acc1);
+        if (lane == 0) {
+            part[p][wave][0] = acc0;
+            part[p][wave][1] = acc1;
+        }
+    };
+    // the next pair's weights are requested before the current pair is reduced
+    if (MULTI) {
+        for (int p = 0; p < ppw; p += 2) {
+            if (p + 1 < ppw) load_pair(unit_of(p + 1), wa1, wb1);
+            finish_pair(p, wa0, wb0);
+            if (p + 1 < ppw) {
+                if (p + 2 < ppw) load_pair(unit_of(p + 2), wa0, wb0);
+                finish_pair(p + 1, wa1, wb1);
+            }
+        }
+    } else {
+        finish_pair(0, wa0, wb0);
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        const float s0 = part[0][0] + part[1][0] + part[2][0] + part[3][0];
-        const float s1 = part[0][1] + part[1][1] + part[2][1] + part[3][1];
+
+    const int p = threadIdx.x;
+    if (p < ppw && unit_of(p) < n_units) {
+        const int unit = unit_of(p);
+        const float s0 = part[p][0][0] + part[p][1][0] + part[p][2][0] + part[p][3][0];
+        const float s1 = part[p][0][1] + part[p][1][1] + part[p][2][1] + part[p][3][1];
         if (SWIGLU) {
             const float g = round_to<T>(s0), u = round_to<T>(s1);
             static_cast<T*>(a.y)[unit] = from_f32<T>(round_to<T>(silu_f32(g)) * u);
         } else {
+            const int r0 = 2 * unit, r1 = r0 + 1;
+            const bool r1_ok = r1 < a.N;
             const T* res = static_cast<const T*>(a.residual);
             float v0 = round_to<T>(s0), v1 = round_to<T>(s1);
             if (res) {
@@ -180,20 +207,36 @@ __global__ __launch_bounds__(256) void gemv1_kernel(Gemv1Args a) {
     }
 }
 
+struct Gemv1Tuning {
+    int pairs_norm = 4;    // pairs per workgroup when a norm prologue has to be amortised
+    int pairs_plain = 1;   // ... and when there is none
+};
+static Gemv1Tuning g_gemv1_tuning;
+
 template <typename T, bool SWIGLU>
-static int launch_gemv1(const Gemv1Args& a, hipStream_t s) {
+static int launch_gemv1(Gemv1Args a, hipStream_t s) {
     constexpr int E = Chunk<T>::N;
     const int n_chunks = a.K / E;
     const int per_wave = (n_chunks + 3) / 4 + 1;  // a quarter, rounded up
     const int c = (per_wave + 63) / 64;
     const int units = SWIGLU ? a.N : (a.N + 1) / 2;
     const bool norm = a.norm_a != nullptr;
-#define RAVEN_GEMV1(CC)                                                                       \
-    do {                                                                                      \
-        if (norm) gemv1_kernel<T, CC, SWIGLU, true><<<dim3(units), dim3(256), 0, s>>>(a);     \
-        else gemv1_kernel<T, CC, SWIGLU, false><<<dim3(units), dim3(256), 0, s>>>(a);         \
+    int ppw = norm ? g_gemv1_tuning.pairs_norm : g_gemv1_tuning.pairs_plain;
+    if (ppw < 1) ppw = 1;
+    if (ppw > kMaxPairsPerWg) ppw = kMaxPairsPerWg;
+    while (ppw > 1 && (units + ppw - 1) / ppw < 1024) --ppw;  // keep at least ~4 workgroups per CU
+    if (c > 3) ppw = 1;  // the double-buffered variant exists for short rows only (registers)
+    a.pairs_per_wg = ppw;
+    const int wgs = (units + ppw - 1) / ppw;
+#define RAVEN_GEMV1(CC)                                                                            \
+    do {                                                                                           \
+        if (norm) gemv1_kernel<T, CC, SWIGLU, true, false><<<dim3(wgs), dim3(256), 0, s>>>(a);     \
+        else gemv1_kernel<T, CC, SWIGLU, false, false><<<dim3(wgs), dim3(256), 0, s>>>(a);         \
     } while (0)
-    if (c <= 3) RAVEN_GEMV1(3);
+    if (c <= 3 && ppw > 1) {
+        if (norm) gemv1_kernel<T, 3, SWIGLU, true, true><<<dim3(wgs), dim3(256), 0, s>>>(a);
+        else gemv1_kernel<T, 3, SWIGLU, false, true><<<dim3(wgs), dim3(256), 0, s>>>(a);
+    } else if (c <= 3) RAVEN_GEMV1(3);
     else if (c <= 6) RAVEN_GEMV1(6);
     else if (c <= 9) RAVEN_GEMV1(9);
     else {
@@ -202,6 +245,14 @@ static int launch_gemv1(const Gemv1Args& a, hipStream_t s) {
     }
 #undef RAVEN_GEMV1
     return raven_host::check_launch("gemv_fused");
+}
+
+int set_gemv1_tuning(const char* key, int value) {
+    const std::string k(key);
+    if (k == "gemv1_pairs_norm") g_gemv1_tuning.pairs_norm = value;
+    else if (k == "gemv1_pairs_plain") g_gemv1_tuning.pairs_plain = value;
+    else return -1;
+    return 0;
 }
 
 }  // namespace raven
