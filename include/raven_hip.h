@@ -127,18 +127,22 @@ int raven_qkv_bias_rope_cache_append(const void* qkv, const void* qk_bias, const
 /* softmax(q K^T / sqrt(hd)) V over the cached positions of one slot, for each of the M = B*S rows
  * (RMM:481-491).  Row m attends to positions 0 .. pos0 + (m % S) inclusive: for S == 1 this is the
  * unmasked decode case, for S > 1 the lower-right-aligned causal case.  The new keys/values must
- * already be in the cache.  q [M, h]; y [M, h] in the layout y.transpose(1,2).reshape(B,S,h) has. */
-int raven_decode_attention(const void* q, void* y, const raven_kv_cache* cache, int32_t slot,
-                           int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
-                           int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream);
+ * already be in the cache.  q [M, h]; y [M, h] in the layout y.transpose(1,2).reshape(B,S,h) has.
+ * workspace (nullable, raven_decode_attention_workspace_bytes): room for partial results when few
+ * (head, row) pairs make a split over positions worthwhile; without it the result is the same, slower. */
+size_t raven_decode_attention_workspace_bytes(int32_t M, int32_t n_heads, int32_t head_dim);
+int    raven_decode_attention(const void* q, void* y, const raven_kv_cache* cache, int32_t slot,
+                              int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
+                              int32_t n_heads, int32_t head_dim, int32_t dtype,
+                              void* workspace, size_t workspace_bytes, void* stream);
 
-/* Decode step (S == 1) of RMM:463-491 in one launch: takes the fused qkv GEMM output [B, 3h], adds
- * the q/k bias, rotates q and k for position pos0, writes the new k and v rows into the cache slot
- * and returns softmax(q K^T / sqrt(hd)) V over positions 0 .. pos0 in y [B, h]. */
+/* Decode step (S == 1) of RMM:463-491: takes the fused qkv GEMM output [B, 3h], adds the q/k bias,
+ * rotates q and k for position pos0, writes the new k and v rows into the cache slot and returns
+ * softmax(q K^T / sqrt(hd)) V over positions 0 .. pos0 in y [B, h].  workspace as above. */
 int raven_qkv_attention_decode(const void* qkv, const void* qk_bias, const float* freqs, void* y,
                                const raven_kv_cache* cache, int32_t slot, int32_t B, int32_t pos0,
                                const int32_t* pos_dev, int32_t n_heads, int32_t head_dim,
-                               int32_t dtype, void* stream);
+                               int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Token embedding times sqrt(h) (RMM:667-671): out[m] = T(wte[ids[m]] * scale); ids are int64. */
 int raven_embed(const void* wte, const int64_t* ids, void* out, int32_t M, int32_t dim,

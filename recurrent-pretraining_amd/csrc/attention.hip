@@ -4,13 +4,13 @@
 // K, V = [n_slots, batch, n_heads, t_max, head_dim]; one head's positions are contiguous, so a
 // workgroup streams [positions x head_dim] with 16-byte lane-contiguous loads.
 //
-// Attention kernel: grid (heads, token rows).  A position occupies one row of 16 lanes
-// (head_dim * sizeof(T) / 16 of them active, 12 for head_dim 96 in bf16); a wave covers 4 positions
-// per load instruction and the waves of a workgroup interleave, so each load step of a workgroup
-// reads 16 or 64 consecutive positions of K and of V.  Scores are reduced with DPP row operations;
-// every 16-lane row runs its own online softmax (one max update per 4 positions) and the rows are
-// merged through LDS.  Nothing is exchanged between workgroups: a split over positions with a
-// device-scope fence per workgroup measured 10x slower than one 16-wave workgroup per head.
+// Attention kernel: a position occupies one row of 16 lanes (head_dim * sizeof(T) / 16 of them active,
+// 12 for head_dim 96 in bf16); a wave covers 4 positions per load instruction and the 4 waves of a
+// workgroup interleave, so each load step of a workgroup reads 16 consecutive positions of K and of V.
+// Scores are reduced with DPP row operations; every 16-lane row runs its own online softmax (one max
+// update per 4 positions) and the rows are merged through LDS.  Small batches split the positions over
+// several workgroups and merge the partials in a second, tiny launch: a merge inside the kernel needs a
+// device-scope fence per workgroup, which measured 10x slower on this part than the extra launch.
 
 #include <math.h>
 
@@ -69,6 +69,9 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(
 
 // ------------------------------------------------------------------------------------------------
 constexpr int kAttnMaxHd = 128;
+}  // namespace raven
+extern "C" size_t raven_decode_attention_workspace_bytes(int32_t M, int32_t n_heads, int32_t head_dim);
+namespace raven {
 
 // bias + RoPE of one 16-byte chunk of a q or k head row (sec 0 = q, 1 = k); d = first column of the chunk
 template <typename T>
@@ -91,27 +94,31 @@ __device__ __forceinline__ Chunk<T> bias_rope_chunk(Chunk<T> x, const T* __restr
     return x;
 }
 
-// One workgroup per (head, token row): no split over positions, so nothing crosses workgroups.
-// WAVES = 16 when there are few (head, row) pairs (a CU then keeps 16 waves of loads in flight for its
-// head), 4 otherwise.  FUSED (decode, S == 1): q, and the new position's k and v, come straight from the
-// fused qkv GEMM output -- bias and RoPE are applied here, the new k/v row is written to the cache by
-// this workgroup and used from registers.
-template <typename T, int WAVES, bool FUSED>
-__global__ __launch_bounds__(WAVES * 64) void decode_attention_kernel(
+// Grid (heads, token rows, splits).  With one split a workgroup owns a whole (head, row) and writes y.
+// With several (few heads x rows, i.e. small batches: one CU cannot pull a head's K/V fast enough) each
+// workgroup covers a contiguous range of positions with all of its loads in flight at once and writes
+// an fp32 partial (max, sum, unnormalised output); combine_kernel, the next launch on the stream, merges
+// them -- the kernel boundary is the only synchronisation.  FUSED (decode, S == 1): q, and the new
+// position's k and v, come straight from the fused qkv GEMM output -- bias and RoPE are applied here,
+// the new k/v row is written to the cache by the workgroup whose range holds it and used from registers.
+template <typename T, bool FUSED>
+__global__ __launch_bounds__(256) void decode_attention_kernel(
     const T* __restrict__ q_or_qkv, const T* __restrict__ qk_bias, const float* __restrict__ freqs, T* __restrict__ y,
-    CacheView cv, int S, int pos0, const int* __restrict__ pos_dev, float scale_log2) {
+    CacheView cv, int S, int pos0, const int* __restrict__ pos_dev, float scale_log2, int n_splits,
+    float* __restrict__ ws_ml, float* __restrict__ ws_o) {
     constexpr int E = Chunk<T>::N;
-    constexpr int G = WAVES * 4;  // 16-lane rows in the workgroup
-    // positions per row and loop iteration: a lone 16-wave workgroup per CU needs every load it can keep in flight
-    constexpr int kAttnU = WAVES == 16 ? 6 : 4;
+    constexpr int G = 16;      // 16-lane rows in the workgroup
+    constexpr int kAttnU = 4;  // positions per row and loop iteration
     __shared__ float sm_m[G], sm_l[G];
     __shared__ float sm_o[G][kAttnMaxHd];
 
-    const int head = blockIdx.x, m = blockIdx.y;
+    const int head = blockIdx.x, m = blockIdx.y, split = blockIdx.z;
     const int hd = cv.hd, h = cv.nh * hd;
     const int b = m / S, s = m - b * S;
     const int pos = (pos_dev ? *pos_dev : pos0) + s;  // position of this row's own token
     const int len = min(pos + 1, cv.t_max);
+    const int per = (len + n_splits - 1) / n_splits;
+    const int start = split * per, end = min(len, start + per);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane >> 4, ci = lane & 15;
@@ -123,36 +130,26 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attention_kernel(
     const T* Kb = static_cast<const T*>(cv.k) + head_off + ci * E;
     const T* Vb = static_cast<const T*>(cv.v) + head_off + ci * E;
 
-    Chunk<T> qc = zero_chunk<T>(), knew = zero_chunk<T>(), vnew = zero_chunk<T>();
+    // q (and the new k, v) first: these loads are the oldest, so their data is back before the K/V tiles
+    Chunk<T> qraw = zero_chunk<T>(), kraw = zero_chunk<T>(), vnew = zero_chunk<T>();
+    const int col = head * hd + ci * E;
     if (active) {
-        const int col = head * hd + ci * E;
         if (FUSED) {
             const T* row = q_or_qkv + (int64_t)m * 3 * h;
-            qc = bias_rope_chunk<T>(load_chunk(row + col), qk_bias, 0, h, col, freqs, pos, hd, ci * E);
-            knew = bias_rope_chunk<T>(load_chunk(row + h + col), qk_bias, 1, h, col, freqs, pos, hd, ci * E);
+            qraw = load_chunk(row + col);
+            kraw = load_chunk(row + h + col);
             vnew = load_chunk(row + 2 * h + col);
-            if (group == 0 && pos < cv.t_max) {
-                store_chunk(static_cast<T*>(cv.k) + head_off + (int64_t)pos * hd + ci * E, knew);
-                store_chunk(static_cast<T*>(cv.v) + head_off + (int64_t)pos * hd + ci * E, vnew);
-            }
         } else {
-            qc = load_chunk(q_or_qkv + (int64_t)m * h + col);
+            qraw = load_chunk(q_or_qkv + (int64_t)m * h + col);
         }
     }
-
-    float m_run = -INFINITY, l_run = 0.f, o[E];
-#pragma unroll
-    for (int e = 0; e < E; ++e) o[e] = 0.f;
-
-    for (int base = 0; base < len; base += G * kAttnU) {  // trip count is uniform over the workgroup
-        Chunk<T> kc[kAttnU], vc[kAttnU];
+    // first K/V tile, requested before q is touched
+    Chunk<T> kc[kAttnU], vc[kAttnU];
+    auto load_tile = [&](int base) {
 #pragma unroll
         for (int j = 0; j < kAttnU; ++j) {
             const int p = base + j * G + group;
-            if (FUSED && p == pos) {
-                kc[j] = knew;
-                vc[j] = vnew;
-            } else if (active && p < len) {
+            if (active && p < end && !(FUSED && p == pos)) {
                 kc[j] = load_chunk(Kb + (int64_t)p * hd);
                 vc[j] = load_chunk(Vb + (int64_t)p * hd);
             } else {
@@ -160,12 +157,35 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attention_kernel(
                 vc[j] = zero_chunk<T>();
             }
         }
+    };
+    load_tile(start);
+
+    Chunk<T> qc = qraw, knew = kraw;
+    if (FUSED && active) {
+        qc = bias_rope_chunk<T>(qraw, qk_bias, 0, h, col, freqs, pos, hd, ci * E);
+        knew = bias_rope_chunk<T>(kraw, qk_bias, 1, h, col, freqs, pos, hd, ci * E);
+        if (group == 0 && pos >= start && pos < end) {
+            store_chunk(static_cast<T*>(cv.k) + head_off + (int64_t)pos * hd + ci * E, knew);
+            store_chunk(static_cast<T*>(cv.v) + head_off + (int64_t)pos * hd + ci * E, vnew);
+        }
+    }
+
+    float m_run = -INFINITY, l_run = 0.f, o[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) o[e] = 0.f;
+
+    for (int base = start; base < end; base += G * kAttnU) {  // trip count is uniform over the workgroup
+        if (base != start) load_tile(base);
         float sc[kAttnU], m_new = m_run;
 #pragma unroll
         for (int j = 0; j < kAttnU; ++j) {
             const int p = base + j * G + group;
+            if (FUSED && p == pos) {
+                kc[j] = knew;
+                vc[j] = vnew;
+            }
             sc[j] = row16_sum(dot_chunk(qc, kc[j], 0.f)) * scale_log2;
-            if (p >= len) sc[j] = -INFINITY;
+            if (p >= end) sc[j] = -INFINITY;
             m_new = fmaxf(m_new, sc[j]);
         }
         if (m_new == -INFINITY) continue;  // this row has not seen a valid position yet
@@ -200,16 +220,56 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attention_kernel(
     const int t = threadIdx.x;
     if (t < hd) {
         float M = -INFINITY, L = 0.f, O = 0.f;
-#pragma unroll 8
+#pragma unroll
         for (int g = 0; g < G; ++g) M = fmaxf(M, sm_m[g]);
-#pragma unroll 8
+#pragma unroll
         for (int g = 0; g < G; ++g) {
             const float wgt = (sm_m[g] == -INFINITY) ? 0.f : exp2f(sm_m[g] - M);
             L += sm_l[g] * wgt;
             O += sm_o[g][t] * wgt;
         }
-        y[(int64_t)m * h + head * hd + t] = from_f32<T>(O / L);
+        if (n_splits == 1) {
+            y[(int64_t)m * h + head * hd + t] = from_f32<T>(O / L);
+        } else {
+            const int64_t idx = ((int64_t)m * cv.nh + head) * n_splits + split;
+            ws_o[idx * hd + t] = O;
+            if (t == 0) {
+                ws_ml[idx * 2] = M;
+                ws_ml[idx * 2 + 1] = L;
+            }
+        }
     }
+}
+
+// y[m, head] = sum_s w_s O_s / sum_s w_s L_s with w_s = 2^(M_s - max M); grid (heads, rows), hd threads
+template <typename T>
+__global__ __launch_bounds__(128) void attention_combine_kernel(const float* __restrict__ ws_ml, const float* __restrict__ ws_o,
+                                                                T* __restrict__ y, int nh, int hd, int n_splits) {
+    const int head = blockIdx.x, m = blockIdx.y, t = threadIdx.x;
+    if (t >= hd) return;
+    const int64_t mh = (int64_t)m * nh + head;
+    float Mg = -INFINITY;
+    for (int sp = 0; sp < n_splits; ++sp) Mg = fmaxf(Mg, ws_ml[(mh * n_splits + sp) * 2]);
+    float Lg = 0.f, Og = 0.f;
+    for (int sp = 0; sp < n_splits; ++sp) {
+        const float ms = ws_ml[(mh * n_splits + sp) * 2];
+        const float wgt = (ms == -INFINITY) ? 0.f : exp2f(ms - Mg);
+        Lg += ws_ml[(mh * n_splits + sp) * 2 + 1] * wgt;
+        Og += ws_o[(mh * n_splits + sp) * hd + t] * wgt;
+    }
+    y[(int64_t)m * nh * hd + head * hd + t] = from_f32<T>(Og / Lg);
+}
+
+constexpr int kAttnMaxSplits = 32;
+
+// Splits are worth their extra launch only while heads x rows cannot fill the chip.
+static int splits_for(int M, int nh, int len_hint) {
+    if ((int64_t)M * nh >= 512) return 1;
+    int ns = (len_hint + 63) / 64;  // 64 positions per workgroup keeps every load in one round trip
+    const int cap = (2048 + M * nh - 1) / (M * nh);
+    if (ns > cap) ns = cap;
+    if (ns > kAttnMaxSplits) ns = kAttnMaxSplits;
+    return ns < 1 ? 1 : ns;
 }
 
 static int make_view(const char* who, const raven_kv_cache* cache, int slot, int B, int nh, int hd, CacheView* cv) {
@@ -262,22 +322,20 @@ extern "C" int raven_qkv_bias_rope_cache_append(const void* qkv, const void* qk_
 
 template <typename T>
 static void launch_attention(bool fused, const void* q, const void* bias, const float* freqs, void* y, const raven::CacheView& cv,
-                             int S, int M, int pos0, const int32_t* pos_dev, float scale_log2, hipStream_t s) {
+                             int S, int M, int pos0, const int32_t* pos_dev, float scale_log2, int ns, float* ws_ml, float* ws_o,
+                             hipStream_t s) {
     using namespace raven;
-    const dim3 grid(cv.nh, M);
-    const bool wide = (int64_t)cv.nh * M < 1024;
-    if (fused) {
-        if (wide) decode_attention_kernel<T, 16, true><<<grid, dim3(1024), 0, s>>>((const T*)q, (const T*)bias, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2);
-        else      decode_attention_kernel<T, 4, true><<<grid, dim3(256), 0, s>>>((const T*)q, (const T*)bias, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2);
-    } else {
-        if (wide) decode_attention_kernel<T, 16, false><<<grid, dim3(1024), 0, s>>>((const T*)q, nullptr, nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2);
-        else      decode_attention_kernel<T, 4, false><<<grid, dim3(256), 0, s>>>((const T*)q, nullptr, nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2);
-    }
+    const dim3 grid(cv.nh, M, ns);
+    if (fused)
+        decode_attention_kernel<T, true><<<grid, dim3(256), 0, s>>>((const T*)q, (const T*)bias, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
+    else
+        decode_attention_kernel<T, false><<<grid, dim3(256), 0, s>>>((const T*)q, nullptr, nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
+    if (ns > 1) attention_combine_kernel<T><<<dim3(cv.nh, M), dim3(128), 0, s>>>(ws_ml, ws_o, (T*)y, cv.nh, cv.hd, ns);
 }
 
 static int attention_common(const char* who, bool fused, const void* q, const void* bias, const float* freqs, void* y,
                             const raven_kv_cache* cache, int slot, int B, int S, int pos0, const int32_t* pos_dev, int n_heads,
-                            int head_dim, int dtype, void* stream) {
+                            int head_dim, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
     using namespace raven;
     if (int rc = check_heads(who, n_heads, head_dim, dtype)) return rc;
     RAVEN_REQUIRE(q && y, "%s: null pointer", who);
@@ -288,24 +346,44 @@ static int attention_common(const char* who, bool fused, const void* q, const vo
     RAVEN_REQUIRE(pos0 + S <= cv.t_max, "%s: positions up to %d exceed the cache length %d", who, pos0 + S - 1, cv.t_max);
     const int M = B * S;
     RAVEN_REQUIRE(M <= 65535, "%s: too many token rows (%d)", who, M);
+    int ns = splits_for(M, n_heads, pos0 + S);
+    float *ws_ml = nullptr, *ws_o = nullptr;
+    if (ns > 1) {
+        const size_t need = raven_decode_attention_workspace_bytes(M, n_heads, head_dim);
+        if (workspace == nullptr || workspace_bytes < need) {
+            ns = 1;  // no room for partials: one workgroup per (head, row) still gives the same result
+        } else {
+            RAVEN_REQUIRE(((uintptr_t)workspace & 255) == 0, "%s: workspace must be 256-byte aligned", who);
+            ws_ml = static_cast<float*>(workspace);
+            ws_o = reinterpret_cast<float*>(static_cast<char*>(workspace) + raven_host::align_up((size_t)M * n_heads * kAttnMaxSplits * 2 * 4));
+        }
+    }
     const float scale_log2 = (float)(1.0 / sqrt((double)head_dim) * 1.4426950408889634);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == RAVEN_BF16) launch_attention<bf16>(fused, q, bias, freqs, y, cv, S, M, pos0, pos_dev, scale_log2, s);
-    else launch_attention<float>(fused, q, bias, freqs, y, cv, S, M, pos0, pos_dev, scale_log2, s);
+    if (dtype == RAVEN_BF16) launch_attention<bf16>(fused, q, bias, freqs, y, cv, S, M, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o, s);
+    else launch_attention<float>(fused, q, bias, freqs, y, cv, S, M, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o, s);
     return raven_host::check_launch(who);
+}
+
+extern "C" size_t raven_decode_attention_workspace_bytes(int32_t M, int32_t n_heads, int32_t head_dim) {
+    using namespace raven;
+    if (M <= 0 || n_heads <= 0 || head_dim <= 0) return 0;
+    if ((int64_t)M * n_heads >= 512) return 0;  // enough (head, row) pairs: never split
+    const size_t mh = (size_t)M * n_heads;
+    return raven_host::align_up(mh * kAttnMaxSplits * 2 * 4) + raven_host::align_up(mh * kAttnMaxSplits * head_dim * 4);
 }
 
 extern "C" int raven_decode_attention(const void* q, void* y, const raven_kv_cache* cache, int32_t slot, int32_t B,
                                       int32_t S, int32_t pos0, const int32_t* pos_dev, int32_t n_heads, int32_t head_dim,
-                                      int32_t dtype, void* stream) {
+                                      int32_t dtype, void* workspace, size_t workspace_bytes, void* stream) {
     return attention_common("decode_attention", false, q, nullptr, nullptr, y, cache, slot, B, S, pos0, pos_dev, n_heads, head_dim,
-                            dtype, stream);
+                            dtype, workspace, workspace_bytes, stream);
 }
 
 extern "C" int raven_qkv_attention_decode(const void* qkv, const void* qk_bias, const float* freqs, void* y,
                                           const raven_kv_cache* cache, int32_t slot, int32_t B, int32_t pos0,
                                           const int32_t* pos_dev, int32_t n_heads, int32_t head_dim, int32_t dtype,
-                                          void* stream) {
+                                          void* workspace, size_t workspace_bytes, void* stream) {
     return attention_common("qkv_attention_decode", true, qkv, qk_bias, freqs, y, cache, slot, B, 1, pos0, pos_dev, n_heads,
-                            head_dim, dtype, stream);
+                            head_dim, dtype, workspace, workspace_bytes, stream);
 }

@@ -21,6 +21,8 @@ namespace raven {
 
 struct BlockScratch {
     char *n1, *qkv, *q, *ya, *x1, *x2, *n3, *g, *x3, *xa, *xr;
+    void* attn_ws;
+    size_t attn_ws_bytes;
 };
 
 static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
@@ -44,6 +46,8 @@ static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
     s.x3 = take(row);
     s.xa = take(row);
     s.xr = take(row);
+    s.attn_ws_bytes = raven_decode_attention_workspace_bytes(M, d->n_heads, d->head_dim);
+    s.attn_ws = s.attn_ws_bytes ? take(s.attn_ws_bytes) : nullptr;
     if (out) *out = s;
     return off;
 }
@@ -82,11 +86,12 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
     if ((rc = raven_gemm(s.n1, w->wqkv, nullptr, s.qkv, M, 3 * h, h, dt, 0, stream))) return rc;
     if (S == 1) {  // decode: bias, RoPE, cache append and attention in one launch
         if ((rc = raven_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, cache, slot, B, pos0, pos_dev, d->n_heads,
-                                             d->head_dim, dt, stream))) return rc;
+                                             d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream))) return rc;
     } else {       // a chunk of S tokens: every row's keys must be in the cache before any row attends
         if ((rc = raven_qkv_bias_rope_cache_append(s.qkv, w->qk_bias, freqs, s.q, cache, slot, B, S, pos0, pos_dev, d->n_heads,
                                                    d->head_dim, dt, stream))) return rc;
-        if ((rc = raven_decode_attention(s.q, s.ya, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, stream))) return rc;
+        if ((rc = raven_decode_attention(s.q, s.ya, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, s.attn_ws,
+                                         s.attn_ws_bytes, stream))) return rc;
     }
     if ((rc = raven_gemm(s.ya, w->proj, x_in, s.x1, M, h, h, dt, 0, stream))) return rc;
     if ((rc = raven_rmsnorm_residual(s.x1, nullptr, w->norm_2, s.x2, nullptr, w->norm_3, s.n3, M, h, d->eps, dt, stream))) return rc;
@@ -110,7 +115,8 @@ static int run_block_one_row(const raven_dims* d, const raven_block_weights* w, 
     } else {
         if ((rc = raven_gemv_fused(x_raw, nullptr, w->norm_1, nullptr, nullptr, w->wqkv, nullptr, s.qkv, 3 * h, h, 0, eps, 0, 0, dt, stream))) return rc;
     }
-    if ((rc = raven_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, cache, slot, 1, pos0, pos_dev, d->n_heads, d->head_dim, dt, stream))) return rc;
+    if ((rc = raven_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, cache, slot, 1, pos0, pos_dev, d->n_heads, d->head_dim, dt,
+                                         s.attn_ws, s.attn_ws_bytes, stream))) return rc;
     if ((rc = raven_gemv_fused(s.ya, nullptr, nullptr, nullptr, nullptr, w->proj, x_res, s.x1, h, h, 0, eps, 0, 0, dt, stream))) return rc;
     if ((rc = raven_gemv_fused(s.x1, nullptr, w->norm_2, w->norm_3, s.x2, w->fc, nullptr, s.g, I, h, 0, eps, 1, 0, dt, stream))) return rc;
     return raven_gemv_fused(s.g, nullptr, nullptr, nullptr, nullptr, w->mlp_proj, s.x2, s.x3, h, I, 0, eps, 0, 0, dt, stream);

@@ -53,9 +53,11 @@ SIGNATURES = {
     "raven_gemv_fused": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _F, _I32, _I32, _I32, _VP]),
     "raven_qkv_bias_rope_cache_append": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32,
                                                    _VP, _I32, _I32, _I32, _VP]),
-    "raven_decode_attention": (C.c_int, [_VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _I32, _I32, _I32, _VP]),
+    "raven_decode_attention_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
+    "raven_decode_attention": (C.c_int, [_VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _I32, _I32, _I32,
+                                         _VP, _SZ, _VP]),
     "raven_qkv_attention_decode": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _VP, _I32, _I32,
-                                             _I32, _VP]),
+                                             _I32, _VP, _SZ, _VP]),
     "raven_embed": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I64, _F, _I32, _VP]),
     "raven_argmax": (C.c_int, [_VP, _VP, _I32, _I64, _VP]),
     "raven_advance_pos": (C.c_int, [_VP, _I32, _VP]),
@@ -218,22 +220,30 @@ def qkv_bias_rope_cache_append(qkv, qk_bias, freqs, cache: KVCache, slot, B, S, 
     return q
 
 
-def decode_attention(q, cache: KVCache, slot, B, S, pos0, n_heads, head_dim, pos_dev=None):
+def attention_workspace(M, n_heads, head_dim, device):
+    """Scratch for split partials (None when the shape never splits)."""
+    n = load().raven_decode_attention_workspace_bytes(M, n_heads, head_dim)
+    return torch.empty(n, dtype=torch.uint8, device=device) if n else None
+
+
+def decode_attention(q, cache: KVCache, slot, B, S, pos0, n_heads, head_dim, pos_dev=None, workspace=None):
     y = torch.empty_like(q)
     rc = load().raven_decode_attention(
         _ptr(q, "q"), _ptr(y, "y"), C.byref(cache), slot, B, S, pos0, _ptr(pos_dev, "pos_dev", torch.int32),
-        n_heads, head_dim, dtype_code(q.dtype), _stream())
+        n_heads, head_dim, dtype_code(q.dtype), _ptr(workspace, "workspace", torch.uint8),
+        0 if workspace is None else workspace.numel(), _stream())
     _check(rc, "raven_decode_attention")
     return y
 
 
-def qkv_attention_decode(qkv, qk_bias, freqs, cache: KVCache, slot, B, pos0, n_heads, head_dim, pos_dev=None):
+def qkv_attention_decode(qkv, qk_bias, freqs, cache: KVCache, slot, B, pos0, n_heads, head_dim, pos_dev=None, workspace=None):
     """Decode step: fused qkv rows [B, 3h] -> attention output [B, h]; appends k, v at pos0."""
     dt = qkv.dtype
     y = torch.empty(B, n_heads * head_dim, device=qkv.device, dtype=dt)
     rc = load().raven_qkv_attention_decode(
         _ptr(qkv, "qkv"), _ptr(qk_bias, "qk_bias", dt), _ptr(freqs, "freqs", torch.float32), _ptr(y, "y"), C.byref(cache),
-        slot, B, pos0, _ptr(pos_dev, "pos_dev", torch.int32), n_heads, head_dim, dtype_code(dt), _stream())
+        slot, B, pos0, _ptr(pos_dev, "pos_dev", torch.int32), n_heads, head_dim, dtype_code(dt),
+        _ptr(workspace, "workspace", torch.uint8), 0 if workspace is None else workspace.numel(), _stream())
     _check(rc, "raven_qkv_attention_decode")
     return y
 

@@ -242,7 +242,8 @@ def test_decode_attention(pkg, dt, nh, hd, B, S, pos0):
     t_max = 1024
     k, v, kd, vd, cache = make_cache(pkg, 2, B, nh, t_max, hd, dt, fill_seed=90)
     q = rnd((B * S, nh * hd), dt, 92)
-    y = pkg.hip.decode_attention(q.cuda(), cache, 1, B, S, pos0, nh, hd)
+    ws = pkg.hip.attention_workspace(B * S, nh, hd, "cuda")
+    y = pkg.hip.decode_attention(q.cuda(), cache, 1, B, S, pos0, nh, hd, workspace=ws)
     T = pos0 + S
     qq = q.view(B, S, nh, hd).transpose(1, 2)
     want = O.sdpa(qq, k[1, :, :, :T], v[1, :, :, :T]).transpose(1, 2).reshape(B * S, nh * hd)
@@ -254,8 +255,11 @@ def test_decode_attention(pkg, dt, nh, hd, B, S, pos0):
         check(y.view(B, nh, hd), v[1, :, :, 0], dt, "T=1 returns v")
     # the device-side position overrides the by-value one
     pos_dev = torch.tensor([pos0], dtype=torch.int32, device="cuda")
-    y2 = pkg.hip.decode_attention(q.cuda(), cache, 1, B, S, t_max - S, nh, hd, pos_dev=pos_dev)
-    assert torch.equal(y2, y), "device-side position must give the identical result"
+    y2 = pkg.hip.decode_attention(q.cuda(), cache, 1, B, S, t_max - S, nh, hd, pos_dev=pos_dev, workspace=ws)
+    check(y2, want, dt, "attention, device-side position (the split count follows the by-value hint)")
+    # without a workspace nothing is split; same values up to the order of the merge
+    y3 = pkg.hip.decode_attention(q.cuda(), cache, 1, B, S, pos0, nh, hd)
+    check(y3, want, dt, "attention without workspace")
 
 
 @pytest.mark.parametrize("dt,nh,hd,B,pos0", [(torch.bfloat16, 55, 96, 1, 1023), (torch.bfloat16, 55, 96, 32, 600),
@@ -270,9 +274,10 @@ def test_qkv_attention_decode_fused(pkg, dt, nh, hd, B, pos0):
     freqs = table.float().reshape(t_max, hd // 2, 2).contiguous().cuda()
     k, v, kd, vd, cache = make_cache(pkg, 2, B, nh, t_max, hd, dt, fill_seed=112)
     k2, v2, kd2, vd2, cache2 = make_cache(pkg, 2, B, nh, t_max, hd, dt, fill_seed=112)
-    y = pkg.hip.qkv_attention_decode(qkv.cuda(), bias.cuda(), freqs, cache, 1, B, pos0, nh, hd)
+    ws = pkg.hip.attention_workspace(B, nh, hd, "cuda")
+    y = pkg.hip.qkv_attention_decode(qkv.cuda(), bias.cuda(), freqs, cache, 1, B, pos0, nh, hd, workspace=ws)
     q = pkg.hip.qkv_bias_rope_cache_append(qkv.cuda(), bias.cuda(), freqs, cache2, 1, B, 1, pos0, nh, hd)
-    y_two = pkg.hip.decode_attention(q, cache2, 1, B, 1, pos0, nh, hd)
+    y_two = pkg.hip.decode_attention(q, cache2, 1, B, 1, pos0, nh, hd, workspace=ws)
     assert torch.equal(kd, kd2) and torch.equal(vd, vd2), "fused and two-step paths must write the same cache bytes"
     check(y, y_two, dt, "fused vs two-step")
     qq, kk, vv = (t.view(B, 1, nh, hd) for t in qkv.view(B, 1, 3 * h).split([h, h, h], dim=2))
@@ -283,8 +288,10 @@ def test_qkv_attention_decode_fused(pkg, dt, nh, hd, B, pos0):
     want = O.sdpa(rq.transpose(1, 2), K, V).transpose(1, 2).reshape(B, h)
     check(y, want, dt, "fused decode attention vs oracle")
     pos_dev = torch.tensor([pos0], dtype=torch.int32, device="cuda")
-    y3 = pkg.hip.qkv_attention_decode(qkv.cuda(), bias.cuda(), freqs, cache, 1, B, t_max - 1, nh, hd, pos_dev=pos_dev)
-    assert torch.equal(y3, y)
+    y3 = pkg.hip.qkv_attention_decode(qkv.cuda(), bias.cuda(), freqs, cache, 1, B, t_max - 1, nh, hd, pos_dev=pos_dev, workspace=ws)
+    check(y3, want, dt, "fused decode attention, device-side position")
+    y4 = pkg.hip.qkv_attention_decode(qkv.cuda(), bias.cuda(), freqs, cache, 1, B, pos0, nh, hd)
+    check(y4, want, dt, "fused decode attention without workspace")
 
 
 def test_decode_attention_zero_query_gives_mean(pkg):
