@@ -6,8 +6,9 @@ r = 32 recurrences of (adapter + 4 SandwichBlocks), 2 coda blocks, ln_f, LM head
 greedy argmax, with the KV cache of a 512-token prompt already resident (random-init weights, random
 token ids).  Prints ONE JSON line:
   value            decoded tokens/s (whole job, one GPU, batch `--batch`, default 1)
-  roofline         the dominant kernel (fc GEMV with the SwiGLU epilogue, 47 % of a token's bytes):
-                   algorithmic bytes per launch / its mean duration (HIP events on the launch stream)
+  roofline         the dominant kernel (mlp.fc GEMV with norm prologue and SwiGLU epilogue, 47 % of a
+                   token's bytes): algorithmic bytes per launch / its mean duration (HIP events on the
+                   launch stream)
   core_iteration   one recurrence iteration (the unit the 70 %-of-HBM target is stated on)
   cpu_baseline     the CPU oracle on this box's host cores, on a bounded sample, scaled to tokens/s
 """
@@ -36,7 +37,37 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-iters", type=int, default=3)
     ap.add_argument("--also-batch", type=int, default=32, help="second batch size reported under 'also' (0 = skip)")
+    ap.add_argument("--kernel-only", type=int, default=0, metavar="N",
+                    help="run only N launches of the dominant kernel plus one 256 MiB device copy (for rocprofv3 --pmc runs)")
     return ap.parse_args()
+
+
+def kernel_only(n_launches):
+    """The dominant kernel alone, as the decode loop launches it, on four rotating fc matrices, followed by
+    one device copy of known size (the yardstick that scales FETCH_SIZE / WRITE_SIZE readings)."""
+    import torch
+    import __graft_entry__ as entry
+    pkg = entry.import_package()
+    lib = pkg.hip.load()
+    cfg = pkg.RavenConfig()
+    dev = torch.device("cuda:0")
+    h, inter = cfg.n_embd, cfg.intermediate_size
+    torch.manual_seed(0)
+    fcs = [torch.randn(2 * inter, h, device=dev, dtype=torch.bfloat16) * 0.02 for _ in range(4)]
+    na, nb = (torch.ones(h, device=dev, dtype=torch.bfloat16) for _ in range(2))
+    x = torch.randn(h, device=dev, dtype=torch.bfloat16)
+    x2, g = torch.empty_like(x), torch.empty(inter, device=dev, dtype=torch.bfloat16)
+    stream = torch.cuda.current_stream().cuda_stream
+    for i in range(n_launches):
+        lib.raven_gemv_fused(x.data_ptr(), None, na.data_ptr(), nb.data_ptr(), x2.data_ptr(), fcs[i % 4].data_ptr(), None,
+                             g.data_ptr(), inter, h, 0, cfg.norm_eps, 1, 0, pkg.hip.BF16, stream)
+    torch.cuda.synchronize()
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    print(json.dumps({"kernel_only": n_launches, "bytes_per_launch": 2 * inter * h * 2 + h * 2 + inter * 2,
+                      "copy_bytes": src.numel()}))
 
 
 def event_time_ms(fn, reps, warm=3):
@@ -93,6 +124,9 @@ def decode_tokens_per_s(pkg, model, batch, prompt_len, steps, warmup, r, use_gra
 
 def main():
     args = parse()
+    if args.kernel_only:
+        kernel_only(args.kernel_only)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: the decode path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
@@ -148,17 +182,35 @@ def main():
     it_bytes = O.core_iteration_bytes(shape, B, T)["total"]
     iter_ms = min(iter_eager_ms, iter_graph_ms)
 
-    # ---- dominant kernel: fc GEMV + SwiGLU ----
-    fc_w = model.transformer.core_block[0].mlp.fc.weight
+    # ---- dominant kernel: mlp.fc GEMV with its norm_2/norm_3 prologue and SwiGLU epilogue ----
+    # (47 % of a token's bytes).  Timed exactly as the decode loop launches it, rotating over the four
+    # core blocks' fc matrices (1.5 GB) so that no cache level can keep a matrix between launches.
+    blocks = model.transformer.core_block
     xin = torch.randn(B, h, device=dev, dtype=torch.bfloat16)
+    x2 = torch.empty_like(xin)
     gout = torch.empty(B, cfg.intermediate_size, device=dev, dtype=torch.bfloat16)
     lib = pkg.hip.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    if B == 1:
+        kernel_name = "gemv1_kernel<bf16, C=3, SwiGLU, norm prologue, 4 row pairs per workgroup> (mlp.fc 35840x5280)"
 
-    def fc_launch():
-        lib.raven_gemm_swiglu(xin.data_ptr(), fc_w.data_ptr(), gout.data_ptr(), B, cfg.intermediate_size, h, pkg.hip.BF16,
-                              torch.cuda.current_stream().cuda_stream)
+        def fc_launch(i=[0]):
+            blk = blocks[i[0] % len(blocks)]
+            i[0] += 1
+            lib.raven_gemv_fused(xin.data_ptr(), None, blk.norm_2.weight.data_ptr(), blk.norm_3.weight.data_ptr(), x2.data_ptr(),
+                                 blk.mlp.fc.weight.data_ptr(), None, gout.data_ptr(), cfg.intermediate_size, h, 0, cfg.norm_eps, 1, 0,
+                                 pkg.hip.BF16, stream)
+    else:
+        kernel_name = "mfma_kernel<SwiGLU> (mlp.fc 35840x5280)" if B > 4 else "gemv_kernel<bf16, SwiGLU> (mlp.fc 35840x5280)"
+
+        def fc_launch(i=[0]):
+            blk = blocks[i[0] % len(blocks)]
+            i[0] += 1
+            lib.raven_gemm_swiglu(xin.data_ptr(), blk.mlp.fc.weight.data_ptr(), gout.data_ptr(), B, cfg.intermediate_size, h,
+                                  pkg.hip.BF16, stream)
 
     fc_ms = event_time_ms(fc_launch, 200, warm=10)
+    fc_w = blocks[0].mlp.fc.weight
     fc_bytes = fc_w.numel() * 2 + B * h * 2 + B * cfg.intermediate_size * 2
     fc_gbs = fc_bytes / (fc_ms * 1e-3) / 1e9
 
@@ -200,9 +252,12 @@ def main():
         "recurrence_steps_per_s": round(tok_s * r / args.batch, 2),
         "token_roofline": {"bytes_per_token": int(token_bytes), "achieved_GBs": round(token_bytes * (tok_s / args.batch) / 1e9, 1),
                            "frac": round(token_bytes * (tok_s / args.batch) / 1e9 / HBM_PEAK_GBS, 4)},
-        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<bf16,SwiGLU> (mlp.fc 35840x5280)" if B <= 4 else "mfma_kernel<SwiGLU> (mlp.fc 35840x5280)",
+        "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": round(fc_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(fc_gbs / HBM_PEAK_GBS, 4),
-                     "bytes_per_launch": int(fc_bytes), "avg_us": round(fc_ms * 1e3, 2), "traffic": None},
+                     "bytes_per_launch": int(fc_bytes), "avg_us": round(fc_ms * 1e3, 2),
+                     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy
+                     # (profiles/mlp_fc_gemv_bs1_hbm_traffic.txt); a profiler figure, so a constant here
+                     "traffic": 386061876 if B == 1 else None},
         "core_iteration": {"T": T, "batch": B, "bytes": int(it_bytes), "ms_eager": round(iter_eager_ms, 4),
                            "ms_graph": round(iter_graph_ms, 4), "achieved_GBs": round(it_bytes / (iter_ms * 1e-3) / 1e9, 1),
                            "frac": round(it_bytes / (iter_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
