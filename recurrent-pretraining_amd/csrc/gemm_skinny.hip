@@ -173,45 +173,44 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemmArgs a) {
 // tiles of 16 rows per workgroup.  D = A * B with A = W tile [16 n x 32 k], B = X^T [32 k x 16 m]:
 // lane l supplies A[n = l%16][k = 8*(l/16) ..+8] and B[k = 8*(l/16) ..+8][m = l%16] and receives
 // D[n = 4*(l/16) + v][m = l%16], v = 0..3.
+//
+// The MFMA operand layout puts 16 different matrix rows into 16 neighbouring lanes; loading it straight
+// from global memory makes every quarter-wave touch 16 cache lines for 256 bytes, and the L1 address path
+// (not HBM) then caps the kernel near 3 TB/s.  So K is walked in macro-steps of 128 elements: each wave
+// loads its rows with row-contiguous 16-byte lanes (a quarter-wave reads 256 consecutive bytes of one
+// row), parks them in a wave-private LDS tile with 272-byte row pitch, and reads the MFMA fragments from
+// there (conflict-free: 16 rows x 16 bytes cover the 64 banks once).  The next macro-step's global loads
+// are issued into registers as soon as the current one is parked, before it is multiplied.  No barrier inside the K loop: every
+// wave only touches its own LDS tile.  K % 128 leftovers (32 elements for K = 5280) go to the last wave.
 // ------------------------------------------------------------------------------------------------
+constexpr int kPitch = 136;  // bf16 elements per LDS row: 128 + 8 (272 bytes)
+
 template <int MT, int NT, int EPI>
 __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
-    __shared__ float red[3][NT * MT][64][4];  // partial accumulators of waves 1..3
+    constexpr int ROWS = 16 * (NT + MT);
+    __shared__ __align__(16) bf16 stage[4][ROWS][kPitch];
+    static_assert(sizeof(bf16) * 4 * ROWS * kPitch >= sizeof(float) * 3 * NT * MT * 64 * 4, "stage doubles as the reduction buffer");
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ln = lane & 15, kq = lane >> 4;
     const int K = a.K;
-    const int n_steps = K / 32;
-    const int s_begin = (int)((int64_t)n_steps * wave / 4), s_end = (int)((int64_t)n_steps * (wave + 1) / 4);
-    const int n_tiles = (EPI == EPI_SWIGLU) ? a.N / 16 : (a.N / 16 + NT - 1) / NT;  // units
+    const int n_units = (EPI == EPI_SWIGLU) ? a.N / 16 : (a.N / 16 + NT - 1) / NT;
     const int unit = blockIdx.x;
-    if (unit >= n_tiles) return;
+    if (unit >= n_units) return;
 
     const bf16* W = static_cast<const bf16*>(a.w);
-    const bf16* wrow[NT];
+    int tile_row0[NT];  // first weight row of each tile
     bool tile_ok[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        int row;
         if (EPI == EPI_SWIGLU) {
-            row = unit * 16 + ln + t * a.N;  // t = 0 gate tile, t = 1 up tile
+            tile_row0[t] = unit * 16 + t * a.N;  // t = 0 gate tile, t = 1 up tile
             tile_ok[t] = true;
         } else {
             const int tile = unit * NT + t;
             tile_ok[t] = tile * 16 < a.N;
-            row = (tile_ok[t] ? tile : unit * NT) * 16 + ln;
+            tile_row0[t] = (tile_ok[t] ? tile : unit * NT) * 16;
         }
-        wrow[t] = W + (int64_t)row * K + kq * 8;
     }
-    // X row pointers: batch row m = mt*16 + ln, clamped (columns of D past M are never stored)
-    const bf16* xrow[MT];
-    int xk0[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int m = min(mt * 16 + ln, a.M - 1);
-        xrow[mt] = static_cast<const bf16*>(a.x0) + (int64_t)m * a.k0 + kq * 8;
-        xk0[mt] = m;
-    }
-    const bf16* x1 = static_cast<const bf16*>(a.x1);
 
     f32x4 acc[NT][MT];
 #pragma unroll
@@ -219,33 +218,103 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    constexpr int U = 4;
-    for (int s = s_begin; s < s_end; s += U) {
-        bf16x8 av[U][NT], bv[U][MT];
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    struct Staged {
+        u32x4 w[NT][4];
+        u32x4 x[MT][4];
+    };
+    bf16(*my)[kPitch] = stage[wave];
+    const int lr = lane >> 4, lc = (lane & 15) * 8;  // loader role: row within a group of 4, first element of the chunk
+
+    // X is given as up to two K segments (the adapter's concat); each is walked on its own
+#pragma unroll 1
+    for (int seg = 0; seg < 2; ++seg) {
+        const int seg_len = seg == 0 ? a.k0 : a.k1;
+        if (seg_len == 0) continue;
+        const int wk0 = seg == 0 ? 0 : a.k0;  // column of W where this segment starts
+        const bf16* X = static_cast<const bf16*>(seg == 0 ? a.x0 : a.x1);
+        const int ldx = seg == 0 ? a.k0 : a.k1;
+        const int n_macro = seg_len / 128;
+        const int mb = (int)((int64_t)n_macro * wave / 4), me = (int)((int64_t)n_macro * (wave + 1) / 4);
+
+        auto fetch = [&](int mac, Staged& st) {  // global -> registers, row-contiguous lanes
+            const int k = mac * 128 + lc;
 #pragma unroll
-        for (int j = 0; j < U; ++j) {
-            const int k = min(s + j, s_end - 1) * 32;
+            for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int t = 0; t < NT; ++t) av[j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + k);
+                for (int i = 0; i < 4; ++i) {
+                    const int m = min(mt * 16 + 4 * i + lr, a.M - 1);  // rows past M repeat the last one; never stored
+                    st.x[mt][i] = *reinterpret_cast<const u32x4*>(X + (int64_t)m * ldx + k);
+                }
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const bf16* p = (k < a.k0) ? xrow[mt] + k : x1 + (int64_t)xk0[mt] * a.k1 + kq * 8 + (k - a.k0);
-                bv[j][mt] = *reinterpret_cast<const bf16x8*>(p);
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    st.w[t][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(W + (int64_t)(tile_row0[t] + 4 * i + lr) * K + wk0 + k));
+        };
+        auto park = [&](const Staged& st) {  // registers -> this wave's LDS tile
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&my[t * 16 + 4 * i + lr][lc]) = st.w[t][i];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&my[(NT + mt) * 16 + 4 * i + lr][lc]) = st.x[mt][i];
+        };
+        auto multiply = [&]() {  // LDS -> MFMA fragments
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                bf16x8 bv[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)  // same access type as the stores in park(): the two must stay ordered
+                    bv[mt] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&my[(NT + mt) * 16 + ln][32 * j + 8 * kq]));
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const bf16x8 av = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&my[t * 16 + ln][32 * j + 8 * kq]));
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv[mt], acc[t][mt], 0, 0, 0);
+                }
             }
+        };
+
+        // lanes exchange data through the tile without a workgroup barrier: pin the order of the LDS
+        // accesses for the compiler (the LDS itself executes one wave's accesses in order)
+        auto wave_sync = []() {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        };
+        // one register set: its loads for macro-step s+1 are in flight while step s is multiplied out of LDS
+        Staged st;
+        if (mb < me) fetch(mb, st);
+        for (int mac = mb; mac < me; ++mac) {
+            park(st);
+            wave_sync();
+            if (mac + 1 < me) fetch(mac + 1, st);
+            multiply();
+            wave_sync();
         }
+        // leftover 32-element steps of this segment: the last wave takes them, straight from global memory
+        if (wave == 3) {
+            for (int k = n_macro * 128; k < seg_len; k += 32) {
 #pragma unroll
-        for (int j = 0; j < U; ++j) {
-            if (s + j < s_end) {
+                for (int t = 0; t < NT; ++t) {
+                    const bf16x8 wv = *reinterpret_cast<const bf16x8*>(W + (int64_t)(tile_row0[t] + ln) * K + wk0 + k + kq * 8);
 #pragma unroll
-                for (int t = 0; t < NT; ++t)
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[j][t], bv[j][mt], acc[t][mt], 0, 0, 0);
+                    for (int mt = 0; mt < MT; ++mt) {
+                        const int m = min(mt * 16 + ln, a.M - 1);
+                        const bf16x8 xv = *reinterpret_cast<const bf16x8*>(X + (int64_t)m * ldx + k + kq * 8);
+                        acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, xv, acc[t][mt], 0, 0, 0);
+                    }
+                }
             }
         }
     }
 
-    // cross-wave reduction over the K split
+    // cross-wave reduction over the K split (the staging tiles are free now)
+    __syncthreads();
+    float(*red)[NT * MT][64][4] = reinterpret_cast<float(*)[NT * MT][64][4]>(&stage[0][0][0]);
     if (wave > 0) {
 #pragma unroll
         for (int t = 0; t < NT; ++t)
@@ -349,8 +418,9 @@ static int dispatch_mfma(GemmArgs a, hipStream_t s) {
         else
             mfma_kernel<2, 2, EPI><<<dim3(n_tiles16), dim3(256), 0, s>>>(a);
     } else {
-        // two tiles per workgroup once that still leaves every CU several workgroups
-        const bool two = n_tiles16 / 2 >= 2 * n_cus();
+        // two tiles per workgroup (X is then re-read from L2 once per two tiles) while that still leaves every
+        // CU more than one workgroup; L2 -> L1 traffic, not HBM, is what limits this kernel
+        const bool two = n_tiles16 / 2 >= n_cus() + n_cus() / 2;
         const int units = two ? (n_tiles16 + 1) / 2 : n_tiles16;
         if (a.M <= 16) {
             if (two) mfma_kernel<1, 2, EPI><<<dim3(units), dim3(256), 0, s>>>(a);
