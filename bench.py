@@ -37,9 +37,67 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-iters", type=int, default=3)
     ap.add_argument("--also-batch", type=int, default=32, help="second batch size reported under 'also' (0 = skip)")
+    ap.add_argument("--prefill", action="store_true",
+                    help="measure the recurrent core over a whole prompt instead (bs=4 x 4096 tokens, r iterations): MFMA-bound regime")
+    ap.add_argument("--prefill-batch", type=int, default=4)
+    ap.add_argument("--prefill-len", type=int, default=4096)
     ap.add_argument("--kernel-only", type=int, default=0, metavar="N",
                     help="run only N launches of the dominant kernel plus one 256 MiB device copy (for rocprofv3 --pmc runs)")
     return ap.parse_args()
+
+
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+
+def prefill(args):
+    """BASELINE configs[4]: the recurrent core over a full prompt.  Token ids uniform over the vocabulary from seed 1,
+    random-init weights; the prelude runs once (untimed), then r core iterations over all B x S rows are timed.
+    FLOPs per iteration: GEMMs 2*M*(params of adapter + 4 blocks) + causal attention 4 * 2*B*nh*hd*S*(S+1)/2 * 2."""
+    import torch
+    import __graft_entry__ as entry
+    pkg = entry.import_package()
+    pkg.hip.load()
+    dev = torch.device("cuda:0")
+    cfg = pkg.RavenConfig()
+    r, B, S = args.recurrence, args.prefill_batch, args.prefill_len
+    model = pkg.RavenForCausalLM(cfg, device=dev, dtype=torch.bfloat16)
+    fill_synthetic(model, 0)
+    ids = torch.randint(0, cfg.vocab_size, (B, S), generator=torch.Generator().manual_seed(1)).cuda()
+    cache = pkg.HuginnDynamicCache(max_length=S)
+    cache.ensure(cfg.n_layers_in_prelude + cfg.n_layers_in_recurrent_block * r, cfg.n_layers_in_coda, B, cfg.n_heads, cfg.head_dim, S,
+                 torch.bfloat16, dev)  # all step slots up front: no reallocation inside the timed region
+    embeds, block_idx = model.embed_inputs(ids, past_key_values=cache, use_cache=True)
+    state = model.initialize_state(embeds, 1.0)
+    torch.cuda.synchronize()
+    print(f"prefill bench: prelude done, KV cache {cache.get_allocated_mb() / 1024:.1f} GiB, timing {r} iterations", file=sys.stderr, flush=True)
+    h, inter, nh, hd = cfg.n_embd, cfg.intermediate_size, cfg.n_heads, cfg.head_dim
+    M = B * S
+    gemm_flops = 2.0 * M * (2 * h * h + 4 * (3 * h * h + h * h + 2 * inter * h + inter * h))
+    attn_flops = 4 * (2.0 * 2.0 * B * nh * hd * S * (S + 1) / 2)
+    # warm-up: one iteration on a scratch copy of the step counter (uses slots of iteration 0, overwritten below)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    cache.lookup_strategy = "compress-s4"   # warm-up writes the same four slots the timed run starts with
+    model.iterate_forward(embeds, state, block_idx=block_idx, past_key_values=cache, num_steps=1)
+    cache.lookup_strategy = "full"
+    cache._filled = {k: v for k, v in cache._filled.items() if k < cfg.n_layers_in_prelude}
+    torch.cuda.synchronize()
+    a.record()
+    model.iterate_forward(embeds, state, block_idx=block_idx, past_key_values=cache, num_steps=r)
+    b.record()
+    torch.cuda.synchronize()
+    ms = a.elapsed_time(b)
+    tflops = (gemm_flops + attn_flops) * r / (ms * 1e-3) / 1e12
+    line = {
+        "metric": "core prefill tokens*iterations/s, raven-3.5b shape bf16; MFMA utilisation",
+        "value": round(M * r / (ms * 1e-3), 1), "unit": "tokens*iterations/s", "n_gpus": 1, "steps": r, "warmup": 1,
+        "ms_per_step": round(ms / r, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"recurrent-core prefill, nebel-raven-3.5b shape, bs={B} x {S} tokens, r={r} (BASELINE configs[4])",
+                   "batch": B, "seq_len": S, "recurrence": r, "gemm": "hipBLASLt via torch.matmul", "attention": "attention_prefill_kernel"},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / MFMA_PEAK_TFLOPS, 4), "flops_per_iteration": gemm_flops + attn_flops, "traffic": None},
+    }
+    print(json.dumps(line))
 
 
 def kernel_only(n_launches):
@@ -126,6 +184,9 @@ def main():
     args = parse()
     if args.kernel_only:
         kernel_only(args.kernel_only)
+        return
+    if args.prefill:
+        prefill(args)
         return
     if args.gpus != 1:
         print("bench.py measures one GPU: the decode path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)

@@ -144,6 +144,18 @@ int raven_qkv_attention_decode(const void* qkv, const void* qk_bias, const float
                                const int32_t* pos_dev, int32_t n_heads, int32_t head_dim,
                                int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Causal attention for a prefill chunk on the matrix cores (bf16; head_dim 64, 96 or 128): the S > 1
+ * cases of RMM:484-491.  Same contract as raven_decode_attention -- row m of sequence b attends to cached
+ * positions 0 .. pos0 + (m % S), the chunk's keys/values are already in the cache -- but one workgroup
+ * serves 64 query rows of a head and streams the keys once for all of them. */
+int raven_prefill_attention(const void* q, void* y, const raven_kv_cache* cache, int32_t slot,
+                            int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
+                            int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream);
+
+/* SiLU-gate of a materialised fc output (RMM:507-508): out[m, j] = T(T(silu(z[m, j])) * z[m, I + j]);
+ * z [M, 2I], out [M, I].  For callers that run mlp.fc as a library GEMM (large M). */
+int raven_swiglu(const void* z, void* out, int32_t M, int32_t I, int32_t dtype, void* stream);
+
 /* Token embedding times sqrt(h) (RMM:667-671): out[m] = T(wte[ids[m]] * scale); ids are int64. */
 int raven_embed(const void* wte, const int64_t* ids, void* out, int32_t M, int32_t dim,
                 int64_t vocab, float scale, int32_t dtype, void* stream);

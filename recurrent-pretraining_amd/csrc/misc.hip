@@ -75,6 +75,21 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ 
     }
 }
 
+// out[m, j] = T(T(silu(z[m, j])) * z[m, I + j])   (recpre/raven_modeling_minimal.py:507-508, after a library GEMM)
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ z, T* __restrict__ out, int inter) {
+    constexpr int E = Chunk<T>::N;
+    const int64_t m = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= inter / E) return;
+    const Chunk<T> g = load_chunk(z + m * 2 * inter + c * E);
+    const Chunk<T> u = load_chunk(z + m * 2 * inter + inter + c * E);
+    Chunk<T> o;
+#pragma unroll
+    for (int e = 0; e < E; ++e) o.v[e] = from_f32<T>(round_to<T>(silu_f32(to_f32(g.v[e]))) * to_f32(u.v[e]));
+    store_chunk(out + m * inter + c * E, o);
+}
+
 __global__ void advance_pos_kernel(int* pos, int delta) {
     if (threadIdx.x == 0 && blockIdx.x == 0) *pos += delta;
 }
@@ -109,6 +124,20 @@ extern "C" int raven_argmax(const float* logits, int64_t* out, int32_t M, int64_
     if (M == 0) return 0;
     argmax_kernel<<<dim3(M), dim3(1024), 0, static_cast<hipStream_t>(stream)>>>(logits, out, vocab);
     return raven_host::check_launch("argmax");
+}
+
+extern "C" int raven_swiglu(const void* z, void* out, int32_t M, int32_t I, int32_t dtype, void* stream) {
+    using namespace raven;
+    RAVEN_REQUIRE(dtype == RAVEN_F32 || dtype == RAVEN_BF16, "swiglu: unknown dtype %d", dtype);
+    if (M == 0) return 0;
+    RAVEN_REQUIRE(z && out, "swiglu: null pointer");
+    const int elts = 16 / (int)raven_host::elt_size(dtype);
+    RAVEN_REQUIRE(M > 0 && M <= 65535 && I > 0 && I % elts == 0, "swiglu: bad shape M=%d I=%d", M, I);
+    dim3 grid((I / elts + 255) / 256, M);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == RAVEN_BF16) swiglu_kernel<bf16><<<grid, dim3(256), 0, s>>>((const bf16*)z, (bf16*)out, I);
+    else swiglu_kernel<float><<<grid, dim3(256), 0, s>>>((const float*)z, (float*)out, I);
+    return raven_host::check_launch("swiglu");
 }
 
 extern "C" int raven_advance_pos(int32_t* pos_dev, int32_t delta, void* stream) {

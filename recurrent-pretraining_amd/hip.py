@@ -58,6 +58,8 @@ SIGNATURES = {
                                          _VP, _SZ, _VP]),
     "raven_qkv_attention_decode": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _VP, _I32, _I32,
                                              _I32, _VP, _SZ, _VP]),
+    "raven_prefill_attention": (C.c_int, [_VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _I32, _I32, _I32, _VP]),
+    "raven_swiglu": (C.c_int, [_VP, _VP, _I32, _I32, _I32, _VP]),
     "raven_embed": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I64, _F, _I32, _VP]),
     "raven_argmax": (C.c_int, [_VP, _VP, _I32, _I64, _VP]),
     "raven_advance_pos": (C.c_int, [_VP, _I32, _VP]),
@@ -246,6 +248,23 @@ def qkv_attention_decode(qkv, qk_bias, freqs, cache: KVCache, slot, B, pos0, n_h
         _ptr(workspace, "workspace", torch.uint8), 0 if workspace is None else workspace.numel(), _stream())
     _check(rc, "raven_qkv_attention_decode")
     return y
+
+
+def prefill_attention(q, cache: KVCache, slot, B, S, pos0, n_heads, head_dim, pos_dev=None):
+    y = torch.empty_like(q)
+    rc = load().raven_prefill_attention(
+        _ptr(q, "q"), _ptr(y, "y"), C.byref(cache), slot, B, S, pos0, _ptr(pos_dev, "pos_dev", torch.int32),
+        n_heads, head_dim, dtype_code(q.dtype), _stream())
+    _check(rc, "raven_prefill_attention")
+    return y
+
+
+def swiglu(z):
+    """z [M, 2I] -> [M, I]."""
+    M, two_i = z.shape
+    out = torch.empty(M, two_i // 2, device=z.device, dtype=z.dtype)
+    _check(load().raven_swiglu(_ptr(z, "z"), _ptr(out, "out"), M, two_i // 2, dtype_code(z.dtype), _stream()), "raven_swiglu")
+    return out
 
 
 def embed(wte, ids, scale, out=None):

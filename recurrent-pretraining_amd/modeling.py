@@ -263,11 +263,57 @@ class RavenForCausalLM(torch.nn.Module):
             return int(num_steps[0]) + int(num_steps[1])
         return int(num_steps)
 
+    # ---- many rows (prefill): library GEMMs for the five nn.Linear products, HIP kernels for the rest ----
+    WIDE_ROWS = 64  # from this many token rows on, the GEMMs are compute-bound and go to hipBLASLt via torch.matmul
+
+    def _is_wide(self, M: int) -> bool:
+        return self.dtype == torch.bfloat16 and M >= self.WIDE_ROWS and self.config.head_dim in (64, 96, 128)
+
+    def _wide_block(self, blk: "SandwichBlock", x: torch.Tensor, kv, slot: int, B: int, S: int, pos0: int,
+                    n1: Optional[torch.Tensor] = None, tail_w: Optional[torch.Tensor] = None):
+        """One SandwichBlock (RMM:525-536) on [B*S, h] rows.  Returns (block output, tail) where tail is one more
+        RMSNorm (weight tail_w: the next block's norm_1, or ln_f) of the output, fused into the closing norm launch."""
+        cfg, eps = self.config, self.config.norm_eps
+        freqs = self._natives()["freqs"]
+        if n1 is None:
+            n1 = hip.rmsnorm_residual(x, blk.norm_1.weight, eps)[0]
+        qkv = torch.matmul(n1, blk.attn.Wqkv.weight.t())
+        bias = blk.attn.qk_bias if hasattr(blk.attn, "qk_bias") else None
+        q = hip.qkv_bias_rope_cache_append(qkv, bias, freqs, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim)
+        ya = hip.prefill_attention(q, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim)
+        a = torch.matmul(ya, blk.attn.proj.weight.t())
+        x2, _, n3 = hip.rmsnorm_residual(a, blk.norm_2.weight, eps, residual=x, weight2=blk.norm_3.weight)
+        g = hip.swiglu(torch.matmul(n3, blk.mlp.fc.weight.t()))
+        m = torch.matmul(g, blk.mlp.proj.weight.t())
+        y, _, tail = hip.rmsnorm_residual(m, blk.norm_4.weight, eps, residual=x2, weight2=tail_w)
+        return y, tail
+
+    def _wide_core(self, x: torch.Tensor, embeds: torch.Tensor, slots, kv, B: int, S: int, pos0: int, ln_f: bool):
+        """One core_block_forward (RMM:764-781) on many rows."""
+        t = self.transformer
+        cur = torch.matmul(torch.cat([x, embeds], dim=-1), t.adapter.weight.t())
+        n1, out = None, cur
+        n_core = len(t.core_block)
+        for j, blk in enumerate(t.core_block):
+            last = j == n_core - 1
+            tail_w = (t.ln_f.weight if ln_f else None) if last else t.core_block[j + 1].norm_1.weight
+            cur, tail = self._wide_block(blk, cur, kv, slots[j], B, S, pos0, n1=n1, tail_w=tail_w)
+            n1 = None if last else tail
+            out = tail if (last and ln_f) else cur
+        if n_core == 0 and ln_f:
+            out = hip.rmsnorm_residual(cur, t.ln_f.weight, self.config.norm_eps)[0]
+        return out
+
     # ---- pieces of the forward --------------------------------------------------------------------
     def _run_block(self, which: str, i: int, step_idx: int, x: torch.Tensor, cache: HuginnDynamicCache, private: bool,
                    B: int, S: int, pos0: int, ln_f: bool = False) -> torch.Tensor:
         nat = self._natives()
         slot = 0 if private else cache.note_append(step_idx, S, pos0)
+        if self._is_wide(B * S):
+            blk = getattr(self.transformer, {"prelude": "prelude", "coda": "coda", "core": "core_block"}[which])[i]
+            y, tail = self._wide_block(blk, x, cache.native(), slot, B, S, pos0,
+                                       tail_w=self.transformer.ln_f.weight if ln_f else None)
+            return tail if ln_f else y
         out = torch.empty_like(x)
         hip.sandwich_block(nat["dims"], nat[which][i], x, out, nat["freqs"], cache.native(), slot, B, S, pos0,
                            self._workspace(B * S), ln_f=self.transformer.ln_f.weight if ln_f else None)
@@ -279,6 +325,8 @@ class RavenForCausalLM(torch.nn.Module):
         nat, t = self._natives(), self.transformer
         n_core = len(t.core_block)
         slots = [0 if private else cache.note_append(first_step + j, S, pos0) for j in range(n_core)]
+        if self._is_wide(B * S):
+            return self._wide_core(x, embeds, slots, cache.native(), B, S, pos0, ln_f)
         out = torch.empty_like(x)
         ws = self._workspace(B * S)
         lnw = t.ln_f.weight if ln_f else None
@@ -380,7 +428,10 @@ class RavenForCausalLM(torch.nn.Module):
         if n_coda == 0:
             x = hip.rmsnorm_residual(x, t.ln_f.weight, cfg.norm_eps)[0]
 
-        logits = hip.gemm(x, self.lm_head.weight, out_f32=True).view(B, S, -1)
+        if self._is_wide(M):
+            logits = torch.matmul(x, self.lm_head.weight.t()).float().view(B, S, -1)
+        else:
+            logits = hip.gemm(x, self.lm_head.weight, out_f32=True).view(B, S, -1)
         if labels is not None:
             loss = torch.nn.functional.cross_entropy(logits.view(-1, logits.shape[-1]), labels.view(-1), ignore_index=-100)
             log_ppl = loss.clone()

@@ -294,6 +294,36 @@ def test_qkv_attention_decode_fused(pkg, dt, nh, hd, B, pos0):
     check(y4, want, dt, "fused decode attention without workspace")
 
 
+@pytest.mark.parametrize("nh,hd,B,S,pos0", [(55, 96, 1, 512, 0), (55, 96, 2, 100, 37), (4, 64, 3, 64, 0), (3, 128, 1, 65, 200),
+                                             (55, 96, 1, 2, 5), (5, 96, 1, 300, 724)])
+def test_prefill_attention_mfma(pkg, nh, hd, B, S, pos0):
+    """The matrix-core chunk kernel against the oracle and against the per-row kernel."""
+    dt, t_max = torch.bfloat16, 1024
+    k, v, kd, vd, cache = make_cache(pkg, 2, B, nh, t_max, hd, dt, fill_seed=130)
+    q = rnd((B * S, nh * hd), dt, 132)
+    y = pkg.hip.prefill_attention(q.cuda(), cache, 1, B, S, pos0, nh, hd)
+    T = pos0 + S
+    qq = q.view(B, S, nh, hd).transpose(1, 2)
+    want = O.sdpa(qq, k[1, :, :, :T], v[1, :, :, :T]).transpose(1, 2).reshape(B * S, nh * hd)
+    check(y, want, dt, f"prefill attention B={B} S={S} pos0={pos0}")
+    y_rows = pkg.hip.decode_attention(q.cuda(), cache, 1, B, S, pos0, nh, hd)
+    check(y, y_rows, dt, "chunk kernel vs per-row kernel")
+    pos_dev = torch.tensor([pos0], dtype=torch.int32, device="cuda")
+    y2 = pkg.hip.prefill_attention(q.cuda(), cache, 1, B, S, t_max - S, nh, hd, pos_dev=pos_dev)
+    assert torch.equal(y2, y)
+    with pytest.raises(pkg.hip.RavenHipError):
+        pkg.hip.prefill_attention(q.float().cuda(), cache, 1, B, S, pos0, nh, hd)
+
+
+def test_swiglu_elementwise(pkg):
+    for dt, M, I in ((torch.bfloat16, 5, 17920), (torch.float32, 3, 704), (torch.bfloat16, 1, 8)):
+        z = rnd((M, 2 * I), dt, 140)
+        got = pkg.hip.swiglu(z.cuda())
+        check(got, F.silu(z[:, :I]) * z[:, I:], dt, "swiglu")
+        if dt == torch.bfloat16:
+            assert bool((got.cpu() == F.silu(z[:, :I]) * z[:, I:]).float().mean() > 0.99)
+
+
 def test_decode_attention_zero_query_gives_mean(pkg):
     dt, nh, hd, T = torch.bfloat16, 55, 96, 513
     k, v, kd, vd, cache = make_cache(pkg, 1, 1, nh, 1024, hd, dt, fill_seed=95)

@@ -142,6 +142,34 @@ def test_forward_tiny_bf16_matches_oracle(tiny16):
     check(got.logits, want.logits, torch.bfloat16, "bf16 logits")
 
 
+@pytest.mark.parametrize("B,S", [(1, 64), (2, 70), (1, 200)])
+def test_wide_prefill_path_bf16(pkg, tiny16, B, S):
+    """From 64 token rows on, the GEMMs go to the library and attention to the matrix-core chunk kernel:
+    same results as the oracle, and as the narrow path, then a decode token on top of the prefilled cache."""
+    s, w, model = tiny16
+    g = torch.Generator().manual_seed(S)
+    ids = torch.randint(0, s.vocab_size, (B, S + 1), generator=g)
+    states = O.initialize_state(torch.empty(B, S + 1, s.n_embd), s, 1.0, g).to(torch.bfloat16)
+    assert model._is_wide(B * S)
+    ref_cache, cache = O.DictCache(), pkg.HuginnDynamicCache()
+    want = O.forward(w, s, input_ids=ids[:, :S], input_states=states[:, :S], past_key_values=ref_cache, use_cache=True)
+    got = model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda(), past_key_values=cache, use_cache=True)
+    check(got.latent_states, want.latent_states, torch.bfloat16, "wide latents")
+    check(got.logits, want.logits, torch.bfloat16, "wide logits")
+    model.WIDE_ROWS = 1 << 30
+    try:
+        narrow = model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda())
+    finally:
+        model.WIDE_ROWS = type(model).WIDE_ROWS
+    check(got.logits, narrow.logits, torch.bfloat16, "wide vs narrow")
+    pos = torch.arange(S, S + 1)
+    want1 = O.forward(w, s, input_ids=ids[:, S:], input_states=states[:, S:], past_key_values=ref_cache, use_cache=True, cache_position=pos)
+    got1 = model(input_ids=ids[:, S:].cuda(), input_states=states[:, S:].cuda(), past_key_values=cache, use_cache=True,
+                 cache_position=pos.cuda())
+    check(got1.logits, want1.logits, torch.bfloat16, "decode after a wide prefill")
+    assert cache.get_seq_length() == ref_cache.get_seq_length() == S + 1
+
+
 def test_piecewise_surface_equals_forward(tiny32):
     """embed_inputs -> iterate_one_step x r -> predict_from_latents reproduces forward (RMM:841-934)."""
     s, w, model = tiny32
