@@ -6,7 +6,7 @@ registers this directory under that name).
 """
 
 from . import hip  # noqa: F401
-from .cache import HuginnDynamicCache, remap_step  # noqa: F401
+from .cache import HuginnDynamicCache, HuginnStaticCache, remap_step  # noqa: F401
 from .config import RavenConfig  # noqa: F401
 from .modeling import (  # noqa: F401
     CausalLMOutputRecurrentLatents,
@@ -17,6 +17,6 @@ from .modeling import (  # noqa: F401
 )
 
 __all__ = [
-    "hip", "HuginnDynamicCache", "remap_step", "RavenConfig", "RavenForCausalLM", "DecodeRunner",
+    "hip", "HuginnDynamicCache", "HuginnStaticCache", "remap_step", "RavenConfig", "RavenForCausalLM", "DecodeRunner",
     "CausalLMOutputRecurrentLatents", "GenerationSettings", "precompute_freqs_cis",
 ]

@@ -220,3 +220,26 @@ class HuginnDynamicCache:
         if self._k is None:
             return 0.0
         return 2 * self._k.nelement() * self._k.element_size() / (1024 * 1024)
+
+
+class HuginnStaticCache(HuginnDynamicCache):
+    """The reference's preallocated cache (RMM:311-433) with its constructor signature.  Storage and
+    behaviour are those of HuginnDynamicCache with `max_length` fixed; `max_num_steps` (= 4 + 4 * recurrences in
+    the reference's callers) only presizes the slots."""
+
+    def __init__(self, max_length: int, max_num_steps: int, num_heads: int, hidden_dim: int, batch_size: int = 1,
+                 lookup_strategy: str = "full", device=None, dtype: torch.dtype = torch.float32) -> None:
+        super().__init__(lookup_strategy=lookup_strategy, max_length=max_length)
+        if "compress-" in lookup_strategy:  # RMM:330-338
+            stage = int(lookup_strategy.split("compress-")[1][1:])
+            steps = 4 + stage if "compress-s" in lookup_strategy else 4 + (max_num_steps - 4 + stage - 1) // stage
+        else:
+            steps = max_num_steps
+        self.max_num_steps = steps
+        n_neg = 2 if steps >= 4 else 1
+        self.ensure(max(steps - n_neg, 1), n_neg, batch_size, num_heads, hidden_dim, max_length, dtype,
+                    device if device is not None else "cpu")
+
+    def get_memory_usage(self) -> float:
+        """Allocated MiB, as the reference's static cache reports (RMM:432-433)."""
+        return self.get_allocated_mb()

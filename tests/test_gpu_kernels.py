@@ -324,6 +324,19 @@ def test_swiglu_elementwise(pkg):
             assert bool((got.cpu() == F.silu(z[:, :I]) * z[:, I:]).float().mean() > 0.99)
 
 
+def test_decode_attention_at_the_maximum_context(pkg):
+    """block_size = 4096 positions (recpre/raven_config_minimal.py:17): the last decode step of a full context."""
+    dt, nh, hd, t_max = torch.bfloat16, 55, 96, 4096
+    k, v, kd, vd, cache = make_cache(pkg, 1, 1, nh, t_max, hd, dt, fill_seed=150)
+    q = rnd((1, nh * hd), dt, 151)
+    ws = pkg.hip.attention_workspace(1, nh, hd, "cuda")
+    y = pkg.hip.decode_attention(q.cuda(), cache, 0, 1, 1, t_max - 1, nh, hd, workspace=ws)
+    want = O.sdpa(q.view(1, 1, nh, hd).transpose(1, 2), k[0], v[0]).transpose(1, 2).reshape(1, nh * hd)
+    check(y, want, dt, "attention over 4096 positions")
+    with pytest.raises(pkg.hip.RavenHipError):
+        pkg.hip.decode_attention(q.cuda(), cache, 0, 1, 1, t_max, nh, hd, workspace=ws)  # one past the end
+
+
 def test_decode_attention_zero_query_gives_mean(pkg):
     dt, nh, hd, T = torch.bfloat16, 55, 96, 513
     k, v, kd, vd, cache = make_cache(pkg, 1, 1, nh, 1024, hd, dt, fill_seed=95)

@@ -131,6 +131,39 @@ def test_greedy_batch_and_zero_state_and_stop(tiny32):
     assert torch.equal(got_s.cpu(), want_s) and got_s.shape[1] < 17
 
 
+def test_generate_options(pkg, tiny32):
+    """Sampling branch, continuous compute, dict output, max_length handling of generate_minimal (RMM:1165-1232)."""
+    s, w, model = tiny32
+    prompt = torch.randint(0, s.vocab_size, (2, 6), generator=torch.Generator().manual_seed(4)).cuda()
+    gc = pkg.GenerationSettings(do_sample=True, temperature=0.8, top_k=50, top_p=0.9, min_p=0.01, return_dict_in_generate=True)
+    outs = []
+    for _ in range(2):
+        torch.manual_seed(123)
+        outs.append(model.generate(prompt, gc, max_new_tokens=8, stop_tokens=set()))
+    assert torch.equal(outs[0].sequences, outs[1].sequences) and outs[0].sequences.shape == (2, 14)
+    assert int(outs[0].sequences.max()) < s.vocab_size and outs[0].past_key_values.get_seq_length() == 13
+    torch.manual_seed(7)
+    other = model.generate(prompt, gc, max_new_tokens=8, stop_tokens=set()).sequences
+    assert not torch.equal(other, outs[0].sequences), "a different seed should sample a different continuation"
+    # top_k = 1 sampling is greedy
+    g1 = pkg.GenerationSettings(do_sample=True, top_k=1)
+    a = model.generate(prompt, g1, max_new_tokens=5, init_scale=0.0, stop_tokens=set())
+    b = model.generate(prompt, max_new_tokens=5, init_scale=0.0, stop_tokens=set())
+    assert torch.equal(a, b)
+    # continuous compute carries the last latent state over (deterministic with a zero initial state)
+    c1 = model.generate(prompt, max_new_tokens=5, init_scale=0.0, continuous_compute=True, stop_tokens=set())
+    c2 = model.generate(prompt, max_new_tokens=5, init_scale=0.0, continuous_compute=True, stop_tokens=set())
+    assert torch.equal(c1, c2) and c1.shape == (2, 11)
+    assert model.generate(prompt, max_length=9, stop_tokens=set()).shape == (2, 9)
+    with pytest.raises(NotImplementedError):
+        model.generate(prompt, criterion="entropy-diff")
+    # the reference's preallocated cache class works as past_key_values too
+    static = pkg.HuginnStaticCache(max_length=32, max_num_steps=4 + 4 * 4, num_heads=s.n_heads, hidden_dim=s.head_dim, batch_size=2,
+                                   device="cuda", dtype=torch.float32)
+    d = model.generate(prompt, max_new_tokens=5, init_scale=0.0, stop_tokens=set(), past_key_values=static)
+    assert torch.equal(d, b)
+
+
 def test_forward_tiny_bf16_matches_oracle(tiny16):
     s, w, model = tiny16
     g = torch.Generator().manual_seed(3)

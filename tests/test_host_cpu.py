@@ -133,3 +133,17 @@ def test_cache_size_known_answers(pkg):
         for step in O.step_indices(s):
             c.note_append(step, 366, 0)
         assert c.get_memory_usage() == want
+
+
+def test_static_cache_known_answer_and_interface(pkg):
+    """examples/inference_demo.ipynb:491 of the reference: 132 steps x 1 x 55 x 1024 x 96, K+V, bf16 = 2722.5 MB."""
+    c = pkg.HuginnStaticCache(max_length=1024, max_num_steps=4 + 32 * 4, num_heads=55, hidden_dim=96, batch_size=1,
+                              dtype=torch.bfloat16)
+    assert c.get_memory_usage() == 2722.5 and c.t_max == 1024 and c.max_num_steps == 132
+    k = torch.ones(1, 55, 3, 96, dtype=torch.bfloat16)
+    gk, gv = c.update(k, 2 * k, torch.tensor(0))
+    assert gk.shape == (1, 55, 3, 96) and c.get_seq_length() == 3
+    gk, _ = c.update(k, k, torch.tensor(-1))
+    assert torch.equal(gk, k) and list(c.key_cache) == [0, -1]
+    s16 = pkg.HuginnStaticCache(max_length=8, max_num_steps=132, num_heads=2, hidden_dim=4, lookup_strategy="latest-m4-compress-s16")
+    assert s16.max_num_steps == 20
