@@ -101,14 +101,15 @@ __device__ __forceinline__ Chunk<T> bias_rope_chunk(Chunk<T> x, const T* __restr
 // them -- the kernel boundary is the only synchronisation.  FUSED (decode, S == 1): q, and the new
 // position's k and v, come straight from the fused qkv GEMM output -- bias and RoPE are applied here,
 // the new k/v row is written to the cache by the workgroup whose range holds it and used from registers.
-template <typename T, bool FUSED>
+template <typename T, bool FUSED, int kAttnU>
 __global__ __launch_bounds__(256) void decode_attention_kernel(
     const T* __restrict__ q_or_qkv, const T* __restrict__ qk_bias, const float* __restrict__ freqs, T* __restrict__ y,
     CacheView cv, int S, int pos0, const int* __restrict__ pos_dev, float scale_log2, int n_splits,
     float* __restrict__ ws_ml, float* __restrict__ ws_o) {
     constexpr int E = Chunk<T>::N;
     constexpr int G = 16;      // 16-lane rows in the workgroup
-    constexpr int kAttnU = 4;  // positions per row and loop iteration
+    // kAttnU = positions per 16-lane row and loop iteration: 4 when a few workgroups must each keep many loads
+    // in flight, 2 when the grid is large and register pressure decides how many workgroups a CU holds
     __shared__ float sm_m[G], sm_l[G];
     __shared__ float sm_o[G][kAttnMaxHd];
 
@@ -320,16 +321,22 @@ extern "C" int raven_qkv_bias_rope_cache_append(const void* qkv, const void* qk_
     return raven_host::check_launch("qkv_append");
 }
 
+static int g_attn_big_grid = 1280;  // workgroups from which the 2-positions-per-row variant is used
+
 template <typename T>
 static void launch_attention(bool fused, const void* q, const void* bias, const float* freqs, void* y, const raven::CacheView& cv,
                              int S, int M, int pos0, const int32_t* pos_dev, float scale_log2, int ns, float* ws_ml, float* ws_o,
                              hipStream_t s) {
     using namespace raven;
     const dim3 grid(cv.nh, M, ns);
-    if (fused)
-        decode_attention_kernel<T, true><<<grid, dim3(256), 0, s>>>((const T*)q, (const T*)bias, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
-    else
-        decode_attention_kernel<T, false><<<grid, dim3(256), 0, s>>>((const T*)q, nullptr, nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
+    const bool big = (int64_t)cv.nh * M * ns >= g_attn_big_grid;
+    if (fused) {
+        if (big) decode_attention_kernel<T, true, 2><<<grid, dim3(256), 0, s>>>((const T*)q, (const T*)bias, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
+        else     decode_attention_kernel<T, true, 4><<<grid, dim3(256), 0, s>>>((const T*)q, (const T*)bias, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
+    } else {
+        if (big) decode_attention_kernel<T, false, 2><<<grid, dim3(256), 0, s>>>((const T*)q, nullptr, nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
+        else     decode_attention_kernel<T, false, 4><<<grid, dim3(256), 0, s>>>((const T*)q, nullptr, nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
+    }
     if (ns > 1) attention_combine_kernel<T><<<dim3(cv.nh, M), dim3(128), 0, s>>>(ws_ml, ws_o, (T*)y, cv.nh, cv.hd, ns);
 }
 
