@@ -70,7 +70,9 @@ const char* raven_last_error(void);
 
 /* Launch-shape overrides for experiments (grid sizing and load hints of the skinny-GEMM kernels);
  * results never depend on them.  Keys: gemv_units_per_wave, gemv_interleave, gemv_nontemporal,
- * gemv_wgs_per_cu, gemv1_pairs_norm, gemv1_pairs_plain.  Not needed in normal use: the defaults are the tuned values. */
+ * gemv_wgs_per_cu, gemv1_pairs_norm, gemv1_pairs_plain, linear_ks (K slices of the split-K kernel behind raven_linear;
+ * non-zero also makes raven_linear use that kernel for every shape it accepts).  Not needed in normal use: the
+ * defaults are the tuned values. */
 int raven_set_tuning(const char* key, int32_t value);
 
 /* RMSNorm with the reference's two roundings, optionally preceded by a residual add and followed by
@@ -101,6 +103,17 @@ int raven_adapter_gemm_concat(const void* x0, const void* x1, const void* w, voi
  *   z = X fc^T, gate = T(z[:, :I]), up = T(z[:, I:]), out[M, I] = T(T(silu(gate)) * up). */
 int raven_gemm_swiglu(const void* x, const void* fc, void* out,
                       int32_t M, int32_t I, int32_t K, int32_t dtype, void* stream);
+
+/* The general form of the three calls above with an optional workspace:
+ *     z = concat(x0, x1) W^T,  y = swiglu ? T(T(silu(T(z[:, :N]))) * T(z[:, N:])) : T(z) [+ residual] [as float]
+ * With a workspace (raven_linear_workspace_bytes(M, widest output: 2N for SwiGLU)) and 5 or more bf16 rows,
+ * K is split across workgroups and the X tile of a K step is shared by the workgroup's waves, which is
+ * what batches of 8..32 rows need to approach HBM bandwidth; partial sums are added in a fixed order.
+ * Without one (or for 1..4 rows, fp32) the call is forwarded to raven_gemm / _adapter_gemm_concat / _gemm_swiglu. */
+size_t raven_linear_workspace_bytes(int32_t M, int32_t n_out_max);
+int    raven_linear(const void* x0, const void* x1, const void* w, const void* residual, void* y,
+                    int32_t M, int32_t N, int32_t K0, int32_t K1, int32_t swiglu, int32_t out_f32,
+                    int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Decode fast path for ONE token row, one launch:
  *     x  = norm_a ? T(rmsnorm(x0) * norm_a) : x0      -> stored to xa_out when non-NULL

@@ -23,6 +23,8 @@ struct BlockScratch {
     char *n1, *qkv, *q, *ya, *x1, *x2, *n3, *g, *x3, *xa, *xr;
     void* attn_ws;
     size_t attn_ws_bytes;
+    void* lin_ws;
+    size_t lin_ws_bytes;
 };
 
 static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
@@ -48,6 +50,9 @@ static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
     s.xr = take(row);
     s.attn_ws_bytes = raven_decode_attention_workspace_bytes(M, d->n_heads, d->head_dim);
     s.attn_ws = s.attn_ws_bytes ? take(s.attn_ws_bytes) : nullptr;
+    const int widest = 3 * d->n_embd > 2 * d->intermediate ? 3 * d->n_embd : 2 * d->intermediate;
+    s.lin_ws_bytes = M > 4 ? raven_linear_workspace_bytes(M, widest) : 0;
+    s.lin_ws = s.lin_ws_bytes ? take(s.lin_ws_bytes) : nullptr;
     if (out) *out = s;
     return off;
 }
@@ -83,7 +88,7 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
     int rc;
     if (!n1_ready)
         if ((rc = raven_rmsnorm_residual(x_in, nullptr, w->norm_1, s.n1, nullptr, nullptr, nullptr, M, h, d->eps, dt, stream))) return rc;
-    if ((rc = raven_gemm(s.n1, w->wqkv, nullptr, s.qkv, M, 3 * h, h, dt, 0, stream))) return rc;
+    if ((rc = raven_linear(s.n1, nullptr, w->wqkv, nullptr, s.qkv, M, 3 * h, h, 0, 0, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
     if (S == 1) {  // decode: bias, RoPE, cache append and attention in one launch
         if ((rc = raven_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, cache, slot, B, pos0, pos_dev, d->n_heads,
                                              d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream))) return rc;
@@ -93,10 +98,10 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
         if ((rc = raven_decode_attention(s.q, s.ya, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, s.attn_ws,
                                          s.attn_ws_bytes, stream))) return rc;
     }
-    if ((rc = raven_gemm(s.ya, w->proj, x_in, s.x1, M, h, h, dt, 0, stream))) return rc;
+    if ((rc = raven_linear(s.ya, nullptr, w->proj, x_in, s.x1, M, h, h, 0, 0, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
     if ((rc = raven_rmsnorm_residual(s.x1, nullptr, w->norm_2, s.x2, nullptr, w->norm_3, s.n3, M, h, d->eps, dt, stream))) return rc;
-    if ((rc = raven_gemm_swiglu(s.n3, w->fc, s.g, M, I, h, dt, stream))) return rc;
-    if ((rc = raven_gemm(s.g, w->mlp_proj, s.x2, s.x3, M, h, I, dt, 0, stream))) return rc;
+    if ((rc = raven_linear(s.n3, nullptr, w->fc, nullptr, s.g, M, I, h, 0, 1, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
+    if ((rc = raven_linear(s.g, nullptr, w->mlp_proj, s.x2, s.x3, M, h, I, 0, 0, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
     return raven_rmsnorm_residual(s.x3, nullptr, w->norm_4, y_out, nullptr, tail_w, tail_out, M, h, d->eps, dt, stream);
 }
 
@@ -187,7 +192,7 @@ extern "C" int raven_core_iteration(const raven_dims* dims, const void* adapter_
         }
         return close_one_row(dims, s, blocks[n_blocks - 1].norm_4, ln_f, state_out, stream);
     }
-    if ((rc = raven_adapter_gemm_concat(state_in, embeds, adapter_w, s.xa, M, h, h, h, dims->dtype, stream))) return rc;
+    if ((rc = raven_linear(state_in, embeds, adapter_w, nullptr, s.xa, M, h, h, h, 0, 0, dims->dtype, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
     for (int j = 0; j < n_blocks; ++j) {
         const bool last = j == n_blocks - 1;
         void* y_out = last ? (ln_f ? nullptr : state_out) : s.xa;

@@ -24,6 +24,7 @@ extern "C" int raven_gemv_fused(const void* x0, const void* x1, const void* norm
 namespace raven {
 
 int set_gemv1_tuning(const char* key, int value);
+extern int g_linear_ks;
 
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
 
@@ -37,6 +38,8 @@ struct GemmArgs {
     int out_f32;
     int units_per_wave;    // gemv: row pairs per wave
     int interleave;        // gemv: unit = u * total_waves + wave (1) or wave * units_per_wave + u (0)
+    int row_stride;        // mfma: 1 = a tile is 16 neighbouring weight rows, 2 = every second row (see mfma_kernel)
+    int line_aligned;      // mfma: the rows of a tile all start at the same offset inside a 128-byte line
 };
 
 // Launch-shape knobs (raven_set_tuning); 0 = automatic.
@@ -181,7 +184,14 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemmArgs a) {
 // row), parks them in a wave-private LDS tile with 272-byte row pitch, and reads the MFMA fragments from
 // there (conflict-free: 16 rows x 16 bytes cover the 64 banks once).  The next macro-step's global loads
 // are issued into registers as soon as the current one is parked, before it is multiplied.  No barrier inside the K loop: every
-// wave only touches its own LDS tile.  K % 128 leftovers (32 elements for K = 5280) go to the last wave.
+// wave only touches its own LDS tile.
+//
+// A quarter-wave's 256 bytes should also be two whole 128-byte lines: a row that starts 64 bytes into a line
+// makes them three, and that alone costs 20 % of the bandwidth.  K = 5280 (10560 bytes per row) puts every
+// second row there.  So with row_stride = 2 a tile is made of 16 rows of the SAME parity, all its rows are
+// misaligned by the same amount, and the macro-steps of such a tile start `shift` elements into the row
+// (at the next line boundary); the `shift` elements before them and whatever is left behind the last full
+// macro-step are single 32-wide MFMA steps straight from global memory (first and last wave).
 // ------------------------------------------------------------------------------------------------
 constexpr int kPitch = 136;  // bf16 elements per LDS row: 128 + 8 (272 bytes)
 
@@ -193,22 +203,26 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ln = lane & 15, kq = lane >> 4;
     const int K = a.K;
-    const int n_units = (EPI == EPI_SWIGLU) ? a.N / 16 : (a.N / 16 + NT - 1) / NT;
-    const int unit = blockIdx.x;
-    if (unit >= n_units) return;
+    const int rs = a.row_stride;
+    // a group is rs units: with rs = 2 the even unit takes the even rows of the group's tiles, the odd unit the odd rows
+    const int group = rs == 2 ? blockIdx.x >> 1 : blockIdx.x;
+    const int parity = rs == 2 ? blockIdx.x & 1 : 0;
 
     const bf16* W = static_cast<const bf16*>(a.w);
-    int tile_row0[NT];  // first weight row of each tile
+    int tile_row0[NT];  // first weight row of each tile; row i of the tile is tile_row0 + i * rs
+    int tile_out0[NT];  // output column of that row
     bool tile_ok[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         if (EPI == EPI_SWIGLU) {
-            tile_row0[t] = unit * 16 + t * a.N;  // t = 0 gate tile, t = 1 up tile
+            tile_out0[t] = group * 16 * rs + parity;
+            tile_row0[t] = tile_out0[t] + t * a.N;  // t = 0 gate tile, t = 1 up tile
             tile_ok[t] = true;
         } else {
-            const int tile = unit * NT + t;
-            tile_ok[t] = tile * 16 < a.N;
-            tile_row0[t] = (tile_ok[t] ? tile : unit * NT) * 16;
+            const int first = (group * NT + t) * 16 * rs;
+            tile_ok[t] = first < a.N;
+            tile_out0[t] = (tile_ok[t] ? first : group * NT * 16 * rs) + parity;
+            tile_row0[t] = tile_out0[t];
         }
     }
 
@@ -234,11 +248,21 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
         const int wk0 = seg == 0 ? 0 : a.k0;  // column of W where this segment starts
         const bf16* X = static_cast<const bf16*>(seg == 0 ? a.x0 : a.x1);
         const int ldx = seg == 0 ? a.k0 : a.k1;
-        const int n_macro = seg_len / 128;
+        // elements in front of the first 128-byte line boundary of this segment's weight rows (0 or 32, else not used)
+        int shift = 0;
+        if (a.line_aligned) {
+            const int mis = (int)(reinterpret_cast<uintptr_t>(W + (int64_t)tile_row0[0] * K + wk0) & 127);
+            shift = mis == 64 ? 32 : 0;
+#pragma unroll
+            for (int t = 1; t < NT; ++t)
+                if ((int)(reinterpret_cast<uintptr_t>(W + (int64_t)tile_row0[t] * K + wk0) & 127) != mis) shift = 0;
+            if (shift > seg_len) shift = 0;
+        }
+        const int n_macro = (seg_len - shift) / 128;
         const int mb = (int)((int64_t)n_macro * wave / 4), me = (int)((int64_t)n_macro * (wave + 1) / 4);
 
         auto fetch = [&](int mac, Staged& st) {  // global -> registers, row-contiguous lanes
-            const int k = mac * 128 + lc;
+            const int k = shift + mac * 128 + lc;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -250,7 +274,7 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
             for (int t = 0; t < NT; ++t)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    st.w[t][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(W + (int64_t)(tile_row0[t] + 4 * i + lr) * K + wk0 + k));
+                    st.w[t][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(W + (int64_t)(tile_row0[t] + (4 * i + lr) * rs) * K + wk0 + k));
         };
         auto park = [&](const Staged& st) {  // registers -> this wave's LDS tile
 #pragma unroll
@@ -295,12 +319,13 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
             multiply();
             wave_sync();
         }
-        // leftover 32-element steps of this segment: the last wave takes them, straight from global memory
-        if (wave == 3) {
-            for (int k = n_macro * 128; k < seg_len; k += 32) {
+        // 32-element steps in front of the first and behind the last macro-step: first and last wave, straight from global memory
+        if (wave == 0 || wave == 3) {
+            const int kb = wave == 0 ? 0 : shift + n_macro * 128, ke = wave == 0 ? shift : seg_len;
+            for (int k = kb; k < ke; k += 32) {
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    const bf16x8 wv = *reinterpret_cast<const bf16x8*>(W + (int64_t)(tile_row0[t] + ln) * K + wk0 + k + kq * 8);
+                    const bf16x8 wv = *reinterpret_cast<const bf16x8*>(W + (int64_t)(tile_row0[t] + ln * rs) * K + wk0 + k + kq * 8);
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt) {
                         const int m = min(mt * 16 + ln, a.M - 1);
@@ -340,7 +365,7 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
         if (EPI == EPI_SWIGLU) {
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const int n = unit * 16 + kq * 4 + v;
+                const int n = tile_out0[0] + (kq * 4 + v) * rs;
                 static_cast<bf16*>(a.y)[(int64_t)m * a.N + n] = from_f32<bf16>(swiglu<bf16>(acc[0][mt][v], acc[NT - 1][mt][v]));
             }
         } else {
@@ -348,7 +373,7 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
             for (int t = 0; t < NT; ++t) {
                 if (!tile_ok[t]) continue;
 #pragma unroll
-                for (int v = 0; v < 4; ++v) store_out<bf16>(a, m, (unit * NT + t) * 16 + kq * 4 + v, acc[t][mt][v]);
+                for (int v = 0; v < 4; ++v) store_out<bf16>(a, m, tile_out0[t] + (kq * 4 + v) * rs, acc[t][mt][v]);
             }
         }
     }
@@ -412,6 +437,11 @@ static int dispatch_gemv(GemmArgs a, hipStream_t s) {
 template <int EPI>
 static int dispatch_mfma(GemmArgs a, hipStream_t s) {
     const int n_tiles16 = a.N / 16;
+    // rows alternate between line-aligned and 64 bytes off when the row pitch is an odd multiple of 64 bytes:
+    // tiles of equal parity then (needs whole pairs of tiles); any multiple of 128 bytes needs nothing special
+    const int pitch = a.K * 2;
+    a.row_stride = (pitch % 128 == 64 && a.N % 32 == 0) ? 2 : 1;
+    a.line_aligned = (pitch * a.row_stride) % 128 == 0;
     if (EPI == EPI_SWIGLU) {
         if (a.M <= 16)
             mfma_kernel<1, 2, EPI><<<dim3(n_tiles16), dim3(256), 0, s>>>(a);
@@ -421,7 +451,8 @@ static int dispatch_mfma(GemmArgs a, hipStream_t s) {
         // two tiles per workgroup (X is then re-read from L2 once per two tiles) while that still leaves every
         // CU more than one workgroup; L2 -> L1 traffic, not HBM, is what limits this kernel
         const bool two = n_tiles16 / 2 >= n_cus() + n_cus() / 2;
-        const int units = two ? (n_tiles16 + 1) / 2 : n_tiles16;
+        const int rs = a.row_stride;  // units come in groups of rs, a group covers rs * (two ? 2 : 1) tiles
+        const int units = two ? (n_tiles16 + 2 * rs - 1) / (2 * rs) * rs : n_tiles16;
         if (a.M <= 16) {
             if (two) mfma_kernel<1, 2, EPI><<<dim3(units), dim3(256), 0, s>>>(a);
             else     mfma_kernel<1, 1, EPI><<<dim3(units), dim3(256), 0, s>>>(a);
@@ -490,6 +521,7 @@ extern "C" int raven_set_tuning(const char* key, int32_t value) {
     else if (k == "gemv_interleave") g_tuning.gemv_interleave = value;
     else if (k == "gemv_nontemporal") g_tuning.gemv_nontemporal = value;
     else if (k == "gemv_wgs_per_cu") g_tuning.gemv_wgs_per_cu = value;
+    else if (k == "linear_ks") g_linear_ks = value;
     else RAVEN_REQUIRE(set_gemv1_tuning(key, value) == 0, "set_tuning: unknown key %s", key);
     return 0;
 }

@@ -50,6 +50,8 @@ SIGNATURES = {
     "raven_gemm": (C.c_int, [_VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _VP]),
     "raven_adapter_gemm_concat": (C.c_int, [_VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _VP]),
     "raven_gemm_swiglu": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I32, _I32, _VP]),
+    "raven_linear_workspace_bytes": (_SZ, [_I32, _I32]),
+    "raven_linear": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _VP, _SZ, _VP]),
     "raven_gemv_fused": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _F, _I32, _I32, _I32, _VP]),
     "raven_qkv_bias_rope_cache_append": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32,
                                                    _VP, _I32, _I32, _I32, _VP]),
@@ -193,6 +195,26 @@ def gemm_swiglu(x, fc):
     y = torch.empty(M, inter, device=x.device, dtype=dt)
     rc = load().raven_gemm_swiglu(_ptr(x, "x"), _ptr(fc, "fc", dt), _ptr(y, "out"), M, inter, K, dtype_code(dt), _stream())
     _check(rc, "raven_gemm_swiglu")
+    return y
+
+
+def linear_workspace(M, n_out_max, device):
+    n = load().raven_linear_workspace_bytes(M, n_out_max)
+    return torch.empty(max(n, 256), dtype=torch.uint8, device=device)
+
+
+def linear(x0, w, x1=None, residual=None, swiglu=False, out_f32=False, workspace=None):
+    """concat(x0, x1) W^T with the plain / residual / float / SwiGLU epilogues; x0 [M, K0], w [N or 2N, K0 + K1]."""
+    dt = x0.dtype
+    M, K0 = x0.shape
+    K1 = 0 if x1 is None else x1.shape[1]
+    N = w.shape[0] // 2 if swiglu else w.shape[0]
+    assert w.shape[1] == K0 + K1
+    y = torch.empty(M, N, device=x0.device, dtype=torch.float32 if out_f32 else dt)
+    rc = load().raven_linear(_ptr(x0, "x0"), _ptr(x1, "x1", dt), _ptr(w, "w", dt), _ptr(residual, "residual", dt), _ptr(y, "y"),
+                             M, N, K0, K1, int(swiglu), int(out_f32), dtype_code(dt), _ptr(workspace, "workspace", torch.uint8),
+                             0 if workspace is None else workspace.numel(), _stream())
+    _check(rc, "raven_linear")
     return y
 
 

@@ -143,6 +143,76 @@ def test_gemm_swiglu(pkg, dt, M, I, K):
     assert close(y, wrong)[1] > 0.1, "the gate must be the first half"
 
 
+@pytest.mark.parametrize("M", [5, 8, 16, 17, 32, 33, 40])
+@pytest.mark.parametrize("ks", [0, 3])
+def test_linear_with_workspace_nebel_shapes(pkg, M, ks):
+    """raven_linear at the 3.5b shapes, every epilogue: with the library's own choice between its two MFMA
+    kernels (ks = 0) and with the split-K, shared-X kernel forced to three K slices for every matrix."""
+    dt, h, I = torch.bfloat16, 5280, 17920
+    pkg.hip.set_tuning("linear_ks", ks)
+    ws = pkg.hip.linear_workspace(M, 2 * I, "cuda")
+    x, xi, x1 = rnd((M, h), dt, 160 + M), rnd((M, I), dt, 161), rnd((M, h), dt, 162)
+    res = rnd((M, h), dt, 163)
+    wqkv, proj, fc, mlp, ada = (rnd(sh, dt, 164 + i, 0.02) for i, sh in enumerate(((3 * h, h), (h, h), (2 * I, h), (h, I), (h, 2 * h))))
+    dev = lambda t: t.cuda()
+    check(pkg.hip.linear(dev(x), dev(wqkv), workspace=ws), lin(x, wqkv).to(dt), dt, "qkv")
+    check(pkg.hip.linear(dev(x), dev(proj), residual=dev(res), workspace=ws), lin(x, proj).to(dt) + res, dt, "proj + residual")
+    z = lin(x, fc).to(dt)
+    check(pkg.hip.linear(dev(x), dev(fc), swiglu=True, workspace=ws), F.silu(z[:, :I]) * z[:, I:], dt, "fc + swiglu")
+    check(pkg.hip.linear(dev(xi), dev(mlp), residual=dev(res), workspace=ws), lin(xi, mlp).to(dt) + res, dt, "mlp.proj + residual")
+    check(pkg.hip.linear(dev(x), dev(ada), x1=dev(x1), workspace=ws), lin(torch.cat([x, x1], -1), ada).to(dt), dt, "adapter")
+    yf = pkg.hip.linear(dev(x), dev(proj), out_f32=True, workspace=ws)
+    assert yf.dtype == torch.float32 and torch.equal(yf, pkg.hip.linear(dev(x), dev(proj), workspace=ws).float())
+    # the same call twice gives the same bits (partials are added in a fixed order), and no workspace gives the same values
+    a, b = pkg.hip.linear(dev(xi), dev(mlp), workspace=ws), pkg.hip.linear(dev(xi), dev(mlp), workspace=ws)
+    assert torch.equal(a, b)
+    check(pkg.hip.linear(dev(xi), dev(mlp)), lin(xi, mlp).to(dt), dt, "no workspace")
+    pkg.hip.set_tuning("linear_ks", 0)
+
+
+def test_linear_small_and_odd_shapes(pkg):
+    dt = torch.bfloat16
+    pkg.hip.set_tuning("linear_ks", 2)  # the split-K kernel for everything it accepts
+    for M, N, K in ((9, 48, 160), (32, 16, 128), (12, 528, 1056), (7, 32, 96), (6, 20, 64)):
+        x, w = rnd((M, K), dt, 170), rnd((N, K), dt, 171, 0.05)
+        ws = pkg.hip.linear_workspace(M, N, "cuda")
+        check(pkg.hip.linear(x.cuda(), w.cuda(), workspace=ws), lin(x, w).to(dt), dt, f"linear {M}x{N}x{K}")
+    x, w = rnd((3, 256), torch.float32, 172), rnd((64, 256), torch.float32, 173, 0.1)
+    check(pkg.hip.linear(x.cuda(), w.cuda(), workspace=pkg.hip.linear_workspace(3, 64, "cuda")), lin(x, w), torch.float32, "fp32 falls through")
+    pkg.hip.set_tuning("linear_ks", 0)
+
+
+@pytest.mark.parametrize("M", [6, 20])
+def test_mfma_gemm_row_alignment_cases(pkg, M):
+    """Row pitches that are odd multiples of 64 bytes (tiles of one row parity, macro-steps shifted to the line
+    boundary), with and without whole tile pairs, a second operand that starts mid-line, and a weight matrix
+    whose base address is not line-aligned; both MFMA kernels (with and without a workspace)."""
+    dt = torch.bfloat16
+    ws = pkg.hip.linear_workspace(M, 4096, "cuda")
+    pkg.hip.set_tuning("linear_ks", 2)  # with a workspace: the split-K kernel
+    for N, K in ((32, 96), (64, 288), (64, 2336), (96, 416), (48, 416), (160, 1184), (64, 256)):
+        x, w = rnd((M, K), dt, 180 + N), rnd((N, K), dt, 181 + K, 0.05)
+        want = lin(x, w).to(dt)
+        for wsp in (None, ws):
+            check(pkg.hip.linear(x.cuda(), w.cuda(), workspace=wsp), want, dt, f"plain {M}x{N}x{K} ws={wsp is not None}")
+        # the same matrix 16 bytes into an allocation
+        flat = torch.zeros(N * K + 8, dtype=dt, device="cuda")
+        flat[8:] = w.cuda().reshape(-1)
+        for wsp in (None, ws):
+            check(pkg.hip.linear(x.cuda(), flat[8:].view(N, K), workspace=wsp), want, dt, f"offset base {M}x{N}x{K}")
+    for I, K in ((64, 160), (96, 416), (48, 288)):
+        x, fc = rnd((M, K), dt, 190), rnd((2 * I, K), dt, 191 + I, 0.05)
+        z = lin(x, fc).to(dt)
+        for wsp in (None, ws):
+            check(pkg.hip.linear(x.cuda(), fc.cuda(), swiglu=True, workspace=wsp), F.silu(z[:, :I]) * z[:, I:], dt, f"swiglu {M}x{I}x{K}")
+    for N, K0, K1 in ((64, 160, 160), (32, 288, 160), (64, 416, 416)):
+        x0, x1, w = rnd((M, K0), dt, 195), rnd((M, K1), dt, 196), rnd((N, K0 + K1), dt, 197 + N, 0.05)
+        for wsp in (None, ws):
+            check(pkg.hip.linear(x0.cuda(), w.cuda(), x1=x1.cuda(), workspace=wsp), lin(torch.cat([x0, x1], -1), w).to(dt), dt,
+                  f"two operands {M}x{N}x({K0}+{K1})")
+    pkg.hip.set_tuning("linear_ks", 0)
+
+
 @pytest.mark.parametrize("dt,h,I", [(torch.bfloat16, 5280, 17920), (torch.float32, 256, 704), (torch.bfloat16, 64, 176)])
 def test_gemv_fused_one_row(pkg, dt, h, I):
     """The one-row kernel with its norm prologues and epilogues, against the oracle's separate ops."""
