@@ -53,14 +53,29 @@ typedef struct raven_block_weights {
 } raven_block_weights;
 
 /* Step-indexed KV cache, the HuginnStaticCache layout (RMM:344-349): K and V are
- * [n_slots, batch, nh, t_max, hd] of T.  Slot s of the reference's step index is s for s >= 0 and
- * n_slots + s for the coda's negative indices (RMM:375-380 index from the end the same way). */
+ * [n_slots, batch, nh, t_max, hd] of T.  The `slot` argument of the calls below is an index into the
+ * first dimension (negative values count from the end); which step index lives in which slot is the
+ * caller's business, except for the partial-fill lookups:
+ *
+ * Tokens computed with different numbers of recurrences leave positions that are not cached at the
+ * deeper steps.  HuginnDynamicCache.update then builds K/V per position according to its lookup strategy
+ * (RMM:199-253).  The attention kernels do the same in place when steps_present is given: steps_present[p]
+ * = how many core steps (step index 2, 3, 4, ... in this order, slots core_slot0, core_slot0 + 1, ...) are
+ * cached for position p, shared by the batch.  It is consulted for positions older than the rows of the
+ * call and for slots >= core_slot0 only; NULL or RAVEN_LOOKUP_NONE = everything is cached (no lookups). */
+enum { RAVEN_LOOKUP_NONE = 0,
+       RAVEN_LOOKUP_SKIP = 1,         /* "skip", and "full" with gaps: leave uncached positions out (RMM:199-204, 247-254) */
+       RAVEN_LOOKUP_LATEST = 2,       /* "latest-m4", "available-m4": deepest cached step <= this one of the same block (RMM:206-232) */
+       RAVEN_LOOKUP_ALWAYS_LAST = 3   /* "always-last-m4": deepest cached step of the same block (RMM:233-246) */ };
 typedef struct raven_kv_cache {
     void*   k;
     void*   v;
     int32_t n_slots;
     int32_t batch;
     int32_t t_max;
+    int32_t lookup_mode;           /* RAVEN_LOOKUP_* */
+    const int32_t* steps_present;  /* device, [t_max], or NULL */
+    int32_t core_slot0;            /* slot of step index 2 */
 } raven_kv_cache;
 
 /* Library identity: version, the gfx arch the kernels were compiled for, last error text. */

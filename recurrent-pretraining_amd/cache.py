@@ -11,6 +11,7 @@ any earlier one only appends slots.
 
 from __future__ import annotations
 
+import bisect
 from typing import Optional
 
 import torch
@@ -31,32 +32,117 @@ def remap_step(step_idx: int, strategy: str) -> int:
     return step_idx
 
 
+class _CoreSteps:
+    """Which core steps (step index 2, 3, ... = bit 0, 1, ...) are cached for which position, as runs
+    [start, end, mask] of neighbouring positions with the same set: a prefill is one run, a decoded token
+    joins the run before it when it was computed with the same number of recurrences."""
+
+    def __init__(self):
+        self.runs: list[list[int]] = []
+
+    def __len__(self) -> int:
+        return self.runs[-1][1] if self.runs else 0
+
+    def _split(self, pos: int) -> int:
+        """Index of the run that starts at pos (splitting the run that holds it); len(runs) when pos is the end."""
+        i = bisect.bisect_right(self.runs, pos, key=lambda r: r[0]) - 1
+        if i < 0 or pos >= self.runs[i][1]:
+            return i + 1
+        if self.runs[i][0] == pos:
+            return i
+        st, en, mask = self.runs[i]
+        self.runs[i][1] = pos
+        self.runs.insert(i + 1, [pos, en, mask])
+        return i + 1
+
+    def add(self, bit: int, first: int, n: int) -> None:
+        """Positions first .. first+n-1 now hold core step `bit`; a second write of the same entry is an error."""
+        if len(self) < first + n:
+            self.runs.append([len(self), first + n, 0])
+        i, j = self._split(first), self._split(first + n)
+        for r in self.runs[i:j]:
+            assert not (r[2] >> bit) & 1, "overwrite of a cached position"  # RMM:192-193
+            r[2] |= 1 << bit
+        for k in range(min(j, len(self.runs) - 1), max(i - 1, 0) - 1, -1):  # re-join equal neighbours
+            if k + 1 < len(self.runs) and self.runs[k][2] == self.runs[k + 1][2]:
+                self.runs[k][1] = self.runs[k + 1][1]
+                del self.runs[k + 1]
+
+    def truncate(self, n: int) -> None:
+        while self.runs and self.runs[-1][0] >= n:
+            self.runs.pop()
+        if self.runs:
+            self.runs[-1][1] = min(self.runs[-1][1], n)
+
+    def has(self, bit: int, pos: int) -> bool:
+        i = bisect.bisect_right(self.runs, pos, key=lambda r: r[0]) - 1
+        return i >= 0 and pos < self.runs[i][1] and bool((self.runs[i][2] >> bit) & 1)
+
+    def count(self, bit: int, n: int) -> int:
+        return sum(min(en, n) - st for st, en, mask in self.runs if st < n and (mask >> bit) & 1)
+
+    @staticmethod
+    def depth(mask: int) -> int:
+        """Number of steps cached without a hole, from the first one on."""
+        return (~mask & (mask + 1)).bit_length() - 1
+
+    def min_depth(self, n: int) -> int:
+        """Smallest depth over positions 0 .. n-1 (0 when some are unknown)."""
+        if n > len(self):
+            return 0
+        return min((self.depth(mask) for st, en, mask in self.runs if st < n), default=0)
+
+    def holes(self, n: int) -> bool:
+        """True when a position below n holds a step but not all the steps before it."""
+        return any(mask & (mask + 1) for st, en, mask in self.runs if st < n)
+
+    def depths(self, n: int) -> list[int]:
+        out: list[int] = []
+        for st, en, mask in self.runs:
+            if st < n:
+                out.extend([self.depth(mask)] * (min(en, n) - st))
+        return out
+
+
+def lookup_mode(strategy: str) -> int:
+    """What to do with positions that are not cached at the step being read (RMM:199-273)."""
+    if strategy == "full" or strategy.startswith("skip"):
+        return hip.LOOKUP_SKIP           # RMM:199-204 stacks whatever is there; RMM:247-254
+    if strategy.startswith("latest-m4") or strategy.startswith("available-m4"):
+        return hip.LOOKUP_LATEST         # RMM:206-232: the same for caches whose positions hold a prefix of the steps
+    if strategy.startswith("always-last-m4"):
+        return hip.LOOKUP_ALWAYS_LAST    # RMM:233-246
+    if strategy.startswith("randomized"):
+        raise NotImplementedError("the 'randomized' lookup (a sanity check in the reference, RMM:255-271) is not built")
+    raise ValueError(f"Unknown lookup strategy: {strategy}")  # RMM:272-273
+
+
 class _PositionView:
     """cache.key_cache[step]: positions -> [B, nh, hd] views into the contiguous storage."""
 
     def __init__(self, owner: "HuginnDynamicCache", store: str, step: int):
         self._o, self._store, self._step = owner, store, step
 
-    def _filled(self) -> int:
-        return self._o._filled.get(self._step, 0)
+    def _positions(self):
+        return [p for p in range(self._o._filled.get(self._step, 0)) if self._o._present(self._step, p)]
 
     def __len__(self):
-        return self._filled()
+        return self._o._n_present(self._step)
 
     def __contains__(self, pos):
-        return 0 <= int(pos) < self._filled()
+        return self._o._present(self._step, int(pos))
 
     def __iter__(self):
-        return iter(range(self._filled()))
+        return iter(self._positions())
 
     def keys(self):
-        return range(self._filled())
+        return self._positions()
 
     def values(self):
-        return [self[p] for p in range(self._filled())]
+        return [self[p] for p in self._positions()]
 
     def items(self):
-        return [(p, self[p]) for p in range(self._filled())]
+        return [(p, self[p]) for p in self._positions()]
 
     def __getitem__(self, pos):
         if pos not in self:
@@ -109,7 +195,14 @@ class HuginnDynamicCache:
         self._k: Optional[torch.Tensor] = None
         self._v: Optional[torch.Tensor] = None
         self._neg_slots = 0          # slots reserved for negative (coda) step indices
-        self._filled: dict[int, int] = {}  # step -> number of positions present (first-touch order)
+        self._filled: dict[int, int] = {}  # step -> 1 + highest position present (first-touch order)
+        # Tokens computed with different numbers of recurrences leave gaps at the deeper core steps.  Kept while no
+        # compress-* remap is in use (those strategies overwrite a few shared steps instead).  A token runs its core
+        # steps in order, so for the kernels "how many of the steps 2, 3, 4, ... are cached" per position says it all.
+        self._core = _CoreSteps()
+        self._sp_dev: Optional[torch.Tensor] = None   # device copy of the per-position depths, built on demand
+        self._sp_valid = 0                            # positions of _sp_dev that are up to date
+        self._min_memo = (0, 0)                       # (n, smallest depth below n): older positions never change
         self.key_cache = _StepView(self, "_k")
         self.value_cache = _StepView(self, "_v")
         self._struct: Optional[hip.KVCache] = None
@@ -156,18 +249,67 @@ class HuginnDynamicCache:
         self._k, self._v, self._neg_slots = k, v, new_neg
         self._struct = None
 
-    def native(self) -> hip.KVCache:
-        """The C-ABI descriptor of the storage (device pointers; rebuilt after every reallocation)."""
+    def native(self, steps=None, first_pos: int = 0) -> hip.KVCache:
+        """The C-ABI descriptor of the storage (device pointers; rebuilt after every reallocation).
+
+        With `steps` (the step indices a launch reads) and the first position of its new rows: the descriptor that
+        makes the attention kernels resolve positions older than `first_pos` which are not cached at those steps
+        according to the lookup strategy -- the plain one when there are no such gaps."""
         if self._k is None:
             raise RuntimeError("cache storage has not been allocated yet")
         if self._struct is None:
             self._struct = hip.make_cache(self._k, self._v)
-        return self._struct
+        if steps is None or not any(self.has_gap(s, first_pos) for s in steps):
+            return self._struct
+        if not all(self.has_gap(s, first_pos) for s in steps):
+            raise ValueError("steps of one launch must agree on whether older positions are missing")
+        mode = lookup_mode(self.lookup_strategy)
+        if self._core.holes(first_pos):
+            raise NotImplementedError("lookups need positions that hold the core steps 2, 3, ... without holes")
+        if mode != hip.LOOKUP_SKIP and self._min_core(first_pos) <= max((remap_step(int(s), self.lookup_strategy) - 2) % 4 for s in steps):
+            raise ValueError("a cached position holds no step to look up")  # the reference's max() of an empty list
+        t_max = self.t_max
+        if self._sp_dev is None or self._sp_dev.numel() < t_max:
+            self._sp_dev, self._sp_valid = torch.zeros(t_max, dtype=torch.int32, device=self._k.device), 0
+        if self._sp_valid < first_pos:
+            self._sp_dev[:first_pos] = torch.tensor(self._core.depths(first_pos), dtype=torch.int32)
+            self._sp_valid = first_pos
+        return hip.make_cache(self._k, self._v, self._sp_dev, mode, self._slot(2))
+
+    def _tracks_core(self, step: int) -> bool:
+        return step >= 2 and "compress-" not in self.lookup_strategy
+
+    def _present(self, step: int, pos: int) -> bool:
+        if not 0 <= pos < self._filled.get(step, 0):
+            return False
+        return self._core.has(step - 2, pos) if self._tracks_core(step) else True
+
+    def _n_present(self, step: int) -> int:
+        n = self._filled.get(step, 0)
+        return self._core.count(step - 2, n) if self._tracks_core(step) else n
+
+    def has_gap(self, step_idx: int, first_pos: int) -> bool:
+        """True when a position older than `first_pos` is not cached at this step."""
+        step = remap_step(int(step_idx), self.lookup_strategy)
+        if first_pos <= 0:
+            return False
+        if not self._tracks_core(step):
+            if self._filled.get(step, 0) < first_pos:
+                raise NotImplementedError(f"positions missing at step {step} under lookup strategy {self.lookup_strategy!r}")
+            return False
+        return self._min_core(first_pos) <= step - 2
+
+    def _min_core(self, n: int) -> int:
+        if self._min_memo[0] != n:
+            self._min_memo = (n, self._core.min_depth(n))
+        return self._min_memo[1]
 
     def note_append(self, step_idx: int, n_new: int, first_pos: int) -> int:
         """Bookkeeping for positions the kernels wrote at `step_idx`; returns the slot used."""
         step = remap_step(int(step_idx), self.lookup_strategy)
-        if "compress-" not in self.lookup_strategy:  # RMM:192-193: no overwrite except for the coda
+        if self._tracks_core(step):
+            self._core.add(step - 2, first_pos, n_new)
+        elif "compress-" not in self.lookup_strategy:  # RMM:192-193: no overwrite except for the coda
             assert step < 0 or self._filled.get(step, 0) <= first_pos, "overwrite of a cached position"
         self._filled[step] = max(self._filled.get(step, 0), first_pos + n_new)
         return self._slot(step)
@@ -189,20 +331,47 @@ class HuginnDynamicCache:
         slot = self.note_append(step, n_new, first)
         self._k[slot, :, :, first:first + n_new] = key_states
         self._v[slot, :, :, first:first + n_new] = value_states
+        if self._n_present(mapped) == self._seen_tokens:
+            return self._k[slot, :, :, :self._seen_tokens], self._v[slot, :, :, :self._seen_tokens]
+        # some positions were never computed at this step: gather per position, as RMM:199-253 does
         lookup = self.lookup_strategy if lookup_strategy is None else lookup_strategy
-        if self._filled[mapped] != self._seen_tokens and self.lookup_strategy != "full":
-            raise NotImplementedError(f"lookup strategy {lookup!r} with positions missing at step {step}")
-        t = self._filled[mapped]
-        return self._k[slot, :, :, :t], self._v[slot, :, :, :t]
+        mode = hip.LOOKUP_SKIP if self.lookup_strategy == "full" else lookup_mode(lookup)
+        if self._core.holes(first):
+            raise NotImplementedError("lookups need positions that hold the core steps 2, 3, ... without holes")
+        depths = self._core.depths(first) if self._tracks_core(mapped) else []
+        src = [self._source_step(mapped, depths[p], mode) if p < len(depths) else mapped for p in range(self._seen_tokens)]
+        pos = torch.tensor([p for p, st in enumerate(src) if st is not None], device=self._k.device)
+        slots = torch.tensor([self._slot(st) for st in src if st is not None], device=self._k.device)
+        return self._k[slots, :, :, pos].permute(1, 2, 0, 3), self._v[slots, :, :, pos].permute(1, 2, 0, 3)
+
+    @staticmethod
+    def _source_step(step: int, depth: int, mode: int):
+        """The step whose entry stands in for `step` (>= 2) at a position of an earlier token that holds `depth` core
+        steps, or None when the position is left out: what the attention kernels compute from steps_present."""
+        cs = step - 2
+        if mode != hip.LOOKUP_ALWAYS_LAST and cs < depth:
+            return step
+        if mode == hip.LOOKUP_SKIP:
+            return None
+        j = cs % 4
+        if depth - 1 - j < 0:
+            raise ValueError("a cached position holds no complete recurrence to look up")
+        return 2 + j + (depth - 1 - j) // 4 * 4
 
     def reset(self) -> None:  # RMM:275-279
         self._seen_tokens = 0
         self._filled.clear()
+        self._core = _CoreSteps()
+        self._sp_valid = 0
+        self._min_memo = (0, 0)
 
     def clear_last_k_entries(self, k: int = 0):  # RMM:281-293
         assert self._seen_tokens >= k
         self._seen_tokens -= k
         self._filled = {s: min(n, self._seen_tokens) for s, n in self._filled.items()}
+        self._core.truncate(self._seen_tokens)
+        self._sp_valid = min(self._sp_valid, self._seen_tokens)
+        self._min_memo = (0, 0)
 
     def get_seq_length(self, step_idx: int = 0) -> int:  # RMM:295-296
         return self._seen_tokens
@@ -213,7 +382,7 @@ class HuginnDynamicCache:
             return 0.0
         _, b, nh, _, hd = self._k.shape
         per_pos = b * nh * hd * self._k.element_size()
-        return sum(self._filled.values()) * per_pos * 2 / (1024 * 1024)
+        return sum(self._n_present(s) for s in self._filled) * per_pos * 2 / (1024 * 1024)
 
     def get_allocated_mb(self) -> float:
         """MiB actually allocated (what HuginnStaticCache.get_memory_usage reports, RMM:432-433)."""

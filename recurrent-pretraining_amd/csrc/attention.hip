@@ -23,7 +23,31 @@ struct CacheView {
     void* v;
     int64_t slot_off;  // element offset of the slot: slot * batch * nh * t_max * hd
     int batch, nh, t_max, hd;
+    // partial fill (tokens computed with different numbers of recurrences): see raven_kv_cache in the header
+    const int* steps_present;  // null: every position below the new rows is cached at this slot
+    int lookup_mode;           // RAVEN_LOOKUP_*
+    int core_step;             // slot's step index - 2 (>= 0 when steps_present is set)
+    int64_t slot_stride;       // elements between two slots
 };
+
+// Where position p (older than the new rows) is read from when the slot holds core step `cs`: the element offset
+// to add (a multiple of the slot stride), or `false` when the position takes no part.  sp = number of core steps
+// cached for p.  The reference's loops over its dict cache (recpre/raven_modeling_minimal.py:206-253), for a
+// cache whose positions each hold a prefix 2, 3, ... of the core steps:
+//   latest-m4 / available-m4: the deepest cached step <= cs of the same block (same step index mod 4);
+//   always-last-m4: the deepest cached step of the same block, also beyond cs;
+//   skip, and `full` with gaps: positions that are not cached at this step are left out.
+__device__ __forceinline__ bool lookup_source(const CacheView& cv, int p, int64_t* delta) {
+    const int sp = cv.steps_present[p], cs = cv.core_step;
+    *delta = 0;
+    if (cv.lookup_mode != RAVEN_LOOKUP_ALWAYS_LAST && cs < sp) return true;
+    if (cv.lookup_mode == RAVEN_LOOKUP_SKIP) return false;
+    const int j = cs & 3;
+    if (sp - 1 - j < 0) return false;  // the block never ran for this position (the host rejects such caches)
+    const int src = j + ((sp - 1 - j) >> 2) * 4;
+    *delta = (int64_t)(src - cs) * cv.slot_stride;
+    return true;
+}
 
 // ------------------------------------------------------------------------------------------------
 template <typename T>
@@ -101,7 +125,8 @@ __device__ __forceinline__ Chunk<T> bias_rope_chunk(Chunk<T> x, const T* __restr
 // them -- the kernel boundary is the only synchronisation.  FUSED (decode, S == 1): q, and the new
 // position's k and v, come straight from the fused qkv GEMM output -- bias and RoPE are applied here,
 // the new k/v row is written to the cache by the workgroup whose range holds it and used from registers.
-template <typename T, bool FUSED, int kAttnU>
+// LOOKUP: some older positions are not cached at this slot (cv.steps_present says which).
+template <typename T, bool FUSED, int kAttnU, bool LOOKUP = false>
 __global__ __launch_bounds__(256) void decode_attention_kernel(
     const T* __restrict__ q_or_qkv, const T* __restrict__ qk_bias, const float* __restrict__ freqs, T* __restrict__ y,
     CacheView cv, int S, int pos0, const int* __restrict__ pos_dev, float scale_log2, int n_splits,
@@ -116,7 +141,8 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
     const int head = blockIdx.x, m = blockIdx.y, split = blockIdx.z;
     const int hd = cv.hd, h = cv.nh * hd;
     const int b = m / S, s = m - b * S;
-    const int pos = (pos_dev ? *pos_dev : pos0) + s;  // position of this row's own token
+    const int first_new = pos_dev ? *pos_dev : pos0;
+    const int pos = first_new + s;  // position of this row's own token
     const int len = min(pos + 1, cv.t_max);
     const int per = (len + n_splits - 1) / n_splits;
     const int start = split * per, end = min(len, start + per);
@@ -146,13 +172,17 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
     }
     // first K/V tile, requested before q is touched
     Chunk<T> kc[kAttnU], vc[kAttnU];
+    bool left_out[kAttnU];  // LOOKUP: the position takes no part
     auto load_tile = [&](int base) {
 #pragma unroll
         for (int j = 0; j < kAttnU; ++j) {
             const int p = base + j * G + group;
-            if (active && p < end && !(FUSED && p == pos)) {
-                kc[j] = load_chunk(Kb + (int64_t)p * hd);
-                vc[j] = load_chunk(Vb + (int64_t)p * hd);
+            int64_t delta = 0;
+            left_out[j] = false;
+            if (LOOKUP && p < end && p < first_new) left_out[j] = !lookup_source(cv, p, &delta);
+            if (active && p < end && !(FUSED && p == pos) && !left_out[j]) {
+                kc[j] = load_chunk(Kb + delta + (int64_t)p * hd);
+                vc[j] = load_chunk(Vb + delta + (int64_t)p * hd);
             } else {
                 kc[j] = zero_chunk<T>();
                 vc[j] = zero_chunk<T>();
@@ -186,7 +216,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
                 vc[j] = vnew;
             }
             sc[j] = row16_sum(dot_chunk(qc, kc[j], 0.f)) * scale_log2;
-            if (p >= end) sc[j] = -INFINITY;
+            if (p >= end || (LOOKUP && left_out[j])) sc[j] = -INFINITY;
             m_new = fmaxf(m_new, sc[j]);
         }
         if (m_new == -INFINITY) continue;  // this row has not seen a valid position yet
@@ -285,7 +315,18 @@ static int make_view(const char* who, const raven_kv_cache* cache, int slot, int
     cv->nh = nh;
     cv->t_max = cache->t_max;
     cv->hd = hd;
-    cv->slot_off = (int64_t)sl * cache->batch * nh * cache->t_max * hd;
+    cv->slot_stride = (int64_t)cache->batch * nh * cache->t_max * hd;
+    cv->slot_off = (int64_t)sl * cv->slot_stride;
+    cv->steps_present = nullptr;
+    cv->lookup_mode = RAVEN_LOOKUP_NONE;
+    cv->core_step = sl - cache->core_slot0;
+    if (cache->steps_present != nullptr && cache->lookup_mode != RAVEN_LOOKUP_NONE && cv->core_step >= 0) {
+        RAVEN_REQUIRE(cache->lookup_mode >= RAVEN_LOOKUP_SKIP && cache->lookup_mode <= RAVEN_LOOKUP_ALWAYS_LAST,
+                      "%s: unknown lookup mode %d", who, cache->lookup_mode);
+        RAVEN_REQUIRE(cache->core_slot0 >= 0, "%s: core_slot0 %d", who, cache->core_slot0);
+        cv->steps_present = cache->steps_present;
+        cv->lookup_mode = cache->lookup_mode;
+    }
     return 0;
 }
 
@@ -330,13 +371,21 @@ static void launch_attention(bool fused, const void* q, const void* bias, const 
     using namespace raven;
     const dim3 grid(cv.nh, M, ns);
     const bool big = (int64_t)cv.nh * M * ns >= g_attn_big_grid;
-    if (fused) {
-        if (big) decode_attention_kernel<T, true, 2><<<grid, dim3(256), 0, s>>>((const T*)q, (const T*)bias, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
-        else     decode_attention_kernel<T, true, 4><<<grid, dim3(256), 0, s>>>((const T*)q, (const T*)bias, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
+    const T* bias_t = (const T*)bias;
+#define RAVEN_ATTN_LAUNCH(FUSED_, U_, LOOKUP_)                                                                            \
+    decode_attention_kernel<T, FUSED_, U_, LOOKUP_><<<grid, dim3(256), 0, s>>>((const T*)q, FUSED_ ? bias_t : nullptr,     \
+        FUSED_ ? freqs : nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o)
+    if (cv.steps_present) {  // partial fill: rare, one variant per entry point
+        if (fused) RAVEN_ATTN_LAUNCH(true, 2, true);
+        else RAVEN_ATTN_LAUNCH(false, 2, true);
+    } else if (fused) {
+        if (big) RAVEN_ATTN_LAUNCH(true, 2, false);
+        else RAVEN_ATTN_LAUNCH(true, 4, false);
     } else {
-        if (big) decode_attention_kernel<T, false, 2><<<grid, dim3(256), 0, s>>>((const T*)q, nullptr, nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
-        else     decode_attention_kernel<T, false, 4><<<grid, dim3(256), 0, s>>>((const T*)q, nullptr, nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
+        if (big) RAVEN_ATTN_LAUNCH(false, 2, false);
+        else RAVEN_ATTN_LAUNCH(false, 4, false);
     }
+#undef RAVEN_ATTN_LAUNCH
     if (ns > 1) attention_combine_kernel<T><<<dim3(cv.nh, M), dim3(128), 0, s>>>(ws_ml, ws_o, (T*)y, cv.nh, cv.hd, ns);
 }
 

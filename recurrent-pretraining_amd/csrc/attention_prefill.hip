@@ -182,6 +182,8 @@ extern "C" int raven_prefill_attention(const void* q, void* y, const raven_kv_ca
     RAVEN_REQUIRE(q && y && cache && cache->k && cache->v, "prefill_attention: null pointer");
     RAVEN_REQUIRE(B > 0 && S > 0 && pos0 >= 0 && n_heads > 0, "prefill_attention: bad B=%d S=%d pos0=%d", B, S, pos0);
     RAVEN_REQUIRE(B <= cache->batch, "prefill_attention: batch %d exceeds the cache's %d", B, cache->batch);
+    RAVEN_REQUIRE(cache->steps_present == nullptr || cache->lookup_mode == RAVEN_LOOKUP_NONE,
+                  "prefill_attention: partially filled caches (steps_present) are served by raven_decode_attention only");
     const int sl = slot >= 0 ? slot : cache->n_slots + slot;
     RAVEN_REQUIRE(sl >= 0 && sl < cache->n_slots, "prefill_attention: slot %d outside [0, %d)", slot, cache->n_slots);
     RAVEN_REQUIRE(pos0 + S <= cache->t_max, "prefill_attention: positions up to %d exceed the cache length %d", pos0 + S - 1, cache->t_max);

@@ -36,7 +36,11 @@ class BlockWeights(C.Structure):
 
 class KVCache(C.Structure):
     _fields_ = [("k", C.c_void_p), ("v", C.c_void_p), ("n_slots", C.c_int32), ("batch", C.c_int32),
-                ("t_max", C.c_int32)]
+                ("t_max", C.c_int32), ("lookup_mode", C.c_int32), ("steps_present", C.c_void_p),
+                ("core_slot0", C.c_int32)]
+
+
+LOOKUP_NONE, LOOKUP_SKIP, LOOKUP_LATEST, LOOKUP_ALWAYS_LAST = 0, 1, 2, 3
 
 
 # name -> (restype, argtypes); kept in one table so the export test can walk it
@@ -129,11 +133,15 @@ def make_dims(n_embd: int, n_heads: int, intermediate: int, eps: float, dtype: t
     return Dims(n_embd, n_heads, n_embd // n_heads, intermediate, eps, dtype_code(dtype))
 
 
-def make_cache(k: torch.Tensor, v: torch.Tensor) -> KVCache:
-    """k, v: [n_slots, batch, nh, t_max, hd], contiguous, on the GPU."""
+def make_cache(k: torch.Tensor, v: torch.Tensor, steps_present: Optional[torch.Tensor] = None, lookup_mode: int = LOOKUP_NONE,
+               core_slot0: int = 0) -> KVCache:
+    """k, v: [n_slots, batch, nh, t_max, hd], contiguous, on the GPU; steps_present: int32 [t_max] or None."""
     if k.shape != v.shape or k.dim() != 5:
         raise RavenHipError("cache tensors must be [n_slots, batch, nh, t_max, hd] and of equal shape")
-    return KVCache(_ptr(k, "cache.k"), _ptr(v, "cache.v", k.dtype), k.shape[0], k.shape[1], k.shape[3])
+    if steps_present is not None and (steps_present.dtype != torch.int32 or steps_present.numel() < k.shape[3]):
+        raise RavenHipError("steps_present must be int32 with one entry per cache position")
+    return KVCache(_ptr(k, "cache.k"), _ptr(v, "cache.v", k.dtype), k.shape[0], k.shape[1], k.shape[3], int(lookup_mode),
+                   _ptr(steps_present, "steps_present", torch.int32), int(core_slot0))
 
 
 def make_block_weights(norm_1, norm_2, norm_3, norm_4, wqkv, qk_bias, proj, fc, mlp_proj) -> BlockWeights:

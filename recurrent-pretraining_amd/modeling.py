@@ -309,13 +309,14 @@ class RavenForCausalLM(torch.nn.Module):
                    B: int, S: int, pos0: int, ln_f: bool = False) -> torch.Tensor:
         nat = self._natives()
         slot = 0 if private else cache.note_append(step_idx, S, pos0)
-        if self._is_wide(B * S):
+        kv = cache.native() if private else cache.native([step_idx], pos0)
+        if self._is_wide(B * S) and kv.steps_present is None:
             blk = getattr(self.transformer, {"prelude": "prelude", "coda": "coda", "core": "core_block"}[which])[i]
-            y, tail = self._wide_block(blk, x, cache.native(), slot, B, S, pos0,
+            y, tail = self._wide_block(blk, x, kv, slot, B, S, pos0,
                                        tail_w=self.transformer.ln_f.weight if ln_f else None)
             return tail if ln_f else y
         out = torch.empty_like(x)
-        hip.sandwich_block(nat["dims"], nat[which][i], x, out, nat["freqs"], cache.native(), slot, B, S, pos0,
+        hip.sandwich_block(nat["dims"], nat[which][i], x, out, nat["freqs"], kv, slot, B, S, pos0,
                            self._workspace(B * S), ln_f=self.transformer.ln_f.weight if ln_f else None)
         return out
 
@@ -325,20 +326,27 @@ class RavenForCausalLM(torch.nn.Module):
         nat, t = self._natives(), self.transformer
         n_core = len(t.core_block)
         slots = [0 if private else cache.note_append(first_step + j, S, pos0) for j in range(n_core)]
-        if self._is_wide(B * S):
-            return self._wide_core(x, embeds, slots, cache.native(), B, S, pos0, ln_f)
+        # positions of earlier tokens that were computed with fewer recurrences are not cached at these steps:
+        # the attention kernels then follow the cache's lookup strategy (one descriptor per launch)
+        steps = [first_step + j for j in range(n_core)]
+        gaps = [False] * n_core if private else [cache.has_gap(s_, pos0) for s_ in steps]
+        uniform = all(g == gaps[0] for g in gaps)
+        kv = cache.native() if private or not uniform else cache.native(steps, pos0)
+        if self._is_wide(B * S) and uniform and kv.steps_present is None:
+            return self._wide_core(x, embeds, slots, kv, B, S, pos0, ln_f)
         out = torch.empty_like(x)
         ws = self._workspace(B * S)
         lnw = t.ln_f.weight if ln_f else None
-        if not private and n_core > 0 and all(slots[j] == slots[0] + j for j in range(n_core)):
-            hip.core_iteration(nat["dims"], t.adapter.weight, nat["core"], x, embeds, out, nat["freqs"], cache.native(),
+        if not private and uniform and n_core > 0 and all(slots[j] == slots[0] + j for j in range(n_core)):
+            hip.core_iteration(nat["dims"], t.adapter.weight, nat["core"], x, embeds, out, nat["freqs"], kv,
                                slots[0], B, S, pos0, ws, ln_f=lnw)
             return out
         cur = hip.adapter_gemm_concat(x, embeds, t.adapter.weight)
         for j in range(n_core):
             last = j == n_core - 1
             nxt = out if last else torch.empty_like(x)
-            hip.sandwich_block(nat["dims"], nat["core"][j], cur, nxt, nat["freqs"], cache.native(), slots[j], B, S, pos0, ws,
+            kv_j = kv if uniform else cache.native([steps[j]], pos0)
+            hip.sandwich_block(nat["dims"], nat["core"][j], cur, nxt, nat["freqs"], kv_j, slots[j], B, S, pos0, ws,
                                ln_f=lnw if last else None)
             cur = nxt
         if n_core == 0:
@@ -769,6 +777,10 @@ class DecodeRunner:
         The returned tensors are the runner's own buffers: copy what must outlive the next step."""
         m, c = self.model, self.cache
         pos0 = c._seen_tokens
+        last_step = m.config.n_layers_in_prelude + m.config.n_layers_in_recurrent_block * self.r - 1
+        if c.has_gap(last_step, pos0):
+            raise NotImplementedError("the decode runner's fixed launch sequence needs a cache whose earlier tokens were all "
+                                      f"computed with at least {self.r} recurrences; use forward() for partially filled caches")
         if pos0 + 1 > c.t_max:
             c.ensure(1, 0, self.B, m.config.n_heads, m.config.head_dim, pos0 + 1, m.dtype, m.device)  # grows; pointers move
             self.graph = None

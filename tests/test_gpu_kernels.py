@@ -407,6 +407,67 @@ def test_decode_attention_at_the_maximum_context(pkg):
         pkg.hip.decode_attention(q.cuda(), cache, 0, 1, 1, t_max, nh, hd, workspace=ws)  # one past the end
 
 
+@pytest.mark.parametrize("B,S,pos0", [(1, 1, 1000), (32, 1, 300), (2, 3, 200)])
+@pytest.mark.parametrize("mode", ["skip", "latest", "always_last"])
+def test_decode_attention_partially_filled_slots(pkg, mode, B, S, pos0):
+    """steps_present: positions of earlier tokens hold different numbers of core steps; the kernel reads each from the
+    slot the lookup rule names (or leaves it out) -- checked against a gather done on the host, at the 3.5b head shape,
+    with and without the split over positions, unfused and fused."""
+    dt, nh, hd, t_max, h = torch.bfloat16, 55, 96, 1024, 55 * 96
+    n_slots, core0 = 14, 2          # slots 0, 1: coda; 2..13: core steps 0..11 (three recurrences of four blocks)
+    k, v = rnd((n_slots, B, nh, t_max, hd), dt, 200), rnd((n_slots, B, nh, t_max, hd), dt, 201)
+    kd, vd = k.cuda(), v.cuda()
+    g = torch.Generator().manual_seed(202)
+    depth = torch.randint(1, 4, (t_max,), generator=g, dtype=torch.int32) * 4  # 4, 8 or 12 core steps per position
+    code = {"skip": pkg.hip.LOOKUP_SKIP, "latest": pkg.hip.LOOKUP_LATEST, "always_last": pkg.hip.LOOKUP_ALWAYS_LAST}[mode]
+    depth_d = depth.cuda()          # the descriptor holds raw pointers: keep the tensors alive
+    cache = pkg.hip.make_cache(kd, vd, depth_d, code, core0)
+    ws = pkg.hip.attention_workspace(B * S, nh, hd, "cuda")
+    T = pos0 + S
+    for cs in (1, 6, 11):           # the step being read: first, second, third recurrence
+        slot = core0 + cs
+        src = torch.full((T,), slot, dtype=torch.long)
+        keep = torch.ones(T, dtype=torch.bool)
+        for p in range(pos0):       # positions from pos0 on are the call's own rows
+            d, j = int(depth[p]), cs % 4
+            if mode != "always_last" and cs < d:
+                continue
+            if mode == "skip":
+                keep[p] = False
+            else:
+                src[p] = core0 + j + (d - 1 - j) // 4 * 4
+        ar = torch.arange(T)
+        kk, vv = k[src, :, :, ar].permute(1, 2, 0, 3), v[src, :, :, ar].permute(1, 2, 0, 3)  # [B, nh, T, hd]
+        q = rnd((B * S, h), dt, 203 + cs)
+        qq = q.view(B, S, nh, hd).transpose(1, 2).float()
+        mask = keep.view(1, T).expand(S, T) & torch.ones(S, T, dtype=torch.bool).tril(T - S)
+        want = F.scaled_dot_product_attention(qq, kk.float(), vv.float(), attn_mask=mask).transpose(1, 2).reshape(B * S, h)
+        y = pkg.hip.decode_attention(q.cuda(), cache, slot, B, S, pos0, nh, hd, workspace=ws)
+        check(y, want, dt, f"{mode} cs={cs}")
+        y = pkg.hip.decode_attention(q.cuda(), cache, slot, B, S, pos0, nh, hd)
+        check(y, want, dt, f"{mode} cs={cs}, no split")
+    # the fused decode step appends its own row and resolves the older ones the same way
+    if S == 1:
+        cs, slot = 6, core0 + 6
+        qkv = rnd((B, 3 * h), dt, 210)
+        table = O.rope_table(hd, t_max, 50000.0).to(dt)
+        freqs = table.float().reshape(t_max, hd // 2, 2).contiguous().cuda()
+        kd2, vd2 = kd.clone(), vd.clone()
+        c2 = pkg.hip.make_cache(kd2, vd2, depth_d, code, core0)
+        y_f = pkg.hip.qkv_attention_decode(qkv.cuda(), None, freqs, cache, slot, B, pos0, nh, hd, workspace=ws)
+        q2 = pkg.hip.qkv_bias_rope_cache_append(qkv.cuda(), None, freqs, c2, slot, B, 1, pos0, nh, hd)
+        y_2 = pkg.hip.decode_attention(q2, c2, slot, B, 1, pos0, nh, hd, workspace=ws)
+        assert torch.equal(kd, kd2) and torch.equal(vd, vd2)
+        check(y_f, y_2.float().cpu(), dt, f"{mode}: fused equals append-then-attend")
+    # prelude / coda slots ignore the lookup table
+    q = rnd((B * S, h), dt, 220)
+    plain = pkg.hip.make_cache(kd, vd)
+    assert torch.equal(pkg.hip.decode_attention(q.cuda(), cache, 0, B, S, pos0, nh, hd, workspace=ws),
+                       pkg.hip.decode_attention(q.cuda(), plain, 0, B, S, pos0, nh, hd, workspace=ws))
+    with pytest.raises(pkg.hip.RavenHipError, match="steps_present"):
+        pkg.hip.prefill_attention(q.cuda(), cache, core0, B, S, pos0, nh, hd)
+
+
 def test_decode_attention_zero_query_gives_mean(pkg):
     dt, nh, hd, T = torch.bfloat16, 55, 96, 513
     k, v, kd, vd, cache = make_cache(pkg, 1, 1, nh, 1024, hd, dt, fill_seed=95)

@@ -203,6 +203,48 @@ def test_wide_prefill_path_bf16(pkg, tiny16, B, S):
     assert cache.get_seq_length() == ref_cache.get_seq_length() == S + 1
 
 
+@pytest.fixture(scope="module")
+def small242(pkg):
+    """2 prelude / 4 core / 2 coda blocks like the 3.5b model (the cache's lookup strategies hard-code that structure)."""
+    s = O.RavenShape(n_embd=128, n_heads=2, intermediate_size=352, vocab_size=512, n_layers_in_prelude=2,
+                     n_layers_in_recurrent_block=4, n_layers_in_coda=2, mean_recurrence=4)
+    w = O.make_weights(s, seed=3, dtype=torch.float32)
+    for k in w:  # weights large enough for attention to matter in the comparison
+        if k.endswith("Wqkv.weight"):
+            w[k] = w[k] * 8
+    cfg = pkg.RavenConfig(n_embd=128, n_heads=2, n_layers=8, n_layers_in_prelude=2, n_layers_in_recurrent_block=4,
+                          n_layers_in_coda=2, intermediate_size=352, vocab_size=512, mean_recurrence=4)
+    return s, w, build_model(pkg, cfg, w, torch.float32)
+
+
+@pytest.mark.parametrize("strategy", ["full", "skip", "latest-m4", "available-m4", "always-last-m4", "latest-m4-compress-s4"])
+def test_partially_filled_cache_lookups_in_the_attention_kernels(pkg, small242, strategy):
+    """Tokens computed with different numbers of recurrences (what per-token adaptive compute leaves behind): the
+    attention kernels resolve positions that are not cached at a step as HuginnDynamicCache.update does (RMM:199-253)."""
+    s, w, model = small242
+    g = torch.Generator().manual_seed(11)
+    B = 2
+    ref_cache, cache = O.DictCache(strategy), pkg.HuginnDynamicCache(strategy)
+    pos = 0
+    # (new tokens, recurrences): prefill, then tokens that stop early or go deeper, one 2-token chunk among them
+    for n_new, r in ((6, 3), (1, 1), (1, 4), (2, 2), (1, 5), (1, 3), (1, 5)):
+        ids = torch.randint(0, s.vocab_size, (B, n_new), generator=g)
+        states = O.initialize_state(torch.empty(B, n_new, s.n_embd), s, 1.0, g)
+        cp = torch.arange(pos, pos + n_new)
+        want = O.forward(w, s, input_ids=ids, input_states=states, past_key_values=ref_cache, use_cache=True,
+                         cache_position=cp, num_steps=r)
+        got = model(input_ids=ids.cuda(), input_states=states.cuda(), past_key_values=cache, use_cache=True,
+                    cache_position=cp.cuda(), num_steps=r)
+        check(got.logits, want.logits, torch.float32, f"{strategy}: logits of {n_new} tokens at {pos} with r={r}")
+        pos += n_new
+    assert cache.get_seq_length() == ref_cache.get_seq_length() == pos
+    for step in ref_cache.key_cache:
+        assert sorted(cache.key_cache[step].keys()) == sorted(ref_cache.key_cache[step].keys()), step
+        for p, kref in ref_cache.key_cache[step].items():
+            check(cache.key_cache[step][p], kref, torch.float32, f"{strategy}: K[{step}][{p}]")
+    assert cache.get_memory_usage() == ref_cache.get_memory_usage()
+
+
 def test_piecewise_surface_equals_forward(tiny32):
     """embed_inputs -> iterate_one_step x r -> predict_from_latents reproduces forward (RMM:841-934)."""
     s, w, model = tiny32

@@ -147,3 +147,49 @@ def test_static_cache_known_answer_and_interface(pkg):
     assert torch.equal(gk, k) and list(c.key_cache) == [0, -1]
     s16 = pkg.HuginnStaticCache(max_length=8, max_num_steps=132, num_heads=2, hidden_dim=4, lookup_strategy="latest-m4-compress-s16")
     assert s16.max_num_steps == 20
+
+
+@pytest.mark.parametrize("strategy", ["full", "skip", "latest-m4", "available-m4", "always-last-m4", "latest-m4-compress-s4"])
+def test_cache_lookups_with_partially_filled_steps_match_dict_model(pkg, strategy):
+    """Tokens computed with different numbers of recurrences: every update of the contiguous cache returns what the
+    brute-force dict model of the reference's cache returns (RMM:199-253)."""
+    g = torch.Generator().manual_seed(5)
+    ours, ref = pkg.HuginnDynamicCache(strategy), O.DictCache(strategy)
+    # (new tokens, recurrences): a prefill, then single tokens that stop earlier or go deeper
+    for n_new, r in ((5, 3), (1, 1), (1, 4), (2, 2), (1, 6), (1, 3)):
+        for step in [0, 1] + list(range(2, 2 + 4 * r)) + [-1, -2]:
+            k, v = torch.randn(2, 3, n_new, 8, generator=g), torch.randn(2, 3, n_new, 8, generator=g)
+            got, want = ours.update(k, v, step), ref.update(k, v, step)
+            assert got[0].shape == want[0].shape, (strategy, step, got[0].shape, want[0].shape)
+            assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]), (strategy, step)
+        assert ours.get_seq_length() == ref.get_seq_length()
+        assert ours.get_memory_usage() == ref.get_memory_usage()
+    for step in ref.key_cache:
+        assert sorted(ours.key_cache[step].keys()) == sorted(ref.key_cache[step].keys()), step
+    ours.clear_last_k_entries(2)
+    ref.clear_last_k_entries(2)
+    k = torch.randn(2, 3, 1, 8, generator=g)
+    for step in [0, 1] + list(range(2, 2 + 4 * 5)):
+        got, want = ours.update(k, k, step), ref.update(k, k, step)
+        assert torch.equal(got[0], want[0]), (strategy, step)
+
+
+def test_cache_lookup_errors(pkg):
+    c = pkg.HuginnDynamicCache("latest-m4")
+    k = torch.zeros(1, 1, 1, 4)
+    for step in (0, 1, 2, 3, 4, 5):
+        c.update(k, k, step)
+    for step in (0, 1, 2, 3, 4, 5, 6):
+        c.update(k, k, step)
+    c2 = pkg.HuginnDynamicCache("randomized")
+    for step in (0, 1, 2, 3, 4, 5):
+        c2.update(k, k, step)
+    for step in (0, 1, 2, 3, 4, 5):
+        c2.update(k, k, step)
+    with pytest.raises(NotImplementedError, match="randomized"):
+        c2.update(k, k, 6)
+    c3 = pkg.HuginnDynamicCache("no-such-strategy")
+    for step in (0, 1, 2, 3, 4, 5, 0, 1, 2, 3, 4, 5):
+        c3.update(k, k, step)
+    with pytest.raises(ValueError, match="Unknown lookup strategy"):
+        c3.update(k, k, 6)

@@ -346,6 +346,40 @@ def test_dict_cache_against_list_model():
     assert cache.get_seq_length() == 0 and not cache.key_cache
 
 
+def test_partial_fill_lookups_closed_form():
+    """Tokens with different numbers of recurrences: entries are tagged with (step, position), so what a lookup
+    returns names its source.  For a token that ran d recurrences, block j of recurrence i (step 2 + 4i + j) must come
+    from recurrence min(i, d - 1) under latest-m4 / available-m4, from recurrence d - 1 under always-last-m4 whenever
+    the step has a gap at all, and is dropped by skip / full when i >= d (RMM:199-253)."""
+    depths = [3, 1, 4, 2, 5]  # recurrences per token; the querying token runs 5
+    for strategy in ("latest-m4", "available-m4", "always-last-m4", "skip", "full"):
+        c = O.DictCache(strategy)
+        for pos, d in enumerate(depths):
+            for step in [0, 1] + list(range(2, 2 + 4 * d)):
+                tag = torch.full((1, 1, 1, 1), float(step * 100 + pos))
+                k, _ = c.update(tag, tag, step)
+                got = [(int(t) // 100, int(t) % 100) for t in k.flatten().tolist()]
+                if step < 2:
+                    assert got == [(step, p) for p in range(pos + 1)]
+                    continue
+                i, j = divmod(step - 2, 4)
+                older = depths[:pos]
+                gap = any(dd <= i for dd in older)
+                want = []
+                for p, dd in enumerate(older):
+                    if not gap or (strategy in ("latest-m4", "available-m4") and i < dd):
+                        want.append((step, p))
+                    elif strategy in ("skip", "full"):
+                        if i < dd:
+                            want.append((step, p))
+                    elif strategy == "always-last-m4":
+                        want.append((2 + 4 * (dd - 1) + j, p))
+                    else:
+                        want.append((2 + 4 * min(i, dd - 1) + j, p))
+                want.append((step, pos))
+                assert got == want, (strategy, pos, step, got, want)
+
+
 def test_step_remap_strategies():
     assert [O.remap_step(i, "full") for i in (0, 1, 2, 129, -1)] == [0, 1, 2, 129, -1]
     assert [O.remap_step(i, "latest-m4-compress-s4") for i in (0, 1, 2, 5, 6, 9, 129, -1, -2)] == [0, 1, 2, 5, 2, 5, 5, -1, -2]
