@@ -130,6 +130,20 @@ int    raven_linear(const void* x0, const void* x1, const void* w, const void* r
                     int32_t M, int32_t N, int32_t K0, int32_t K1, int32_t swiglu, int32_t out_f32,
                     int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Statistics behind the per-iteration exit criteria of adaptive compute (RMM:2128-2260), one value per row.
+ * raven_exit_logit_stats on logits [rows, V] float:
+ *   RAVEN_EXIT_ENTROPY  out = -sum p log(p + 1e-10), p = softmax(logits)                       (RMM:2142-2144)
+ *   RAVEN_EXIT_KL       lp = log_softmax(logits); out = sum exp(prev) (prev - lp); prev <- lp  (RMM:2182-2186)
+ *   RAVEN_EXIT_MINP_KL  the same with p[p < 0.1 max p] = 1/V, renormalised, before the log     (RMM:2200-2216)
+ * prev_log_probs [rows, V] float is read and overwritten by the KL kinds (NULL for the entropy).
+ * raven_exit_latent_stats on latents, prev [rows, h] of T: rel_change = |latents - prev| / |latents| (RMM:2162),
+ * cosine = <latents, prev> / |latents| / |prev| (RMM:2256), each [rows] of T, either may be NULL. */
+enum { RAVEN_EXIT_ENTROPY = 0, RAVEN_EXIT_KL = 1, RAVEN_EXIT_MINP_KL = 2 };
+int raven_exit_logit_stats(const float* logits, float* prev_log_probs, float* out, int32_t rows, int32_t V,
+                           int32_t kind, void* stream);
+int raven_exit_latent_stats(const void* latents, const void* prev, void* rel_change, void* cosine,
+                            int32_t rows, int32_t h, int32_t dtype, void* stream);
+
 /* Decode fast path for ONE token row, one launch:
  *     x  = norm_a ? T(rmsnorm(x0) * norm_a) : x0      -> stored to xa_out when non-NULL
  *     x  = norm_b ? T(rmsnorm(x)  * norm_b) : x

@@ -24,6 +24,14 @@ How each function is pinned (tests/test_oracle_pins.py), without running the ref
   block/iterate/forward/greedy   composition laws (r=0, cache vs no-cache,
                      prefill-then-decode vs token-by-token)                       -> pinned
   initialize_state   bounds, std, scale=0, generator determinism                  -> pinned
+  DictCache lookups  (latest-m4, available-m4, always-last-m4, skip) closed form on
+                     step-tagged entries                                          -> pinned
+  ExitCriterion      entropy of uniform / one-hot rows, KL(p, p) = 0 and two-point closed
+                     form, fp64 brute force, min-p floor by hand, latent ratios of scaled /
+                     orthogonal vectors, argmax streak counting                    -> pinned
+  embed_inputs / iterate_one_step / predict_from_latents / generate_with_adaptive_compute
+                     pieces compose to forward(); criterion "none" equals greedy_generate;
+                     num-steps evaluator equals forward(num_steps=k) token by token -> pinned
 The reference holds no golden vectors for this path (it has no test suite); the only
 exact numbers it publishes are three KV-cache sizes, used as known-answer tests.
 """
@@ -445,6 +453,230 @@ def greedy_generate(w, s: RavenShape, input_ids: torch.Tensor, max_new_tokens: i
         record["margins"] = margins
         record["cache"] = cache
     return ids
+
+
+# --------------------------------------------------------------------------------------
+# adaptive compute: per-iteration exit criteria and the generate loop around them
+# (RMM:841-934 pieces of the forward, 1552-1749 the loop, 2099-2307 the criteria)
+# --------------------------------------------------------------------------------------
+def embed_inputs(w, s: RavenShape, input_ids, cache=None, cache_position=None, position_ids=None):
+    """RMM:902-934: embedding times sqrt(h), then the prelude; returns (embeds, block_idx)."""
+    freqs = pick_freqs(w["freqs_cis"], input_ids.shape[1], position_ids, cache_position)
+    x = F.embedding(input_ids, w["transformer.wte.weight"]) * s.emb_scale
+    block_idx = -1
+    for i in range(s.n_layers_in_prelude):
+        block_idx += 1
+        x = sandwich_block(x, w, f"transformer.prelude.{i}", freqs, block_idx, cache, s)
+    return x, block_idx
+
+
+def iterate_one_step(w, s: RavenShape, embeds, states, block_idx: int, cache=None, cache_position=None, position_ids=None):
+    """RMM:841-868: one recurrence; returns (state, block_idx)."""
+    freqs = pick_freqs(w["freqs_cis"], embeds.shape[1], position_ids, cache_position)
+    return core_block_forward(states, embeds, w, freqs, cache, block_idx, s)
+
+
+def predict_from_latents(w, s: RavenShape, latents, cache=None, cache_position=None, position_ids=None) -> OracleOutput:
+    """RMM:870-900: ln_f, coda (step indices -1, -2, ...), ln_f, tied head, float logits."""
+    freqs = pick_freqs(w["freqs_cis"], latents.shape[1], position_ids, cache_position)
+    x = rmsnorm(latents, w["transformer.ln_f.weight"], s.norm_eps)
+    block_idx = 0
+    for i in range(s.n_layers_in_coda):
+        block_idx -= 1
+        x = sandwich_block(x, w, f"transformer.coda.{i}", freqs, block_idx, cache, s)
+    x = rmsnorm(x, w["transformer.ln_f.weight"], s.norm_eps)
+    return OracleOutput(logits=linear(x, w["lm_head.weight"]).float(), latent_states=x, past_key_values=cache)
+
+
+EXIT_AUTO = {"entropy-diff": 1e-3, "latent-diff": 0.03, "cosine": 1e-3, "kl": 1e-3, "minp-kl": 1e-5, "argmax-stability": 5}
+
+
+class ExitCriterion:
+    """The per-iteration exit evaluators of RMM:2099-2307 behind one class (reduce=True, the generate loop's use).
+
+    check(latents, predict) -> (exit?[B] bool, outputs or None, value[B]); `predict` maps latents to an
+    OracleOutput (the coda and the head) and is only called by the criteria that look at logits."""
+
+    def __init__(self, criterion: str, threshold="auto", vocab: int = 0, steps_fn=None):
+        if criterion == "none" or criterion == "num-steps":
+            self.kind = criterion
+        elif criterion in ("entropy-diff", "latent-diff", "cosine", "argmax-stability"):
+            self.kind = criterion
+        elif "kl" in criterion:                      # RMM:2295-2299: any other name containing "kl" is the plain KL
+            self.kind = "minp-kl" if criterion == "minp-kl" else "kl"
+        else:
+            raise ValueError(f"Invalid adaptive compute strategy: {criterion}")
+        if self.kind in EXIT_AUTO:
+            t = EXIT_AUTO[self.kind] if threshold == "auto" else threshold
+            self.threshold = int(t) if self.kind == "argmax-stability" else float(t)
+        self.V, self.steps_fn, self.counter = vocab, steps_fn, 0
+
+    def init(self, latents: torch.Tensor) -> None:
+        B = latents.shape[0]
+        if self.kind == "entropy-diff":
+            self.prev = torch.ones(B) * 100.0                                    # RMM:2135-2137
+        elif self.kind in ("latent-diff", "cosine"):
+            self.prev = latents.clone()                                          # RMM:2156-2157, 2250-2251
+        elif self.kind in ("kl", "minp-kl"):
+            self.prev = ((1 / self.V) * torch.ones(B, self.V)).log()             # RMM:2175-2177
+        elif self.kind == "argmax-stability":
+            self.prev = torch.ones(B, dtype=torch.long) * -1                     # RMM:2225-2228
+            self.stable = torch.zeros(B, dtype=torch.long)
+        elif self.kind == "num-steps":                                           # RMM:2269-2272
+            self.target, self.current = self.steps_fn(self.counter), 0
+            self.counter += 1
+
+    def check(self, latents: torch.Tensor, predict):
+        B = latents.shape[0]
+        if self.kind == "none":                                                  # RMM:2120-2125
+            return torch.zeros(B, dtype=torch.bool), None, torch.zeros(B)
+        if self.kind == "num-steps":                                             # RMM:2274-2281
+            self.current += 1
+            return torch.full((B,), self.current >= self.target, dtype=torch.bool), None, torch.zeros(B)
+        if self.kind == "latent-diff":                                           # RMM:2159-2167
+            v = ((latents - self.prev).norm(dim=-1) / latents.norm(dim=-1)).mean(dim=-1)
+            self.prev = latents.clone()
+            return v < self.threshold, None, v
+        if self.kind == "cosine":                                                # RMM:2253-2260
+            cos = (latents * self.prev).sum(dim=-1) / latents.norm(dim=-1) / self.prev.norm(dim=-1)
+            v = 1 - cos.mean(dim=1)
+            self.prev = latents.clone()
+            return v < self.threshold, None, v
+        out = predict(latents)
+        last = out.logits[:, -1, :]
+        if self.kind == "entropy-diff":                                          # RMM:2139-2148
+            probs = F.softmax(last, dim=-1)
+            entropy = -torch.sum(probs * torch.log(probs + 1e-10), dim=-1)
+            v = (entropy - self.prev).abs()
+            self.prev = entropy
+            return v < self.threshold, out, v
+        if self.kind == "argmax-stability":                                      # RMM:2230-2241
+            cur = last.argmax(dim=-1)
+            self.stable = torch.where(cur == self.prev, self.stable + 1, torch.zeros_like(self.stable))
+            self.prev = cur
+            return self.stable >= self.threshold, out, self.stable
+        if self.kind == "kl":                                                    # RMM:2179-2187
+            logp = F.log_softmax(last, dim=-1)
+        else:                                                                    # RMM:2200-2216
+            probs = F.softmax(last, dim=-1)
+            small = probs < 0.1 * probs.max(dim=-1, keepdim=True)[0]
+            probs = torch.where(small, torch.full_like(probs, 1 / self.V), probs)
+            logp = (probs / probs.sum(dim=-1, keepdim=True)).log()
+        v = F.kl_div(logp, self.prev, reduction="none", log_target=True).sum(dim=-1)
+        self.prev = logp
+        return v < self.threshold, out, v
+
+
+def generate_with_adaptive_compute(w, s: RavenShape, input_ids: torch.Tensor, max_new_tokens: int, criterion="none",
+                                   exit_threshold="auto", num_steps=None, state_fn=None, continuous_compute=False,
+                                   cache_lookup_strategy="full", do_not_exit_in_prefill=False, min_steps=0,
+                                   check_criterion_every_n_steps=1, stop_tokens=(), init_scale=1.0, evaluator=None,
+                                   record: Optional[dict] = None):
+    """Greedy generate_with_adaptive_compute, RMM:1552-1749.  Every sequence of a batch keeps iterating until all
+    have met the criterion (or max_steps); a sequence's logits are frozen at the step where it met it.
+    `state_fn(call, shape)` supplies the initial latent state of each token step (call 0 is the prompt).
+    Returns (ids, [per token: per sequence compute steps])."""
+    cache = DictCache(cache_lookup_strategy)
+    max_steps = s.mean_recurrence if num_steps is None else num_steps
+    ids = input_ids.clone()
+    B = ids.shape[0]
+    draw = (lambda call, shape: state_fn(call, shape)) if state_fn is not None else \
+        (lambda call, shape: initialize_state(torch.empty(shape), s, init_scale))
+    carried = draw(0, (B, ids.shape[1], s.n_embd)) if continuous_compute else None      # RMM:1589-1591
+    unfinished = torch.ones(B, dtype=torch.bool)
+    ev = evaluator if evaluator is not None else ExitCriterion(criterion, exit_threshold, s.vocab_size)
+    steps_log, values_log = [], []
+    for token_step in range(max_new_tokens):
+        seen = cache.get_seq_length()
+        pos = torch.arange(seen, ids.shape[1])
+        aux = dict(cache=cache, cache_position=pos)
+        embeds, block_idx = embed_inputs(w, s, ids[:, pos], **aux)
+        latents = carried if continuous_compute else draw(token_step, tuple(embeds.shape))
+        if continuous_compute:
+            next_states = latents[:, -1:, :].clone()
+        predict = lambda lat: predict_from_latents(w, s, lat, **aux)
+        steps_per_seq, values_per_seq = [0] * B, [[] for _ in range(B)]
+        exit_reached = torch.zeros(B, dtype=torch.bool)
+        outputs, next_logits = None, None
+        ev.init(latents)
+        broke = False
+        for compute_step in range(max_steps):
+            latents, block_idx = iterate_one_step(w, s, embeds, latents, block_idx, **aux)
+            if (compute_step < min_steps or (compute_step - min_steps) % check_criterion_every_n_steps != 0
+                    or (do_not_exit_in_prefill and token_step == 0)):
+                continue
+            new_exits, outputs, values = ev.check(latents, predict)
+            for i in range(B):
+                if not exit_reached[i] and unfinished[i]:
+                    values_per_seq[i].append(float(values[i]))
+            new_exits = new_exits & ~exit_reached & unfinished
+            if new_exits.any():
+                exit_reached = exit_reached | new_exits
+                if outputs is None:
+                    outputs = predict(latents)
+                if next_logits is None:
+                    next_logits = outputs.logits[:, -1, :].float().clone()
+                else:
+                    next_logits[new_exits] = outputs.logits[new_exits, -1, :].float()
+                for i in range(B):
+                    if new_exits[i]:
+                        steps_per_seq[i] = compute_step + 1
+                if continuous_compute:
+                    next_states[new_exits] = latents[new_exits, -1:, :]
+            if (exit_reached | ~unfinished).all():
+                broke = True
+                break
+        if not broke:                                                                   # the loop's else branch
+            if outputs is None:
+                outputs = predict(latents)
+            if next_logits is None:
+                next_logits = outputs.logits[:, -1, :].float().clone()
+                steps_per_seq = [max_steps] * B
+            else:
+                for i in range(B):
+                    if not exit_reached[i] and unfinished[i]:
+                        next_logits[i] = outputs.logits[i, -1, :].float()
+                        steps_per_seq[i] = max_steps
+        if continuous_compute:
+            running = ~exit_reached & unfinished
+            next_states[running] = latents[running, -1:, :]
+            carried = next_states
+        steps_log.append(steps_per_seq)
+        values_log.append(values_per_seq)
+        nxt = next_logits.argmax(dim=-1, keepdim=True)
+        ids = torch.cat([ids, nxt], dim=-1)
+        for i in range(B):
+            if unfinished[i] and int(nxt[i, 0]) in stop_tokens:
+                unfinished[i] = False
+        if not unfinished.any():
+            break
+    if record is not None:
+        record["cache"], record["exit_values"] = cache, values_log
+    return ids, steps_log
+
+
+def prefill_with_varied_exit_steps(w, s: RavenShape, input_ids: torch.Tensor, evaluator: ExitCriterion, state_fn=None,
+                                   init_scale: float = 1.0, cache: Optional[DictCache] = None):
+    """RMM:937-996: token by token, each token leaves the recurrence when the evaluator says so.
+    Returns (logits [1, S, V], cache, compute steps per token)."""
+    assert input_ids.shape[0] == 1
+    cache = DictCache() if cache is None else cache
+    rows, steps = [], []
+    for p in range(input_ids.shape[1]):
+        aux = dict(cache=cache, cache_position=torch.tensor([p]))
+        embeds, block_idx = embed_inputs(w, s, input_ids[:, p:p + 1], **aux)
+        latents = state_fn(p, tuple(embeds.shape)) if state_fn is not None else initialize_state(embeds, s, init_scale)
+        evaluator.init(latents)
+        predict = lambda lat: predict_from_latents(w, s, lat, **aux)
+        step = -1
+        for step in range(s.mean_recurrence):
+            latents, block_idx = iterate_one_step(w, s, embeds, latents, block_idx, **aux)
+            exits, _, _ = evaluator.check(latents, predict)
+            if exits.any():
+                break
+        steps.append(step + 1)
+        rows.append(predict(latents).logits)
+    return torch.cat(rows, dim=1), cache, steps
 
 
 # --------------------------------------------------------------------------------------

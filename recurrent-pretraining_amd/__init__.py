@@ -6,6 +6,19 @@ registers this directory under that name).
 """
 
 from . import hip  # noqa: F401
+from . import adaptive  # noqa: F401
+from .adaptive import (  # noqa: F401
+    ArgmaxStabilityExitEvaluator,
+    CosineExitEvaluator,
+    EntropyDiffExitEvaluator,
+    KLExitEvaluator,
+    LatentDiffExitEvaluator,
+    MinKLExitEvaluator,
+    NoOpExitEvaluator,
+    NumStepsGenerator,
+    PerIterationExitEvaluator,
+    get_adaptive_exit_evaluator,
+)
 from .cache import HuginnDynamicCache, HuginnStaticCache, remap_step  # noqa: F401
 from .config import RavenConfig  # noqa: F401
 from .modeling import (  # noqa: F401
@@ -18,5 +31,8 @@ from .modeling import (  # noqa: F401
 
 __all__ = [
     "hip", "HuginnDynamicCache", "HuginnStaticCache", "remap_step", "RavenConfig", "RavenForCausalLM", "DecodeRunner",
-    "CausalLMOutputRecurrentLatents", "GenerationSettings", "precompute_freqs_cis",
+    "CausalLMOutputRecurrentLatents", "GenerationSettings", "precompute_freqs_cis", "adaptive",
+    "PerIterationExitEvaluator", "NoOpExitEvaluator", "EntropyDiffExitEvaluator", "LatentDiffExitEvaluator",
+    "KLExitEvaluator", "MinKLExitEvaluator", "ArgmaxStabilityExitEvaluator", "CosineExitEvaluator", "NumStepsGenerator",
+    "get_adaptive_exit_evaluator",
 ]

@@ -56,6 +56,8 @@ SIGNATURES = {
     "raven_gemm_swiglu": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I32, _I32, _VP]),
     "raven_linear_workspace_bytes": (_SZ, [_I32, _I32]),
     "raven_linear": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _VP, _SZ, _VP]),
+    "raven_exit_logit_stats": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I32, _VP]),
+    "raven_exit_latent_stats": (C.c_int, [_VP, _VP, _VP, _VP, _I32, _I32, _I32, _VP]),
     "raven_gemv_fused": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _F, _I32, _I32, _I32, _VP]),
     "raven_qkv_bias_rope_cache_append": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32,
                                                    _VP, _I32, _I32, _I32, _VP]),
@@ -224,6 +226,30 @@ def linear(x0, w, x1=None, residual=None, swiglu=False, out_f32=False, workspace
                              0 if workspace is None else workspace.numel(), _stream())
     _check(rc, "raven_linear")
     return y
+
+
+EXIT_ENTROPY, EXIT_KL, EXIT_MINP_KL = 0, 1, 2
+
+
+def exit_logit_stats(logits, kind: int, prev_log_probs=None):
+    """One float per row of logits [rows, V] (float): entropy, or KL against prev_log_probs, which is overwritten."""
+    rows, V = logits.shape
+    out = torch.empty(rows, device=logits.device, dtype=torch.float32)
+    rc = load().raven_exit_logit_stats(_ptr(logits, "logits", torch.float32), _ptr(prev_log_probs, "prev_log_probs", torch.float32),
+                                       _ptr(out, "out"), rows, V, int(kind), _stream())
+    _check(rc, "raven_exit_logit_stats")
+    return out
+
+
+def exit_latent_stats(latents, prev, want_rel=True, want_cos=False):
+    """latents, prev [rows, h] -> (|latents - prev| / |latents|, cosine), each [rows] in the inputs' dtype or None."""
+    rows, h = latents.shape
+    rel = torch.empty(rows, device=latents.device, dtype=latents.dtype) if want_rel else None
+    cos = torch.empty(rows, device=latents.device, dtype=latents.dtype) if want_cos else None
+    rc = load().raven_exit_latent_stats(_ptr(latents, "latents"), _ptr(prev, "prev", latents.dtype), _ptr(rel, "rel"), _ptr(cos, "cos"),
+                                        rows, h, dtype_code(latents.dtype), _stream())
+    _check(rc, "raven_exit_latent_stats")
+    return rel, cos
 
 
 def gemv_fused(x0, w, x1=None, norm_a=None, norm_b=None, want_xa=False, residual=None, swiglu=False, out_f32=False, eps=1e-6):

@@ -602,13 +602,32 @@ class RavenForCausalLM(torch.nn.Module):
 
     @torch.no_grad()
     def generate(self, input_ids: torch.Tensor, generation_config=None, **kwargs):
-        """Dispatcher of RMM:1112-1127.  The adaptive-compute, speculative and diffusion-style loops
-        of the reference are not part of this package; everything else goes to generate_minimal."""
-        for k in ("criterion", "exit_threshold", "exit_evaluator", "draft_steps", "lookahead_for_draft",
-                  "verification_threshold", "headway", "state_noise_mixing", "inner_recurrence", "freeze_strategy"):
+        """Dispatcher of RMM:1112-1127: `criterion` / `exit_threshold` / `exit_evaluator` select the adaptive-compute
+        loop; the speculative and diffusion-style loops of the reference are not part of this package; everything else
+        goes to generate_minimal (the reference hands those calls to transformers' GenerationMixin)."""
+        if any(k in kwargs for k in ("criterion", "exit_threshold", "exit_evaluator")):
+            return self.generate_with_adaptive_compute(input_ids, generation_config, **kwargs)
+        for k in ("draft_steps", "lookahead_for_draft", "verification_threshold", "headway", "state_noise_mixing",
+                  "inner_recurrence", "freeze_strategy"):
             if k in kwargs:
                 raise NotImplementedError(f"generate(..., {k}=...) selects a sampler this package does not provide")
         return self.generate_minimal(input_ids, generation_config, **kwargs)
+
+    def generate_with_adaptive_compute(self, input_ids: torch.Tensor, generation_config=None, **kwargs):
+        """RMM:1552-1749; see adaptive.generate_with_adaptive_compute."""
+        from . import adaptive
+        return adaptive.generate_with_adaptive_compute(self, input_ids, generation_config, **kwargs)
+
+    def forward_with_adaptive_compute(self, input_ids: torch.Tensor, exit_evaluator, **kwargs):
+        """RMM:998-1035; see adaptive.forward_with_adaptive_compute."""
+        from . import adaptive
+        return adaptive.forward_with_adaptive_compute(self, input_ids, exit_evaluator, **kwargs)
+
+    def _prefill_with_varied_exit_steps(self, input_ids: torch.Tensor, exit_evaluator, past_key_values=None,
+                                        init_scale: float = 1.0, **kwargs):
+        """RMM:937-996; see adaptive.prefill_with_varied_exit_steps."""
+        from . import adaptive
+        return adaptive.prefill_with_varied_exit_steps(self, input_ids, exit_evaluator, past_key_values, init_scale, **kwargs)
 
     @torch.no_grad()
     def generate_minimal(self, input_ids: torch.Tensor, generation_config=None, tokenizer=None, streamer=None,

@@ -491,3 +491,61 @@ def test_embed_and_argmax(pkg):
     assert torch.equal(pkg.hip.argmax(logits.cuda()).cpu(), logits.argmax(-1))
     small = rnd((3, 1024), torch.float32, 102)
     assert torch.equal(pkg.hip.argmax(small.cuda()).cpu(), small.argmax(-1))
+
+
+# ----------------------------------------------------------------------------- adaptive-compute exit statistics
+@pytest.mark.parametrize("B,V", [(1, 65536), (3, 65536), (32, 1024), (2, 1000)])
+def test_exit_logit_stats(pkg, B, V):
+    """Entropy, KL and min-p KL of successive logits rows against the oracle's evaluators (fp32; sums over V terms
+    in another order: absolute 2e-5 + relative 1e-4)."""
+    g = torch.Generator().manual_seed(300 + B)
+    steps = [torch.randn(B, V, generator=g) * 3 for _ in range(2)]
+    steps.append(steps[-1] + torch.randn(B, V, generator=g) * 1e-2)     # a small change: KL of the order 1e-4
+    steps.append(steps[-1].clone())                                     # no change: KL 0
+    fake = lambda lg: (lambda lat: O.OracleOutput(logits=lg.unsqueeze(1), latent_states=lat))
+    lat = torch.zeros(B, 1, 4)
+    for kind, code in (("entropy-diff", pkg.hip.EXIT_ENTROPY), ("kl", pkg.hip.EXIT_KL), ("minp-kl", pkg.hip.EXIT_MINP_KL)):
+        ev = O.ExitCriterion(kind, "auto", V)
+        ev.init(lat)
+        prev = ((1 / V) * torch.ones(B, V)).log().cuda()
+        for i, lg in enumerate(steps):
+            ev.check(lat, fake(lg))
+            got = pkg.hip.exit_logit_stats(lg.cuda(), code, None if kind == "entropy-diff" else prev)
+            want = ev.prev if kind == "entropy-diff" else None
+            if kind == "entropy-diff":
+                assert torch.allclose(got.cpu(), want, rtol=1e-4, atol=2e-5), (kind, i, got, want)
+            else:
+                break
+        # KL kinds: compare the values and the stored log-probabilities step by step
+        if kind != "entropy-diff":
+            ev.init(lat)
+            prev = ((1 / V) * torch.ones(B, V)).log().cuda()
+            for i, lg in enumerate(steps):
+                _, _, v = ev.check(lat, fake(lg))
+                got = pkg.hip.exit_logit_stats(lg.cuda(), code, prev)
+                assert torch.allclose(got.cpu(), v, rtol=1e-3, atol=2e-5), (kind, i, got, v)
+                assert torch.allclose(prev.cpu(), ev.prev, rtol=1e-5, atol=1e-5), (kind, i)
+            assert float(got.abs().max()) < 1e-6                        # identical successive rows
+    with pytest.raises(pkg.hip.RavenHipError):
+        pkg.hip.exit_logit_stats(steps[0].cuda(), pkg.hip.EXIT_KL)      # KL without the previous log-probabilities
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_exit_latent_stats(pkg, dt):
+    B, S, h = 3, 5, 5280
+    a, b = rnd((B, S, h), dt, 310), rnd((B, S, h), dt, 311)
+    b = (a.float() * 0.9 + b.float() * 0.3).to(dt)
+    rel, cos = pkg.hip.exit_latent_stats(a.view(-1, h).cuda(), b.view(-1, h).cuda(), want_rel=True, want_cos=True)
+    want_rel = (a - b).norm(dim=-1) / a.norm(dim=-1)                     # the reference's expressions, in dtype
+    want_cos = (a * b).sum(dim=-1) / a.norm(dim=-1) / b.norm(dim=-1)
+    tol = dict(rtol=2e-2, atol=1e-2) if dt == torch.bfloat16 else dict(rtol=1e-5, atol=1e-6)
+    assert rel.dtype == dt and torch.allclose(rel.float().cpu().view(B, S), want_rel.float(), **tol)
+    assert torch.allclose(cos.float().cpu().view(B, S), want_cos.float(), **tol)
+    # closed forms: a = 2 b -> 1/2 and cosine 1; orthogonal rows -> cosine 0
+    x = torch.zeros(2, h, dtype=dt)
+    x[0, :7], x[1, 0] = 1.0, 3.0
+    y = x.clone() * 0.5
+    y[1] = 0
+    y[1, 1] = 2.0
+    rel, cos = pkg.hip.exit_latent_stats(x.cuda(), y.cuda(), want_rel=True, want_cos=True)
+    assert abs(float(rel[0]) - 0.5) < 1e-6 and abs(float(cos[0]) - 1.0) < 1e-2 and float(cos[1]) == 0.0

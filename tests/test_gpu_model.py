@@ -156,7 +156,7 @@ def test_generate_options(pkg, tiny32):
     assert torch.equal(c1, c2) and c1.shape == (2, 11)
     assert model.generate(prompt, max_length=9, stop_tokens=set()).shape == (2, 9)
     with pytest.raises(NotImplementedError):
-        model.generate(prompt, criterion="entropy-diff")
+        model.generate(prompt, draft_steps=4)       # the speculative sampler is not part of the package
     # the reference's preallocated cache class works as past_key_values too
     static = pkg.HuginnStaticCache(max_length=32, max_num_steps=4 + 4 * 4, num_heads=s.n_heads, hidden_dim=s.head_dim, batch_size=2,
                                    device="cuda", dtype=torch.float32)
@@ -243,6 +243,108 @@ def test_partially_filled_cache_lookups_in_the_attention_kernels(pkg, small242, 
         for p, kref in ref_cache.key_cache[step].items():
             check(cache.key_cache[step][p], kref, torch.float32, f"{strategy}: K[{step}][{p}]")
     assert cache.get_memory_usage() == ref_cache.get_memory_usage()
+
+
+def _adaptive_case(pkg, small242, B, prompt, n_new, oracle_kw, ours_kw, seed=21):
+    s, w, model = small242
+    g = torch.Generator().manual_seed(seed)
+    ids = torch.randint(0, s.vocab_size, (B, prompt), generator=g)
+    sf = lambda c, sh: O.initialize_state(torch.empty(sh), s, 1.0, torch.Generator().manual_seed(1000 * seed + c))
+    rec = {}
+    want_ids, want_steps = O.generate_with_adaptive_compute(w, s, ids, n_new, state_fn=sf, record=rec, stop_tokens=(),
+                                                            **oracle_kw)
+    gc = pkg.GenerationSettings(max_new_tokens=n_new, return_dict_in_generate=True)
+    out = model.generate_with_adaptive_compute(ids.cuda(), gc, input_states_fn=sf, stop_tokens=set(), **ours_kw)
+    return want_ids, want_steps, rec, out
+
+
+@pytest.mark.parametrize("criterion,threshold", [("entropy-diff", 2e-3), ("latent-diff", 0.35), ("cosine", 0.08), ("kl", 4e-3),
+                                                 ("minp-kl", 4e-3), ("argmax-stability", 2), ("none", "auto")])
+def test_generate_with_adaptive_compute_matches_oracle(pkg, small242, criterion, threshold):
+    """Per-token adaptive compute, batch of 2, up to 8 recurrences: the same tokens, the same number of recurrences
+    per token and sequence, exit values within fp32 reduction-order distance.  A flip of an exit decision would
+    need an exit value within that distance of the threshold; the test states the smallest margin it saw."""
+    kw = dict(criterion=criterion, exit_threshold=threshold, num_steps=8, cache_lookup_strategy="latest-m4")
+    want_ids, want_steps, rec, out = _adaptive_case(pkg, small242, 2, 5, 6, kw, kw)
+    got_steps, got_values = out.scores["compute_steps"], out.scores["exit_values"]
+    margins = []
+    for t, per_seq in enumerate(rec["exit_values"]):
+        for b, vals in enumerate(per_seq):
+            assert len(got_values[t][b]) == len(vals), (t, b, got_values[t][b], vals)
+            for a, v in zip(got_values[t][b], vals):
+                assert abs(a - v) <= 5e-5 + 2e-3 * abs(v), (criterion, t, b, a, v)
+                if criterion not in ("none", "argmax-stability"):
+                    margins.append(abs(v - threshold))
+    if margins:
+        assert min(margins) > 1e-4, f"an exit value sits within 1e-4 of the threshold ({min(margins):.2e}): pick another seed"
+    assert got_steps == want_steps, (criterion, got_steps, want_steps)
+    assert torch.equal(out.sequences.cpu(), want_ids)
+    if criterion not in ("none",):
+        flat = [k for per_tok in want_steps for k in per_tok]
+        assert min(flat) < 8, f"{criterion}: no early exit happened in this case, the test exercises nothing"
+    # the cache holds what the oracle's holds: positions present per step, and the same keys
+    ref_cache = rec["cache"]
+    for step in ref_cache.key_cache:
+        assert sorted(out.past_key_values.key_cache[step].keys()) == sorted(ref_cache.key_cache[step].keys()), step
+
+
+def test_adaptive_compute_options(pkg, small242):
+    """min_steps, checks every second step, no exit in prefill, warm-started states, a lookup strategy that skips
+    missing positions, and the dispatcher."""
+    s, w, model = small242
+    base = dict(criterion="kl", exit_threshold=4e-3, num_steps=8)
+    for extra in (dict(min_steps=3), dict(check_criterion_every_n_steps=2), dict(do_not_exit_in_prefill=True),
+                  dict(continuous_compute=True), dict(cache_lookup_strategy="skip"), dict(cache_lookup_strategy="always-last-m4"),
+                  dict(min_steps=2, check_criterion_every_n_steps=3, continuous_compute=True, cache_lookup_strategy="latest-m4")):
+        kw = {**base, **extra}
+        want_ids, want_steps, rec, out = _adaptive_case(pkg, small242, 2, 4, 5, kw, kw, seed=33)
+        assert out.scores["compute_steps"] == want_steps, (extra, out.scores["compute_steps"], want_steps)
+        assert torch.equal(out.sequences.cpu(), want_ids), extra
+    g = torch.Generator().manual_seed(4)
+    ids = torch.randint(0, s.vocab_size, (1, 4), generator=g)
+    sf = lambda c, sh: O.initialize_state(torch.empty(sh), s, 1.0, torch.Generator().manual_seed(c))
+    gc = pkg.GenerationSettings(max_new_tokens=3)
+    a = model.generate(ids.cuda(), gc, criterion="argmax-stability", exit_threshold=2, num_steps=6, input_states_fn=sf, stop_tokens=set())
+    b, _ = O.generate_with_adaptive_compute(w, s, ids, 3, criterion="argmax-stability", exit_threshold=2, num_steps=6, state_fn=sf)
+    assert torch.equal(a.cpu(), b)
+    # a plug-in evaluator with a fixed schedule; stop tokens end a sequence
+    sched = [3, 1, 4, 2]
+    ev = pkg.NumStepsGenerator(lambda i: sched[i])
+    out = model.generate_with_adaptive_compute(ids.cuda(), pkg.GenerationSettings(max_new_tokens=4, return_dict_in_generate=True),
+                                               exit_evaluator=ev, num_steps=4, input_states_fn=sf, stop_tokens=set())
+    want, steps = O.generate_with_adaptive_compute(w, s, ids, 4, num_steps=4, state_fn=sf,
+                                                   evaluator=O.ExitCriterion("num-steps", steps_fn=lambda i: sched[i]))
+    assert out.scores["compute_steps"] == steps == [[k] for k in sched] and torch.equal(out.sequences.cpu(), want)
+    free = model.generate_with_adaptive_compute(ids.cuda(), pkg.GenerationSettings(max_new_tokens=4), criterion="none",
+                                                num_steps=2, input_states_fn=sf, stop_tokens=set())
+    first = int(free[0, 4])
+    stopped = model.generate_with_adaptive_compute(ids.cuda(), pkg.GenerationSettings(max_new_tokens=4), criterion="none",
+                                                   num_steps=2, input_states_fn=sf, stop_tokens={first})
+    assert stopped.shape[1] == 5 and int(stopped[0, 4]) == first
+    with pytest.raises(ValueError, match="Invalid adaptive compute strategy"):
+        model.generate(ids.cuda(), gc, criterion="no-such-criterion")
+    with pytest.raises(NotImplementedError):
+        pkg.EntropyDiffExitEvaluator(reduce=False)
+
+
+def test_forward_with_adaptive_compute_token_by_token(pkg, small242):
+    s, w, model = small242
+    g = torch.Generator().manual_seed(9)
+    ids = torch.randint(0, s.vocab_size, (1, 6), generator=g)
+    sf = lambda c, sh: O.initialize_state(torch.empty(sh), s, 1.0, torch.Generator().manual_seed(70 + c))
+    sched = [2, 4, 1, 3, 4, 2]
+    want, _, steps = O.prefill_with_varied_exit_steps(w, s, ids, O.ExitCriterion("num-steps", steps_fn=lambda i: sched[i]), state_fn=sf)
+    out = model.forward_with_adaptive_compute(ids.cuda(), pkg.NumStepsGenerator(lambda i: sched[i]), input_states_fn=sf,
+                                              labels=ids)
+    assert out.stats["compute_steps"] == steps == sched
+    check(out.logits, want, torch.float32, "token-by-token logits")
+    ce = torch.nn.functional.cross_entropy(want.view(-1, want.shape[-1]), ids.view(-1))
+    assert abs(float(out.loss) - float(ce)) < 1e-3
+    ev = pkg.KLExitEvaluator(model, 4e-3)
+    want, _, steps = O.prefill_with_varied_exit_steps(w, s, ids, O.ExitCriterion("kl", 4e-3, s.vocab_size), state_fn=sf)
+    got, cache, got_steps = model._prefill_with_varied_exit_steps(ids.cuda(), ev, input_states_fn=sf)
+    assert got_steps == steps
+    check(got, want, torch.float32, "kl exits, token by token")
 
 
 def test_piecewise_surface_equals_forward(tiny32):

@@ -424,3 +424,131 @@ def test_make_weights_layout_and_determinism():
     assert abs(w["transformer.ln_f.weight"].mean().item() - 1.0) < 0.01
     n_params = sum(math.prod(sh) for _, sh in O.state_dict_layout(O.RavenShape.nebel()))
     assert n_params == 3_564_976_800 + 0  # tied head counted once
+
+
+# ----------------------------------------------------------------------------- adaptive compute
+def _fake_predict(logits):
+    return lambda lat: O.OracleOutput(logits=logits.unsqueeze(1), latent_states=lat)
+
+
+def test_exit_entropy_closed_forms():
+    V = 1000
+    ev = O.ExitCriterion("entropy-diff", "auto", V)
+    ev.init(torch.zeros(2, 1, 4))
+    logits = torch.zeros(2, V)
+    logits[1, 7] = 200.0                                   # one-hot: entropy 0; uniform: log V
+    exits, out, v = ev.check(torch.zeros(2, 1, 4), _fake_predict(logits))
+    assert out is not None and not exits.any()
+    assert torch.allclose(ev.prev, torch.tensor([math.log(V), 0.0]), atol=2e-4)
+    assert torch.allclose(v, torch.tensor([100 - math.log(V), 100.0]), atol=2e-4)   # |entropy - 100| on the first check
+    exits, _, v = ev.check(torch.zeros(2, 1, 4), _fake_predict(logits))             # unchanged distribution: difference 0
+    assert exits.all() and float(v.abs().max()) == 0.0
+    p = torch.tensor([0.5, 0.25, 0.25])                    # entropy 1.5 ln 2
+    ev3 = O.ExitCriterion("entropy-diff", 0.5, 3)
+    ev3.init(torch.zeros(1, 1, 4))
+    ev3.check(torch.zeros(1, 1, 4), _fake_predict(p.log().unsqueeze(0)))
+    assert abs(float(ev3.prev) - 1.5 * math.log(2)) < 1e-6
+
+
+def test_exit_kl_closed_forms_and_direction():
+    V = 4
+    ev = O.ExitCriterion("kl", "auto", V)
+    ev.init(torch.zeros(1, 1, 2))
+    q = torch.tensor([[0.7, 0.1, 0.1, 0.1]])
+    _, _, v = ev.check(torch.zeros(1, 1, 2), _fake_predict(q.log()))
+    want = sum(0.25 * (math.log(0.25) - math.log(x)) for x in q[0].tolist())       # KL(previous || current), previous uniform
+    assert abs(float(v) - want) < 1e-6
+    r = torch.tensor([[0.4, 0.3, 0.2, 0.1]])
+    _, _, v = ev.check(torch.zeros(1, 1, 2), _fake_predict(r.log() + 3.0))         # shift invariance of log_softmax
+    want = sum(a * (math.log(a) - math.log(b)) for a, b in zip(q[0].tolist(), r[0].tolist()))
+    wrong = sum(b * (math.log(b) - math.log(a)) for a, b in zip(q[0].tolist(), r[0].tolist()))
+    assert abs(float(v) - want) < 1e-6 and abs(want - wrong) > 1e-2                # not the reverse direction
+    exits, _, v = ev.check(torch.zeros(1, 1, 2), _fake_predict(r.log()))
+    assert abs(float(v)) < 1e-7 and exits.all()
+    assert O.ExitCriterion("some-kl-name", "auto", V).kind == "kl" and O.ExitCriterion("minp-kl", "auto", V).kind == "minp-kl"
+    with pytest.raises(ValueError):
+        O.ExitCriterion("nonsense")
+
+
+def test_exit_minp_kl_by_hand():
+    V = 4
+    ev = O.ExitCriterion("minp-kl", "auto", V)
+    ev.init(torch.zeros(1, 1, 2))
+    p = torch.tensor([[0.6, 0.3, 0.05, 0.05]])             # below 0.1 * 0.6: floored to 1/V, then renormalised
+    _, _, v = ev.check(torch.zeros(1, 1, 2), _fake_predict(p.log()))
+    filt = [0.6 / 1.4, 0.3 / 1.4, 0.25 / 1.4, 0.25 / 1.4]
+    assert torch.allclose(ev.prev.exp(), torch.tensor([filt]), atol=1e-6)
+    want = sum(0.25 * (math.log(0.25) - math.log(x)) for x in filt)
+    assert abs(float(v) - want) < 1e-6
+    assert ev.threshold == 1e-5 and O.ExitCriterion("kl", "auto", V).threshold == 1e-3
+
+
+def test_exit_latent_criteria_closed_forms():
+    prev = torch.tensor([[[3.0, 4.0, 0.0, 0.0], [1.0, 0.0, 0.0, 0.0]]])            # [1, 2, 4]
+    ev = O.ExitCriterion("latent-diff", 0.6)
+    ev.init(prev)
+    _, out, v = ev.check(2 * prev, None)                   # |2x - x| / |2x| = 1/2 at both positions
+    assert out is None and abs(float(v) - 0.5) < 1e-7
+    cur = torch.tensor([[[6.0, 8.0, 0.0, 0.0], [2.0, 0.0, 2.0, 0.0]]])
+    _, _, v = ev.check(cur, None)                          # position 0: 10/10... |cur - 2 prev| = 0 -> 0; position 1: 2 / sqrt 8
+    assert abs(float(v) - (0.0 + 2 / math.sqrt(8)) / 2) < 1e-6
+    ec = O.ExitCriterion("cosine", "auto")
+    ec.init(prev)
+    exits, _, v = ec.check(torch.tensor([[[-4.0, 3.0, 0.0, 0.0], [5.0, 0.0, 0.0, 0.0]]]), None)
+    assert abs(float(v) - 0.5) < 1e-6 and not exits.any()  # orthogonal and parallel: mean cosine 1/2
+    assert ec.threshold == 1e-3 and ev.threshold == 0.6 and O.ExitCriterion("latent-diff").threshold == 0.03
+
+
+def test_exit_argmax_stability_and_num_steps_counting():
+    ev = O.ExitCriterion("argmax-stability", 2, 5)
+    ev.init(torch.zeros(1, 1, 2))
+    streaks = []
+    for tok in (3, 3, 1, 1, 1, 1):
+        logits = torch.zeros(1, 5)
+        logits[0, tok] = 1.0
+        exits, _, v = ev.check(torch.zeros(1, 1, 2), _fake_predict(logits))
+        streaks.append((int(v), bool(exits)))
+    assert streaks == [(0, False), (1, False), (0, False), (1, False), (2, True), (3, True)]
+    assert O.ExitCriterion("argmax-stability", "auto", 5).threshold == 5
+    ns = O.ExitCriterion("num-steps", steps_fn=lambda i: [2, 1][i])
+    ns.init(torch.zeros(3, 1, 2))
+    assert not ns.check(torch.zeros(3, 1, 2), None)[0].any() and ns.check(torch.zeros(3, 1, 2), None)[0].all()
+    ns.init(torch.zeros(3, 1, 2))
+    assert ns.check(torch.zeros(3, 1, 2), None)[0].all()
+
+
+def test_adaptive_pieces_compose_to_forward_and_greedy():
+    s = O.RavenShape.tiny()
+    w = O.make_weights(s, seed=0, dtype=torch.float32)
+    g = torch.Generator().manual_seed(3)
+    ids = torch.randint(0, s.vocab_size, (2, 6), generator=g)
+    states = O.initialize_state(torch.empty(2, 6, s.n_embd), s, 1.0, g)
+    want = O.forward(w, s, input_ids=ids, input_states=states, num_steps=3)
+    embeds, b = O.embed_inputs(w, s, ids)
+    x = states
+    for _ in range(3):
+        x, b = O.iterate_one_step(w, s, embeds, x, b)
+    assert b == s.n_layers_in_prelude - 1 + 3 * s.n_layers_in_recurrent_block
+    got = O.predict_from_latents(w, s, x)
+    assert torch.equal(got.logits, want.logits)            # ln_f is applied inside predict_from_latents (RMM:886)
+    sf = lambda c, sh: O.initialize_state(torch.empty(sh), s, 1.0, torch.Generator().manual_seed(50 + c))
+    a = O.greedy_generate(w, s, ids, 5, state_fn=sf)
+    b_ids, steps = O.generate_with_adaptive_compute(w, s, ids, 5, criterion="none", state_fn=sf)
+    assert torch.equal(a, b_ids) and steps == [[s.mean_recurrence] * 2] * 5
+    # a fixed schedule of recurrences per token equals forward(num_steps=k) token by token on a shared cache
+    sched = [3, 1, 4, 2]
+    c_ids, steps = O.generate_with_adaptive_compute(w, s, ids, 4, num_steps=4, state_fn=sf,
+                                                    evaluator=O.ExitCriterion("num-steps", steps_fn=lambda i: sched[i]))
+    assert steps == [[k, k] for k in sched]
+    cache, cur = O.DictCache(), ids.clone()
+    for call, k in enumerate(sched):
+        seen = cache.get_seq_length()
+        pos = torch.arange(seen, cur.shape[1])
+        out = O.forward(w, s, input_ids=cur[:, pos], input_states=sf(call, (2, len(pos), s.n_embd)), num_steps=k,
+                        past_key_values=cache, use_cache=True, cache_position=pos)
+        cur = torch.cat([cur, out.logits[:, -1].argmax(-1, keepdim=True)], dim=-1)
+    assert torch.equal(cur, c_ids)
+    # token-by-token prefill with exits: same schedule, logits of each token equal the forward's
+    ev = O.ExitCriterion("num-steps", steps_fn=lambda i: sched[i % 4])
+    logits, _, st = O.prefill_with_varied_exit_steps(w, s, ids[:1, :4], ev, state_fn=sf)
+    assert st == sched and logits.shape == (1, 4, s.vocab_size)
