@@ -679,6 +679,102 @@ def prefill_with_varied_exit_steps(w, s: RavenShape, input_ids: torch.Tensor, ev
     return torch.cat(rows, dim=1), cache, steps
 
 
+def generate_speculative(w, s: RavenShape, input_ids: torch.Tensor, max_new_tokens: int, draft_steps: int, lookahead_for_draft: int,
+                         num_steps: int, verification_threshold=1, state_fn=None, init_scale: float = 1.0,
+                         continuous_compute=False, cache_lookup_strategy="full", stop_tokens=(), pad_id: int = 65509,
+                         record: Optional[dict] = None):
+    """Greedy generate_speculative, RMM:1750-1927: draft `lookahead_for_draft` tokens with `draft_steps` recurrences,
+    drop them from the cache, verify all of them in one forward with `num_steps` recurrences, keep each sequence's
+    agreeing prefix plus the verifier's own token at the first disagreement.  `state_fn(call, shape)` supplies the
+    initial latent state of the call-th forward (prefill, drafts and verifications counted in order)."""
+    assert lookahead_for_draft > 0
+    L = lookahead_for_draft
+    cache = DictCache(cache_lookup_strategy)
+    ids = input_ids.clone()
+    B = ids.shape[0]
+    calls = [0]
+
+    def run(tokens, pos, steps, carried):
+        st = carried if carried is not None else (None if state_fn is None else state_fn(calls[0], (B, tokens.shape[1], s.n_embd)))
+        calls[0] += 1
+        return forward(w, s, input_ids=tokens, input_states=st, num_steps=steps, past_key_values=cache, use_cache=True,
+                       cache_position=pos, init_scale=init_scale)
+
+    carried = None
+    if continuous_compute:                                              # RMM:1781-1783
+        carried = state_fn(-1, (B, ids.shape[1], s.n_embd)) if state_fn is not None else \
+            initialize_state(torch.empty(B, ids.shape[1], s.n_embd), s, init_scale)
+    unfinished = torch.ones(B, dtype=torch.bool)
+    generated = 0
+    pos = torch.arange(0, ids.shape[1])
+    out = run(ids, pos, num_steps, carried)                              # prefill with the full number of steps
+    ids = torch.cat([ids, out.logits[:, -1, :].argmax(-1, keepdim=True)], dim=-1)
+    generated += 1
+    cache_position = torch.tensor([cache.get_seq_length()])
+    if continuous_compute:
+        carried = out.latent_states[:, -1:, :]
+    prefix_len = ids.shape[1]
+    accepted = []
+    while generated < max_new_tokens:
+        drafted = ids.clone()
+        current_len = ids.shape[1]
+        for _ in range(L):                                               # RMM:1809-1817
+            out = run(drafted[:, cache_position], cache_position, draft_steps, carried)
+            drafted = torch.cat([drafted, out.logits[:, -1, :].argmax(-1, keepdim=True)], dim=-1)
+            cache_position = cache_position[-1:] + 1
+            if continuous_compute:
+                carried = out.latent_states[:, -1:, :]
+        cache.clear_last_k_entries(L)
+        cache_position = torch.arange(current_len - 1, current_len + L - 1)
+        out = run(drafted[:, cache_position], cache_position, num_steps, carried)
+        preds = out.logits.argmax(dim=-1)
+        if verification_threshold >= 1:
+            mismatched = preds[:, -L:] != drafted[:, current_len:]
+            not_all, first_mismatch = torch.max(mismatched, dim=1)
+        else:
+            probs = F.softmax(out.logits[:, -L:, :], dim=-1)
+            drafted_p = torch.gather(probs, -1, drafted[:, current_len:].unsqueeze(-1)).squeeze(-1)
+            passed = drafted_p >= verification_threshold * probs.max(dim=-1)[0]
+            not_all, first_mismatch = torch.max(~passed, dim=1)
+        accept = torch.where(not_all, first_mismatch, L)
+        per_seq = []
+        for i in range(B):
+            a = int(accept[i])
+            if not_all[i] and a < L:
+                final = out.logits[i:i + 1, a, :].argmax(-1, keepdim=True)
+                part = drafted[i:i + 1, current_len:current_len + a]
+                per_seq.append(torch.cat([part, final], dim=-1) if a > 0 else final)
+            else:
+                per_seq.append(drafted[i:i + 1, current_len:current_len + a])
+        if not_all.any():
+            cache.clear_last_k_entries(L - int(first_mismatch.min()) - 1)
+        counts = [t.shape[1] for t in per_seq]
+        width = max(counts)
+        rows = [torch.cat([t, pad_id * torch.ones((1, width - t.shape[1]), dtype=t.dtype)], dim=-1) if t.shape[1] < width else t
+                for t in per_seq]
+        ids = torch.cat([ids, torch.cat(rows, dim=0)], dim=-1)
+        accepted.append(counts)
+        generated += width
+        cache_position = torch.tensor([cache.get_seq_length()])
+        if continuous_compute:
+            carried = out.latent_states[:, -1:, :]
+        for i in range(B):
+            if unfinished[i] and any(int(t) in stop_tokens for t in per_seq[i].flatten()):
+                unfinished[i] = False
+        if not unfinished.any():
+            break
+    for i in range(B):                                                   # RMM:1903-1912: cut after the first stop token
+        hits = [j for j, t in enumerate(ids[i, prefix_len:].tolist()) if t in stop_tokens]
+        if hits:
+            ids[i, prefix_len + hits[0] + 1:] = pad_id
+    real = (ids != pad_id).any(dim=0).nonzero()
+    if len(real) > 0:
+        ids = ids[:, :int(real[-1]) + 1]
+    if record is not None:
+        record["accepted"], record["cache"], record["forwards"] = accepted, cache, calls[0]
+    return ids
+
+
 # --------------------------------------------------------------------------------------
 # closed-form accounting used as known-answer tests and by the roofline arithmetic
 # --------------------------------------------------------------------------------------

@@ -603,12 +603,14 @@ class RavenForCausalLM(torch.nn.Module):
     @torch.no_grad()
     def generate(self, input_ids: torch.Tensor, generation_config=None, **kwargs):
         """Dispatcher of RMM:1112-1127: `criterion` / `exit_threshold` / `exit_evaluator` select the adaptive-compute
-        loop; the speculative and diffusion-style loops of the reference are not part of this package; everything else
-        goes to generate_minimal (the reference hands those calls to transformers' GenerationMixin)."""
+        loop, `draft_steps` / `lookahead_for_draft` / `verification_threshold` the self-speculative one; the
+        diffusion-style loop of the reference is not part of this package; everything else goes to generate_minimal
+        (the reference hands those calls to transformers' GenerationMixin)."""
         if any(k in kwargs for k in ("criterion", "exit_threshold", "exit_evaluator")):
             return self.generate_with_adaptive_compute(input_ids, generation_config, **kwargs)
-        for k in ("draft_steps", "lookahead_for_draft", "verification_threshold", "headway", "state_noise_mixing",
-                  "inner_recurrence", "freeze_strategy"):
+        if any(k in kwargs for k in ("draft_steps", "lookahead_for_draft", "verification_threshold")):
+            return self.generate_speculative(input_ids, generation_config, **kwargs)
+        for k in ("headway", "state_noise_mixing", "inner_recurrence", "freeze_strategy"):
             if k in kwargs:
                 raise NotImplementedError(f"generate(..., {k}=...) selects a sampler this package does not provide")
         return self.generate_minimal(input_ids, generation_config, **kwargs)
@@ -617,6 +619,11 @@ class RavenForCausalLM(torch.nn.Module):
         """RMM:1552-1749; see adaptive.generate_with_adaptive_compute."""
         from . import adaptive
         return adaptive.generate_with_adaptive_compute(self, input_ids, generation_config, **kwargs)
+
+    def generate_speculative(self, input_ids: torch.Tensor, generation_config=None, **kwargs):
+        """RMM:1750-1927; see speculative.generate_speculative."""
+        from . import speculative
+        return speculative.generate_speculative(self, input_ids, generation_config, **kwargs)
 
     def forward_with_adaptive_compute(self, input_ids: torch.Tensor, exit_evaluator, **kwargs):
         """RMM:998-1035; see adaptive.forward_with_adaptive_compute."""

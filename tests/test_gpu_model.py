@@ -156,7 +156,7 @@ def test_generate_options(pkg, tiny32):
     assert torch.equal(c1, c2) and c1.shape == (2, 11)
     assert model.generate(prompt, max_length=9, stop_tokens=set()).shape == (2, 9)
     with pytest.raises(NotImplementedError):
-        model.generate(prompt, draft_steps=4)       # the speculative sampler is not part of the package
+        model.generate(prompt, headway=2)           # the diffusion-style sampler is not part of the package
     # the reference's preallocated cache class works as past_key_values too
     static = pkg.HuginnStaticCache(max_length=32, max_num_steps=4 + 4 * 4, num_heads=s.n_heads, hidden_dim=s.head_dim, batch_size=2,
                                    device="cuda", dtype=torch.float32)
@@ -345,6 +345,37 @@ def test_forward_with_adaptive_compute_token_by_token(pkg, small242):
     got, cache, got_steps = model._prefill_with_varied_exit_steps(ids.cuda(), ev, input_states_fn=sf)
     assert got_steps == steps
     check(got, want, torch.float32, "kl exits, token by token")
+
+
+@pytest.mark.parametrize("B,draft_steps,L,vt", [(1, 1, 3, 1), (1, 2, 4, 1), (2, 4, 3, 1), (1, 4, 3, 1), (1, 2, 3, 0.5)])
+def test_generate_speculative_matches_oracle(pkg, small242, B, draft_steps, L, vt):
+    """Self-speculative decoding: drafts with few recurrences, rollback, one verifying chunk with all of them.
+    Same sequences and the same accepted counts per round as the oracle's restatement of the loop; for one
+    sequence with zero initial states it also equals plain greedy decoding (what speculation must preserve).
+    Batches are covered where all sequences accept the same number of tokens: once they differ, the reference feeds
+    RoPE positions that no longer equal the cache positions, which this package's forward refuses."""
+    s, w, model = small242
+    g = torch.Generator().manual_seed(40 + B)
+    ids = torch.randint(0, s.vocab_size, (B, 5), generator=g)
+    sf = lambda c, sh: O.initialize_state(torch.empty(sh), s, 1.0, torch.Generator().manual_seed(500 + c))
+    if B > 1:   # zero states and a draft as deep as the verifier: every token is accepted, the batch stays in step
+        sf = lambda c, sh: torch.zeros(sh)
+    rec = {}
+    want = O.generate_speculative(w, s, ids, 9, draft_steps=draft_steps, lookahead_for_draft=L, num_steps=4,
+                                  verification_threshold=vt, state_fn=sf, record=rec, pad_id=s.vocab_size - 1)
+    gc = pkg.GenerationSettings(max_new_tokens=9, return_dict_in_generate=True)
+    out = model.generate(ids.cuda(), gc, draft_steps=draft_steps, lookahead_for_draft=L, num_steps=4, verification_threshold=vt,
+                         input_states_fn=sf, stop_tokens=set(), pad_id=s.vocab_size - 1)
+    assert out.scores["accepted_tokens"] == rec["accepted"], (out.scores["accepted_tokens"], rec["accepted"])
+    assert torch.equal(out.sequences.cpu(), want)
+    assert out.past_key_values.get_seq_length() == rec["cache"].get_seq_length()
+    if B == 1:
+        plain = model.generate_minimal(ids.cuda(), pkg.GenerationSettings(max_new_tokens=9), num_steps=4, init_scale=0.0,
+                                       stop_tokens=set(), use_graph=False)
+        spec = model.generate_speculative(ids.cuda(), pkg.GenerationSettings(max_new_tokens=9), draft_steps=draft_steps,
+                                          lookahead_for_draft=L, num_steps=4, init_scale=0.0, stop_tokens=set())
+        n = min(plain.shape[1], spec.shape[1])
+        assert n >= 5 + 9 and torch.equal(plain[:, :n], spec[:, :n])
 
 
 def test_piecewise_surface_equals_forward(tiny32):

@@ -552,3 +552,24 @@ def test_adaptive_pieces_compose_to_forward_and_greedy():
     ev = O.ExitCriterion("num-steps", steps_fn=lambda i: sched[i % 4])
     logits, _, st = O.prefill_with_varied_exit_steps(w, s, ids[:1, :4], ev, state_fn=sf)
     assert st == sched and logits.shape == (1, 4, s.vocab_size)
+
+
+def test_speculative_decoding_preserves_greedy_output():
+    """With deterministic (zero) initial states, drafting and verifying must reproduce plain greedy decoding, whatever
+    the draft depth and the look-ahead; with the draft as deep as the verifier every drafted token is accepted."""
+    s = O.RavenShape.tiny()
+    w = O.make_weights(s, seed=0, dtype=torch.float32)
+    ids = torch.randint(0, s.vocab_size, (1, 6), generator=torch.Generator().manual_seed(2))
+    plain = O.greedy_generate(w, s, ids, 12, num_steps=4)
+    for draft_steps, look in ((4, 3), (1, 3), (2, 4)):
+        rec = {}
+        spec = O.generate_speculative(w, s, ids, 12, draft_steps=draft_steps, lookahead_for_draft=look, num_steps=4,
+                                      init_scale=0.0, record=rec)
+        n = min(plain.shape[1], spec.shape[1])
+        assert n >= 6 + 12 and torch.equal(plain[:, :n], spec[:, :n])
+        if draft_steps == 4:
+            assert all(c == [look] for c in rec["accepted"])
+        assert rec["cache"].get_seq_length() == spec.shape[1] - 1       # exactly one token is still unseen by the cache
+    stop = int(plain[0, 8])
+    cut = O.generate_speculative(w, s, ids, 12, draft_steps=1, lookahead_for_draft=3, num_steps=4, init_scale=0.0, stop_tokens=(stop,))
+    assert int(cut[0, -1]) == stop and torch.equal(cut[0], plain[0, :cut.shape[1]])
