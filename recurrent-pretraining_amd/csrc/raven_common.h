@@ -34,6 +34,14 @@ __device__ __forceinline__ Chunk<T> load_chunk(const T* p) {
     *reinterpret_cast<uint4*>(&c) = *reinterpret_cast<const uint4*>(p);
     return c;
 }
+// for data that is read once per launch: a load hinted to stream past the caches
+template <typename T>
+__device__ __forceinline__ Chunk<T> load_chunk_stream(const T* p) {
+    typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+    Chunk<T> c;
+    *reinterpret_cast<u32x4_t*>(&c) = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+    return c;
+}
 template <typename T>
 __device__ __forceinline__ void store_chunk(T* p, const Chunk<T>& c) {
     *reinterpret_cast<uint4*>(p) = *reinterpret_cast<const uint4*>(&c);
