@@ -48,6 +48,7 @@ struct Tuning {
     int gemv_interleave = 1;
     int gemv_nontemporal = 1;
     int gemv_wgs_per_cu = 4;
+    int gemm_four_tiles = 1;
 };
 static Tuning g_tuning;
 
@@ -193,11 +194,17 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemmArgs a) {
 // (at the next line boundary); the `shift` elements before them and whatever is left behind the last full
 // macro-step are single 32-wide MFMA steps straight from global memory (first and last wave).
 // ------------------------------------------------------------------------------------------------
-constexpr int kPitch = 136;  // bf16 elements per LDS row: 128 + 8 (272 bytes)
-
-template <int MT, int NT, int EPI>
+// KM = k-values per macro-step: 128, or 64 for the variants with four weight tiles per workgroup (the same
+// bytes per macro-step; a quarter-wave then reads two rows of 128 bytes).  LDS rows are KM + 8 elements long
+// (272 or 144 bytes: both spread 16 rows over the 64 banks without conflicts for 16-byte reads).
+template <int MT, int NT, int EPI, int KM = 128>
 __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
     constexpr int ROWS = 16 * (NT + MT);
+    constexpr int kPitch = KM + 8;
+    constexpr int LPR = KM / 8;        // lanes per row of a macro-step
+    constexpr int RPI = 64 / LPR;      // rows per load instruction
+    constexpr int IPT = 16 / RPI;      // load instructions per 16-row tile
+    constexpr int NG = EPI == EPI_SWIGLU ? NT / 2 : NT;  // tiles side by side along N (SwiGLU: NG gate tiles + their NG up tiles)
     __shared__ __align__(16) bf16 stage[4][ROWS][kPitch];
     static_assert(sizeof(bf16) * 4 * ROWS * kPitch >= sizeof(float) * 3 * NT * MT * 64 * 4, "stage doubles as the reduction buffer");
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -215,9 +222,10 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         if (EPI == EPI_SWIGLU) {
-            tile_out0[t] = group * 16 * rs + parity;
-            tile_row0[t] = tile_out0[t] + t * a.N;  // t = 0 gate tile, t = 1 up tile
-            tile_ok[t] = true;
+            const int first = (group * NG + t % NG) * 16 * rs;
+            tile_ok[t] = first < a.N;
+            tile_out0[t] = (tile_ok[t] ? first : group * NG * 16 * rs) + parity;
+            tile_row0[t] = tile_out0[t] + (t / NG) * a.N;  // the first NG tiles are gate tiles, the others their up tiles
         } else {
             const int first = (group * NT + t) * 16 * rs;
             tile_ok[t] = first < a.N;
@@ -234,11 +242,11 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
 
     typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
     struct Staged {
-        u32x4 w[NT][4];
-        u32x4 x[MT][4];
+        u32x4 w[NT][IPT];
+        u32x4 x[MT][IPT];
     };
     bf16(*my)[kPitch] = stage[wave];
-    const int lr = lane >> 4, lc = (lane & 15) * 8;  // loader role: row within a group of 4, first element of the chunk
+    const int lr = lane / LPR, lc = (lane % LPR) * 8;  // loader role: row within a group of RPI, first element of the chunk
 
     // X is given as up to two K segments (the adapter's concat); each is walked on its own
 #pragma unroll 1
@@ -258,37 +266,37 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
                 if ((int)(reinterpret_cast<uintptr_t>(W + (int64_t)tile_row0[t] * K + wk0) & 127) != mis) shift = 0;
             if (shift > seg_len) shift = 0;
         }
-        const int n_macro = (seg_len - shift) / 128;
+        const int n_macro = (seg_len - shift) / KM;
         const int mb = (int)((int64_t)n_macro * wave / 4), me = (int)((int64_t)n_macro * (wave + 1) / 4);
 
         auto fetch = [&](int mac, Staged& st) {  // global -> registers, row-contiguous lanes
-            const int k = shift + mac * 128 + lc;
+            const int k = shift + mac * KM + lc;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int m = min(mt * 16 + 4 * i + lr, a.M - 1);  // rows past M repeat the last one; never stored
+                for (int i = 0; i < IPT; ++i) {
+                    const int m = min(mt * 16 + RPI * i + lr, a.M - 1);  // rows past M repeat the last one; never stored
                     st.x[mt][i] = *reinterpret_cast<const u32x4*>(X + (int64_t)m * ldx + k);
                 }
 #pragma unroll
             for (int t = 0; t < NT; ++t)
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    st.w[t][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(W + (int64_t)(tile_row0[t] + (4 * i + lr) * rs) * K + wk0 + k));
+                for (int i = 0; i < IPT; ++i)
+                    st.w[t][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(W + (int64_t)(tile_row0[t] + (RPI * i + lr) * rs) * K + wk0 + k));
         };
         auto park = [&](const Staged& st) {  // registers -> this wave's LDS tile
 #pragma unroll
             for (int t = 0; t < NT; ++t)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&my[t * 16 + 4 * i + lr][lc]) = st.w[t][i];
+                for (int i = 0; i < IPT; ++i) *reinterpret_cast<u32x4*>(&my[t * 16 + RPI * i + lr][lc]) = st.w[t][i];
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&my[(NT + mt) * 16 + 4 * i + lr][lc]) = st.x[mt][i];
+                for (int i = 0; i < IPT; ++i) *reinterpret_cast<u32x4*>(&my[(NT + mt) * 16 + RPI * i + lr][lc]) = st.x[mt][i];
         };
         auto multiply = [&]() {  // LDS -> MFMA fragments
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < KM / 32; ++j) {
                 bf16x8 bv[MT];
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)  // same access type as the stores in park(): the two must stay ordered
@@ -321,7 +329,7 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
         }
         // 32-element steps in front of the first and behind the last macro-step: first and last wave, straight from global memory
         if (wave == 0 || wave == 3) {
-            const int kb = wave == 0 ? 0 : shift + n_macro * 128, ke = wave == 0 ? shift : seg_len;
+            const int kb = wave == 0 ? 0 : shift + n_macro * KM, ke = wave == 0 ? shift : seg_len;
             for (int k = kb; k < ke; k += 32) {
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
@@ -364,9 +372,13 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
         if (m >= a.M) continue;
         if (EPI == EPI_SWIGLU) {
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int n = tile_out0[0] + (kq * 4 + v) * rs;
-                static_cast<bf16*>(a.y)[(int64_t)m * a.N + n] = from_f32<bf16>(swiglu<bf16>(acc[0][mt][v], acc[NT - 1][mt][v]));
+            for (int g = 0; g < NG; ++g) {
+                if (!tile_ok[g]) continue;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int n = tile_out0[g] + (kq * 4 + v) * rs;
+                    static_cast<bf16*>(a.y)[(int64_t)m * a.N + n] = from_f32<bf16>(swiglu<bf16>(acc[g][mt][v], acc[NG + g][mt][v]));
+                }
             }
         } else {
 #pragma unroll
@@ -442,17 +454,32 @@ static int dispatch_mfma(GemmArgs a, hipStream_t s) {
     const int pitch = a.K * 2;
     a.row_stride = (pitch % 128 == 64 && a.N % 32 == 0) ? 2 : 1;
     a.line_aligned = (pitch * a.row_stride) % 128 == 0;
-    if (EPI == EPI_SWIGLU) {
-        if (a.M <= 16)
+    const int rs = a.row_stride;
+    // Four tiles per workgroup (64-wide K steps) halve the X re-reads per weight byte: 5.0 -> 5.7 TB/s in steady state
+    // at 32 rows.  Their workgroups are twice as long, so the gain only survives where the grid is balanced: at most
+    // one workgroup per CU (Wqkv: 248), or so many that the last round does not matter.  Tuning key gemm_four_tiles:
+    // 0 never, 1 by this rule, 2 whenever the shape allows.
+    const int groups4 = (n_tiles16 + 4 * rs - 1) / (4 * rs) * rs;       // plain epilogue: 4 tiles side by side
+    const int groups2 = (n_tiles16 + 2 * rs - 1) / (2 * rs) * rs;       // SwiGLU with 4 tiles: 2 gate + 2 up
+    const int g4 = EPI == EPI_SWIGLU ? groups2 : groups4;
+    const bool four = g_tuning.gemm_four_tiles == 2 ||
+                      (g_tuning.gemm_four_tiles == 1 && a.M > 16 && g4 >= n_cus() / 2 && (g4 <= n_cus() || g4 >= 8 * n_cus()));
+    if constexpr (EPI == EPI_SWIGLU) {
+        if (four) {
+            if (a.M <= 16) mfma_kernel<1, 4, EPI, 64><<<dim3(groups2), dim3(256), 0, s>>>(a);
+            else           mfma_kernel<2, 4, EPI, 64><<<dim3(groups2), dim3(256), 0, s>>>(a);
+        } else if (a.M <= 16)
             mfma_kernel<1, 2, EPI><<<dim3(n_tiles16), dim3(256), 0, s>>>(a);
         else
             mfma_kernel<2, 2, EPI><<<dim3(n_tiles16), dim3(256), 0, s>>>(a);
+    } else if (four) {
+        if (a.M <= 16) mfma_kernel<1, 4, EPI, 64><<<dim3(groups4), dim3(256), 0, s>>>(a);
+        else           mfma_kernel<2, 4, EPI, 64><<<dim3(groups4), dim3(256), 0, s>>>(a);
     } else {
         // two tiles per workgroup (X is then re-read from L2 once per two tiles) while that still leaves every
         // CU more than one workgroup; L2 -> L1 traffic, not HBM, is what limits this kernel
         const bool two = n_tiles16 / 2 >= n_cus() + n_cus() / 2;
-        const int rs = a.row_stride;  // units come in groups of rs, a group covers rs * (two ? 2 : 1) tiles
-        const int units = two ? (n_tiles16 + 2 * rs - 1) / (2 * rs) * rs : n_tiles16;
+        const int units = two ? groups2 : n_tiles16;
         if (a.M <= 16) {
             if (two) mfma_kernel<1, 2, EPI><<<dim3(units), dim3(256), 0, s>>>(a);
             else     mfma_kernel<1, 1, EPI><<<dim3(units), dim3(256), 0, s>>>(a);
@@ -522,6 +549,7 @@ extern "C" int raven_set_tuning(const char* key, int32_t value) {
     else if (k == "gemv_nontemporal") g_tuning.gemv_nontemporal = value;
     else if (k == "gemv_wgs_per_cu") g_tuning.gemv_wgs_per_cu = value;
     else if (k == "linear_ks") g_linear_ks = value;
+    else if (k == "gemm_four_tiles") g_tuning.gemm_four_tiles = value;
     else RAVEN_REQUIRE(set_gemv1_tuning(key, value) == 0, "set_tuning: unknown key %s", key);
     return 0;
 }

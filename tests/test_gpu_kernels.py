@@ -183,12 +183,14 @@ def test_linear_small_and_odd_shapes(pkg):
 
 
 @pytest.mark.parametrize("M", [6, 20])
-def test_mfma_gemm_row_alignment_cases(pkg, M):
+@pytest.mark.parametrize("four", [1, 2])
+def test_mfma_gemm_row_alignment_cases(pkg, M, four):
     """Row pitches that are odd multiples of 64 bytes (tiles of one row parity, macro-steps shifted to the line
     boundary), with and without whole tile pairs, a second operand that starts mid-line, and a weight matrix
     whose base address is not line-aligned; both MFMA kernels (with and without a workspace)."""
     dt = torch.bfloat16
     ws = pkg.hip.linear_workspace(M, 4096, "cuda")
+    pkg.hip.set_tuning("gemm_four_tiles", four)  # 2: the four-tile, 64-wide-step variant wherever there is no workspace
     pkg.hip.set_tuning("linear_ks", 2)  # with a workspace: the split-K kernel
     for N, K in ((32, 96), (64, 288), (64, 2336), (96, 416), (48, 416), (160, 1184), (64, 256)):
         x, w = rnd((M, K), dt, 180 + N), rnd((N, K), dt, 181 + K, 0.05)
@@ -211,6 +213,22 @@ def test_mfma_gemm_row_alignment_cases(pkg, M):
             check(pkg.hip.linear(x0.cuda(), w.cuda(), x1=x1.cuda(), workspace=wsp), lin(torch.cat([x0, x1], -1), w).to(dt), dt,
                   f"two operands {M}x{N}x({K0}+{K1})")
     pkg.hip.set_tuning("linear_ks", 0)
+    pkg.hip.set_tuning("gemm_four_tiles", 1)
+
+
+@pytest.mark.parametrize("M", [8, 32])
+def test_mfma_four_tile_variant_nebel_shapes(pkg, M):
+    dt, h, I = torch.bfloat16, 5280, 17920
+    pkg.hip.set_tuning("gemm_four_tiles", 2)
+    x, xi, res = rnd((M, h), dt, 230 + M), rnd((M, I), dt, 231), rnd((M, h), dt, 232)
+    wqkv, fc, mlp = rnd((3 * h, h), dt, 233, 0.02), rnd((2 * I, h), dt, 234, 0.02), rnd((h, I), dt, 235, 0.02)
+    check(pkg.hip.gemm(x.cuda(), wqkv.cuda()), lin(x, wqkv).to(dt), dt, "qkv")
+    z = lin(x, fc).to(dt)
+    check(pkg.hip.gemm_swiglu(x.cuda(), fc.cuda()), F.silu(z[:, :I]) * z[:, I:], dt, "fc + swiglu")
+    check(pkg.hip.gemm(xi.cuda(), mlp.cuda(), residual=res.cuda()), lin(xi, mlp).to(dt) + res, dt, "mlp.proj + residual")
+    yf = pkg.hip.gemm(x.cuda(), wqkv.cuda(), out_f32=True)
+    assert yf.dtype == torch.float32 and torch.equal(yf, pkg.hip.gemm(x.cuda(), wqkv.cuda()).float())
+    pkg.hip.set_tuning("gemm_four_tiles", 1)
 
 
 @pytest.mark.parametrize("dt,h,I", [(torch.bfloat16, 5280, 17920), (torch.float32, 256, 704), (torch.bfloat16, 64, 176)])
