@@ -25,7 +25,7 @@ namespace raven {
 constexpr int kPfKeys = 64;     // keys per tile
 constexpr int kPfRows = 64;     // query rows per workgroup
 constexpr int kPfMaxHd = 128;
-constexpr int kVtPitch = 68;    // bf16 elements per V^T row: 64 + 4 (136 bytes, 8-byte aligned reads)
+constexpr int kVtPitch = 72;    // bf16 elements per V^T row: 64 + 8 (144 bytes: the 8-byte reads of a half-wave hit 32 different bank pairs)
 
 struct PrefillArgs {
     const bf16* q;   // [B*S, h]
@@ -79,19 +79,54 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(PrefillArgs a) {
     const int n_keys = min(pos0 + last_row + 1, a.t_max);
     const int my_limit = pos0 + my_row;  // this lane's query sees keys <= my_limit
 
+    // Global -> registers -> LDS, one tile ahead: the loads of tile kt + 64 are in flight while tile kt is multiplied.
+    // K: 16-byte chunks, row-major.  V: a thread takes the same 8 columns of 4 consecutive keys and writes, per
+    // column, the 4 keys as one 8-byte piece of the transposed tile.
+    constexpr int CPR = HD / 8;                          // chunks per key row
+    constexpr int KCH = (kPfKeys * CPR + 255) / 256;     // K chunks per thread
+    constexpr int VTASKS = (kPfKeys / 4) * CPR;          // V tasks per tile (at most 256)
+    static_assert(VTASKS <= 256, "one V task per thread");
+    u32x4 kreg[KCH];
+    Chunk<bf16> vreg[4];
+    const int v_kg = threadIdx.x % (kPfKeys / 4), v_dc = threadIdx.x / (kPfKeys / 4);
+    auto fetch = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < KCH; ++i) {
+            const int c = threadIdx.x + 256 * i;
+            if (c < kPfKeys * CPR) {
+                const int key = c / CPR, dc = c - key * CPR;
+                const int kpos = min(kt + key, a.t_max - 1);  // rows past n_keys are masked below; stay in bounds
+                kreg[i] = *reinterpret_cast<const u32x4*>(Kb + (int64_t)kpos * HD + dc * 8);
+            }
+        }
+        if (threadIdx.x < VTASKS) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) vreg[i] = load_chunk(Vb + (int64_t)min(kt + 4 * v_kg + i, a.t_max - 1) * HD + v_dc * 8);
+        }
+    };
+    auto park = [&]() {
+#pragma unroll
+        for (int i = 0; i < KCH; ++i) {
+            const int c = threadIdx.x + 256 * i;
+            if (c < kPfKeys * CPR) {
+                const int key = c / CPR, dc = c - key * CPR;
+                *reinterpret_cast<u32x4*>(&sk[key][dc * 8]) = kreg[i];
+            }
+        }
+        if (threadIdx.x < VTASKS) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                bf16 four[4] = {vreg[0].v[e], vreg[1].v[e], vreg[2].v[e], vreg[3].v[e]};
+                typedef unsigned int u32x2s __attribute__((ext_vector_type(2)));
+                *reinterpret_cast<u32x2s*>(&svt[v_dc * 8 + e][4 * v_kg]) = *reinterpret_cast<const u32x2s*>(four);
+            }
+        }
+    };
+    if (n_keys > 0) fetch(0);
     for (int kt = 0; kt < n_keys; kt += kPfKeys) {
         __syncthreads();  // the previous tile has been consumed
-        // stage K (row-major) and V (transposed); 16-byte chunks, 256 threads
-        constexpr int CPR = HD / 8;  // chunks per key row
-        for (int c = threadIdx.x; c < kPfKeys * CPR; c += 256) {
-            const int key = c / CPR, dc = c - key * CPR;
-            const int kpos = min(kt + key, a.t_max - 1);  // rows past n_keys are masked below; stay in bounds
-            const u32x4 kv = *reinterpret_cast<const u32x4*>(Kb + (int64_t)kpos * HD + dc * 8);
-            *reinterpret_cast<u32x4*>(&sk[key][dc * 8]) = kv;
-            Chunk<bf16> vv = load_chunk(Vb + (int64_t)kpos * HD + dc * 8);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) svt[dc * 8 + e][key] = vv.v[e];
-        }
+        park();
+        if (kt + kPfKeys < n_keys) fetch(kt + kPfKeys);
         __syncthreads();
 
         // S^T sub-tiles: sc[t][v] = score of key kt + 16 t + 4 s4 + v against query qc
@@ -105,45 +140,59 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(PrefillArgs a) {
                 sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], sc[t], 0, 0, 0);
             }
         }
-        // scale, causal mask, tile maximum for this query
+        // scale, causal mask (only tiles that reach past the wave's first query need it), tile maximum for this query
         float mx = -INFINITY;
+        if (kt + kPfKeys - 1 <= pos0 + row0) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int key = kt + 16 * t + 4 * s4 + v;
-                float x = sc[t][v] * a.scale_log2;
-                if (key > my_limit) x = -INFINITY;
-                sc[t][v] = x;
-                mx = fmaxf(mx, x);
-            }
+                for (int v = 0; v < 4; ++v) {
+                    sc[t][v] *= a.scale_log2;
+                    mx = fmaxf(mx, sc[t][v]);
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int key = kt + 16 * t + 4 * s4 + v;
+                    float x = sc[t][v] * a.scale_log2;
+                    if (key > my_limit) x = -INFINITY;
+                    sc[t][v] = x;
+                    mx = fmaxf(mx, x);
+                }
+        }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m_run, mx);
-        // a query with no visible key yet (rows past S only) keeps weights of zero
-        const float corr = (m_new == -INFINITY) ? 1.f : exp2f(m_run - m_new);
-        float psum = 0.f;
+        // a query with no visible key yet (rows past S only) has m_new = -inf: subtract 0 instead, every weight is then 0
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        float psum = 0.f;  // over this lane's 16 keys; the four lanes of a query are added up once, after the last tile
         bf16x8 pf[2];
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const float p = (m_new == -INFINITY) ? 0.f : exp2f(sc[t][v] - m_new);
+                const float p = __builtin_amdgcn_exp2f(sc[t][v] - m_use);
                 psum += p;
                 pf[t >> 1][(t & 1) * 4 + v] = static_cast<bf16>(p);
             }
-        psum += __shfl_xor(psum, 16, 64);
-        psum += __shfl_xor(psum, 32, 64);
-        l_run = l_run * corr + psum;
+        // the running maximum of most queries stops moving after a few tiles: rescale only when some lane's did
+        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+            const float corr = __builtin_amdgcn_exp2f(m_run - m_use);  // 0 for the first visible tile (m_run = -inf)
+            l_run = l_run * corr + psum;
+            // O rows are queries 4*s4 + v: fetch their rescale factor from the lane that tracks that query
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const float cv = __shfl(corr, 4 * s4 + v, 64);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) o[nt][v] *= cv;
+            }
+        } else {
+            l_run += psum;
+        }
         m_run = m_new;
 
-        // O rows are queries 4*s4 + v: fetch their rescale factor from the lane that tracks that query
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const float cv = __shfl(corr, 4 * s4 + v, 64);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) o[nt][v] *= cv;
-        }
         // O += P V: k-step c covers sub-tiles (2c, 2c+1); slot (s4, e) is key 16*(2c + e/4) + 4*s4 + e%4
 #pragma unroll
         for (int c = 0; c < 2; ++c)
@@ -159,6 +208,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(PrefillArgs a) {
     }
 
     // normalise and store: O row v of this lane is query 4*s4 + v, column 16*nt + qc
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
         const float lv = __shfl(l_run, 4 * s4 + v, 64);
