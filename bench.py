@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-iters", type=int, default=3)
     ap.add_argument("--also-batch", type=int, default=32, help="second batch size reported under 'also' (0 = skip)")
+    ap.add_argument("--adaptive", action="store_true",
+                    help="per-token adaptive compute at bs=1 with a fixed cycle of recurrences per token (a next-row measurement)")
     ap.add_argument("--prefill", action="store_true",
                     help="measure the recurrent core over a whole prompt instead (bs=4 x 4096 tokens, r iterations): MFMA-bound regime")
     ap.add_argument("--prefill-batch", type=int, default=4)
@@ -96,6 +98,52 @@ def prefill(args):
                    "batch": B, "seq_len": S, "recurrence": r, "gemm": "hipBLASLt via torch.matmul", "attention": "attention_prefill_kernel"},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / MFMA_PEAK_TFLOPS, 4), "flops_per_iteration": gemm_flops + attn_flops, "traffic": None},
+    }
+    print(json.dumps(line))
+
+
+def adaptive(args):
+    """Per-token adaptive compute at bs=1 (next-row measurement, not the headline line): tokens stop after a fixed
+    cycle of 8 / 16 / 32 / 12 recurrences (a NumStepsGenerator, so the work does not depend on what random weights
+    predict), the cache lookup is latest-m4, i.e. deeper tokens read shallower tokens' last recurrence through the
+    attention kernel's steps_present path.  Each recurrence is one eager raven_core_iteration call."""
+    import torch
+    import __graft_entry__ as entry
+    pkg = entry.import_package()
+    pkg.hip.load()
+    dev = torch.device("cuda:0")
+    cfg = pkg.RavenConfig()
+    model = pkg.RavenForCausalLM(cfg, device=dev, dtype=torch.bfloat16)
+    fill_synthetic(model, 0)
+    sched = [8, 16, 32, 12]
+    n_new = args.steps
+    ids = torch.randint(0, cfg.vocab_size, (1, args.prompt), generator=torch.Generator().manual_seed(1)).cuda()
+    gc = pkg.GenerationSettings(max_new_tokens=n_new + 1, return_dict_in_generate=True)
+    ev = pkg.NumStepsGenerator(lambda i: 32 if i == 0 else sched[(i - 1) % len(sched)])
+    # the prompt (token step 0, all 32 recurrences) is part of the call; time it separately and subtract
+    for _ in range(2):  # the first pass warms up (allocations, lazy initialisation)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        model.generate_with_adaptive_compute(ids, pkg.GenerationSettings(max_new_tokens=1, return_dict_in_generate=True),
+                                             exit_evaluator=pkg.NumStepsGenerator(lambda i: 32), num_steps=32,
+                                             cache_lookup_strategy="latest-m4", stop_tokens=set())
+        torch.cuda.synchronize()
+        t_prompt = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    out = model.generate_with_adaptive_compute(ids, gc, exit_evaluator=ev, num_steps=32, cache_lookup_strategy="latest-m4",
+                                               stop_tokens=set())
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0 - t_prompt
+    steps = [s_[0] for s_ in out.scores["compute_steps"]][1:]
+    line = {
+        "metric": "adaptive-compute decode, raven-3.5b shape bf16 bs=1: tokens/s and recurrences/s",
+        "value": round(len(steps) / dt, 3), "unit": "tokens/s", "n_gpus": 1, "steps": len(steps), "warmup": 0,
+        "ms_per_step": round(dt / len(steps) * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"generate_with_adaptive_compute, nebel-raven-3.5b shape, bs=1, {args.prompt}-token prompt, "
+                               f"recurrences per token cycle {sched}, cache lookup latest-m4", "schedule": sched},
+        "recurrences_per_s": round(sum(steps) / dt, 1), "mean_recurrences": round(sum(steps) / len(steps), 2),
+        "ms_per_recurrence_incl_coda_and_head": round(dt / sum(steps) * 1e3, 4), "prompt_s": round(t_prompt, 3),
     }
     print(json.dumps(line))
 
@@ -187,6 +235,9 @@ def main():
         return
     if args.prefill:
         prefill(args)
+        return
+    if args.adaptive:
+        adaptive(args)
         return
     if args.gpus != 1:
         print("bench.py measures one GPU: the decode path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
