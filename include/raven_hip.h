@@ -86,7 +86,8 @@ const char* raven_last_error(void);
 /* Launch-shape overrides for experiments (grid sizing and load hints of the skinny-GEMM kernels);
  * results never depend on them.  Keys: gemv_units_per_wave, gemv_interleave, gemv_nontemporal,
  * gemv_wgs_per_cu, gemv1_pairs_norm, gemv1_pairs_plain, gemm_four_tiles (0 / 1 / 2 = never / by rule / always use
- * the four-tile MFMA variant), linear_ks (K slices of the split-K kernel behind raven_linear;
+ * the four-tile MFMA variant), attn_split_target / attn_big_grid (workgroups a split decode-attention launch aims
+ * for / from which its 2-positions-per-row variant is used), linear_ks (K slices of the split-K kernel behind raven_linear;
  * non-zero also makes raven_linear use that kernel for every shape it accepts).  Not needed in normal use: the
  * defaults are the tuned values. */
 int raven_set_tuning(const char* key, int32_t value);

@@ -293,12 +293,14 @@ __global__ __launch_bounds__(128) void attention_combine_kernel(const float* __r
 }
 
 constexpr int kAttnMaxSplits = 32;
+int g_attn_split_target = 2048;  // workgroups a split launch aims for (raven_set_tuning "attn_split_target")
+int g_attn_big_grid = 1280;      // workgroups from which the 2-positions-per-row variant is used ("attn_big_grid")
 
 // Splits are worth their extra launch only while heads x rows cannot fill the chip.
 static int splits_for(int M, int nh, int len_hint) {
     if ((int64_t)M * nh >= 512) return 1;
     int ns = (len_hint + 63) / 64;  // 64 positions per workgroup keeps every load in one round trip
-    const int cap = (2048 + M * nh - 1) / (M * nh);
+    const int cap = (g_attn_split_target + M * nh - 1) / (M * nh);
     if (ns > cap) ns = cap;
     if (ns > kAttnMaxSplits) ns = kAttnMaxSplits;
     return ns < 1 ? 1 : ns;
@@ -363,7 +365,6 @@ extern "C" int raven_qkv_bias_rope_cache_append(const void* qkv, const void* qk_
     return raven_host::check_launch("qkv_append");
 }
 
-static int g_attn_big_grid = 1280;  // workgroups from which the 2-positions-per-row variant is used
 
 template <typename T>
 static void launch_attention(bool fused, const void* q, const void* bias, const float* freqs, void* y, const raven::CacheView& cv,

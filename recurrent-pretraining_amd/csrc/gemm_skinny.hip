@@ -25,6 +25,7 @@ namespace raven {
 
 int set_gemv1_tuning(const char* key, int value);
 extern int g_linear_ks;
+extern int g_attn_split_target, g_attn_big_grid;
 
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
 
@@ -550,6 +551,8 @@ extern "C" int raven_set_tuning(const char* key, int32_t value) {
     else if (k == "gemv_wgs_per_cu") g_tuning.gemv_wgs_per_cu = value;
     else if (k == "linear_ks") g_linear_ks = value;
     else if (k == "gemm_four_tiles") g_tuning.gemm_four_tiles = value;
+    else if (k == "attn_split_target" && value > 0) g_attn_split_target = value;
+    else if (k == "attn_big_grid" && value > 0) g_attn_big_grid = value;
     else RAVEN_REQUIRE(set_gemv1_tuning(key, value) == 0, "set_tuning: unknown key %s", key);
     return 0;
 }
