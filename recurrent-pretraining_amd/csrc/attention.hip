@@ -118,6 +118,39 @@ __device__ __forceinline__ Chunk<T> bias_rope_chunk(Chunk<T> x, const T* __restr
     return x;
 }
 
+// What one lane holds of a position's head row: CPL neighbouring 16-byte chunks (1, or 2 for fp32 heads wider than
+// 64 elements, whose rows are more than 16 chunks long).
+template <typename T, int CPL>
+struct Piece {
+    Chunk<T> c[CPL];
+};
+template <typename T, int CPL, bool STREAM = false>
+__device__ __forceinline__ Piece<T, CPL> load_piece(const T* p) {
+    Piece<T, CPL> r;
+#pragma unroll
+    for (int i = 0; i < CPL; ++i) r.c[i] = STREAM ? load_chunk_stream(p + i * Chunk<T>::N) : load_chunk(p + i * Chunk<T>::N);
+    return r;
+}
+template <typename T, int CPL>
+__device__ __forceinline__ void store_piece(T* p, const Piece<T, CPL>& v) {
+#pragma unroll
+    for (int i = 0; i < CPL; ++i) store_chunk(p + i * Chunk<T>::N, v.c[i]);
+}
+template <typename T, int CPL>
+__device__ __forceinline__ Piece<T, CPL> zero_piece() {
+    Piece<T, CPL> r;
+#pragma unroll
+    for (int i = 0; i < CPL; ++i) r.c[i] = zero_chunk<T>();
+    return r;
+}
+template <typename T, int CPL>
+__device__ __forceinline__ float dot_piece(const Piece<T, CPL>& a, const Piece<T, CPL>& b) {
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < CPL; ++i) acc = dot_chunk(a.c[i], b.c[i], acc);
+    return acc;
+}
+
 // Grid (heads, token rows, splits).  With one split a workgroup owns a whole (head, row) and writes y.
 // With several (few heads x rows, i.e. small batches: one CU cannot pull a head's K/V fast enough) each
 // workgroup covers a contiguous range of positions with all of its loads in flight at once and writes
@@ -126,12 +159,13 @@ __device__ __forceinline__ Chunk<T> bias_rope_chunk(Chunk<T> x, const T* __restr
 // position's k and v, come straight from the fused qkv GEMM output -- bias and RoPE are applied here,
 // the new k/v row is written to the cache by the workgroup whose range holds it and used from registers.
 // LOOKUP: some older positions are not cached at this slot (cv.steps_present says which).
-template <typename T, bool FUSED, int kAttnU, bool LOOKUP = false>
+template <typename T, bool FUSED, int kAttnU, bool LOOKUP = false, int CPL = 1>
 __global__ __launch_bounds__(256) void decode_attention_kernel(
     const T* __restrict__ q_or_qkv, const T* __restrict__ qk_bias, const float* __restrict__ freqs, T* __restrict__ y,
     CacheView cv, int S, int pos0, const int* __restrict__ pos_dev, float scale_log2, int n_splits,
     float* __restrict__ ws_ml, float* __restrict__ ws_o) {
-    constexpr int E = Chunk<T>::N;
+    constexpr int EC = Chunk<T>::N;   // elements per 16-byte chunk
+    constexpr int E = EC * CPL;       // elements per lane and position
     constexpr int G = 16;      // 16-lane rows in the workgroup
     // kAttnU = positions per 16-lane row and loop iteration: 4 when a few workgroups must each keep many loads
     // in flight, 2 when the grid is large and register pressure decides how many workgroups a CU holds
@@ -158,20 +192,21 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
     const T* Vb = static_cast<const T*>(cv.v) + head_off + ci * E;
 
     // q (and the new k, v) first: these loads are the oldest, so their data is back before the K/V tiles
-    Chunk<T> qraw = zero_chunk<T>(), kraw = zero_chunk<T>(), vnew = zero_chunk<T>();
+    typedef Piece<T, CPL> P;
+    P qraw = zero_piece<T, CPL>(), kraw = zero_piece<T, CPL>(), vnew = zero_piece<T, CPL>();
     const int col = head * hd + ci * E;
     if (active) {
         if (FUSED) {
             const T* row = q_or_qkv + (int64_t)m * 3 * h;
-            qraw = load_chunk(row + col);
-            kraw = load_chunk(row + h + col);
-            vnew = load_chunk(row + 2 * h + col);
+            qraw = load_piece<T, CPL>(row + col);
+            kraw = load_piece<T, CPL>(row + h + col);
+            vnew = load_piece<T, CPL>(row + 2 * h + col);
         } else {
-            qraw = load_chunk(q_or_qkv + (int64_t)m * h + col);
+            qraw = load_piece<T, CPL>(q_or_qkv + (int64_t)m * h + col);
         }
     }
     // first K/V tile, requested before q is touched
-    Chunk<T> kc[kAttnU], vc[kAttnU];
+    P kc[kAttnU], vc[kAttnU];
     bool left_out[kAttnU];  // LOOKUP: the position takes no part
     auto load_tile = [&](int base) {
 #pragma unroll
@@ -179,26 +214,29 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
             const int p = base + j * G + group;
             int64_t delta = 0;
             left_out[j] = false;
-            if (LOOKUP && p < end && p < first_new) left_out[j] = !lookup_source(cv, p, &delta);
+            if (LOOKUP && cv.steps_present != nullptr && p < end && p < first_new) left_out[j] = !lookup_source(cv, p, &delta);
             if (active && p < end && !(FUSED && p == pos) && !left_out[j]) {
                 // large grids (the 2-position variant) stream K/V past the caches: +8 % at batch 32; small ones do not gain
-                kc[j] = kAttnU == 2 ? load_chunk_stream(Kb + delta + (int64_t)p * hd) : load_chunk(Kb + delta + (int64_t)p * hd);
-                vc[j] = kAttnU == 2 ? load_chunk_stream(Vb + delta + (int64_t)p * hd) : load_chunk(Vb + delta + (int64_t)p * hd);
+                kc[j] = load_piece<T, CPL, kAttnU == 2>(Kb + delta + (int64_t)p * hd);
+                vc[j] = load_piece<T, CPL, kAttnU == 2>(Vb + delta + (int64_t)p * hd);
             } else {
-                kc[j] = zero_chunk<T>();
-                vc[j] = zero_chunk<T>();
+                kc[j] = zero_piece<T, CPL>();
+                vc[j] = zero_piece<T, CPL>();
             }
         }
     };
     load_tile(start);
 
-    Chunk<T> qc = qraw, knew = kraw;
+    P qc = qraw, knew = kraw;
     if (FUSED && active) {
-        qc = bias_rope_chunk<T>(qraw, qk_bias, 0, h, col, freqs, pos, hd, ci * E);
-        knew = bias_rope_chunk<T>(kraw, qk_bias, 1, h, col, freqs, pos, hd, ci * E);
+#pragma unroll
+        for (int i = 0; i < CPL; ++i) {
+            qc.c[i] = bias_rope_chunk<T>(qraw.c[i], qk_bias, 0, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
+            knew.c[i] = bias_rope_chunk<T>(kraw.c[i], qk_bias, 1, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
+        }
         if (group == 0 && pos >= start && pos < end) {
-            store_chunk(static_cast<T*>(cv.k) + head_off + (int64_t)pos * hd + ci * E, knew);
-            store_chunk(static_cast<T*>(cv.v) + head_off + (int64_t)pos * hd + ci * E, vnew);
+            store_piece<T, CPL>(static_cast<T*>(cv.k) + head_off + (int64_t)pos * hd + ci * E, knew);
+            store_piece<T, CPL>(static_cast<T*>(cv.v) + head_off + (int64_t)pos * hd + ci * E, vnew);
         }
     }
 
@@ -216,7 +254,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
                 kc[j] = knew;
                 vc[j] = vnew;
             }
-            sc[j] = row16_sum(dot_chunk(qc, kc[j], 0.f)) * scale_log2;
+            sc[j] = row16_sum(dot_piece<T, CPL>(qc, kc[j])) * scale_log2;
             if (p >= end || (LOOKUP && left_out[j])) sc[j] = -INFINITY;
             m_new = fmaxf(m_new, sc[j]);
         }
@@ -233,7 +271,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
         for (int e = 0; e < E; ++e) {
             float acc = o[e] * corr;
 #pragma unroll
-            for (int j = 0; j < kAttnU; ++j) acc = __builtin_fmaf(pe[j], to_f32(vc[j].v[e]), acc);
+            for (int j = 0; j < kAttnU; ++j) acc = __builtin_fmaf(pe[j], to_f32(vc[j].c[e / EC].v[e % EC]), acc);
             o[e] = acc;
         }
         m_run = m_new;
@@ -337,7 +375,8 @@ static int check_heads(const char* who, int nh, int hd, int dtype) {
     RAVEN_REQUIRE(dtype == RAVEN_F32 || dtype == RAVEN_BF16, "%s: unknown dtype %d", who, dtype);
     const int elts = 16 / (int)raven_host::elt_size(dtype);
     RAVEN_REQUIRE(nh > 0 && hd > 0 && hd % elts == 0 && hd % 2 == 0, "%s: head_dim %d must be an even multiple of %d", who, hd, elts);
-    RAVEN_REQUIRE(hd / elts <= 16 && hd <= kAttnMaxHd, "%s: head_dim %d too large for one 16-lane row", who, hd);
+    RAVEN_REQUIRE(hd / elts <= 32 && hd <= kAttnMaxHd, "%s: head_dim %d too large for one 16-lane row", who, hd);
+    RAVEN_REQUIRE(hd / elts <= 16 || hd % (2 * elts) == 0, "%s: head_dim %d must be a multiple of %d", who, hd, 2 * elts);
     return 0;
 }
 
@@ -377,7 +416,12 @@ static void launch_attention(bool fused, const void* q, const void* bias, const 
 #define RAVEN_ATTN_LAUNCH(FUSED_, U_, LOOKUP_)                                                                            \
     decode_attention_kernel<T, FUSED_, U_, LOOKUP_><<<grid, dim3(256), 0, s>>>((const T*)q, FUSED_ ? bias_t : nullptr,     \
         FUSED_ ? freqs : nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o)
-    if (cv.steps_present) {  // partial fill: rare, one variant per entry point
+    if (cv.hd / Chunk<T>::N > 16) {  // fp32 heads wider than 64 elements: two chunks per lane, one variant per entry point
+        if constexpr (sizeof(T) == 4) {
+            if (fused) decode_attention_kernel<T, true, 2, true, 2><<<grid, dim3(256), 0, s>>>((const T*)q, bias_t, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
+            else decode_attention_kernel<T, false, 2, true, 2><<<grid, dim3(256), 0, s>>>((const T*)q, nullptr, nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
+        }
+    } else if (cv.steps_present) {  // partial fill: rare, one variant per entry point
         if (fused) RAVEN_ATTN_LAUNCH(true, 2, true);
         else RAVEN_ATTN_LAUNCH(false, 2, true);
     } else if (fused) {

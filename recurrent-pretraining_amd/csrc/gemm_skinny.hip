@@ -513,8 +513,13 @@ static int run_gemm(GemmArgs a, int dtype, hipStream_t s) {
         }
         const bool use_mfma = mfma_ok && left > 4;
         if (use_mfma) pass = left < 32 ? left : 32;
-        else if (dtype == RAVEN_BF16) pass = left < 4 ? left : 4;
-        else pass = left < 8 ? left : 8;
+        else {
+            pass = dtype == RAVEN_BF16 ? (left < 4 ? left : 4) : (left < 8 ? left : 8);
+            // the vector kernel keeps its X rows in LDS: as many rows per pass (1, 2, 4 or 8) as fit
+            const size_t row_bytes = (size_t)a.K * es;
+            RAVEN_REQUIRE(row_bytes <= 160 * 1024, "gemm: one row of K=%d elements does not fit the 160 KB LDS", a.K);
+            while (pass > 1 && (size_t)(pass <= 2 ? 2 : pass <= 4 ? 4 : 8) * row_bytes > 160 * 1024) pass = pass > 4 ? 4 : pass > 2 ? 2 : 1;
+        }
         GemmArgs p = a;
         p.M = pass;
         p.x0 = static_cast<const char*>(a.x0) + (size_t)m0 * a.k0 * es;

@@ -9,7 +9,7 @@
 namespace raven {
 
 constexpr int kNormThreads = 256;
-constexpr int kNormMaxChunks = 4;  // per thread: dim <= 256 * 4 * (16 / sizeof(T)) elements
+constexpr int kNormMaxChunks = 16;  // per thread, in the largest variant: dim <= 256 * 16 * (16 / sizeof(T)) elements
 
 __device__ __forceinline__ float block_sum_256(float v, float* red) {
     v = wave_sum(v);
@@ -20,7 +20,8 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
     return red[0] + red[1] + red[2] + red[3];
 }
 
-template <typename T>
+// MC = 16-byte chunks a thread keeps of its row (4 covers 5280 bf16 elements; fp32 rows of that length need 8)
+template <typename T, int MC>
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
     const T* __restrict__ x, const T* __restrict__ residual, const T* __restrict__ weight, T* __restrict__ y,
     T* __restrict__ sum_out, const T* __restrict__ weight2, T* __restrict__ y2, int dim, float eps) {
@@ -31,10 +32,10 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
     const T* xr = x + row * dim;
     const T* rr = residual ? residual + row * dim : nullptr;
 
-    float v[kNormMaxChunks][E];
+    float v[MC][E];
     float ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < kNormMaxChunks; ++i) {
+    for (int i = 0; i < MC; ++i) {
         const int c = threadIdx.x + i * kNormThreads;
         if (c < n_chunks) {
             Chunk<T> cx = load_chunk(xr + c * E);
@@ -55,7 +56,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
 
     float ss2 = 0.f;
 #pragma unroll
-    for (int i = 0; i < kNormMaxChunks; ++i) {
+    for (int i = 0; i < MC; ++i) {
         const int c = threadIdx.x + i * kNormThreads;
         if (c < n_chunks) {
             Chunk<T> cw = load_chunk(weight + c * E);
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
 
     inv = rsqrtf(block_sum_256(ss2, red) / (float)dim + eps);
 #pragma unroll
-    for (int i = 0; i < kNormMaxChunks; ++i) {
+    for (int i = 0; i < MC; ++i) {
         const int c = threadIdx.x + i * kNormThreads;
         if (c < n_chunks) {
             Chunk<T> cw = load_chunk(weight2 + c * E);
@@ -102,14 +103,19 @@ extern "C" int raven_rmsnorm_residual(const void* x, const void* residual, const
                   kNormThreads * kNormMaxChunks * elts);
     RAVEN_REQUIRE(rows > 0 && rows < (1ll << 31), "rmsnorm: bad row count %lld", (long long)rows);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const int per_thread = (dim / elts + kNormThreads - 1) / kNormThreads;
+#define RAVEN_NORM_LAUNCH(T_, MC_)                                                                                       \
+    rmsnorm_kernel<T_, MC_><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                                          \
+        (const T_*)x, (const T_*)residual, (const T_*)weight, (T_*)y, (T_*)sum_out, (const T_*)weight2, (T_*)y2, dim, eps)
     if (dtype == RAVEN_BF16) {
-        rmsnorm_kernel<bf16><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(
-            (const bf16*)x, (const bf16*)residual, (const bf16*)weight, (bf16*)y, (bf16*)sum_out, (const bf16*)weight2,
-            (bf16*)y2, dim, eps);
+        if (per_thread <= 4) RAVEN_NORM_LAUNCH(bf16, 4);
+        else if (per_thread <= 8) RAVEN_NORM_LAUNCH(bf16, 8);
+        else RAVEN_NORM_LAUNCH(bf16, 16);
     } else {
-        rmsnorm_kernel<float><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(
-            (const float*)x, (const float*)residual, (const float*)weight, (float*)y, (float*)sum_out,
-            (const float*)weight2, (float*)y2, dim, eps);
+        if (per_thread <= 4) RAVEN_NORM_LAUNCH(float, 4);
+        else if (per_thread <= 8) RAVEN_NORM_LAUNCH(float, 8);
+        else RAVEN_NORM_LAUNCH(float, 16);
     }
+#undef RAVEN_NORM_LAUNCH
     return raven_host::check_launch("rmsnorm");
 }

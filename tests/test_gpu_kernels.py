@@ -567,3 +567,38 @@ def test_exit_latent_stats(pkg, dt):
     y[1, 1] = 2.0
     rel, cos = pkg.hip.exit_latent_stats(x.cuda(), y.cuda(), want_rel=True, want_cos=True)
     assert abs(float(rel[0]) - 0.5) < 1e-6 and abs(float(cos[0]) - 1.0) < 1e-2 and float(cos[1]) == 0.0
+
+
+# ----------------------------------------------------------------------------- fp32 at the 3.5b shape
+def test_fp32_kernels_at_the_3_5b_shape(pkg):
+    """The reference runs in fp32 at any shape; the fp32 variants here need more registers / LDS per row at h = 5280,
+    hd = 96, I = 17920: rows of 1320 chunks for the norm, 24 chunks per head row (two per lane) for attention, X rows
+    of up to 71680 bytes in the vector GEMM's LDS."""
+    dt, h, nh, hd, I = torch.float32, 5280, 55, 96, 17920
+    x, res, w = rnd((3, h), dt, 400), rnd((3, h), dt, 401), 1 + rnd((h,), dt, 402, 0.02)
+    y, _, _ = pkg.hip.rmsnorm_residual(x.cuda(), w.cuda(), 1e-6, residual=res.cuda())
+    check(y, O.rmsnorm(x + res, w, 1e-6), dt, "rmsnorm fp32 5280")
+    for M in (1, 3, 8):
+        xi, wm = rnd((M, I), dt, 403 + M), rnd((256, I), dt, 404, 0.02)
+        check(pkg.hip.gemm(xi.cuda(), wm.cuda()), lin(xi, wm), dt, f"fp32 gemm K=17920 M={M}")
+        xa, wa = rnd((M, 2 * h), dt, 405 + M), rnd((128, 2 * h), dt, 406, 0.02)
+        check(pkg.hip.gemm(xa.cuda(), wa.cuda()), lin(xa, wa), dt, f"fp32 gemm K=10560 M={M}")
+    # attention: decode step (fused and two-step), a chunk of rows, with and without the split over positions
+    t_max, B = 300, 2
+    k, v, kd, vd, cache = make_cache(pkg, 2, B, nh, t_max, hd, dt, fill_seed=410)
+    ws = pkg.hip.attention_workspace(B * 3, nh, hd, "cuda")
+    for S, pos0 in ((1, 200), (3, 100), (1, 0)):
+        q = rnd((B * S, nh * hd), dt, 412 + S)
+        T = pos0 + S
+        want = O.sdpa(q.view(B, S, nh, hd).transpose(1, 2), k[1, :, :, :T], v[1, :, :, :T]).transpose(1, 2).reshape(B * S, nh * hd)
+        check(pkg.hip.decode_attention(q.cuda(), cache, 1, B, S, pos0, nh, hd, workspace=ws), want, dt, f"fp32 hd=96 attention S={S}")
+        check(pkg.hip.decode_attention(q.cuda(), cache, 1, B, S, pos0, nh, hd), want, dt, f"fp32 hd=96 attention S={S}, no split")
+    qkv, bias = rnd((B, 3 * nh * hd), dt, 420), rnd((2, 1, nh, hd), dt, 421, 0.5)
+    table = O.rope_table(hd, t_max, 50000.0)
+    freqs = table.reshape(t_max, hd // 2, 2).contiguous().cuda()
+    k2, v2, kd2, vd2, cache2 = make_cache(pkg, 2, B, nh, t_max, hd, dt, fill_seed=410)
+    y_f = pkg.hip.qkv_attention_decode(qkv.cuda(), bias.cuda(), freqs, cache, 1, B, 150, nh, hd, workspace=ws)
+    q2 = pkg.hip.qkv_bias_rope_cache_append(qkv.cuda(), bias.cuda(), freqs, cache2, 1, B, 1, 150, nh, hd)
+    y_2 = pkg.hip.decode_attention(q2, cache2, 1, B, 1, 150, nh, hd, workspace=ws)
+    assert torch.equal(kd, kd2) and torch.equal(vd, vd2)
+    check(y_f, y_2.cpu(), dt, "fp32 hd=96 fused decode step")
