@@ -231,6 +231,17 @@ int raven_core_iteration(const raven_dims* dims, const void* adapter_w,
                          int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
                          void* workspace, size_t workspace_bytes, void* stream);
 
+/* n_iterations recurrences in a row (the loop of iterate_forward, RMM:751-761): iteration i reads and appends to the
+ * cache slots slots[i * n_blocks + j], j = 0 .. n_blocks - 1 (a host array, read before the call returns).  The same
+ * results as n_iterations calls of raven_core_iteration with ln_f on the last one; for one token row the closing
+ * norm_4 of an iteration runs as the prologue of the next adapter product instead of a launch of its own.
+ * state_out may not alias state_in or embeds. */
+int raven_core_iterations(const raven_dims* dims, const void* adapter_w, const raven_block_weights* blocks,
+                          int32_t n_blocks, const void* ln_f, const void* state_in, const void* embeds,
+                          void* state_out, const float* freqs, const raven_kv_cache* cache, const int32_t* slots,
+                          int32_t n_iterations, int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -162,44 +162,75 @@ extern "C" int raven_sandwich_block(const raven_dims* dims, const raven_block_we
     return run_block(dims, w, s, false, x_in, x_out, nullptr, nullptr, freqs, cache, slot, B, S, pos0, pos_dev, stream);
 }
 
+extern "C" int raven_core_iterations(const raven_dims* dims, const void* adapter_w, const raven_block_weights* blocks,
+                                     int32_t n_blocks, const void* ln_f, const void* state_in, const void* embeds,
+                                     void* state_out, const float* freqs, const raven_kv_cache* cache, const int32_t* slots,
+                                     int32_t n_iterations, int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace raven;
+    if (int rc = check_dims("core_iterations", dims)) return rc;
+    RAVEN_REQUIRE(adapter_w && state_in && embeds && state_out && freqs && slots, "core_iterations: null pointer");
+    RAVEN_REQUIRE(n_blocks >= 1 && blocks, "core_iterations: needs at least one block");
+    RAVEN_REQUIRE(n_iterations >= 1, "core_iterations: needs at least one iteration (got %d)", n_iterations);
+    RAVEN_REQUIRE(B > 0 && S > 0, "core_iterations: bad B=%d S=%d", B, S);
+    for (int j = 0; j < n_blocks; ++j)
+        if (int rc = check_block_weights("core_iterations", &blocks[j])) return rc;
+    const int M = B * S, h = dims->n_embd;
+    const size_t need = carve(dims, M, nullptr, nullptr);
+    RAVEN_REQUIRE(workspace && workspace_bytes >= need, "core_iterations: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    RAVEN_REQUIRE(((uintptr_t)workspace & 255) == 0, "core_iterations: workspace must be 256-byte aligned");
+    BlockScratch s;
+    carve(dims, M, static_cast<char*>(workspace), &s);
+    const raven_block_weights& last_blk = blocks[n_blocks - 1];
+
+    int rc;
+    if (M == 1 && one_row_fits(dims)) {
+        // One row: between two iterations the last block's closing norm_4 is the prologue of the next adapter product
+        // (no launch of its own); only the last iteration closes with a norm launch (norm_4, then ln_f if asked for).
+        for (int it = 0; it < n_iterations; ++it) {
+            const int32_t* sl = slots + (size_t)it * n_blocks;
+            if (it == 0)
+                rc = raven_gemv_fused(state_in, embeds, nullptr, nullptr, nullptr, adapter_w, nullptr, s.xa, h, h, h, dims->eps, 0, 0,
+                                      dims->dtype, stream);
+            else
+                rc = raven_gemv_fused(s.x3, embeds, last_blk.norm_4, nullptr, nullptr, adapter_w, nullptr, s.xa, h, h, h, dims->eps, 0, 0,
+                                      dims->dtype, stream);
+            if (rc) return rc;
+            for (int j = 0; j < n_blocks; ++j) {
+                const void* x_raw = j == 0 ? (const void*)s.xa : (const void*)s.x3;
+                const void* pre = j == 0 ? nullptr : blocks[j - 1].norm_4;
+                if ((rc = run_block_one_row(dims, &blocks[j], s, x_raw, pre, freqs, cache, sl[j], pos0, pos_dev, stream))) return rc;
+            }
+        }
+        return close_one_row(dims, s, last_blk.norm_4, ln_f, state_out, stream);
+    }
+    for (int it = 0; it < n_iterations; ++it) {
+        const int32_t* sl = slots + (size_t)it * n_blocks;
+        const bool last_it = it == n_iterations - 1;
+        // the adapter product consumes the state before the last block of this iteration overwrites state_out
+        if ((rc = raven_linear(it == 0 ? state_in : state_out, embeds, adapter_w, nullptr, s.xa, M, h, h, h, 0, 0, dims->dtype, s.lin_ws,
+                               s.lin_ws_bytes, stream))) return rc;
+        const void* lnw = last_it ? ln_f : nullptr;
+        for (int j = 0; j < n_blocks; ++j) {
+            const bool last = j == n_blocks - 1;
+            void* y_out = last ? (lnw ? nullptr : state_out) : s.xa;
+            const void* tail_w = last ? lnw : blocks[j + 1].norm_1;
+            void* tail_out = last ? (lnw ? state_out : nullptr) : s.n1;
+            if ((rc = run_block(dims, &blocks[j], s, j > 0, s.xa, y_out, tail_w, tail_out, freqs, cache, sl[j], B, S, pos0, pos_dev,
+                                stream))) return rc;
+        }
+    }
+    return 0;
+}
+
 extern "C" int raven_core_iteration(const raven_dims* dims, const void* adapter_w, const raven_block_weights* blocks,
                                     int32_t n_blocks, const void* ln_f, const void* state_in, const void* embeds,
                                     void* state_out, const float* freqs, const raven_kv_cache* cache, int32_t first_slot,
                                     int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev, void* workspace,
                                     size_t workspace_bytes, void* stream) {
-    using namespace raven;
-    if (int rc = check_dims("core_iteration", dims)) return rc;
-    RAVEN_REQUIRE(adapter_w && state_in && embeds && state_out && freqs, "core_iteration: null pointer");
-    RAVEN_REQUIRE(n_blocks >= 1 && blocks, "core_iteration: needs at least one block");
-    RAVEN_REQUIRE(B > 0 && S > 0, "core_iteration: bad B=%d S=%d", B, S);
-    for (int j = 0; j < n_blocks; ++j)
-        if (int rc = check_block_weights("core_iteration", &blocks[j])) return rc;
-    const int M = B * S, h = dims->n_embd;
-    const size_t need = carve(dims, M, nullptr, nullptr);
-    RAVEN_REQUIRE(workspace && workspace_bytes >= need, "core_iteration: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-    RAVEN_REQUIRE(((uintptr_t)workspace & 255) == 0, "core_iteration: workspace must be 256-byte aligned");
-    BlockScratch s;
-    carve(dims, M, static_cast<char*>(workspace), &s);
-
-    int rc;
-    if (M == 1 && one_row_fits(dims)) {
-        if ((rc = raven_gemv_fused(state_in, embeds, nullptr, nullptr, nullptr, adapter_w, nullptr, s.xa, h, h, h, dims->eps, 0, 0,
-                                   dims->dtype, stream))) return rc;
-        for (int j = 0; j < n_blocks; ++j) {
-            const void* x_raw = j == 0 ? (const void*)s.xa : (const void*)s.x3;
-            const void* pre = j == 0 ? nullptr : blocks[j - 1].norm_4;
-            if ((rc = run_block_one_row(dims, &blocks[j], s, x_raw, pre, freqs, cache, first_slot + j, pos0, pos_dev, stream))) return rc;
-        }
-        return close_one_row(dims, s, blocks[n_blocks - 1].norm_4, ln_f, state_out, stream);
-    }
-    if ((rc = raven_linear(state_in, embeds, adapter_w, nullptr, s.xa, M, h, h, h, 0, 0, dims->dtype, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
-    for (int j = 0; j < n_blocks; ++j) {
-        const bool last = j == n_blocks - 1;
-        void* y_out = last ? (ln_f ? nullptr : state_out) : s.xa;
-        const void* tail_w = last ? ln_f : blocks[j + 1].norm_1;
-        void* tail_out = last ? (ln_f ? state_out : nullptr) : s.n1;
-        if ((rc = run_block(dims, &blocks[j], s, j > 0, s.xa, y_out, tail_w, tail_out, freqs, cache, first_slot + j, B, S, pos0,
-                            pos_dev, stream))) return rc;
-    }
-    return 0;
+    RAVEN_REQUIRE(n_blocks >= 1 && n_blocks <= 64, "core_iteration: needs 1..64 blocks (got %d)", n_blocks);
+    int32_t slots[64];
+    for (int j = 0; j < n_blocks; ++j) slots[j] = first_slot + j;
+    return raven_core_iterations(dims, adapter_w, blocks, n_blocks, ln_f, state_in, embeds, state_out, freqs, cache, slots, 1, B, S,
+                                 pos0, pos_dev, workspace, workspace_bytes, stream);
 }

@@ -76,6 +76,8 @@ SIGNATURES = {
                                        C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _VP, _SZ, _VP]),
     "raven_core_iteration": (C.c_int, [C.POINTER(Dims), _VP, C.POINTER(BlockWeights), _I32, _VP, _VP, _VP, _VP, _VP,
                                        C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _VP, _SZ, _VP]),
+    "raven_core_iterations": (C.c_int, [C.POINTER(Dims), _VP, C.POINTER(BlockWeights), _I32, _VP, _VP, _VP, _VP, _VP,
+                                        C.POINTER(KVCache), C.POINTER(C.c_int32), _I32, _I32, _I32, _I32, _VP, _VP, _SZ, _VP]),
 }
 
 _lib: Optional[C.CDLL] = None
@@ -371,4 +373,20 @@ def core_iteration(dims: Dims, adapter_w, blocks, state_in, embeds, state_out, f
         _ptr(freqs, "freqs", torch.float32), C.byref(cache), first_slot, B, S, pos0,
         _ptr(pos_dev, "pos_dev", torch.int32), _ptr(workspace, "workspace", torch.uint8), workspace.numel(), _stream())
     _check(rc, "raven_core_iteration")
+    return state_out
+
+
+def core_iterations(dims: Dims, adapter_w, blocks, state_in, embeds, state_out, freqs, cache: KVCache, slots, B, S, pos0,
+                    workspace, ln_f=None, pos_dev=None):
+    """slots: one list of len(blocks) cache slots per recurrence; runs len(slots) recurrences."""
+    flat = [int(v) for it in slots for v in it]
+    if len(flat) != len(slots) * len(blocks):
+        raise RavenHipError("core_iterations: every recurrence needs one slot per block")
+    arr = (C.c_int32 * len(flat))(*flat)
+    rc = load().raven_core_iterations(
+        C.byref(dims), _ptr(adapter_w, "adapter_w", state_in.dtype), blocks, len(blocks), _ptr(ln_f, "ln_f", state_in.dtype),
+        _ptr(state_in, "state_in"), _ptr(embeds, "embeds", state_in.dtype), _ptr(state_out, "state_out", state_in.dtype),
+        _ptr(freqs, "freqs", torch.float32), C.byref(cache), arr, len(slots), B, S, pos0,
+        _ptr(pos_dev, "pos_dev", torch.int32), _ptr(workspace, "workspace", torch.uint8), workspace.numel(), _stream())
+    _check(rc, "raven_core_iterations")
     return state_out

@@ -766,18 +766,13 @@ class DecodeRunner:
                                pos_dev=self.pos)
         x = self.state
         n_core = len(t.core_block)
-        for it, slots in enumerate(core):
-            lnw = t.ln_f.weight if it == self.r - 1 else None
-            if n_core > 0 and all(slots[j] == slots[0] + j for j in range(n_core)):
-                hip.core_iteration(nat["dims"], t.adapter.weight, nat["core"], x, self.embeds, self.x, nat["freqs"], kv, slots[0],
-                                   B, 1, hint, self.ws, ln_f=lnw, pos_dev=self.pos)
-            else:
-                hip_x = hip.adapter_gemm_concat(x, self.embeds, t.adapter.weight)
-                for j in range(n_core):
-                    last = j == n_core - 1
-                    hip.sandwich_block(nat["dims"], nat["core"][j], hip_x, self.x if last else hip_x, nat["freqs"], kv, slots[j],
-                                       B, 1, hint, self.ws, ln_f=lnw if last else None, pos_dev=self.pos)
+        if n_core > 0 and self.r > 0:
+            # all recurrences in one call: for one row the library folds each closing norm into the next adapter product
+            hip.core_iterations(nat["dims"], t.adapter.weight, nat["core"], x, self.embeds, self.x, nat["freqs"], kv, core, B, 1, hint,
+                                self.ws, ln_f=t.ln_f.weight, pos_dev=self.pos)
             x = self.x
+        elif self.r > 0:
+            raise NotImplementedError("the decode runner needs at least one core block; use forward() for such a model")
         if self.r == 0:
             hip.load().raven_rmsnorm_residual(x.data_ptr(), None, t.ln_f.weight.data_ptr(), self.x.data_ptr(), None, None, None,
                                               B, cfg.n_embd, cfg.norm_eps, hip.dtype_code(m.dtype), hip._stream())

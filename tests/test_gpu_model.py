@@ -378,6 +378,37 @@ def test_generate_speculative_matches_oracle(pkg, small242, B, draft_steps, L, v
         assert n >= 5 + 9 and torch.equal(plain[:, :n], spec[:, :n])
 
 
+@pytest.mark.parametrize("dt,B", [(torch.float32, 1), (torch.bfloat16, 1), (torch.bfloat16, 3), (torch.float32, 6)])
+def test_core_iterations_equal_single_iterations(pkg, tiny32, tiny16, dt, B):
+    """raven_core_iterations (all recurrences in one call; for one row the closing norm rides in the next adapter
+    product) gives the bits of the same recurrences called one by one, and leaves the same cache."""
+    s, w, model = tiny32 if dt == torch.float32 else tiny16
+    nat, t = model._natives(), model.transformer
+    n_core, r, T, h = len(t.core_block), 3, 9, s.n_embd
+    g = torch.Generator().manual_seed(60 + B)
+    state = O.initialize_state(torch.empty(B, 1, h), s, 1.0, g).to(dt).view(B, h).cuda()
+    emb = torch.randn(B, h, generator=g).to(dt).cuda()
+    caches = []
+    for _ in range(2):
+        k = rnd((r * n_core, B, s.n_heads, T + 1, s.head_dim), dt, 61).cuda()
+        v = rnd((r * n_core, B, s.n_heads, T + 1, s.head_dim), dt, 62).cuda()
+        caches.append((k, v, pkg.hip.make_cache(k, v)))
+    ws = pkg.hip.block_workspace(nat["dims"], B, "cuda")
+    slots = [[it * n_core + j for j in range(n_core)] for it in range(r)]
+    many = torch.empty_like(state)
+    pkg.hip.core_iterations(nat["dims"], t.adapter.weight, nat["core"], state, emb, many, nat["freqs"], caches[0][2], slots, B, 1, T, ws,
+                            ln_f=t.ln_f.weight)
+    x, one = state, torch.empty_like(state)
+    for it in range(r):
+        pkg.hip.core_iteration(nat["dims"], t.adapter.weight, nat["core"], x, emb, one, nat["freqs"], caches[1][2], slots[it][0], B, 1, T, ws,
+                               ln_f=t.ln_f.weight if it == r - 1 else None)
+        x = one.clone()
+    assert torch.equal(many, one)
+    assert torch.equal(caches[0][0], caches[1][0]) and torch.equal(caches[0][1], caches[1][1])
+    with pytest.raises(pkg.hip.RavenHipError):
+        pkg.hip.core_iterations(nat["dims"], t.adapter.weight, nat["core"], state, emb, many, nat["freqs"], caches[0][2], [[0]], B, 1, T, ws)
+
+
 def test_piecewise_surface_equals_forward(tiny32):
     """embed_inputs -> iterate_one_step x r -> predict_from_latents reproduces forward (RMM:841-934)."""
     s, w, model = tiny32
