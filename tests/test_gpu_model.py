@@ -409,6 +409,34 @@ def test_core_iterations_equal_single_iterations(pkg, tiny32, tiny16, dt, B):
         pkg.hip.core_iterations(nat["dims"], t.adapter.weight, nat["core"], state, emb, many, nat["freqs"], caches[0][2], [[0]], B, 1, T, ws)
 
 
+def test_committed_fixture_without_the_oracle(pkg, tiny32):
+    """tests/golden/tiny_fp32_oracle.json (stored oracle outputs): logits, greedy, adaptive and speculative token streams
+    from the HIP path against the stored values; the oracle only supplies the seeded weights and latent states."""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "tiny_fp32_oracle.json")) as f:
+        fx = json.load(f)
+    s, w, model = tiny32
+    ids = torch.tensor(fx["prompt"])
+    states = O.initialize_state(torch.empty(2, 6, s.n_embd), s, 1.0, torch.Generator().manual_seed(12))
+    out = model(input_ids=ids.cuda(), input_states=states.cuda())
+    assert torch.allclose(out.logits[:, -1, :8].cpu(), torch.tensor(fx["forward_last_logits_first8"]), atol=2e-4)
+    assert out.logits[:, -1].argmax(-1).tolist() == fx["forward_last_argmax"]
+    assert torch.allclose(out.latent_states[:, -1].norm(dim=-1).cpu(), torch.tensor(fx["forward_latent_l2"]), rtol=1e-4)
+    sf = lambda call, shape: O.initialize_state(torch.empty(shape), s, 1.0, torch.Generator().manual_seed(7000 + call))
+    gc = pkg.GenerationSettings(max_new_tokens=16)
+    got = model.generate_minimal(ids.cuda(), gc, input_states_fn=sf, stop_tokens=set())
+    assert got[:, 6:].tolist() == fx["greedy_16_tokens"]
+    ad = model.generate_with_adaptive_compute(ids.cuda(), pkg.GenerationSettings(max_new_tokens=6, return_dict_in_generate=True),
+                                              criterion="kl", exit_threshold=5e-3, num_steps=8, input_states_fn=sf,
+                                              cache_lookup_strategy="latest-m4", stop_tokens=set())
+    assert ad.sequences[:, 6:].tolist() == fx["adaptive_kl_5e-3_tokens"]
+    assert ad.scores["compute_steps"] == fx["adaptive_kl_5e-3_compute_steps"]
+    spec = model.generate_speculative(ids[:1].cuda(), pkg.GenerationSettings(max_new_tokens=10), draft_steps=1, lookahead_for_draft=3,
+                                      num_steps=4, init_scale=0.0, stop_tokens=set())
+    assert spec[:, 6:].tolist() == fx["speculative_draft1_look3_tokens"]
+
+
 def test_piecewise_surface_equals_forward(tiny32):
     """embed_inputs -> iterate_one_step x r -> predict_from_latents reproduces forward (RMM:841-934)."""
     s, w, model = tiny32

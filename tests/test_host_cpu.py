@@ -193,3 +193,52 @@ def test_cache_lookup_errors(pkg):
         c3.update(k, k, step)
     with pytest.raises(ValueError, match="Unknown lookup strategy"):
         c3.update(k, k, 6)
+
+
+# ----------------------------------------------------------------------------- committed fixtures (tests/golden)
+def _golden(name):
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name)) as f:
+        return json.load(f)
+
+
+def test_oracle_reproduces_the_committed_fixture():
+    """tests/golden/tiny_fp32_oracle.json was written by tests/golden/make_fixtures.py: a change of the oracle's
+    arithmetic, of its seeded draws or of its generate loops shows up here."""
+    fx = _golden("tiny_fp32_oracle.json")
+    s = O.RavenShape.tiny()
+    w = O.make_weights(s, seed=0, dtype=torch.float32)
+    ids = torch.tensor(fx["prompt"])
+    states = O.initialize_state(torch.empty(2, 6, s.n_embd), s, 1.0, torch.Generator().manual_seed(12))
+    out = O.forward(w, s, input_ids=ids, input_states=states)
+    assert torch.allclose(out.logits[:, -1, :8], torch.tensor(fx["forward_last_logits_first8"]), atol=2e-5)
+    assert out.logits[:, -1].argmax(-1).tolist() == fx["forward_last_argmax"]
+    sf = lambda call, shape: O.initialize_state(torch.empty(shape), s, 1.0, torch.Generator().manual_seed(7000 + call))
+    assert O.greedy_generate(w, s, ids, 16, state_fn=sf)[:, 6:].tolist() == fx["greedy_16_tokens"]
+    toks, steps = O.generate_with_adaptive_compute(w, s, ids, 6, criterion="kl", exit_threshold=5e-3, num_steps=8, state_fn=sf,
+                                                   cache_lookup_strategy="latest-m4")
+    assert toks[:, 6:].tolist() == fx["adaptive_kl_5e-3_tokens"] and steps == fx["adaptive_kl_5e-3_compute_steps"]
+    spec = O.generate_speculative(w, s, ids[:1], 10, draft_steps=1, lookahead_for_draft=3, num_steps=4, init_scale=0.0)
+    assert spec[:, 6:].tolist() == fx["speculative_draft1_look3_tokens"]
+
+
+def test_reference_published_cache_sizes_from_the_fixture(pkg):
+    """The three cache sizes the reference's notebook prints, from the fixture file, against the oracle's dict cache
+    and this package's two cache classes."""
+    ka = _golden("reference_known_answers.json")
+    s = O.RavenShape.nebel()
+    for case in ka["cases"][:2]:
+        c = pkg.HuginnDynamicCache(case["strategy"])
+        c._k = torch.empty(1, 1, s.n_heads, 1, s.head_dim, dtype=torch.bfloat16)  # shape carrier only
+        for step in O.step_indices(s):
+            c.note_append(step, case["tokens"], 0)
+        assert c.get_memory_usage() == case["MB"]
+        d = O.DictCache(case["strategy"])
+        one = torch.zeros(1, s.n_heads, 1, s.head_dim, dtype=torch.bfloat16)
+        for step in O.step_indices(s):
+            d.update(one.expand(1, s.n_heads, case["tokens"], s.head_dim), one.expand(1, s.n_heads, case["tokens"], s.head_dim), step)
+        assert d.get_memory_usage() == case["MB"]
+    static = pkg.HuginnStaticCache(max_length=1024, max_num_steps=4 + 4 * 32, num_heads=s.n_heads, hidden_dim=s.head_dim,
+                                   batch_size=1, device="meta", dtype=torch.bfloat16)
+    assert static.get_memory_usage() == ka["cases"][2]["MB"]
