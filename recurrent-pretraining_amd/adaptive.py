@@ -201,7 +201,9 @@ def generate_with_adaptive_compute(model, input_ids: torch.Tensor, generation_co
     the exit evaluator after each; a sequence's next-token logits are frozen at the step where it met the criterion
     while the batch keeps iterating until every sequence has (or max_steps).  Tokens that stop early leave their
     deeper cache steps empty; later tokens that go deeper resolve them through the cache's lookup strategy, inside
-    the attention kernels.
+    the attention kernels.  The recurrences are launched eagerly: replaying them from captured HIP graphs (one per
+    recurrence index) was built and measured and gained nothing at the 3.5b shape -- the host reads the exit decision
+    after every recurrence, and the GPU is not waiting for launches in between.
 
     Extensions: input_states_fn(token_step, (B, S, h)) supplies the initial latent state of each token step
     (the reference draws it from the device RNG); stop_tokens overrides the reference's fixed stop set; with
@@ -224,7 +226,8 @@ def generate_with_adaptive_compute(model, input_ids: torch.Tensor, generation_co
     stops = model._get_stops(gc) if stop_tokens is None else set(stop_tokens)
     dev = model.device
     input_ids = input_ids.to(dev)
-    cache = model_kwargs.get("past_key_values") or HuginnDynamicCache(cache_lookup_strategy)
+    total = min(prompt_len + max_new, model.config.block_size)
+    cache = model_kwargs.get("past_key_values") or HuginnDynamicCache(cache_lookup_strategy, max_length=total)
     h = model.config.n_embd
 
     def draw(token_step: int, shape, embeds):
@@ -236,7 +239,7 @@ def generate_with_adaptive_compute(model, input_ids: torch.Tensor, generation_co
     if continuous_compute:  # RMM:1589-1591: the first state covers the whole prompt
         embeds0 = None if input_states_fn is not None else model.embed_inputs(input_ids)[0]
         next_states = draw(0, (B, prompt_len, h), embeds0)
-    unfinished = torch.ones(B, dtype=torch.bool, device=dev)
+    unfinished = [True] * B
     if exit_evaluator is None:
         exit_evaluator = get_adaptive_exit_evaluator(model, criterion, exit_threshold)
     compute_steps = []
@@ -251,10 +254,15 @@ def generate_with_adaptive_compute(model, input_ids: torch.Tensor, generation_co
             next_states = current[:, -1:, :].clone()
         exit_values_per_seq = [[] for _ in range(B)]
         compute_steps_per_seq = [0] * B
-        exit_reached = torch.zeros(B, dtype=torch.bool, device=dev)
+        # who has left / finished is kept on the host: one device-to-host read per check (its exit flags and values)
+        exit_reached = [False] * B
         outputs, next_token_logits = None, None
         exit_evaluator.init(current)
         finished_loop = True
+
+        def rows(flags):
+            return torch.tensor(flags, dtype=torch.bool, device=dev)
+
         for compute_step in range(max_steps):
             current, block_idx, _ = model.iterate_one_step(embedded, current, block_idx=block_idx, **aux_inputs,
                                                            current_step=compute_step)
@@ -262,26 +270,31 @@ def generate_with_adaptive_compute(model, input_ids: torch.Tensor, generation_co
                     or (do_not_exit_in_prefill and token_step == 0)):
                 continue
             new_exits, outputs, exit_values = exit_evaluator.check(model, current, aux_inputs)
-            counted = (~exit_reached & unfinished).tolist()
-            for i, v in enumerate(exit_values.tolist()):
-                if counted[i]:
-                    exit_values_per_seq[i].append(v)
-            new_exits = new_exits & ~exit_reached & unfinished
-            if bool(new_exits.any()):
-                exit_reached = exit_reached | new_exits
+            host = torch.stack([new_exits.to(torch.float64), exit_values.to(torch.float64)]).tolist()
+            running = [not exit_reached[i] and unfinished[i] for i in range(B)]
+            for i in range(B):
+                if running[i]:
+                    exit_values_per_seq[i].append(host[1][i])
+            leaving = [bool(host[0][i]) and running[i] for i in range(B)]
+            if any(leaving):
+                exit_reached = [exit_reached[i] or leaving[i] for i in range(B)]
                 if outputs is None:  # latent criteria: the coda and the head run only when somebody leaves
                     outputs = model.predict_from_latents(current, **aux_inputs)
                 logits = outputs.logits
                 if next_token_logits is None:
                     next_token_logits = logits[:, -1, :].to(torch.float32).clone()
+                elif all(leaving):
+                    next_token_logits.copy_(logits[:, -1, :])
                 else:
-                    next_token_logits[new_exits] = logits[new_exits, -1, :].to(torch.float32)
-                for i, e in enumerate(new_exits.tolist()):
-                    if e:
+                    mask = rows(leaving)
+                    next_token_logits[mask] = logits[mask, -1, :].to(torch.float32)
+                for i in range(B):
+                    if leaving[i]:
                         compute_steps_per_seq[i] = compute_step + 1
                 if continuous_compute:
-                    next_states[new_exits] = current[new_exits, -1:, :]
-            if bool((exit_reached | ~unfinished).all()):
+                    mask = rows(leaving)
+                    next_states[mask] = current[mask, -1:, :]
+            if all(exit_reached[i] or not unfinished[i] for i in range(B)):
                 finished_loop = False
                 break
         if finished_loop:  # nobody ended the loop early: the remaining sequences take the last outputs
@@ -291,12 +304,12 @@ def generate_with_adaptive_compute(model, input_ids: torch.Tensor, generation_co
                 next_token_logits = outputs.logits[:, -1, :].to(torch.float32).clone()
                 compute_steps_per_seq = [max_steps] * B
             else:
-                for i, run in enumerate((~exit_reached & unfinished).tolist()):
-                    if run:
+                for i in range(B):
+                    if not exit_reached[i] and unfinished[i]:
                         next_token_logits[i] = outputs.logits[i, -1, :].to(torch.float32)
                         compute_steps_per_seq[i] = max_steps
         if continuous_compute:
-            still_running = ~exit_reached & unfinished
+            still_running = rows([not exit_reached[i] and unfinished[i] for i in range(B)])
             next_states[still_running] = current[still_running, -1:, :]
         compute_steps.append([compute_steps_per_seq, exit_values_per_seq])
 
@@ -309,8 +322,9 @@ def generate_with_adaptive_compute(model, input_ids: torch.Tensor, generation_co
                 if v in stops:
                     unfinished[i] = False
         if "stopping_criteria" in model_kwargs:
-            unfinished = unfinished & ~model_kwargs["stopping_criteria"](input_ids, None)
-        if not bool(unfinished.any()):
+            done = model_kwargs["stopping_criteria"](input_ids, None).tolist()
+            unfinished = [unfinished[i] and not done[i] for i in range(B)]
+        if not any(unfinished):
             break
     if streamer:
         streamer.end()
