@@ -52,7 +52,7 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
 def prefill(args):
-    """BASELINE configs[4]: the recurrent core over a full prompt.  Token ids uniform over the vocabulary from seed 1,
+    """BASELINE.json configs[4]: the recurrent core over a full prompt.  Token ids uniform over the vocabulary from seed 1,
     random-init weights; the prelude runs once (untimed), then r core iterations over all B x S rows are timed.
     FLOPs per iteration: GEMMs 2*M*(params of adapter + 4 blocks) + causal attention 4 * 2*B*nh*hd*S*(S+1)/2 * 2."""
     import torch
@@ -94,7 +94,7 @@ def prefill(args):
         "value": round(M * r / (ms * 1e-3), 1), "unit": "tokens*iterations/s", "n_gpus": 1, "steps": r, "warmup": 1,
         "ms_per_step": round(ms / r, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": f"recurrent-core prefill, nebel-raven-3.5b shape, bs={B} x {S} tokens, r={r} (BASELINE configs[4])",
+        "config": {"workload": f"recurrent-core prefill, nebel-raven-3.5b shape, bs={B} x {S} tokens, r={r} (BASELINE.json configs[4])",
                    "batch": B, "seq_len": S, "recurrence": r, "gemm": "hipBLASLt via torch.matmul", "attention": "attention_prefill_kernel"},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / MFMA_PEAK_TFLOPS, 4), "flops_per_iteration": gemm_flops + attn_flops, "traffic": None},
@@ -361,7 +361,7 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"full-token greedy decode, nebel-raven-3.5b shape, r={r}, bs={args.batch}, "
-                               f"{args.prompt}-token random prompt, {args.steps} timed tokens (BASELINE configs[3])",
+                               f"{args.prompt}-token random prompt, {args.steps} timed tokens (BASELINE.json configs[3])",
                    "batch": args.batch, "recurrence": r, "prompt": args.prompt, "hip_graph": use_graph},
         "recurrence_steps_per_s": round(tok_s * r / args.batch, 2),
         "token_roofline": {"bytes_per_token": int(token_bytes), "achieved_GBs": round(token_bytes * (tok_s / args.batch) / 1e9, 1),
