@@ -335,6 +335,23 @@ def main():
     copy_gbs = 2 * src.numel() / (copy_ms * 1e-3) / 1e9
     del src, dst, kc, vc
 
+    # ---- the isolated norm kernel (BASELINE.json configs[1]): x + residual -> RMSNorm, [T, 5280] bf16, 31,680 B per row ----
+    norm_w = model.transformer.core_block[0].norm_1.weight
+    norm_cfg2 = {}
+    for T_rows in (1, 32, 4096):
+        xs = [torch.randn(T_rows, h, device=dev, dtype=torch.bfloat16) for _ in range(8)]  # rotate: 8 x 43 MB at T = 4096
+        rs = torch.randn(T_rows, h, device=dev, dtype=torch.bfloat16)
+        yo = torch.empty_like(rs)
+
+        def norm_launch(i=[0]):
+            i[0] += 1
+            lib.raven_rmsnorm_residual(xs[i[0] % 8].data_ptr(), rs.data_ptr(), norm_w.data_ptr(), yo.data_ptr(), None, None, None, T_rows, h,
+                                       cfg.norm_eps, pkg.hip.BF16, stream)
+
+        t_ms = event_time_ms(norm_launch, 100, warm=10)
+        norm_cfg2[f"T={T_rows}"] = {"us": round(t_ms * 1e3, 2), "GBs": round(T_rows * 3 * h * 2 / (t_ms * 1e-3) / 1e9, 1)}
+        del xs, rs, yo
+
     also = None
     if args.also_batch and args.also_batch != args.batch:
         torch.cuda.empty_cache()
@@ -375,6 +392,7 @@ def main():
         "core_iteration": {"T": T, "batch": B, "bytes": int(it_bytes), "ms_eager": round(iter_eager_ms, 4),
                            "ms_graph": round(iter_graph_ms, 4), "achieved_GBs": round(it_bytes / (iter_ms * 1e-3) / 1e9, 1),
                            "frac": round(it_bytes / (iter_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+        "rmsnorm_residual_5280": norm_cfg2,
         "device_copy_GBs": round(copy_gbs, 1),
         "prefill_s": round(prefill_s, 3),
         "also": also,
