@@ -146,6 +146,22 @@ int raven_exit_logit_stats(const float* logits, float* prev_log_probs, float* ou
 int raven_exit_latent_stats(const void* latents, const void* prev, void* rel_change, void* cosine,
                             int32_t rows, int32_t h, int32_t dtype, void* stream);
 
+/* Paged KV cache, the layout the attention layer of the reference's vLLM plugin is given (vllm/raven_vllm.py:174-201
+ * hands rotated q, k and v to vLLM's Attention, which owns a block-paged cache): k_cache and v_cache are
+ * [num_blocks, block_size, n_heads, head_dim] of T; position p of sequence b lives in block
+ * block_table[b * max_blocks + p / block_size] at offset p % block_size.
+ * raven_paged_kv_append: rows k, v [T, n_heads * head_dim] (k already biased and rotated) go to the flat slots
+ *   slot_mapping[t] = block * block_size + offset (negative: skipped).
+ * raven_paged_decode_attention: one query row per sequence, q / y [B, n_heads * head_dim]; sequence b attends to its
+ *   first seq_lens[b] positions (its own new token included; 0 gives zeros).  max_seq_len >= every seq_lens[b] sizes the
+ *   launch.  workspace as for raven_decode_attention (raven_decode_attention_workspace_bytes(B, ...)). */
+int raven_paged_kv_append(const void* k, const void* v, void* k_cache, void* v_cache, const int64_t* slot_mapping,
+                          int32_t T, int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream);
+int raven_paged_decode_attention(const void* q, void* y, const void* k_cache, const void* v_cache,
+                                 const int32_t* block_table, const int32_t* seq_lens, int32_t B, int32_t max_blocks,
+                                 int32_t block_size, int32_t max_seq_len, int32_t n_heads, int32_t head_dim,
+                                 int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Decode fast path for ONE token row, one launch:
  *     x  = norm_a ? T(rmsnorm(x0) * norm_a) : x0      -> stored to xa_out when non-NULL
  *     x  = norm_b ? T(rmsnorm(x)  * norm_b) : x

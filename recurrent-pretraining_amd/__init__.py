@@ -7,6 +7,7 @@ registers this directory under that name).
 
 from . import hip  # noqa: F401
 from . import adaptive  # noqa: F401
+from . import vllm_binding  # noqa: F401
 from .adaptive import (  # noqa: F401
     ArgmaxStabilityExitEvaluator,
     CosineExitEvaluator,
@@ -31,7 +32,7 @@ from .modeling import (  # noqa: F401
 
 __all__ = [
     "hip", "HuginnDynamicCache", "HuginnStaticCache", "remap_step", "RavenConfig", "RavenForCausalLM", "DecodeRunner",
-    "CausalLMOutputRecurrentLatents", "GenerationSettings", "precompute_freqs_cis", "adaptive",
+    "CausalLMOutputRecurrentLatents", "GenerationSettings", "precompute_freqs_cis", "adaptive", "vllm_binding",
     "PerIterationExitEvaluator", "NoOpExitEvaluator", "EntropyDiffExitEvaluator", "LatentDiffExitEvaluator",
     "KLExitEvaluator", "MinKLExitEvaluator", "ArgmaxStabilityExitEvaluator", "CosineExitEvaluator", "NumStepsGenerator",
     "get_adaptive_exit_evaluator",

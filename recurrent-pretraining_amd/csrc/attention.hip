@@ -327,7 +327,132 @@ __global__ __launch_bounds__(128) void attention_combine_kernel(const float* __r
         Lg += ws_ml[(mh * n_splits + sp) * 2 + 1] * wgt;
         Og += ws_o[(mh * n_splits + sp) * hd + t] * wgt;
     }
-    y[(int64_t)m * nh * hd + head * hd + t] = from_f32<T>(Og / Lg);
+    y[(int64_t)m * nh * hd + head * hd + t] = from_f32<T>(Lg > 0.f ? Og / Lg : 0.f);  // no position at all (an empty paged sequence): zeros
+}
+
+// ------------------------------------------------------------------------------------------------
+// Paged KV cache (the layout vLLM's attention layer owns): K and V are [num_blocks, block_size, n_heads, head_dim];
+// a sequence's position p lives in block block_table[seq][p / block_size] at offset p % block_size, and every
+// sequence has its own length.  One new query row per sequence (decode).  Same arithmetic as decode_attention_kernel:
+// 16 lanes per position, online softmax per 16-lane row, rows merged through LDS, splits merged by
+// attention_combine_kernel.
+// ------------------------------------------------------------------------------------------------
+struct PagedView {
+    const void* k;
+    const void* v;
+    const int* block_table;  // [B, max_blocks]
+    const int* seq_lens;     // [B]: positions to attend to, the new token's own included
+    int max_blocks, block_size, nh, hd;
+};
+
+template <typename T, int CPL>
+__global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __restrict__ q, T* __restrict__ y, PagedView pv,
+                                                                     float scale_log2, int n_splits, float* __restrict__ ws_ml,
+                                                                     float* __restrict__ ws_o) {
+    constexpr int EC = Chunk<T>::N, E = EC * CPL, G = 16, U = 2;
+    __shared__ float sm_m[G], sm_l[G];
+    __shared__ float sm_o[G][kAttnMaxHd];
+    typedef Piece<T, CPL> P;
+    const int head = blockIdx.x, b = blockIdx.y, split = blockIdx.z;
+    const int hd = pv.hd, h = pv.nh * hd;
+    const int len = pv.seq_lens[b];
+    const int per = (len + n_splits - 1) / n_splits;
+    const int start = split * per, end = min(len, start + per);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane >> 4, ci = lane & 15;
+    const bool active = ci < hd / E;
+    const int group = wave * 4 + r;
+    const int* table = pv.block_table + (int64_t)b * pv.max_blocks;
+    const T* K = static_cast<const T*>(pv.k);
+    const T* V = static_cast<const T*>(pv.v);
+    const P qc = active ? load_piece<T, CPL>(q + (int64_t)b * h + head * hd + ci * E) : zero_piece<T, CPL>();
+
+    float m_run = -INFINITY, l_run = 0.f, o[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) o[e] = 0.f;
+    for (int base = start; base < end; base += G * U) {  // trip count is uniform over the workgroup
+        P kc[U], vc[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int p = base + j * G + group;
+            if (active && p < end) {
+                const int64_t row = (int64_t)table[p / pv.block_size] * pv.block_size + p % pv.block_size;
+                const int64_t off = (row * pv.nh + head) * hd + ci * E;
+                kc[j] = load_piece<T, CPL, true>(K + off);
+                vc[j] = load_piece<T, CPL, true>(V + off);
+            } else {
+                kc[j] = zero_piece<T, CPL>();
+                vc[j] = zero_piece<T, CPL>();
+            }
+        }
+        float sc[U], m_new = m_run;
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            sc[j] = row16_sum(dot_piece<T, CPL>(qc, kc[j])) * scale_log2;
+            if (base + j * G + group >= end) sc[j] = -INFINITY;
+            m_new = fmaxf(m_new, sc[j]);
+        }
+        if (m_new == -INFINITY) continue;
+        const float corr = exp2f(m_run - m_new);
+        float pe[U], psum = 0.f;
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            pe[j] = exp2f(sc[j] - m_new);
+            psum += pe[j];
+        }
+        l_run = l_run * corr + psum;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float acc = o[e] * corr;
+#pragma unroll
+            for (int j = 0; j < U; ++j) acc = __builtin_fmaf(pe[j], to_f32(vc[j].c[e / EC].v[e % EC]), acc);
+            o[e] = acc;
+        }
+        m_run = m_new;
+    }
+    if (ci == 0) {
+        sm_m[group] = m_run;
+        sm_l[group] = l_run;
+    }
+    if (active) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) sm_o[group][ci * E + e] = o[e];
+    }
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t < hd) {
+        float M = -INFINITY, L = 0.f, O = 0.f;
+#pragma unroll
+        for (int g = 0; g < G; ++g) M = fmaxf(M, sm_m[g]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float wgt = (sm_m[g] == -INFINITY) ? 0.f : exp2f(sm_m[g] - M);
+            L += sm_l[g] * wgt;
+            O += sm_o[g][t] * wgt;
+        }
+        if (n_splits == 1) {
+            y[(int64_t)b * h + head * hd + t] = from_f32<T>(L > 0.f ? O / L : 0.f);  // an empty sequence gives zeros
+        } else {
+            const int64_t idx = ((int64_t)b * pv.nh + head) * n_splits + split;
+            ws_o[idx * hd + t] = O;
+            if (t == 0) {
+                ws_ml[idx * 2] = M;
+                ws_ml[idx * 2 + 1] = L;
+            }
+        }
+    }
+}
+
+// cache[slot_mapping[t]] = row t, for K and V: rows of [n_heads * head_dim] elements; negative slots are skipped
+template <typename T>
+__global__ __launch_bounds__(256) void paged_kv_append_kernel(const T* __restrict__ k, const T* __restrict__ v, T* __restrict__ kc,
+                                                              T* __restrict__ vc, const int64_t* __restrict__ slots, int h) {
+    constexpr int E = Chunk<T>::N;
+    const int t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    const int64_t slot = slots[t];
+    if (c >= h / E || slot < 0) return;
+    store_chunk(kc + slot * h + c * E, load_chunk(k + (int64_t)t * h + c * E));
+    store_chunk(vc + slot * h + c * E, load_chunk(v + (int64_t)t * h + c * E));
 }
 
 constexpr int kAttnMaxSplits = 32;
@@ -488,4 +613,57 @@ extern "C" int raven_qkv_attention_decode(const void* qkv, const void* qk_bias, 
                                           void* workspace, size_t workspace_bytes, void* stream) {
     return attention_common("qkv_attention_decode", true, qkv, qk_bias, freqs, y, cache, slot, B, 1, pos0, pos_dev, n_heads,
                             head_dim, dtype, workspace, workspace_bytes, stream);
+}
+
+
+extern "C" int raven_paged_kv_append(const void* k, const void* v, void* k_cache, void* v_cache, const int64_t* slot_mapping,
+                                     int32_t T, int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream) {
+    using namespace raven;
+    if (int rc = check_heads("paged_kv_append", n_heads, head_dim, dtype)) return rc;
+    RAVEN_REQUIRE(T >= 0 && T <= 65535, "paged_kv_append: bad row count %d", T);
+    if (T == 0) return 0;
+    RAVEN_REQUIRE(k && v && k_cache && v_cache && slot_mapping, "paged_kv_append: null pointer");
+    const int h = n_heads * head_dim, elts = 16 / (int)raven_host::elt_size(dtype);
+    const dim3 grid((h / elts + 255) / 256, T);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == RAVEN_BF16) paged_kv_append_kernel<bf16><<<grid, dim3(256), 0, s>>>((const bf16*)k, (const bf16*)v, (bf16*)k_cache, (bf16*)v_cache, slot_mapping, h);
+    else paged_kv_append_kernel<float><<<grid, dim3(256), 0, s>>>((const float*)k, (const float*)v, (float*)k_cache, (float*)v_cache, slot_mapping, h);
+    return raven_host::check_launch("paged_kv_append");
+}
+
+extern "C" int raven_paged_decode_attention(const void* q, void* y, const void* k_cache, const void* v_cache,
+                                            const int32_t* block_table, const int32_t* seq_lens, int32_t B, int32_t max_blocks,
+                                            int32_t block_size, int32_t max_seq_len, int32_t n_heads, int32_t head_dim, int32_t dtype,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace raven;
+    if (int rc = check_heads("paged_decode_attention", n_heads, head_dim, dtype)) return rc;
+    RAVEN_REQUIRE(B >= 0 && B <= 65535 && max_blocks > 0 && block_size > 0 && max_seq_len > 0, "paged_decode_attention: bad B=%d max_blocks=%d block_size=%d max_seq_len=%d", B, max_blocks, block_size, max_seq_len);
+    if (B == 0) return 0;
+    RAVEN_REQUIRE(q && y && k_cache && v_cache && block_table && seq_lens, "paged_decode_attention: null pointer");
+    RAVEN_REQUIRE((int64_t)max_blocks * block_size >= max_seq_len, "paged_decode_attention: %d blocks of %d cannot hold %d positions", max_blocks, block_size, max_seq_len);
+    int ns = splits_for(B, n_heads, max_seq_len);
+    float *ws_ml = nullptr, *ws_o = nullptr;
+    if (ns > 1) {
+        const size_t need = raven_decode_attention_workspace_bytes(B, n_heads, head_dim);
+        if (workspace == nullptr || workspace_bytes < need) {
+            ns = 1;
+        } else {
+            RAVEN_REQUIRE(((uintptr_t)workspace & 255) == 0, "paged_decode_attention: workspace must be 256-byte aligned");
+            ws_ml = static_cast<float*>(workspace);
+            ws_o = reinterpret_cast<float*>(static_cast<char*>(workspace) + raven_host::align_up((size_t)B * n_heads * kAttnMaxSplits * 2 * 4));
+        }
+    }
+    PagedView pv{k_cache, v_cache, block_table, seq_lens, max_blocks, block_size, n_heads, head_dim};
+    const float scale_log2 = (float)(1.0 / sqrt((double)head_dim) * 1.4426950408889634);
+    const dim3 grid(n_heads, B, ns);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == RAVEN_BF16) {
+        paged_decode_attention_kernel<bf16, 1><<<grid, dim3(256), 0, s>>>((const bf16*)q, (bf16*)y, pv, scale_log2, ns, ws_ml, ws_o);
+        if (ns > 1) attention_combine_kernel<bf16><<<dim3(n_heads, B), dim3(128), 0, s>>>(ws_ml, ws_o, (bf16*)y, n_heads, head_dim, ns);
+    } else {
+        if (head_dim / 4 > 16) paged_decode_attention_kernel<float, 2><<<grid, dim3(256), 0, s>>>((const float*)q, (float*)y, pv, scale_log2, ns, ws_ml, ws_o);
+        else paged_decode_attention_kernel<float, 1><<<grid, dim3(256), 0, s>>>((const float*)q, (float*)y, pv, scale_log2, ns, ws_ml, ws_o);
+        if (ns > 1) attention_combine_kernel<float><<<dim3(n_heads, B), dim3(128), 0, s>>>(ws_ml, ws_o, (float*)y, n_heads, head_dim, ns);
+    }
+    return raven_host::check_launch("paged_decode_attention");
 }

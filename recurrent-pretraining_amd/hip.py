@@ -58,6 +58,8 @@ SIGNATURES = {
     "raven_linear": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _VP, _SZ, _VP]),
     "raven_exit_logit_stats": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I32, _VP]),
     "raven_exit_latent_stats": (C.c_int, [_VP, _VP, _VP, _VP, _I32, _I32, _I32, _VP]),
+    "raven_paged_kv_append": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _VP]),
+    "raven_paged_decode_attention": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _VP, _SZ, _VP]),
     "raven_gemv_fused": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _F, _I32, _I32, _I32, _VP]),
     "raven_qkv_bias_rope_cache_append": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32,
                                                    _VP, _I32, _I32, _I32, _VP]),
@@ -227,6 +229,29 @@ def linear(x0, w, x1=None, residual=None, swiglu=False, out_f32=False, workspace
                              M, N, K0, K1, int(swiglu), int(out_f32), dtype_code(dt), _ptr(workspace, "workspace", torch.uint8),
                              0 if workspace is None else workspace.numel(), _stream())
     _check(rc, "raven_linear")
+    return y
+
+
+def paged_kv_append(k, v, k_cache, v_cache, slot_mapping):
+    """k, v [T, nh * hd] -> k_cache / v_cache [num_blocks, block_size, nh, hd] at the flat slots slot_mapping [T] (int64)."""
+    T = k.shape[0]
+    nh, hd = k_cache.shape[2], k_cache.shape[3]
+    rc = load().raven_paged_kv_append(_ptr(k, "k"), _ptr(v, "v", k.dtype), _ptr(k_cache, "k_cache", k.dtype), _ptr(v_cache, "v_cache", k.dtype),
+                                      _ptr(slot_mapping, "slot_mapping", torch.int64), T, nh, hd, dtype_code(k.dtype), _stream())
+    _check(rc, "raven_paged_kv_append")
+
+
+def paged_decode_attention(q, k_cache, v_cache, block_table, seq_lens, max_seq_len, workspace=None):
+    """q [B, nh * hd]; k_cache / v_cache [num_blocks, block_size, nh, hd]; block_table [B, max_blocks] int32; seq_lens [B] int32."""
+    B = q.shape[0]
+    _, block_size, nh, hd = k_cache.shape
+    y = torch.empty_like(q)
+    rc = load().raven_paged_decode_attention(
+        _ptr(q, "q"), _ptr(y, "y"), _ptr(k_cache, "k_cache", q.dtype), _ptr(v_cache, "v_cache", q.dtype),
+        _ptr(block_table, "block_table", torch.int32), _ptr(seq_lens, "seq_lens", torch.int32), B, block_table.shape[1], block_size,
+        int(max_seq_len), nh, hd, dtype_code(q.dtype), _ptr(workspace, "workspace", torch.uint8),
+        0 if workspace is None else workspace.numel(), _stream())
+    _check(rc, "raven_paged_decode_attention")
     return y
 
 

@@ -602,3 +602,71 @@ def test_fp32_kernels_at_the_3_5b_shape(pkg):
     y_2 = pkg.hip.decode_attention(q2, cache2, 1, B, 1, 150, nh, hd, workspace=ws)
     assert torch.equal(kd, kd2) and torch.equal(vd, vd2)
     check(y_f, y_2.cpu(), dt, "fp32 hd=96 fused decode step")
+
+
+# ----------------------------------------------------------------------------- paged KV cache (vLLM layout)
+@pytest.mark.parametrize("dt,nh,hd,B,block_size", [(torch.bfloat16, 55, 96, 1, 16), (torch.bfloat16, 55, 96, 32, 16),
+                                                   (torch.bfloat16, 55, 96, 5, 32), (torch.float32, 4, 64, 3, 8),
+                                                   (torch.float32, 5, 96, 2, 16)])
+def test_paged_decode_attention_and_append(pkg, dt, nh, hd, B, block_size):
+    """Block-paged K/V with shuffled block tables and a different length per sequence (1 and 0 among them): appended rows
+    land in their slots, attention equals torch SDPA per sequence, and -- for equal lengths -- the contiguous kernel's bits."""
+    h = nh * hd
+    g = torch.Generator().manual_seed(600 + B)
+    max_len = 700
+    max_blocks = (max_len + block_size - 1) // block_size
+    num_blocks = B * max_blocks + 3
+    lens = torch.randint(2, max_len + 1, (B,), generator=g, dtype=torch.int32)
+    lens[0] = max_len
+    if B > 2:
+        lens[1], lens[2] = 1, 0
+    table = torch.randperm(num_blocks, generator=g)[:B * max_blocks].view(B, max_blocks).to(torch.int32)
+    k_seq, v_seq = rnd((B, max_len, nh, hd), dt, 601), rnd((B, max_len, nh, hd), dt, 602)
+    kc = torch.zeros(num_blocks, block_size, nh, hd, dtype=dt, device="cuda")
+    vc = torch.zeros_like(kc)
+    # fill the cache through the append kernel: every sequence's positions, in one call, plus a skipped row
+    rows_k, rows_v, slots = [], [], []
+    for b in range(B):
+        for p in range(int(lens[b])):
+            rows_k.append(k_seq[b, p].reshape(-1))
+            rows_v.append(v_seq[b, p].reshape(-1))
+            slots.append(int(table[b, p // block_size]) * block_size + p % block_size)
+    rows_k.append(torch.ones(h, dtype=dt))
+    rows_v.append(torch.ones(h, dtype=dt))
+    slots.append(-1)
+    kk, vv, sl = torch.stack(rows_k).cuda(), torch.stack(rows_v).cuda(), torch.tensor(slots, dtype=torch.int64).cuda()
+    for lo in range(0, kk.shape[0], 60000):
+        pkg.hip.paged_kv_append(kk[lo:lo + 60000].contiguous(), vv[lo:lo + 60000].contiguous(), kc, vc, sl[lo:lo + 60000].contiguous())
+    flat_k = kc.view(-1, nh, hd).cpu()
+    for b in range(B):
+        for p in (0, int(lens[b]) - 1):
+            if p >= 0 and int(lens[b]) > 0:
+                assert torch.equal(flat_k[int(table[b, p // block_size]) * block_size + p % block_size], k_seq[b, p])
+    assert int((flat_k.abs().amax(dim=(1, 2)) > 0).sum()) == int(lens.sum())  # nothing written anywhere else (the -1 row is skipped)
+    q = rnd((B, h), dt, 603)
+    ws = pkg.hip.attention_workspace(B, nh, hd, "cuda")
+    for wsp in (ws, None):
+        y = pkg.hip.paged_decode_attention(q.cuda(), kc, vc, table.cuda(), lens.cuda(), max_len, workspace=wsp)
+        for b in range(B):
+            n = int(lens[b])
+            if n == 0:
+                assert float(y[b].abs().max()) == 0.0
+                continue
+            want = F.scaled_dot_product_attention(q[b].view(1, nh, 1, hd).float(), k_seq[b, :n].transpose(0, 1).unsqueeze(0).float(),
+                                                  v_seq[b, :n].transpose(0, 1).unsqueeze(0).float()).reshape(h)
+            check(y[b], want, dt, f"paged attention, sequence {b} of length {n}")
+    # equal lengths: the same numbers as the contiguous cache kernel gives (same arithmetic, other addresses)
+    n = 300
+    eq = torch.full((B,), n, dtype=torch.int32)
+    y = pkg.hip.paged_decode_attention(q.cuda(), kc, vc, table.cuda(), eq.cuda(), n)
+    kd = torch.zeros(1, B, nh, n, hd, dtype=dt)
+    vd = torch.zeros_like(kd)
+    for b in range(B):
+        m = min(n, int(lens[b]))
+        kd[0, b, :, :m], vd[0, b, :, :m] = k_seq[b, :m].transpose(0, 1), v_seq[b, :m].transpose(0, 1)
+    kdd, vdd = kd.cuda(), vd.cuda()
+    want = pkg.hip.decode_attention(q.cuda(), pkg.hip.make_cache(kdd, vdd), 0, B, 1, n - 1, nh, hd)
+    full = [b for b in range(B) if int(lens[b]) >= n]
+    check(y[full], want[full].float().cpu(), dt, "paged vs contiguous")
+    with pytest.raises(pkg.hip.RavenHipError):
+        pkg.hip.paged_decode_attention(q.cuda(), kc, vc, table.cuda(), lens.cuda(), max_blocks * block_size + 1)

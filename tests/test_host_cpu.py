@@ -242,3 +242,39 @@ def test_reference_published_cache_sizes_from_the_fixture(pkg):
     static = pkg.HuginnStaticCache(max_length=1024, max_num_steps=4 + 4 * 32, num_heads=s.n_heads, hidden_dim=s.head_dim,
                                    batch_size=1, device="meta", dtype=torch.bfloat16)
     assert static.get_memory_usage() == ka["cases"][2]["MB"]
+
+
+# ----------------------------------------------------------------------------- vLLM plugin naming
+def test_vllm_flat_layer_names_and_schedule(pkg):
+    """Hugging Face names -> the vLLM plugin's flat names (vllm/raven_vllm.py:481-526), spot values by hand, a full
+    round trip over the 3.5b state-dict layout, and the order of a forward over the flat layers (raven_vllm.py:389-411)."""
+    vb = pkg.vllm_binding
+    cfg = pkg.RavenConfig()
+    hand = {
+        "transformer.wte.weight": "model.embed_tokens.weight",
+        "lm_head.weight": "model.embed_tokens.weight",
+        "transformer.prelude.1.attn.Wqkv.weight": "model.layers.1.self_attn.qkv_proj.weight",
+        "transformer.core_block.0.mlp.fc.weight": "model.layers.2.mlp.gate_up_proj.weight",
+        "transformer.core_block.3.attn.qk_bias": "model.layers.5.self_attn.qk_bias",
+        "transformer.coda.1.mlp.proj.weight": "model.layers.7.mlp.down_proj.weight",
+        "transformer.coda.0.attn.proj.weight": "model.layers.6.self_attn.o_proj.weight",
+        "transformer.core_block.2.norm_3.weight": "model.layers.4.norm_3.weight",
+        "transformer.ln_f.weight": "model.ln_f.weight",
+        "transformer.adapter.weight": "model.adapter.weight",
+        "freqs_cis": None,
+    }
+    for hf, want in hand.items():
+        assert vb.vllm_name(hf, cfg) == want, hf
+    names = [n for n, _ in O.state_dict_layout(O.RavenShape.nebel())]
+    mapped = [vb.vllm_name(n, cfg) for n in names]
+    assert len(set(mapped)) == len(names) and all(vb.hf_name(m, cfg) == n for m, n in zip(mapped, names))
+    assert sum(m.startswith("model.layers.") for m in mapped) == 8 * 9
+    sd = {"transformer.core_block.1.attn.qk_bias": torch.zeros(2, 1, 55, 96), "freqs_cis": torch.zeros(1), "lm_head.weight": torch.ones(3),
+          "transformer.wte.weight": torch.ones(3)}
+    out = vb.to_vllm_state_dict(sd, cfg)
+    assert set(out) == {"model.layers.3.self_attn.qk_bias", "model.embed_tokens.weight"}
+    assert out["model.layers.3.self_attn.qk_bias"].shape == (2, 55, 96)
+    plan = vb.flat_layer_schedule(cfg, num_steps=2)
+    assert plan == ([("layer", 0), ("layer", 1)] + [("adapter", 0)] + [("layer", i) for i in (2, 3, 4, 5)] + [("adapter", 1)]
+                    + [("layer", i) for i in (2, 3, 4, 5)] + [("ln_f", 0), ("layer", 6), ("layer", 7), ("ln_f", 1)])
+    assert len(vb.flat_layer_schedule(cfg)) == 2 + 32 * 5 + 1 + 2 + 1
