@@ -19,8 +19,12 @@ extern "C" int raven_gemv_fused(const void* x0, const void* x1, const void* norm
 
 namespace raven {
 
+int gemv1_column_block(const void* x, const void* norm_a, const void* w_block, int ldw, const float* acc_in, void* y, int raw_out,
+                       int N, int K, float eps, int dtype, hipStream_t s);
+
 struct BlockScratch {
     char *n1, *qkv, *q, *ya, *x1, *x2, *n3, *g, *x3, *xa, *xr;
+    float* e_sums;  // one row: fp32 sums of the adapter's embedding half, computed once for all recurrences
     void* attn_ws;
     size_t attn_ws_bytes;
     void* lin_ws;
@@ -48,6 +52,7 @@ static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
     s.x3 = take(row);
     s.xa = take(row);
     s.xr = take(row);
+    s.e_sums = reinterpret_cast<float*>(take(M == 1 ? (size_t)d->n_embd * sizeof(float) : 0));
     s.attn_ws_bytes = raven_decode_attention_workspace_bytes(M, d->n_heads, d->head_dim);
     s.attn_ws = s.attn_ws_bytes ? take(s.attn_ws_bytes) : nullptr;
     const int widest = 3 * d->n_embd > 2 * d->intermediate ? 3 * d->n_embd : 2 * d->intermediate;
@@ -187,13 +192,22 @@ extern "C" int raven_core_iterations(const raven_dims* dims, const void* adapter
     if (M == 1 && one_row_fits(dims)) {
         // One row: between two iterations the last block's closing norm_4 is the prologue of the next adapter product
         // (no launch of its own); only the last iteration closes with a norm launch (norm_4, then ln_f if asked for).
+        // The embedding half of the adapter product is the same in every recurrence: with two or more of them its fp32
+        // sums are formed once, and each recurrence streams the state half of the weight only.
+        const bool split = n_iterations >= 2;
+        const size_t es = raven_host::elt_size(dims->dtype);
+        hipStream_t hs = static_cast<hipStream_t>(stream);
+        if (split)
+            if ((rc = gemv1_column_block(embeds, nullptr, static_cast<const char*>(adapter_w) + (size_t)h * es, 2 * h, nullptr, s.e_sums,
+                                         1, h, h, dims->eps, dims->dtype, hs))) return rc;
         for (int it = 0; it < n_iterations; ++it) {
             const int32_t* sl = slots + (size_t)it * n_blocks;
-            if (it == 0)
-                rc = raven_gemv_fused(state_in, embeds, nullptr, nullptr, nullptr, adapter_w, nullptr, s.xa, h, h, h, dims->eps, 0, 0,
-                                      dims->dtype, stream);
+            const void* x_in = it == 0 ? state_in : (const void*)s.x3;
+            const void* pre_norm = it == 0 ? nullptr : last_blk.norm_4;
+            if (split)
+                rc = gemv1_column_block(x_in, pre_norm, adapter_w, 2 * h, s.e_sums, s.xa, 0, h, h, dims->eps, dims->dtype, hs);
             else
-                rc = raven_gemv_fused(s.x3, embeds, last_blk.norm_4, nullptr, nullptr, adapter_w, nullptr, s.xa, h, h, h, dims->eps, 0, 0,
+                rc = raven_gemv_fused(x_in, embeds, pre_norm, nullptr, nullptr, adapter_w, nullptr, s.xa, h, h, h, dims->eps, 0, 0,
                                       dims->dtype, stream);
             if (rc) return rc;
             for (int j = 0; j < n_blocks; ++j) {

@@ -33,6 +33,9 @@ struct Gemv1Args {
     int out_f32;
     float eps;
     int pairs_per_wg;      // weight-row pairs each workgroup walks through
+    int ldw;               // elements between two weight rows (K, or more for a column block of a wider matrix)
+    const float* acc_in;   // [N] or null: fp32 sums of the remaining columns, added before the result is rounded
+    int raw_out;           // y receives the unrounded fp32 sums (the other half of acc_in)
 };
 
 template <bool NT, typename T>
@@ -76,8 +79,8 @@ __global__ __launch_bounds__(256) void gemv1_kernel(Gemv1Args a) {
     auto load_pair = [&](int unit, Chunk<T>* wa, Chunk<T>* wb) {
         const int r0 = SWIGLU ? unit : 2 * unit;
         const int r1 = SWIGLU ? unit + a.N : min(r0 + 1, a.N - 1);
-        const T* w0 = W + (int64_t)r0 * a.K;
-        const T* w1 = W + (int64_t)r1 * a.K;
+        const T* w0 = W + (int64_t)r0 * a.ldw;
+        const T* w1 = W + (int64_t)r1 * a.ldw;
 #pragma unroll
         for (int j = 0; j < C; ++j) {
             const int c = cb + lane + 64 * j;
@@ -182,8 +185,20 @@ __global__ __launch_bounds__(256) void gemv1_kernel(Gemv1Args a) {
     const int p = threadIdx.x;
     if (p < ppw && unit_of(p) < n_units) {
         const int unit = unit_of(p);
-        const float s0 = part[p][0][0] + part[p][1][0] + part[p][2][0] + part[p][3][0];
-        const float s1 = part[p][0][1] + part[p][1][1] + part[p][2][1] + part[p][3][1];
+        float s0 = part[p][0][0] + part[p][1][0] + part[p][2][0] + part[p][3][0];
+        float s1 = part[p][0][1] + part[p][1][1] + part[p][2][1] + part[p][3][1];
+        if (!SWIGLU && (a.acc_in || a.raw_out)) {
+            const int r0 = 2 * unit, r1 = r0 + 1;
+            if (a.acc_in) {
+                s0 += a.acc_in[r0];
+                if (r1 < a.N) s1 += a.acc_in[r1];
+            }
+            if (a.raw_out) {
+                static_cast<float*>(a.y)[r0] = s0;
+                if (r1 < a.N) static_cast<float*>(a.y)[r1] = s1;
+                return;
+            }
+        }
         if (SWIGLU) {
             const float g = round_to<T>(s0), u = round_to<T>(s1);
             static_cast<T*>(a.y)[unit] = from_f32<T>(round_to<T>(silu_f32(g)) * u);
@@ -255,6 +270,18 @@ int set_gemv1_tuning(const char* key, int value) {
     return 0;
 }
 
+// One column block of a wider weight matrix: y = round(norm_a(x) W[:, c0 : c0 + K]^T + acc_in), or the unrounded
+// fp32 sums when raw_out is set.  A product over concatenated inputs (the adapter's [state, embedding],
+// recpre/raven_modeling_minimal.py:776) whose second input does not change between calls is split with it: the sums of
+// the unchanged half are kept in fp32 and enter the other half's accumulator before the one rounding the product has.
+int gemv1_column_block(const void* x, const void* norm_a, const void* w_block, int ldw, const float* acc_in, void* y, int raw_out,
+                       int N, int K, float eps, int dtype, hipStream_t s) {
+    Gemv1Args a{};
+    a.w = w_block; a.x0 = x; a.norm_a = norm_a; a.y = y; a.N = N; a.K = K; a.k0 = K; a.eps = eps;
+    a.ldw = ldw; a.acc_in = acc_in; a.raw_out = raw_out;
+    return dtype == RAVEN_BF16 ? launch_gemv1<bf16, false>(a, s) : launch_gemv1<float, false>(a, s);
+}
+
 }  // namespace raven
 
 extern "C" int raven_gemv_fused(const void* x0, const void* x1, const void* norm_a, const void* norm_b, void* xa_out,
@@ -272,6 +299,7 @@ extern "C" int raven_gemv_fused(const void* x0, const void* x1, const void* norm
     Gemv1Args a{};
     a.w = w; a.x0 = x0; a.x1 = x1; a.norm_a = norm_a; a.norm_b = norm_b; a.xa_out = xa_out;
     a.residual = residual; a.y = y; a.N = N; a.K = K0 + K1; a.k0 = K0; a.out_f32 = out_f32; a.eps = eps;
+    a.ldw = a.K;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == RAVEN_BF16) return swiglu ? launch_gemv1<bf16, true>(a, s) : launch_gemv1<bf16, false>(a, s);
     return swiglu ? launch_gemv1<float, true>(a, s) : launch_gemv1<float, false>(a, s);

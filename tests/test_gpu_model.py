@@ -380,8 +380,11 @@ def test_generate_speculative_matches_oracle(pkg, small242, B, draft_steps, L, v
 
 @pytest.mark.parametrize("dt,B", [(torch.float32, 1), (torch.bfloat16, 1), (torch.bfloat16, 3), (torch.float32, 6)])
 def test_core_iterations_equal_single_iterations(pkg, tiny32, tiny16, dt, B):
-    """raven_core_iterations (all recurrences in one call; for one row the closing norm rides in the next adapter
-    product) gives the bits of the same recurrences called one by one, and leaves the same cache."""
+    """raven_core_iterations (all recurrences in one call) against the same recurrences called one by one.  Several rows:
+    the same bits and the same cache.  One row: the closing norm rides in the next adapter product and the embedding
+    half of that product is summed once for all recurrences, in fp32, entering the accumulator before the product's one
+    rounding; only the order of the fp32 additions differs, so the results agree to rounding (rel-L2 1e-5 in fp32, the
+    per-kernel bar of 1e-2 in bf16), and so do the cache entries."""
     s, w, model = tiny32 if dt == torch.float32 else tiny16
     nat, t = model._natives(), model.transformer
     n_core, r, T, h = len(t.core_block), 3, 9, s.n_embd
@@ -403,8 +406,17 @@ def test_core_iterations_equal_single_iterations(pkg, tiny32, tiny16, dt, B):
         pkg.hip.core_iteration(nat["dims"], t.adapter.weight, nat["core"], x, emb, one, nat["freqs"], caches[1][2], slots[it][0], B, 1, T, ws,
                                ln_f=t.ln_f.weight if it == r - 1 else None)
         x = one.clone()
-    assert torch.equal(many, one)
-    assert torch.equal(caches[0][0], caches[1][0]) and torch.equal(caches[0][1], caches[1][1])
+    if B > 1:
+        assert torch.equal(many, one)
+        assert torch.equal(caches[0][0], caches[1][0]) and torch.equal(caches[0][1], caches[1][1])
+    else:
+        tol = 1e-5 if dt == torch.float32 else 1e-2
+        assert close(many, one, "state")[1] <= tol
+        assert close(caches[0][0], caches[1][0], "keys")[1] <= tol and close(caches[0][1], caches[1][1], "values")[1] <= tol
+        # a single recurrence takes the unsplit product: the same bits as raven_core_iteration
+        pkg.hip.core_iterations(nat["dims"], t.adapter.weight, nat["core"], state, emb, many, nat["freqs"], caches[0][2], slots[:1], B, 1, T, ws)
+        pkg.hip.core_iteration(nat["dims"], t.adapter.weight, nat["core"], state, emb, one, nat["freqs"], caches[1][2], 0, B, 1, T, ws)
+        assert torch.equal(many, one)
     with pytest.raises(pkg.hip.RavenHipError):
         pkg.hip.core_iterations(nat["dims"], t.adapter.weight, nat["core"], state, emb, many, nat["freqs"], caches[0][2], [[0]], B, 1, T, ws)
 
