@@ -22,9 +22,12 @@ namespace raven {
 int gemv1_column_block(const void* x, const void* norm_a, const void* w_block, int ldw, const float* acc_in, void* y, int raw_out,
                        int N, int K, float eps, int dtype, hipStream_t s);
 
+int linear_column_block(const void* x, const void* w_block, int ldw, const float* extra, void* y, int raw_out, int M, int N, int K,
+                        void* workspace, size_t workspace_bytes, hipStream_t s);
+
 struct BlockScratch {
     char *n1, *qkv, *q, *ya, *x1, *x2, *n3, *g, *x3, *xa, *xr;
-    float* e_sums;  // one row: fp32 sums of the adapter's embedding half, computed once for all recurrences
+    float* e_sums;  // up to 32 rows: fp32 sums of the adapter's embedding half, computed once for all recurrences
     void* attn_ws;
     size_t attn_ws_bytes;
     void* lin_ws;
@@ -52,7 +55,7 @@ static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
     s.x3 = take(row);
     s.xa = take(row);
     s.xr = take(row);
-    s.e_sums = reinterpret_cast<float*>(take(M == 1 ? (size_t)d->n_embd * sizeof(float) : 0));
+    s.e_sums = reinterpret_cast<float*>(take(M <= 32 ? (size_t)M * d->n_embd * sizeof(float) : 0));
     s.attn_ws_bytes = raven_decode_attention_workspace_bytes(M, d->n_heads, d->head_dim);
     s.attn_ws = s.attn_ws_bytes ? take(s.attn_ws_bytes) : nullptr;
     const int widest = 3 * d->n_embd > 2 * d->intermediate ? 3 * d->n_embd : 2 * d->intermediate;
@@ -218,12 +221,20 @@ extern "C" int raven_core_iterations(const raven_dims* dims, const void* adapter
         }
         return close_one_row(dims, s, last_blk.norm_4, ln_f, state_out, stream);
     }
+    // 5..32 rows in bf16: the adapter is split by columns as for one row (embedding half summed once, in fp32)
+    const bool split = n_iterations >= 2 && dims->dtype == RAVEN_BF16 && M >= 5 && M <= 32 && h % 32 == 0 && h >= 256 && s.lin_ws;
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    if (split)
+        if ((rc = linear_column_block(embeds, static_cast<const char*>(adapter_w) + (size_t)h * 2, 2 * h, nullptr, s.e_sums, 1, M, h, h,
+                                      s.lin_ws, s.lin_ws_bytes, hs))) return rc;
     for (int it = 0; it < n_iterations; ++it) {
         const int32_t* sl = slots + (size_t)it * n_blocks;
         const bool last_it = it == n_iterations - 1;
         // the adapter product consumes the state before the last block of this iteration overwrites state_out
-        if ((rc = raven_linear(it == 0 ? state_in : state_out, embeds, adapter_w, nullptr, s.xa, M, h, h, h, 0, 0, dims->dtype, s.lin_ws,
-                               s.lin_ws_bytes, stream))) return rc;
+        const void* st = it == 0 ? state_in : state_out;
+        if (split) rc = linear_column_block(st, adapter_w, 2 * h, s.e_sums, s.xa, 0, M, h, h, s.lin_ws, s.lin_ws_bytes, hs);
+        else rc = raven_linear(st, embeds, adapter_w, nullptr, s.xa, M, h, h, h, 0, 0, dims->dtype, s.lin_ws, s.lin_ws_bytes, stream);
+        if (rc) return rc;
         const void* lnw = last_it ? ln_f : nullptr;
         for (int j = 0; j < n_blocks; ++j) {
             const bool last = j == n_blocks - 1;

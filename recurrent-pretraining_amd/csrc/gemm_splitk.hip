@@ -40,6 +40,9 @@ struct NsArgs {
     int out_f32, ks;
     int row_stride;        // 1 = a tile is 16 neighbouring weight rows, 2 = every second row (rows of one parity)
     int line_aligned;      // the rows of a tile all start at the same offset inside a 128-byte line
+    int ldw;               // elements between two weight rows: K, or more for a column block of a wider matrix
+    const float* extra;    // [M, N] or null: fp32 sums of the remaining columns, added with the K-slice partials
+    int raw_out;           // y receives the unrounded fp32 sums (what `extra` of a later call holds)
 };
 
 template <bool SWIGLU>
@@ -63,7 +66,7 @@ __global__ __launch_bounds__(256) void mfma_ns_kernel(NsArgs a) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ln = lane & 15, kq = lane >> 4;
     const int lr = lane >> 4, lc = (lane & 15) * 8;  // loader role inside a wave: row of a group of 4, first element of the chunk
-    const int K = a.K;
+    const int K = a.ldw;  // row pitch of W
 
     // this wave's weight tile(s): row i of the tile is tile_row0 + i * rs, its output column out0 + i * rs
     const int rs = a.row_stride;
@@ -222,13 +225,14 @@ __global__ __launch_bounds__(256) void splitk_finalize_kernel(NsArgs a) {
     if (idx >= (int64_t)a.M * a.N) return;
     const int m = (int)(idx / a.N), n = (int)(idx - (int64_t)m * a.N);
     const int n_total = SWIGLU ? 2 * a.N : a.N;
-    float v0 = 0.f, v1 = 0.f;
+    float v0 = a.extra ? a.extra[idx] : 0.f, v1 = 0.f;
     for (int s = 0; s < a.ks; ++s) {
         const float* p = a.partial + ((int64_t)s * a.M + m) * n_total;
         v0 += p[n];
         if (SWIGLU) v1 += p[a.N + n];
     }
-    ns_epilogue<SWIGLU>(a, m, n, v0, v1);
+    if (a.raw_out) static_cast<float*>(a.y)[idx] = v0;
+    else ns_epilogue<SWIGLU>(a, m, n, v0, v1);
 }
 
 static int ns_cus() {
@@ -247,8 +251,9 @@ int g_linear_ks = 0;  // raven_set_tuning("linear_ks"): K slices per weight tile
 template <bool SWIGLU>
 static int launch_ns(NsArgs a, void* workspace, size_t workspace_bytes, hipStream_t s) {
     // tiles of one row parity when the row pitch is an odd multiple of 64 bytes (needs whole pairs of tiles)
-    a.row_stride = ((a.K * 2) % 128 == 64 && a.N % 32 == 0) ? 2 : 1;
-    a.line_aligned = (a.K * 2 * a.row_stride) % 128 == 0;
+    if (a.ldw == 0) a.ldw = a.K;
+    a.row_stride = ((a.ldw * 2) % 128 == 64 && a.N % 32 == 0) ? 2 : 1;
+    a.line_aligned = (a.ldw * 2 * a.row_stride) % 128 == 0;
     const int rs = a.row_stride;
     const int blocks = (a.N / 16 + 4 * rs - 1) / (4 * rs) * rs;
     const int n_mac = a.k0 / 128 + a.k1 / 128;
@@ -259,6 +264,13 @@ static int launch_ns(NsArgs a, void* workspace, size_t workspace_bytes, hipStrea
     if (ks > 8) ks = 8;
     if (ks < 1) ks = 1;
     while (ks > 1 && (size_t)ks * a.M * n_total * sizeof(float) > workspace_bytes) --ks;
+    if ((a.extra || a.raw_out) && ks < 2) {  // those go through the second launch
+        ks = 2;
+        if (n_mac < 2 || (size_t)ks * a.M * n_total * sizeof(float) > workspace_bytes) {
+            raven_host::set_error("linear: a column block needs two K slices (K=%d) and their workspace", a.K);
+            return -1;
+        }
+    }
     a.ks = ks;
     a.partial = ks > 1 ? static_cast<float*>(workspace) : nullptr;
     const dim3 grid(blocks, ks);
@@ -269,6 +281,24 @@ static int launch_ns(NsArgs a, void* workspace, size_t workspace_bytes, hipStrea
         splitk_finalize_kernel<SWIGLU><<<dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s>>>(a);
     }
     return raven_host::check_launch("linear (split-K MFMA)");
+}
+
+// Column block [c0, c0 + K) of a wider bf16 weight matrix with row pitch ldw, for 5..32 rows:
+// y = round(x W[:, c0 : c0 + K]^T + extra), or the unrounded fp32 sums (raw_out) that a later call takes as `extra`.
+// The adapter product over [state, embedding] (recpre/raven_modeling_minimal.py:776) is split with it when the
+// embedding half stays the same over many calls; the product keeps its single rounding.
+int linear_column_block(const void* x, const void* w_block, int ldw, const float* extra, void* y, int raw_out, int M, int N, int K,
+                        void* workspace, size_t workspace_bytes, hipStream_t s) {
+    if (M < 5 || M > 32 || N % 16 || K % 32 || K < 256 || !workspace || ((uintptr_t)workspace & 255)) {
+        raven_host::set_error("linear_column_block: unsupported shape M=%d N=%d K=%d", M, N, K);
+        return -1;
+    }
+    NsArgs a{};
+    a.w = static_cast<const bf16*>(w_block);
+    a.x0 = static_cast<const bf16*>(x);
+    a.y = y;
+    a.M = M; a.N = N; a.K = K; a.k0 = K; a.k1 = 0; a.ldw = ldw; a.extra = extra; a.raw_out = raw_out;
+    return launch_ns<false>(a, workspace, workspace_bytes, s);
 }
 
 }  // namespace raven
