@@ -39,6 +39,8 @@ def parse():
     ap.add_argument("--also-batch", type=int, default=32, help="second batch size reported under 'also' (0 = skip)")
     ap.add_argument("--adaptive", action="store_true",
                     help="per-token adaptive compute at bs=1 with a fixed cycle of recurrences per token (a next-row measurement)")
+    ap.add_argument("--paged", action="store_true",
+                    help="decode over block-paged caches, --batch sequences of different lengths around --prompt (a next-row measurement)")
     ap.add_argument("--prefill", action="store_true",
                     help="measure the recurrent core over a whole prompt instead (bs=4 x 4096 tokens, r iterations): MFMA-bound regime")
     ap.add_argument("--prefill-batch", type=int, default=4)
@@ -148,6 +150,63 @@ def adaptive(args):
     print(json.dumps(line))
 
 
+def paged(args):
+    """Decode steps over block-paged caches (one per flat layer, 16 positions per block, shuffled block tables), the
+    sequences of the batch at different lengths drawn uniformly from [prompt / 2, 3 prompt / 2].  The pages hold
+    synthetic keys and values (N(0, 1)); every step appends one position per sequence and feeds back the greedy token."""
+    import torch
+    import __graft_entry__ as entry
+    pkg = entry.import_package()
+    pkg.hip.load()
+    dev = torch.device("cuda:0")
+    cfg = pkg.RavenConfig()
+    model = pkg.RavenForCausalLM(cfg, device=dev, dtype=torch.bfloat16)
+    fill_synthetic(model, 0)
+    B, bs, r = args.batch, 16, args.recurrence
+    g = torch.Generator().manual_seed(1)
+    lens = torch.randint(args.prompt // 2, args.prompt * 3 // 2 + 1, (B,), generator=g, dtype=torch.int32)
+    total = args.steps + args.warmup
+    max_blocks = (int(lens.max()) + total + bs - 1) // bs
+    n_blocks = B * max_blocks
+    table = torch.randperm(n_blocks, generator=g).view(B, max_blocks).to(torch.int32).to(dev)
+    dec = pkg.PagedDecoder(model, num_blocks=n_blocks, block_size=bs, num_steps=r)
+    for t in dec.k + dec.v:
+        t.normal_(0.0, 1.0)
+    ids = torch.randint(0, cfg.vocab_size, (B,), generator=g).to(dev)
+    seq_lens = (lens + 1).to(dev)
+    nxt = torch.zeros(B, dtype=torch.int64, device=dev)
+    state = torch.zeros(B, cfg.n_embd, dtype=torch.bfloat16, device=dev)
+
+    def one():
+        state.normal_(0.0, 0.632)  # a fresh latent state per token, as the reference draws it (scale of its default initialisation)
+        logits, _ = dec.step(ids, table, seq_lens, input_states=state)
+        pkg.hip.argmax(logits, out=nxt)
+        ids.copy_(nxt)
+        seq_lens.add_(1)
+
+    for _ in range(args.warmup):
+        one()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        one()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    mean_len = float(lens.float().mean()) + args.warmup + args.steps / 2
+    n_flat, core = dec.n_flat, cfg.n_layers_in_recurrent_block
+    kv_bytes = B * mean_len * cfg.n_embd * 2 * 2 * (n_flat - core + core * r)  # K and V of every attention call of a step
+    line = {
+        "metric": "paged-KV decode, raven-3.5b shape bf16: tokens/s over sequences of different lengths",
+        "value": round(B * args.steps / dt, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(dt / args.steps * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"PagedDecoder.step, nebel-raven-3.5b shape, r={r}, {B} sequences, lengths {int(lens.min())}..{int(lens.max())} "
+                               f"(mean {float(lens.float().mean()):.0f}), block size {bs}, eager launches", "batch": B, "recurrence": r},
+        "kv_GB_per_step": round(kv_bytes / 1e9, 2),
+    }
+    print(json.dumps(line))
+
+
 def kernel_only(n_launches):
     """The dominant kernel alone, as the decode loop launches it, on four rotating fc matrices, followed by
     one device copy of known size (the yardstick that scales FETCH_SIZE / WRITE_SIZE readings)."""
@@ -238,6 +297,9 @@ def main():
         return
     if args.adaptive:
         adaptive(args)
+        return
+    if args.paged:
+        paged(args)
         return
     if args.gpus != 1:
         print("bench.py measures one GPU: the decode path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)

@@ -154,13 +154,42 @@ int raven_exit_latent_stats(const void* latents, const void* prev, void* rel_cha
  *   slot_mapping[t] = block * block_size + offset (negative: skipped).
  * raven_paged_decode_attention: one query row per sequence, q / y [B, n_heads * head_dim]; sequence b attends to its
  *   first seq_lens[b] positions (its own new token included; 0 gives zeros).  max_seq_len >= every seq_lens[b] sizes the
- *   launch.  workspace as for raven_decode_attention (raven_decode_attention_workspace_bytes(B, ...)). */
+ *   launch.  workspace as for raven_decode_attention (raven_decode_attention_workspace_bytes(B, ...)).
+ * raven_paged_qkv_attention_decode: the whole decode step of the plugin's attention layer in one launch
+ *   (vllm/raven_vllm.py:186-201: split, q/k bias, RoPE, cache write, attention): qkv [B, 3 * n_heads * head_dim] is the
+ *   fused projection's output, qk_bias [2, n_heads, head_dim] or NULL, freqs the (cos, sin) table; sequence b's new
+ *   token sits at position seq_lens[b] - 1: its rotated k and its v are written to that position's page and the row
+ *   attends to positions 0..seq_lens[b] - 1 (seq_lens[b] = 0: nothing written, zeros returned). */
 int raven_paged_kv_append(const void* k, const void* v, void* k_cache, void* v_cache, const int64_t* slot_mapping,
                           int32_t T, int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream);
 int raven_paged_decode_attention(const void* q, void* y, const void* k_cache, const void* v_cache,
                                  const int32_t* block_table, const int32_t* seq_lens, int32_t B, int32_t max_blocks,
                                  int32_t block_size, int32_t max_seq_len, int32_t n_heads, int32_t head_dim,
                                  int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
+int raven_paged_qkv_attention_decode(const void* qkv, const void* qk_bias, const float* freqs, void* y, void* k_cache,
+                                     void* v_cache, const int32_t* block_table, const int32_t* seq_lens, int32_t B,
+                                     int32_t max_blocks, int32_t block_size, int32_t max_seq_len, int32_t n_heads,
+                                     int32_t head_dim, int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* A stack of SandwichBlocks over block-paged caches, one decode row per sequence (the flat layer list the plugin's
+ * model runs, vllm/raven_vllm.py:365-432: every flat layer owns ONE paged cache, which the recurrences of a token
+ * overwrite in turn, so older positions hold their last recurrence).  k_caches / v_caches: HOST arrays of n_blocks
+ * device pointers, block j's cache [num_blocks, block_size, n_heads, head_dim]; block_table [B, max_blocks] and
+ * seq_lens [B] (new token included) in device memory, shared by all blocks.
+ * adapter_w / embeds non-NULL: n_iterations x (adapter([x, embeds]) then the blocks), i.e. the recurrent core;
+ * both NULL: the blocks once (prelude, coda).  ln_f non-NULL: applied to the result.  x_in, embeds, x_out [B, h].
+ * workspace: raven_block_workspace_bytes(dims, B). */
+typedef struct raven_paged_kv {
+    void* const* k_caches;
+    void* const* v_caches;
+    const int32_t* block_table;
+    const int32_t* seq_lens;
+    int32_t max_blocks, block_size, max_seq_len;
+} raven_paged_kv;
+int raven_paged_decode_blocks(const raven_dims* dims, const void* adapter_w, const raven_block_weights* blocks,
+                              int32_t n_blocks, const void* ln_f, const void* x_in, const void* embeds, void* x_out,
+                              const float* freqs, const raven_paged_kv* kv, int32_t n_iterations, int32_t B,
+                              void* workspace, size_t workspace_bytes, void* stream);
 
 /* Decode fast path for ONE token row, one launch:
  *     x  = norm_a ? T(rmsnorm(x0) * norm_a) : x0      -> stored to xa_out when non-NULL

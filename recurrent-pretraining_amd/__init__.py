@@ -29,11 +29,12 @@ from .modeling import (  # noqa: F401
     RavenForCausalLM,
     precompute_freqs_cis,
 )
+from .paged import PagedDecoder  # noqa: F401
 
 __all__ = [
     "hip", "HuginnDynamicCache", "HuginnStaticCache", "remap_step", "RavenConfig", "RavenForCausalLM", "DecodeRunner",
     "CausalLMOutputRecurrentLatents", "GenerationSettings", "precompute_freqs_cis", "adaptive", "vllm_binding",
     "PerIterationExitEvaluator", "NoOpExitEvaluator", "EntropyDiffExitEvaluator", "LatentDiffExitEvaluator",
     "KLExitEvaluator", "MinKLExitEvaluator", "ArgmaxStabilityExitEvaluator", "CosineExitEvaluator", "NumStepsGenerator",
-    "get_adaptive_exit_evaluator",
+    "get_adaptive_exit_evaluator", "PagedDecoder",
 ]

@@ -345,8 +345,12 @@ struct PagedView {
     int max_blocks, block_size, nh, hd;
 };
 
-template <typename T, int CPL>
-__global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __restrict__ q, T* __restrict__ y, PagedView pv,
+// FUSED: q_or_qkv is the fused projection's output [B, 3 * h]; bias and RoPE (row seq_lens[b] - 1 of the table) are
+// applied here, the new position's k / v row is written to its page by the workgroup whose range holds it and used
+// from registers (the paged counterpart of decode_attention_kernel<FUSED>).
+template <typename T, int CPL, bool FUSED = false>
+__global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __restrict__ q_or_qkv, const T* __restrict__ qk_bias,
+                                                                     const float* __restrict__ freqs, T* __restrict__ y, PagedView pv,
                                                                      float scale_log2, int n_splits, float* __restrict__ ws_ml,
                                                                      float* __restrict__ ws_o) {
     constexpr int EC = Chunk<T>::N, E = EC * CPL, G = 16, U = 2;
@@ -365,7 +369,27 @@ __global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __
     const int* table = pv.block_table + (int64_t)b * pv.max_blocks;
     const T* K = static_cast<const T*>(pv.k);
     const T* V = static_cast<const T*>(pv.v);
-    const P qc = active ? load_piece<T, CPL>(q + (int64_t)b * h + head * hd + ci * E) : zero_piece<T, CPL>();
+    const int col = head * hd + ci * E;
+    const int pos = len - 1;  // FUSED: the new token's position
+    P qc = zero_piece<T, CPL>(), knew = zero_piece<T, CPL>(), vnew = zero_piece<T, CPL>();
+    if (active && !FUSED) qc = load_piece<T, CPL>(q_or_qkv + (int64_t)b * h + col);
+    if (FUSED && active && len > 0) {
+        const T* row = q_or_qkv + (int64_t)b * 3 * h;
+        qc = load_piece<T, CPL>(row + col);
+        knew = load_piece<T, CPL>(row + h + col);
+        vnew = load_piece<T, CPL>(row + 2 * h + col);
+#pragma unroll
+        for (int i = 0; i < CPL; ++i) {
+            qc.c[i] = bias_rope_chunk<T>(qc.c[i], qk_bias, 0, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
+            knew.c[i] = bias_rope_chunk<T>(knew.c[i], qk_bias, 1, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
+        }
+        if (group == 0 && pos >= start && pos < end) {
+            const int64_t row_new = (int64_t)table[pos / pv.block_size] * pv.block_size + pos % pv.block_size;
+            const int64_t off = (row_new * pv.nh + head) * hd + ci * E;
+            store_piece<T, CPL>(const_cast<T*>(K) + off, knew);
+            store_piece<T, CPL>(const_cast<T*>(V) + off, vnew);
+        }
+    }
 
     float m_run = -INFINITY, l_run = 0.f, o[E];
 #pragma unroll
@@ -375,7 +399,10 @@ __global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __
 #pragma unroll
         for (int j = 0; j < U; ++j) {
             const int p = base + j * G + group;
-            if (active && p < end) {
+            if (FUSED && p == pos) {
+                kc[j] = knew;
+                vc[j] = vnew;
+            } else if (active && p < end) {
                 const int64_t row = (int64_t)table[p / pv.block_size] * pv.block_size + p % pv.block_size;
                 const int64_t off = (row * pv.nh + head) * hd + ci * E;
                 kc[j] = load_piece<T, CPL, true>(K + off);
@@ -631,16 +658,17 @@ extern "C" int raven_paged_kv_append(const void* k, const void* v, void* k_cache
     return raven_host::check_launch("paged_kv_append");
 }
 
-extern "C" int raven_paged_decode_attention(const void* q, void* y, const void* k_cache, const void* v_cache,
-                                            const int32_t* block_table, const int32_t* seq_lens, int32_t B, int32_t max_blocks,
-                                            int32_t block_size, int32_t max_seq_len, int32_t n_heads, int32_t head_dim, int32_t dtype,
-                                            void* workspace, size_t workspace_bytes, void* stream) {
+static int paged_attention_common(const char* who, bool fused, const void* q, const void* bias, const float* freqs, void* y,
+                                  const void* k_cache, const void* v_cache, const int32_t* block_table, const int32_t* seq_lens,
+                                  int32_t B, int32_t max_blocks, int32_t block_size, int32_t max_seq_len, int32_t n_heads,
+                                  int32_t head_dim, int32_t dtype, void* workspace, size_t workspace_bytes, void* stream) {
     using namespace raven;
-    if (int rc = check_heads("paged_decode_attention", n_heads, head_dim, dtype)) return rc;
-    RAVEN_REQUIRE(B >= 0 && B <= 65535 && max_blocks > 0 && block_size > 0 && max_seq_len > 0, "paged_decode_attention: bad B=%d max_blocks=%d block_size=%d max_seq_len=%d", B, max_blocks, block_size, max_seq_len);
+    if (int rc = check_heads(who, n_heads, head_dim, dtype)) return rc;
+    RAVEN_REQUIRE(B >= 0 && B <= 65535 && max_blocks > 0 && block_size > 0 && max_seq_len > 0, "%s: bad B=%d max_blocks=%d block_size=%d max_seq_len=%d", who, B, max_blocks, block_size, max_seq_len);
     if (B == 0) return 0;
-    RAVEN_REQUIRE(q && y && k_cache && v_cache && block_table && seq_lens, "paged_decode_attention: null pointer");
-    RAVEN_REQUIRE((int64_t)max_blocks * block_size >= max_seq_len, "paged_decode_attention: %d blocks of %d cannot hold %d positions", max_blocks, block_size, max_seq_len);
+    RAVEN_REQUIRE(q && y && k_cache && v_cache && block_table && seq_lens, "%s: null pointer", who);
+    RAVEN_REQUIRE(!fused || freqs, "%s: null RoPE table", who);
+    RAVEN_REQUIRE((int64_t)max_blocks * block_size >= max_seq_len, "%s: %d blocks of %d cannot hold %d positions", who, max_blocks, block_size, max_seq_len);
     int ns = splits_for(B, n_heads, max_seq_len);
     float *ws_ml = nullptr, *ws_o = nullptr;
     if (ns > 1) {
@@ -648,7 +676,7 @@ extern "C" int raven_paged_decode_attention(const void* q, void* y, const void* 
         if (workspace == nullptr || workspace_bytes < need) {
             ns = 1;
         } else {
-            RAVEN_REQUIRE(((uintptr_t)workspace & 255) == 0, "paged_decode_attention: workspace must be 256-byte aligned");
+            RAVEN_REQUIRE(((uintptr_t)workspace & 255) == 0, "%s: workspace must be 256-byte aligned", who);
             ws_ml = static_cast<float*>(workspace);
             ws_o = reinterpret_cast<float*>(static_cast<char*>(workspace) + raven_host::align_up((size_t)B * n_heads * kAttnMaxSplits * 2 * 4));
         }
@@ -657,13 +685,35 @@ extern "C" int raven_paged_decode_attention(const void* q, void* y, const void* 
     const float scale_log2 = (float)(1.0 / sqrt((double)head_dim) * 1.4426950408889634);
     const dim3 grid(n_heads, B, ns);
     hipStream_t s = static_cast<hipStream_t>(stream);
+#define RAVEN_PAGED_LAUNCH(T_, CPL_)                                                                                            \
+    do {                                                                                                                        \
+        if (fused) paged_decode_attention_kernel<T_, CPL_, true><<<grid, dim3(256), 0, s>>>((const T_*)q, (const T_*)bias, freqs, (T_*)y, pv, scale_log2, ns, ws_ml, ws_o); \
+        else paged_decode_attention_kernel<T_, CPL_, false><<<grid, dim3(256), 0, s>>>((const T_*)q, nullptr, nullptr, (T_*)y, pv, scale_log2, ns, ws_ml, ws_o); \
+    } while (0)
     if (dtype == RAVEN_BF16) {
-        paged_decode_attention_kernel<bf16, 1><<<grid, dim3(256), 0, s>>>((const bf16*)q, (bf16*)y, pv, scale_log2, ns, ws_ml, ws_o);
+        RAVEN_PAGED_LAUNCH(bf16, 1);
         if (ns > 1) attention_combine_kernel<bf16><<<dim3(n_heads, B), dim3(128), 0, s>>>(ws_ml, ws_o, (bf16*)y, n_heads, head_dim, ns);
     } else {
-        if (head_dim / 4 > 16) paged_decode_attention_kernel<float, 2><<<grid, dim3(256), 0, s>>>((const float*)q, (float*)y, pv, scale_log2, ns, ws_ml, ws_o);
-        else paged_decode_attention_kernel<float, 1><<<grid, dim3(256), 0, s>>>((const float*)q, (float*)y, pv, scale_log2, ns, ws_ml, ws_o);
+        if (head_dim / 4 > 16) RAVEN_PAGED_LAUNCH(float, 2);
+        else RAVEN_PAGED_LAUNCH(float, 1);
         if (ns > 1) attention_combine_kernel<float><<<dim3(n_heads, B), dim3(128), 0, s>>>(ws_ml, ws_o, (float*)y, n_heads, head_dim, ns);
     }
-    return raven_host::check_launch("paged_decode_attention");
+#undef RAVEN_PAGED_LAUNCH
+    return raven_host::check_launch(who);
+}
+
+extern "C" int raven_paged_decode_attention(const void* q, void* y, const void* k_cache, const void* v_cache,
+                                            const int32_t* block_table, const int32_t* seq_lens, int32_t B, int32_t max_blocks,
+                                            int32_t block_size, int32_t max_seq_len, int32_t n_heads, int32_t head_dim, int32_t dtype,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+    return paged_attention_common("paged_decode_attention", false, q, nullptr, nullptr, y, k_cache, v_cache, block_table, seq_lens, B,
+                                  max_blocks, block_size, max_seq_len, n_heads, head_dim, dtype, workspace, workspace_bytes, stream);
+}
+
+extern "C" int raven_paged_qkv_attention_decode(const void* qkv, const void* qk_bias, const float* freqs, void* y, void* k_cache,
+                                                void* v_cache, const int32_t* block_table, const int32_t* seq_lens, int32_t B,
+                                                int32_t max_blocks, int32_t block_size, int32_t max_seq_len, int32_t n_heads,
+                                                int32_t head_dim, int32_t dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    return paged_attention_common("paged_qkv_attention_decode", true, qkv, qk_bias, freqs, y, k_cache, v_cache, block_table, seq_lens,
+                                  B, max_blocks, block_size, max_seq_len, n_heads, head_dim, dtype, workspace, workspace_bytes, stream);
 }

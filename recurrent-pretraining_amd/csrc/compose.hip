@@ -91,13 +91,18 @@ static bool one_row_fits(const raven_dims* d) {
 // result is wanted.
 static int run_block(const raven_dims* d, const raven_block_weights* w, const BlockScratch& s, bool n1_ready,
                      const void* x_in, void* y_out, const void* tail_w, void* tail_out, const float* freqs,
-                     const raven_kv_cache* cache, int slot, int B, int S, int pos0, const int32_t* pos_dev, void* stream) {
+                     const raven_kv_cache* cache, int slot, int B, int S, int pos0, const int32_t* pos_dev, void* stream,
+                     const raven_paged_kv* paged = nullptr, int layer = 0) {
     const int M = B * S, h = d->n_embd, I = d->intermediate, dt = d->dtype;
     int rc;
     if (!n1_ready)
         if ((rc = raven_rmsnorm_residual(x_in, nullptr, w->norm_1, s.n1, nullptr, nullptr, nullptr, M, h, d->eps, dt, stream))) return rc;
     if ((rc = raven_linear(s.n1, nullptr, w->wqkv, nullptr, s.qkv, M, 3 * h, h, 0, 0, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
-    if (S == 1) {  // decode: bias, RoPE, cache append and attention in one launch
+    if (paged) {   // decode over block-paged caches, every sequence at its own position
+        if ((rc = raven_paged_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, paged->k_caches[layer], paged->v_caches[layer],
+                                                   paged->block_table, paged->seq_lens, B, paged->max_blocks, paged->block_size,
+                                                   paged->max_seq_len, d->n_heads, d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream))) return rc;
+    } else if (S == 1) {  // decode: bias, RoPE, cache append and attention in one launch
         if ((rc = raven_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, cache, slot, B, pos0, pos_dev, d->n_heads,
                                              d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream))) return rc;
     } else {       // a chunk of S tokens: every row's keys must be in the cache before any row attends
@@ -117,7 +122,7 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
 // the input itself).  Leaves the block output BEFORE its norm_4 in scratch.x3.
 static int run_block_one_row(const raven_dims* d, const raven_block_weights* w, const BlockScratch& s, const void* x_raw,
                              const void* pre_norm, const float* freqs, const raven_kv_cache* cache, int slot, int pos0,
-                             const int32_t* pos_dev, void* stream) {
+                             const int32_t* pos_dev, void* stream, const raven_paged_kv* paged = nullptr, int layer = 0) {
     const int h = d->n_embd, I = d->intermediate, dt = d->dtype;
     const float eps = d->eps;
     int rc;
@@ -128,8 +133,14 @@ static int run_block_one_row(const raven_dims* d, const raven_block_weights* w, 
     } else {
         if ((rc = raven_gemv_fused(x_raw, nullptr, w->norm_1, nullptr, nullptr, w->wqkv, nullptr, s.qkv, 3 * h, h, 0, eps, 0, 0, dt, stream))) return rc;
     }
-    if ((rc = raven_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, cache, slot, 1, pos0, pos_dev, d->n_heads, d->head_dim, dt,
-                                         s.attn_ws, s.attn_ws_bytes, stream))) return rc;
+    if (paged)
+        rc = raven_paged_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, paged->k_caches[layer], paged->v_caches[layer],
+                                              paged->block_table, paged->seq_lens, 1, paged->max_blocks, paged->block_size,
+                                              paged->max_seq_len, d->n_heads, d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream);
+    else
+        rc = raven_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, cache, slot, 1, pos0, pos_dev, d->n_heads, d->head_dim, dt,
+                                        s.attn_ws, s.attn_ws_bytes, stream);
+    if (rc) return rc;
     if ((rc = raven_gemv_fused(s.ya, nullptr, nullptr, nullptr, nullptr, w->proj, x_res, s.x1, h, h, 0, eps, 0, 0, dt, stream))) return rc;
     if ((rc = raven_gemv_fused(s.x1, nullptr, w->norm_2, w->norm_3, s.x2, w->fc, nullptr, s.g, I, h, 0, eps, 1, 0, dt, stream))) return rc;
     return raven_gemv_fused(s.g, nullptr, nullptr, nullptr, nullptr, w->mlp_proj, s.x2, s.x3, h, I, 0, eps, 0, 0, dt, stream);
@@ -170,26 +181,33 @@ extern "C" int raven_sandwich_block(const raven_dims* dims, const raven_block_we
     return run_block(dims, w, s, false, x_in, x_out, nullptr, nullptr, freqs, cache, slot, B, S, pos0, pos_dev, stream);
 }
 
-extern "C" int raven_core_iterations(const raven_dims* dims, const void* adapter_w, const raven_block_weights* blocks,
-                                     int32_t n_blocks, const void* ln_f, const void* state_in, const void* embeds,
-                                     void* state_out, const float* freqs, const raven_kv_cache* cache, const int32_t* slots,
-                                     int32_t n_iterations, int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
-                                     void* workspace, size_t workspace_bytes, void* stream) {
-    using namespace raven;
-    if (int rc = check_dims("core_iterations", dims)) return rc;
-    RAVEN_REQUIRE(adapter_w && state_in && embeds && state_out && freqs && slots, "core_iterations: null pointer");
-    RAVEN_REQUIRE(n_blocks >= 1 && blocks, "core_iterations: needs at least one block");
-    RAVEN_REQUIRE(n_iterations >= 1, "core_iterations: needs at least one iteration (got %d)", n_iterations);
-    RAVEN_REQUIRE(B > 0 && S > 0, "core_iterations: bad B=%d S=%d", B, S);
+namespace raven {
+
+// n_iterations x ([adapter product] + n_blocks blocks), the closing norm(s) at the end.  The K/V of block j live either
+// in slot slots[it * n_blocks + j] of a contiguous cache (all sequences at position pos0 / *pos_dev) or, with `paged`,
+// in the j-th block-paged cache (every sequence at its own position, the same cache in every iteration).
+static int iterations_impl(const char* who, const raven_dims* dims, const void* adapter_w, const raven_block_weights* blocks,
+                           int32_t n_blocks, const void* ln_f, const void* state_in, const void* embeds, void* state_out,
+                           const float* freqs, const raven_kv_cache* cache, const int32_t* slots, const raven_paged_kv* paged,
+                           int32_t n_iterations, int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+    if (int rc = check_dims(who, dims)) return rc;
+    RAVEN_REQUIRE(state_in && state_out && freqs && (slots || paged), "%s: null pointer", who);
+    RAVEN_REQUIRE((adapter_w == nullptr) == (embeds == nullptr), "%s: the adapter weight and its second input come together", who);
+    RAVEN_REQUIRE(n_blocks >= 1 && blocks, "%s: needs at least one block", who);
+    RAVEN_REQUIRE(n_iterations >= 1, "%s: needs at least one iteration (got %d)", who, n_iterations);
+    RAVEN_REQUIRE(adapter_w || n_iterations == 1, "%s: several iterations need the adapter", who);
+    RAVEN_REQUIRE(B > 0 && S > 0, "%s: bad B=%d S=%d", who, B, S);
     for (int j = 0; j < n_blocks; ++j)
-        if (int rc = check_block_weights("core_iterations", &blocks[j])) return rc;
+        if (int rc = check_block_weights(who, &blocks[j])) return rc;
     const int M = B * S, h = dims->n_embd;
     const size_t need = carve(dims, M, nullptr, nullptr);
-    RAVEN_REQUIRE(workspace && workspace_bytes >= need, "core_iterations: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-    RAVEN_REQUIRE(((uintptr_t)workspace & 255) == 0, "core_iterations: workspace must be 256-byte aligned");
+    RAVEN_REQUIRE(workspace && workspace_bytes >= need, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+    RAVEN_REQUIRE(((uintptr_t)workspace & 255) == 0, "%s: workspace must be 256-byte aligned", who);
     BlockScratch s;
     carve(dims, M, static_cast<char*>(workspace), &s);
     const raven_block_weights& last_blk = blocks[n_blocks - 1];
+    hipStream_t hs = static_cast<hipStream_t>(stream);
 
     int rc;
     if (M == 1 && one_row_fits(dims)) {
@@ -199,53 +217,82 @@ extern "C" int raven_core_iterations(const raven_dims* dims, const void* adapter
         // sums are formed once, and each recurrence streams the state half of the weight only.
         const bool split = n_iterations >= 2;
         const size_t es = raven_host::elt_size(dims->dtype);
-        hipStream_t hs = static_cast<hipStream_t>(stream);
         if (split)
             if ((rc = gemv1_column_block(embeds, nullptr, static_cast<const char*>(adapter_w) + (size_t)h * es, 2 * h, nullptr, s.e_sums,
                                          1, h, h, dims->eps, dims->dtype, hs))) return rc;
         for (int it = 0; it < n_iterations; ++it) {
-            const int32_t* sl = slots + (size_t)it * n_blocks;
+            const int32_t* sl = slots ? slots + (size_t)it * n_blocks : nullptr;
             const void* x_in = it == 0 ? state_in : (const void*)s.x3;
             const void* pre_norm = it == 0 ? nullptr : last_blk.norm_4;
-            if (split)
-                rc = gemv1_column_block(x_in, pre_norm, adapter_w, 2 * h, s.e_sums, s.xa, 0, h, h, dims->eps, dims->dtype, hs);
-            else
-                rc = raven_gemv_fused(x_in, embeds, pre_norm, nullptr, nullptr, adapter_w, nullptr, s.xa, h, h, h, dims->eps, 0, 0,
-                                      dims->dtype, stream);
-            if (rc) return rc;
+            if (adapter_w) {
+                if (split)
+                    rc = gemv1_column_block(x_in, pre_norm, adapter_w, 2 * h, s.e_sums, s.xa, 0, h, h, dims->eps, dims->dtype, hs);
+                else
+                    rc = raven_gemv_fused(x_in, embeds, pre_norm, nullptr, nullptr, adapter_w, nullptr, s.xa, h, h, h, dims->eps, 0, 0,
+                                          dims->dtype, stream);
+                if (rc) return rc;
+            }
             for (int j = 0; j < n_blocks; ++j) {
-                const void* x_raw = j == 0 ? (const void*)s.xa : (const void*)s.x3;
+                const void* x_raw = j == 0 ? (adapter_w ? (const void*)s.xa : state_in) : (const void*)s.x3;
                 const void* pre = j == 0 ? nullptr : blocks[j - 1].norm_4;
-                if ((rc = run_block_one_row(dims, &blocks[j], s, x_raw, pre, freqs, cache, sl[j], pos0, pos_dev, stream))) return rc;
+                if ((rc = run_block_one_row(dims, &blocks[j], s, x_raw, pre, freqs, cache, sl ? sl[j] : 0, pos0, pos_dev, stream, paged, j)))
+                    return rc;
             }
         }
         return close_one_row(dims, s, last_blk.norm_4, ln_f, state_out, stream);
     }
     // 5..32 rows in bf16: the adapter is split by columns as for one row (embedding half summed once, in fp32)
-    const bool split = n_iterations >= 2 && dims->dtype == RAVEN_BF16 && M >= 5 && M <= 32 && h % 32 == 0 && h >= 256 && s.lin_ws;
-    hipStream_t hs = static_cast<hipStream_t>(stream);
+    const bool split = adapter_w && n_iterations >= 2 && dims->dtype == RAVEN_BF16 && M >= 5 && M <= 32 && h % 32 == 0 && h >= 256 &&
+                       s.lin_ws;
     if (split)
         if ((rc = linear_column_block(embeds, static_cast<const char*>(adapter_w) + (size_t)h * 2, 2 * h, nullptr, s.e_sums, 1, M, h, h,
                                       s.lin_ws, s.lin_ws_bytes, hs))) return rc;
     for (int it = 0; it < n_iterations; ++it) {
-        const int32_t* sl = slots + (size_t)it * n_blocks;
+        const int32_t* sl = slots ? slots + (size_t)it * n_blocks : nullptr;
         const bool last_it = it == n_iterations - 1;
         // the adapter product consumes the state before the last block of this iteration overwrites state_out
         const void* st = it == 0 ? state_in : state_out;
-        if (split) rc = linear_column_block(st, adapter_w, 2 * h, s.e_sums, s.xa, 0, M, h, h, s.lin_ws, s.lin_ws_bytes, hs);
-        else rc = raven_linear(st, embeds, adapter_w, nullptr, s.xa, M, h, h, h, 0, 0, dims->dtype, s.lin_ws, s.lin_ws_bytes, stream);
-        if (rc) return rc;
+        if (adapter_w) {
+            if (split) rc = linear_column_block(st, adapter_w, 2 * h, s.e_sums, s.xa, 0, M, h, h, s.lin_ws, s.lin_ws_bytes, hs);
+            else rc = raven_linear(st, embeds, adapter_w, nullptr, s.xa, M, h, h, h, 0, 0, dims->dtype, s.lin_ws, s.lin_ws_bytes, stream);
+            if (rc) return rc;
+        }
         const void* lnw = last_it ? ln_f : nullptr;
         for (int j = 0; j < n_blocks; ++j) {
             const bool last = j == n_blocks - 1;
+            const void* x_in = (j == 0 && !adapter_w) ? state_in : (const void*)s.xa;
             void* y_out = last ? (lnw ? nullptr : state_out) : s.xa;
             const void* tail_w = last ? lnw : blocks[j + 1].norm_1;
             void* tail_out = last ? (lnw ? state_out : nullptr) : s.n1;
-            if ((rc = run_block(dims, &blocks[j], s, j > 0, s.xa, y_out, tail_w, tail_out, freqs, cache, sl[j], B, S, pos0, pos_dev,
-                                stream))) return rc;
+            if ((rc = run_block(dims, &blocks[j], s, j > 0, x_in, y_out, tail_w, tail_out, freqs, cache, sl ? sl[j] : 0, B, S, pos0,
+                                pos_dev, stream, paged, j))) return rc;
         }
     }
     return 0;
+}
+
+}  // namespace raven
+
+extern "C" int raven_core_iterations(const raven_dims* dims, const void* adapter_w, const raven_block_weights* blocks,
+                                     int32_t n_blocks, const void* ln_f, const void* state_in, const void* embeds,
+                                     void* state_out, const float* freqs, const raven_kv_cache* cache, const int32_t* slots,
+                                     int32_t n_iterations, int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+    RAVEN_REQUIRE(adapter_w && embeds && slots, "core_iterations: null pointer");
+    return raven::iterations_impl("core_iterations", dims, adapter_w, blocks, n_blocks, ln_f, state_in, embeds, state_out, freqs, cache,
+                                  slots, nullptr, n_iterations, B, S, pos0, pos_dev, workspace, workspace_bytes, stream);
+}
+
+extern "C" int raven_paged_decode_blocks(const raven_dims* dims, const void* adapter_w, const raven_block_weights* blocks,
+                                         int32_t n_blocks, const void* ln_f, const void* x_in, const void* embeds, void* x_out,
+                                         const float* freqs, const raven_paged_kv* kv, int32_t n_iterations, int32_t B,
+                                         void* workspace, size_t workspace_bytes, void* stream) {
+    RAVEN_REQUIRE(kv && kv->k_caches && kv->v_caches && kv->block_table && kv->seq_lens, "paged_decode_blocks: null cache description");
+    RAVEN_REQUIRE(n_blocks >= 1 && n_blocks <= 64, "paged_decode_blocks: needs 1..64 blocks (got %d)", n_blocks);
+    for (int j = 0; j < n_blocks; ++j)
+        RAVEN_REQUIRE(kv->k_caches[j] && kv->v_caches[j], "paged_decode_blocks: null cache for block %d", j);
+    return raven::iterations_impl("paged_decode_blocks", dims, adapter_w, blocks, n_blocks, ln_f, x_in, embeds, x_out, freqs, nullptr,
+                                  nullptr, kv, n_iterations, B, 1, 0, nullptr, workspace, workspace_bytes, stream);
 }
 
 extern "C" int raven_core_iteration(const raven_dims* dims, const void* adapter_w, const raven_block_weights* blocks,

@@ -40,6 +40,11 @@ class KVCache(C.Structure):
                 ("core_slot0", C.c_int32)]
 
 
+class PagedKV(C.Structure):
+    _fields_ = [("k_caches", C.POINTER(C.c_void_p)), ("v_caches", C.POINTER(C.c_void_p)), ("block_table", C.c_void_p),
+                ("seq_lens", C.c_void_p), ("max_blocks", C.c_int32), ("block_size", C.c_int32), ("max_seq_len", C.c_int32)]
+
+
 LOOKUP_NONE, LOOKUP_SKIP, LOOKUP_LATEST, LOOKUP_ALWAYS_LAST = 0, 1, 2, 3
 
 
@@ -60,6 +65,8 @@ SIGNATURES = {
     "raven_exit_latent_stats": (C.c_int, [_VP, _VP, _VP, _VP, _I32, _I32, _I32, _VP]),
     "raven_paged_kv_append": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _VP]),
     "raven_paged_decode_attention": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _VP, _SZ, _VP]),
+    "raven_paged_qkv_attention_decode": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _VP, _SZ,
+                                                   _VP]),
     "raven_gemv_fused": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _F, _I32, _I32, _I32, _VP]),
     "raven_qkv_bias_rope_cache_append": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32,
                                                    _VP, _I32, _I32, _I32, _VP]),
@@ -80,6 +87,8 @@ SIGNATURES = {
                                        C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _VP, _SZ, _VP]),
     "raven_core_iterations": (C.c_int, [C.POINTER(Dims), _VP, C.POINTER(BlockWeights), _I32, _VP, _VP, _VP, _VP, _VP,
                                         C.POINTER(KVCache), C.POINTER(C.c_int32), _I32, _I32, _I32, _I32, _VP, _VP, _SZ, _VP]),
+    "raven_paged_decode_blocks": (C.c_int, [C.POINTER(Dims), _VP, C.POINTER(BlockWeights), _I32, _VP, _VP, _VP, _VP, _VP,
+                                            C.POINTER(PagedKV), _I32, _I32, _VP, _SZ, _VP]),
 }
 
 _lib: Optional[C.CDLL] = None
@@ -255,6 +264,21 @@ def paged_decode_attention(q, k_cache, v_cache, block_table, seq_lens, max_seq_l
     return y
 
 
+def paged_qkv_attention_decode(qkv, qk_bias, freqs, k_cache, v_cache, block_table, seq_lens, max_seq_len, workspace=None):
+    """The decode step of a paged attention layer in one launch: qkv [B, 3 * nh * hd] from the fused projection; bias, RoPE at
+    position seq_lens[b] - 1, write of the new k / v row to its page, attention over seq_lens[b] positions.  Returns y [B, nh * hd]."""
+    B = qkv.shape[0]
+    _, block_size, nh, hd = k_cache.shape
+    y = torch.empty(B, nh * hd, device=qkv.device, dtype=qkv.dtype)
+    rc = load().raven_paged_qkv_attention_decode(
+        _ptr(qkv, "qkv"), _ptr(qk_bias, "qk_bias", qkv.dtype), _ptr(freqs, "freqs", torch.float32), _ptr(y, "y"),
+        _ptr(k_cache, "k_cache", qkv.dtype), _ptr(v_cache, "v_cache", qkv.dtype), _ptr(block_table, "block_table", torch.int32),
+        _ptr(seq_lens, "seq_lens", torch.int32), B, block_table.shape[1], block_size, int(max_seq_len), nh, hd, dtype_code(qkv.dtype),
+        _ptr(workspace, "workspace", torch.uint8), 0 if workspace is None else workspace.numel(), _stream())
+    _check(rc, "raven_paged_qkv_attention_decode")
+    return y
+
+
 EXIT_ENTROPY, EXIT_KL, EXIT_MINP_KL = 0, 1, 2
 
 
@@ -415,3 +439,33 @@ def core_iterations(dims: Dims, adapter_w, blocks, state_in, embeds, state_out, 
         _ptr(pos_dev, "pos_dev", torch.int32), _ptr(workspace, "workspace", torch.uint8), workspace.numel(), _stream())
     _check(rc, "raven_core_iterations")
     return state_out
+
+
+def make_paged_kv(k_caches, v_caches, block_table, seq_lens, max_seq_len: int) -> PagedKV:
+    """k_caches / v_caches: one [num_blocks, block_size, nh, hd] tensor per block of the stack; block_table [B, max_blocks] and
+    seq_lens [B] int32 on the GPU.  The returned structure holds pointers only: keep the tensors alive."""
+    if len(k_caches) != len(v_caches) or not k_caches:
+        raise RavenHipError("make_paged_kv: one key and one value cache per block")
+    shape, dt = k_caches[0].shape, k_caches[0].dtype
+    for t in list(k_caches) + list(v_caches):
+        if t.shape != shape or t.dtype != dt:
+            raise RavenHipError("make_paged_kv: all caches must share shape and dtype")
+    ka = (C.c_void_p * len(k_caches))(*[_ptr(t, "k_cache") for t in k_caches])
+    va = (C.c_void_p * len(v_caches))(*[_ptr(t, "v_cache") for t in v_caches])
+    if block_table.dim() != 2 or seq_lens.shape != (block_table.shape[0],):
+        raise RavenHipError("make_paged_kv: block_table [B, max_blocks], seq_lens [B]")
+    kv = PagedKV(C.cast(ka, C.POINTER(C.c_void_p)), C.cast(va, C.POINTER(C.c_void_p)), _ptr(block_table, "block_table", torch.int32),
+                 _ptr(seq_lens, "seq_lens", torch.int32), block_table.shape[1], shape[1], int(max_seq_len))
+    kv._keep = (ka, va)  # the pointer arrays live in host memory owned by this object
+    return kv
+
+
+def paged_decode_blocks(dims: Dims, blocks, x_in, x_out, freqs, kv: PagedKV, B, workspace, adapter_w=None, embeds=None, n_iterations=1,
+                        ln_f=None):
+    """The blocks once (adapter_w None: prelude, coda) or n_iterations x (adapter([x, embeds]) + blocks) over paged caches."""
+    rc = load().raven_paged_decode_blocks(
+        C.byref(dims), _ptr(adapter_w, "adapter_w", x_in.dtype), blocks, len(blocks), _ptr(ln_f, "ln_f", x_in.dtype), _ptr(x_in, "x_in"),
+        _ptr(embeds, "embeds", x_in.dtype), _ptr(x_out, "x_out", x_in.dtype), _ptr(freqs, "freqs", torch.float32), C.byref(kv),
+        int(n_iterations), B, _ptr(workspace, "workspace", torch.uint8), workspace.numel(), _stream())
+    _check(rc, "raven_paged_decode_blocks")
+    return x_out

@@ -1,0 +1,128 @@
+"""Decode over block-paged KV caches: what the model of the reference's vLLM plugin does for a batch of decode rows
+(RavenModel.forward, vllm/raven_vllm.py:374-411), without vLLM.
+
+Every flat layer (prelude, core and coda blocks in forward order) owns ONE paged cache [num_blocks, block_size, n_heads,
+head_dim] for keys and one for values; the recurrences of a token overwrite the core layers' entries in turn, so older
+positions hold the keys and values of their last recurrence -- the cache sharing that the Hugging Face surface calls
+`latest-m4-compress-s4` (raven_modeling_minimal.py:169-182), which is why a prompt processed through that surface can be
+copied into the pages (`load_prompt`).  A sequence is a row of the block table plus a length; sequences of different
+lengths decode together, each at its own position (the contiguous cache of the Hugging Face surface shares one position
+across the batch, raven_modeling_minimal.py:660-665).
+
+The arithmetic of a step is the contiguous decode path's: the same SandwichBlock launches with the paged decode-attention
+kernel in place of the contiguous one (raven_paged_decode_blocks)."""
+
+from __future__ import annotations
+
+from typing import Optional, Sequence
+
+import torch
+
+from . import hip
+from .cache import HuginnDynamicCache, remap_step
+
+PAGED_STRATEGY = "latest-m4-compress-s4"
+
+
+class PagedDecoder:
+    def __init__(self, model, num_blocks: int, block_size: int = 16, num_steps: Optional[int] = None):
+        cfg = model.config
+        if (cfg.n_layers_in_prelude, cfg.n_layers_in_recurrent_block) != (2, 4):
+            # the equivalence with the cache-sharing strategy of the other surface hard-codes these counts (RMM:169-182)
+            raise NotImplementedError("the paged decoder mirrors a model with 2 prelude and 4 core blocks")
+        self.model, self.cfg = model, cfg
+        self.r = cfg.mean_recurrence if num_steps is None else int(num_steps)
+        if self.r < 1:
+            raise ValueError("num_steps must be at least 1")
+        self.block_size, self.num_blocks = int(block_size), int(num_blocks)
+        dev, dt = model.device, model.dtype
+        self.n_flat = cfg.n_layers_in_prelude + cfg.n_layers_in_recurrent_block + cfg.n_layers_in_coda
+        shape = (self.num_blocks, self.block_size, cfg.n_heads, cfg.head_dim)
+        self.k = [torch.zeros(shape, dtype=dt, device=dev) for _ in range(self.n_flat)]
+        self.v = [torch.zeros(shape, dtype=dt, device=dev) for _ in range(self.n_flat)]
+        self._ws = {}
+
+    # ------------------------------------------------------------------ prompts
+    def _flat_steps(self):
+        """Step index, in the other surface's cache, of each flat layer's final entries."""
+        cfg = self.cfg
+        n_pre, n_core = cfg.n_layers_in_prelude, cfg.n_layers_in_recurrent_block
+        last = n_pre + (self.r - 1) * n_core
+        return ([i for i in range(n_pre)] + [remap_step(last + j, PAGED_STRATEGY) for j in range(n_core)] +
+                [-(i + 1) for i in range(cfg.n_layers_in_coda)])
+
+    def load_prompt(self, cache: HuginnDynamicCache, row: int, table_row: Sequence[int]) -> int:
+        """Copies sequence `row` of a cache filled through the other surface with lookup_strategy `latest-m4-compress-s4`
+        into the pages listed in table_row; returns the number of positions."""
+        if cache.lookup_strategy != PAGED_STRATEGY:
+            raise ValueError(f"a prompt for the paged decoder must be cached with lookup_strategy={PAGED_STRATEGY!r}")
+        n = cache.get_seq_length()
+        if n > len(table_row) * self.block_size:
+            raise ValueError(f"{len(table_row)} blocks of {self.block_size} cannot hold {n} positions")
+        pos = torch.arange(n)
+        table = torch.as_tensor(list(table_row), dtype=torch.int64)
+        slots = (table[pos // self.block_size] * self.block_size + pos % self.block_size).to(self.model.device)
+        h = self.cfg.n_heads * self.cfg.head_dim
+        for f, step in enumerate(self._flat_steps()):
+            s = cache._slot(step)
+            k = cache._k[s, row, :, :n].transpose(0, 1).reshape(n, h).contiguous()
+            v = cache._v[s, row, :, :n].transpose(0, 1).reshape(n, h).contiguous()
+            hip.paged_kv_append(k, v, self.k[f], self.v[f], slots)
+        return n
+
+    def prefill(self, input_ids: torch.Tensor, table_row: Sequence[int], input_states: Optional[torch.Tensor] = None):
+        """One prompt [1, n] through the chunk kernels of the other surface, then into the pages.  Returns its output."""
+        cache = HuginnDynamicCache(lookup_strategy=PAGED_STRATEGY)
+        n = input_ids.shape[1]
+        out = self.model(input_ids=input_ids, input_states=input_states, past_key_values=cache, use_cache=True,
+                         cache_position=torch.arange(n, device=input_ids.device), num_steps=self.r)
+        self.load_prompt(cache, 0, table_row)
+        return out
+
+    # ------------------------------------------------------------------ decode
+    def _buffers(self, B: int):
+        if B not in self._ws:
+            m, cfg = self.model, self.cfg
+            dev, dt, h = m.device, m.dtype, cfg.n_embd
+            nat = m._natives()
+            mk = lambda: torch.empty(B, h, dtype=dt, device=dev)
+            self._ws[B] = {
+                "embeds": mk(), "pre": mk(), "x": mk(), "y": mk(),
+                "logits": torch.empty(B, cfg.padded_vocab_size, dtype=torch.float32, device=dev),
+                "ws": hip.block_workspace(nat["dims"], B, dev),
+            }
+        return self._ws[B]
+
+    def step(self, ids: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor, input_states: Optional[torch.Tensor] = None,
+             init_scale: float = 1.0):
+        """One new token per sequence.  ids [B]; block_table [B, max_blocks] int32; seq_lens [B] int32 = each sequence's
+        length INCLUDING the new token (its position is seq_lens - 1; the page for it must be in the table).
+        Returns (logits [B, V] float32, latents [B, h]); both are buffers reused by the next step of the same batch size."""
+        m, cfg, t = self.model, self.cfg, self.model.transformer
+        B = ids.shape[0]
+        nat = m._natives()
+        buf = self._buffers(B)
+        max_len = block_table.shape[1] * self.block_size  # sizes the launch only; lengths are read on the device
+        n_pre, n_core = cfg.n_layers_in_prelude, cfg.n_layers_in_recurrent_block
+        kvs = [hip.make_paged_kv(self.k[a:b], self.v[a:b], block_table, seq_lens, max_len)
+               for a, b in ((0, n_pre), (n_pre, n_pre + n_core), (n_pre + n_core, self.n_flat))]
+        hip.embed(t.wte.weight, ids.view(-1), m.emb_scale, out=buf["embeds"])
+        pre = (hip.BlockWeights * n_pre)(*nat["prelude"])
+        hip.paged_decode_blocks(nat["dims"], pre, buf["embeds"], buf["pre"], nat["freqs"], kvs[0], B, buf["ws"])
+        if input_states is None:
+            state = m.initialize_state(buf["pre"], init_scale) if init_scale > 0 else torch.zeros_like(buf["pre"])
+        else:
+            state = input_states.reshape(B, -1).to(m.dtype).contiguous()
+        hip.paged_decode_blocks(nat["dims"], nat["core"], state, buf["x"], nat["freqs"], kvs[1], B, buf["ws"], adapter_w=t.adapter.weight,
+                                embeds=buf["pre"], n_iterations=self.r, ln_f=t.ln_f.weight)
+        if cfg.n_layers_in_coda > 0:
+            coda = (hip.BlockWeights * cfg.n_layers_in_coda)(*nat["coda"])
+            hip.paged_decode_blocks(nat["dims"], coda, buf["x"], buf["y"], nat["freqs"], kvs[2], B, buf["ws"], ln_f=t.ln_f.weight)
+        else:
+            rc = hip.load().raven_rmsnorm_residual(buf["x"].data_ptr(), None, t.ln_f.weight.data_ptr(), buf["y"].data_ptr(), None, None,
+                                                   None, B, cfg.n_embd, cfg.norm_eps, hip.dtype_code(m.dtype), hip._stream())
+            hip._check(rc, "raven_rmsnorm_residual")
+        rc = hip.load().raven_gemm(buf["y"].data_ptr(), m.lm_head.weight.data_ptr(), None, buf["logits"].data_ptr(), B,
+                                   cfg.padded_vocab_size, cfg.n_embd, hip.dtype_code(m.dtype), 1, hip._stream())
+        hip._check(rc, "raven_gemm")
+        return buf["logits"], buf["x"]

@@ -670,3 +670,32 @@ def test_paged_decode_attention_and_append(pkg, dt, nh, hd, B, block_size):
     check(y[full], want[full].float().cpu(), dt, "paged vs contiguous")
     with pytest.raises(pkg.hip.RavenHipError):
         pkg.hip.paged_decode_attention(q.cuda(), kc, vc, table.cuda(), lens.cuda(), max_blocks * block_size + 1)
+
+    # The fused decode step: sequence b's new token at position lens[b] - 1 (its page currently holds k_seq / v_seq of
+    # that position, which the step overwrites).  Against the oracle's bias + RoPE per sequence, the append kernel and
+    # the attention kernel above -- same results, and the same cache afterwards.
+    qkv = rnd((B, 3 * h), dt, 604)
+    bias = rnd((2, nh, hd), dt, 605, 0.5)
+    rope = O.rope_table(hd, max_len, 50000.0).to(dt)
+    freqs = rope.float().reshape(max_len, hd // 2, 2).contiguous().cuda()
+    kc2, vc2 = kc.clone(), vc.clone()
+    for wsp in (ws, None):
+        y_f = pkg.hip.paged_qkv_attention_decode(qkv.cuda(), bias.cuda(), freqs, kc, vc, table.cuda(), lens.cuda(), max_len, workspace=wsp)
+    rows_q, rows_k, rows_v, slots = [], [], [], []
+    for b in range(B):
+        n = int(lens[b])
+        qq, kk, vv = (t.view(1, 1, nh, hd) for t in qkv[b].split([h, h, h]))
+        if n == 0:
+            rows_q.append(torch.zeros(h, dtype=dt)); rows_k.append(torch.zeros(h, dtype=dt)); rows_v.append(torch.zeros(h, dtype=dt))
+            slots.append(-1)
+            continue
+        qq, kk = (qq + bias[0]).to(dt), (kk + bias[1]).to(dt)
+        rq, rk = O.apply_rope(qq, kk, rope[:, n - 1:n])
+        rows_q.append(rq.reshape(h)); rows_k.append(rk.reshape(h)); rows_v.append(vv.reshape(h))
+        slots.append(int(table[b, (n - 1) // block_size]) * block_size + (n - 1) % block_size)
+    pkg.hip.paged_kv_append(torch.stack(rows_k).cuda(), torch.stack(rows_v).cuda(), kc2, vc2, torch.tensor(slots, dtype=torch.int64).cuda())
+    y_2 = pkg.hip.paged_decode_attention(torch.stack(rows_q).cuda(), kc2, vc2, table.cuda(), lens.cuda(), max_len, workspace=ws)
+    check(y_f, y_2.float().cpu(), dt, "fused paged step vs rope + append + attention")
+    check(kc, kc2.float().cpu(), dt, "keys after the fused paged step")
+    assert torch.equal(vc, vc2)
+    assert int((kc.view(-1, nh, hd).abs().amax(dim=(1, 2)) > 0).sum()) == int(lens.sum())  # no other row was touched

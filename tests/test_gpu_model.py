@@ -378,6 +378,51 @@ def test_generate_speculative_matches_oracle(pkg, small242, B, draft_steps, L, v
         assert n >= 5 + 9 and torch.equal(plain[:, :n], spec[:, :n])
 
 
+@pytest.mark.parametrize("lens", [(7, 3, 12, 5, 9, 2), (6,), (4, 4)])
+def test_paged_decoder_serves_sequences_of_different_lengths(pkg, small242, lens):
+    """Block-paged caches, one per flat layer, shared by all recurrences (the cache of the reference's vLLM plugin):
+    every sequence is prefilled on its own, then all decode together, each at its own position.  Per sequence the
+    logits equal the oracle's forward with the cache-sharing strategy that has the same semantics on the other surface
+    (`latest-m4-compress-s4`), run on that sequence alone."""
+    s, w, model = small242
+    B, n_new, bs, r = len(lens), 4, 4, 3
+    g = torch.Generator().manual_seed(77 + B)
+    max_blocks = (max(lens) + n_new + bs - 1) // bs
+    table = torch.randperm(B * max_blocks + 5, generator=g)[:B * max_blocks].view(B, max_blocks).to(torch.int32)
+    dec = pkg.PagedDecoder(model, num_blocks=B * max_blocks + 5, block_size=bs, num_steps=r)
+    prompts = [torch.randint(0, s.vocab_size, (1, n), generator=g) for n in lens]
+    new_ids = torch.randint(0, s.vocab_size, (B, n_new), generator=g)
+    states = [O.initialize_state(torch.empty(1, n + n_new, s.n_embd), s, 1.0, g) for n in lens]
+    want = []  # per sequence: logits of each decode step
+    for b, n in enumerate(lens):
+        ref = O.DictCache("latest-m4-compress-s4")
+        o = O.forward(w, s, input_ids=prompts[b], input_states=states[b][:, :n], past_key_values=ref, use_cache=True,
+                      cache_position=torch.arange(n), num_steps=r)
+        got = dec.prefill(prompts[b].cuda(), table[b].tolist(), input_states=states[b][:, :n].cuda())
+        check(got.logits, o.logits, torch.float32, f"prompt {b}")
+        steps = []
+        for t in range(n_new):
+            o = O.forward(w, s, input_ids=new_ids[b:b + 1, t:t + 1], input_states=states[b][:, n + t:n + t + 1], past_key_values=ref,
+                          use_cache=True, cache_position=torch.tensor([n + t]), num_steps=r)
+            steps.append(o.logits[0, 0])
+        want.append(steps)
+    table_d = table.cuda()
+    for t in range(n_new):
+        seq_lens = torch.tensor([n + t + 1 for n in lens], dtype=torch.int32).cuda()
+        st = torch.cat([states[b][:, lens[b] + t] for b in range(B)]).cuda()
+        logits, latents = dec.step(new_ids[:, t].cuda(), table_d, seq_lens, input_states=st)
+        for b in range(B):
+            check(logits[b], want[b][t], torch.float32, f"sequence {b} (length {lens[b]}), decode step {t}")
+        assert latents.shape == (B, s.n_embd)
+    # a position outside the table is an error of the caller that the entry point catches by size
+    with pytest.raises(pkg.hip.RavenHipError):
+        pkg.hip.paged_decode_blocks(model._natives()["dims"], model._natives()["core"], latents, latents.clone(), model._natives()["freqs"],
+                                    pkg.hip.make_paged_kv(dec.k[2:6], dec.v[2:6], table_d, seq_lens, max_blocks * bs), B,
+                                    torch.empty(16, dtype=torch.uint8, device="cuda"))
+    with pytest.raises(ValueError):
+        dec.load_prompt(pkg.HuginnDynamicCache(), 0, table[0].tolist())
+
+
 @pytest.mark.parametrize("dt,B", [(torch.float32, 1), (torch.bfloat16, 1), (torch.bfloat16, 3), (torch.float32, 6), (torch.bfloat16, 6),
                                   (torch.bfloat16, 32)])
 def test_core_iterations_equal_single_iterations(pkg, tiny32, tiny16, dt, B):
