@@ -25,7 +25,7 @@ PAGED_STRATEGY = "latest-m4-compress-s4"
 
 
 class PagedDecoder:
-    def __init__(self, model, num_blocks: int, block_size: int = 16, num_steps: Optional[int] = None):
+    def __init__(self, model, num_blocks: int, block_size: int = 16, num_steps: Optional[int] = None, use_graph: bool = False):
         cfg = model.config
         if (cfg.n_layers_in_prelude, cfg.n_layers_in_recurrent_block) != (2, 4):
             # the equivalence with the cache-sharing strategy of the other surface hard-codes these counts (RMM:169-182)
@@ -41,6 +41,9 @@ class PagedDecoder:
         self.k = [torch.zeros(shape, dtype=dt, device=dev) for _ in range(self.n_flat)]
         self.v = [torch.zeros(shape, dtype=dt, device=dev) for _ in range(self.n_flat)]
         self._ws = {}
+        # use_graph: a step's launches are captured once per (batch size, table width) and replayed; ids, block table,
+        # lengths and latent state are copied into fixed buffers that the captured kernels read
+        self.use_graph = use_graph
 
     # ------------------------------------------------------------------ prompts
     def _flat_steps(self):
@@ -80,41 +83,36 @@ class PagedDecoder:
         return out
 
     # ------------------------------------------------------------------ decode
-    def _buffers(self, B: int):
-        if B not in self._ws:
+    def _buffers(self, B: int, max_blocks: int):
+        key = (B, max_blocks)
+        if key not in self._ws:
             m, cfg = self.model, self.cfg
             dev, dt, h = m.device, m.dtype, cfg.n_embd
             nat = m._natives()
             mk = lambda: torch.empty(B, h, dtype=dt, device=dev)
-            self._ws[B] = {
-                "embeds": mk(), "pre": mk(), "x": mk(), "y": mk(),
+            self._ws[key] = {
+                "ids": torch.zeros(B, dtype=torch.int64, device=dev),
+                "table": torch.zeros(B, max_blocks, dtype=torch.int32, device=dev),
+                "lens": torch.zeros(B, dtype=torch.int32, device=dev),
+                "state": mk(), "embeds": mk(), "pre": mk(), "x": mk(), "y": mk(),
                 "logits": torch.empty(B, cfg.padded_vocab_size, dtype=torch.float32, device=dev),
                 "ws": hip.block_workspace(nat["dims"], B, dev),
+                "graph": None, "warm": False,
             }
-        return self._ws[B]
+        return self._ws[key]
 
-    def step(self, ids: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor, input_states: Optional[torch.Tensor] = None,
-             init_scale: float = 1.0):
-        """One new token per sequence.  ids [B]; block_table [B, max_blocks] int32; seq_lens [B] int32 = each sequence's
-        length INCLUDING the new token (its position is seq_lens - 1; the page for it must be in the table).
-        Returns (logits [B, V] float32, latents [B, h]); both are buffers reused by the next step of the same batch size."""
+    def _enqueue(self, buf, B: int):
         m, cfg, t = self.model, self.cfg, self.model.transformer
-        B = ids.shape[0]
         nat = m._natives()
-        buf = self._buffers(B)
-        max_len = block_table.shape[1] * self.block_size  # sizes the launch only; lengths are read on the device
+        max_len = buf["table"].shape[1] * self.block_size  # sizes the launch only; lengths are read on the device
         n_pre, n_core = cfg.n_layers_in_prelude, cfg.n_layers_in_recurrent_block
-        kvs = [hip.make_paged_kv(self.k[a:b], self.v[a:b], block_table, seq_lens, max_len)
+        kvs = [hip.make_paged_kv(self.k[a:b], self.v[a:b], buf["table"], buf["lens"], max_len)
                for a, b in ((0, n_pre), (n_pre, n_pre + n_core), (n_pre + n_core, self.n_flat))]
-        hip.embed(t.wte.weight, ids.view(-1), m.emb_scale, out=buf["embeds"])
+        hip.embed(t.wte.weight, buf["ids"], m.emb_scale, out=buf["embeds"])
         pre = (hip.BlockWeights * n_pre)(*nat["prelude"])
         hip.paged_decode_blocks(nat["dims"], pre, buf["embeds"], buf["pre"], nat["freqs"], kvs[0], B, buf["ws"])
-        if input_states is None:
-            state = m.initialize_state(buf["pre"], init_scale) if init_scale > 0 else torch.zeros_like(buf["pre"])
-        else:
-            state = input_states.reshape(B, -1).to(m.dtype).contiguous()
-        hip.paged_decode_blocks(nat["dims"], nat["core"], state, buf["x"], nat["freqs"], kvs[1], B, buf["ws"], adapter_w=t.adapter.weight,
-                                embeds=buf["pre"], n_iterations=self.r, ln_f=t.ln_f.weight)
+        hip.paged_decode_blocks(nat["dims"], nat["core"], buf["state"], buf["x"], nat["freqs"], kvs[1], B, buf["ws"],
+                                adapter_w=t.adapter.weight, embeds=buf["pre"], n_iterations=self.r, ln_f=t.ln_f.weight)
         if cfg.n_layers_in_coda > 0:
             coda = (hip.BlockWeights * cfg.n_layers_in_coda)(*nat["coda"])
             hip.paged_decode_blocks(nat["dims"], coda, buf["x"], buf["y"], nat["freqs"], kvs[2], B, buf["ws"], ln_f=t.ln_f.weight)
@@ -125,4 +123,34 @@ class PagedDecoder:
         rc = hip.load().raven_gemm(buf["y"].data_ptr(), m.lm_head.weight.data_ptr(), None, buf["logits"].data_ptr(), B,
                                    cfg.padded_vocab_size, cfg.n_embd, hip.dtype_code(m.dtype), 1, hip._stream())
         hip._check(rc, "raven_gemm")
+
+    def step(self, ids: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor, input_states: Optional[torch.Tensor] = None,
+             init_scale: float = 1.0):
+        """One new token per sequence.  ids [B]; block_table [B, max_blocks] int32; seq_lens [B] int32 = each sequence's
+        length INCLUDING the new token (its position is seq_lens - 1; the page for it must be in the table).
+        Returns (logits [B, V] float32, latents [B, h]); both are buffers reused by the next step of the same batch size."""
+        m = self.model
+        B = ids.shape[0]
+        if block_table.dim() != 2 or block_table.shape[0] != B or seq_lens.shape != (B,):
+            raise ValueError("block_table [B, max_blocks] and seq_lens [B] must match ids [B]")
+        buf = self._buffers(B, block_table.shape[1])
+        buf["ids"].copy_(ids.view(-1))
+        buf["table"].copy_(block_table)
+        buf["lens"].copy_(seq_lens)
+        if input_states is None:
+            if init_scale > 0:
+                buf["state"].copy_(m.initialize_state(buf["state"], init_scale))
+            else:
+                buf["state"].zero_()
+        else:
+            buf["state"].copy_(input_states.reshape(B, -1))
+        if self.use_graph and buf["warm"]:
+            if buf["graph"] is None:
+                buf["graph"] = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(buf["graph"]):
+                    self._enqueue(buf, B)
+            buf["graph"].replay()
+        else:
+            self._enqueue(buf, B)
+            buf["warm"] = True
         return buf["logits"], buf["x"]

@@ -378,18 +378,20 @@ def test_generate_speculative_matches_oracle(pkg, small242, B, draft_steps, L, v
         assert n >= 5 + 9 and torch.equal(plain[:, :n], spec[:, :n])
 
 
-@pytest.mark.parametrize("lens", [(7, 3, 12, 5, 9, 2), (6,), (4, 4)])
-def test_paged_decoder_serves_sequences_of_different_lengths(pkg, small242, lens):
+@pytest.mark.parametrize("lens,use_graph", [((7, 3, 12, 5, 9, 2), False), ((6,), False), ((4, 4), False), ((7, 3, 12, 5, 9, 2), True),
+                                            ((6,), True)])
+def test_paged_decoder_serves_sequences_of_different_lengths(pkg, small242, lens, use_graph):
     """Block-paged caches, one per flat layer, shared by all recurrences (the cache of the reference's vLLM plugin):
     every sequence is prefilled on its own, then all decode together, each at its own position.  Per sequence the
     logits equal the oracle's forward with the cache-sharing strategy that has the same semantics on the other surface
-    (`latest-m4-compress-s4`), run on that sequence alone."""
+    (`latest-m4-compress-s4`), run on that sequence alone.  use_graph: the step's launches replayed from a HIP graph
+    (captured at the second step; lengths, table and ids are read from device buffers)."""
     s, w, model = small242
     B, n_new, bs, r = len(lens), 4, 4, 3
     g = torch.Generator().manual_seed(77 + B)
     max_blocks = (max(lens) + n_new + bs - 1) // bs
     table = torch.randperm(B * max_blocks + 5, generator=g)[:B * max_blocks].view(B, max_blocks).to(torch.int32)
-    dec = pkg.PagedDecoder(model, num_blocks=B * max_blocks + 5, block_size=bs, num_steps=r)
+    dec = pkg.PagedDecoder(model, num_blocks=B * max_blocks + 5, block_size=bs, num_steps=r, use_graph=use_graph)
     prompts = [torch.randint(0, s.vocab_size, (1, n), generator=g) for n in lens]
     new_ids = torch.randint(0, s.vocab_size, (B, n_new), generator=g)
     states = [O.initialize_state(torch.empty(1, n + n_new, s.n_embd), s, 1.0, g) for n in lens]
