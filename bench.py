@@ -41,6 +41,7 @@ def parse():
                     help="per-token adaptive compute at bs=1 with a fixed cycle of recurrences per token (a next-row measurement)")
     ap.add_argument("--paged", action="store_true",
                     help="decode over block-paged caches, --batch sequences of different lengths around --prompt (a next-row measurement)")
+    ap.add_argument("--paged-layout", default="HND", choices=["NHD", "HND"])
     ap.add_argument("--prefill", action="store_true",
                     help="measure the recurrent core over a whole prompt instead (bs=4 x 4096 tokens, r iterations): MFMA-bound regime")
     ap.add_argument("--prefill-batch", type=int, default=4)
@@ -169,7 +170,7 @@ def paged(args):
     max_blocks = (int(lens.max()) + total + bs - 1) // bs
     n_blocks = B * max_blocks
     table = torch.randperm(n_blocks, generator=g).view(B, max_blocks).to(torch.int32).to(dev)
-    dec = pkg.PagedDecoder(model, num_blocks=n_blocks, block_size=bs, num_steps=r, use_graph=not args.no_graph)
+    dec = pkg.PagedDecoder(model, num_blocks=n_blocks, block_size=bs, num_steps=r, use_graph=not args.no_graph, layout=args.paged_layout)
     for t in dec.k + dec.v:
         t.normal_(0.0, 1.0)
     ids = torch.randint(0, cfg.vocab_size, (B,), generator=g).to(dev)
@@ -201,7 +202,8 @@ def paged(args):
         "ms_per_step": round(dt / args.steps * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"PagedDecoder.step, nebel-raven-3.5b shape, r={r}, {B} sequences, lengths {int(lens.min())}..{int(lens.max())} "
-                               f"(mean {float(lens.float().mean()):.0f}), block size {bs}", "batch": B, "recurrence": r, "hip_graph": not args.no_graph},
+                               f"(mean {float(lens.float().mean()):.0f}), block size {bs}", "batch": B, "recurrence": r, "hip_graph": not args.no_graph,
+                   "layout": args.paged_layout},
         "kv_GB_per_step": round(kv_bytes / 1e9, 2),
     }
     print(json.dumps(line))

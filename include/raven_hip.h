@@ -148,8 +148,9 @@ int raven_exit_latent_stats(const void* latents, const void* prev, void* rel_cha
 
 /* Paged KV cache, the layout the attention layer of the reference's vLLM plugin is given (vllm/raven_vllm.py:174-201
  * hands rotated q, k and v to vLLM's Attention, which owns a block-paged cache): k_cache and v_cache are
- * [num_blocks, block_size, n_heads, head_dim] of T; position p of sequence b lives in block
- * block_table[b * max_blocks + p / block_size] at offset p % block_size.
+ * [num_blocks, block_size, n_heads, head_dim] of T (kv_layout RAVEN_PAGED_NHD) or [num_blocks, n_heads, block_size,
+ * head_dim] (RAVEN_PAGED_HND: a head's positions of a block are contiguous, which the attention kernel reads faster);
+ * position p of sequence b lives in block block_table[b * max_blocks + p / block_size] at offset p % block_size.
  * raven_paged_kv_append: rows k, v [T, n_heads * head_dim] (k already biased and rotated) go to the flat slots
  *   slot_mapping[t] = block * block_size + offset (negative: skipped).
  * raven_paged_decode_attention: one query row per sequence, q / y [B, n_heads * head_dim]; sequence b attends to its
@@ -160,21 +161,24 @@ int raven_exit_latent_stats(const void* latents, const void* prev, void* rel_cha
  *   fused projection's output, qk_bias [2, n_heads, head_dim] or NULL, freqs the (cos, sin) table; sequence b's new
  *   token sits at position seq_lens[b] - 1: its rotated k and its v are written to that position's page and the row
  *   attends to positions 0..seq_lens[b] - 1 (seq_lens[b] = 0: nothing written, zeros returned). */
+enum { RAVEN_PAGED_NHD = 0, RAVEN_PAGED_HND = 1 };
 int raven_paged_kv_append(const void* k, const void* v, void* k_cache, void* v_cache, const int64_t* slot_mapping,
-                          int32_t T, int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream);
+                          int32_t T, int32_t n_heads, int32_t head_dim, int32_t block_size, int32_t kv_layout,
+                          int32_t dtype, void* stream);
 int raven_paged_decode_attention(const void* q, void* y, const void* k_cache, const void* v_cache,
                                  const int32_t* block_table, const int32_t* seq_lens, int32_t B, int32_t max_blocks,
-                                 int32_t block_size, int32_t max_seq_len, int32_t n_heads, int32_t head_dim,
-                                 int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
+                                 int32_t block_size, int32_t kv_layout, int32_t max_seq_len, int32_t n_heads,
+                                 int32_t head_dim, int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
 int raven_paged_qkv_attention_decode(const void* qkv, const void* qk_bias, const float* freqs, void* y, void* k_cache,
                                      void* v_cache, const int32_t* block_table, const int32_t* seq_lens, int32_t B,
-                                     int32_t max_blocks, int32_t block_size, int32_t max_seq_len, int32_t n_heads,
-                                     int32_t head_dim, int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
+                                     int32_t max_blocks, int32_t block_size, int32_t kv_layout, int32_t max_seq_len,
+                                     int32_t n_heads, int32_t head_dim, int32_t dtype, void* workspace,
+                                     size_t workspace_bytes, void* stream);
 
 /* A stack of SandwichBlocks over block-paged caches, one decode row per sequence (the flat layer list the plugin's
  * model runs, vllm/raven_vllm.py:365-432: every flat layer owns ONE paged cache, which the recurrences of a token
  * overwrite in turn, so older positions hold their last recurrence).  k_caches / v_caches: HOST arrays of n_blocks
- * device pointers, block j's cache [num_blocks, block_size, n_heads, head_dim]; block_table [B, max_blocks] and
+ * device pointers, block j's cache in the layout kv_layout names; block_table [B, max_blocks] and
  * seq_lens [B] (new token included) in device memory, shared by all blocks.
  * adapter_w / embeds non-NULL: n_iterations x (adapter([x, embeds]) then the blocks), i.e. the recurrent core;
  * both NULL: the blocks once (prelude, coda).  ln_f non-NULL: applied to the result.  x_in, embeds, x_out [B, h].
@@ -185,6 +189,7 @@ typedef struct raven_paged_kv {
     const int32_t* block_table;
     const int32_t* seq_lens;
     int32_t max_blocks, block_size, max_seq_len;
+    int32_t kv_layout; /* RAVEN_PAGED_NHD or RAVEN_PAGED_HND */
 } raven_paged_kv;
 int raven_paged_decode_blocks(const raven_dims* dims, const void* adapter_w, const raven_block_weights* blocks,
                               int32_t n_blocks, const void* ln_f, const void* x_in, const void* embeds, void* x_out,

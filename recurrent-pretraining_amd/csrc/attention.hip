@@ -343,6 +343,9 @@ struct PagedView {
     const int* block_table;  // [B, max_blocks]
     const int* seq_lens;     // [B]: positions to attend to, the new token's own included
     int max_blocks, block_size, nh, hd;
+    int block_shift;         // log2(block_size), or -1 when it is not a power of two
+    int64_t pos_stride;      // elements between two positions of a block: nh * hd (RAVEN_PAGED_NHD) or hd (RAVEN_PAGED_HND)
+    int64_t head_stride;     // elements between two heads: hd (NHD) or block_size * hd (HND)
 };
 
 // FUSED: q_or_qkv is the fused projection's output [B, 3 * h]; bias and RoPE (row seq_lens[b] - 1 of the table) are
@@ -371,6 +374,24 @@ __global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __
     const T* V = static_cast<const T*>(pv.v);
     const int col = head * hd + ci * E;
     const int pos = len - 1;  // FUSED: the new token's position
+    // this workgroup's part of the block table, read once: the loop's addresses then depend on LDS only
+    constexpr int kTbl = 1024;
+    __shared__ int tbl[kTbl];
+    auto block_of = [&](int p) { return pv.block_shift >= 0 ? p >> pv.block_shift : p / pv.block_size; };
+    auto offset_of = [&](int p) { return pv.block_shift >= 0 ? p & (pv.block_size - 1) : p % pv.block_size; };
+    const int blk0 = block_of(start);
+    if (start < end) {
+        const int n_blk = block_of(end - 1) - blk0 + 1;
+        for (int i = threadIdx.x; i < min(n_blk, kTbl); i += 256) tbl[i] = table[blk0 + i];
+    }
+    __syncthreads();
+    const int64_t blk_stride = (int64_t)pv.block_size * pv.nh * hd;
+    const int64_t lane_off = head * pv.head_stride + ci * E;
+    auto elem_of = [&](int p) {  // this lane's first element of position p
+        const int i = block_of(p) - blk0;
+        const int blk = i < kTbl ? tbl[i] : table[blk0 + i];
+        return (int64_t)blk * blk_stride + offset_of(p) * pv.pos_stride + lane_off;
+    };
     P qc = zero_piece<T, CPL>(), knew = zero_piece<T, CPL>(), vnew = zero_piece<T, CPL>();
     if (active && !FUSED) qc = load_piece<T, CPL>(q_or_qkv + (int64_t)b * h + col);
     if (FUSED && active && len > 0) {
@@ -384,8 +405,7 @@ __global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __
             knew.c[i] = bias_rope_chunk<T>(knew.c[i], qk_bias, 1, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
         }
         if (group == 0 && pos >= start && pos < end) {
-            const int64_t row_new = (int64_t)table[pos / pv.block_size] * pv.block_size + pos % pv.block_size;
-            const int64_t off = (row_new * pv.nh + head) * hd + ci * E;
+            const int64_t off = elem_of(pos);
             store_piece<T, CPL>(const_cast<T*>(K) + off, knew);
             store_piece<T, CPL>(const_cast<T*>(V) + off, vnew);
         }
@@ -403,8 +423,7 @@ __global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __
                 kc[j] = knew;
                 vc[j] = vnew;
             } else if (active && p < end) {
-                const int64_t row = (int64_t)table[p / pv.block_size] * pv.block_size + p % pv.block_size;
-                const int64_t off = (row * pv.nh + head) * hd + ci * E;
+                const int64_t off = elem_of(p);
                 kc[j] = load_piece<T, CPL, true>(K + off);
                 vc[j] = load_piece<T, CPL, true>(V + off);
             } else {
@@ -470,16 +489,21 @@ __global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __
     }
 }
 
-// cache[slot_mapping[t]] = row t, for K and V: rows of [n_heads * head_dim] elements; negative slots are skipped
+// cache[slot_mapping[t]] = row t, for K and V: rows of [n_heads * head_dim] elements; negative slots are skipped.
+// slot = block * block_size + offset; pos_stride / head_stride as in PagedView.
 template <typename T>
 __global__ __launch_bounds__(256) void paged_kv_append_kernel(const T* __restrict__ k, const T* __restrict__ v, T* __restrict__ kc,
-                                                              T* __restrict__ vc, const int64_t* __restrict__ slots, int h) {
+                                                              T* __restrict__ vc, const int64_t* __restrict__ slots, int h, int hd,
+                                                              int block_size, int64_t pos_stride, int64_t head_stride) {
     constexpr int E = Chunk<T>::N;
     const int t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
     const int64_t slot = slots[t];
     if (c >= h / E || slot < 0) return;
-    store_chunk(kc + slot * h + c * E, load_chunk(k + (int64_t)t * h + c * E));
-    store_chunk(vc + slot * h + c * E, load_chunk(v + (int64_t)t * h + c * E));
+    const int64_t blk = slot / block_size, off = slot - blk * block_size;
+    const int head = c * E / hd, d = c * E - head * hd;
+    const int64_t dst = blk * block_size * h + off * pos_stride + head * head_stride + d;
+    store_chunk(kc + dst, load_chunk(k + (int64_t)t * h + c * E));
+    store_chunk(vc + dst, load_chunk(v + (int64_t)t * h + c * E));
 }
 
 constexpr int kAttnMaxSplits = 32;
@@ -643,27 +667,41 @@ extern "C" int raven_qkv_attention_decode(const void* qkv, const void* qk_bias, 
 }
 
 
+static int paged_strides(const char* who, int kv_layout, int block_size, int n_heads, int head_dim, int64_t* pos_stride, int64_t* head_stride) {
+    RAVEN_REQUIRE(kv_layout == RAVEN_PAGED_NHD || kv_layout == RAVEN_PAGED_HND, "%s: unknown kv_layout %d", who, kv_layout);
+    RAVEN_REQUIRE(block_size > 0, "%s: bad block_size %d", who, block_size);
+    *pos_stride = kv_layout == RAVEN_PAGED_NHD ? (int64_t)n_heads * head_dim : head_dim;
+    *head_stride = kv_layout == RAVEN_PAGED_NHD ? head_dim : (int64_t)block_size * head_dim;
+    return 0;
+}
+
 extern "C" int raven_paged_kv_append(const void* k, const void* v, void* k_cache, void* v_cache, const int64_t* slot_mapping,
-                                     int32_t T, int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream) {
+                                     int32_t T, int32_t n_heads, int32_t head_dim, int32_t block_size, int32_t kv_layout,
+                                     int32_t dtype, void* stream) {
     using namespace raven;
     if (int rc = check_heads("paged_kv_append", n_heads, head_dim, dtype)) return rc;
+    int64_t ps, hs;
+    if (int rc = paged_strides("paged_kv_append", kv_layout, block_size, n_heads, head_dim, &ps, &hs)) return rc;
     RAVEN_REQUIRE(T >= 0 && T <= 65535, "paged_kv_append: bad row count %d", T);
     if (T == 0) return 0;
     RAVEN_REQUIRE(k && v && k_cache && v_cache && slot_mapping, "paged_kv_append: null pointer");
     const int h = n_heads * head_dim, elts = 16 / (int)raven_host::elt_size(dtype);
     const dim3 grid((h / elts + 255) / 256, T);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == RAVEN_BF16) paged_kv_append_kernel<bf16><<<grid, dim3(256), 0, s>>>((const bf16*)k, (const bf16*)v, (bf16*)k_cache, (bf16*)v_cache, slot_mapping, h);
-    else paged_kv_append_kernel<float><<<grid, dim3(256), 0, s>>>((const float*)k, (const float*)v, (float*)k_cache, (float*)v_cache, slot_mapping, h);
+    if (dtype == RAVEN_BF16) paged_kv_append_kernel<bf16><<<grid, dim3(256), 0, s>>>((const bf16*)k, (const bf16*)v, (bf16*)k_cache, (bf16*)v_cache, slot_mapping, h, head_dim, block_size, ps, hs);
+    else paged_kv_append_kernel<float><<<grid, dim3(256), 0, s>>>((const float*)k, (const float*)v, (float*)k_cache, (float*)v_cache, slot_mapping, h, head_dim, block_size, ps, hs);
     return raven_host::check_launch("paged_kv_append");
 }
 
 static int paged_attention_common(const char* who, bool fused, const void* q, const void* bias, const float* freqs, void* y,
                                   const void* k_cache, const void* v_cache, const int32_t* block_table, const int32_t* seq_lens,
-                                  int32_t B, int32_t max_blocks, int32_t block_size, int32_t max_seq_len, int32_t n_heads,
-                                  int32_t head_dim, int32_t dtype, void* workspace, size_t workspace_bytes, void* stream) {
+                                  int32_t B, int32_t max_blocks, int32_t block_size, int32_t kv_layout, int32_t max_seq_len,
+                                  int32_t n_heads, int32_t head_dim, int32_t dtype, void* workspace, size_t workspace_bytes,
+                                  void* stream) {
     using namespace raven;
     if (int rc = check_heads(who, n_heads, head_dim, dtype)) return rc;
+    int64_t ps, hs;
+    if (int rc = paged_strides(who, kv_layout, block_size, n_heads, head_dim, &ps, &hs)) return rc;
     RAVEN_REQUIRE(B >= 0 && B <= 65535 && max_blocks > 0 && block_size > 0 && max_seq_len > 0, "%s: bad B=%d max_blocks=%d block_size=%d max_seq_len=%d", who, B, max_blocks, block_size, max_seq_len);
     if (B == 0) return 0;
     RAVEN_REQUIRE(q && y && k_cache && v_cache && block_table && seq_lens, "%s: null pointer", who);
@@ -681,7 +719,10 @@ static int paged_attention_common(const char* who, bool fused, const void* q, co
             ws_o = reinterpret_cast<float*>(static_cast<char*>(workspace) + raven_host::align_up((size_t)B * n_heads * kAttnMaxSplits * 2 * 4));
         }
     }
-    PagedView pv{k_cache, v_cache, block_table, seq_lens, max_blocks, block_size, n_heads, head_dim};
+    int shift = -1;
+    for (int b = 0; b < 31; ++b)
+        if (block_size == (1 << b)) shift = b;
+    PagedView pv{k_cache, v_cache, block_table, seq_lens, max_blocks, block_size, n_heads, head_dim, shift, ps, hs};
     const float scale_log2 = (float)(1.0 / sqrt((double)head_dim) * 1.4426950408889634);
     const dim3 grid(n_heads, B, ns);
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -704,16 +745,19 @@ static int paged_attention_common(const char* who, bool fused, const void* q, co
 
 extern "C" int raven_paged_decode_attention(const void* q, void* y, const void* k_cache, const void* v_cache,
                                             const int32_t* block_table, const int32_t* seq_lens, int32_t B, int32_t max_blocks,
-                                            int32_t block_size, int32_t max_seq_len, int32_t n_heads, int32_t head_dim, int32_t dtype,
-                                            void* workspace, size_t workspace_bytes, void* stream) {
+                                            int32_t block_size, int32_t kv_layout, int32_t max_seq_len, int32_t n_heads,
+                                            int32_t head_dim, int32_t dtype, void* workspace, size_t workspace_bytes, void* stream) {
     return paged_attention_common("paged_decode_attention", false, q, nullptr, nullptr, y, k_cache, v_cache, block_table, seq_lens, B,
-                                  max_blocks, block_size, max_seq_len, n_heads, head_dim, dtype, workspace, workspace_bytes, stream);
+                                  max_blocks, block_size, kv_layout, max_seq_len, n_heads, head_dim, dtype, workspace, workspace_bytes,
+                                  stream);
 }
 
 extern "C" int raven_paged_qkv_attention_decode(const void* qkv, const void* qk_bias, const float* freqs, void* y, void* k_cache,
                                                 void* v_cache, const int32_t* block_table, const int32_t* seq_lens, int32_t B,
-                                                int32_t max_blocks, int32_t block_size, int32_t max_seq_len, int32_t n_heads,
-                                                int32_t head_dim, int32_t dtype, void* workspace, size_t workspace_bytes, void* stream) {
+                                                int32_t max_blocks, int32_t block_size, int32_t kv_layout, int32_t max_seq_len,
+                                                int32_t n_heads, int32_t head_dim, int32_t dtype, void* workspace,
+                                                size_t workspace_bytes, void* stream) {
     return paged_attention_common("paged_qkv_attention_decode", true, qkv, qk_bias, freqs, y, k_cache, v_cache, block_table, seq_lens,
-                                  B, max_blocks, block_size, max_seq_len, n_heads, head_dim, dtype, workspace, workspace_bytes, stream);
+                                  B, max_blocks, block_size, kv_layout, max_seq_len, n_heads, head_dim, dtype, workspace, workspace_bytes,
+                                  stream);
 }

@@ -101,7 +101,7 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
     if (paged) {   // decode over block-paged caches, every sequence at its own position
         if ((rc = raven_paged_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, paged->k_caches[layer], paged->v_caches[layer],
                                                    paged->block_table, paged->seq_lens, B, paged->max_blocks, paged->block_size,
-                                                   paged->max_seq_len, d->n_heads, d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream))) return rc;
+                                                   paged->kv_layout, paged->max_seq_len, d->n_heads, d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream))) return rc;
     } else if (S == 1) {  // decode: bias, RoPE, cache append and attention in one launch
         if ((rc = raven_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, cache, slot, B, pos0, pos_dev, d->n_heads,
                                              d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream))) return rc;
@@ -136,7 +136,7 @@ static int run_block_one_row(const raven_dims* d, const raven_block_weights* w, 
     if (paged)
         rc = raven_paged_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, paged->k_caches[layer], paged->v_caches[layer],
                                               paged->block_table, paged->seq_lens, 1, paged->max_blocks, paged->block_size,
-                                              paged->max_seq_len, d->n_heads, d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream);
+                                              paged->kv_layout, paged->max_seq_len, d->n_heads, d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream);
     else
         rc = raven_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, cache, slot, 1, pos0, pos_dev, d->n_heads, d->head_dim, dt,
                                         s.attn_ws, s.attn_ws_bytes, stream);

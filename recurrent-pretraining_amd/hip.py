@@ -42,7 +42,22 @@ class KVCache(C.Structure):
 
 class PagedKV(C.Structure):
     _fields_ = [("k_caches", C.POINTER(C.c_void_p)), ("v_caches", C.POINTER(C.c_void_p)), ("block_table", C.c_void_p),
-                ("seq_lens", C.c_void_p), ("max_blocks", C.c_int32), ("block_size", C.c_int32), ("max_seq_len", C.c_int32)]
+                ("seq_lens", C.c_void_p), ("max_blocks", C.c_int32), ("block_size", C.c_int32), ("max_seq_len", C.c_int32),
+                ("kv_layout", C.c_int32)]
+
+
+PAGED_NHD, PAGED_HND = 0, 1
+
+
+def _paged_dims(cache: torch.Tensor, layout: int):
+    """(block_size, n_heads, head_dim) of a paged cache tensor: [blocks, block_size, nh, hd] (NHD) or [blocks, nh, block_size, hd]."""
+    if layout == PAGED_NHD:
+        _, bs, nh, hd = cache.shape
+    elif layout == PAGED_HND:
+        _, nh, bs, hd = cache.shape
+    else:
+        raise RavenHipError(f"unknown paged layout {layout}")
+    return bs, nh, hd
 
 
 LOOKUP_NONE, LOOKUP_SKIP, LOOKUP_LATEST, LOOKUP_ALWAYS_LAST = 0, 1, 2, 3
@@ -63,10 +78,11 @@ SIGNATURES = {
     "raven_linear": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _VP, _SZ, _VP]),
     "raven_exit_logit_stats": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I32, _VP]),
     "raven_exit_latent_stats": (C.c_int, [_VP, _VP, _VP, _VP, _I32, _I32, _I32, _VP]),
-    "raven_paged_kv_append": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _VP]),
-    "raven_paged_decode_attention": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _VP, _SZ, _VP]),
-    "raven_paged_qkv_attention_decode": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _VP, _SZ,
-                                                   _VP]),
+    "raven_paged_kv_append": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _VP]),
+    "raven_paged_decode_attention": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _VP, _SZ,
+                                               _VP]),
+    "raven_paged_qkv_attention_decode": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32,
+                                                   _VP, _SZ, _VP]),
     "raven_gemv_fused": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _F, _I32, _I32, _I32, _VP]),
     "raven_qkv_bias_rope_cache_append": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32,
                                                    _VP, _I32, _I32, _I32, _VP]),
@@ -241,39 +257,41 @@ def linear(x0, w, x1=None, residual=None, swiglu=False, out_f32=False, workspace
     return y
 
 
-def paged_kv_append(k, v, k_cache, v_cache, slot_mapping):
-    """k, v [T, nh * hd] -> k_cache / v_cache [num_blocks, block_size, nh, hd] at the flat slots slot_mapping [T] (int64)."""
+def paged_kv_append(k, v, k_cache, v_cache, slot_mapping, layout: int = PAGED_NHD):
+    """k, v [T, nh * hd] -> k_cache / v_cache (layout NHD: [num_blocks, block_size, nh, hd], HND: [num_blocks, nh, block_size, hd])
+    at the flat slots slot_mapping [T] (int64, block * block_size + offset)."""
     T = k.shape[0]
-    nh, hd = k_cache.shape[2], k_cache.shape[3]
+    bs, nh, hd = _paged_dims(k_cache, layout)
     rc = load().raven_paged_kv_append(_ptr(k, "k"), _ptr(v, "v", k.dtype), _ptr(k_cache, "k_cache", k.dtype), _ptr(v_cache, "v_cache", k.dtype),
-                                      _ptr(slot_mapping, "slot_mapping", torch.int64), T, nh, hd, dtype_code(k.dtype), _stream())
+                                      _ptr(slot_mapping, "slot_mapping", torch.int64), T, nh, hd, bs, layout, dtype_code(k.dtype), _stream())
     _check(rc, "raven_paged_kv_append")
 
 
-def paged_decode_attention(q, k_cache, v_cache, block_table, seq_lens, max_seq_len, workspace=None):
-    """q [B, nh * hd]; k_cache / v_cache [num_blocks, block_size, nh, hd]; block_table [B, max_blocks] int32; seq_lens [B] int32."""
+def paged_decode_attention(q, k_cache, v_cache, block_table, seq_lens, max_seq_len, workspace=None, layout: int = PAGED_NHD):
+    """q [B, nh * hd]; k_cache / v_cache as in paged_kv_append; block_table [B, max_blocks] int32; seq_lens [B] int32."""
     B = q.shape[0]
-    _, block_size, nh, hd = k_cache.shape
+    block_size, nh, hd = _paged_dims(k_cache, layout)
     y = torch.empty_like(q)
     rc = load().raven_paged_decode_attention(
         _ptr(q, "q"), _ptr(y, "y"), _ptr(k_cache, "k_cache", q.dtype), _ptr(v_cache, "v_cache", q.dtype),
         _ptr(block_table, "block_table", torch.int32), _ptr(seq_lens, "seq_lens", torch.int32), B, block_table.shape[1], block_size,
-        int(max_seq_len), nh, hd, dtype_code(q.dtype), _ptr(workspace, "workspace", torch.uint8),
+        layout, int(max_seq_len), nh, hd, dtype_code(q.dtype), _ptr(workspace, "workspace", torch.uint8),
         0 if workspace is None else workspace.numel(), _stream())
     _check(rc, "raven_paged_decode_attention")
     return y
 
 
-def paged_qkv_attention_decode(qkv, qk_bias, freqs, k_cache, v_cache, block_table, seq_lens, max_seq_len, workspace=None):
+def paged_qkv_attention_decode(qkv, qk_bias, freqs, k_cache, v_cache, block_table, seq_lens, max_seq_len, workspace=None,
+                               layout: int = PAGED_NHD):
     """The decode step of a paged attention layer in one launch: qkv [B, 3 * nh * hd] from the fused projection; bias, RoPE at
     position seq_lens[b] - 1, write of the new k / v row to its page, attention over seq_lens[b] positions.  Returns y [B, nh * hd]."""
     B = qkv.shape[0]
-    _, block_size, nh, hd = k_cache.shape
+    block_size, nh, hd = _paged_dims(k_cache, layout)
     y = torch.empty(B, nh * hd, device=qkv.device, dtype=qkv.dtype)
     rc = load().raven_paged_qkv_attention_decode(
         _ptr(qkv, "qkv"), _ptr(qk_bias, "qk_bias", qkv.dtype), _ptr(freqs, "freqs", torch.float32), _ptr(y, "y"),
         _ptr(k_cache, "k_cache", qkv.dtype), _ptr(v_cache, "v_cache", qkv.dtype), _ptr(block_table, "block_table", torch.int32),
-        _ptr(seq_lens, "seq_lens", torch.int32), B, block_table.shape[1], block_size, int(max_seq_len), nh, hd, dtype_code(qkv.dtype),
+        _ptr(seq_lens, "seq_lens", torch.int32), B, block_table.shape[1], block_size, layout, int(max_seq_len), nh, hd, dtype_code(qkv.dtype),
         _ptr(workspace, "workspace", torch.uint8), 0 if workspace is None else workspace.numel(), _stream())
     _check(rc, "raven_paged_qkv_attention_decode")
     return y
@@ -441,8 +459,8 @@ def core_iterations(dims: Dims, adapter_w, blocks, state_in, embeds, state_out, 
     return state_out
 
 
-def make_paged_kv(k_caches, v_caches, block_table, seq_lens, max_seq_len: int) -> PagedKV:
-    """k_caches / v_caches: one [num_blocks, block_size, nh, hd] tensor per block of the stack; block_table [B, max_blocks] and
+def make_paged_kv(k_caches, v_caches, block_table, seq_lens, max_seq_len: int, layout: int = PAGED_NHD) -> PagedKV:
+    """k_caches / v_caches: one paged cache tensor (as in paged_kv_append) per block of the stack; block_table [B, max_blocks] and
     seq_lens [B] int32 on the GPU.  The returned structure holds pointers only: keep the tensors alive."""
     if len(k_caches) != len(v_caches) or not k_caches:
         raise RavenHipError("make_paged_kv: one key and one value cache per block")
@@ -455,7 +473,7 @@ def make_paged_kv(k_caches, v_caches, block_table, seq_lens, max_seq_len: int) -
     if block_table.dim() != 2 or seq_lens.shape != (block_table.shape[0],):
         raise RavenHipError("make_paged_kv: block_table [B, max_blocks], seq_lens [B]")
     kv = PagedKV(C.cast(ka, C.POINTER(C.c_void_p)), C.cast(va, C.POINTER(C.c_void_p)), _ptr(block_table, "block_table", torch.int32),
-                 _ptr(seq_lens, "seq_lens", torch.int32), block_table.shape[1], shape[1], int(max_seq_len))
+                 _ptr(seq_lens, "seq_lens", torch.int32), block_table.shape[1], _paged_dims(k_caches[0], layout)[0], int(max_seq_len), layout)
     kv._keep = (ka, va)  # the pointer arrays live in host memory owned by this object
     return kv
 

@@ -25,7 +25,8 @@ PAGED_STRATEGY = "latest-m4-compress-s4"
 
 
 class PagedDecoder:
-    def __init__(self, model, num_blocks: int, block_size: int = 16, num_steps: Optional[int] = None, use_graph: bool = False):
+    def __init__(self, model, num_blocks: int, block_size: int = 16, num_steps: Optional[int] = None, use_graph: bool = False,
+                 layout: str = "HND"):
         cfg = model.config
         if (cfg.n_layers_in_prelude, cfg.n_layers_in_recurrent_block) != (2, 4):
             # the equivalence with the cache-sharing strategy of the other surface hard-codes these counts (RMM:169-182)
@@ -37,7 +38,13 @@ class PagedDecoder:
         self.block_size, self.num_blocks = int(block_size), int(num_blocks)
         dev, dt = model.device, model.dtype
         self.n_flat = cfg.n_layers_in_prelude + cfg.n_layers_in_recurrent_block + cfg.n_layers_in_coda
-        shape = (self.num_blocks, self.block_size, cfg.n_heads, cfg.head_dim)
+        # "NHD": [num_blocks, block_size, n_heads, head_dim]; "HND": [num_blocks, n_heads, block_size, head_dim], where a
+        # head's positions of a block are contiguous (the attention kernel reads it about 15 % faster)
+        if layout not in ("NHD", "HND"):
+            raise ValueError(f"unknown layout {layout!r}")
+        self.layout = hip.PAGED_NHD if layout == "NHD" else hip.PAGED_HND
+        shape = ((self.num_blocks, self.block_size, cfg.n_heads, cfg.head_dim) if layout == "NHD" else
+                 (self.num_blocks, cfg.n_heads, self.block_size, cfg.head_dim))
         self.k = [torch.zeros(shape, dtype=dt, device=dev) for _ in range(self.n_flat)]
         self.v = [torch.zeros(shape, dtype=dt, device=dev) for _ in range(self.n_flat)]
         self._ws = {}
@@ -70,7 +77,7 @@ class PagedDecoder:
             s = cache._slot(step)
             k = cache._k[s, row, :, :n].transpose(0, 1).reshape(n, h).contiguous()
             v = cache._v[s, row, :, :n].transpose(0, 1).reshape(n, h).contiguous()
-            hip.paged_kv_append(k, v, self.k[f], self.v[f], slots)
+            hip.paged_kv_append(k, v, self.k[f], self.v[f], slots, layout=self.layout)
         return n
 
     def prefill(self, input_ids: torch.Tensor, table_row: Sequence[int], input_states: Optional[torch.Tensor] = None):
@@ -106,7 +113,7 @@ class PagedDecoder:
         nat = m._natives()
         max_len = buf["table"].shape[1] * self.block_size  # sizes the launch only; lengths are read on the device
         n_pre, n_core = cfg.n_layers_in_prelude, cfg.n_layers_in_recurrent_block
-        kvs = [hip.make_paged_kv(self.k[a:b], self.v[a:b], buf["table"], buf["lens"], max_len)
+        kvs = [hip.make_paged_kv(self.k[a:b], self.v[a:b], buf["table"], buf["lens"], max_len, layout=self.layout)
                for a, b in ((0, n_pre), (n_pre, n_pre + n_core), (n_pre + n_core, self.n_flat))]
         hip.embed(t.wte.weight, buf["ids"], m.emb_scale, out=buf["embeds"])
         pre = (hip.BlockWeights * n_pre)(*nat["prelude"])

@@ -605,13 +605,17 @@ def test_fp32_kernels_at_the_3_5b_shape(pkg):
 
 
 # ----------------------------------------------------------------------------- paged KV cache (vLLM layout)
-@pytest.mark.parametrize("dt,nh,hd,B,block_size", [(torch.bfloat16, 55, 96, 1, 16), (torch.bfloat16, 55, 96, 32, 16),
-                                                   (torch.bfloat16, 55, 96, 5, 32), (torch.float32, 4, 64, 3, 8),
-                                                   (torch.float32, 5, 96, 2, 16)])
-def test_paged_decode_attention_and_append(pkg, dt, nh, hd, B, block_size):
+@pytest.mark.parametrize("dt,nh,hd,B,block_size,layout", [(torch.bfloat16, 55, 96, 1, 16, "NHD"), (torch.bfloat16, 55, 96, 32, 16, "NHD"),
+                                                          (torch.bfloat16, 55, 96, 5, 32, "HND"), (torch.float32, 4, 64, 3, 8, "NHD"),
+                                                          (torch.float32, 5, 96, 2, 16, "HND"), (torch.bfloat16, 55, 96, 32, 16, "HND"),
+                                                          (torch.bfloat16, 4, 64, 3, 12, "HND"), (torch.bfloat16, 4, 64, 3, 12, "NHD")])
+def test_paged_decode_attention_and_append(pkg, dt, nh, hd, B, block_size, layout):
     """Block-paged K/V with shuffled block tables and a different length per sequence (1 and 0 among them): appended rows
-    land in their slots, attention equals torch SDPA per sequence, and -- for equal lengths -- the contiguous kernel's bits."""
+    land in their slots, attention equals torch SDPA per sequence, and -- for equal lengths -- the contiguous kernel's bits.
+    Both page layouts ([blocks, block_size, heads, hd] and [blocks, heads, block_size, hd]); a block size that is no power of two."""
     h = nh * hd
+    lay = pkg.hip.PAGED_NHD if layout == "NHD" else pkg.hip.PAGED_HND
+    rows_of = (lambda c: c.view(-1, nh, hd)) if layout == "NHD" else (lambda c: c.permute(0, 2, 1, 3).reshape(-1, nh, hd))
     g = torch.Generator().manual_seed(600 + B)
     max_len = 700
     max_blocks = (max_len + block_size - 1) // block_size
@@ -622,7 +626,7 @@ def test_paged_decode_attention_and_append(pkg, dt, nh, hd, B, block_size):
         lens[1], lens[2] = 1, 0
     table = torch.randperm(num_blocks, generator=g)[:B * max_blocks].view(B, max_blocks).to(torch.int32)
     k_seq, v_seq = rnd((B, max_len, nh, hd), dt, 601), rnd((B, max_len, nh, hd), dt, 602)
-    kc = torch.zeros(num_blocks, block_size, nh, hd, dtype=dt, device="cuda")
+    kc = torch.zeros((num_blocks, block_size, nh, hd) if layout == "NHD" else (num_blocks, nh, block_size, hd), dtype=dt, device="cuda")
     vc = torch.zeros_like(kc)
     # fill the cache through the append kernel: every sequence's positions, in one call, plus a skipped row
     rows_k, rows_v, slots = [], [], []
@@ -636,8 +640,9 @@ def test_paged_decode_attention_and_append(pkg, dt, nh, hd, B, block_size):
     slots.append(-1)
     kk, vv, sl = torch.stack(rows_k).cuda(), torch.stack(rows_v).cuda(), torch.tensor(slots, dtype=torch.int64).cuda()
     for lo in range(0, kk.shape[0], 60000):
-        pkg.hip.paged_kv_append(kk[lo:lo + 60000].contiguous(), vv[lo:lo + 60000].contiguous(), kc, vc, sl[lo:lo + 60000].contiguous())
-    flat_k = kc.view(-1, nh, hd).cpu()
+        pkg.hip.paged_kv_append(kk[lo:lo + 60000].contiguous(), vv[lo:lo + 60000].contiguous(), kc, vc, sl[lo:lo + 60000].contiguous(),
+                                layout=lay)
+    flat_k = rows_of(kc).cpu()
     for b in range(B):
         for p in (0, int(lens[b]) - 1):
             if p >= 0 and int(lens[b]) > 0:
@@ -646,7 +651,7 @@ def test_paged_decode_attention_and_append(pkg, dt, nh, hd, B, block_size):
     q = rnd((B, h), dt, 603)
     ws = pkg.hip.attention_workspace(B, nh, hd, "cuda")
     for wsp in (ws, None):
-        y = pkg.hip.paged_decode_attention(q.cuda(), kc, vc, table.cuda(), lens.cuda(), max_len, workspace=wsp)
+        y = pkg.hip.paged_decode_attention(q.cuda(), kc, vc, table.cuda(), lens.cuda(), max_len, workspace=wsp, layout=lay)
         for b in range(B):
             n = int(lens[b])
             if n == 0:
@@ -658,7 +663,7 @@ def test_paged_decode_attention_and_append(pkg, dt, nh, hd, B, block_size):
     # equal lengths: the same numbers as the contiguous cache kernel gives (same arithmetic, other addresses)
     n = 300
     eq = torch.full((B,), n, dtype=torch.int32)
-    y = pkg.hip.paged_decode_attention(q.cuda(), kc, vc, table.cuda(), eq.cuda(), n)
+    y = pkg.hip.paged_decode_attention(q.cuda(), kc, vc, table.cuda(), eq.cuda(), n, layout=lay)
     kd = torch.zeros(1, B, nh, n, hd, dtype=dt)
     vd = torch.zeros_like(kd)
     for b in range(B):
@@ -669,7 +674,7 @@ def test_paged_decode_attention_and_append(pkg, dt, nh, hd, B, block_size):
     full = [b for b in range(B) if int(lens[b]) >= n]
     check(y[full], want[full].float().cpu(), dt, "paged vs contiguous")
     with pytest.raises(pkg.hip.RavenHipError):
-        pkg.hip.paged_decode_attention(q.cuda(), kc, vc, table.cuda(), lens.cuda(), max_blocks * block_size + 1)
+        pkg.hip.paged_decode_attention(q.cuda(), kc, vc, table.cuda(), lens.cuda(), max_blocks * block_size + 1, layout=lay)
 
     # The fused decode step: sequence b's new token at position lens[b] - 1 (its page currently holds k_seq / v_seq of
     # that position, which the step overwrites).  Against the oracle's bias + RoPE per sequence, the append kernel and
@@ -680,7 +685,8 @@ def test_paged_decode_attention_and_append(pkg, dt, nh, hd, B, block_size):
     freqs = rope.float().reshape(max_len, hd // 2, 2).contiguous().cuda()
     kc2, vc2 = kc.clone(), vc.clone()
     for wsp in (ws, None):
-        y_f = pkg.hip.paged_qkv_attention_decode(qkv.cuda(), bias.cuda(), freqs, kc, vc, table.cuda(), lens.cuda(), max_len, workspace=wsp)
+        y_f = pkg.hip.paged_qkv_attention_decode(qkv.cuda(), bias.cuda(), freqs, kc, vc, table.cuda(), lens.cuda(), max_len, workspace=wsp,
+                                                 layout=lay)
     rows_q, rows_k, rows_v, slots = [], [], [], []
     for b in range(B):
         n = int(lens[b])
@@ -693,9 +699,10 @@ def test_paged_decode_attention_and_append(pkg, dt, nh, hd, B, block_size):
         rq, rk = O.apply_rope(qq, kk, rope[:, n - 1:n])
         rows_q.append(rq.reshape(h)); rows_k.append(rk.reshape(h)); rows_v.append(vv.reshape(h))
         slots.append(int(table[b, (n - 1) // block_size]) * block_size + (n - 1) % block_size)
-    pkg.hip.paged_kv_append(torch.stack(rows_k).cuda(), torch.stack(rows_v).cuda(), kc2, vc2, torch.tensor(slots, dtype=torch.int64).cuda())
-    y_2 = pkg.hip.paged_decode_attention(torch.stack(rows_q).cuda(), kc2, vc2, table.cuda(), lens.cuda(), max_len, workspace=ws)
+    pkg.hip.paged_kv_append(torch.stack(rows_k).cuda(), torch.stack(rows_v).cuda(), kc2, vc2, torch.tensor(slots, dtype=torch.int64).cuda(),
+                            layout=lay)
+    y_2 = pkg.hip.paged_decode_attention(torch.stack(rows_q).cuda(), kc2, vc2, table.cuda(), lens.cuda(), max_len, workspace=ws, layout=lay)
     check(y_f, y_2.float().cpu(), dt, "fused paged step vs rope + append + attention")
     check(kc, kc2.float().cpu(), dt, "keys after the fused paged step")
     assert torch.equal(vc, vc2)
-    assert int((kc.view(-1, nh, hd).abs().amax(dim=(1, 2)) > 0).sum()) == int(lens.sum())  # no other row was touched
+    assert int((rows_of(kc).abs().amax(dim=(1, 2)) > 0).sum()) == int(lens.sum())  # no other row was touched

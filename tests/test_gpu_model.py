@@ -378,9 +378,9 @@ def test_generate_speculative_matches_oracle(pkg, small242, B, draft_steps, L, v
         assert n >= 5 + 9 and torch.equal(plain[:, :n], spec[:, :n])
 
 
-@pytest.mark.parametrize("lens,use_graph", [((7, 3, 12, 5, 9, 2), False), ((6,), False), ((4, 4), False), ((7, 3, 12, 5, 9, 2), True),
-                                            ((6,), True)])
-def test_paged_decoder_serves_sequences_of_different_lengths(pkg, small242, lens, use_graph):
+@pytest.mark.parametrize("lens,use_graph,layout", [((7, 3, 12, 5, 9, 2), False, "HND"), ((6,), False, "NHD"), ((4, 4), False, "HND"),
+                                                   ((7, 3, 12, 5, 9, 2), True, "NHD"), ((6,), True, "HND")])
+def test_paged_decoder_serves_sequences_of_different_lengths(pkg, small242, lens, use_graph, layout):
     """Block-paged caches, one per flat layer, shared by all recurrences (the cache of the reference's vLLM plugin):
     every sequence is prefilled on its own, then all decode together, each at its own position.  Per sequence the
     logits equal the oracle's forward with the cache-sharing strategy that has the same semantics on the other surface
@@ -391,7 +391,7 @@ def test_paged_decoder_serves_sequences_of_different_lengths(pkg, small242, lens
     g = torch.Generator().manual_seed(77 + B)
     max_blocks = (max(lens) + n_new + bs - 1) // bs
     table = torch.randperm(B * max_blocks + 5, generator=g)[:B * max_blocks].view(B, max_blocks).to(torch.int32)
-    dec = pkg.PagedDecoder(model, num_blocks=B * max_blocks + 5, block_size=bs, num_steps=r, use_graph=use_graph)
+    dec = pkg.PagedDecoder(model, num_blocks=B * max_blocks + 5, block_size=bs, num_steps=r, use_graph=use_graph, layout=layout)
     prompts = [torch.randint(0, s.vocab_size, (1, n), generator=g) for n in lens]
     new_ids = torch.randint(0, s.vocab_size, (B, n_new), generator=g)
     states = [O.initialize_state(torch.empty(1, n + n_new, s.n_embd), s, 1.0, g) for n in lens]
@@ -419,7 +419,7 @@ def test_paged_decoder_serves_sequences_of_different_lengths(pkg, small242, lens
     # a position outside the table is an error of the caller that the entry point catches by size
     with pytest.raises(pkg.hip.RavenHipError):
         pkg.hip.paged_decode_blocks(model._natives()["dims"], model._natives()["core"], latents, latents.clone(), model._natives()["freqs"],
-                                    pkg.hip.make_paged_kv(dec.k[2:6], dec.v[2:6], table_d, seq_lens, max_blocks * bs), B,
+                                    pkg.hip.make_paged_kv(dec.k[2:6], dec.v[2:6], table_d, seq_lens, max_blocks * bs, layout=dec.layout), B,
                                     torch.empty(16, dtype=torch.uint8, device="cuda"))
     with pytest.raises(ValueError):
         dec.load_prompt(pkg.HuginnDynamicCache(), 0, table[0].tolist())
