@@ -18,6 +18,19 @@
 
 namespace raven {
 
+// One RoPE pair, adjacent elements (recpre/raven_modeling_minimal.py:118-131): products and sums rounded one by one in
+// fp32, as the reference's separate elementwise kernels do; every kernel that rotates uses this one function, so that
+// the fused and the two-launch paths write the same bits.
+template <typename T>
+__device__ __forceinline__ void rope_pair(T& a, T& b, float cs, float sn) {
+#pragma clang fp contract(off)
+    const float x0 = to_f32(a), x1 = to_f32(b);
+    const float r0 = x0 * cs - x1 * sn;
+    const float r1 = x1 * cs + x0 * sn;
+    a = from_f32<T>(r0);
+    b = from_f32<T>(r1);
+}
+
 struct CacheView {
     void* k;
     void* v;
@@ -75,12 +88,7 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(
         }
         const float* f = freqs + ((int64_t)pos * (cv.hd / 2) + d / 2) * 2;
 #pragma unroll
-        for (int e = 0; e < E; e += 2) {
-            const float cs = f[e], sn = f[e + 1];
-            const float x0 = to_f32(x.v[e]), x1 = to_f32(x.v[e + 1]);
-            x.v[e] = from_f32<T>(x0 * cs - x1 * sn);
-            x.v[e + 1] = from_f32<T>(x1 * cs + x0 * sn);
-        }
+        for (int e = 0; e < E; e += 2) rope_pair<T>(x.v[e], x.v[e + 1], f[e], f[e + 1]);
     }
     if (sec == 0) {
         store_chunk(q_out + (int64_t)m * h + col, x);
@@ -97,25 +105,40 @@ constexpr int kAttnMaxHd = 128;
 extern "C" size_t raven_decode_attention_workspace_bytes(int32_t M, int32_t n_heads, int32_t head_dim);
 namespace raven {
 
-// bias + RoPE of one 16-byte chunk of a q or k head row (sec 0 = q, 1 = k); d = first column of the chunk
+// bias + RoPE of one 16-byte chunk of a q or k head row (sec 0 = q, 1 = k); d = first column of the chunk.
+// The operands (bias chunk, cos/sin pairs) are loaded by rope_operands so that a caller can issue those loads
+// ahead of others it will wait for anyway.
+template <typename T>
+struct RopeOperands {
+    Chunk<T> bias;
+    float cs[Chunk<T>::N];  // (cos, sin) of the chunk's N / 2 pairs
+};
+template <typename T>
+__device__ __forceinline__ RopeOperands<T> rope_operands(const T* __restrict__ qk_bias, int sec, int h, int col,
+                                                         const float* __restrict__ freqs, int pos, int hd, int d) {
+    constexpr int E = Chunk<T>::N;
+    RopeOperands<T> r;
+    r.bias = qk_bias ? load_chunk(qk_bias + sec * h + col) : zero_chunk<T>();
+    const float* f = freqs + ((int64_t)pos * (hd / 2) + d / 2) * 2;
+#pragma unroll
+    for (int e = 0; e < E; e += 4) *reinterpret_cast<float4*>(&r.cs[e]) = *reinterpret_cast<const float4*>(f + e);
+    return r;
+}
+template <typename T>
+__device__ __forceinline__ Chunk<T> bias_rope_apply(Chunk<T> x, const RopeOperands<T>& op, bool has_bias) {
+    constexpr int E = Chunk<T>::N;
+    if (has_bias) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) x.v[e] = from_f32<T>(to_f32(x.v[e]) + to_f32(op.bias.v[e]));
+    }
+#pragma unroll
+    for (int e = 0; e < E; e += 2) rope_pair<T>(x.v[e], x.v[e + 1], op.cs[e], op.cs[e + 1]);
+    return x;
+}
 template <typename T>
 __device__ __forceinline__ Chunk<T> bias_rope_chunk(Chunk<T> x, const T* __restrict__ qk_bias, int sec, int h, int col,
                                                     const float* __restrict__ freqs, int pos, int hd, int d) {
-    constexpr int E = Chunk<T>::N;
-    if (qk_bias) {
-        const Chunk<T> bch = load_chunk(qk_bias + sec * h + col);
-#pragma unroll
-        for (int e = 0; e < E; ++e) x.v[e] = from_f32<T>(to_f32(x.v[e]) + to_f32(bch.v[e]));
-    }
-    const float* f = freqs + ((int64_t)pos * (hd / 2) + d / 2) * 2;
-#pragma unroll
-    for (int e = 0; e < E; e += 2) {
-        const float cs = f[e], sn = f[e + 1];
-        const float x0 = to_f32(x.v[e]), x1 = to_f32(x.v[e + 1]);
-        x.v[e] = from_f32<T>(x0 * cs - x1 * sn);
-        x.v[e + 1] = from_f32<T>(x1 * cs + x0 * sn);
-    }
-    return x;
+    return bias_rope_apply<T>(x, rope_operands<T>(qk_bias, sec, h, col, freqs, pos, hd, d), qk_bias != nullptr);
 }
 
 // What one lane holds of a position's head row: CPL neighbouring 16-byte chunks (1, or 2 for fp32 heads wider than
@@ -225,14 +248,22 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
             }
         }
     };
+    RopeOperands<T> opq[CPL], opk[CPL];
+    if (FUSED && active) {
+#pragma unroll
+        for (int i = 0; i < CPL; ++i) {
+            opq[i] = rope_operands<T>(qk_bias, 0, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
+            opk[i] = rope_operands<T>(qk_bias, 1, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
+        }
+    }
     load_tile(start);
 
     P qc = qraw, knew = kraw;
     if (FUSED && active) {
 #pragma unroll
         for (int i = 0; i < CPL; ++i) {
-            qc.c[i] = bias_rope_chunk<T>(qraw.c[i], qk_bias, 0, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
-            knew.c[i] = bias_rope_chunk<T>(kraw.c[i], qk_bias, 1, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
+            qc.c[i] = bias_rope_apply<T>(qraw.c[i], opq[i], qk_bias != nullptr);
+            knew.c[i] = bias_rope_apply<T>(kraw.c[i], opk[i], qk_bias != nullptr);
         }
         if (group == 0 && pos >= start && pos < end) {
             store_piece<T, CPL>(static_cast<T*>(cv.k) + head_off + (int64_t)pos * hd + ci * E, knew);
