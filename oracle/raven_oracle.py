@@ -32,6 +32,12 @@ How each function is pinned (tests/test_oracle_pins.py), without running the ref
   embed_inputs / iterate_one_step / predict_from_latents / generate_with_adaptive_compute
                      pieces compose to forward(); criterion "none" equals greedy_generate;
                      num-steps evaluator equals forward(num_steps=k) token by token -> pinned
+  generate_diffusion_style   the first position of the wave followed by hand (its embedding average, noise
+                     mixing and recurrences over several steps, on a private copy of the prompt cache)
+                     gives the token the loop freezes there; schedule / counter closed forms for the
+                     "fixed" strategy and for exit thresholds 0 and infinity.  The later positions' tokens
+                     (whose inputs change from step to step) have no independent check: parity unpinned
+                     beyond that                                                     -> partly pinned
 The reference holds no golden vectors for this path (it has no test suite); the only
 exact numbers it publishes are three KV-cache sizes, used as known-answer tests.
 """
@@ -773,6 +779,194 @@ def generate_speculative(w, s: RavenShape, input_ids: torch.Tensor, max_new_toke
     if record is not None:
         record["accepted"], record["cache"], record["forwards"] = accepted, cache, calls[0]
     return ids
+
+
+# --------------------------------------------------------------------------------------
+# diffusion-style sampler (RMM:1234-1549): a wave of not-yet-frozen positions is re-run
+# every step with a few recurrences, its cache entries are rolled back, positions freeze
+# from the left
+# --------------------------------------------------------------------------------------
+def generate_diffusion_style(w, s: RavenShape, input_ids: torch.Tensor, max_new_tokens: int, *, num_steps: int = 32,
+                             inner_recurrence: int = 4, headway: int = 1, freeze_strategy: str = "latent-diff",
+                             exit_t: float = 0.03, ema_embeds: float = 0.1, state_noise_mixing: float = 0.5,
+                             dampened_state_mixer: bool = True, sqrt_mixer: bool = False, continuous_compute: bool = False,
+                             full_prefill: bool = True, max_wavefront: int = 128, max_diffusion_steps: int = 4096,
+                             init_scale: float = 1.0, cache_lookup_strategy: str = "latest-m4-compress-s4", state_fn=None,
+                             extra_token_fn=None, extra_token_high: int = 65510, stop_tokens=(), record: Optional[dict] = None):
+    """Greedy generate_diffusion_style for one sequence.  `state_fn(draw, shape)` supplies the draw-th random latent state
+    (the prefill's initial state, the first wave state, then per step the noise states and the states of new positions,
+    in the order the loop draws them); `extra_token_fn(step, n)` the n = headway - 1 filler tokens of a step."""
+    assert input_ids.shape[0] == 1, "one sequence"
+    n_prompt, h = input_ids.shape[1], s.n_embd
+    dt = w["transformer.wte.weight"].dtype
+    cache = DictCache(cache_lookup_strategy)
+    draws = [0]
+
+    def draw(shape, via_bf16=False):
+        x = state_fn(draws[0], shape) if state_fn is not None else initialize_state(torch.empty(shape), s, init_scale)
+        draws[0] += 1
+        # new positions and the prompt-wide wave are drawn from a bf16 template in the reference (RMM:1302, 1375-1378)
+        return (x.to(torch.bfloat16) if via_bf16 else x).to(dt)
+
+    width = max(s.block_size, n_prompt + max_new_tokens + headway + int(full_prefill))
+    rec_count = torch.zeros(1, width, dtype=torch.long)   # recurrences spent per position
+    stable = torch.zeros(1, width, dtype=torch.long)      # steps in which a position's token did not change
+    passes = tokens_forward = clears = standing = 0
+
+    if full_prefill:                                                      # RMM:1289-1299
+        out = forward(w, s, input_ids=input_ids, input_states=draw((1, n_prompt, h)), num_steps=num_steps, past_key_values=cache,
+                      use_cache=True, cache_position=torch.arange(n_prompt), init_scale=init_scale)
+        passes, tokens_forward = passes + 1, tokens_forward + n_prompt
+        frozen = current = torch.cat([input_ids, out.logits[:, -1, :].argmax(-1, keepdim=True)], dim=-1)
+        rec_count[:, :frozen.shape[1]] += num_steps
+        states = draw((1, 1, h))
+    else:                                                                 # RMM:1300-1309
+        states = draw((1, n_prompt, h), via_bf16=True)
+        frozen, current = input_ids.clone(), input_ids.clone()
+        if 0 < max_wavefront < states.shape[1]:
+            raise ValueError("prompt longer than max_wavefront: use full_prefill")
+
+    if ema_embeds > 0.0:
+        old_embeds, _ = embed_inputs(w, s, current)                        # without a cache (RMM:1311-1312)
+    latent = "latent" in freeze_strategy
+    accel = "latent-acceleration" in freeze_strategy
+    if latent:
+        prev_states = states.clone()
+    if accel:
+        prev_delta, prev_prev_states, old_old_ci = torch.zeros_like(states), torch.zeros_like(states), 0
+    old_ci, old_k, k, step = 0, 0, 0, 0
+    log = []
+
+    while frozen.shape[1] - n_prompt < max_new_tokens and current.shape[1] <= s.block_size:
+        ci = cache.get_seq_length()
+        n_wave = states.shape[1]
+        pos = torch.arange(ci, ci + n_wave)
+        new_embeds, block_idx = embed_inputs(w, s, current[:, pos], cache=cache, cache_position=pos)
+        if ema_embeds > 0.0:                                               # RMM:1337-1342
+            carry = old_embeds[:, ci - old_ci:]
+            embeds = new_embeds.clone() * (1 - ema_embeds)
+            embeds[:, :carry.shape[1], :] += carry * ema_embeds
+            old_embeds = embeds.clone()
+        else:
+            embeds = new_embeds
+        if state_noise_mixing > 0:                                         # RMM:1346-1357
+            noise_states = draw(tuple(states.shape))
+            if dampened_state_mixer:
+                mix = (state_noise_mixing / (1 + rec_count[:, ci:ci + n_wave]))[:, :, None].to(states.dtype)
+            else:
+                mix = torch.as_tensor(state_noise_mixing, dtype=states.dtype)
+            if sqrt_mixer:
+                states = states * F.relu(1 - mix).sqrt() + mix.sqrt() * noise_states
+            else:
+                states = states * (1 - mix) + mix * noise_states
+        for _ in range(inner_recurrence):                                  # RMM:1358-1362
+            states, block_idx = iterate_one_step(w, s, embeds, states, block_idx, cache=cache, cache_position=pos)
+            rec_count[:, ci:ci + n_wave] += 1
+            passes, tokens_forward = passes + 1, tokens_forward + n_wave
+        logits = predict_from_latents(w, s, states, cache=cache, cache_position=pos).logits
+        first_state, first_logits = states[0, 0].clone(), logits[0, 0].clone()  # of the wave's leftmost position, for the record
+        # positions whose prediction is not frozen yet: from the last frozen token on (RMM:1366-1369)
+        new_tokens = logits[0, max(frozen.shape[1] - 1 - ci, 0):, :].argmax(-1, keepdim=True).T
+        guess = torch.cat([frozen, new_tokens[:, :-1]], dim=1)
+        stable[:, :current.shape[1]] += current == guess
+        if extra_token_fn is not None:
+            extra = extra_token_fn(step, headway - 1).view(1, headway - 1)
+        else:
+            extra = torch.randint(0, extra_token_high, (1, headway - 1))
+        current = torch.cat([frozen, new_tokens, extra], dim=1)
+        if continuous_compute and states.shape[1] >= headway:
+            fresh = states[:, -headway:].clone()
+        else:
+            fresh = draw((1, headway, h), via_bf16=True)
+        states = torch.cat([states, fresh], dim=1)
+        headway_now = headway
+        if max_wavefront > 0 and states.shape[1] > max_wavefront:          # RMM:1384-1394: the wave stops growing
+            headway_now = max_wavefront - (states.shape[1] - headway)
+            states = states[:, :max_wavefront]
+            current = current[:, :ci + max_wavefront]
+            standing += 1
+
+        def freeze_up_to(k_new):                                           # RMM:1437-1444 and its two siblings
+            nonlocal states, frozen, clears
+            n_clear = current.shape[1] - headway_now - k_new + 1
+            cache.clear_last_k_entries(n_clear)
+            clears += n_clear
+            states = states[:, k_new - ci - 1:, :]
+            frozen = current[:, :k_new]
+
+        def freeze_nothing():
+            nonlocal clears
+            cache.clear_last_k_entries(states.shape[1] - headway_now)
+            clears += states.shape[1] - headway_now
+
+        if latent:
+            if freeze_strategy == "latent-diff":                           # RMM:1396-1400
+                old = prev_states[:, ci - old_ci:]
+                cur = states[:, :old.shape[1], :]
+                criterion = (cur - old).norm(dim=-1) / cur.norm(dim=-1)
+            elif freeze_strategy == "latent-acceleration-1":               # RMM:1401-1412
+                old = prev_states[:, ci - old_ci:]
+                cur = states[:, :old.shape[1], :]
+                delta = cur - old
+                m = min(delta.shape[1], prev_delta.shape[1])
+                criterion = (delta[:, :m, :] - prev_delta[:, :m, :]).norm(dim=-1) / cur[:, :m, :].norm(dim=-1)
+                prev_delta = delta.clone()
+            elif freeze_strategy == "latent-acceleration-2":               # RMM:1414-1435
+                lo = max(ci, old_ci, old_old_ci)
+                hi = min(ci + states.shape[1], old_ci + prev_states.shape[1], old_old_ci + prev_prev_states.shape[1])
+                a, b, c = states[:, lo - ci:hi - ci], prev_states[:, lo - old_ci:hi - old_ci], \
+                    prev_prev_states[:, lo - old_old_ci:hi - old_old_ci]
+                criterion = ((a - b) - (b - c)).norm(dim=-1) / (a.norm(dim=-1) + 1e-6)
+            else:
+                raise ValueError(freeze_strategy)
+            exits = criterion < exit_t
+            if exits.sum() > 0:
+                k = ci + int(exits.nonzero()[-1][1]) + 1
+                freeze_up_to(k)
+            else:
+                freeze_nothing()
+        elif freeze_strategy == "token-stability":                         # RMM:1450-1463
+            ripe = stable > num_steps // inner_recurrence
+            if torch.any(ripe):
+                k = int(ripe.nonzero()[-1][1]) + 1
+                freeze_up_to(k)
+            else:
+                freeze_nothing()
+                k = 0
+        elif freeze_strategy == "fixed":                                   # RMM:1464-1474
+            if step > num_steps // inner_recurrence:
+                n_clear = states.shape[1] - headway - headway_now
+                cache.clear_last_k_entries(n_clear)
+                clears += n_clear
+                states = states[:, headway_now:, :]
+                frozen = torch.cat([frozen, new_tokens[:, :headway_now]], dim=-1)
+            else:
+                freeze_nothing()
+        else:
+            raise ValueError(f"Invalid freeze strategy {freeze_strategy}")
+        log.append(dict(step=step, cache_index=ci, wave=n_wave, frozen=frozen.shape[1], current=current[0].tolist(),
+                        first_state=first_state, first_logits=first_logits))
+
+        if step > num_steps:                                               # RMM:1478-1492
+            seen = frozen[0, old_k:k].tolist() if latent else frozen[0, -headway:].tolist()
+            if any(t in stop_tokens for t in seen):
+                break
+        if step > max_diffusion_steps:
+            break
+        if accel:
+            prev_prev_states, old_old_ci = prev_states.clone(), old_ci
+        if latent:
+            prev_states = states.clone()
+        old_ci = ci
+        step += 1
+        old_k = k
+
+    if record is not None:
+        record.update(num_core_forward_passes=passes, num_tokens_forward=tokens_forward, num_cache_clears=clears,
+                      num_standing_waves=standing, diffusion_steps=step, gen_seq_length=current.shape[1], len_prefill=n_prompt,
+                      recurrence_per_position=rec_count[:, :frozen.shape[1]].clone(),
+                      token_stable_per_position=stable[:, :frozen.shape[1]].clone(), cache=cache, log=log, draws=draws[0])
+    return frozen
 
 
 # --------------------------------------------------------------------------------------

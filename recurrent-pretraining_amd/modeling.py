@@ -603,17 +603,21 @@ class RavenForCausalLM(torch.nn.Module):
     @torch.no_grad()
     def generate(self, input_ids: torch.Tensor, generation_config=None, **kwargs):
         """Dispatcher of RMM:1112-1127: `criterion` / `exit_threshold` / `exit_evaluator` select the adaptive-compute
-        loop, `draft_steps` / `lookahead_for_draft` / `verification_threshold` the self-speculative one; the
-        diffusion-style loop of the reference is not part of this package; everything else goes to generate_minimal
-        (the reference hands those calls to transformers' GenerationMixin)."""
+        loop, `draft_steps` / `lookahead_for_draft` / `verification_threshold` the self-speculative one, `headway` /
+        `state_noise_mixing` / `inner_recurrence` / `freeze_strategy` the diffusion-style one; everything else goes to
+        generate_minimal (the reference hands those calls to transformers' GenerationMixin)."""
         if any(k in kwargs for k in ("criterion", "exit_threshold", "exit_evaluator")):
             return self.generate_with_adaptive_compute(input_ids, generation_config, **kwargs)
         if any(k in kwargs for k in ("draft_steps", "lookahead_for_draft", "verification_threshold")):
             return self.generate_speculative(input_ids, generation_config, **kwargs)
-        for k in ("headway", "state_noise_mixing", "inner_recurrence", "freeze_strategy"):
-            if k in kwargs:
-                raise NotImplementedError(f"generate(..., {k}=...) selects a sampler this package does not provide")
+        if any(k in kwargs for k in ("headway", "state_noise_mixing", "inner_recurrence", "freeze_strategy")):
+            return self.generate_diffusion_style(input_ids, generation_config, **kwargs)
         return self.generate_minimal(input_ids, generation_config, **kwargs)
+
+    def generate_diffusion_style(self, input_ids: torch.Tensor, generation_config=None, **kwargs):
+        """RMM:1234-1549; see diffusion.generate_diffusion_style."""
+        from . import diffusion
+        return diffusion.generate_diffusion_style(self, input_ids, generation_config, **kwargs)
 
     def generate_with_adaptive_compute(self, input_ids: torch.Tensor, generation_config=None, **kwargs):
         """RMM:1552-1749; see adaptive.generate_with_adaptive_compute."""

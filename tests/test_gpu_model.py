@@ -156,7 +156,7 @@ def test_generate_options(pkg, tiny32):
     assert torch.equal(c1, c2) and c1.shape == (2, 11)
     assert model.generate(prompt, max_length=9, stop_tokens=set()).shape == (2, 9)
     with pytest.raises(NotImplementedError):
-        model.generate(prompt, headway=2)           # the diffusion-style sampler is not part of the package
+        model.generate(prompt, headway=2)           # the diffusion-style sampler takes one sequence, as the reference's does
     # the reference's preallocated cache class works as past_key_values too
     static = pkg.HuginnStaticCache(max_length=32, max_num_steps=4 + 4 * 4, num_heads=s.n_heads, hidden_dim=s.head_dim, batch_size=2,
                                    device="cuda", dtype=torch.float32)
@@ -376,6 +376,60 @@ def test_generate_speculative_matches_oracle(pkg, small242, B, draft_steps, L, v
                                           lookahead_for_draft=L, num_steps=4, init_scale=0.0, stop_tokens=set())
         n = min(plain.shape[1], spec.shape[1])
         assert n >= 5 + 9 and torch.equal(plain[:, :n], spec[:, :n])
+
+
+DIFFUSION_CASES = [
+    dict(freeze_strategy="fixed"),
+    dict(freeze_strategy="latent-diff", exit_t=0.5),
+    dict(freeze_strategy="latent-diff", exit_t=1e9, ema_embeds=0.0),
+    dict(freeze_strategy="latent-diff", exit_t=0.5, headway=3, max_wavefront=6),
+    dict(freeze_strategy="latent-diff", exit_t=0.5, sqrt_mixer=True, continuous_compute=True, headway=2),
+    dict(freeze_strategy="latent-diff", exit_t=0.5, dampened_state_mixer=False, state_noise_mixing=0.25),
+    dict(freeze_strategy="token-stability", state_noise_mixing=0.0),
+    dict(freeze_strategy="latent-acceleration-1", exit_t=0.5),
+    dict(freeze_strategy="latent-acceleration-2", exit_t=0.5),
+    dict(freeze_strategy="latent-diff", exit_t=0.5, full_prefill=False),
+]
+
+
+@pytest.mark.parametrize("case", range(len(DIFFUSION_CASES)))
+def test_generate_diffusion_style_matches_oracle(pkg, small242, case):
+    """The diffusion-style sampler: a wave of positions advanced by a few recurrences per step over a cache whose wave
+    entries are rolled back every step.  The same frozen tokens, steps, passes, cache clears and per-position recurrence
+    counts as the oracle's restatement of the loop, with the same injected random states and filler tokens."""
+    s, w, model = small242
+    kw = dict(num_steps=8, inner_recurrence=4)
+    kw.update(DIFFUSION_CASES[case])
+    g = torch.Generator().manual_seed(300 + case)
+    ids = torch.randint(0, s.vocab_size, (1, 5), generator=g)
+    sf = lambda c, sh: O.initialize_state(torch.empty(sh), s, 1.0, torch.Generator().manual_seed(7000 + 50 * case + c))
+    ef = lambda step, n: torch.randint(0, s.vocab_size, (1, n), generator=torch.Generator().manual_seed(9000 + step))
+    rec = {}
+    want = O.generate_diffusion_style(w, s, ids, 6, state_fn=sf, extra_token_fn=ef, record=rec, **kw)
+    out = model.generate_diffusion_style(ids.cuda(), pkg.GenerationSettings(max_new_tokens=6, return_dict_in_generate=True),
+                                         input_states_fn=sf, extra_tokens_fn=ef, stop_tokens=set(), **kw)
+    assert torch.equal(out.sequences.cpu(), want), (out.sequences.tolist(), want.tolist())
+    for key in ("num_core_forward_passes", "num_tokens_forward", "num_cache_clears", "num_standing_waves", "diffusion_steps",
+                "gen_seq_length", "len_prefill"):
+        assert out.scores[key] == rec[key], key
+    assert torch.equal(out.scores["recurrence_per_position"], rec["recurrence_per_position"])
+    assert torch.equal(out.scores["token_stable_per_position"], rec["token_stable_per_position"])
+    assert out.past_key_values.get_seq_length() == rec["cache"].get_seq_length()
+
+
+def test_generate_dispatches_to_the_diffusion_sampler(pkg, small242):
+    s, w, model = small242
+    ids = torch.randint(0, s.vocab_size, (1, 4), generator=torch.Generator().manual_seed(5)).cuda()
+    sf = lambda c, sh: O.initialize_state(torch.empty(sh), s, 1.0, torch.Generator().manual_seed(40 + c))
+    a = model.generate(ids, pkg.GenerationSettings(max_new_tokens=4), freeze_strategy="fixed", inner_recurrence=2, num_steps=4,
+                       input_states_fn=sf, stop_tokens=set())
+    b = model.generate_diffusion_style(ids, pkg.GenerationSettings(max_new_tokens=4), freeze_strategy="fixed", inner_recurrence=2,
+                                       num_steps=4, input_states_fn=sf, stop_tokens=set())
+    assert torch.equal(a, b) and a.shape == (1, 8) and torch.equal(a[:, :4], ids)
+    with pytest.raises(ValueError, match="Invalid freeze strategy"):
+        model.generate(ids, pkg.GenerationSettings(max_new_tokens=4), freeze_strategy="no-such-strategy")
+    with pytest.raises(ValueError, match="max_wavefront"):
+        model.generate_diffusion_style(ids, pkg.GenerationSettings(max_new_tokens=4), full_prefill=False, max_wavefront=2)
 
 
 @pytest.mark.parametrize("lens,use_graph,layout", [((7, 3, 12, 5, 9, 2), False, "HND"), ((6,), False, "NHD"), ((4, 4), False, "HND"),

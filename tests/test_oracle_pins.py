@@ -573,3 +573,107 @@ def test_speculative_decoding_preserves_greedy_output():
     stop = int(plain[0, 8])
     cut = O.generate_speculative(w, s, ids, 12, draft_steps=1, lookahead_for_draft=3, num_steps=4, init_scale=0.0, stop_tokens=(stop,))
     assert int(cut[0, -1]) == stop and torch.equal(cut[0], plain[0, :cut.shape[1]])
+
+
+# --------------------------------------------------------------------------------------
+# diffusion-style sampler
+# --------------------------------------------------------------------------------------
+def _diffusion_model():
+    s = O.RavenShape(n_embd=64, n_heads=2, intermediate_size=96, vocab_size=128, n_layers_in_prelude=2, n_layers_in_recurrent_block=4,
+                     n_layers_in_coda=2, mean_recurrence=4, block_size=64)
+    w = O.make_weights(s, seed=3, dtype=torch.float32)
+    ids = torch.randint(0, s.vocab_size, (1, 5), generator=torch.Generator().manual_seed(8))
+    sf = lambda c, sh: O.initialize_state(torch.empty(sh), s, 1.0, torch.Generator().manual_seed(600 + c))
+    return s, w, ids, sf
+
+
+def test_diffusion_sampler_first_wave_position_followed_by_hand():
+    """The leftmost wave position never sees the positions to its right (causal attention), and its token does not
+    change while it waits, so everything the loop does to it can be restated for that position alone, each step on a
+    private copy of the prompt's cache: embedding average with the previous step's, noise mixing damped by the
+    recurrences it has had, `inner_recurrence` recurrences, coda and head.  Its latent state and its logits after every
+    step must be the ones this hand computation gives (the token alone would not do: with random weights the argmax
+    hardly moves), and the token the loop freezes at the next position their argmax.  A wrong wave offset, a cache
+    rollback that drops too little or too much, a wrong damping count or mixing order, a recurrence too many or too
+    few, or noise states handed out in the wrong order all change the state by far more than the tolerance (checked:
+    each of these moves the top-2 logit margin in the second decimal)."""
+    import copy
+    s, w, ids, sf = _diffusion_model()
+    n, h = ids.shape[1], s.n_embd
+    num_steps, inner, a, m = 4, 2, 0.1, 0.5
+    rec = {}
+    got = O.generate_diffusion_style(w, s, ids, 3, num_steps=num_steps, inner_recurrence=inner, freeze_strategy="fixed", ema_embeds=a,
+                                     state_noise_mixing=m, state_fn=sf, record=rec)
+    # by hand
+    cache0 = O.DictCache("latest-m4-compress-s4")
+    out = O.forward(w, s, input_ids=ids, input_states=sf(0, (1, n, h)), num_steps=num_steps, past_key_values=cache0, use_cache=True,
+                    cache_position=torch.arange(n))
+    tok1 = out.logits[:, -1, :].argmax(-1, keepdim=True)
+    assert int(got[0, n]) == int(tok1)
+    state = sf(1, (1, 1, h))
+    old_e = O.embed_inputs(w, s, torch.cat([ids, tok1], dim=1))[0][:, n:]
+    pos = torch.tensor([n])
+    n_hold = num_steps // inner                       # steps 0 .. n_hold freeze nothing, step n_hold + 1 freezes one position
+    for t in range(n_hold + 2):
+        cache = copy.deepcopy(cache0)
+        e_new, block_idx = O.embed_inputs(w, s, tok1, cache=cache, cache_position=pos)
+        e = e_new * (1 - a) + old_e * a
+        old_e = e
+        noise = sf(2 + 2 * t, (1, t + 1, h))[:, :1]   # draws: prefill, first state, then (noise, new position) per step
+        mix = m / (1 + num_steps + inner * t)
+        state = state * (1 - mix) + mix * noise
+        for _ in range(inner):
+            state, block_idx = O.iterate_one_step(w, s, e, state, block_idx, cache=cache, cache_position=pos)
+        logits = O.predict_from_latents(w, s, state, cache=cache, cache_position=pos).logits[0, 0]
+        assert rec["log"][t]["cache_index"] == n and rec["log"][t]["wave"] == t + 1
+        assert torch.allclose(rec["log"][t]["first_state"], state[0, 0], rtol=1e-4, atol=1e-5), t
+        assert torch.allclose(rec["log"][t]["first_logits"], logits, rtol=1e-4, atol=1e-5), t
+    assert int(got[0, n + 1]) == int(logits.argmax())
+    assert rec["log"][n_hold + 2]["cache_index"] == n + 1      # the position is frozen: the next wave starts behind it
+    assert rec["draws"] == 2 + 2 * rec["diffusion_steps"]
+
+
+def test_diffusion_sampler_fixed_schedule_closed_form():
+    """freeze_strategy "fixed", headway 1: nothing freezes during steps 0 .. num_steps // inner, then one position per
+    step; the wave grows to num_steps // inner + 2 positions and stays there.  Counters follow in closed form."""
+    s, w, ids, sf = _diffusion_model()
+    n, num_steps, inner, max_new = ids.shape[1], 4, 2, 5
+    rec = {}
+    out = O.generate_diffusion_style(w, s, ids, max_new, num_steps=num_steps, inner_recurrence=inner, freeze_strategy="fixed",
+                                     state_fn=sf, record=rec)
+    hold = num_steps // inner                         # 2
+    steps = hold + 1 + (max_new - 1)                  # the prefill froze one token already
+    waves = [min(t + 1, hold + 2) for t in range(steps)]
+    assert out.shape == (1, n + max_new) and torch.equal(out[:, :n], ids)
+    assert rec["diffusion_steps"] == steps and rec["num_standing_waves"] == 0
+    assert rec["num_core_forward_passes"] == 1 + inner * steps
+    assert rec["num_tokens_forward"] == n + inner * sum(waves)
+    assert rec["num_cache_clears"] == sum(wv if t <= hold else wv - 1 for t, wv in enumerate(waves))
+    per_pos = [num_steps] * n + [num_steps + inner * (hold + 2)] + [inner * (hold + 2)] * (max_new - 2) + [inner * (hold + 1)]
+    assert rec["recurrence_per_position"].tolist() == [per_pos]
+    assert rec["cache"].get_seq_length() == n + max_new - 1      # every frozen position but the newest is cached
+    # the cache holds, for the frozen positions, one entry per prelude / core slot / coda block
+    assert sorted(rec["cache"].key_cache.keys()) == [-2, -1, 0, 1, 2, 3, 4, 5]
+    assert all(sorted(c.keys()) == list(range(n + max_new - 1)) for c in rec["cache"].key_cache.values())
+
+
+def test_diffusion_sampler_never_freezing_and_standing_waves():
+    """exit_t = 0 never freezes a position: the wave grows by `headway` per step up to max_wavefront and then stands;
+    the loop ends at max_diffusion_steps with the prompt and the prefill's token only, and an empty wave in the cache."""
+    s, w, ids, sf = _diffusion_model()
+    n = ids.shape[1]
+    rec = {}
+    out = O.generate_diffusion_style(w, s, ids, 4, num_steps=4, inner_recurrence=1, freeze_strategy="latent-diff", exit_t=0.0,
+                                     max_wavefront=3, max_diffusion_steps=5, state_fn=sf, record=rec)
+    assert out.shape == (1, n + 1)
+    assert rec["diffusion_steps"] == 6                          # leaves in the step after the limit, before counting it
+    assert [e["wave"] for e in rec["log"]] == [1, 2, 3, 3, 3, 3, 3]
+    assert rec["num_standing_waves"] == 5
+    assert rec["cache"].get_seq_length() == n
+    assert rec["num_cache_clears"] == 1 + 2 + 3 * 5
+    # a huge threshold freezes every position that has a previous state to compare with; the prefill's token stays
+    rec2 = {}
+    out2 = O.generate_diffusion_style(w, s, ids, 4, num_steps=4, inner_recurrence=1, freeze_strategy="latent-diff", exit_t=1e9,
+                                      state_fn=sf, record=rec2)
+    assert out2.shape == (1, n + 4) and int(out2[0, n]) == int(out[0, n])
+    assert all(e["frozen"] >= b["frozen"] for b, e in zip(rec2["log"], rec2["log"][1:]))
