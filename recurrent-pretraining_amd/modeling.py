@@ -204,6 +204,93 @@ class RavenForCausalLM(torch.nn.Module):
             mean = 1.0 if (name.endswith("weight") and p.dim() == 1) else 0.0
             p.copy_(torch.empty(p.shape, dtype=torch.float32).normal_(mean, std, generator=g).to(p.dtype))
 
+    # ---- checkpoints -----------------------------------------------------------------------------
+    @classmethod
+    def from_pretrained(cls, path: str, device: Union[str, torch.device] = "cuda", dtype: Optional[torch.dtype] = None,
+                        **config_overrides) -> "RavenForCausalLM":
+        """Builds the model from a LOCAL directory laid out like the reference's published checkpoints (what
+        `AutoModelForCausalLM.from_pretrained(..., trust_remote_code=True)` reads for raven_modeling_minimal.py:2312-2323):
+        `config.json` plus `model.safetensors`, or sharded `model-XXXXX-of-YYYYY.safetensors` with
+        `model.safetensors.index.json`, or `pytorch_model.bin` (read with weights_only=True).  Nothing is downloaded.
+        The parameter names are the reference's, so the tensors load unchanged; a tied head may be absent from the file."""
+        import json
+        import os
+        with open(os.path.join(path, "config.json")) as f:
+            cfg_dict = json.load(f)
+        cfg_dict.update(config_overrides)
+        config = RavenConfig(**cfg_dict)
+        model = cls(config, device=device, dtype=dtype)
+        index = os.path.join(path, "model.safetensors.index.json")
+        single = os.path.join(path, "model.safetensors")
+        legacy = os.path.join(path, "pytorch_model.bin")
+        if os.path.exists(index):
+            with open(index) as f:
+                shards = sorted(set(json.load(f)["weight_map"].values()))
+            files = [os.path.join(path, s) for s in shards]
+        elif os.path.exists(single):
+            files = [single]
+        elif os.path.exists(legacy):
+            files = [legacy]
+        else:
+            raise FileNotFoundError(f"no model.safetensors(.index.json) or pytorch_model.bin under {path}")
+        own = model.state_dict()
+        seen, unexpected = set(), []
+        for file in files:  # shard by shard: at most one shard is held besides the model
+            if file.endswith(".safetensors"):
+                from safetensors.torch import load_file
+                part = load_file(file, device="cpu")
+            else:
+                part = torch.load(file, map_location="cpu", weights_only=True)
+            for name, tensor in part.items():
+                if name not in own:
+                    unexpected.append(name)
+                    continue
+                if own[name].shape != tensor.shape:
+                    raise ValueError(f"{name}: checkpoint shape {tuple(tensor.shape)} != model shape {tuple(own[name].shape)}")
+                own[name].copy_(tensor)
+                seen.add(name)
+            del part
+        optional = {"freqs_cis"} | ({"lm_head.weight", "transformer.wte.weight"} if config.tie_embeddings else set())
+        missing = [n for n in own if n not in seen and n not in optional]
+        if config.tie_embeddings and not ({"lm_head.weight", "transformer.wte.weight"} & seen):
+            missing.append("transformer.wte.weight")
+        if missing or unexpected:
+            raise KeyError(f"checkpoint does not match the model: missing {missing[:8]}, unexpected {unexpected[:8]}")
+        model._native_key = None
+        return model
+
+    def save_pretrained(self, path: str, max_shard_bytes: int = 5 * 2 ** 30) -> None:
+        """Writes `config.json` and safetensors shards (with an index when there are several) that from_pretrained and
+        the reference's loader read.  The tied head is stored once, under the embedding's name."""
+        import json
+        import os
+        from safetensors.torch import save_file
+        os.makedirs(path, exist_ok=True)
+        with open(os.path.join(path, "config.json"), "w") as f:
+            json.dump({**self.config.to_dict(), "architectures": ["RavenForCausalLM"]}, f, indent=1)
+        sd = {k: v.detach().to("cpu").contiguous() for k, v in self.state_dict().items()
+              if not (self.config.tie_embeddings and k == "lm_head.weight")}
+        shards, cur, size = [], {}, 0
+        for name, t in sd.items():
+            nbytes = t.numel() * t.element_size()
+            if cur and size + nbytes > max_shard_bytes:
+                shards.append(cur)
+                cur, size = {}, 0
+            cur[name] = t
+            size += nbytes
+        shards.append(cur)
+        if len(shards) == 1:
+            save_file(shards[0], os.path.join(path, "model.safetensors"), metadata={"format": "pt"})
+            return
+        weight_map = {}
+        for i, part in enumerate(shards):
+            fname = f"model-{i + 1:05d}-of-{len(shards):05d}.safetensors"
+            save_file(part, os.path.join(path, fname), metadata={"format": "pt"})
+            weight_map.update({k: fname for k in part})
+        with open(os.path.join(path, "model.safetensors.index.json"), "w") as f:
+            json.dump({"metadata": {"total_size": sum(t.numel() * t.element_size() for t in sd.values())}, "weight_map": weight_map}, f,
+                      indent=1)
+
     def _natives(self) -> dict:
         """ctypes views of the weights; rebuilt when a parameter's storage has moved."""
         key = (self.transformer.wte.weight.data_ptr(), self.transformer.adapter.weight.data_ptr(),

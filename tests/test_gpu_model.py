@@ -524,6 +524,19 @@ def test_core_iterations_equal_single_iterations(pkg, tiny32, tiny16, dt, B):
         pkg.hip.core_iterations(nat["dims"], t.adapter.weight, nat["core"], state, emb, many, nat["freqs"], caches[0][2], [[0]], B, 1, T, ws)
 
 
+def test_from_pretrained_directory_gives_the_same_model(pkg, tiny32, tmp_path):
+    """A checkpoint directory written by save_pretrained (the layout of the reference's published checkpoints) loads
+    onto the GPU into a model with the same bits in every output."""
+    s, w, model = tiny32
+    model.save_pretrained(str(tmp_path / "ckpt"), max_shard_bytes=2_000_000)
+    again = pkg.RavenForCausalLM.from_pretrained(str(tmp_path / "ckpt"), device="cuda:0", dtype=torch.float32)
+    ids = torch.randint(0, s.vocab_size, (2, 7), generator=torch.Generator().manual_seed(12)).cuda()
+    states = O.initialize_state(torch.empty(2, 7, s.n_embd), s, 1.0, torch.Generator().manual_seed(13)).cuda()
+    a = model(input_ids=ids, input_states=states, num_steps=3)
+    b = again(input_ids=ids, input_states=states, num_steps=3)
+    assert torch.equal(a.logits, b.logits) and torch.equal(a.latent_states, b.latent_states)
+
+
 def test_committed_fixture_without_the_oracle(pkg, tiny32):
     """tests/golden/tiny_fp32_oracle.json (stored oracle outputs): logits, greedy, adaptive and speculative token streams
     from the HIP path against the stored values; the oracle only supplies the seeded weights and latent states."""

@@ -278,3 +278,55 @@ def test_vllm_flat_layer_names_and_schedule(pkg):
     assert plan == ([("layer", 0), ("layer", 1)] + [("adapter", 0)] + [("layer", i) for i in (2, 3, 4, 5)] + [("adapter", 1)]
                     + [("layer", i) for i in (2, 3, 4, 5)] + [("ln_f", 0), ("layer", 6), ("layer", 7), ("ln_f", 1)])
     assert len(vb.flat_layer_schedule(cfg)) == 2 + 32 * 5 + 1 + 2 + 1
+
+
+def test_checkpoint_directory_round_trip(pkg, tmp_path):
+    """from_pretrained / save_pretrained on a local directory in the layout of the reference's published checkpoints:
+    config.json + safetensors (one file, or shards with an index) or pytorch_model.bin; tied head stored once; the
+    parameter containers need no GPU."""
+    import json
+    import torch
+    cfg = pkg.RavenConfig.tiny()
+    model = pkg.RavenForCausalLM(cfg, device="cpu", dtype=torch.float32)
+    model.init_weights(seed=3)
+    want = {k: v.clone() for k, v in model.state_dict().items()}
+    one, many = tmp_path / "one", tmp_path / "many"
+    model.save_pretrained(str(one))
+    model.save_pretrained(str(many), max_shard_bytes=600_000)
+    assert (one / "model.safetensors").exists() and not (one / "model.safetensors.index.json").exists()
+    index = json.loads((many / "model.safetensors.index.json").read_text())
+    assert len(set(index["weight_map"].values())) > 2 and "lm_head.weight" not in index["weight_map"]
+    for d in (one, many):
+        got = pkg.RavenForCausalLM.from_pretrained(str(d), device="cpu", dtype=torch.float32)
+        assert {k: v for k, v in got.config.to_dict().items() if k != "architectures"} == cfg.to_dict()
+        sd = got.state_dict()
+        assert sd.keys() == want.keys() and all(torch.equal(sd[k], want[k]) for k in want)
+        assert got.lm_head.weight.data_ptr() == got.transformer.wte.weight.data_ptr()          # still tied
+    # a config override and a dtype change on load
+    half = pkg.RavenForCausalLM.from_pretrained(str(one), device="cpu", dtype=torch.bfloat16, mean_recurrence=7)
+    assert half.config.mean_recurrence == 7 and half.transformer.adapter.weight.dtype == torch.bfloat16
+    assert torch.equal(half.transformer.adapter.weight, want["transformer.adapter.weight"].bfloat16())
+    # the legacy single-file layout, read without unpickling code
+    legacy = tmp_path / "legacy"
+    legacy.mkdir()
+    (legacy / "config.json").write_text((one / "config.json").read_text())
+    torch.save({k: v for k, v in want.items() if k != "lm_head.weight"}, str(legacy / "pytorch_model.bin"))
+    got = pkg.RavenForCausalLM.from_pretrained(str(legacy), device="cpu", dtype=torch.float32)
+    assert all(torch.equal(got.state_dict()[k], want[k]) for k in want)
+    # mismatches are errors, not silent partial loads
+    from safetensors.torch import save_file
+    bad = tmp_path / "bad"
+    bad.mkdir()
+    (bad / "config.json").write_text((one / "config.json").read_text())
+    save_file({"transformer.ln_f.weight": want["transformer.ln_f.weight"], "transformer.nonsense": torch.zeros(1)}, str(bad / "model.safetensors"))
+    with pytest.raises(KeyError, match="missing"):
+        pkg.RavenForCausalLM.from_pretrained(str(bad), device="cpu")
+    wrong = dict(cfg.to_dict(), n_embd=128, n_heads=2)
+    (bad / "config.json").write_text(json.dumps(wrong))
+    save_file({k: v for k, v in want.items() if k != "lm_head.weight"}, str(bad / "model.safetensors"))
+    with pytest.raises(ValueError, match="shape"):
+        pkg.RavenForCausalLM.from_pretrained(str(bad), device="cpu")
+    with pytest.raises(FileNotFoundError):
+        (tmp_path / "empty").mkdir()
+        (tmp_path / "empty" / "config.json").write_text((one / "config.json").read_text())
+        pkg.RavenForCausalLM.from_pretrained(str(tmp_path / "empty"), device="cpu")
