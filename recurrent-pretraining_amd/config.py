@@ -31,8 +31,14 @@ class RavenConfig:
         qk_bias: bool = True,
         rope_base: float = 50_000,
         torch_dtype: str = "bfloat16",
+        test_time_noise: float = 0,
+        test_time_noise_type: str = "fixed",
         **kwargs,
     ):
+        if test_time_noise:
+            # RMM:815-838 perturbs the latent state before every recurrence when this is set; the recurrence launches of
+            # this package have no such step
+            raise NotImplementedError("test_time_noise > 0 (noise injected before every recurrence) is not supported")
         if bias:
             raise ValueError("bias=True is not supported: the reference model family has no Linear biases")
         self.n_embd = n_embd
@@ -54,7 +60,7 @@ class RavenConfig:
         self.rope_base = rope_base
         self.torch_dtype = torch_dtype
         self.test_time_noise = 0
-        self.test_time_noise_type = "fixed"
+        self.test_time_noise_type = test_time_noise_type
         self.extra = dict(kwargs)  # keys of the reference config that only matter for training
         # derived (raven_config_minimal.py:78-91)
         if n_embd % n_heads:

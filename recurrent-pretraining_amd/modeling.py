@@ -53,6 +53,9 @@ class GenerationSettings:
     top_p: Optional[float] = None
     min_p: Optional[float] = None
     repetition_penalty: Optional[float] = None
+    dry_multiplier: float = 0.0        # > 0 selects the n-gram penalty instead (RMM:2003-2046)
+    dry_base: float = 1.75
+    dry_allowed_length: int = 2
     eos_token_id: Any = None
     return_dict_in_generate: bool = False
 
@@ -667,6 +670,8 @@ class RavenForCausalLM(torch.nn.Module):
     def _sample_next_token(self, next_token_logits: torch.Tensor, input_ids, generation_config) -> torch.Tensor:
         """RMM:1944-1989.  Greedy selection runs in the HIP argmax kernel."""
         gc = generation_config
+        if getattr(gc, "repetition_penalty", None) is not None and gc.repetition_penalty != 1.0:
+            next_token_logits = self._apply_repetition_penalty(next_token_logits, input_ids, gc)
         if not getattr(gc, "do_sample", False):
             return hip.argmax(next_token_logits.float().contiguous()).unsqueeze(-1)
         logits = next_token_logits.to(torch.float32)
@@ -686,6 +691,19 @@ class RavenForCausalLM(torch.nn.Module):
             probs = torch.where(probs < gc.min_p * probs.max(dim=-1, keepdim=True).values, torch.zeros_like(probs), probs)
         probs = probs / probs.sum(dim=-1, keepdim=True).clamp(min=1e-10)
         return torch.multinomial(probs, num_samples=1)
+
+    def _apply_repetition_penalty(self, original_logits, input_ids, generation_config, use_candidates: bool = False):
+        """RMM:1991-2070; see sampling.apply_repetition_penalty."""
+        from .sampling import apply_repetition_penalty
+        return apply_repetition_penalty(original_logits, input_ids, generation_config, use_candidates)
+
+    def get_stats(self, logits, x, latent_states, xk, input_embeds, num_steps_no_grad, num_steps_with_grad) -> dict:
+        """RMM:1037-1049: entropy of the predictive distribution and the distance between two latent states."""
+        probs = torch.softmax(logits.float(), dim=-1)
+        residual_diff = (x - latent_states).norm(dim=-1)
+        return {"entropy": torch.where(probs > 0, -probs * probs.log(), 0).sum(dim=-1), "residual_diff": residual_diff,
+                "rel_residual": residual_diff / latent_states.norm(dim=-1), "num_steps_no_grad": num_steps_no_grad,
+                "num_steps_with_grad": num_steps_with_grad}
 
     @torch.no_grad()
     def generate(self, input_ids: torch.Tensor, generation_config=None, **kwargs):

@@ -150,6 +150,16 @@ def test_generate_options(pkg, tiny32):
     a = model.generate(prompt, g1, max_new_tokens=5, init_scale=0.0, stop_tokens=set())
     b = model.generate(prompt, max_new_tokens=5, init_scale=0.0, stop_tokens=set())
     assert torch.equal(a, b)
+    # repetition penalties change which token wins; a huge penalty keeps every generated token new
+    rp = pkg.GenerationSettings(repetition_penalty=1e6)
+    r1 = model.generate(prompt, rp, max_new_tokens=6, init_scale=0.0, stop_tokens=set())
+    for row in r1.tolist():
+        assert len(set(row[6:])) == 6 and not (set(row[6:]) & set(row[:6]))
+    dry = pkg.GenerationSettings(repetition_penalty=1.0001, dry_multiplier=50.0)
+    assert model.generate(prompt, dry, max_new_tokens=4, init_scale=0.0, stop_tokens=set()).shape == (2, 10)
+    lg = model(input_ids=prompt, input_states=torch.zeros(2, 6, s.n_embd, device="cuda"), num_steps=2)
+    st = model.get_stats(lg.logits, lg.latent_states, lg.latent_states * 2, None, None, 2, 0)
+    assert st["entropy"].shape == (2, 6) and torch.allclose(st["rel_residual"], torch.full((2, 6), 0.5, device="cuda"))
     # continuous compute carries the last latent state over (deterministic with a zero initial state)
     c1 = model.generate(prompt, max_new_tokens=5, init_scale=0.0, continuous_compute=True, stop_tokens=set())
     c2 = model.generate(prompt, max_new_tokens=5, init_scale=0.0, continuous_compute=True, stop_tokens=set())

@@ -330,3 +330,57 @@ def test_checkpoint_directory_round_trip(pkg, tmp_path):
         (tmp_path / "empty").mkdir()
         (tmp_path / "empty" / "config.json").write_text((one / "config.json").read_text())
         pkg.RavenForCausalLM.from_pretrained(str(tmp_path / "empty"), device="cpu")
+
+
+def test_repetition_penalties_against_the_reference_loops(pkg):
+    """The standard repetition penalty and the n-gram penalty against a literal restatement of the reference's loops
+    (RMM:2003-2060, per vocabulary entry and start position) on a small vocabulary."""
+    import types
+    import torch
+    from recurrent_pretraining_amd.sampling import apply_repetition_penalty
+    g = torch.Generator().manual_seed(5)
+    V = 14
+    ids = torch.tensor([[3, 4, 5, 3, 4, 5, 3, 4, 9, 3, 4], [1, 1, 1, 1, 2, 2, 7, 7, 1, 1, 1]])
+    logits = torch.randn(2, V, generator=g) * 3
+
+    def brute_dry(row_logits, context, mult, base, allowed):
+        out = row_logits.clone()
+        n = len(context)
+        for vocab_idx in range(V):
+            max_match = 0
+            for start in range(max(0, n - 128), n - 1):
+                match = 0
+                while start + match < n and match < 32 and context[start + match] == context[n - match - 1]:
+                    match += 1
+                if match > 0 and start + match < n and context[start + match] == vocab_idx:
+                    max_match = max(max_match, match + 1)
+            if max_match >= allowed:
+                out[vocab_idx] -= mult * base ** (max_match - allowed)
+        return out
+
+    dry = types.SimpleNamespace(repetition_penalty=1.0, dry_multiplier=0.8, dry_base=1.75, dry_allowed_length=2)
+    got = apply_repetition_penalty(logits, ids, dry)
+    for b in range(2):
+        assert torch.allclose(got[b], brute_dry(logits[b], ids[b].tolist(), 0.8, 1.75, 2)), b
+    assert not torch.equal(got, logits)   # the sequences do repeat
+    # several positions of one sequence ([T, V] logits, batch of one): every position gets the row's penalty
+    multi = torch.randn(3, V, generator=g)
+    got = apply_repetition_penalty(multi, ids[:1], dry)
+    for t in range(3):
+        assert torch.allclose(got[t], brute_dry(multi[t], ids[0].tolist(), 0.8, 1.75, 2))
+    # standard penalty: seen tokens' positive logits are divided, negative ones multiplied
+    std = types.SimpleNamespace(repetition_penalty=1.3, dry_multiplier=0.0)
+    got = apply_repetition_penalty(logits, ids, std)
+    for b in range(2):
+        seen = set(ids[b].tolist())
+        for v in range(V):
+            x = float(logits[b, v])
+            want = (x * 1.3 if x < 0 else x / 1.3) if v in seen else x
+            assert abs(float(got[b, v]) - want) < 1e-6
+    # with the positions' own argmax tokens added to the context
+    got = apply_repetition_penalty(logits.view(2, 1, V), ids, std, use_candidates=True)
+    b0 = int(logits[0].argmax())
+    x = float(logits[0, b0])
+    assert abs(float(got[0, 0, b0]) - (x * 1.3 if x < 0 else x / 1.3)) < 1e-6
+    with pytest.raises(NotImplementedError):
+        pkg.RavenConfig(test_time_noise=0.1)
