@@ -209,7 +209,6 @@ def generate_with_adaptive_compute(model, input_ids: torch.Tensor, generation_co
     (the reference draws it from the device RNG); stop_tokens overrides the reference's fixed stop set; with
     return_dict_in_generate the output's `scores` carries "compute_steps" and "exit_values" per token and sequence
     (the reference builds both and then drops them)."""
-    from .cache import HuginnDynamicCache
     from .modeling import GenerateOutput
 
     gc = generation_config if generation_config is not None else model.generation_config
@@ -227,7 +226,7 @@ def generate_with_adaptive_compute(model, input_ids: torch.Tensor, generation_co
     dev = model.device
     input_ids = input_ids.to(dev)
     total = min(prompt_len + max_new, model.config.block_size)
-    cache = model_kwargs.get("past_key_values") or HuginnDynamicCache(cache_lookup_strategy, max_length=total)
+    cache = model._generation_cache(model_kwargs, cache_lookup_strategy, input_ids.shape[0], total)
     h = model.config.n_embd
 
     def draw(token_step: int, shape, embeds):

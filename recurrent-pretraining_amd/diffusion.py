@@ -36,7 +36,6 @@ def generate_diffusion_style(model, input_ids: torch.Tensor, generation_config=N
     hard-coded 65510, here `extra_token_high`); stop_tokens overrides the reference's stop set.  With
     return_dict_in_generate the output's `scores` holds the reference's summary (passes, tokens forwarded, cache
     clears, standing waves, steps, recurrences and stable steps per position)."""
-    from .cache import HuginnDynamicCache
     from .modeling import GenerateOutput
 
     if input_ids.shape[0] != 1:
@@ -57,7 +56,7 @@ def generate_diffusion_style(model, input_ids: torch.Tensor, generation_config=N
     else:
         max_new = model_kwargs.get("max_length", gc.max_length) - n_prompt
     stops = model._get_stops(gc) if stop_tokens is None else set(stop_tokens)
-    cache = model_kwargs.get("past_key_values") or HuginnDynamicCache(cache_lookup_strategy)
+    cache = model._generation_cache(model_kwargs, cache_lookup_strategy, 1)
     draws = [0]
 
     def draw(shape, via_bf16: bool = False):

@@ -23,7 +23,7 @@ from typing import Any, Callable, Optional, Union
 import torch
 
 from . import hip
-from .cache import HuginnDynamicCache, remap_step
+from .cache import HuginnDynamicCache, HuginnStaticCache, remap_step
 from .config import RavenConfig
 
 
@@ -692,6 +692,21 @@ class RavenForCausalLM(torch.nn.Module):
         probs = probs / probs.sum(dim=-1, keepdim=True).clamp(min=1e-10)
         return torch.multinomial(probs, num_samples=1)
 
+    def _generation_cache(self, model_kwargs: dict, cache_lookup_strategy: str, batch: int, max_length: Optional[int] = None):
+        """The cache a generate loop works on (RMM:1146-1160): the caller's `past_key_values`, or a new one --
+        HuginnStaticCache when `cache_implementation="static"` is asked for, else HuginnDynamicCache."""
+        given = model_kwargs.get("past_key_values")
+        if given is not None:
+            return given
+        if model_kwargs.get("cache_implementation", "dynamic") == "static":
+            cfg = self.config
+            length = max_length if max_length is not None else model_kwargs.get("max_length", self.generation_config.max_length)
+            steps = 4 + model_kwargs.get("num_steps", cfg.mean_recurrence) * 4
+            return HuginnStaticCache(max_length=min(length, cfg.block_size), max_num_steps=steps, num_heads=cfg.num_key_value_heads,
+                                     hidden_dim=cfg.head_dim, batch_size=batch, device=self.device, dtype=self.dtype,
+                                     lookup_strategy=cache_lookup_strategy)
+        return HuginnDynamicCache(cache_lookup_strategy, max_length=max_length)
+
     def _apply_repetition_penalty(self, original_logits, input_ids, generation_config, use_candidates: bool = False):
         """RMM:1991-2070; see sampling.apply_repetition_penalty."""
         from .sampling import apply_repetition_penalty
@@ -772,7 +787,7 @@ class RavenForCausalLM(torch.nn.Module):
         if max_new <= 0:
             return input_ids
         total = min(prompt_len + max_new, self.config.block_size)
-        cache = model_kwargs.get("past_key_values") or HuginnDynamicCache(cache_lookup_strategy, max_length=total)
+        cache = self._generation_cache(model_kwargs, cache_lookup_strategy, B, total)
 
         def state_for(call: int, S: int, embeds_like=None):
             if input_states_fn is not None:

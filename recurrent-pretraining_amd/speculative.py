@@ -26,7 +26,6 @@ def generate_speculative(model, input_ids: torch.Tensor, generation_config=None,
     compute); stop_tokens overrides the reference's fixed stop set; pad_id (the reference hard-codes 65509) fills the
     rows of sequences that accepted fewer tokens than others; with return_dict_in_generate the output's
     `scores` carries "accepted_tokens" per round and sequence."""
-    from .cache import HuginnDynamicCache
     from .modeling import GenerateOutput
 
     assert lookahead_for_draft > 0
@@ -44,7 +43,7 @@ def generate_speculative(model, input_ids: torch.Tensor, generation_config=None,
     stops = model._get_stops(gc) if stop_tokens is None else set(stop_tokens)
     dev, h = model.device, model.config.n_embd
     input_ids = input_ids.to(dev)
-    cache = model_kwargs.get("past_key_values") or HuginnDynamicCache(cache_lookup_strategy)
+    cache = model._generation_cache(model_kwargs, cache_lookup_strategy, B)
     calls = [0]
 
     def run(tokens, pos, steps, carried):

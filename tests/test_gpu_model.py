@@ -172,6 +172,10 @@ def test_generate_options(pkg, tiny32):
                                    device="cuda", dtype=torch.float32)
     d = model.generate(prompt, max_new_tokens=5, init_scale=0.0, stop_tokens=set(), past_key_values=static)
     assert torch.equal(d, b)
+    # ... and is what cache_implementation="static" builds (RMM:1150-1160)
+    e = model.generate(prompt, pkg.GenerationSettings(return_dict_in_generate=True), max_new_tokens=5, init_scale=0.0, stop_tokens=set(),
+                       cache_implementation="static", max_length=32)
+    assert torch.equal(e.sequences, b) and isinstance(e.past_key_values, pkg.HuginnStaticCache)
 
 
 def test_forward_tiny_bf16_matches_oracle(tiny16):
