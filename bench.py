@@ -46,6 +46,8 @@ def parse():
                     help="measure the recurrent core over a whole prompt instead (bs=4 x 4096 tokens, r iterations): MFMA-bound regime")
     ap.add_argument("--prefill-batch", type=int, default=4)
     ap.add_argument("--prefill-len", type=int, default=4096)
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                    help="launch-shape override passed to raven_set_tuning before the run (experiments only)")
     ap.add_argument("--kernel-only", type=int, default=0, metavar="N",
                     help="run only N launches of the dominant kernel plus one 256 MiB device copy (for rocprofv3 --pmc runs)")
     return ap.parse_args()
@@ -289,8 +291,19 @@ def decode_tokens_per_s(pkg, model, batch, prompt_len, steps, warmup, r, use_gra
     return batch * steps / dt, dt / steps * 1e3, prefill_s, cache
 
 
+def apply_tuning(args):
+    if not args.tune:
+        return
+    import __graft_entry__ as entry
+    hip = entry.import_package().hip
+    for item in args.tune:
+        key, value = item.split("=")
+        hip.set_tuning(key, int(value))
+
+
 def main():
     args = parse()
+    apply_tuning(args)
     if args.kernel_only:
         kernel_only(args.kernel_only)
         return

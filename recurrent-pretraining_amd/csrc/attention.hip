@@ -105,40 +105,20 @@ constexpr int kAttnMaxHd = 128;
 extern "C" size_t raven_decode_attention_workspace_bytes(int32_t M, int32_t n_heads, int32_t head_dim);
 namespace raven {
 
-// bias + RoPE of one 16-byte chunk of a q or k head row (sec 0 = q, 1 = k); d = first column of the chunk.
-// The operands (bias chunk, cos/sin pairs) are loaded by rope_operands so that a caller can issue those loads
-// ahead of others it will wait for anyway.
-template <typename T>
-struct RopeOperands {
-    Chunk<T> bias;
-    float cs[Chunk<T>::N];  // (cos, sin) of the chunk's N / 2 pairs
-};
-template <typename T>
-__device__ __forceinline__ RopeOperands<T> rope_operands(const T* __restrict__ qk_bias, int sec, int h, int col,
-                                                         const float* __restrict__ freqs, int pos, int hd, int d) {
-    constexpr int E = Chunk<T>::N;
-    RopeOperands<T> r;
-    r.bias = qk_bias ? load_chunk(qk_bias + sec * h + col) : zero_chunk<T>();
-    const float* f = freqs + ((int64_t)pos * (hd / 2) + d / 2) * 2;
-#pragma unroll
-    for (int e = 0; e < E; e += 4) *reinterpret_cast<float4*>(&r.cs[e]) = *reinterpret_cast<const float4*>(f + e);
-    return r;
-}
-template <typename T>
-__device__ __forceinline__ Chunk<T> bias_rope_apply(Chunk<T> x, const RopeOperands<T>& op, bool has_bias) {
-    constexpr int E = Chunk<T>::N;
-    if (has_bias) {
-#pragma unroll
-        for (int e = 0; e < E; ++e) x.v[e] = from_f32<T>(to_f32(x.v[e]) + to_f32(op.bias.v[e]));
-    }
-#pragma unroll
-    for (int e = 0; e < E; e += 2) rope_pair<T>(x.v[e], x.v[e + 1], op.cs[e], op.cs[e + 1]);
-    return x;
-}
+// bias + RoPE of one 16-byte chunk of a q or k head row (sec 0 = q, 1 = k); d = first column of the chunk
 template <typename T>
 __device__ __forceinline__ Chunk<T> bias_rope_chunk(Chunk<T> x, const T* __restrict__ qk_bias, int sec, int h, int col,
                                                     const float* __restrict__ freqs, int pos, int hd, int d) {
-    return bias_rope_apply<T>(x, rope_operands<T>(qk_bias, sec, h, col, freqs, pos, hd, d), qk_bias != nullptr);
+    constexpr int E = Chunk<T>::N;
+    if (qk_bias) {
+        const Chunk<T> bch = load_chunk(qk_bias + sec * h + col);
+#pragma unroll
+        for (int e = 0; e < E; ++e) x.v[e] = from_f32<T>(to_f32(x.v[e]) + to_f32(bch.v[e]));
+    }
+    const float* f = freqs + ((int64_t)pos * (hd / 2) + d / 2) * 2;
+#pragma unroll
+    for (int e = 0; e < E; e += 2) rope_pair<T>(x.v[e], x.v[e + 1], f[e], f[e + 1]);
+    return x;
 }
 
 // What one lane holds of a position's head row: CPL neighbouring 16-byte chunks (1, or 2 for fp32 heads wider than
@@ -174,6 +154,27 @@ __device__ __forceinline__ float dot_piece(const Piece<T, CPL>& a, const Piece<T
     return acc;
 }
 
+// Online-softmax state (running maximum, sum, unnormalised output) of a wave's four 16-lane rows merged into one, in
+// registers; afterwards every row of the wave holds the merged state.
+template <int E>
+__device__ __forceinline__ void merge_wave_rows(float& m_run, float& l_run, float (&o)[E]) {
+    float m4 = fmaxf(m_run, __shfl_xor(m_run, 16, 64));
+    m4 = fmaxf(m4, __shfl_xor(m4, 32, 64));
+    const float w = (m_run == -INFINITY) ? 0.f : exp2f(m_run - m4);
+    float l4 = l_run * w;
+    l4 += __shfl_xor(l4, 16, 64);
+    l4 += __shfl_xor(l4, 32, 64);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        float v = o[e] * w;
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        o[e] = v;
+    }
+    m_run = m4;
+    l_run = l4;
+}
+
 // Grid (heads, token rows, splits).  With one split a workgroup owns a whole (head, row) and writes y.
 // With several (few heads x rows, i.e. small batches: one CU cannot pull a head's K/V fast enough) each
 // workgroup covers a contiguous range of positions with all of its loads in flight at once and writes
@@ -182,18 +183,20 @@ __device__ __forceinline__ float dot_piece(const Piece<T, CPL>& a, const Piece<T
 // position's k and v, come straight from the fused qkv GEMM output -- bias and RoPE are applied here,
 // the new k/v row is written to the cache by the workgroup whose range holds it and used from registers.
 // LOOKUP: some older positions are not cached at this slot (cv.steps_present says which).
-template <typename T, bool FUSED, int kAttnU, bool LOOKUP = false, int CPL = 1>
-__global__ __launch_bounds__(256) void decode_attention_kernel(
+// G = 16-lane rows per workgroup (16 x G threads): 16, or 64 for the variant that gives a whole (head, row) to one
+// workgroup of 1024 threads whose every load is in flight at once -- what the split launch achieves with several
+// workgroups and a second launch, without that launch.
+template <typename T, bool FUSED, int kAttnU, bool LOOKUP = false, int CPL = 1, int G = 16>
+__global__ __launch_bounds__(16 * G) void decode_attention_kernel(
     const T* __restrict__ q_or_qkv, const T* __restrict__ qk_bias, const float* __restrict__ freqs, T* __restrict__ y,
     CacheView cv, int S, int pos0, const int* __restrict__ pos_dev, float scale_log2, int n_splits,
     float* __restrict__ ws_ml, float* __restrict__ ws_o) {
     constexpr int EC = Chunk<T>::N;   // elements per 16-byte chunk
     constexpr int E = EC * CPL;       // elements per lane and position
-    constexpr int G = 16;      // 16-lane rows in the workgroup
     // kAttnU = positions per 16-lane row and loop iteration: 4 when a few workgroups must each keep many loads
     // in flight, 2 when the grid is large and register pressure decides how many workgroups a CU holds
-    __shared__ float sm_m[G], sm_l[G];
-    __shared__ float sm_o[G][kAttnMaxHd];
+    __shared__ float sm_m[G / 4], sm_l[G / 4];  // one entry per wave
+    __shared__ float sm_o[G / 4][kAttnMaxHd];
 
     const int head = blockIdx.x, m = blockIdx.y, split = blockIdx.z;
     const int hd = cv.hd, h = cv.nh * hd;
@@ -248,22 +251,14 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
             }
         }
     };
-    RopeOperands<T> opq[CPL], opk[CPL];
-    if (FUSED && active) {
-#pragma unroll
-        for (int i = 0; i < CPL; ++i) {
-            opq[i] = rope_operands<T>(qk_bias, 0, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
-            opk[i] = rope_operands<T>(qk_bias, 1, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
-        }
-    }
     load_tile(start);
 
     P qc = qraw, knew = kraw;
     if (FUSED && active) {
 #pragma unroll
         for (int i = 0; i < CPL; ++i) {
-            qc.c[i] = bias_rope_apply<T>(qraw.c[i], opq[i], qk_bias != nullptr);
-            knew.c[i] = bias_rope_apply<T>(kraw.c[i], opk[i], qk_bias != nullptr);
+            qc.c[i] = bias_rope_chunk<T>(qraw.c[i], qk_bias, 0, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
+            knew.c[i] = bias_rope_chunk<T>(kraw.c[i], qk_bias, 1, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
         }
         if (group == 0 && pos >= start && pos < end) {
             store_piece<T, CPL>(static_cast<T*>(cv.k) + head_off + (int64_t)pos * hd + ci * E, knew);
@@ -308,23 +303,26 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(
         m_run = m_new;
     }
 
-    // merge the G rows of the workgroup
-    if (ci == 0) {
-        sm_m[group] = m_run;
-        sm_l[group] = l_run;
-    }
-    if (active) {
+    // merge: first the wave's four 16-lane rows in registers, then the waves through LDS
+    merge_wave_rows<E>(m_run, l_run, o);
+    if (r == 0) {
+        if (ci == 0) {
+            sm_m[wave] = m_run;
+            sm_l[wave] = l_run;
+        }
+        if (active) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) sm_o[group][ci * E + e] = o[e];
+            for (int e = 0; e < E; ++e) sm_o[wave][ci * E + e] = o[e];
+        }
     }
     __syncthreads();
     const int t = threadIdx.x;
     if (t < hd) {
         float M = -INFINITY, L = 0.f, O = 0.f;
 #pragma unroll
-        for (int g = 0; g < G; ++g) M = fmaxf(M, sm_m[g]);
+        for (int g = 0; g < G / 4; ++g) M = fmaxf(M, sm_m[g]);
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
+        for (int g = 0; g < G / 4; ++g) {
             const float wgt = (sm_m[g] == -INFINITY) ? 0.f : exp2f(sm_m[g] - M);
             L += sm_l[g] * wgt;
             O += sm_o[g][t] * wgt;
@@ -388,8 +386,8 @@ __global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __
                                                                      float scale_log2, int n_splits, float* __restrict__ ws_ml,
                                                                      float* __restrict__ ws_o) {
     constexpr int EC = Chunk<T>::N, E = EC * CPL, G = 16, U = 2;
-    __shared__ float sm_m[G], sm_l[G];
-    __shared__ float sm_o[G][kAttnMaxHd];
+    __shared__ float sm_m[G / 4], sm_l[G / 4];
+    __shared__ float sm_o[G / 4][kAttnMaxHd];
     typedef Piece<T, CPL> P;
     const int head = blockIdx.x, b = blockIdx.y, split = blockIdx.z;
     const int hd = pv.hd, h = pv.nh * hd;
@@ -487,22 +485,25 @@ __global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __
         }
         m_run = m_new;
     }
-    if (ci == 0) {
-        sm_m[group] = m_run;
-        sm_l[group] = l_run;
-    }
-    if (active) {
+    merge_wave_rows<E>(m_run, l_run, o);
+    if (r == 0) {
+        if (ci == 0) {
+            sm_m[wave] = m_run;
+            sm_l[wave] = l_run;
+        }
+        if (active) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) sm_o[group][ci * E + e] = o[e];
+            for (int e = 0; e < E; ++e) sm_o[wave][ci * E + e] = o[e];
+        }
     }
     __syncthreads();
     const int t = threadIdx.x;
     if (t < hd) {
         float M = -INFINITY, L = 0.f, O = 0.f;
 #pragma unroll
-        for (int g = 0; g < G; ++g) M = fmaxf(M, sm_m[g]);
+        for (int g = 0; g < G / 4; ++g) M = fmaxf(M, sm_m[g]);
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
+        for (int g = 0; g < G / 4; ++g) {
             const float wgt = (sm_m[g] == -INFINITY) ? 0.f : exp2f(sm_m[g] - M);
             L += sm_l[g] * wgt;
             O += sm_o[g][t] * wgt;
@@ -540,6 +541,11 @@ __global__ __launch_bounds__(256) void paged_kv_append_kernel(const T* __restric
 constexpr int kAttnMaxSplits = 32;
 int g_attn_split_target = 2048;  // workgroups a split launch aims for (raven_set_tuning "attn_split_target")
 int g_attn_big_grid = 1280;      // workgroups from which the 2-positions-per-row variant is used ("attn_big_grid")
+// Few (head, row) pairs and a short cache: one 1024-thread workgroup per pair instead of a split launch and its merge
+// launch.  Alone the step is faster (bs=1, 513 positions: 11.5 us against 13.8; bs=4: 13.9 against 19.1; it loses beyond
+// about 2000 positions and from 8 sequences on), inside a decoded token the gain does not show (bs=1: 18.9-19.1 ms per
+// token either way; bs=4: -0.4 %), so it is off unless asked for.  "attn_wide" = longest cache it is used for, 0 = never.
+int g_attn_wide = 0;
 
 // Splits are worth their extra launch only while heads x rows cannot fill the chip.
 static int splits_for(int M, int nh, int len_hint) {
@@ -615,8 +621,15 @@ extern "C" int raven_qkv_bias_rope_cache_append(const void* qkv, const void* qk_
 template <typename T>
 static void launch_attention(bool fused, const void* q, const void* bias, const float* freqs, void* y, const raven::CacheView& cv,
                              int S, int M, int pos0, const int32_t* pos_dev, float scale_log2, int ns, float* ws_ml, float* ws_o,
-                             hipStream_t s) {
+                             bool wide, hipStream_t s) {
     using namespace raven;
+    if (wide) {  // one 1024-thread workgroup per (head, row), 384 positions per round trip, no second launch
+        constexpr int WIDE_G = 64, WIDE_U = 6;  // 6 positions per 16-lane row: what 128 registers per lane hold without spilling
+        const dim3 g1(cv.nh, M, 1);
+        decode_attention_kernel<T, true, WIDE_U, false, 1, WIDE_G><<<g1, dim3(16 * WIDE_G), 0, s>>>((const T*)q, (const T*)bias, freqs, (T*)y, cv, S, pos0,
+                                                                                   pos_dev, scale_log2, 1, nullptr, nullptr);
+        return;
+    }
     const dim3 grid(cv.nh, M, ns);
     const bool big = (int64_t)cv.nh * M * ns >= g_attn_big_grid;
     const T* bias_t = (const T*)bias;
@@ -656,6 +669,9 @@ static int attention_common(const char* who, bool fused, const void* q, const vo
     const int M = B * S;
     RAVEN_REQUIRE(M <= 65535, "%s: too many token rows (%d)", who, M);
     int ns = splits_for(M, n_heads, pos0 + S);
+    const int elts = 16 / (int)raven_host::elt_size(dtype);
+    const bool wide = fused && ns > 1 && pos0 + S <= g_attn_wide && M * n_heads <= 256 && !cv.steps_present && head_dim / elts <= 16;
+    if (wide) ns = 1;
     float *ws_ml = nullptr, *ws_o = nullptr;
     if (ns > 1) {
         const size_t need = raven_decode_attention_workspace_bytes(M, n_heads, head_dim);
@@ -669,8 +685,8 @@ static int attention_common(const char* who, bool fused, const void* q, const vo
     }
     const float scale_log2 = (float)(1.0 / sqrt((double)head_dim) * 1.4426950408889634);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == RAVEN_BF16) launch_attention<bf16>(fused, q, bias, freqs, y, cv, S, M, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o, s);
-    else launch_attention<float>(fused, q, bias, freqs, y, cv, S, M, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o, s);
+    if (dtype == RAVEN_BF16) launch_attention<bf16>(fused, q, bias, freqs, y, cv, S, M, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o, wide, s);
+    else launch_attention<float>(fused, q, bias, freqs, y, cv, S, M, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o, wide, s);
     return raven_host::check_launch(who);
 }
 

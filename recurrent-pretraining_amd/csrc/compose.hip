@@ -59,7 +59,7 @@ static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
     s.attn_ws_bytes = raven_decode_attention_workspace_bytes(M, d->n_heads, d->head_dim);
     s.attn_ws = s.attn_ws_bytes ? take(s.attn_ws_bytes) : nullptr;
     const int widest = 3 * d->n_embd > 2 * d->intermediate ? 3 * d->n_embd : 2 * d->intermediate;
-    s.lin_ws_bytes = M > 4 ? raven_linear_workspace_bytes(M, widest) : 0;
+    s.lin_ws_bytes = M > 1 ? raven_linear_workspace_bytes(M, widest) : 0;
     s.lin_ws = s.lin_ws_bytes ? take(s.lin_ws_bytes) : nullptr;
     if (out) *out = s;
     return off;
@@ -241,8 +241,8 @@ static int iterations_impl(const char* who, const raven_dims* dims, const void* 
         }
         return close_one_row(dims, s, last_blk.norm_4, ln_f, state_out, stream);
     }
-    // 5..32 rows in bf16: the adapter is split by columns as for one row (embedding half summed once, in fp32)
-    const bool split = adapter_w && n_iterations >= 2 && dims->dtype == RAVEN_BF16 && M >= 5 && M <= 32 && h % 32 == 0 && h >= 256 &&
+    // 2..32 rows in bf16: the adapter is split by columns as for one row (embedding half summed once, in fp32)
+    const bool split = adapter_w && n_iterations >= 2 && dims->dtype == RAVEN_BF16 && M >= 2 && M <= 32 && h % 32 == 0 && h >= 256 &&
                        s.lin_ws;
     if (split)
         if ((rc = linear_column_block(embeds, static_cast<const char*>(adapter_w) + (size_t)h * 2, 2 * h, nullptr, s.e_sums, 1, M, h, h,

@@ -25,7 +25,7 @@ namespace raven {
 
 int set_gemv1_tuning(const char* key, int value);
 extern int g_linear_ks;
-extern int g_attn_split_target, g_attn_big_grid;
+extern int g_attn_split_target, g_attn_big_grid, g_attn_wide, g_linear_min_rows;
 
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
 
@@ -50,6 +50,7 @@ struct Tuning {
     int gemv_nontemporal = 1;
     int gemv_wgs_per_cu = 4;
     int gemm_four_tiles = 1;
+    int gemm_mfma_min_rows = 2;  // fewer rows go to the vector kernels (one row: the K-split GEMV)
 };
 static Tuning g_tuning;
 
@@ -511,7 +512,7 @@ static int run_gemm(GemmArgs a, int dtype, hipStream_t s) {
             return raven_gemv_fused(x0, x1, nullptr, nullptr, nullptr, a.w, res, y, a.N, a.k0, a.k1, 0.f, EPI == EPI_SWIGLU, a.out_f32,
                                     dtype, s);
         }
-        const bool use_mfma = mfma_ok && left > 4;
+        const bool use_mfma = mfma_ok && left >= g_tuning.gemm_mfma_min_rows;
         if (use_mfma) pass = left < 32 ? left : 32;
         else {
             pass = dtype == RAVEN_BF16 ? (left < 4 ? left : 4) : (left < 8 ? left : 8);
@@ -556,8 +557,11 @@ extern "C" int raven_set_tuning(const char* key, int32_t value) {
     else if (k == "gemv_wgs_per_cu") g_tuning.gemv_wgs_per_cu = value;
     else if (k == "linear_ks") g_linear_ks = value;
     else if (k == "gemm_four_tiles") g_tuning.gemm_four_tiles = value;
+    else if (k == "gemm_mfma_min_rows" && value >= 2) g_tuning.gemm_mfma_min_rows = value;
     else if (k == "attn_split_target" && value > 0) g_attn_split_target = value;
     else if (k == "attn_big_grid" && value > 0) g_attn_big_grid = value;
+    else if (k == "attn_wide") g_attn_wide = value;
+    else if (k == "linear_min_rows" && value >= 1) g_linear_min_rows = value;
     else RAVEN_REQUIRE(set_gemv1_tuning(key, value) == 0, "set_tuning: unknown key %s", key);
     return 0;
 }

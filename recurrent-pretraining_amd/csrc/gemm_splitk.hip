@@ -246,6 +246,7 @@ static int ns_cus() {
     return cus;
 }
 
+int g_linear_min_rows = 1;  // raven_set_tuning("linear_min_rows"): up to this many rows go to the kernels without a workspace
 int g_linear_ks = 0;  // raven_set_tuning("linear_ks"): K slices per weight tile, 0 = choose from the grid size
 
 template <bool SWIGLU>
@@ -283,13 +284,13 @@ static int launch_ns(NsArgs a, void* workspace, size_t workspace_bytes, hipStrea
     return raven_host::check_launch("linear (split-K MFMA)");
 }
 
-// Column block [c0, c0 + K) of a wider bf16 weight matrix with row pitch ldw, for 5..32 rows:
+// Column block [c0, c0 + K) of a wider bf16 weight matrix with row pitch ldw, for 2..32 rows:
 // y = round(x W[:, c0 : c0 + K]^T + extra), or the unrounded fp32 sums (raw_out) that a later call takes as `extra`.
 // The adapter product over [state, embedding] (recpre/raven_modeling_minimal.py:776) is split with it when the
 // embedding half stays the same over many calls; the product keeps its single rounding.
 int linear_column_block(const void* x, const void* w_block, int ldw, const float* extra, void* y, int raw_out, int M, int N, int K,
                         void* workspace, size_t workspace_bytes, hipStream_t s) {
-    if (M < 5 || M > 32 || N % 16 || K % 32 || K < 256 || !workspace || ((uintptr_t)workspace & 255)) {
+    if (M < 2 || M > 32 || N % 16 || K % 32 || K < 256 || !workspace || ((uintptr_t)workspace & 255)) {
         raven_host::set_error("linear_column_block: unsupported shape M=%d N=%d K=%d", M, N, K);
         return -1;
     }
@@ -320,7 +321,7 @@ extern "C" int raven_linear(const void* x0, const void* x1, const void* w, const
     RAVEN_REQUIRE((K1 == 0) == (x1 == nullptr), "linear: x1 and K1 must be given together");
     RAVEN_REQUIRE(!(swiglu && (residual || out_f32 || K1)), "linear: the SwiGLU epilogue takes one operand, no residual, and stores T");
     RAVEN_REQUIRE(!(K1 && (residual || out_f32)), "linear: the two-operand form has a plain epilogue");
-    bool fits = dtype == RAVEN_BF16 && M > 4 && N % 16 == 0 && K0 % 32 == 0 && K1 % 32 == 0 && workspace != nullptr &&
+    bool fits = dtype == RAVEN_BF16 && M > g_linear_min_rows && N % 16 == 0 && K0 % 32 == 0 && K1 % 32 == 0 && workspace != nullptr &&
                 ((uintptr_t)workspace & 255) == 0 && K0 / 128 + K1 / 128 >= 1;
     // Matrices with many rows give the kernel without a workspace enough workgroups and it is then the faster one
     // (its waves never wait for each other); the K split pays for few rows, once X re-reads (more than 16 token
@@ -336,7 +337,7 @@ extern "C" int raven_linear(const void* x0, const void* x1, const void* w, const
     for (int m0 = 0; m0 < M; m0 += 32) {  // the weight matrix is streamed once per 32 rows
         NsArgs a{};
         a.M = (M - m0) < 32 ? (M - m0) : 32;
-        if (a.M <= 4) {  // a short last pass
+        if (a.M <= g_linear_min_rows) {  // a short last pass
             const char* r = residual ? static_cast<const char*>(residual) + (size_t)m0 * N * 2 : nullptr;
             char* yy = static_cast<char*>(y) + (size_t)m0 * N * out_es;
             const char* xa = static_cast<const char*>(x0) + (size_t)m0 * K0 * 2;

@@ -100,7 +100,7 @@ def test_gemm_bf16_all_row_counts(pkg, M):
     assert torch.equal(yf.cpu(), y.float().cpu()), "float store must be the upcast of the rounded result"
 
 
-@pytest.mark.parametrize("M", [1, 4, 8, 32])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 8, 32])
 @pytest.mark.parametrize("N,K", [(5280, 5280), (15840, 5280), (5280, 17920)])
 def test_gemm_bf16_nebel_shapes(pkg, M, N, K):
     dt = torch.bfloat16
@@ -143,7 +143,7 @@ def test_gemm_swiglu(pkg, dt, M, I, K):
     assert close(y, wrong)[1] > 0.1, "the gate must be the first half"
 
 
-@pytest.mark.parametrize("M", [5, 8, 16, 17, 32, 33, 40])
+@pytest.mark.parametrize("M", [2, 3, 4, 5, 8, 16, 17, 32, 33, 34, 40])
 @pytest.mark.parametrize("ks", [0, 3])
 def test_linear_with_workspace_nebel_shapes(pkg, M, ks):
     """raven_linear at the 3.5b shapes, every epilogue: with the library's own choice between its two MFMA
@@ -380,6 +380,14 @@ def test_qkv_attention_decode_fused(pkg, dt, nh, hd, B, pos0):
     check(y3, want, dt, "fused decode attention, device-side position")
     y4 = pkg.hip.qkv_attention_decode(qkv.cuda(), bias.cuda(), freqs, cache, 1, B, pos0, nh, hd)
     check(y4, want, dt, "fused decode attention without workspace")
+    # the single-launch variant for few (head, row) pairs: one 1024-thread workgroup each
+    pkg.hip.set_tuning("attn_wide", 4096)
+    try:
+        y5 = pkg.hip.qkv_attention_decode(qkv.cuda(), bias.cuda(), freqs, cache, 1, B, pos0, nh, hd, workspace=ws)
+    finally:
+        pkg.hip.set_tuning("attn_wide", 0)
+    check(y5, want, dt, "fused decode attention, one workgroup per head and row")
+    assert torch.equal(kd, kd2) and torch.equal(vd, vd2)
 
 
 @pytest.mark.parametrize("nh,hd,B,S,pos0", [(55, 96, 1, 512, 0), (55, 96, 2, 100, 37), (4, 64, 3, 64, 0), (3, 128, 1, 65, 200),
