@@ -631,7 +631,9 @@ static void launch_attention(bool fused, const void* q, const void* bias, const 
         return;
     }
     const dim3 grid(cv.nh, M, ns);
-    const bool big = (int64_t)cv.nh * M * ns >= g_attn_big_grid;
+    // the 2-positions-per-row variant streams K/V past the caches and keeps more workgroups per CU: it wins whenever
+    // the launch is not split (512 or more (head, row) pairs), and for split launches from g_attn_big_grid workgroups on
+    const bool big = ns == 1 ? (int64_t)cv.nh * M >= 512 : (int64_t)cv.nh * M * ns >= g_attn_big_grid;
     const T* bias_t = (const T*)bias;
 #define RAVEN_ATTN_LAUNCH(FUSED_, U_, LOOKUP_)                                                                            \
     decode_attention_kernel<T, FUSED_, U_, LOOKUP_><<<grid, dim3(256), 0, s>>>((const T*)q, FUSED_ ? bias_t : nullptr,     \
