@@ -354,7 +354,10 @@ class RavenForCausalLM(torch.nn.Module):
         return int(num_steps)
 
     # ---- many rows (prefill): library GEMMs for the five nn.Linear products, HIP kernels for the rest ----
-    WIDE_ROWS = 64  # from this many token rows on, the GEMMs are compute-bound and go to hipBLASLt via torch.matmul
+    # From this many token rows on the five nn.Linear products go to hipBLASLt via torch.matmul: the skinny kernels take
+    # at most 32 rows per pass over the weights, and from the second pass on the library is faster (33 rows: 1.25 ms per
+    # recurrence against 1.39; 56 rows: 1.25 against 1.60; 24 rows: 1.10 against 0.82).
+    WIDE_ROWS = 33
 
     def _is_wide(self, M: int) -> bool:
         return self.dtype == torch.bfloat16 and M >= self.WIDE_ROWS and self.config.head_dim in (64, 96, 128)
@@ -370,7 +373,10 @@ class RavenForCausalLM(torch.nn.Module):
         qkv = torch.matmul(n1, blk.attn.Wqkv.weight.t())
         bias = blk.attn.qk_bias if hasattr(blk.attn, "qk_bias") else None
         q = hip.qkv_bias_rope_cache_append(qkv, bias, freqs, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim)
-        ya = hip.prefill_attention(q, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim)
+        if S >= 16:  # chunks: the MFMA kernel (64 query rows of one sequence per workgroup)
+            ya = hip.prefill_attention(q, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim)
+        else:        # many sequences with a few rows each: the per-row kernel
+            ya = hip.decode_attention(q, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim)
         a = torch.matmul(ya, blk.attn.proj.weight.t())
         x2, _, n3 = hip.rmsnorm_residual(a, blk.norm_2.weight, eps, residual=x, weight2=blk.norm_3.weight)
         g = hip.swiglu(torch.matmul(n3, blk.mlp.fc.weight.t()))
