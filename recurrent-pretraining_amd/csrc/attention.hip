@@ -539,7 +539,7 @@ __global__ __launch_bounds__(256) void paged_kv_append_kernel(const T* __restric
 }
 
 constexpr int kAttnMaxSplits = 32;
-int g_attn_split_target = 2048;  // workgroups a split launch aims for (raven_set_tuning "attn_split_target")
+int g_attn_split_target = 1536;  // workgroups a split launch aims for (raven_set_tuning "attn_split_target"); 1536 beats 2048 by 2-6 us at 3..9 sequences
 int g_attn_big_grid = 1280;      // workgroups from which the 2-positions-per-row variant is used ("attn_big_grid")
 // Few (head, row) pairs and a short cache: one 1024-thread workgroup per pair instead of a split launch and its merge
 // launch.  Alone the step is faster (bs=1, 513 positions: 11.5 us against 13.8; bs=4: 13.9 against 19.1; it loses beyond
