@@ -539,6 +539,7 @@ __global__ __launch_bounds__(256) void paged_kv_append_kernel(const T* __restric
 }
 
 constexpr int kAttnMaxSplits = 32;
+int g_attn_nosplit_pairs = 1024;  // (head, row) pairs from which a launch is never split ("attn_nosplit_pairs", at most 1024)
 int g_attn_split_target = 1536;  // workgroups a split launch aims for (raven_set_tuning "attn_split_target"); 1536 beats 2048 by 2-6 us at 3..9 sequences
 int g_attn_big_grid = 1280;      // workgroups from which the 2-positions-per-row variant is used ("attn_big_grid")
 // Few (head, row) pairs and a short cache: one 1024-thread workgroup per pair instead of a split launch and its merge
@@ -549,7 +550,7 @@ int g_attn_wide = 0;
 
 // Splits are worth their extra launch only while heads x rows cannot fill the chip.
 static int splits_for(int M, int nh, int len_hint) {
-    if ((int64_t)M * nh >= 512) return 1;
+    if ((int64_t)M * nh >= g_attn_nosplit_pairs) return 1;
     int ns = (len_hint + 63) / 64;  // 64 positions per workgroup keeps every load in one round trip
     const int cap = (g_attn_split_target + M * nh - 1) / (M * nh);
     if (ns > cap) ns = cap;
@@ -695,7 +696,7 @@ static int attention_common(const char* who, bool fused, const void* q, const vo
 extern "C" size_t raven_decode_attention_workspace_bytes(int32_t M, int32_t n_heads, int32_t head_dim) {
     using namespace raven;
     if (M <= 0 || n_heads <= 0 || head_dim <= 0) return 0;
-    if ((int64_t)M * n_heads >= 512) return 0;  // enough (head, row) pairs: never split
+    if ((int64_t)M * n_heads >= 1024) return 0;  // enough (head, row) pairs: never split
     const size_t mh = (size_t)M * n_heads;
     return raven_host::align_up(mh * kAttnMaxSplits * 2 * 4) + raven_host::align_up(mh * kAttnMaxSplits * head_dim * 4);
 }
