@@ -88,7 +88,8 @@ const char* raven_last_error(void);
  * gemv_wgs_per_cu, gemv1_pairs_norm, gemv1_pairs_plain, gemm_four_tiles (0 / 1 / 2 = never / by rule / always use
  * the four-tile MFMA variant), attn_split_target / attn_big_grid (workgroups a split decode-attention launch aims
  * for / from which its 2-positions-per-row variant is used), attn_nosplit_pairs ((head, row) pairs from which a launch is
- * never split, at most 1024), attn_wide (longest cache for which few (head, row) pairs get
+ * never split, at most 1024), rope_tiled_rows (chunk length from which raven_qkv_bias_rope_cache_append works on tiles
+ * of one head and 64 positions), attn_wide (longest cache for which few (head, row) pairs get
  * one 1024-thread workgroup each instead of a split launch; 0 = never), gemm_mfma_min_rows (fewest rows the MFMA
  * kernels take; fewer go to the vector kernels), linear_min_rows (most rows raven_linear still hands to the kernels
  * without a workspace), linear_ks (K slices of the split-K kernel behind raven_linear;

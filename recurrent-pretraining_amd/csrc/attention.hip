@@ -539,6 +539,7 @@ __global__ __launch_bounds__(256) void paged_kv_append_kernel(const T* __restric
 }
 
 constexpr int kAttnMaxSplits = 32;
+int g_rope_tiled_rows = 16;       // chunk length from which the append kernel works on (head, 16 positions) tiles ("rope_tiled_rows")
 int g_attn_nosplit_pairs = 1024;  // (head, row) pairs from which a launch is never split ("attn_nosplit_pairs", at most 1024)
 int g_attn_split_target = 1536;  // workgroups a split launch aims for (raven_set_tuning "attn_split_target"); 1536 beats 2048 by 2-6 us at 3..9 sequences
 int g_attn_big_grid = 1280;      // workgroups from which the 2-positions-per-row variant is used ("attn_big_grid")
@@ -594,6 +595,57 @@ static int check_heads(const char* who, int nh, int hd, int dtype) {
     return 0;
 }
 
+// The same for chunks of many positions: a workgroup takes one (section, head) and 64 consecutive positions, 16 lanes
+// per position and four positions per lane (all four loads issued before the first is used), so that what it writes to
+// the cache is one contiguous run of 64 head rows (the kernel above writes a token's heads to 55 places, one 192-byte
+// piece each).  Grid (position tiles, 3 * heads, sequences).
+template <typename T>
+__global__ __launch_bounds__(256) void qkv_rope_append_tiled_kernel(
+    const T* __restrict__ qkv, const T* __restrict__ qk_bias, const float* __restrict__ freqs, T* __restrict__ q_out,
+    CacheView cv, int S, int pos0, const int* __restrict__ pos_dev) {
+    constexpr int E = Chunk<T>::N, PPL = 4;
+    const int h = cv.nh * cv.hd;
+    const int s0 = blockIdx.x * 16 * PPL + (threadIdx.x >> 4), ci = threadIdx.x & 15;
+    const int sec = blockIdx.y / cv.nh, head = blockIdx.y - sec * cv.nh;  // 0 q, 1 k, 2 v
+    const int b = blockIdx.z;
+    const int d = ci * E;
+    if (d >= cv.hd) return;
+    const int first = pos_dev ? *pos_dev : pos0;
+    const int col = head * cv.hd + d;
+    Chunk<T> x[PPL];
+#pragma unroll
+    for (int j = 0; j < PPL; ++j) {
+        const int s = s0 + 16 * j;
+        x[j] = s < S ? load_chunk(qkv + ((int64_t)b * S + s) * 3 * h + sec * h + col) : zero_chunk<T>();
+    }
+    if (sec < 2) {
+        Chunk<T> bch = zero_chunk<T>();
+        if (qk_bias) bch = load_chunk(qk_bias + sec * h + col);
+#pragma unroll
+        for (int j = 0; j < PPL; ++j) {
+            const int s = min(s0 + 16 * j, S - 1);
+            if (qk_bias) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) x[j].v[e] = from_f32<T>(to_f32(x[j].v[e]) + to_f32(bch.v[e]));
+            }
+            const float* f = freqs + ((int64_t)(first + s) * (cv.hd / 2) + d / 2) * 2;
+#pragma unroll
+            for (int e = 0; e < E; e += 2) rope_pair<T>(x[j].v[e], x[j].v[e + 1], f[e], f[e + 1]);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < PPL; ++j) {
+        const int s = s0 + 16 * j, pos = first + s;
+        if (s >= S) continue;
+        if (sec == 0) {
+            store_chunk(q_out + ((int64_t)b * S + s) * h + col, x[j]);
+        } else if (pos < cv.t_max) {
+            T* base = static_cast<T*>(sec == 1 ? cv.k : cv.v);
+            store_chunk(base + cv.slot_off + (((int64_t)b * cv.nh + head) * cv.t_max + pos) * cv.hd + d, x[j]);
+        }
+    }
+}
+
 }  // namespace raven
 
 extern "C" int raven_qkv_bias_rope_cache_append(const void* qkv, const void* qk_bias, const float* freqs, void* q_out,
@@ -611,6 +663,14 @@ extern "C" int raven_qkv_bias_rope_cache_append(const void* qkv, const void* qk_
     const int chunks = 3 * n_heads * head_dim / elts;
     dim3 grid((chunks + 255) / 256, B * S);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (S >= g_rope_tiled_rows && head_dim / elts <= 16 && B <= 65535 && 3 * n_heads <= 65535) {
+        const dim3 tiles((S + 63) / 64, 3 * n_heads, B);
+        if (dtype == RAVEN_BF16)
+            qkv_rope_append_tiled_kernel<bf16><<<tiles, dim3(256), 0, s>>>((const bf16*)qkv, (const bf16*)qk_bias, freqs, (bf16*)q_out, cv, S, pos0, pos_dev);
+        else
+            qkv_rope_append_tiled_kernel<float><<<tiles, dim3(256), 0, s>>>((const float*)qkv, (const float*)qk_bias, freqs, (float*)q_out, cv, S, pos0, pos_dev);
+        return raven_host::check_launch("qkv_append");
+    }
     if (dtype == RAVEN_BF16)
         qkv_rope_append_kernel<bf16><<<grid, dim3(256), 0, s>>>((const bf16*)qkv, (const bf16*)qk_bias, freqs, (bf16*)q_out, cv, S, pos0, pos_dev);
     else

@@ -25,7 +25,7 @@ namespace raven {
 
 int set_gemv1_tuning(const char* key, int value);
 extern int g_linear_ks;
-extern int g_attn_split_target, g_attn_big_grid, g_attn_wide, g_linear_min_rows, g_attn_nosplit_pairs;
+extern int g_attn_split_target, g_attn_big_grid, g_attn_wide, g_linear_min_rows, g_attn_nosplit_pairs, g_rope_tiled_rows;
 
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
 
@@ -561,6 +561,7 @@ extern "C" int raven_set_tuning(const char* key, int32_t value) {
     else if (k == "attn_split_target" && value > 0) g_attn_split_target = value;
     else if (k == "attn_big_grid" && value > 0) g_attn_big_grid = value;
     else if (k == "attn_wide") g_attn_wide = value;
+    else if (k == "rope_tiled_rows" && value > 0) g_rope_tiled_rows = value;
     else if (k == "attn_nosplit_pairs" && value > 0 && value <= 1024) g_attn_nosplit_pairs = value;
     else if (k == "linear_min_rows" && value >= 1) g_linear_min_rows = value;
     else RAVEN_REQUIRE(set_gemv1_tuning(key, value) == 0, "set_tuning: unknown key %s", key);
