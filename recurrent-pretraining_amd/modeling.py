@@ -15,8 +15,6 @@ What differs from the reference on purpose:
 
 from __future__ import annotations
 
-import ctypes
-import math
 from dataclasses import dataclass
 from typing import Any, Callable, Optional, Union
 

@@ -9,7 +9,7 @@ vLLM is not installed where this package is built and tested: nothing here impor
 
 from __future__ import annotations
 
-from typing import Dict, Iterable, List, Tuple
+from typing import Dict, List, Tuple
 
 import torch
 
