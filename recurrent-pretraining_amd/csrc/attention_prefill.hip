@@ -24,7 +24,6 @@ namespace raven {
 
 constexpr int kPfKeys = 64;     // keys per tile
 constexpr int kPfRows = 64;     // query rows per workgroup
-constexpr int kPfMaxHd = 128;
 constexpr int kVtPitch = 72;    // bf16 elements per V^T row: 64 + 8 (144 bytes: the 8-byte reads of a half-wave hit 32 different bank pairs)
 
 struct PrefillArgs {
@@ -54,7 +53,6 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(PrefillArgs a) {
 
     const int row0 = qb * kPfRows + wave * 16;         // first query row (within the sequence) of this wave
     const int my_row = row0 + qc;                      // the query whose scores this lane holds
-    const bool row_ok = my_row < a.S;
     const int64_t head_off = a.slot_off + ((int64_t)b * a.nh + head) * a.t_max * HD;
     const bf16* Kb = a.k + head_off;
     const bf16* Vb = a.v + head_off;
