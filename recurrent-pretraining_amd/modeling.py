@@ -361,7 +361,7 @@ class RavenForCausalLM(torch.nn.Module):
         return self.dtype == torch.bfloat16 and M >= self.WIDE_ROWS and self.config.head_dim in (64, 96, 128)
 
     def _wide_block(self, blk: "SandwichBlock", x: torch.Tensor, kv, slot: int, B: int, S: int, pos0: int,
-                    n1: Optional[torch.Tensor] = None, tail_w: Optional[torch.Tensor] = None):
+                    n1: Optional[torch.Tensor] = None, tail_w: Optional[torch.Tensor] = None, pos_dev: Optional[torch.Tensor] = None):
         """One SandwichBlock (RMM:525-536) on [B*S, h] rows.  Returns (block output, tail) where tail is one more
         RMSNorm (weight tail_w: the next block's norm_1, or ln_f) of the output, fused into the closing norm launch."""
         cfg, eps = self.config, self.config.norm_eps
@@ -370,11 +370,14 @@ class RavenForCausalLM(torch.nn.Module):
             n1 = hip.rmsnorm_residual(x, blk.norm_1.weight, eps)[0]
         qkv = torch.matmul(n1, blk.attn.Wqkv.weight.t())
         bias = blk.attn.qk_bias if hasattr(blk.attn, "qk_bias") else None
-        q = hip.qkv_bias_rope_cache_append(qkv, bias, freqs, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim)
-        if S >= 16:  # chunks: the MFMA kernel (64 query rows of one sequence per workgroup)
-            ya = hip.prefill_attention(q, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim)
-        else:        # many sequences with a few rows each: the per-row kernel
-            ya = hip.decode_attention(q, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim)
+        if S == 1:   # one new row per sequence: bias, RoPE, cache append and attention in one launch
+            ya = hip.qkv_attention_decode(qkv, bias, freqs, kv, slot, B, pos0, cfg.n_heads, cfg.head_dim, pos_dev=pos_dev)
+        else:
+            q = hip.qkv_bias_rope_cache_append(qkv, bias, freqs, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim, pos_dev=pos_dev)
+            if S >= 16:  # chunks: the MFMA kernel (64 query rows of one sequence per workgroup)
+                ya = hip.prefill_attention(q, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim, pos_dev=pos_dev)
+            else:        # many sequences with a few rows each: the per-row kernel
+                ya = hip.decode_attention(q, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim, pos_dev=pos_dev)
         a = torch.matmul(ya, blk.attn.proj.weight.t())
         x2, _, n3 = hip.rmsnorm_residual(a, blk.norm_2.weight, eps, residual=x, weight2=blk.norm_3.weight)
         g = hip.swiglu(torch.matmul(n3, blk.mlp.fc.weight.t()))
@@ -382,7 +385,8 @@ class RavenForCausalLM(torch.nn.Module):
         y, _, tail = hip.rmsnorm_residual(m, blk.norm_4.weight, eps, residual=x2, weight2=tail_w)
         return y, tail
 
-    def _wide_core(self, x: torch.Tensor, embeds: torch.Tensor, slots, kv, B: int, S: int, pos0: int, ln_f: bool):
+    def _wide_core(self, x: torch.Tensor, embeds: torch.Tensor, slots, kv, B: int, S: int, pos0: int, ln_f: bool,
+                   pos_dev: Optional[torch.Tensor] = None):
         """One core_block_forward (RMM:764-781) on many rows."""
         t = self.transformer
         cur = torch.matmul(torch.cat([x, embeds], dim=-1), t.adapter.weight.t())
@@ -391,7 +395,7 @@ class RavenForCausalLM(torch.nn.Module):
         for j, blk in enumerate(t.core_block):
             last = j == n_core - 1
             tail_w = (t.ln_f.weight if ln_f else None) if last else t.core_block[j + 1].norm_1.weight
-            cur, tail = self._wide_block(blk, cur, kv, slots[j], B, S, pos0, n1=n1, tail_w=tail_w)
+            cur, tail = self._wide_block(blk, cur, kv, slots[j], B, S, pos0, n1=n1, tail_w=tail_w, pos_dev=pos_dev)
             n1 = None if last else tail
             out = tail if (last and ln_f) else cur
         if n_core == 0 and ln_f:
@@ -880,10 +884,40 @@ class DecodeRunner:
         coda = [c._slot(-(i + 1)) for i in range(n_coda)]
         return pre, core, coda
 
+    def _enqueue_wide(self):
+        """The same step for more sequences than the skinny kernels take in one pass over the weights: library GEMMs
+        around the norm / RoPE-append / attention / SwiGLU kernels (forward's path for many rows), position on the device."""
+        m, t = self.model, self.model.transformer
+        cfg, B = m.config, self.B
+        kv = self.cache.native()
+        hint = self.cache.t_max - 1
+        pre, core, coda = self._slots()
+        hip.embed(t.wte.weight, self.ids, m.emb_scale, out=self.embeds)
+        x = self.embeds
+        for i, slot in enumerate(pre):
+            x, _ = m._wide_block(t.prelude[i], x, kv, slot, B, 1, hint, pos_dev=self.pos)
+        embeds = x
+        x = self.state
+        for it in range(self.r):
+            x = m._wide_core(x, embeds, core[it], kv, B, 1, hint, ln_f=(it == self.r - 1), pos_dev=self.pos)
+        self.latents.copy_(x)
+        n_coda = len(coda)
+        for i, slot in enumerate(coda):
+            last = i == n_coda - 1
+            y, tail = m._wide_block(t.coda[i], x, kv, slot, B, 1, hint, tail_w=t.ln_f.weight if last else None, pos_dev=self.pos)
+            x = tail if last else y
+        if n_coda == 0:
+            x = hip.rmsnorm_residual(x, t.ln_f.weight, cfg.norm_eps)[0]
+        self.logits.copy_(torch.matmul(x, m.lm_head.weight.t()))
+        hip.argmax(self.logits, out=self.next_ids)
+        hip.advance_pos(self.pos, 1)
+
     def _enqueue(self):
         """Launches one token's kernels; reads the position from self.pos."""
         m, t = self.model, self.model.transformer
         nat, cfg, B = m._natives(), m.config, self.B
+        if m._is_wide(B) and self.r > 0 and len(t.core_block) > 0:
+            return self._enqueue_wide()
         kv = self.cache.native()
         hint = self.cache.t_max - 1  # sizes grids; the kernels take the true position from the device
         pre, core, coda = self._slots()

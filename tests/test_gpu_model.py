@@ -217,6 +217,36 @@ def test_wide_prefill_path_bf16(pkg, tiny16, B, S):
     assert cache.get_seq_length() == ref_cache.get_seq_length() == S + 1
 
 
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_decode_runner_beyond_one_pass_of_rows_bf16(pkg, tiny16, use_graph):
+    """More sequences than the skinny kernels take per pass over the weights: the runner's step goes through the library
+    GEMMs with the position on the device.  Teacher-forced tokens; every step's logits against the oracle and against
+    forward() on the same cache contents; the graph is captured at the second step and replayed at the third."""
+    s, w, model = tiny16
+    B, S, n_new = 40, 5, 3
+    assert model._is_wide(B)
+    g = torch.Generator().manual_seed(77)
+    ids = torch.randint(0, s.vocab_size, (B, S + n_new), generator=g)
+    states = O.initialize_state(torch.empty(B, S + n_new, s.n_embd), s, 1.0, g).to(torch.bfloat16)
+    ref_cache, cache, cache2 = O.DictCache(), pkg.HuginnDynamicCache(), pkg.HuginnDynamicCache()
+    O.forward(w, s, input_ids=ids[:, :S], input_states=states[:, :S], past_key_values=ref_cache, use_cache=True)
+    for c in (cache, cache2):
+        model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda(), past_key_values=c, use_cache=True)
+    runner = pkg.DecodeRunner(model, cache, B, s.mean_recurrence, use_graph=use_graph)
+    for i in range(n_new):
+        pos = torch.arange(S + i, S + i + 1)
+        tok, st = ids[:, S + i:S + i + 1], states[:, S + i:S + i + 1]
+        want = O.forward(w, s, input_ids=tok, input_states=st, past_key_values=ref_cache, use_cache=True, cache_position=pos)
+        fwd = model(input_ids=tok.cuda(), input_states=st.cuda(), past_key_values=cache2, use_cache=True, cache_position=pos.cuda())
+        logits, nxt, lat = runner.step(tok.cuda(), st.cuda())
+        check(logits, want.logits[:, 0], torch.bfloat16, f"runner logits, token {i}")
+        check(lat, want.latent_states[:, 0], torch.bfloat16, f"runner latents, token {i}")
+        assert torch.equal(logits, fwd.logits[:, 0]), f"token {i}: runner and forward() launch the same kernels"
+        assert torch.equal(nxt.cpu(), logits.argmax(-1).cpu())
+    assert cache.get_seq_length() == ref_cache.get_seq_length() == S + n_new
+    assert (runner.graph is not None) == use_graph
+
+
 @pytest.fixture(scope="module")
 def small242(pkg):
     """2 prelude / 4 core / 2 coda blocks like the 3.5b model (the cache's lookup strategies hard-code that structure)."""
