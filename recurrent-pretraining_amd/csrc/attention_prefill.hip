@@ -18,12 +18,13 @@
 
 #include <math.h>
 
+#include <type_traits>
+
 #include "raven_common.h"
 
 namespace raven {
 
 constexpr int kPfKeys = 64;     // keys per tile
-constexpr int kPfRows = 64;     // query rows per workgroup
 constexpr int kVtPitch = 72;    // bf16 elements per V^T row: 64 + 8 (144 bytes: the 8-byte reads of a half-wave hit 32 different bank pairs)
 
 struct PrefillArgs {
@@ -37,186 +38,272 @@ struct PrefillArgs {
     float scale_log2;
 };
 
-template <int HD>
-__global__ __launch_bounds__(256) void attention_prefill_kernel(PrefillArgs a) {
+template <int HD, int RG>
+__global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a) {
     constexpr int KS = HD / 32;      // k-steps of the score MFMA
-    constexpr int NT = HD / 16;      // 16-wide output tiles of O
+    constexpr int NT = HD / 16;      // 16-wide output tiles of O; tile NT holds the row sums
     constexpr int KP = HD + 8;       // K tile row pitch (elements): (HD*2+16) bytes, 16-byte aligned rows
-    __shared__ __align__(16) bf16 sk[kPfKeys][KP];
-    __shared__ __align__(16) bf16 svt[HD][kVtPitch];
+    constexpr int WR = 16 * RG;      // query rows per wave
+    constexpr int ROWS = 4 * WR;     // query rows per workgroup
+    __shared__ __align__(16) bf16 sk[2][kPfKeys][KP];
+    __shared__ __align__(16) bf16 svt[2][HD][kVtPitch];
 
-    const int qb = blockIdx.x, head = blockIdx.y, b = blockIdx.z;
+    const int qb = gridDim.x - 1 - blockIdx.x;  // the blocks with the most keys start first
+    const int head = blockIdx.y, b = blockIdx.z;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int qc = lane & 15, s4 = lane >> 4;
     const int h = a.nh * HD;
     const int pos0 = a.pos_dev ? *a.pos_dev : a.pos0;
 
-    const int row0 = qb * kPfRows + wave * 16;         // first query row (within the sequence) of this wave
-    const int my_row = row0 + qc;                      // the query whose scores this lane holds
+    const int row0 = qb * ROWS + wave * WR;            // first query row (within the sequence) of this wave
     const int64_t head_off = a.slot_off + ((int64_t)b * a.nh + head) * a.t_max * HD;
     const bf16* Kb = a.k + head_off;
     const bf16* Vb = a.v + head_off;
 
-    // Q fragments (B operand of S^T = K Q^T): lane supplies Q[q = l%16][d = 32*ks + 8*(l/16) ..+8]
+    // Q fragments (B operand of S^T = K Q^T): lane supplies Q[q = l%16][d = 32*ks + 8*(l/16) ..+8] of each row group
     typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-    bf16x8 qf[KS];
-    {
-        const int r = min(my_row, a.S - 1);
-        const bf16* qp = a.q + ((int64_t)b * a.S + r) * h + head * HD + 8 * s4;
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    bf16x8 qf[RG][KS];
+    int my_limit[RG];  // the query of group g whose scores this lane holds sees keys <= my_limit[g]
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + 32 * ks);
+    for (int g = 0; g < RG; ++g) {
+        const int my_row = row0 + 16 * g + qc;
+        my_limit[g] = pos0 + my_row;
+        const bf16* qp = a.q + ((int64_t)b * a.S + min(my_row, a.S - 1)) * h + head * HD + 8 * s4;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qf[g][ks] = *reinterpret_cast<const bf16x8*>(qp + 32 * ks);
     }
 
-    f32x4 o[NT];
+    f32x4 o[RG][NT + 1];
+    float ms_run[RG];  // reference maximum of each query's scores, in scaled log2 units
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) o[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;
+    for (int g = 0; g < RG; ++g) {
+        ms_run[g] = -INFINITY;
+#pragma unroll
+        for (int nt = 0; nt <= NT; ++nt) o[g][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    bf16x8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ones[e] = static_cast<bf16>(1.0f);
 
     // keys this workgroup needs: everything up to the last row's own position
-    const int last_row = min(qb * kPfRows + kPfRows, a.S) - 1;
+    const int last_row = min(qb * ROWS + ROWS, a.S) - 1;
     const int n_keys = min(pos0 + last_row + 1, a.t_max);
-    const int my_limit = pos0 + my_row;  // this lane's query sees keys <= my_limit
+    const int wave_last = pos0 + row0 + WR - 1;  // the last key that any row of this wave sees
 
-    // Global -> registers -> LDS, one tile ahead: the loads of tile kt + 64 are in flight while tile kt is multiplied.
-    // K: 16-byte chunks, row-major.  V: a thread takes the same 8 columns of 4 consecutive keys and writes, per
-    // column, the 4 keys as one 8-byte piece of the transposed tile.
-    constexpr int CPR = HD / 8;                          // chunks per key row
-    constexpr int KCH = (kPfKeys * CPR + 255) / 256;     // K chunks per thread
-    constexpr int VTASKS = (kPfKeys / 4) * CPR;          // V tasks per tile (at most 256)
-    static_assert(VTASKS <= 256, "one V task per thread");
+    // Global -> registers -> LDS, two tiles ahead of the multiply and two LDS buffers: the loads of tile i + 2 are in
+    // flight while tile i is multiplied and tile i + 1 sits in the other buffer; one barrier per tile.
+    // K: the tile is one contiguous piece of the cache, 16-byte chunks.  V: a thread takes the same 8 columns of 4
+    // consecutive keys and writes, per column, the 4 keys as one 8-byte piece of the transposed tile; threads beyond
+    // the number of such tasks repeat the first ones (same values to the same addresses), so no wave branches.
+    constexpr int CPR = HD / 8;                     // chunks per key row
+    constexpr int KCH = kPfKeys * CPR / 256;        // K chunks per thread
+    constexpr int VTASKS = (kPfKeys / 4) * CPR;     // V tasks per tile (at most 256)
+    static_assert(kPfKeys * CPR % 256 == 0 && VTASKS <= 256, "staging shape");
     u32x4 kreg[KCH];
-    Chunk<bf16> vreg[4];
-    const int v_kg = threadIdx.x % (kPfKeys / 4), v_dc = threadIdx.x / (kPfKeys / 4);
+    u32x4 vreg[4];
+    const int v_task = threadIdx.x < VTASKS ? threadIdx.x : threadIdx.x - VTASKS;
+    const int v_kg = v_task % (kPfKeys / 4), v_dc = v_task / (kPfKeys / 4);
+    const bf16* k_src = Kb + threadIdx.x * 8;
+    const bf16* v_src = Vb + (int64_t)(4 * v_kg) * HD + v_dc * 8;
+    int k_dst[KCH];  // element offsets inside one K buffer
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+        const int c = threadIdx.x + 256 * i;
+        k_dst[i] = (c / CPR) * KP + (c % CPR) * 8;
+    }
+    // Inside each block of 32 keys the transposed tile keeps the 4-key pieces in the order the P fragments want them:
+    // piece r = 4*(t&1) + s4 (keys 16*(t&1) + 4*s4 ..+3) sits at 8*s4 + 4*(t&1), so a lane's 8 keys of a k-step are
+    // one 16-byte read.
+    const int v_dst = (v_dc * 8) * kVtPitch + 32 * (v_kg / 8) + 8 * (v_kg % 4) + 4 * ((v_kg % 8) / 4);
     auto fetch = [&](int kt) {
+        if (kt + kPfKeys <= a.t_max) {
 #pragma unroll
-        for (int i = 0; i < KCH; ++i) {
-            const int c = threadIdx.x + 256 * i;
-            if (c < kPfKeys * CPR) {
+            for (int i = 0; i < KCH; ++i) kreg[i] = *reinterpret_cast<const u32x4*>(k_src + (int64_t)kt * HD + 2048 * i);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) vreg[i] = *reinterpret_cast<const u32x4*>(v_src + (int64_t)kt * HD + i * HD);
+        } else {  // the cache ends inside this tile: rows past it are masked below, their loads stay in bounds
+#pragma unroll
+            for (int i = 0; i < KCH; ++i) {
+                const int c = threadIdx.x + 256 * i;
                 const int key = c / CPR, dc = c - key * CPR;
-                const int kpos = min(kt + key, a.t_max - 1);  // rows past n_keys are masked below; stay in bounds
-                kreg[i] = *reinterpret_cast<const u32x4*>(Kb + (int64_t)kpos * HD + dc * 8);
+                kreg[i] = *reinterpret_cast<const u32x4*>(Kb + (int64_t)min(kt + key, a.t_max - 1) * HD + dc * 8);
             }
-        }
-        if (threadIdx.x < VTASKS) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) vreg[i] = load_chunk(Vb + (int64_t)min(kt + 4 * v_kg + i, a.t_max - 1) * HD + v_dc * 8);
+            for (int i = 0; i < 4; ++i)
+                vreg[i] = *reinterpret_cast<const u32x4*>(Vb + (int64_t)min(kt + 4 * v_kg + i, a.t_max - 1) * HD + v_dc * 8);
         }
     };
-    auto park = [&]() {
+    auto park = [&](int buf) {
+        bf16* kb = &sk[buf][0][0];
 #pragma unroll
-        for (int i = 0; i < KCH; ++i) {
-            const int c = threadIdx.x + 256 * i;
-            if (c < kPfKeys * CPR) {
-                const int key = c / CPR, dc = c - key * CPR;
-                *reinterpret_cast<u32x4*>(&sk[key][dc * 8]) = kreg[i];
-            }
-        }
-        if (threadIdx.x < VTASKS) {
+        for (int i = 0; i < KCH; ++i) *reinterpret_cast<u32x4*>(kb + k_dst[i]) = kreg[i];
+        bf16* vb = &svt[buf][0][0] + v_dst;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                bf16 four[4] = {vreg[0].v[e], vreg[1].v[e], vreg[2].v[e], vreg[3].v[e]};
-                typedef unsigned int u32x2s __attribute__((ext_vector_type(2)));
-                *reinterpret_cast<u32x2s*>(&svt[v_dc * 8 + e][4 * v_kg]) = *reinterpret_cast<const u32x2s*>(four);
-            }
+        for (int e = 0; e < 4; ++e) {  // 32-bit word e of the four chunks holds columns 2e, 2e+1
+            const unsigned w0 = vreg[0][e], w1 = vreg[1][e], w2 = vreg[2][e], w3 = vreg[3][e];
+            const u32x2 even = {__builtin_amdgcn_perm(w1, w0, 0x05040100u), __builtin_amdgcn_perm(w3, w2, 0x05040100u)};
+            const u32x2 odd = {__builtin_amdgcn_perm(w1, w0, 0x07060302u), __builtin_amdgcn_perm(w3, w2, 0x07060302u)};
+            *reinterpret_cast<u32x2*>(vb + (2 * e) * kVtPitch) = even;
+            *reinterpret_cast<u32x2*>(vb + (2 * e + 1) * kVtPitch) = odd;
         }
     };
-    if (n_keys > 0) fetch(0);
-    for (int kt = 0; kt < n_keys; kt += kPfKeys) {
-        __syncthreads();  // the previous tile has been consumed
-        park();
-        if (kt + kPfKeys < n_keys) fetch(kt + kPfKeys);
+
+    // One key tile against the wave's rows.  MASKED: some key of the tile is hidden from some row (the tiles on the
+    // diagonal); all other tiles run the same code without the comparisons.
+    auto tile = [&](int kt, int buf, auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        // S^T sub-tiles: sc[g][t][v] = score of key kt + 16 t + 4 s4 + v against query qc of group g
+        f32x4 sc[RG][4];
+#pragma unroll
+        for (int g = 0; g < RG; ++g)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) sc[g][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&sk[buf][16 * t + qc][32 * ks + 8 * s4]));
+#pragma unroll
+                for (int g = 0; g < RG; ++g) sc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[g][ks], sc[g][t], 0, 0, 0);
+            }
+        float ms_new[RG];
+        bool moved = false;
+#pragma unroll
+        for (int g = 0; g < RG; ++g) {
+            if (MASKED) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (kt + 16 * t + 4 * s4 + v > my_limit[g]) sc[g][t][v] = -INFINITY;
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) mx = fmaxf(mx, sc[g][t][v]);
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            // The reference maximum follows the scores lazily: it moves only when a tile exceeds it by more than 2^8
+            // (weights stay below 256, far inside the range of float and bf16), so O is rescaled a few times per query
+            // instead of whenever any of its 16 queries sees a new maximum.
+            const float mxs = mx * a.scale_log2;
+            const bool up = mxs > ms_run[g] + 8.f;
+            ms_new[g] = up ? mxs : ms_run[g];
+            moved |= up;
+        }
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+            for (int g = 0; g < RG; ++g) {
+                // 0 for the first tile, 1 where nothing moved (also for a query that has not seen a key yet)
+                const float corr = (ms_new[g] == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(ms_run[g] - ms_new[g]);
+                // O rows are queries 4*s4 + v: fetch their factor from the lane that tracks that query
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float cv = __shfl(corr, 4 * s4 + v, 64);
+#pragma unroll
+                    for (int nt = 0; nt <= NT; ++nt) o[g][nt][v] *= cv;
+                }
+                ms_run[g] = ms_new[g];
+            }
+        }
+        // O += P V in 2*NT steps: step i multiplies V fragment i = (k-step c = i / NT, columns 16*(i % NT) ..+15) into both
+        // row groups.  Three fragments are in flight (the first ones are requested before the exponentials), and the
+        // exponentials of the second k-step sit between the products of the first; scheduling fences keep that order.
+        constexpr int NF = 2 * NT;
+        auto vfrag = [&](int i) {
+            return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&svt[buf][16 * (i % NT) + qc][32 * (i / NT) + 8 * s4]));
+        };
+        bf16x8 vf[3];
+#pragma unroll
+        for (int i = 0; i < 3; ++i) vf[i] = vfrag(i);
+        float ms[RG];
+        bf16x8 pf[RG][2];
+#pragma unroll
+        for (int g = 0; g < RG; ++g) {
+            // a query with no visible key yet (rows past S only) still has -inf: subtract 0 instead, every weight is then 0
+            ms[g] = (ms_run[g] == -INFINITY) ? 0.f : ms_run[g];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    pf[g][0][t * 4 + v] = static_cast<bf16>(__builtin_amdgcn_exp2f(__builtin_fmaf(sc[g][t][v], a.scale_log2, -ms[g])));
+        }
+        constexpr int LATE = RG * 8;                 // weights of the second k-step
+        constexpr int PER = (LATE + NT - 1) / NT;    // of them per step of the first k-step
+#pragma unroll
+        for (int i = 0; i < NF; ++i) {
+            __builtin_amdgcn_sched_barrier(0);
+            const int c = i / NT, nt = i % NT;
+#pragma unroll
+            for (int g = 0; g < RG; ++g) o[g][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[g][c], vf[i % 3], o[g][nt], 0, 0, 0);
+            // the row sums, in O's layout, from the weights as rounded for the product: a tile of ones as V
+            if (nt == NT - 1) {
+#pragma unroll
+                for (int g = 0; g < RG; ++g) o[g][NT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[g][c], ones, o[g][NT], 0, 0, 0);
+            }
+            if (i + 3 < NF) vf[i % 3] = vfrag(i + 3);
+            if (c == 0) {
+#pragma unroll
+                for (int j = nt * PER; j < (nt + 1) * PER && j < LATE; ++j) {
+                    const int g = j / 8, e = j % 8;
+                    pf[g][1][e] = static_cast<bf16>(__builtin_amdgcn_exp2f(__builtin_fmaf(sc[g][2 + e / 4][e % 4], a.scale_log2, -ms[g])));
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    if (n_keys > 0) {
+        fetch(0);
+        park(0);
+    }
+    // The Q fragments pass through an empty asm statement: the compiler waits for their loads here, once, and inside
+    // the loop they are no longer load results -- otherwise its wait for them (counted from the newest load) sits in the
+    // loop and drains the tile fetched ahead on every trip.
+#pragma unroll
+    for (int g = 0; g < RG; ++g)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            u32x4 t = __builtin_bit_cast(u32x4, qf[g][ks]);
+            asm volatile("" : "+v"(t));
+            qf[g][ks] = __builtin_bit_cast(bf16x8, t);
+        }
+    if (kPfKeys < n_keys) fetch(kPfKeys);
+    __syncthreads();
+    int buf = 0;
+    for (int kt = 0; kt < n_keys; kt += kPfKeys, buf ^= 1) {
+        if (kt + kPfKeys - 1 <= pos0 + row0) tile(kt, buf, std::false_type{});
+        else if (kt <= wave_last) tile(kt, buf, std::true_type{});
+        if (kt + kPfKeys < n_keys) {
+            park(buf ^ 1);  // last read two tiles ago; every wave has passed the barrier since
+            if (kt + 2 * kPfKeys < n_keys) fetch(kt + 2 * kPfKeys);
+        }
         __syncthreads();
-
-        // S^T sub-tiles: sc[t][v] = score of key kt + 16 t + 4 s4 + v against query qc
-        f32x4 sc[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            sc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&sk[16 * t + qc][32 * ks + 8 * s4]));
-                sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], sc[t], 0, 0, 0);
-            }
-        }
-        // scale, causal mask (only tiles that reach past the wave's first query need it), tile maximum for this query
-        float mx = -INFINITY;
-        if (kt + kPfKeys - 1 <= pos0 + row0) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    sc[t][v] *= a.scale_log2;
-                    mx = fmaxf(mx, sc[t][v]);
-                }
-        } else {
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int key = kt + 16 * t + 4 * s4 + v;
-                    float x = sc[t][v] * a.scale_log2;
-                    if (key > my_limit) x = -INFINITY;
-                    sc[t][v] = x;
-                    mx = fmaxf(mx, x);
-                }
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);
-        // a query with no visible key yet (rows past S only) has m_new = -inf: subtract 0 instead, every weight is then 0
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        float psum = 0.f;  // over this lane's 16 keys; the four lanes of a query are added up once, after the last tile
-        bf16x8 pf[2];
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const float p = __builtin_amdgcn_exp2f(sc[t][v] - m_use);
-                psum += p;
-                pf[t >> 1][(t & 1) * 4 + v] = static_cast<bf16>(p);
-            }
-        // the running maximum of most queries stops moving after a few tiles: rescale only when some lane's did
-        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
-            const float corr = __builtin_amdgcn_exp2f(m_run - m_use);  // 0 for the first visible tile (m_run = -inf)
-            l_run = l_run * corr + psum;
-            // O rows are queries 4*s4 + v: fetch their rescale factor from the lane that tracks that query
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const float cv = __shfl(corr, 4 * s4 + v, 64);
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) o[nt][v] *= cv;
-            }
-        } else {
-            l_run += psum;
-        }
-        m_run = m_new;
-
-        // O += P V: k-step c covers sub-tiles (2c, 2c+1); slot (s4, e) is key 16*(2c + e/4) + 4*s4 + e%4
-#pragma unroll
-        for (int c = 0; c < 2; ++c)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const bf16* vrow = &svt[16 * nt + qc][0];
-                typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-                const u32x2 lo = *reinterpret_cast<const u32x2*>(vrow + 32 * c + 4 * s4);
-                const u32x2 hi = *reinterpret_cast<const u32x2*>(vrow + 32 * c + 16 + 4 * s4);
-                const u32x4 both = {lo.x, lo.y, hi.x, hi.y};
-                o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[c], __builtin_bit_cast(bf16x8, both), o[nt], 0, 0, 0);
-            }
     }
 
-    // normalise and store: O row v of this lane is query 4*s4 + v, column 16*nt + qc
-    l_run += __shfl_xor(l_run, 16, 64);
-    l_run += __shfl_xor(l_run, 32, 64);
+    // Normalise and store.  O row v of this lane is query 4*s4 + v of its group, column 16*nt + qc: the wave turns its
+    // rows round through LDS (the K buffers are free after the last barrier; each wave has its own WR x KP piece) and
+    // writes 16-byte pieces of whole rows.
+    bf16* ot = &sk[0][0][0] + wave * (WR * KP);
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        const float lv = __shfl(l_run, 4 * s4 + v, 64);
-        const int row = row0 + 4 * s4 + v;
-        if (row < a.S) {
-            bf16* yp = a.y + ((int64_t)b * a.S + row) * h + head * HD + qc;
+    for (int g = 0; g < RG; ++g)
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) yp[16 * nt] = from_f32<bf16>(o[nt][v] / lv);
+        for (int v = 0; v < 4; ++v) {
+            const float inv = __builtin_amdgcn_rcpf(o[g][NT][v]);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) ot[(16 * g + 4 * s4 + v) * KP + 16 * nt + qc] = from_f32<bf16>(o[g][nt][v] * inv);
         }
+    // the wave reads only what it wrote itself: no barrier, the LDS operations of a wave complete in order
+    constexpr int OCH = WR * CPR / 64;  // 16-byte pieces per lane
+#pragma unroll
+    for (int i = 0; i < OCH; ++i) {
+        const int c = lane + 64 * i;
+        const int r = c / CPR, dc = c - r * CPR;
+        const int row = row0 + r;
+        if (row < a.S)
+            *reinterpret_cast<u32x4*>(a.y + ((int64_t)b * a.S + row) * h + head * HD + dc * 8) = *reinterpret_cast<const u32x4*>(ot + r * KP + dc * 8);
     }
 }
 
@@ -245,10 +332,17 @@ extern "C" int raven_prefill_attention(const void* q, void* y, const raven_kv_ca
     a.slot_off = (int64_t)sl * cache->batch * n_heads * cache->t_max * head_dim;
     a.nh = n_heads; a.hd = head_dim; a.t_max = cache->t_max; a.S = S; a.pos0 = pos0; a.pos_dev = pos_dev;
     a.scale_log2 = (float)(1.0 / sqrt((double)head_dim) * 1.4426950408889634);
-    const dim3 grid((S + kPfRows - 1) / kPfRows, n_heads, B);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (head_dim == 64) attention_prefill_kernel<64><<<grid, dim3(256), 0, s>>>(a);
-    else if (head_dim == 96) attention_prefill_kernel<96><<<grid, dim3(256), 0, s>>>(a);
-    else attention_prefill_kernel<128><<<grid, dim3(256), 0, s>>>(a);
+    // two row groups of 16 per wave (128 query rows per workgroup) share every K and V fragment read from LDS
+    const bool two = S > 64;
+    const int rows = two ? 128 : 64;
+    const dim3 grid((S + rows - 1) / rows, n_heads, B);
+#define RAVEN_PREFILL(HD)                                                                  \
+    if (two) attention_prefill_kernel<HD, 2><<<grid, dim3(256), 0, s>>>(a);                \
+    else attention_prefill_kernel<HD, 1><<<grid, dim3(256), 0, s>>>(a)
+    if (head_dim == 64) { RAVEN_PREFILL(64); }
+    else if (head_dim == 96) { RAVEN_PREFILL(96); }
+    else { RAVEN_PREFILL(128); }
+#undef RAVEN_PREFILL
     return raven_host::check_launch("prefill_attention");
 }
