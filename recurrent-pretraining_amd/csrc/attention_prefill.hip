@@ -5,16 +5,22 @@
 // S > 1: plain causal when the cache was empty, lower-right-aligned causal otherwise).  The new
 // keys/values are already in the cache (raven_qkv_bias_rope_cache_append ran before).
 //
-// Grid (query blocks of 64, heads, sequences); 4 waves, each owns 16 query rows and walks all key
-// tiles of 64 positions on its own (no cross-wave softmax state).  Per key tile:
-//   * the workgroup stages K [64 x hd] and V transposed [hd x 64] in LDS;
-//   * S^T = K Q^T with v_mfma_f32_16x16x32_bf16: a lane then holds, for ONE query (l % 16), the scores
-//     of keys 4*(l/16) + v of each 16-key sub-tile -- exactly the lane-row / k-slice shape the A operand
-//     of the next MFMA wants, so P never leaves registers: the 32 "k" slots of a P V MFMA are mapped to
-//     keys (sub-tile pair, 4*(l/16) + v), and V^T is read from LDS with the same mapping;
-//   * online softmax per query: max/sum across the 4 lanes that share a query (two shuffles each),
-//     exp2 with the scale folded in; the output tile O [16 q x hd] lives in the MFMA accumulator layout
-//     (q = 4*(l/16) + v), so the per-query rescale factors are fetched with one shuffle per v.
+// Grid (query blocks of 64 or 128 rows, heads, sequences), the blocks with the most keys first; 4 waves, each owns
+// RG groups of 16 query rows (RG = 1 or 2) and walks all key tiles of 64 positions on its own (no cross-wave softmax
+// state).  Per key tile:
+//   * the workgroup stages K [64 x hd] and V transposed [hd x 64] in one of two LDS buffers, through registers that
+//     were loaded one tile earlier (so the tile two ahead is in flight during the products; one barrier per tile);
+//   * S^T = K Q^T with v_mfma_f32_16x16x32_bf16, every K fragment multiplied into all row groups: a lane then holds,
+//     for ONE query (l % 16) of each group, the scores of keys 4*(l/16) + v of each 16-key sub-tile -- exactly the
+//     lane-row / k-slice shape the A operand of the next MFMA wants, so P never leaves registers: the 32 "k" slots
+//     of a P V MFMA are mapped to keys (sub-tile pair, 4*(l/16) + v), and V^T is laid out in LDS in that order;
+//   * online softmax per query against a reference maximum that moves only when a tile exceeds it by 2^8 (O is then
+//     rescaled, with factors fetched by one shuffle per row); exp2 with the scale folded in; the row sums come from
+//     one more MFMA against a tile of ones, in O's own layout;
+//   * O += P V with three V fragments in flight and the exponentials of the second k-step between the products of
+//     the first; the wave raises its priority for the product phases so that the other wave of the SIMD fills the
+//     gaps with its softmax.
+// The output goes through LDS once, to be written as 16-byte pieces of whole rows.
 
 #include <math.h>
 
@@ -25,7 +31,7 @@
 namespace raven {
 
 constexpr int kPfKeys = 64;     // keys per tile
-constexpr int kVtPitch = 72;    // bf16 elements per V^T row: 64 + 8 (144 bytes: the 8-byte reads of a half-wave hit 32 different bank pairs)
+constexpr int kVtPitch = 72;    // bf16 elements per V^T row: 64 + 8 (144 bytes: the 16-byte reads of 16 rows hit 64 different banks)
 
 struct PrefillArgs {
     const bf16* q;   // [B*S, h]
@@ -37,6 +43,18 @@ struct PrefillArgs {
     const int* pos_dev;
     float scale_log2;
 };
+
+// Maximum over the four lanes l, l^16, l^32, l^48 (the lanes that share a query), in every lane, with the two row-swap
+// instructions of gfx950 instead of two round trips through the LDS crossbar: after v_permlane16_swap of a register
+// with a copy of itself the pair holds rows (0,0,2,2) and (1,1,3,3) of 16 lanes, after v_permlane32_swap the two halves.
+__device__ __forceinline__ float max_over_quarters(float x) {
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    unsigned u = __builtin_bit_cast(unsigned, x);
+    const u32x2 r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    u = __builtin_bit_cast(unsigned, fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1])));
+    const u32x2 q = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__builtin_bit_cast(float, q[0]), __builtin_bit_cast(float, q[1]));
+}
 
 template <int HD, int RG>
 __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a) {
@@ -159,6 +177,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
         for (int g = 0; g < RG; ++g)
 #pragma unroll
             for (int t = 0; t < 4; ++t) sc[g][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        __builtin_amdgcn_s_setprio(3);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
@@ -167,6 +186,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
 #pragma unroll
                 for (int g = 0; g < RG; ++g) sc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[g][ks], sc[g][t], 0, 0, 0);
             }
+        __builtin_amdgcn_s_setprio(0);
         float ms_new[RG];
         bool moved = false;
 #pragma unroll
@@ -183,8 +203,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
             for (int t = 0; t < 4; ++t)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) mx = fmaxf(mx, sc[g][t][v]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = max_over_quarters(mx);
             // The reference maximum follows the scores lazily: it moves only when a tile exceeds it by more than 2^8
             // (weights stay below 256, far inside the range of float and bf16), so O is rescaled a few times per query
             // instead of whenever any of its 16 queries sees a new maximum.
@@ -232,6 +251,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
         }
         constexpr int LATE = RG * 8;                 // weights of the second k-step
         constexpr int PER = (LATE + NT - 1) / NT;    // of them per step of the first k-step
+        __builtin_amdgcn_s_setprio(3);
 #pragma unroll
         for (int i = 0; i < NF; ++i) {
             __builtin_amdgcn_sched_barrier(0);
@@ -253,6 +273,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
             }
         }
         __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(0);
     };
 
     if (n_keys > 0) {
@@ -286,24 +307,29 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
     // Normalise and store.  O row v of this lane is query 4*s4 + v of its group, column 16*nt + qc: the wave turns its
     // rows round through LDS (the K buffers are free after the last barrier; each wave has its own WR x KP piece) and
     // writes 16-byte pieces of whole rows.
-    bf16* ot = &sk[0][0][0] + wave * (WR * KP);
+    constexpr int ER = RG == 1 ? 16 : 32;  // rows per pass
+    bf16* ot = &sk[0][0][0] + wave * (ER * KP);
 #pragma unroll
-    for (int g = 0; g < RG; ++g)
+    for (int g0 = 0; g0 < RG; g0 += ER / 16) {
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const float inv = __builtin_amdgcn_rcpf(o[g][NT][v]);
+        for (int gg = 0; gg < ER / 16; ++gg)
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) ot[(16 * g + 4 * s4 + v) * KP + 16 * nt + qc] = from_f32<bf16>(o[g][nt][v] * inv);
+            for (int v = 0; v < 4; ++v) {
+                const float inv = __builtin_amdgcn_rcpf(o[g0 + gg][NT][v]);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    ot[(16 * gg + 4 * s4 + v) * KP + 16 * nt + qc] = from_f32<bf16>(o[g0 + gg][nt][v] * inv);
+            }
+        // the wave reads only what it wrote itself: no barrier, the LDS operations of a wave complete in order
+        constexpr int OCH = ER * CPR / 64;  // 16-byte pieces per lane
+#pragma unroll
+        for (int i = 0; i < OCH; ++i) {
+            const int c = lane + 64 * i;
+            const int r = c / CPR, dc = c - r * CPR;
+            const int row = row0 + 16 * g0 + r;
+            if (row < a.S)
+                *reinterpret_cast<u32x4*>(a.y + ((int64_t)b * a.S + row) * h + head * HD + dc * 8) = *reinterpret_cast<const u32x4*>(ot + r * KP + dc * 8);
         }
-    // the wave reads only what it wrote itself: no barrier, the LDS operations of a wave complete in order
-    constexpr int OCH = WR * CPR / 64;  // 16-byte pieces per lane
-#pragma unroll
-    for (int i = 0; i < OCH; ++i) {
-        const int c = lane + 64 * i;
-        const int r = c / CPR, dc = c - r * CPR;
-        const int row = row0 + r;
-        if (row < a.S)
-            *reinterpret_cast<u32x4*>(a.y + ((int64_t)b * a.S + row) * h + head * HD + dc * 8) = *reinterpret_cast<const u32x4*>(ot + r * KP + dc * 8);
     }
 }
 
@@ -334,11 +360,14 @@ extern "C" int raven_prefill_attention(const void* q, void* y, const raven_kv_ca
     a.scale_log2 = (float)(1.0 / sqrt((double)head_dim) * 1.4426950408889634);
     hipStream_t s = static_cast<hipStream_t>(stream);
     // two row groups of 16 per wave (128 query rows per workgroup) share every K and V fragment read from LDS
-    const bool two = S > 64;
-    const int rows = two ? 128 : 64;
+    // Two row groups of 16 per wave (128 query rows per workgroup) share every K and V fragment read from LDS; short
+    // launches keep 64 rows per workgroup so that there are more workgroups than compute units.
+    const int64_t wgs128 = (int64_t)((S + 127) / 128) * n_heads * B;
+    const int rg = wgs128 >= 512 ? 2 : 1;
+    const int rows = 64 * rg;
     const dim3 grid((S + rows - 1) / rows, n_heads, B);
 #define RAVEN_PREFILL(HD)                                                                  \
-    if (two) attention_prefill_kernel<HD, 2><<<grid, dim3(256), 0, s>>>(a);                \
+    if (rg == 2) attention_prefill_kernel<HD, 2><<<grid, dim3(256), 0, s>>>(a);            \
     else attention_prefill_kernel<HD, 1><<<grid, dim3(256), 0, s>>>(a)
     if (head_dim == 64) { RAVEN_PREFILL(64); }
     else if (head_dim == 96) { RAVEN_PREFILL(96); }
