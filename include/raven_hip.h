@@ -246,7 +246,7 @@ int raven_qkv_attention_decode(const void* qkv, const void* qk_bias, const float
 /* Causal attention for a prefill chunk on the matrix cores (bf16; head_dim 64, 96 or 128): the S > 1
  * cases of RMM:484-491.  Same contract as raven_decode_attention -- row m of sequence b attends to cached
  * positions 0 .. pos0 + (m % S), the chunk's keys/values are already in the cache -- but one workgroup
- * serves 64 query rows of a head and streams the keys once for all of them. */
+ * serves 64 or 128 query rows of a head and streams the keys once for all of them. */
 int raven_prefill_attention(const void* q, void* y, const raven_kv_cache* cache, int32_t slot,
                             int32_t B, int32_t S, int32_t pos0, const int32_t* pos_dev,
                             int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream);
@@ -254,6 +254,13 @@ int raven_prefill_attention(const void* q, void* y, const raven_kv_cache* cache,
 /* SiLU-gate of a materialised fc output (RMM:507-508): out[m, j] = T(T(silu(z[m, j])) * z[m, I + j]);
  * z [M, 2I], out [M, I].  For callers that run mlp.fc as a library GEMM (large M). */
 int raven_swiglu(const void* z, void* out, int32_t M, int32_t I, int32_t dtype, void* stream);
+
+/* The state perturbation in front of a recurrence when the config's test_time_noise is set (RMM:815-833, before the
+ * renormalisation, which is raven_rmsnorm_residual with the last core block's norm_4): y = T(T(x * keep) + m) with
+ * m = T(noise * a), and m = T(m / d) when d != 0 -- one rounding per torch operation of the reference's expression
+ * `x * (1 - c) + randn_like(x) * n [/ step]`; the caller draws `noise` and computes keep, a, d for the noise type. */
+int raven_noise_mix(const void* x, const void* noise, void* y, int64_t n, float keep, float a, float d,
+                    int32_t dtype, void* stream);
 
 /* Token embedding times sqrt(h) (RMM:667-671): out[m] = T(wte[ids[m]] * scale); ids are int64. */
 int raven_embed(const void* wte, const int64_t* ids, void* out, int32_t M, int32_t dim,

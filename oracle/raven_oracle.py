@@ -38,6 +38,11 @@ How each function is pinned (tests/test_oracle_pins.py), without running the ref
                      "fixed" strategy and for exit thresholds 0 and infinity.  The later positions' tokens
                      (whose inputs change from step to step) have no independent check: parity unpinned
                      beyond that                                                     -> partly pinned
+  inject_noise       amplitude n = t * sqrt(2/5) and the per-type coefficients (n/(k+1), n/sqrt(k+1), max(n, (r-k)/r),
+                     2un) by closed form on x = 0 / noise = 1; zero noise leaves norm_4(x) (scale invariance);
+                     "line" at step 0 replaces the state, so forward() no longer depends on input_states;
+                     the roundings against the reference's expression evaluated by torch ON THE GPU
+                     (tests/test_gpu_model.py)                                        -> pinned
 The reference holds no golden vectors for this path (it has no test suite); the only
 exact numbers it publishes are three KV-cache sizes, used as known-answer tests.
 """
@@ -69,6 +74,8 @@ class RavenShape:
     rope_base: float = 50000.0
     norm_eps: float = 1e-6
     qk_bias: bool = True
+    test_time_noise: float = 0.0
+    test_time_noise_type: str = "fixed"
 
     @property
     def head_dim(self) -> int:
@@ -337,8 +344,51 @@ def sandwich_block(x, w, prefix, freqs, step_idx, cache, s: RavenShape):
     return rmsnorm(m + x, w[f"{prefix}.norm_4.weight"], eps)
 
 
-def core_block_forward(x, embeds, w, freqs, cache, block_idx: int, s: RavenShape):
-    """RMM:764-781 with test_time_noise == 0.  Adapter input order is (state, embedded input)."""
+def inject_noise(x, current_step: int, w, s: RavenShape, draws=None, renorm: bool = True):
+    """RMM:815-837: x <- x * (1 - c) + randn_like(x) * c with c from the noise type and the recurrence index, then the
+    last core block's norm_4 again.  `draws` supplies the random numbers (normal(x), uniform(x)) so that a checker and a
+    checked run can share them.
+
+    Every product, quotient and sum of the reference's expression is one elementwise torch op and rounds to the state's
+    dtype.  Its operands are Python floats (the elementwise GPU kernels take them as float32) and, for "geom" and
+    "sqrt", 0-dim float32 tensors ON THE DEVICE: ATen's GPU kernels convert such an operand to the result dtype before
+    the operation (torch on the CPU keeps it in float32 -- the two differ, so the roundings are spelled out here
+    rather than left to CPU torch's promotion)."""
+    if s.test_time_noise <= 0:
+        return x
+    dt = x.dtype
+    f = lambda v: torch.tensor(v, dtype=torch.float32)
+    dev0 = lambda v: v.to(dt).float()          # a 0-dim device tensor as the GPU kernel takes it
+    rnd = lambda v: v.to(dt).float()           # the rounding of an op's result
+    n = s.test_time_noise * s.init_std * s.emb_scale
+    kind = s.test_time_noise_type
+    if kind == "chi":                          # the reference draws the amplitude before the noise
+        u = (draws.uniform(x) if draws is not None else torch.rand(1, dtype=dt)).to(dt).float()
+    noise = (draws.normal(x) if draws is not None else torch.randn_like(x)).to(dt).float()
+    if kind in ("geom", "sqrt"):               # RMM:818-823
+        d = f(current_step + 1) if kind == "geom" else f(current_step + 1).sqrt()
+        keep = dev0(1 - f(n) / d)
+        mixed = rnd(rnd(noise * f(n)) / dev0(d))
+    elif kind == "line":                       # RMM:824-826
+        c = max(n, (s.mean_recurrence - current_step) / s.mean_recurrence)
+        keep, mixed = f(1 - c), rnd(noise * f(c))
+    elif kind == "chi":                        # RMM:827-829
+        c = rnd(rnd(2 * u) * f(n))
+        keep, mixed = rnd(1 - c), rnd(noise * c)
+    elif kind == "fixed":                      # RMM:830-831
+        keep, mixed = f(1 - n), rnd(noise * f(n))
+    else:
+        raise ValueError(kind)
+    x = (rnd(x.float() * keep) + mixed).to(dt)
+    if renorm:
+        last = s.n_layers_in_recurrent_block - 1
+        x = rmsnorm(x, w[f"transformer.core_block.{last}.norm_4.weight"], s.norm_eps)
+    return x
+
+
+def core_block_forward(x, embeds, w, freqs, cache, block_idx: int, s: RavenShape, current_step: int = 0, noise_draws=None):
+    """RMM:764-781.  Adapter input order is (state, embedded input)."""
+    x = inject_noise(x, current_step, w, s, noise_draws)
     x = linear(torch.cat([x, embeds], dim=-1), w["transformer.adapter.weight"])
     for j in range(s.n_layers_in_recurrent_block):
         block_idx += 1
@@ -371,12 +421,12 @@ def split_num_steps(num_steps, s: RavenShape) -> tuple[int, int]:
 
 
 def iterate_forward(embeds, input_states, w, freqs, block_idx: int, cache, num_steps, s: RavenShape,
-                    init_scale: float = 1.0, generator=None):
-    """RMM:726-762 (inference: the no-grad and grad loops do the same arithmetic)."""
+                    init_scale: float = 1.0, generator=None, noise_draws=None):
+    """RMM:726-762 (inference: the no-grad and grad loops do the same arithmetic and number their steps through)."""
     x = initialize_state(embeds, s, init_scale, generator) if input_states is None else input_states.clone()
     n0, n1 = split_num_steps(num_steps, s)
-    for _ in range(n0 + n1):
-        x, block_idx = core_block_forward(x, embeds, w, freqs, cache, block_idx, s)
+    for step in range(n0 + n1):
+        x, block_idx = core_block_forward(x, embeds, w, freqs, cache, block_idx, s, step, noise_draws)
     return rmsnorm(x, w["transformer.ln_f.weight"], s.norm_eps), block_idx
 
 
@@ -399,7 +449,7 @@ class OracleOutput:
 
 def forward(w, s: RavenShape, input_ids=None, input_embeds=None, input_states=None, position_ids=None,
             num_steps=None, past_key_values=None, use_cache=False, cache_position=None, init_scale=1.0,
-            generator=None) -> OracleOutput:
+            generator=None, noise_draws=None) -> OracleOutput:
     """RavenForCausalLM.forward, RMM:638-724 (labels / stats branches left out; attention_mask is ignored there)."""
     n_tok = input_ids.shape[1] if input_ids is not None else input_embeds.shape[1]
     freqs = pick_freqs(w["freqs_cis"], n_tok, position_ids, cache_position)
@@ -414,7 +464,7 @@ def forward(w, s: RavenShape, input_ids=None, input_embeds=None, input_states=No
         block_idx += 1
         input_embeds = sandwich_block(input_embeds, w, f"transformer.prelude.{i}", freqs, block_idx, cache, s)
     x, block_idx = iterate_forward(input_embeds, input_states, w, freqs, block_idx, cache, num_steps, s,
-                                   init_scale, generator)
+                                   init_scale, generator, noise_draws)
     latents = x.clone()
     block_idx = 0
     for i in range(s.n_layers_in_coda):
@@ -476,10 +526,11 @@ def embed_inputs(w, s: RavenShape, input_ids, cache=None, cache_position=None, p
     return x, block_idx
 
 
-def iterate_one_step(w, s: RavenShape, embeds, states, block_idx: int, cache=None, cache_position=None, position_ids=None):
+def iterate_one_step(w, s: RavenShape, embeds, states, block_idx: int, cache=None, cache_position=None, position_ids=None,
+                     current_step: int = 0, noise_draws=None):
     """RMM:841-868: one recurrence; returns (state, block_idx)."""
     freqs = pick_freqs(w["freqs_cis"], embeds.shape[1], position_ids, cache_position)
-    return core_block_forward(states, embeds, w, freqs, cache, block_idx, s)
+    return core_block_forward(states, embeds, w, freqs, cache, block_idx, s, current_step, noise_draws)
 
 
 def predict_from_latents(w, s: RavenShape, latents, cache=None, cache_position=None, position_ids=None) -> OracleOutput:

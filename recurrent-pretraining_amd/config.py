@@ -35,10 +35,10 @@ class RavenConfig:
         test_time_noise_type: str = "fixed",
         **kwargs,
     ):
-        if test_time_noise:
-            # RMM:815-838 perturbs the latent state before every recurrence when this is set; the recurrence launches of
-            # this package have no such step
-            raise NotImplementedError("test_time_noise > 0 (noise injected before every recurrence) is not supported")
+        if test_time_noise_type not in ("geom", "sqrt", "line", "chi", "fixed"):  # RMM:818-833
+            raise ValueError(f"unknown test_time_noise_type {test_time_noise_type!r}")
+        if test_time_noise < 0:
+            raise ValueError("test_time_noise must not be negative")
         if bias:
             raise ValueError("bias=True is not supported: the reference model family has no Linear biases")
         self.n_embd = n_embd
@@ -59,7 +59,7 @@ class RavenConfig:
         self.qk_bias = qk_bias
         self.rope_base = rope_base
         self.torch_dtype = torch_dtype
-        self.test_time_noise = 0
+        self.test_time_noise = test_time_noise
         self.test_time_noise_type = test_time_noise_type
         self.extra = dict(kwargs)  # keys of the reference config that only matter for training
         # derived (raven_config_minimal.py:78-91)
@@ -99,5 +99,6 @@ class RavenConfig:
     def to_dict(self) -> dict:
         keys = ("n_embd", "n_heads", "n_layers", "block_size", "vocab_size", "padding_multiple", "tie_embeddings",
                 "intermediate_size", "bias", "norm_eps", "n_layers_in_recurrent_block", "mean_recurrence",
-                "mean_backprop_depth", "n_layers_in_prelude", "n_layers_in_coda", "qk_bias", "rope_base", "torch_dtype")
+                "mean_backprop_depth", "n_layers_in_prelude", "n_layers_in_coda", "qk_bias", "rope_base", "torch_dtype",
+                "test_time_noise", "test_time_noise_type")
         return {**self.extra, **{k: getattr(self, k) for k in keys}, "model_type": self.model_type}

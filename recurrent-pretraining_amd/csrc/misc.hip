@@ -90,6 +90,26 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ z, T*
     store_chunk(out + m * inter + c * E, o);
 }
 
+// Test-time noise (recpre/raven_modeling_minimal.py:815-833): y = T(T(x * keep) + n) with n = T(noise * a), divided once
+// more by d and rounded again when d != 0 -- the reference's elementwise torch expression, one rounding per operation.
+template <typename T>
+__global__ __launch_bounds__(256) void noise_mix_kernel(const T* __restrict__ x, const T* __restrict__ noise, T* __restrict__ y,
+                                                        int64_t chunks, float keep, float a, float d) {
+#pragma clang fp contract(off)  // float32 states: the product and the sum are two roundings, never one fused multiply-add
+    constexpr int E = Chunk<T>::N;
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= chunks) return;
+    const Chunk<T> xv = load_chunk(x + c * E), nv = load_chunk(noise + c * E);
+    Chunk<T> o;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        float n = round_to<T>(to_f32(nv.v[e]) * a);
+        if (d != 0.f) n = round_to<T>(n / d);
+        o.v[e] = from_f32<T>(round_to<T>(to_f32(xv.v[e]) * keep) + n);
+    }
+    store_chunk(y + c * E, o);
+}
+
 __global__ void advance_pos_kernel(int* pos, int delta) {
     if (threadIdx.x == 0 && blockIdx.x == 0) *pos += delta;
 }
@@ -138,6 +158,23 @@ extern "C" int raven_swiglu(const void* z, void* out, int32_t M, int32_t I, int3
     if (dtype == RAVEN_BF16) swiglu_kernel<bf16><<<grid, dim3(256), 0, s>>>((const bf16*)z, (bf16*)out, I);
     else swiglu_kernel<float><<<grid, dim3(256), 0, s>>>((const float*)z, (float*)out, I);
     return raven_host::check_launch("swiglu");
+}
+
+extern "C" int raven_noise_mix(const void* x, const void* noise, void* y, int64_t n, float keep, float a, float d, int32_t dtype,
+                               void* stream) {
+    using namespace raven;
+    RAVEN_REQUIRE(dtype == RAVEN_F32 || dtype == RAVEN_BF16, "noise_mix: unknown dtype %d", dtype);
+    RAVEN_REQUIRE(x && noise && y, "noise_mix: null pointer");
+    const int elts = 16 / (int)raven_host::elt_size(dtype);
+    RAVEN_REQUIRE(n >= 0 && n % elts == 0, "noise_mix: %lld elements are not a multiple of %d", (long long)n, elts);
+    if (n == 0) return 0;
+    const int64_t chunks = n / elts;
+    RAVEN_REQUIRE((chunks + 255) / 256 <= 0x7fffffff, "noise_mix: too many elements");
+    const dim3 grid((unsigned)((chunks + 255) / 256));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == RAVEN_BF16) noise_mix_kernel<bf16><<<grid, dim3(256), 0, s>>>((const bf16*)x, (const bf16*)noise, (bf16*)y, chunks, keep, a, d);
+    else noise_mix_kernel<float><<<grid, dim3(256), 0, s>>>((const float*)x, (const float*)noise, (float*)y, chunks, keep, a, d);
+    return raven_host::check_launch("noise_mix");
 }
 
 extern "C" int raven_advance_pos(int32_t* pos_dev, int32_t delta, void* stream) {

@@ -93,6 +93,7 @@ SIGNATURES = {
                                              _I32, _VP, _SZ, _VP]),
     "raven_prefill_attention": (C.c_int, [_VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _I32, _I32, _I32, _VP]),
     "raven_swiglu": (C.c_int, [_VP, _VP, _I32, _I32, _I32, _VP]),
+    "raven_noise_mix": (C.c_int, [_VP, _VP, _VP, _I64, _F, _F, _F, _I32, _VP]),
     "raven_embed": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I64, _F, _I32, _VP]),
     "raven_argmax": (C.c_int, [_VP, _VP, _I32, _I64, _VP]),
     "raven_advance_pos": (C.c_int, [_VP, _I32, _VP]),
@@ -390,6 +391,17 @@ def swiglu(z):
     out = torch.empty(M, two_i // 2, device=z.device, dtype=z.dtype)
     _check(load().raven_swiglu(_ptr(z, "z"), _ptr(out, "out"), M, two_i // 2, dtype_code(z.dtype), _stream()), "raven_swiglu")
     return out
+
+
+def noise_mix(x, noise, keep: float, a: float, d: float = 0.0):
+    """T(T(x * keep) + T(noise * a) [/ d, rounded again]) elementwise; x and noise of one shape and dtype."""
+    if noise.shape != x.shape:
+        raise RavenHipError(f"noise_mix: noise {tuple(noise.shape)} against x {tuple(x.shape)}")
+    y = torch.empty_like(x)
+    rc = load().raven_noise_mix(_ptr(x, "x"), _ptr(noise, "noise", x.dtype), _ptr(y, "y"), x.numel(), float(keep), float(a), float(d),
+                                dtype_code(x.dtype), _stream())
+    _check(rc, "raven_noise_mix")
+    return y
 
 
 def embed(wte, ids, scale, out=None):

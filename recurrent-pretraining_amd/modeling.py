@@ -15,6 +15,7 @@ What differs from the reference on purpose:
 
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass
 from typing import Any, Callable, Optional, Union
 
@@ -152,6 +153,7 @@ class RavenForCausalLM(torch.nn.Module):
             self.register_buffer("freqs_cis", table.to(device), persistent=True)
         self.to(dtype)  # casts the RoPE table too, as nn.Module.to does for the reference (RMM:577)
         self.generation_config = GenerationSettings()
+        self.noise_source = None  # test-time noise draws: an object with normal(x) and uniform(x); None = torch's generator
         self._native_key = None
         self._native: dict = {}
         self._scratch: dict = {}
@@ -418,10 +420,45 @@ class RavenForCausalLM(torch.nn.Module):
                            self._workspace(B * S), ln_f=self.transformer.ln_f.weight if ln_f else None)
         return out
 
+    def _maybe_inject_noise(self, x: torch.Tensor, current_step: int, renorm: bool = True) -> torch.Tensor:
+        """RMM:815-837: with test_time_noise set, the state is mixed with fresh Gaussian noise in front of every
+        recurrence and passed through the last core block's norm_4 again.  The draws come from self.noise_source
+        (`normal(x)`, `uniform(x)`) when that is set, otherwise from torch's generator of the device."""
+        cfg = self.config
+        if cfg.test_time_noise <= 0:
+            return x
+        n = cfg.test_time_noise * cfg.init_values["std"] * self.emb_scale
+        src = self.noise_source
+        kind = cfg.test_time_noise_type
+        # The reference's expression mixes Python floats (taken as float32 operands by the elementwise kernels) with 0-dim
+        # device tensors (converted to the state's dtype first, as ATen's GPU kernels do); every product, quotient and
+        # sum is rounded to the state's dtype.
+        f32 = lambda v: float(torch.tensor(v, dtype=torch.float32))
+        as_state = lambda v: float(torch.tensor(v, dtype=torch.float32).to(x.dtype))
+        d = 0.0
+        if kind in ("geom", "sqrt"):  # n / (step + 1) or n / sqrt(step + 1): float32 0-dim tensors (RMM:819-823)
+            d32 = f32(current_step + 1) if kind == "geom" else f32(math.sqrt(current_step + 1))
+            keep, a, d = as_state(1.0 - f32(f32(n) / d32)), n, as_state(d32)
+        elif kind == "line":          # RMM:825-826, a Python float
+            c = max(n, (cfg.mean_recurrence - current_step) / cfg.mean_recurrence)
+            keep, a = 1.0 - c, c
+        elif kind == "chi":           # RMM:828-829: 2 * rand(1) * n, a tensor of the state's dtype
+            u = src.uniform(x) if src is not None else torch.rand(1, device=x.device, dtype=x.dtype)
+            c = as_state(as_state(2.0 * float(u)) * f32(n))
+            keep, a = as_state(1.0 - c), c
+        else:                         # "fixed", RMM:831
+            keep, a = 1.0 - n, n
+        noise = src.normal(x).to(device=x.device, dtype=x.dtype) if src is not None else torch.randn_like(x)
+        x = hip.noise_mix(x, noise.reshape(x.shape).contiguous(), keep, a, d)
+        if renorm:
+            x = hip.rmsnorm_residual(x, self.transformer.core_block[-1].norm_4.weight, cfg.norm_eps)[0]
+        return x
+
     def _run_core(self, x: torch.Tensor, embeds: torch.Tensor, first_step: int, cache: HuginnDynamicCache, private: bool,
-                  B: int, S: int, pos0: int, ln_f: bool) -> torch.Tensor:
+                  B: int, S: int, pos0: int, ln_f: bool, current_step: int = 0) -> torch.Tensor:
         """One core_block_forward (RMM:764-781) on [B*S, h] rows."""
         nat, t = self._natives(), self.transformer
+        x = self._maybe_inject_noise(x, current_step)
         n_core = len(t.core_block)
         slots = [0 if private else cache.note_append(first_step + j, S, pos0) for j in range(n_core)]
         # positions of earlier tokens that were computed with fewer recurrences are not cached at these steps:
@@ -556,7 +593,7 @@ class RavenForCausalLM(torch.nn.Module):
         n_core = len(self.transformer.core_block)
         x = state
         for it in range(r):
-            x = self._run_core(x, embeds, block_idx + 1 + it * n_core, cache, private, B, S, pos0, ln_f=(it == r - 1))
+            x = self._run_core(x, embeds, block_idx + 1 + it * n_core, cache, private, B, S, pos0, ln_f=(it == r - 1), current_step=it)
         if r == 0:
             x = hip.rmsnorm_residual(x, self.transformer.ln_f.weight, self.config.norm_eps)[0]
         return x
@@ -601,7 +638,7 @@ class RavenForCausalLM(torch.nn.Module):
         cache, private, pos0 = self._cache_for_piece(past_key_values, B, S, b0 + 1 + n_core)
         out = self._run_core(x.to(self.dtype).reshape(B * S, h).contiguous(),
                              input_embeds.to(self.dtype).reshape(B * S, h).contiguous(), b0 + 1, cache, private, B, S, pos0,
-                             ln_f=False)
+                             ln_f=False, current_step=_as_int(current_step))
         return out.view(B, S, h), torch.tensor(b0 + n_core, dtype=torch.long)
 
     @torch.no_grad()
@@ -870,7 +907,7 @@ class DecodeRunner:
         self.logits = torch.empty(batch, cfg.padded_vocab_size, dtype=torch.float32, device=dev)
         self.next_ids = torch.zeros(batch, dtype=torch.int64, device=dev)
         self.ws = hip.block_workspace(model._natives()["dims"], batch, dev)
-        self.use_graph = use_graph
+        self.use_graph = use_graph and cfg.test_time_noise <= 0  # the noise draws are not part of a replayable launch sequence
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self._graph_t_max = None
         self._warm = False
@@ -899,7 +936,7 @@ class DecodeRunner:
         embeds = x
         x = self.state
         for it in range(self.r):
-            x = m._wide_core(x, embeds, core[it], kv, B, 1, hint, ln_f=(it == self.r - 1), pos_dev=self.pos)
+            x = m._wide_core(m._maybe_inject_noise(x, it), embeds, core[it], kv, B, 1, hint, ln_f=(it == self.r - 1), pos_dev=self.pos)
         self.latents.copy_(x)
         n_coda = len(coda)
         for i, slot in enumerate(coda):
@@ -928,7 +965,14 @@ class DecodeRunner:
                                pos_dev=self.pos)
         x = self.state
         n_core = len(t.core_block)
-        if n_core > 0 and self.r > 0:
+        if n_core > 0 and self.r > 0 and cfg.test_time_noise > 0:
+            # the state is perturbed in front of every recurrence (RMM:775): one call per recurrence
+            for it in range(self.r):
+                x = m._maybe_inject_noise(x, it)
+                hip.core_iterations(nat["dims"], t.adapter.weight, nat["core"], x, self.embeds, self.x, nat["freqs"], kv, [core[it]], B, 1,
+                                    hint, self.ws, ln_f=t.ln_f.weight if it == self.r - 1 else None, pos_dev=self.pos)
+                x = self.x
+        elif n_core > 0 and self.r > 0:
             # all recurrences in one call: for one row the library folds each closing norm into the next adapter product
             hip.core_iterations(nat["dims"], t.adapter.weight, nat["core"], x, self.embeds, self.x, nat["freqs"], kv, core, B, 1, hint,
                                 self.ws, ln_f=t.ln_f.weight, pos_dev=self.pos)

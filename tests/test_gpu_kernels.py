@@ -420,6 +420,35 @@ def test_swiglu_elementwise(pkg):
             assert bool((got.cpu() == F.silu(z[:, :I]) * z[:, I:]).float().mean() > 0.99)
 
 
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+def test_noise_mix_rounds_like_the_elementwise_expression_on_the_device(pkg, dt):
+    """raven_noise_mix against the five forms of the state perturbation (recpre/raven_modeling_minimal.py:818-831)
+    evaluated by torch on the GPU, where a 0-dim device tensor operand is converted to the result dtype first and a
+    Python float is a float32 operand: bit-exact."""
+    x, noise = rnd((3, 5280), dt, 160).cuda(), rnd((3, 5280), dt, 161).cuda()
+    n = 0.3 * math.sqrt(0.4)
+    f32 = lambda v: float(torch.tensor(v, dtype=torch.float32))
+    st = lambda v: float(torch.tensor(v, dtype=torch.float32).to(dt))
+    for step in (0, 2, 6):
+        step1 = torch.as_tensor(step + 1, device="cuda")
+        want = x * (1 - n / step1) + noise * n / step1
+        got = pkg.hip.noise_mix(x, noise, st(1.0 - f32(f32(n) / (step + 1))), n, float(step + 1))
+        assert torch.equal(got, want), f"geom, step {step}"
+        root = step1.sqrt()
+        want = x * (1 - n / root) + noise * n / root
+        d32 = f32(math.sqrt(step + 1))
+        got = pkg.hip.noise_mix(x, noise, st(1.0 - f32(f32(n) / d32)), n, st(d32))
+        assert torch.equal(got, want), f"sqrt, step {step}"
+        c = max(n, (8 - step) / 8)
+        assert torch.equal(pkg.hip.noise_mix(x, noise, 1.0 - c, c), x * (1 - c) + noise * c), f"line, step {step}"
+    assert torch.equal(pkg.hip.noise_mix(x, noise, 1.0 - n, n), x * (1 - n) + noise * n), "fixed"
+    u = torch.tensor([0.3671875], device="cuda", dtype=dt)
+    amp = 2 * u * n
+    want = x * (1 - amp) + noise * amp
+    c = st(st(2.0 * float(u)) * f32(n))
+    assert torch.equal(pkg.hip.noise_mix(x, noise, st(1.0 - c), c), want), "chi"
+
+
 def test_decode_attention_at_the_maximum_context(pkg):
     """block_size = 4096 positions (recpre/raven_config_minimal.py:17): the last decode step of a full context."""
     dt, nh, hd, t_max = torch.bfloat16, 55, 96, 4096

@@ -247,6 +247,61 @@ def test_decode_runner_beyond_one_pass_of_rows_bf16(pkg, tiny16, use_graph):
     assert (runner.graph is not None) == use_graph
 
 
+class SharedDraws:
+    """The random numbers of the test-time noise, drawn on the CPU from one seeded generator: the oracle and the model
+    consume them in the same order (per recurrence: the amplitude for "chi", then the noise)."""
+
+    def __init__(self, seed):
+        self.g = torch.Generator().manual_seed(seed)
+
+    def normal(self, x):
+        return torch.randn(tuple(x.shape), generator=self.g).to(x.dtype)
+
+    def uniform(self, x):
+        return torch.rand(1, generator=self.g).to(x.dtype)
+
+
+@pytest.mark.parametrize("kind", ["geom", "sqrt", "line", "chi", "fixed"])
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_forward_and_decode_with_test_time_noise(pkg, kind, dt):
+    """test_time_noise > 0 (RMM:815-837): the state is mixed with noise and renormalised in front of every recurrence.
+    Prefill through forward(), two decode tokens through the preallocated runner (one launch sequence per recurrence
+    then), all against the oracle fed with the same draws."""
+    import dataclasses
+    s = dataclasses.replace(O.RavenShape.tiny(), test_time_noise=0.4, test_time_noise_type=kind)
+    w = O.make_weights(s, seed=3, dtype=dt)
+    if dt == torch.bfloat16:
+        w["freqs_cis"] = w["freqs_cis"].to(dt)
+    cfg = pkg.RavenConfig.tiny()
+    cfg.test_time_noise, cfg.test_time_noise_type = 0.4, kind
+    model = build_model(pkg, cfg, w, dt)
+    B, S = 2, 5
+    g = torch.Generator().manual_seed(21)
+    ids = torch.randint(0, s.vocab_size, (B, S + 2), generator=g)
+    states = O.initialize_state(torch.empty(B, S + 2, s.n_embd), s, 1.0, g).to(dt)
+    ref_draws, model.noise_source = SharedDraws(77), SharedDraws(77)
+    ref_cache, cache = O.DictCache(), pkg.HuginnDynamicCache()
+    want = O.forward(w, s, input_ids=ids[:, :S], input_states=states[:, :S], past_key_values=ref_cache, use_cache=True,
+                     noise_draws=ref_draws)
+    got = model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda(), past_key_values=cache, use_cache=True)
+    check(got.latent_states, want.latent_states, dt, f"{kind} latents")
+    check(got.logits, want.logits, dt, f"{kind} logits")
+    runner = pkg.DecodeRunner(model, cache, B, s.mean_recurrence, use_graph=True)
+    assert not runner.use_graph
+    for i in range(2):
+        pos = torch.arange(S + i, S + i + 1)
+        tok, st = ids[:, S + i:S + i + 1], states[:, S + i:S + i + 1]
+        want = O.forward(w, s, input_ids=tok, input_states=st, past_key_values=ref_cache, use_cache=True, cache_position=pos,
+                         noise_draws=ref_draws)
+        logits, _, lat = runner.step(tok.cuda(), st.cuda())
+        check(logits, want.logits[:, 0], dt, f"{kind} runner logits, token {i}")
+        check(lat, want.latent_states[:, 0], dt, f"{kind} runner latents, token {i}")
+    # without the noise the same model gives something else: the option is not silently ignored
+    model.config.test_time_noise = 0.0
+    plain = model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda())
+    assert close(plain.logits, got.logits)[1] > 1e-2
+
+
 @pytest.fixture(scope="module")
 def small242(pkg):
     """2 prelude / 4 core / 2 coda blocks like the 3.5b model (the cache's lookup strategies hard-code that structure)."""

@@ -382,5 +382,7 @@ def test_repetition_penalties_against_the_reference_loops(pkg):
     b0 = int(logits[0].argmax())
     x = float(logits[0, b0])
     assert abs(float(got[0, 0, b0]) - (x * 1.3 if x < 0 else x / 1.3)) < 1e-6
-    with pytest.raises(NotImplementedError):
-        pkg.RavenConfig(test_time_noise=0.1)
+    cfg = pkg.RavenConfig(test_time_noise=0.1, test_time_noise_type="geom")
+    assert cfg.to_dict()["test_time_noise"] == 0.1 and cfg.to_dict()["test_time_noise_type"] == "geom"
+    with pytest.raises(ValueError):
+        pkg.RavenConfig(test_time_noise=0.1, test_time_noise_type="pink")

@@ -677,3 +677,74 @@ def test_diffusion_sampler_never_freezing_and_standing_waves():
                                       state_fn=sf, record=rec2)
     assert out2.shape == (1, n + 4) and int(out2[0, n]) == int(out[0, n])
     assert all(e["frozen"] >= b["frozen"] for b, e in zip(rec2["log"], rec2["log"][1:]))
+
+
+# ----------------------------------------------------------------------------- test-time noise
+class _Draws:
+    """Deterministic stand-ins for randn_like / rand(1)."""
+
+    def __init__(self, normal=None, uniform=0.25, seed=None):
+        self._n, self._u = normal, uniform
+        self._g = None if seed is None else torch.Generator().manual_seed(seed)
+
+    def normal(self, x):
+        if self._g is not None:
+            return torch.randn(x.shape, generator=self._g).to(x.dtype)
+        return torch.full_like(x, self._n)
+
+    def uniform(self, x):
+        return torch.tensor([self._u], dtype=x.dtype)
+
+
+def _noisy(kind, t=0.3):
+    import dataclasses
+    s = dataclasses.replace(O.RavenShape.tiny(), test_time_noise=t, test_time_noise_type=kind)
+    return s, O.make_weights(s, seed=0, dtype=torch.float32)
+
+
+def test_noise_amplitude_and_per_type_coefficients_closed_form():
+    """x = 0, noise = 1, no renormalisation: the output is the coefficient c itself.  n = t * std * sqrt(h) with
+    std = sqrt(2/(5h)) is t * sqrt(2/5) whatever the width (RMM:817, raven_config_minimal.py:86)."""
+    t = 0.3
+    n = t * math.sqrt(0.4)
+    want = {("fixed", 0): n, ("fixed", 5): n, ("geom", 0): n, ("geom", 2): n / 3, ("sqrt", 0): n, ("sqrt", 3): n / 2,
+            ("line", 0): 1.0, ("line", 1): 0.75, ("line", 3): max(n, 0.25), ("chi", 0): 2 * 0.25 * n}
+    for (kind, k), c in want.items():
+        s, w = _noisy(kind, t)
+        x = torch.zeros(1, 2, s.n_embd)
+        y = O.inject_noise(x, k, w, s, _Draws(normal=1.0), renorm=False)
+        assert torch.allclose(y, torch.full_like(y, c), rtol=1e-6, atol=0), (kind, k)
+        # and the state keeps 1 - c: x = 1, noise = 0
+        y = O.inject_noise(torch.ones(1, 2, s.n_embd), k, w, s, _Draws(normal=0.0), renorm=False)
+        assert torch.allclose(y, torch.full_like(y, 1 - c), rtol=1e-6, atol=1e-7), (kind, k)
+
+
+def test_noise_off_is_identity_and_zero_noise_leaves_the_norm():
+    s, w = _noisy("fixed", 0.0)
+    x = torch.randn(2, 3, s.n_embd)
+    assert O.inject_noise(x, 1, w, s, _Draws(normal=1.0)) is x
+    # RMSNorm does not see a scale: x * (1 - n) + 0 renormalises to norm_4(x)
+    s, w = _noisy("fixed", 0.3)
+    got = O.inject_noise(x, 1, w, s, _Draws(normal=0.0))
+    want = O.rmsnorm(x, w[f"transformer.core_block.{s.n_layers_in_recurrent_block - 1}.norm_4.weight"], s.norm_eps)
+    assert torch.allclose(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_line_noise_replaces_the_state_at_step_zero_inside_forward():
+    """With "line" the first recurrence sees pure noise (c = 1 at step 0): the forward pass no longer depends on
+    input_states, which also fixes WHERE the injection sits (in front of the adapter) and that steps count from 0."""
+    s, w = _noisy("line", 0.3)
+    g = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, s.vocab_size, (1, 6), generator=g)
+    a = torch.randn(1, 6, s.n_embd, generator=g)
+    b = torch.randn(1, 6, s.n_embd, generator=g)
+    out_a = O.forward(w, s, input_ids=ids, input_states=a, noise_draws=_Draws(seed=9))
+    out_b = O.forward(w, s, input_ids=ids, input_states=b, noise_draws=_Draws(seed=9))
+    assert torch.equal(out_a.logits, out_b.logits)
+    other = O.forward(w, s, input_ids=ids, input_states=a, noise_draws=_Draws(seed=10))
+    assert not torch.equal(out_a.logits, other.logits)
+    # "fixed" keeps 1 - n of the state: there the two do differ
+    s2, _ = _noisy("fixed", 0.3)
+    out_c = O.forward(w, s2, input_ids=ids, input_states=a, noise_draws=_Draws(seed=9))
+    out_d = O.forward(w, s2, input_ids=ids, input_states=b, noise_draws=_Draws(seed=9))
+    assert not torch.equal(out_c.logits, out_d.logits)
