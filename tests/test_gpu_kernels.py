@@ -390,13 +390,19 @@ def test_qkv_attention_decode_fused(pkg, dt, nh, hd, B, pos0):
     assert torch.equal(kd, kd2) and torch.equal(vd, vd2)
 
 
-@pytest.mark.parametrize("nh,hd,B,S,pos0", [(55, 96, 1, 512, 0), (55, 96, 2, 100, 37), (4, 64, 3, 64, 0), (3, 128, 1, 65, 200),
-                                             (55, 96, 1, 2, 5), (5, 96, 1, 300, 724)])
-def test_prefill_attention_mfma(pkg, nh, hd, B, S, pos0):
+@pytest.mark.parametrize("nh,hd,B,S,pos0,t_max,qscale", [
+    (55, 96, 1, 512, 0, 1024, 1), (55, 96, 2, 100, 37, 1024, 1), (4, 64, 3, 64, 0, 1024, 1), (3, 128, 1, 65, 200, 1024, 1),
+    (55, 96, 1, 2, 5, 1024, 1), (5, 96, 1, 300, 724, 1024, 1),
+    # 128 query rows per workgroup (launches of 512 workgroups and more): ragged last block, a cache that ends inside the
+    # last key tile, all three head sizes, and scores spread widely enough that the reference maximum moves (and O is
+    # rescaled) in many tiles
+    (55, 96, 2, 650, 300, 1024, 1), (16, 64, 4, 1000, 24, 1024, 1), (16, 128, 4, 900, 77, 1000, 1), (55, 96, 2, 640, 0, 640, 8),
+    (55, 96, 1, 512, 0, 1024, 8)])
+def test_prefill_attention_mfma(pkg, nh, hd, B, S, pos0, t_max, qscale):
     """The matrix-core chunk kernel against the oracle and against the per-row kernel."""
-    dt, t_max = torch.bfloat16, 1024
+    dt = torch.bfloat16
     k, v, kd, vd, cache = make_cache(pkg, 2, B, nh, t_max, hd, dt, fill_seed=130)
-    q = rnd((B * S, nh * hd), dt, 132)
+    q = (rnd((B * S, nh * hd), dt, 132) * qscale).to(dt)
     y = pkg.hip.prefill_attention(q.cuda(), cache, 1, B, S, pos0, nh, hd)
     T = pos0 + S
     qq = q.view(B, S, nh, hd).transpose(1, 2)
