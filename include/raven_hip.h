@@ -165,7 +165,17 @@ int raven_exit_latent_stats(const void* latents, const void* prev, void* rel_cha
  *   (vllm/raven_vllm.py:186-201: split, q/k bias, RoPE, cache write, attention): qkv [B, 3 * n_heads * head_dim] is the
  *   fused projection's output, qk_bias [2, n_heads, head_dim] or NULL, freqs the (cos, sin) table; sequence b's new
  *   token sits at position seq_lens[b] - 1: its rotated k and its v are written to that position's page and the row
- *   attends to positions 0..seq_lens[b] - 1 (seq_lens[b] = 0: nothing written, zeros returned). */
+ *   attends to positions 0..seq_lens[b] - 1 (seq_lens[b] = 0: nothing written, zeros returned).
+ * raven_paged_qkv_rope_append: the same layer up to the cache write for ANY rows (prompt chunks and decode rows of
+ *   several sequences in one launch, vllm/raven_vllm.py:186-199): row t of qkv [T, 3 * n_heads * head_dim] gets the q/k
+ *   bias and the rotation of positions[t] (a row of freqs; the caller keeps it inside the table), q goes to
+ *   q_out [T, n_heads * head_dim], k and v to slot slot_mapping[t] of the pages (negative: not stored).
+ * raven_paged_prefill_attention: causal attention of such rows on the matrix cores (bf16, head_dim 64 / 96 / 128), the
+ *   variable-length form vLLM's backends call: sequence b owns rows q_start[b] .. q_start[b + 1] - 1 of q / y
+ *   [T, n_heads * head_dim]; they are the LAST positions of its seq_lens[b] cached positions (already appended), so row
+ *   r of the sequence attends to positions 0 .. seq_lens[b] - (rows of b) + r.  max_q_len >= every sequence's row count
+ *   sizes the launch; a sequence with no rows, or more rows than positions, is left alone.  Same kernel as
+ *   raven_prefill_attention with the key tiles gathered through the block table. */
 enum { RAVEN_PAGED_NHD = 0, RAVEN_PAGED_HND = 1 };
 int raven_paged_kv_append(const void* k, const void* v, void* k_cache, void* v_cache, const int64_t* slot_mapping,
                           int32_t T, int32_t n_heads, int32_t head_dim, int32_t block_size, int32_t kv_layout,
@@ -179,6 +189,15 @@ int raven_paged_qkv_attention_decode(const void* qkv, const void* qk_bias, const
                                      int32_t max_blocks, int32_t block_size, int32_t kv_layout, int32_t max_seq_len,
                                      int32_t n_heads, int32_t head_dim, int32_t dtype, void* workspace,
                                      size_t workspace_bytes, void* stream);
+
+int raven_paged_qkv_rope_append(const void* qkv, const void* qk_bias, const float* freqs, const int64_t* positions,
+                                const int64_t* slot_mapping, void* q_out, void* k_cache, void* v_cache, int32_t T,
+                                int32_t n_heads, int32_t head_dim, int32_t block_size, int32_t kv_layout,
+                                int32_t dtype, void* stream);
+int raven_paged_prefill_attention(const void* q, void* y, const void* k_cache, const void* v_cache,
+                                  const int32_t* block_table, const int32_t* seq_lens, const int32_t* q_start,
+                                  int32_t B, int32_t max_q_len, int32_t max_blocks, int32_t block_size,
+                                  int32_t kv_layout, int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream);
 
 /* A stack of SandwichBlocks over block-paged caches, one decode row per sequence (the flat layer list the plugin's
  * model runs, vllm/raven_vllm.py:365-432: every flat layer owns ONE paged cache, which the recurrences of a token

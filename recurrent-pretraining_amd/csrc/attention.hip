@@ -538,6 +538,31 @@ __global__ __launch_bounds__(256) void paged_kv_append_kernel(const T* __restric
     store_chunk(vc + dst, load_chunk(v + (int64_t)t * h + c * E));
 }
 
+// Rows of a fused projection [T, 3 * h] on their way into block-paged caches: q and k get the bias and the rotation of
+// their own position (positions[t], any order -- rows of several sequences in one launch), q goes to q_out [T, h], k and
+// v to slot slots[t] of the pages (negative slot: not stored).  blockIdx.z = 0 / 1 / 2 for q / k / v.
+template <typename T>
+__global__ __launch_bounds__(256) void paged_qkv_rope_append_kernel(const T* __restrict__ qkv, const T* __restrict__ qk_bias,
+                                                                    const float* __restrict__ freqs, const int64_t* __restrict__ positions,
+                                                                    const int64_t* __restrict__ slots, T* __restrict__ q_out,
+                                                                    T* __restrict__ kc, T* __restrict__ vc, int h, int hd, int block_size,
+                                                                    int64_t pos_stride, int64_t head_stride) {
+    constexpr int E = Chunk<T>::N;
+    const int t = blockIdx.y, sec = blockIdx.z, c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= h / E) return;
+    const int col = c * E, head = col / hd, d = col - head * hd;
+    Chunk<T> x = load_chunk(qkv + (int64_t)t * 3 * h + (int64_t)sec * h + col);
+    if (sec < 2) x = bias_rope_chunk<T>(x, qk_bias, sec, h, col, freqs, (int)positions[t], hd, d);
+    if (sec == 0) {
+        store_chunk(q_out + (int64_t)t * h + col, x);
+        return;
+    }
+    const int64_t slot = slots[t];
+    if (slot < 0) return;
+    const int64_t blk = slot / block_size, off = slot - blk * block_size;
+    store_chunk((sec == 1 ? kc : vc) + blk * block_size * h + off * pos_stride + head * head_stride + d, x);
+}
+
 constexpr int kAttnMaxSplits = 32;
 int g_rope_tiled_rows = 16;       // chunk length from which the append kernel works on (head, 16 positions) tiles ("rope_tiled_rows")
 int g_attn_nosplit_pairs = 1024;  // (head, row) pairs from which a launch is never split ("attn_nosplit_pairs", at most 1024)
@@ -801,6 +826,29 @@ extern "C" int raven_paged_kv_append(const void* k, const void* v, void* k_cache
     if (dtype == RAVEN_BF16) paged_kv_append_kernel<bf16><<<grid, dim3(256), 0, s>>>((const bf16*)k, (const bf16*)v, (bf16*)k_cache, (bf16*)v_cache, slot_mapping, h, head_dim, block_size, ps, hs);
     else paged_kv_append_kernel<float><<<grid, dim3(256), 0, s>>>((const float*)k, (const float*)v, (float*)k_cache, (float*)v_cache, slot_mapping, h, head_dim, block_size, ps, hs);
     return raven_host::check_launch("paged_kv_append");
+}
+
+extern "C" int raven_paged_qkv_rope_append(const void* qkv, const void* qk_bias, const float* freqs, const int64_t* positions,
+                                           const int64_t* slot_mapping, void* q_out, void* k_cache, void* v_cache, int32_t T,
+                                           int32_t n_heads, int32_t head_dim, int32_t block_size, int32_t kv_layout, int32_t dtype,
+                                           void* stream) {
+    using namespace raven;
+    if (int rc = check_heads("paged_qkv_rope_append", n_heads, head_dim, dtype)) return rc;
+    int64_t ps, hs;
+    if (int rc = paged_strides("paged_qkv_rope_append", kv_layout, block_size, n_heads, head_dim, &ps, &hs)) return rc;
+    RAVEN_REQUIRE(T >= 0 && T <= 65535, "paged_qkv_rope_append: bad row count %d", T);
+    if (T == 0) return 0;
+    RAVEN_REQUIRE(qkv && freqs && positions && slot_mapping && q_out && k_cache && v_cache, "paged_qkv_rope_append: null pointer");
+    const int h = n_heads * head_dim, elts = 16 / (int)raven_host::elt_size(dtype);
+    const dim3 grid((h / elts + 255) / 256, T, 3);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == RAVEN_BF16)
+        paged_qkv_rope_append_kernel<bf16><<<grid, dim3(256), 0, s>>>((const bf16*)qkv, (const bf16*)qk_bias, freqs, positions, slot_mapping,
+                                                                      (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, h, head_dim, block_size, ps, hs);
+    else
+        paged_qkv_rope_append_kernel<float><<<grid, dim3(256), 0, s>>>((const float*)qkv, (const float*)qk_bias, freqs, positions, slot_mapping,
+                                                                       (float*)q_out, (float*)k_cache, (float*)v_cache, h, head_dim, block_size, ps, hs);
+    return raven_host::check_launch("paged_qkv_rope_append");
 }
 
 static int paged_attention_common(const char* who, bool fused, const void* q, const void* bias, const float* freqs, void* y,

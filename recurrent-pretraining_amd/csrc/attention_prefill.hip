@@ -42,7 +42,16 @@ struct PrefillArgs {
     int nh, hd, t_max, S, pos0;
     const int* pos_dev;
     float scale_log2;
+    // block-paged caches (the PAGED kernels): sequence b's query rows are q_start[b] .. q_start[b + 1] - 1 of q, they are
+    // the LAST positions of its seq_lens[b] cached positions, and position p lives in page block_table[b][p / block_size]
+    const int* block_table;  // [B, max_blocks]
+    const int* seq_lens;     // [B]
+    const int* q_start;      // [B + 1]
+    int max_blocks, block_size, block_shift;  // block_shift = log2(block_size), or -1 when that is not a power of two
+    int64_t page_stride, pos_stride, head_stride;  // elements between two pages / positions of a page / heads
 };
+
+constexpr int kPfTable = 1024;  // block-table entries of a sequence held in LDS (beyond that they are read from memory)
 
 // Maximum over the four lanes l, l^16, l^32, l^48 (the lanes that share a query), in every lane, with the two row-swap
 // instructions of gfx950 instead of two round trips through the LDS crossbar: after v_permlane16_swap of a register
@@ -56,7 +65,7 @@ __device__ __forceinline__ float max_over_quarters(float x) {
     return fmaxf(__builtin_bit_cast(float, q[0]), __builtin_bit_cast(float, q[1]));
 }
 
-template <int HD, int RG>
+template <int HD, int RG, bool PAGED = false>
 __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a) {
     constexpr int KS = HD / 32;      // k-steps of the score MFMA
     constexpr int NT = HD / 16;      // 16-wide output tiles of O; tile NT holds the row sums
@@ -71,10 +80,28 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int qc = lane & 15, s4 = lane >> 4;
     const int h = a.nh * HD;
-    const int pos0 = a.pos_dev ? *a.pos_dev : a.pos0;
+    __shared__ int tbl[PAGED ? kPfTable : 1];
+    // rows of this sequence in q / y, their number, the number of cached positions that may be read, and the position
+    // of the first row
+    int64_t q_row0;
+    int n_rows, t_lim, pos0;
+    const int* table_row = nullptr;
+    if constexpr (PAGED) {
+        q_row0 = a.q_start[b];
+        n_rows = a.q_start[b + 1] - (int)q_row0;
+        t_lim = a.seq_lens[b];
+        pos0 = t_lim - n_rows;
+        table_row = a.block_table + (int64_t)b * a.max_blocks;
+        if (n_rows <= 0 || pos0 < 0 || qb * (64 * RG) >= n_rows) return;  // the grid is sized for the longest sequence
+    } else {
+        q_row0 = (int64_t)b * a.S;
+        n_rows = a.S;
+        t_lim = a.t_max;
+        pos0 = a.pos_dev ? *a.pos_dev : a.pos0;
+    }
 
     const int row0 = qb * ROWS + wave * WR;            // first query row (within the sequence) of this wave
-    const int64_t head_off = a.slot_off + ((int64_t)b * a.nh + head) * a.t_max * HD;
+    const int64_t head_off = PAGED ? (int64_t)head * a.head_stride : a.slot_off + ((int64_t)b * a.nh + head) * a.t_max * HD;
     const bf16* Kb = a.k + head_off;
     const bf16* Vb = a.v + head_off;
 
@@ -87,7 +114,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
     for (int g = 0; g < RG; ++g) {
         const int my_row = row0 + 16 * g + qc;
         my_limit[g] = pos0 + my_row;
-        const bf16* qp = a.q + ((int64_t)b * a.S + min(my_row, a.S - 1)) * h + head * HD + 8 * s4;
+        const bf16* qp = a.q + (q_row0 + min(my_row, n_rows - 1)) * h + head * HD + 8 * s4;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qf[g][ks] = *reinterpret_cast<const bf16x8*>(qp + 32 * ks);
     }
@@ -105,8 +132,8 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
     for (int e = 0; e < 8; ++e) ones[e] = static_cast<bf16>(1.0f);
 
     // keys this workgroup needs: everything up to the last row's own position
-    const int last_row = min(qb * ROWS + ROWS, a.S) - 1;
-    const int n_keys = min(pos0 + last_row + 1, a.t_max);
+    const int last_row = min(qb * ROWS + ROWS, n_rows) - 1;
+    const int n_keys = min(pos0 + last_row + 1, t_lim);
     const int wave_last = pos0 + row0 + WR - 1;  // the last key that any row of this wave sees
 
     // Global -> registers -> LDS, two tiles ahead of the multiply and two LDS buffers: the loads of tile i + 2 are in
@@ -134,8 +161,25 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
     // piece r = 4*(t&1) + s4 (keys 16*(t&1) + 4*s4 ..+3) sits at 8*s4 + 4*(t&1), so a lane's 8 keys of a k-step are
     // one 16-byte read.
     const int v_dst = (v_dc * 8) * kVtPitch + 32 * (v_kg / 8) + 8 * (v_kg % 4) + 4 * ((v_kg % 8) / 4);
+    // paged: element offset of position p's head row.  Positions past the last key this workgroup needs repeat that key
+    // (they are masked): only the pages up to it are in `tbl`, and only those are known to exist.
+    auto paged_off = [&](int p) {
+        p = min(p, n_keys - 1);
+        const int pg = a.block_shift >= 0 ? p >> a.block_shift : p / a.block_size;
+        const int page = pg < kPfTable ? tbl[pg] : table_row[pg];
+        return (int64_t)page * a.page_stride + (int64_t)(p - pg * a.block_size) * a.pos_stride;
+    };
     auto fetch = [&](int kt) {
-        if (kt + kPfKeys <= a.t_max) {
+        if constexpr (PAGED) {
+#pragma unroll
+            for (int i = 0; i < KCH; ++i) {
+                const int c = threadIdx.x + 256 * i;
+                const int key = c / CPR, dc = c - key * CPR;
+                kreg[i] = *reinterpret_cast<const u32x4*>(Kb + paged_off(kt + key) + dc * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) vreg[i] = *reinterpret_cast<const u32x4*>(Vb + paged_off(kt + 4 * v_kg + i) + v_dc * 8);
+        } else if (kt + kPfKeys <= a.t_max) {
 #pragma unroll
             for (int i = 0; i < KCH; ++i) kreg[i] = *reinterpret_cast<const u32x4*>(k_src + (int64_t)kt * HD + 2048 * i);
 #pragma unroll
@@ -276,6 +320,11 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
         __builtin_amdgcn_s_setprio(0);
     };
 
+    if constexpr (PAGED) {
+        const int n_pages = min((n_keys + a.block_size - 1) / a.block_size, kPfTable);
+        for (int i = threadIdx.x; i < n_pages; i += 256) tbl[i] = table_row[i];
+        __syncthreads();
+    }
     if (n_keys > 0) {
         fetch(0);
         park(0);
@@ -327,8 +376,8 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
             const int c = lane + 64 * i;
             const int r = c / CPR, dc = c - r * CPR;
             const int row = row0 + 16 * g0 + r;
-            if (row < a.S)
-                *reinterpret_cast<u32x4*>(a.y + ((int64_t)b * a.S + row) * h + head * HD + dc * 8) = *reinterpret_cast<const u32x4*>(ot + r * KP + dc * 8);
+            if (row < n_rows)
+                *reinterpret_cast<u32x4*>(a.y + (q_row0 + row) * h + head * HD + dc * 8) = *reinterpret_cast<const u32x4*>(ot + r * KP + dc * 8);
         }
     }
 }
@@ -350,7 +399,7 @@ extern "C" int raven_prefill_attention(const void* q, void* y, const raven_kv_ca
     RAVEN_REQUIRE(sl >= 0 && sl < cache->n_slots, "prefill_attention: slot %d outside [0, %d)", slot, cache->n_slots);
     RAVEN_REQUIRE(pos0 + S <= cache->t_max, "prefill_attention: positions up to %d exceed the cache length %d", pos0 + S - 1, cache->t_max);
     RAVEN_REQUIRE(B <= 65535 && n_heads <= 65535, "prefill_attention: grid too large");
-    PrefillArgs a;
+    PrefillArgs a{};
     a.q = static_cast<const bf16*>(q);
     a.y = static_cast<bf16*>(y);
     a.k = static_cast<const bf16*>(cache->k);
@@ -359,7 +408,6 @@ extern "C" int raven_prefill_attention(const void* q, void* y, const raven_kv_ca
     a.nh = n_heads; a.hd = head_dim; a.t_max = cache->t_max; a.S = S; a.pos0 = pos0; a.pos_dev = pos_dev;
     a.scale_log2 = (float)(1.0 / sqrt((double)head_dim) * 1.4426950408889634);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // two row groups of 16 per wave (128 query rows per workgroup) share every K and V fragment read from LDS
     // Two row groups of 16 per wave (128 query rows per workgroup) share every K and V fragment read from LDS; short
     // launches keep 64 rows per workgroup so that there are more workgroups than compute units.
     const int64_t wgs128 = (int64_t)((S + 127) / 128) * n_heads * B;
@@ -374,4 +422,45 @@ extern "C" int raven_prefill_attention(const void* q, void* y, const raven_kv_ca
     else { RAVEN_PREFILL(128); }
 #undef RAVEN_PREFILL
     return raven_host::check_launch("prefill_attention");
+}
+
+extern "C" int raven_paged_prefill_attention(const void* q, void* y, const void* k_cache, const void* v_cache,
+                                             const int32_t* block_table, const int32_t* seq_lens, const int32_t* q_start, int32_t B,
+                                             int32_t max_q_len, int32_t max_blocks, int32_t block_size, int32_t kv_layout,
+                                             int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream) {
+    using namespace raven;
+    RAVEN_REQUIRE(dtype == RAVEN_BF16, "paged_prefill_attention: bf16 only (dtype %d)", dtype);
+    RAVEN_REQUIRE(head_dim == 64 || head_dim == 96 || head_dim == 128, "paged_prefill_attention: head_dim %d not in {64, 96, 128}", head_dim);
+    RAVEN_REQUIRE(kv_layout == RAVEN_PAGED_NHD || kv_layout == RAVEN_PAGED_HND, "paged_prefill_attention: unknown kv_layout %d", kv_layout);
+    RAVEN_REQUIRE(B >= 0 && B <= 65535 && n_heads > 0 && n_heads <= 65535 && max_q_len >= 0 && max_blocks > 0 && block_size > 0,
+                  "paged_prefill_attention: bad B=%d max_q_len=%d max_blocks=%d block_size=%d", B, max_q_len, max_blocks, block_size);
+    if (B == 0 || max_q_len == 0) return 0;
+    RAVEN_REQUIRE(q && y && k_cache && v_cache && block_table && seq_lens && q_start, "paged_prefill_attention: null pointer");
+    PrefillArgs a{};
+    a.q = static_cast<const bf16*>(q);
+    a.y = static_cast<bf16*>(y);
+    a.k = static_cast<const bf16*>(k_cache);
+    a.v = static_cast<const bf16*>(v_cache);
+    a.nh = n_heads; a.hd = head_dim;
+    a.scale_log2 = (float)(1.0 / sqrt((double)head_dim) * 1.4426950408889634);
+    a.block_table = block_table; a.seq_lens = seq_lens; a.q_start = q_start;
+    a.max_blocks = max_blocks; a.block_size = block_size; a.block_shift = -1;
+    for (int sh = 0; sh < 31; ++sh)
+        if (block_size == (1 << sh)) a.block_shift = sh;
+    a.page_stride = (int64_t)block_size * n_heads * head_dim;
+    a.pos_stride = kv_layout == RAVEN_PAGED_NHD ? (int64_t)n_heads * head_dim : head_dim;
+    a.head_stride = kv_layout == RAVEN_PAGED_NHD ? head_dim : (int64_t)block_size * head_dim;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t wgs128 = (int64_t)((max_q_len + 127) / 128) * n_heads * B;
+    const int rg = wgs128 >= 512 ? 2 : 1;
+    const int rows = 64 * rg;
+    const dim3 grid((max_q_len + rows - 1) / rows, n_heads, B);
+#define RAVEN_PREFILL(HD)                                                                        \
+    if (rg == 2) attention_prefill_kernel<HD, 2, true><<<grid, dim3(256), 0, s>>>(a);            \
+    else attention_prefill_kernel<HD, 1, true><<<grid, dim3(256), 0, s>>>(a)
+    if (head_dim == 64) { RAVEN_PREFILL(64); }
+    else if (head_dim == 96) { RAVEN_PREFILL(96); }
+    else { RAVEN_PREFILL(128); }
+#undef RAVEN_PREFILL
+    return raven_host::check_launch("paged_prefill_attention");
 }

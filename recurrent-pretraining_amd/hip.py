@@ -104,6 +104,8 @@ SIGNATURES = {
                                        C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _VP, _SZ, _VP]),
     "raven_core_iterations": (C.c_int, [C.POINTER(Dims), _VP, C.POINTER(BlockWeights), _I32, _VP, _VP, _VP, _VP, _VP,
                                         C.POINTER(KVCache), C.POINTER(C.c_int32), _I32, _I32, _I32, _I32, _VP, _VP, _SZ, _VP]),
+    "raven_paged_qkv_rope_append": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _VP]),
+    "raven_paged_prefill_attention": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _VP]),
     "raven_paged_decode_blocks": (C.c_int, [C.POINTER(Dims), _VP, C.POINTER(BlockWeights), _I32, _VP, _VP, _VP, _VP, _VP,
                                             C.POINTER(PagedKV), _I32, _I32, _VP, _SZ, _VP]),
 }
@@ -266,6 +268,38 @@ def paged_kv_append(k, v, k_cache, v_cache, slot_mapping, layout: int = PAGED_NH
     rc = load().raven_paged_kv_append(_ptr(k, "k"), _ptr(v, "v", k.dtype), _ptr(k_cache, "k_cache", k.dtype), _ptr(v_cache, "v_cache", k.dtype),
                                       _ptr(slot_mapping, "slot_mapping", torch.int64), T, nh, hd, bs, layout, dtype_code(k.dtype), _stream())
     _check(rc, "raven_paged_kv_append")
+
+
+def paged_qkv_rope_append(qkv, qk_bias, freqs, positions, slot_mapping, k_cache, v_cache, layout: int = PAGED_NHD):
+    """Rows qkv [T, 3 * nh * hd] of any sequences: bias and rotation of positions [T] (int64) on q and k; returns q [T, nh * hd]
+    and writes k, v to the flat slots slot_mapping [T] (int64) of the pages."""
+    T = qkv.shape[0]
+    bs, nh, hd = _paged_dims(k_cache, layout)
+    if qkv.shape[1] != 3 * nh * hd or positions.shape != (T,) or slot_mapping.shape != (T,):
+        raise RavenHipError("paged_qkv_rope_append: qkv [T, 3 * nh * hd], positions [T] and slot_mapping [T] do not fit together")
+    q = torch.empty(T, nh * hd, device=qkv.device, dtype=qkv.dtype)
+    rc = load().raven_paged_qkv_rope_append(
+        _ptr(qkv, "qkv"), _ptr(qk_bias, "qk_bias", qkv.dtype), _ptr(freqs, "freqs", torch.float32), _ptr(positions, "positions", torch.int64),
+        _ptr(slot_mapping, "slot_mapping", torch.int64), _ptr(q, "q"), _ptr(k_cache, "k_cache", qkv.dtype), _ptr(v_cache, "v_cache", qkv.dtype),
+        T, nh, hd, bs, layout, dtype_code(qkv.dtype), _stream())
+    _check(rc, "raven_paged_qkv_rope_append")
+    return q
+
+
+def paged_prefill_attention(q, k_cache, v_cache, block_table, seq_lens, q_start, max_q_len: int, layout: int = PAGED_NHD):
+    """Causal attention of the rows q [T, nh * hd] (bf16) of several sequences over their pages: sequence b owns rows
+    q_start[b] .. q_start[b + 1] - 1 (q_start [B + 1] int32), the last positions of its seq_lens[b] cached ones."""
+    B = seq_lens.shape[0]
+    if q_start.shape != (B + 1,) or block_table.dim() != 2 or block_table.shape[0] != B:
+        raise RavenHipError("paged_prefill_attention: block_table [B, max_blocks], seq_lens [B] and q_start [B + 1] do not fit together")
+    block_size, nh, hd = _paged_dims(k_cache, layout)
+    y = torch.empty_like(q)
+    rc = load().raven_paged_prefill_attention(
+        _ptr(q, "q"), _ptr(y, "y"), _ptr(k_cache, "k_cache", q.dtype), _ptr(v_cache, "v_cache", q.dtype),
+        _ptr(block_table, "block_table", torch.int32), _ptr(seq_lens, "seq_lens", torch.int32), _ptr(q_start, "q_start", torch.int32),
+        B, int(max_q_len), block_table.shape[1], block_size, layout, nh, hd, dtype_code(q.dtype), _stream())
+    _check(rc, "raven_paged_prefill_attention")
+    return y
 
 
 def paged_decode_attention(q, k_cache, v_cache, block_table, seq_lens, max_seq_len, workspace=None, layout: int = PAGED_NHD):

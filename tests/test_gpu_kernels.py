@@ -749,3 +749,83 @@ def test_paged_decode_attention_and_append(pkg, dt, nh, hd, B, block_size, layou
     check(kc, kc2.float().cpu(), dt, "keys after the fused paged step")
     assert torch.equal(vc, vc2)
     assert int((rows_of(kc).abs().amax(dim=(1, 2)) > 0).sum()) == int(lens.sum())  # no other row was touched
+
+
+@pytest.mark.parametrize("nh,hd,block_size,layout,chunks", [
+    (55, 96, 16, "HND", ((0, 300), (212, 40), (699, 1), (0, 0), (64, 64), (5, 130))),
+    (55, 96, 16, "NHD", ((0, 200), (100, 100))),
+    (4, 64, 12, "HND", ((0, 77), (30, 300))),
+    (3, 128, 32, "NHD", ((1, 129), (500, 200), (0, 1))),
+    (55, 96, 16, "HND", tuple((37 * i % 200, 640) for i in range(10))),   # 128-row workgroups
+])
+def test_paged_rope_append_and_prefill_attention_of_several_sequences(pkg, nh, hd, block_size, layout, chunks):
+    """Prompt chunks and decode rows of several sequences in one launch each, over shuffled pages: chunk (context, rows)
+    means the sequence already holds `context` positions and `rows` new ones arrive.  raven_paged_qkv_rope_append against
+    the oracle's bias + RoPE per row (and the slots it must fill), raven_paged_prefill_attention against torch SDPA with a
+    lower-right aligned causal mask per sequence, and against the contiguous-cache kernel's bits."""
+    dt, h = torch.bfloat16, nh * hd
+    lay = pkg.hip.PAGED_NHD if layout == "NHD" else pkg.hip.PAGED_HND
+    B = len(chunks)
+    g = torch.Generator().manual_seed(700 + B + block_size)
+    max_len = max(c + r for c, r in chunks) + 3
+    max_blocks = (max_len + block_size - 1) // block_size
+    num_blocks = B * max_blocks + 2
+    table = torch.randperm(num_blocks, generator=g)[:B * max_blocks].view(B, max_blocks).to(torch.int32)
+    shape = (num_blocks, block_size, nh, hd) if layout == "NHD" else (num_blocks, nh, block_size, hd)
+    kc, vc = torch.zeros(shape, dtype=dt, device="cuda"), torch.zeros(shape, dtype=dt, device="cuda")
+    slot_of = lambda b, p: int(table[b, p // block_size]) * block_size + p % block_size
+    # the contexts: already rotated keys, through the plain append kernel
+    k_ctx = [rnd((c, nh, hd), dt, 710 + b) for b, (c, r) in enumerate(chunks)]
+    v_ctx = [rnd((c, nh, hd), dt, 740 + b) for b, (c, r) in enumerate(chunks)]
+    rows = [(b, p) for b, (c, r) in enumerate(chunks) for p in range(c)]
+    if rows:
+        pkg.hip.paged_kv_append(torch.stack([k_ctx[b][p].reshape(-1) for b, p in rows]).cuda(),
+                                torch.stack([v_ctx[b][p].reshape(-1) for b, p in rows]).cuda(), kc, vc,
+                                torch.tensor([slot_of(b, p) for b, p in rows], dtype=torch.int64).cuda(), layout=lay)
+    # the new rows of all sequences, flattened as a serving engine hands them over, plus one row that is not stored
+    T = sum(r for c, r in chunks)
+    qkv = rnd((T + 1, 3 * h), dt, 770)
+    bias = rnd((2, nh, hd), dt, 771, 0.5)
+    rope = O.rope_table(hd, max_len, 50000.0).to(dt)
+    freqs = rope.float().reshape(max_len, hd // 2, 2).contiguous().cuda()
+    positions = torch.tensor([c + i for c, r in chunks for i in range(r)] + [0], dtype=torch.int64)
+    slots = torch.tensor([slot_of(b, c + i) for b, (c, r) in enumerate(chunks) for i in range(r)] + [-1], dtype=torch.int64)
+    before = kc.clone()
+    q = pkg.hip.paged_qkv_rope_append(qkv.cuda(), bias.cuda(), freqs, positions.cuda(), slots.cuda(), kc, vc, layout=lay)
+    qq, kk, vv = (t.view(T + 1, 1, nh, hd) for t in qkv.split([h, h, h], dim=1))
+    qq, kk = (qq + bias[0]).to(dt), (kk + bias[1]).to(dt)
+    want_q, want_k = torch.empty(T + 1, nh, hd, dtype=dt), torch.empty(T + 1, nh, hd, dtype=dt)
+    for t in range(T + 1):
+        rq, rk = O.apply_rope(qq[t:t + 1], kk[t:t + 1], rope[:, int(positions[t]):int(positions[t]) + 1])
+        want_q[t], want_k[t] = rq.view(nh, hd), rk.view(nh, hd)
+    assert torch.equal(q.cpu().view(T + 1, nh, hd), want_q)
+    rows_of = (lambda c: c.view(-1, nh, hd)) if layout == "NHD" else (lambda c: c.permute(0, 2, 1, 3).reshape(-1, nh, hd))
+    flat_k, flat_v = rows_of(kc).cpu(), rows_of(vc).cpu()
+    for t in range(T):
+        assert torch.equal(flat_k[int(slots[t])], want_k[t]) and torch.equal(flat_v[int(slots[t])], vv[t, 0])
+    untouched = torch.ones(flat_k.shape[0], dtype=torch.bool)
+    untouched[slots[:T]] = False
+    assert torch.equal(flat_k[untouched], rows_of(before).cpu()[untouched])  # the row with slot -1 went nowhere
+
+    lens = torch.tensor([c + r for c, r in chunks], dtype=torch.int32)
+    q_start = torch.tensor([0] + list(torch.tensor([r for c, r in chunks]).cumsum(0)), dtype=torch.int32)
+    max_q = max(r for c, r in chunks)
+    y = pkg.hip.paged_prefill_attention(q[:T].contiguous(), kc, vc, table.cuda(), lens.cuda(), q_start.cuda(), max_q, layout=lay)
+    t0 = 0
+    for b, (c, r) in enumerate(chunks):
+        if r == 0:
+            continue
+        keys = torch.cat([k_ctx[b], want_k[t0:t0 + r]]).transpose(0, 1).unsqueeze(0)      # [1, nh, c + r, hd]
+        vals = torch.cat([v_ctx[b], vv[t0:t0 + r, 0]]).transpose(0, 1).unsqueeze(0)
+        want = O.sdpa(want_q[t0:t0 + r].transpose(0, 1).unsqueeze(0), keys, vals).transpose(1, 2).reshape(r, h)
+        check(y[t0:t0 + r], want, dt, f"paged prefill attention, sequence {b}: {r} rows after {c}")
+        if r >= 2:   # the contiguous-cache kernel on the same keys: same arithmetic, other addresses
+            kd, vd = keys.unsqueeze(0).contiguous().cuda(), vals.unsqueeze(0).contiguous().cuda()
+            same = pkg.hip.prefill_attention(q[t0:t0 + r].contiguous(), pkg.hip.make_cache(kd, vd), 0, 1, r, c, nh, hd)
+            if (max_q + 127) // 128 * nh * B >= 512 and (r + 127) // 128 * nh < 512:
+                check(y[t0:t0 + r], same, dt, "paged vs contiguous (other rows per workgroup)")
+            else:
+                assert torch.equal(y[t0:t0 + r], same), f"paged vs contiguous, sequence {b}"
+        t0 += r
+    with pytest.raises(pkg.hip.RavenHipError):
+        pkg.hip.paged_prefill_attention(q[:T].float(), kc.float(), vc.float(), table.cuda(), lens.cuda(), q_start.cuda(), max_q, layout=lay)
