@@ -171,14 +171,34 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
     };
     auto fetch = [&](int kt) {
         if constexpr (PAGED) {
+            if (a.block_shift >= 2 && kt + kPfKeys <= n_keys) {
+                // a whole tile of needed keys, pages of 4 * 2^n positions: shifts instead of divisions, no clamping, and
+                // the four consecutive keys of a V task share a page
+                const int mask = a.block_size - 1;
+                auto off = [&](int p) {
+                    const int pg = p >> a.block_shift;
+                    const int page = pg < kPfTable ? tbl[pg] : table_row[pg];
+                    return (int64_t)page * a.page_stride + (int64_t)((p & mask) * (int)a.pos_stride);
+                };
 #pragma unroll
-            for (int i = 0; i < KCH; ++i) {
-                const int c = threadIdx.x + 256 * i;
-                const int key = c / CPR, dc = c - key * CPR;
-                kreg[i] = *reinterpret_cast<const u32x4*>(Kb + paged_off(kt + key) + dc * 8);
+                for (int i = 0; i < KCH; ++i) {
+                    const int c = threadIdx.x + 256 * i;
+                    const int key = c / CPR, dc = c - key * CPR;
+                    kreg[i] = *reinterpret_cast<const u32x4*>(Kb + off(kt + key) + dc * 8);
+                }
+                const bf16* vp = Vb + off(kt + 4 * v_kg) + v_dc * 8;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) vreg[i] = *reinterpret_cast<const u32x4*>(vp + i * a.pos_stride);
+            } else {
+#pragma unroll
+                for (int i = 0; i < KCH; ++i) {
+                    const int c = threadIdx.x + 256 * i;
+                    const int key = c / CPR, dc = c - key * CPR;
+                    kreg[i] = *reinterpret_cast<const u32x4*>(Kb + paged_off(kt + key) + dc * 8);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) vreg[i] = *reinterpret_cast<const u32x4*>(Vb + paged_off(kt + 4 * v_kg + i) + v_dc * 8);
             }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) vreg[i] = *reinterpret_cast<const u32x4*>(Vb + paged_off(kt + 4 * v_kg + i) + v_dc * 8);
         } else if (kt + kPfKeys <= a.t_max) {
 #pragma unroll
             for (int i = 0; i < KCH; ++i) kreg[i] = *reinterpret_cast<const u32x4*>(k_src + (int64_t)kt * HD + 2048 * i);
@@ -447,6 +467,7 @@ extern "C" int raven_paged_prefill_attention(const void* q, void* y, const void*
     a.max_blocks = max_blocks; a.block_size = block_size; a.block_shift = -1;
     for (int sh = 0; sh < 31; ++sh)
         if (block_size == (1 << sh)) a.block_shift = sh;
+    RAVEN_REQUIRE((int64_t)block_size * n_heads * head_dim < (1ll << 31), "paged_prefill_attention: a page of %d positions is too large", block_size);
     a.page_stride = (int64_t)block_size * n_heads * head_dim;
     a.pos_stride = kv_layout == RAVEN_PAGED_NHD ? (int64_t)n_heads * head_dim : head_dim;
     a.head_stride = kv_layout == RAVEN_PAGED_NHD ? head_dim : (int64_t)block_size * head_dim;

@@ -10,7 +10,9 @@ lengths decode together, each at its own position (the contiguous cache of the H
 across the batch, raven_modeling_minimal.py:660-665).
 
 The arithmetic of a step is the contiguous decode path's: the same SandwichBlock launches with the paged decode-attention
-kernel in place of the contiguous one (raven_paged_decode_blocks)."""
+kernel in place of the contiguous one (raven_paged_decode_blocks).  forward_tokens takes any mix of prompt chunks and decode
+rows of several sequences, flattened as a serving engine hands them over, through the paged chunk kernels
+(raven_paged_qkv_rope_append, raven_paged_prefill_attention)."""
 
 from __future__ import annotations
 
@@ -28,9 +30,6 @@ class PagedDecoder:
     def __init__(self, model, num_blocks: int, block_size: int = 16, num_steps: Optional[int] = None, use_graph: bool = False,
                  layout: str = "HND"):
         cfg = model.config
-        if (cfg.n_layers_in_prelude, cfg.n_layers_in_recurrent_block) != (2, 4):
-            # the equivalence with the cache-sharing strategy of the other surface hard-codes these counts (RMM:169-182)
-            raise NotImplementedError("the paged decoder mirrors a model with 2 prelude and 4 core blocks")
         self.model, self.cfg = model, cfg
         self.r = cfg.mean_recurrence if num_steps is None else int(num_steps)
         if self.r < 1:
@@ -64,6 +63,10 @@ class PagedDecoder:
     def load_prompt(self, cache: HuginnDynamicCache, row: int, table_row: Sequence[int]) -> int:
         """Copies sequence `row` of a cache filled through the other surface with lookup_strategy `latest-m4-compress-s4`
         into the pages listed in table_row; returns the number of positions."""
+        if (self.cfg.n_layers_in_prelude, self.cfg.n_layers_in_recurrent_block) != (2, 4):
+            # the equivalence with the cache-sharing strategy of the other surface hard-codes these counts (RMM:169-182)
+            raise NotImplementedError("prompts come over from the other surface only for a model with 2 prelude and 4 core blocks; "
+                                      "forward_tokens() has no such limit")
         if cache.lookup_strategy != PAGED_STRATEGY:
             raise ValueError(f"a prompt for the paged decoder must be cached with lookup_strategy={PAGED_STRATEGY!r}")
         n = cache.get_seq_length()
@@ -88,6 +91,85 @@ class PagedDecoder:
                          cache_position=torch.arange(n, device=input_ids.device), num_steps=self.r)
         self.load_prompt(cache, 0, table_row)
         return out
+
+    # ------------------------------------------------------------------ rows of any sequences (prompt chunks, decode rows)
+    def _mm(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        """x [T, K] times w [N, K] transposed: the library for many rows, the skinny kernels for few."""
+        return torch.matmul(x, w.t()) if x.shape[0] >= self.model.WIDE_ROWS else hip.gemm(x, w)
+
+    def _token_block(self, blk, f: int, x: torch.Tensor, meta) -> torch.Tensor:
+        """One SandwichBlock (vllm/raven_vllm.py:289-294 around its attention layer, :184-203) on flat rows, flat layer f."""
+        eps = self.cfg.norm_eps
+        positions, slots, table, lens, q_start, max_q = meta
+        n1 = hip.rmsnorm_residual(x, blk.norm_1.weight, eps)[0]
+        qkv = self._mm(n1, blk.attn.Wqkv.weight)
+        bias = blk.attn.qk_bias if hasattr(blk.attn, "qk_bias") else None
+        q = hip.paged_qkv_rope_append(qkv, bias, self.model._natives()["freqs"], positions, slots, self.k[f], self.v[f], layout=self.layout)
+        ya = hip.paged_prefill_attention(q, self.k[f], self.v[f], table, lens, q_start, max_q, layout=self.layout)
+        a = self._mm(ya, blk.attn.proj.weight)
+        x2, _, n3 = hip.rmsnorm_residual(a, blk.norm_2.weight, eps, residual=x, weight2=blk.norm_3.weight)
+        m = self._mm(hip.swiglu(self._mm(n3, blk.mlp.fc.weight)), blk.mlp.proj.weight)
+        return hip.rmsnorm_residual(m, blk.norm_4.weight, eps, residual=x2)[0]
+
+    @torch.no_grad()
+    def forward_tokens(self, input_ids: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor, block_table: torch.Tensor,
+                       seq_lens: torch.Tensor, query_start_loc: torch.Tensor, max_query_len: int,
+                       input_states: Optional[torch.Tensor] = None, init_scale: float = 1.0):
+        """What the plugin's model computes for one scheduler step (RavenModel.forward, vllm/raven_vllm.py:374-411), straight on
+        the pages: input_ids [T] are the new rows of B sequences, flattened (prompt chunks of any length and decode rows
+        together); positions [T] and slot_mapping [T] (int64) say where each row sits; sequence b owns rows
+        query_start_loc[b] .. query_start_loc[b + 1] - 1 and holds seq_lens[b] positions once they are appended.
+        Returns (logits [T, V] float32, latents [T, h]).  bf16 models with head_dim 64 / 96 / 128."""
+        m, cfg, t = self.model, self.cfg, self.model.transformer
+        if m.dtype != torch.bfloat16:
+            raise NotImplementedError("forward_tokens: the paged chunk attention kernel is bf16 only")
+        T = input_ids.numel()
+        B = seq_lens.shape[0]
+        if positions.shape != (T,) or slot_mapping.shape != (T,) or query_start_loc.shape != (B + 1,) or block_table.shape[0] != B:
+            raise ValueError("positions [T], slot_mapping [T], block_table [B, max_blocks], seq_lens [B], query_start_loc [B + 1]")
+        dev = m.device
+        meta = (positions.to(dev, torch.int64), slot_mapping.to(dev, torch.int64), block_table.to(dev, torch.int32).contiguous(),
+                seq_lens.to(dev, torch.int32), query_start_loc.to(dev, torch.int32), int(max_query_len))
+        n_pre, n_core = cfg.n_layers_in_prelude, cfg.n_layers_in_recurrent_block
+        x = hip.embed(t.wte.weight, input_ids.reshape(-1).to(dev, torch.int64).contiguous(), m.emb_scale)
+        for i in range(n_pre):
+            x = self._token_block(t.prelude[i], i, x, meta)
+        embeds = x
+        if input_states is None:
+            state = m.initialize_state(embeds, init_scale) if init_scale > 0 else torch.zeros_like(embeds)
+        else:
+            state = input_states.reshape(T, -1).to(dev, m.dtype)
+        for _ in range(self.r):
+            state = self._mm(torch.cat([state, embeds], dim=-1), t.adapter.weight)
+            for j in range(n_core):
+                state = self._token_block(t.core_block[j], n_pre + j, state, meta)
+        latents = hip.rmsnorm_residual(state, t.ln_f.weight, cfg.norm_eps)[0]
+        x = latents
+        for i in range(cfg.n_layers_in_coda):
+            x = self._token_block(t.coda[i], n_pre + n_core + i, x, meta)
+        x = hip.rmsnorm_residual(x, t.ln_f.weight, cfg.norm_eps)[0]
+        logits = torch.matmul(x, m.lm_head.weight.t()).float() if T >= m.WIDE_ROWS else hip.gemm(x, m.lm_head.weight, out_f32=True)
+        return logits, latents
+
+    def prefill_paged(self, input_ids: torch.Tensor, table_row: Sequence[int], input_states: Optional[torch.Tensor] = None,
+                      chunk: Optional[int] = None):
+        """One prompt [1, n] straight into the pages of table_row, `chunk` rows at a time (all at once by default).
+        Returns (logits [n, V], latents [n, h])."""
+        n = input_ids.shape[1]
+        if n > len(table_row) * self.block_size:
+            raise ValueError(f"{len(table_row)} blocks of {self.block_size} cannot hold {n} positions")
+        chunk = n if chunk is None else int(chunk)
+        table = torch.as_tensor([list(table_row)], dtype=torch.int32)
+        row = torch.as_tensor(list(table_row), dtype=torch.int64)
+        outs = []
+        for lo in range(0, n, chunk):
+            hi = min(n, lo + chunk)
+            pos = torch.arange(lo, hi)
+            slots = row[pos // self.block_size] * self.block_size + pos % self.block_size
+            st = None if input_states is None else input_states[:, lo:hi]
+            outs.append(self.forward_tokens(input_ids[0, lo:hi], pos, slots, table, torch.tensor([hi], dtype=torch.int32),
+                                            torch.tensor([0, hi - lo], dtype=torch.int32), hi - lo, input_states=st))
+        return torch.cat([o[0] for o in outs]), torch.cat([o[1] for o in outs])
 
     # ------------------------------------------------------------------ decode
     def _buffers(self, B: int, max_blocks: int):

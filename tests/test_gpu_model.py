@@ -578,6 +578,92 @@ def test_paged_decoder_serves_sequences_of_different_lengths(pkg, small242, lens
         dec.load_prompt(pkg.HuginnDynamicCache(), 0, table[0].tolist())
 
 
+@pytest.mark.parametrize("layout,bs", [("HND", 16), ("NHD", 8)])
+def test_paged_forward_tokens_prompt_chunks_and_decode_rows_together(pkg, layout, bs):
+    """forward_tokens: what the reference's vLLM model computes for one scheduler step, on the pages.  A bf16 model with the
+    3.5b model's 2/4/2 structure; three sequences.  (1) Every prompt straight into its pages, whole or in chunks: logits
+    and page contents equal those of the other route (the prompt through forward() with the cache-sharing strategy of the
+    same semantics, then copied into pages).  (2) One mixed step -- a decode row of sequence 0, a prompt chunk of
+    sequence 1 on top of its cached part, a fresh prompt of sequence 2 -- equals the three done one by one.  (3) The
+    decode kernels continue from pages that forward_tokens filled.  One recurrence against the oracle within the bf16
+    bar; deeper chains are compared between the package's own routes (same kernels, other addresses)."""
+    dt = torch.bfloat16
+
+    def loose(got, want, what):
+        """Routes that give the GEMMs other row counts (a chunk of 12 rows, a batch of 64) go through other GEMM kernels;
+        the 12 blocks of a pass amplify their rounding differences (the oracle run in bf16 moves as much when its
+        accumulation order changes): 5e-2 instead of 1e-2 on the relative L2 error, the first layer's keys at the full bar."""
+        max_abs, rel = close(got, want, what)
+        assert rel <= 5e-2, f"{what}: rel-L2 {rel:.3e}"
+
+    s = O.RavenShape(n_embd=128, n_heads=2, intermediate_size=352, vocab_size=512, n_layers_in_prelude=2,
+                     n_layers_in_recurrent_block=4, n_layers_in_coda=2, mean_recurrence=4)
+    w = O.make_weights(s, seed=5, dtype=dt)
+    w["freqs_cis"] = w["freqs_cis"].to(dt)
+    cfg = pkg.RavenConfig(n_embd=128, n_heads=2, n_layers=8, n_layers_in_prelude=2, n_layers_in_recurrent_block=4,
+                          n_layers_in_coda=2, intermediate_size=352, vocab_size=512, mean_recurrence=4)
+    model = build_model(pkg, cfg, w, dt)
+    r, lens = 2, (70, 45, 38)
+    g = torch.Generator().manual_seed(91)
+    max_blocks = (max(lens) + 4 + bs - 1) // bs
+    n_blocks = 3 * max_blocks + 4
+    table = torch.randperm(n_blocks, generator=g)[:3 * max_blocks].view(3, max_blocks).to(torch.int32)
+    prompts = [torch.randint(0, s.vocab_size, (1, n), generator=g) for n in lens]
+    states = [O.initialize_state(torch.empty(1, n + 1, s.n_embd), s, 1.0, g).to(dt) for n in lens]
+    a = pkg.PagedDecoder(model, num_blocks=n_blocks, block_size=bs, num_steps=r, layout=layout)   # the route under test
+    b = pkg.PagedDecoder(model, num_blocks=n_blocks, block_size=bs, num_steps=r, layout=layout)   # prompts through forward()
+    for i, n in enumerate(lens):
+        other = b.prefill(prompts[i].cuda(), table[i].tolist(), input_states=states[i][:, :n].cuda())
+        logits, _ = a.prefill_paged(prompts[i].cuda(), table[i].tolist(), input_states=states[i][:, :n].cuda(),
+                                    chunk=33 if i == 1 else None)
+        (loose if i == 1 else check)(logits, other.logits[0], *(() if i == 1 else (dt,)), f"prompt {i}: straight into the pages vs through forward()")
+    check(a.k[0], b.k[0], dt, "keys of the first flat layer")
+    check(a.v[0], b.v[0], dt, "values of the first flat layer")
+    for f in range(1, a.n_flat):
+        loose(a.k[f], b.k[f], f"keys of flat layer {f}")
+        loose(a.v[f], b.v[f], f"values of flat layer {f}")
+    # one recurrence against the oracle
+    one = pkg.PagedDecoder(model, num_blocks=n_blocks, block_size=bs, num_steps=1, layout=layout)
+    want = O.forward(w, s, input_ids=prompts[2], input_states=states[2][:, :lens[2]], num_steps=1)
+    logits, latents = one.prefill_paged(prompts[2].cuda(), table[2].tolist(), input_states=states[2][:, :lens[2]].cuda())
+    check(latents, want.latent_states[0], dt, "one recurrence, latents")
+    check(logits, want.logits[0], dt, "one recurrence, logits")
+
+    # (2) a mixed step on fresh pages: sequence 0 has its prompt cached and decodes one row, sequence 1 has 20 rows cached
+    # and brings the other 25, sequence 2 brings its whole prompt
+    mixed = pkg.PagedDecoder(model, num_blocks=n_blocks, block_size=bs, num_steps=r, layout=layout)
+    mixed.prefill_paged(prompts[0].cuda(), table[0].tolist(), input_states=states[0][:, :lens[0]].cuda())
+    mixed.prefill_paged(prompts[1][:, :20].cuda(), table[1].tolist(), input_states=states[1][:, :20].cuda())
+    tok0 = torch.randint(0, s.vocab_size, (1,), generator=g)
+    rows = [(0, lens[0], tok0, states[0][0, lens[0]:lens[0] + 1])] + \
+           [(1, p, prompts[1][0, p:p + 1], states[1][0, p:p + 1]) for p in range(20, lens[1])] + \
+           [(2, p, prompts[2][0, p:p + 1], states[2][0, p:p + 1]) for p in range(lens[2])]
+    ids = torch.cat([t for _, _, t, _ in rows])
+    pos = torch.tensor([p for _, p, _, _ in rows])
+    slots = torch.tensor([int(table[q, p // bs]) * bs + p % bs for q, p, _, _ in rows])
+    st = torch.cat([x for _, _, _, x in rows])
+    counts = [1, lens[1] - 20, lens[2]]
+    logits, latents = mixed.forward_tokens(ids, pos, slots, table, torch.tensor([lens[0] + 1, lens[1], lens[2]], dtype=torch.int32),
+                                           torch.tensor([0, 1, 1 + counts[1], 1 + counts[1] + counts[2]], dtype=torch.int32),
+                                           max(counts), input_states=st)
+    # the same three pieces one by one on the decoder filled in (1)
+    l1, _ = a.forward_tokens(prompts[1][0, 20:], torch.arange(20, lens[1]),
+                             torch.tensor([int(table[1, p // bs]) * bs + p % bs for p in range(20, lens[1])]), table[1:2],
+                             torch.tensor([lens[1]], dtype=torch.int32), torch.tensor([0, counts[1]], dtype=torch.int32), counts[1],
+                             input_states=states[1][0, 20:lens[1]])
+    loose(logits[1:1 + counts[1]], l1, "mixed step, the prompt chunk")
+    l2, _ = a.prefill_paged(prompts[2].cuda(), table[2].tolist(), input_states=states[2][:, :lens[2]].cuda())
+    loose(logits[1 + counts[1]:], l2, "mixed step, the fresh prompt")
+    # (3) the decode row: the decode kernels on the pages of `a` give the same
+    step_logits, _ = a.step(tok0.cuda(), table[0:1].cuda(), torch.tensor([lens[0] + 1], dtype=torch.int32).cuda(),
+                            input_states=states[0][0, lens[0]:lens[0] + 1].cuda())
+    loose(logits[0], step_logits[0], "mixed step, the decode row vs the decode kernels")
+    with pytest.raises(NotImplementedError):
+        pkg.PagedDecoder(build_model(pkg, pkg.RavenConfig.tiny(), O.make_weights(O.RavenShape.tiny(), seed=0, dtype=torch.float32),
+                                     torch.float32), num_blocks=8, block_size=4).forward_tokens(
+            ids[:1], pos[:1], slots[:1], table[:1], torch.tensor([1], dtype=torch.int32), torch.tensor([0, 1], dtype=torch.int32), 1)
+
+
 @pytest.mark.parametrize("dt,B", [(torch.float32, 1), (torch.bfloat16, 1), (torch.bfloat16, 3), (torch.float32, 6), (torch.bfloat16, 6),
                                   (torch.bfloat16, 32)])
 def test_core_iterations_equal_single_iterations(pkg, tiny32, tiny16, dt, B):
