@@ -173,6 +173,20 @@ def paged(args):
     n_blocks = B * max_blocks
     table = torch.randperm(n_blocks, generator=g).view(B, max_blocks).to(torch.int32).to(dev)
     dec = pkg.PagedDecoder(model, num_blocks=n_blocks, block_size=bs, num_steps=r, use_graph=not args.no_graph, layout=args.paged_layout)
+    # prompt processing on the pages first: up to four prompts of --prompt tokens in one forward_tokens call
+    n_p, n_tok = min(B, 4), min(args.prompt, int(lens.min()))
+    p_ids = torch.randint(0, cfg.vocab_size, (n_p * n_tok,), generator=g).to(dev)
+    p_pos = torch.arange(n_tok).repeat(n_p)
+    p_slots = torch.cat([table[b].cpu().to(torch.int64)[torch.arange(n_tok) // bs] * bs + torch.arange(n_tok) % bs for b in range(n_p)])
+    p_args = (p_ids, p_pos.to(dev), p_slots.to(dev), table[:n_p], torch.full((n_p,), n_tok, dtype=torch.int32, device=dev),
+              (torch.arange(n_p + 1, dtype=torch.int32) * n_tok).to(dev), n_tok)
+    p_state = torch.zeros(n_p * n_tok, cfg.n_embd, dtype=torch.bfloat16, device=dev)
+    dec.forward_tokens(*p_args, input_states=p_state)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dec.forward_tokens(*p_args, input_states=p_state)
+    torch.cuda.synchronize()
+    prompt_dt = time.perf_counter() - t0
     for t in dec.k + dec.v:
         t.normal_(0.0, 1.0)
     ids = torch.randint(0, cfg.vocab_size, (B,), generator=g).to(dev)
@@ -207,6 +221,8 @@ def paged(args):
                                f"(mean {float(lens.float().mean()):.0f}), block size {bs}", "batch": B, "recurrence": r, "hip_graph": not args.no_graph,
                    "layout": args.paged_layout},
         "kv_GB_per_step": round(kv_bytes / 1e9, 2),
+        "prompt_chunks": {"call": "PagedDecoder.forward_tokens", "sequences": n_p, "rows": n_p * n_tok, "ms": round(prompt_dt * 1e3, 2),
+                          "prompt_tokens_per_s": round(n_p * n_tok / prompt_dt, 1)},
     }
     print(json.dumps(line))
 
