@@ -50,7 +50,7 @@ exact numbers it publishes are three KV-cache sizes, used as known-answer tests.
 from __future__ import annotations
 
 import math
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Optional
 
 import torch
