@@ -172,7 +172,7 @@ __global__ __launch_bounds__(256) void mfma_ns_kernel(NsArgs a) {
 
     // k-values in front of the first and behind the last full macro-step of each segment (32 for K = 5280):
     // the last K slice takes them, straight from global memory
-    if (blockIdx.y == a.ks - 1) {
+    if ((int)blockIdx.y == a.ks - 1) {
 #pragma unroll 1
         for (int part = 0; part < 4; ++part) {
             const int seg = part >> 1;
