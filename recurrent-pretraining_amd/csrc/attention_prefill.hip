@@ -8,12 +8,12 @@
 // Grid (query blocks of 64 or 128 rows, heads, sequences), the blocks with the most keys first; 4 waves, each owns
 // RG groups of 16 query rows (RG = 1 or 2) and walks all key tiles of 64 positions on its own (no cross-wave softmax
 // state).  Per key tile:
-//   * the workgroup stages K [64 x hd] and V transposed [hd x 64] in one of two LDS buffers, through registers that
+//   * the workgroup stages K [64 x hd] and V [64 x hd] in one of two LDS buffers, through registers that
 //     were loaded one tile earlier (so the tile two ahead is in flight during the products; one barrier per tile);
 //   * S^T = K Q^T with v_mfma_f32_16x16x32_bf16, every K fragment multiplied into all row groups: a lane then holds,
 //     for ONE query (l % 16) of each group, the scores of keys 4*(l/16) + v of each 16-key sub-tile -- exactly the
 //     lane-row / k-slice shape the A operand of the next MFMA wants, so P never leaves registers: the 32 "k" slots
-//     of a P V MFMA are mapped to keys (sub-tile pair, 4*(l/16) + v), and V^T is laid out in LDS in that order;
+//     of a P V MFMA are mapped to keys (sub-tile pair, 4*(l/16) + v), and V is read from LDS with ds_read_b64_tr_b16 in that order (no transposed copy);
 //   * online softmax per query against a reference maximum that moves only when a tile exceeds it by 2^8 (O is then
 //     rescaled, with factors fetched by one shuffle per row); exp2 with the scale folded in; the row sums come from
 //     one more MFMA against a tile of ones, in O's own layout;
@@ -31,7 +31,7 @@
 namespace raven {
 
 constexpr int kPfKeys = 64;     // keys per tile
-constexpr int kVtPitch = 72;    // bf16 elements per V^T row: 64 + 8 (144 bytes: the 16-byte reads of 16 rows hit 64 different banks)
+constexpr int kVPitch = 144;    // bf16 elements per V row in LDS (288 bytes = 72 banks: the 8 key rows that 32 lanes read transposed hit 64 different banks)
 
 struct PrefillArgs {
     const bf16* q;   // [B*S, h]
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
     constexpr int WR = 16 * RG;      // query rows per wave
     constexpr int ROWS = 4 * WR;     // query rows per workgroup
     __shared__ __align__(16) bf16 sk[2][kPfKeys][KP];
-    __shared__ __align__(16) bf16 svt[2][HD][kVtPitch];
+    __shared__ __align__(16) bf16 sv[2][kPfKeys][kVPitch];
 
     const int qb = gridDim.x - 1 - blockIdx.x;  // the blocks with the most keys start first
     const int head = blockIdx.y, b = blockIdx.z;
@@ -138,29 +138,22 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
 
     // Global -> registers -> LDS, two tiles ahead of the multiply and two LDS buffers: the loads of tile i + 2 are in
     // flight while tile i is multiplied and tile i + 1 sits in the other buffer; one barrier per tile.
-    // K: the tile is one contiguous piece of the cache, 16-byte chunks.  V: a thread takes the same 8 columns of 4
-    // consecutive keys and writes, per column, the 4 keys as one 8-byte piece of the transposed tile; threads beyond
-    // the number of such tasks repeat the first ones (same values to the same addresses), so no wave branches.
+    // K and V tiles are contiguous pieces of the cache (or gathered page rows), moved as 16-byte chunks of key rows; V
+    // stays row-major in LDS and is read through ds_read_b64_tr_b16, which hands a lane four keys of one column.
     constexpr int CPR = HD / 8;                     // chunks per key row
-    constexpr int KCH = kPfKeys * CPR / 256;        // K chunks per thread
-    constexpr int VTASKS = (kPfKeys / 4) * CPR;     // V tasks per tile (at most 256)
-    static_assert(kPfKeys * CPR % 256 == 0 && VTASKS <= 256, "staging shape");
+    constexpr int KCH = kPfKeys * CPR / 256;        // chunks per thread, of K and of V
+    static_assert(kPfKeys * CPR % 256 == 0, "staging shape");
     u32x4 kreg[KCH];
-    u32x4 vreg[4];
-    const int v_task = threadIdx.x < VTASKS ? threadIdx.x : threadIdx.x - VTASKS;
-    const int v_kg = v_task % (kPfKeys / 4), v_dc = v_task / (kPfKeys / 4);
+    u32x4 vreg[KCH];
     const bf16* k_src = Kb + threadIdx.x * 8;
-    const bf16* v_src = Vb + (int64_t)(4 * v_kg) * HD + v_dc * 8;
-    int k_dst[KCH];  // element offsets inside one K buffer
+    const bf16* v_src = Vb + threadIdx.x * 8;
+    int k_dst[KCH], v_dst[KCH];  // element offsets inside one buffer
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
         const int c = threadIdx.x + 256 * i;
         k_dst[i] = (c / CPR) * KP + (c % CPR) * 8;
+        v_dst[i] = (c / CPR) * kVPitch + (c % CPR) * 8;
     }
-    // Inside each block of 32 keys the transposed tile keeps the 4-key pieces in the order the P fragments want them:
-    // piece r = 4*(t&1) + s4 (keys 16*(t&1) + 4*s4 ..+3) sits at 8*s4 + 4*(t&1), so a lane's 8 keys of a k-step are
-    // one 16-byte read.
-    const int v_dst = (v_dc * 8) * kVtPitch + 32 * (v_kg / 8) + 8 * (v_kg % 4) + 4 * ((v_kg % 8) / 4);
     // paged: element offset of position p's head row.  Positions past the last key this workgroup needs repeat that key
     // (they are masked): only the pages up to it are in `tbl`, and only those are known to exist.
     auto paged_off = [&](int p) {
@@ -171,9 +164,8 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
     };
     auto fetch = [&](int kt) {
         if constexpr (PAGED) {
-            if (a.block_shift >= 2 && kt + kPfKeys <= n_keys) {
-                // a whole tile of needed keys, pages of 4 * 2^n positions: shifts instead of divisions, no clamping, and
-                // the four consecutive keys of a V task share a page
+            if (a.block_shift >= 0 && kt + kPfKeys <= n_keys) {
+                // a whole tile of needed keys, pages of 2^n positions: shifts instead of divisions, no clamping
                 const int mask = a.block_size - 1;
                 auto off = [&](int p) {
                     const int pg = p >> a.block_shift;
@@ -184,51 +176,43 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
                 for (int i = 0; i < KCH; ++i) {
                     const int c = threadIdx.x + 256 * i;
                     const int key = c / CPR, dc = c - key * CPR;
-                    kreg[i] = *reinterpret_cast<const u32x4*>(Kb + off(kt + key) + dc * 8);
+                    const int64_t o = off(kt + key);
+                    kreg[i] = *reinterpret_cast<const u32x4*>(Kb + o + dc * 8);
+                    vreg[i] = *reinterpret_cast<const u32x4*>(Vb + o + dc * 8);
                 }
-                const bf16* vp = Vb + off(kt + 4 * v_kg) + v_dc * 8;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) vreg[i] = *reinterpret_cast<const u32x4*>(vp + i * a.pos_stride);
             } else {
 #pragma unroll
                 for (int i = 0; i < KCH; ++i) {
                     const int c = threadIdx.x + 256 * i;
                     const int key = c / CPR, dc = c - key * CPR;
-                    kreg[i] = *reinterpret_cast<const u32x4*>(Kb + paged_off(kt + key) + dc * 8);
+                    const int64_t o = paged_off(kt + key);
+                    kreg[i] = *reinterpret_cast<const u32x4*>(Kb + o + dc * 8);
+                    vreg[i] = *reinterpret_cast<const u32x4*>(Vb + o + dc * 8);
                 }
-#pragma unroll
-                for (int i = 0; i < 4; ++i) vreg[i] = *reinterpret_cast<const u32x4*>(Vb + paged_off(kt + 4 * v_kg + i) + v_dc * 8);
             }
         } else if (kt + kPfKeys <= a.t_max) {
 #pragma unroll
             for (int i = 0; i < KCH; ++i) kreg[i] = *reinterpret_cast<const u32x4*>(k_src + (int64_t)kt * HD + 2048 * i);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) vreg[i] = *reinterpret_cast<const u32x4*>(v_src + (int64_t)kt * HD + i * HD);
+            for (int i = 0; i < KCH; ++i) vreg[i] = *reinterpret_cast<const u32x4*>(v_src + (int64_t)kt * HD + 2048 * i);
         } else {  // the cache ends inside this tile: rows past it are masked below, their loads stay in bounds
 #pragma unroll
             for (int i = 0; i < KCH; ++i) {
                 const int c = threadIdx.x + 256 * i;
                 const int key = c / CPR, dc = c - key * CPR;
-                kreg[i] = *reinterpret_cast<const u32x4*>(Kb + (int64_t)min(kt + key, a.t_max - 1) * HD + dc * 8);
+                const int64_t o = (int64_t)min(kt + key, a.t_max - 1) * HD + dc * 8;
+                kreg[i] = *reinterpret_cast<const u32x4*>(Kb + o);
+                vreg[i] = *reinterpret_cast<const u32x4*>(Vb + o);
             }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                vreg[i] = *reinterpret_cast<const u32x4*>(Vb + (int64_t)min(kt + 4 * v_kg + i, a.t_max - 1) * HD + v_dc * 8);
         }
     };
     auto park = [&](int buf) {
         bf16* kb = &sk[buf][0][0];
 #pragma unroll
         for (int i = 0; i < KCH; ++i) *reinterpret_cast<u32x4*>(kb + k_dst[i]) = kreg[i];
-        bf16* vb = &svt[buf][0][0] + v_dst;
+        bf16* vb = &sv[buf][0][0];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {  // 32-bit word e of the four chunks holds columns 2e, 2e+1
-            const unsigned w0 = vreg[0][e], w1 = vreg[1][e], w2 = vreg[2][e], w3 = vreg[3][e];
-            const u32x2 even = {__builtin_amdgcn_perm(w1, w0, 0x05040100u), __builtin_amdgcn_perm(w3, w2, 0x05040100u)};
-            const u32x2 odd = {__builtin_amdgcn_perm(w1, w0, 0x07060302u), __builtin_amdgcn_perm(w3, w2, 0x07060302u)};
-            *reinterpret_cast<u32x2*>(vb + (2 * e) * kVtPitch) = even;
-            *reinterpret_cast<u32x2*>(vb + (2 * e + 1) * kVtPitch) = odd;
-        }
+        for (int i = 0; i < KCH; ++i) *reinterpret_cast<u32x4*>(vb + v_dst[i]) = vreg[i];
     };
 
     // One key tile against the wave's rows.  MASKED: some key of the tile is hidden from some row (the tiles on the
@@ -295,8 +279,16 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
         // row groups.  Three fragments are in flight (the first ones are requested before the exponentials), and the
         // exponentials of the second k-step sit between the products of the first; scheduling fences keep that order.
         constexpr int NF = 2 * NT;
+        // V fragment i, the B operand [32 key slots x 16 columns]: two transposing reads.  In each, lane l of a group of 16
+        // points at four columns (4 * (l % 4) ..+3 of the tile's 16) of key row l / 4 of four, and receives the four keys
+        // of column l % 16; the four keys are 4 * s4 ..+3 of sub-tile 2c (first read) and 2c + 1 (second), P's order.
+        typedef short s16x4 __attribute__((ext_vector_type(4)));
+        const bf16* vtr = &sv[buf][4 * s4 + (qc >> 2)][4 * (qc & 3)];
         auto vfrag = [&](int i) {
-            return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&svt[buf][16 * (i % NT) + qc][32 * (i / NT) + 8 * s4]));
+            const bf16* p0 = vtr + (32 * (i / NT)) * kVPitch + 16 * (i % NT);
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0 + 16 * kVPitch));
+            return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         };
         bf16x8 vf[3];
 #pragma unroll
