@@ -48,6 +48,8 @@ def parse():
     ap.add_argument("--prefill-len", type=int, default=4096)
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="launch-shape override passed to raven_set_tuning before the run (experiments only)")
+    ap.add_argument("--attention-only", type=int, default=0, metavar="N",
+                    help="with --prefill: run only N launches of the chunk attention kernel at that shape (for rocprofv3 --pmc runs)")
     ap.add_argument("--kernel-only", type=int, default=0, metavar="N",
                     help="run only N launches of the dominant kernel plus one 256 MiB device copy (for rocprofv3 --pmc runs)")
     return ap.parse_args()
@@ -227,6 +229,28 @@ def paged(args):
     print(json.dumps(line))
 
 
+def attention_only(args):
+    """The chunk attention kernel alone at the prefill shape (--prefill-batch sequences of --prefill-len rows, 55 heads of
+    96): synthetic q, K, V ~ N(0, 1) in a contiguous cache of one step slot; HIP events around --attention-only launches."""
+    import torch
+    import __graft_entry__ as entry
+    pkg = entry.import_package()
+    pkg.hip.load()
+    cfg = pkg.RavenConfig()
+    dev = torch.device("cuda:0")
+    B, S, nh, hd = args.prefill_batch, args.prefill_len, cfg.n_heads, cfg.head_dim
+    torch.manual_seed(0)
+    k = torch.randn(1, B, nh, S, hd, device=dev, dtype=torch.bfloat16)
+    v = torch.randn_like(k)
+    kv = pkg.hip.make_cache(k, v)
+    q = torch.randn(B * S, nh * hd, device=dev, dtype=torch.bfloat16)
+    ms = event_time_ms(lambda: pkg.hip.prefill_attention(q, kv, 0, B, S, 0, nh, hd), args.attention_only, warm=2)
+    flops = 4.0 * B * nh * hd * S * (S + 1) / 2
+    print(json.dumps({"attention_only": args.attention_only, "kernel": "attention_prefill_kernel", "batch": B, "seq_len": S,
+                      "ms_per_launch": round(ms, 4), "causal_flops_per_launch": flops, "TFLOP/s": round(flops / ms / 1e9, 1),
+                      "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4)}))
+
+
 def kernel_only(n_launches):
     """The dominant kernel alone, as the decode loop launches it, on four rotating fc matrices, followed by
     one device copy of known size (the yardstick that scales FETCH_SIZE / WRITE_SIZE readings)."""
@@ -322,6 +346,9 @@ def main():
     apply_tuning(args)
     if args.kernel_only:
         kernel_only(args.kernel_only)
+        return
+    if args.prefill and args.attention_only:
+        attention_only(args)
         return
     if args.prefill:
         prefill(args)
