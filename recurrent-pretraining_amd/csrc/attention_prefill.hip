@@ -31,7 +31,6 @@
 namespace raven {
 
 constexpr int kPfKeys = 64;     // keys per tile
-constexpr int kVPitch = 144;    // bf16 elements per V row in LDS (288 bytes = 72 banks: the 8 key rows that 32 lanes read transposed hit 64 different banks)
 
 struct PrefillArgs {
     const bf16* q;   // [B*S, h]
@@ -73,6 +72,9 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
     constexpr int WR = 16 * RG;      // query rows per wave
     constexpr int ROWS = 4 * WR;     // query rows per workgroup
     __shared__ __align__(16) bf16 sk[2][kPfKeys][KP];
+    // bf16 elements per V row in LDS: HD + 16, i.e. 40 / 56 / 72 banks -- an odd multiple of 8, so that the 8 key rows that
+    // 32 lanes read transposed (8 banks each) hit 64 different banks
+    constexpr int kVPitch = HD + 16;
     __shared__ __align__(16) bf16 sv[2][kPfKeys][kVPitch];
 
     const int qb = gridDim.x - 1 - blockIdx.x;  // the blocks with the most keys start first
