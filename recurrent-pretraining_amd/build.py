@@ -11,7 +11,7 @@ ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libraven_hip.so")
-SOURCES = ["rmsnorm.hip", "gemm_skinny.hip", "gemm_splitk.hip", "gemv_decode.hip", "attention.hip", "attention_prefill.hip", "misc.hip", "exit_stats.hip", "compose.hip"]
+SOURCES = ["rmsnorm.hip", "gemm_skinny.hip", "gemm_splitk.hip", "gemm_tiled.hip", "gemv_decode.hip", "attention.hip", "attention_prefill.hip", "misc.hip", "exit_stats.hip", "compose.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -25,6 +25,10 @@ namespace raven {
 
 int set_gemv1_tuning(const char* key, int value);
 extern int g_linear_ks;
+extern int g_tiled_min_rows, g_tiled_variant;
+bool tiled_gemm_fits(int M, int N, int K0, int K1, int dtype);
+int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residual, void* y, int M, int N, int K0, int K1, int swiglu,
+               int out_f32, hipStream_t s);
 extern int g_attn_split_target, g_attn_big_grid, g_attn_wide, g_linear_min_rows, g_attn_nosplit_pairs, g_rope_tiled_rows;
 
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
@@ -564,6 +568,8 @@ extern "C" int raven_set_tuning(const char* key, int32_t value) {
     else if (k == "rope_tiled_rows" && value > 0) g_rope_tiled_rows = value;
     else if (k == "attn_nosplit_pairs" && value > 0 && value <= 1024) g_attn_nosplit_pairs = value;
     else if (k == "linear_min_rows" && value >= 1) g_linear_min_rows = value;
+    else if (k == "gemm_tiled_min_rows" && value >= 33) g_tiled_min_rows = value;
+    else if (k == "gemm_tiled_variant" && value >= 0 && value <= 2) g_tiled_variant = value;
     else RAVEN_REQUIRE(set_gemv1_tuning(key, value) == 0, "set_tuning: unknown key %s", key);
     return 0;
 }
@@ -574,6 +580,8 @@ extern "C" int raven_gemm(const void* x, const void* w, const void* residual, vo
     if (int rc = check_common("gemm", M, N, K, dtype)) return rc;
     if (M == 0) return 0;
     RAVEN_REQUIRE(x && w && y, "gemm: null pointer");
+    if (M >= g_tiled_min_rows && tiled_gemm_fits(M, N, K, 0, dtype))
+        return tiled_gemm(x, nullptr, w, residual, y, M, N, K, 0, 0, out_f32, static_cast<hipStream_t>(stream));
     GemmArgs a{};
     a.w = w; a.x0 = x; a.x1 = nullptr; a.residual = residual; a.y = y;
     a.M = M; a.N = N; a.K = K; a.k0 = K; a.k1 = 0; a.out_f32 = out_f32;
@@ -588,7 +596,8 @@ extern "C" int raven_adapter_gemm_concat(const void* x0, const void* x1, const v
     RAVEN_REQUIRE(x0 && x1 && w && y, "adapter: null pointer");
     const int elts = 16 / (int)raven_host::elt_size(dtype);
     RAVEN_REQUIRE(K0 > 0 && K1 > 0 && K0 % elts == 0 && K1 % elts == 0, "adapter: K0=%d, K1=%d must be positive multiples of %d", K0, K1, elts);
-    if (M == 0) return 0;
+    if (M >= g_tiled_min_rows && tiled_gemm_fits(M, N, K0, K1, dtype))
+        return tiled_gemm(x0, x1, w, nullptr, y, M, N, K0, K1, 0, 0, static_cast<hipStream_t>(stream));
     GemmArgs a{};
     a.w = w; a.x0 = x0; a.x1 = x1; a.residual = nullptr; a.y = y;
     a.M = M; a.N = N; a.K = K0 + K1; a.k0 = K0; a.k1 = K1; a.out_f32 = 0;
@@ -601,6 +610,8 @@ extern "C" int raven_gemm_swiglu(const void* x, const void* fc, void* out, int32
     if (int rc = check_common("gemm_swiglu", M, I, K, dtype)) return rc;
     if (M == 0) return 0;
     RAVEN_REQUIRE(x && fc && out, "gemm_swiglu: null pointer");
+    if (M >= g_tiled_min_rows && tiled_gemm_fits(M, I, K, 0, dtype))
+        return tiled_gemm(x, nullptr, fc, nullptr, out, M, I, K, 0, 1, 0, static_cast<hipStream_t>(stream));
     GemmArgs a{};
     a.w = fc; a.x0 = x; a.x1 = nullptr; a.residual = nullptr; a.y = out;
     a.M = M; a.N = I; a.K = K; a.k0 = K; a.k1 = 0; a.out_f32 = 0;

@@ -26,6 +26,11 @@ extern "C" int raven_gemm_swiglu(const void* x, const void* fc, void* out, int32
 
 namespace raven {
 
+extern int g_tiled_min_rows;
+bool tiled_gemm_fits(int M, int N, int K0, int K1, int dtype);
+int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residual, void* y, int M, int N, int K0, int K1, int swiglu,
+               int out_f32, hipStream_t s);
+
 constexpr int kNsPitch = 136;  // bf16 elements per LDS row: 128 + 8 (272 bytes)
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
@@ -321,6 +326,8 @@ extern "C" int raven_linear(const void* x0, const void* x1, const void* w, const
     RAVEN_REQUIRE((K1 == 0) == (x1 == nullptr), "linear: x1 and K1 must be given together");
     RAVEN_REQUIRE(!(swiglu && (residual || out_f32 || K1)), "linear: the SwiGLU epilogue takes one operand, no residual, and stores T");
     RAVEN_REQUIRE(!(K1 && (residual || out_f32)), "linear: the two-operand form has a plain epilogue");
+    if (M >= g_tiled_min_rows && tiled_gemm_fits(M, N, K0, K1, dtype))  // many rows: tiles of the whole product on the matrix cores
+        return tiled_gemm(x0, x1, w, residual, y, M, N, K0, K1, swiglu, out_f32, static_cast<hipStream_t>(stream));
     bool fits = dtype == RAVEN_BF16 && M > g_linear_min_rows && N % 16 == 0 && K0 % 32 == 0 && K1 % 32 == 0 && workspace != nullptr &&
                 ((uintptr_t)workspace & 255) == 0 && K0 / 128 + K1 / 128 >= 1;
     // Matrices with many rows give the kernel without a workspace enough workgroups and it is then the faster one
