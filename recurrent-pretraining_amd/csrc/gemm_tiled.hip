@@ -45,6 +45,7 @@ struct TiledArgs {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) unsigned char lds_byte;
+typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
 
 template <int... I, typename F>
 __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
@@ -53,13 +54,6 @@ __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>
 template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
-}
-
-// LDS read that the compiler does not see as one: it would otherwise order every such read behind all outstanding
-// global -> LDS loads.  The result is valid after wait_lds().
-template <int OFF>
-__device__ __forceinline__ void lds_read16(u32x4& dst, unsigned addr) {
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
 
 // Epilogue of both kernels.  A lane holds, for token row m = .. + l32, output columns 8 j + 4 hi + (0 .. 3) of each
@@ -118,17 +112,16 @@ __device__ __forceinline__ void store_tiles(const TiledArgs& a, const f32x16 (&a
 
 __device__ __align__(16) unsigned int g_zero_piece[4];  // what a 16-byte piece past the end of K is loaded from
 
-template <bool SWIGLU, int TM, int TN, int EXP = 0, int PFD = 0>
+template <bool SWIGLU, int TM, int TN, int EXP = 0>
 __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
     constexpr int BM = 2 * TM * 32, BN = 4 * TN * 32;
     constexpr int ROWS = BN + BM;              // LDS rows of a stage: the W tile, then the X tile
     constexpr int STAGE_BYTES = ROWS * 128;
-    constexpr int LPW = ROWS / 8 / 8;          // global -> LDS instructions (8 rows each) per wave and stage
-    static_assert(ROWS % 64 == 0 && (BN / 8) % LPW == 0 && LPW % 2 == 0, "a wave loads rows of one operand only");
+    constexpr int LPW = ROWS / 8 / 8;          // 16-byte pieces per lane and step: piece p of a wave = 8 rows x 128 bytes
+    static_assert(ROWS % 256 == 0 && (BN / 8) % LPW == 0, "a wave loads rows of one operand only, the same number under every k-slice");
     constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
     constexpr int NM = TN * TM;                // MFMAs per k-slice
-    // the loads of a step are issued in three portions, under the products of three k-slices
-    constexpr int P0 = (LPW * 3 + 7) / 8, P1 = (LPW * 6 + 7) / 8;
+    constexpr int PPS = LPW / 4;               // pieces handled under the products of one k-slice
     extern __shared__ __align__(1024) unsigned char smem[];
 
     // ---- which tile -----------------------------------------------------------------------------------------------
@@ -150,105 +143,74 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
     const int K = a.K0 + a.K1;
     const int nk = (K + 63) >> 6;
 
-    // ---- global -> LDS: this wave fills rows (wave * LPW + jj) * 8 ..+7 of every stage -------------------------------
+    // ---- global -> registers -> LDS: this wave moves rows (wave * LPW + p) * 8 ..+7 of every stage, piece p = one
+    // instruction; lane l brings bytes 16 (l & 7) ..+15 of the 128-byte row step of row l >> 3 --------------------------
     const bool loads_w = wave * LPW < BN / 8;
-    int rowidx[LPW];
+    const int col8 = (lane & 7) * 8;           // this lane's column inside a step, in elements
+    unsigned goff[LPW];                        // byte offset of this lane's row + column inside its operand (both segments
+                                               // of the token rows have one row pitch)
+    const unsigned ld2 = 2u * (loads_w ? K : a.K0);
 #pragma unroll
-    for (int jj = 0; jj < LPW; ++jj) {
-        const int r = (wave * LPW + jj) * 8 + (lane >> 3);
+    for (int p = 0; p < LPW; ++p) {
+        const int r = (wave * LPW + p) * 8 + (lane >> 3);
+        int row;
         if (loads_w) {
-            if (SWIGLU) {
-                const int col = min(tile_n * BN_OUT + (r >> 5) * 16 + (r & 15), a.N - 1);
-                rowidx[jj] = col + ((r & 16) ? a.N : 0);
-            } else {
-                rowidx[jj] = min(tile_n * BN + r, a.N - 1);
-            }
+            if (SWIGLU) row = min(tile_n * BN_OUT + (r >> 5) * 16 + (r & 15), a.N - 1) + ((r & 16) ? a.N : 0);
+            else row = min(tile_n * BN + r, a.N - 1);
         } else {
-            rowidx[jj] = min(tile_m * BM + (r - BN), a.M - 1);
+            row = min(tile_m * BM + (r - BN), a.M - 1);
         }
+        goff[p] = (unsigned)row * ld2 + 2u * col8;
     }
-    // column (in elements) of the piece this lane fetches, for instructions of even / odd index: slot (lane & 7) of row
-    // r holds piece (lane & 7) ^ ((r >> 1) & 7)
-    int pcol[2];
+    // LDS slot of the piece: row r keeps piece c at position c ^ ((r >> 1) & 7); (r >> 1) & 7 = (lane >> 4) | 4 (p & 1)
+    const unsigned lds_base = (unsigned)(uintptr_t)(lds_byte*)smem;
+    unsigned wr_addr[2];
 #pragma unroll
-    for (int par = 0; par < 2; ++par) pcol[par] = ((lane & 7) ^ ((4 * par) | (lane >> 4))) * 8;
-    lds_byte* const lds0 = (lds_byte*)smem;
-    const bf16* const zero = reinterpret_cast<const bf16*>(g_zero_piece);
-    // where a step's pieces come from: when the whole step lies inside one segment, one base pointer for all lanes
-    // and a 32-bit offset per lane
+    for (int par = 0; par < 2; ++par)
+        wr_addr[par] = lds_base + (wave * LPW * 8 + (lane >> 3)) * 128 + (((lane & 7) ^ ((lane >> 4) | (4 * par))) * 16);
+    const char* const zero = reinterpret_cast<const char*>(g_zero_piece);
+    const char* const seg0 = reinterpret_cast<const char*>(loads_w ? a.w : a.x0);
+    const char* const seg1 = reinterpret_cast<const char*>(a.x1) - 2 * (int64_t)a.K0;  // column c >= K0 of the token rows
+    const int k_split = loads_w ? K : a.K0;    // columns from here on come from the second segment
+
+    // Plain loads and stores, and no branch inside the K loop: the compiler then knows the order of all outstanding loads
+    // and waits, in front of the LDS write of a piece, for exactly that piece's load (issued one step earlier).
+    // Where this lane's 16 bytes of step kk come from: its segment's pointer (rebased so that the piece's offset is
+    // goff[p] + 2 * 64 kk), or the zero page for columns past K -- which is every column of a step past the last one.
     struct StepSrc {
         const char* base;
-        unsigned ld2;  // row pitch in bytes
-        int kk;
-        bool uniform, live;
+        bool past;  // this lane's column lies past K
     };
     auto step_src = [&](int kk) {
+        const int col = (kk << 6) + col8;
         StepSrc s;
-        const int k0 = kk << 6;
-        s.kk = kk;
-        s.live = kk < nk;
-        s.uniform = loads_w ? (k0 + 64 <= K) : (k0 + 64 <= a.K0 || (k0 >= a.K0 && k0 + 64 <= K));
-        if (loads_w) { s.base = reinterpret_cast<const char*>(a.w + k0); s.ld2 = 2u * K; }
-        else if (k0 < a.K0) { s.base = reinterpret_cast<const char*>(a.x0 + k0); s.ld2 = 2u * a.K0; }
-        else { s.base = reinterpret_cast<const char*>(a.x1 + (k0 - a.K0)); s.ld2 = 2u * a.K1; }
+        s.past = col >= K;
+        s.base = s.past ? zero : (col < k_split ? seg0 : seg1) + 2 * (kk << 6);
         return s;
     };
-    // one instruction: piece jj of a step into stage kk & 1
-    auto issue = [&](const StepSrc& s, auto jj_tag) {
-        constexpr int jj = decltype(jj_tag)::value;
-        if ((EXP & 2) || !s.live) return;
-        lds_byte* dst = lds0 + (s.kk & 1) * STAGE_BYTES + wave * (LPW * 1024) + jj * 1024;
-        if (s.uniform) {
-            const unsigned off = __umul24((unsigned)rowidx[jj], s.ld2) + 2u * pcol[jj & 1];
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(s.base + off), dst, 16, 0, 0);
-        } else {
-            const int col = (s.kk << 6) + pcol[jj & 1];
-            const bool second = !loads_w && col >= a.K0;
-            const bf16* b = loads_w ? a.w : (second ? a.x1 : a.x0);
-            const int ld = loads_w ? K : (second ? a.K1 : a.K0);
-            const bf16* src = b + ((int64_t)rowidx[jj] * ld + (second ? col - a.K0 : col));
-            if (col >= K) src = zero;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src, dst, 16, 0, 0);
-        }
+    u32x4 stg[LPW];
+    auto load_piece = [&](const StepSrc& src, auto p_tag) {
+        constexpr int p = decltype(p_tag)::value;
+        if (EXP & 2) return;
+        stg[p] = *reinterpret_cast<const u32x4*>(src.base + (src.past ? 0u : goff[p]));
     };
-
-    // ---- L2 prefetch (PFD > 0): PFD steps beyond the loads, one lane touches one 128-byte line.  The workgroups that run
-    // together on an XCD share panels (8 token-row tiles per weight panel, 4 weight tiles per token-row panel): each of
-    // them touches its share of the lines, wave 0 of the weight panel, wave 4 of the token-row panel.
-    const bool does_pf = PFD > 0 && (wave == 0 || wave == 4);
-    const char* pf_ptr = nullptr;
-    bool pf_lane = false;
-    if (PFD > 0) {
-        if (wave == 0) {
-            const int r = (tile_m & 7) * (BN / 8) + lane;
-            pf_lane = lane < BN / 8;
-            int g;
-            if (SWIGLU) g = min(tile_n * BN_OUT + (r >> 5) * 16 + (r & 15), a.N - 1) + ((r & 16) ? a.N : 0);
-            else g = min(tile_n * BN + r, a.N - 1);
-            pf_ptr = reinterpret_cast<const char*>(a.w + (int64_t)g * K);
-        } else if (wave == 4) {
-            const int r = (tile_n & 3) * (BM / 4) + lane;
-            pf_lane = lane < BM / 4;
-            pf_ptr = reinterpret_cast<const char*>(a.x0 + (int64_t)min(tile_m * BM + r, a.M - 1) * a.K0);
-        }
-    }
-    lds_byte* const pf_dst = lds0 + 2 * STAGE_BYTES;
-    const int pf_limit = wave == 0 ? K : a.K0;  // the token-row operand is prefetched inside its first segment only
-    auto prefetch = [&](int kk) {  // always one instruction, so that the count of outstanding loads stays uniform
-        int k0 = kk << 6;
-        if (kk >= nk || k0 + 64 > pf_limit) k0 = 0;
-        if (pf_lane) __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(pf_ptr + 2 * k0), pf_dst, 4, 0, 0);
+    auto store_piece = [&](int kk, auto p_tag) {
+        constexpr int p = decltype(p_tag)::value;
+        if (EXP & 2) return;
+        *reinterpret_cast<lds_u32x4*>(wr_addr[p & 1] + (kk & 1) * STAGE_BYTES + p * 1024) = stg[p];
+    };
+    // Piece p of step j moves on: into stage j & 1; the registers take the piece of step j + 1 (source: next).
+    auto move_piece = [&](int j, const StepSrc& next, auto p_tag) {
+        store_piece(j, p_tag);
+        load_piece(next, p_tag);
     };
 
     // ---- LDS -> registers -------------------------------------------------------------------------------------------
     const int l32 = lane & 31, hi = lane >> 5;
     const int swz = (l32 >> 1) & 7;
-    const unsigned lds_base = (unsigned)(uintptr_t)lds0;
     const unsigned a_row = lds_base + (wn * TN * 32 + l32) * 128;
     const unsigned b_row = lds_base + (BN + wm * TM * 32 + l32) * 128;
-    unsigned pos[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) pos[ks] = ((2 * ks + hi) ^ swz) * 16;
+    const unsigned pos0 = (hi ^ swz) * 16;     // position of k-slice ks: pos0 ^ (32 ks)
 
     f32x16 acc[TN][TM];
 #pragma unroll
@@ -262,15 +224,11 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
     auto read_frags = [&](auto ks_tag, int buf) {  // k-slice ks of stage buf into fragment set ks & 1
         constexpr int ks = decltype(ks_tag)::value;
         if (EXP & 4) return;
-        const unsigned off = buf * STAGE_BYTES + pos[ks];
-        static_for<TN>([&](auto t) { lds_read16<decltype(t)::value * 4096>(fa[ks & 1][decltype(t)::value], a_row + off); });
-        static_for<TM>([&](auto t) { lds_read16<decltype(t)::value * 4096>(fb[ks & 1][decltype(t)::value], b_row + off); });
-    };
-    auto settle = [&](int set) {  // the fragments of this set are valid from here on (behind a wait for the LDS counter)
+        const unsigned off = buf * STAGE_BYTES + (pos0 ^ (32 * ks));
 #pragma unroll
-        for (int t = 0; t < TN; ++t) asm volatile("" : "+v"(fa[set][t]));
+        for (int t = 0; t < TN; ++t) fa[ks & 1][t] = *reinterpret_cast<const lds_u32x4*>(a_row + off + t * 4096);
 #pragma unroll
-        for (int t = 0; t < TM; ++t) asm volatile("" : "+v"(fb[set][t]));
+        for (int t = 0; t < TM; ++t) fb[ks & 1][t] = *reinterpret_cast<const lds_u32x4*>(b_row + off + t * 4096);
     };
     // the NM products of one k-slice; after(i) is called behind product i
     auto products = [&](int set, auto&& after) {
@@ -284,81 +242,72 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
             __builtin_amdgcn_sched_barrier(0);
         });
     };
-    // portion [LO, HI) of the loads of step kk, spread behind the products 1, 3, 5, ... of a slice
-    auto spread = [&](auto it, const StepSrc& src, auto lo_tag, auto hi_tag) {
-        constexpr int i = decltype(it)::value, LO = decltype(lo_tag)::value, HI = decltype(hi_tag)::value;
-        static_for<HI - LO>([&](auto p) {
-            constexpr int slot = 1 + 2 * decltype(p)::value < NM - 1 ? 1 + 2 * decltype(p)::value : NM - 1;
-            if (slot == i) issue(src, std::integral_constant<int, LO + decltype(p)::value>{});
+    // pieces FIRST .. FIRST + PPS - 1 of step j, behind products 1, 1 + NM / PPS, ... of a slice
+    auto move_under = [&](auto it, int j, const StepSrc& next, auto first_tag) {
+        constexpr int i = decltype(it)::value, FIRST = decltype(first_tag)::value;
+        static_for<PPS>([&](auto q) {
+            constexpr int slot = 1 + decltype(q)::value * (NM / PPS) < NM - 1 ? 1 + decltype(q)::value * (NM / PPS) : NM - 1;
+            if (slot == i) move_piece(j, next, std::integral_constant<int, FIRST + decltype(q)::value>{});
         });
     };
     using ic0 = std::integral_constant<int, 0>;
 
-    // ---- the K loop: two stages, one barrier per step -----------------------------------------------------------------
-    // Step k is multiplied out of stage k & 1 in four k-slices of 16.  The barrier of step k sits between the products
-    // of slices 2 and 3: in front of it every wave has all fragments of the step in registers and its loads of step k + 1
-    // have landed, so behind it stage k & 1 may be overwritten (loads of step k + 2: a first portion under the products
-    // of slice 3, the rest under slices 0 and 1 of the next step) and stage (k + 1) & 1 may be read.
-    StepSrc src1 = step_src(0), src2 = step_src(1);  // inside the loop: the sources of steps k + 1 and k + 2
-    static_for<LPW>([&](auto jj) { issue(src1, jj); });
-    if (1 < nk) {
-        static_for<P0>([&](auto jj) { issue(src2, jj); });
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(P0) : "memory");
-    } else {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // ---- the K loop: two LDS stages and one set of staging registers, one barrier per step --------------------------
+    // Step k is multiplied out of stage k & 1 in four k-slices of 16.  The barrier of step k sits between the products of
+    // slices 2 and 3: in front of it every wave has all fragments of step k in registers and has written its pieces of
+    // step k + 1; behind it stage k & 1 is free for step k + 2 and stage (k + 1) & 1 may be read.  Every piece goes round
+    // once per step: under slice 3 of step k the pieces 0 .. PPS - 1 of step k + 2 are written and reloaded for step
+    // k + 3, under slices 0 .. 2 of the next step the others -- each load has a whole step to land and the loads flow
+    // evenly.
+    {
+        const StepSrc s0 = step_src(0), s1 = step_src(1), s2 = step_src(2);
+        static_for<LPW>([&](auto p) { load_piece(s0, p); });
+        static_for<LPW>([&](auto p) { move_piece(0, s1, p); });
+        static_for<PPS>([&](auto p) { move_piece(1, s2, p); });  // as under slice 3 of a step in front of the first
     }
+    if (EXP & 4) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int t = 0; t < TN; ++t) fa[ks][t] = u32x4{0, 0, 0, 0};
+#pragma unroll
+            for (int t = 0; t < TM; ++t) fb[ks][t] = u32x4{0, 0, 0, 0};
+        }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
-    if (does_pf) prefetch(2);  // from here on a prefetch is this wave's youngest load at every wait
+    asm volatile("" ::: "memory");
     unsigned long long dbg_vm = 0, dbg_bar = 0, dbg_t0 = 0;
     unsigned long long dbg_r0 = 0;
     if (EXP & 64) { dbg_t0 = __builtin_readcyclecounter(); dbg_r0 = __builtin_amdgcn_s_memrealtime(); }
     read_frags(ic0{}, 0);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    settle(0);
     for (int k = 0; k < nk; ++k) {
         const int cur = k & 1;
-        src1 = src2;
-        src2 = step_src(k + 2);
+        const StepSrc src2 = step_src(k + 2), src3 = step_src(k + 3);
         static_for<3>([&](auto ks_tag) {
             constexpr int ks = decltype(ks_tag)::value;
             products(ks & 1, [&](auto it) {
                 if (decltype(it)::value == 0) read_frags(std::integral_constant<int, ks + 1>{}, cur);
-                if (ks == 0) spread(it, src1, std::integral_constant<int, P0>{}, std::integral_constant<int, P1>{});
-                if (ks == 1) {
-                    spread(it, src1, std::integral_constant<int, P1>{}, std::integral_constant<int, LPW>{});
-                    if (decltype(it)::value == NM - 1 && does_pf) prefetch(k + 2 + PFD);
-                }
+                move_under(it, k + 1, src2, std::integral_constant<int, PPS * (ks + 1)>{});
             });
-            if (ks < 2) {
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                settle((ks + 1) & 1);
-            }
         });
-        unsigned long long t0 = 0, t1 = 0, t2 = 0;
-        if (EXP & 64) {
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            t0 = __builtin_readcyclecounter();
-        }
-        if (does_pf) asm volatile("s_waitcnt vmcnt(1) lgkmcnt(0)" ::: "memory");  // the prefetch issued last may still be out
-        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        settle(1);
+        unsigned long long t1 = 0, t2 = 0;
+        // every LDS write of step k + 1 and every read of step k has completed in front of the barrier
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (EXP & 64) t1 = __builtin_readcyclecounter();
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
+        asm volatile("" ::: "memory");
         if (EXP & 64) {
             t2 = __builtin_readcyclecounter();
-            dbg_vm += t1 - t0;
             dbg_bar += t2 - t1;
         }
         products(1, [&](auto it) {
-            if (decltype(it)::value == 0 && k + 1 < nk) read_frags(ic0{}, cur ^ 1);
-            spread(it, src2, ic0{}, std::integral_constant<int, P0>{});
+            if (decltype(it)::value == 0) read_frags(ic0{}, cur ^ 1);  // behind the last step: zeros, not used
+            move_under(it, k + 2, src3, ic0{});
         });
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        settle(0);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if ((EXP & 64) && a.dbg && lane == 0 && blockIdx.x < 64) {
         unsigned long long* d = a.dbg + ((size_t)blockIdx.x * 8 + wave) * 4;
         d[0] = __builtin_readcyclecounter() - dbg_t0;
@@ -373,13 +322,13 @@ int g_tiled_min_rows = 33;  // raven_set_tuning("gemm_tiled_min_rows"): fewest r
 int g_tiled_variant = 0;    // raven_set_tuning("gemm_tiled_variant"): 0 = by shape, 1 = 256 x 256 tiles, 2 = 128 x 128 tiles
 int g_tiled_exp = 0;
 
-template <bool SWIGLU, int TM, int TN, int EXP = 0, int PFD = 0>
+template <bool SWIGLU, int TM, int TN, int EXP = 0>
 static int launch_tiled(TiledArgs a, hipStream_t s) {
     constexpr int BM = 2 * TM * 32, BN = 4 * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
-    constexpr size_t lds = (size_t)2 * (BM + BN) * 128 + 256;
+    constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<SWIGLU, TM, TN, EXP, PFD>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<SWIGLU, TM, TN, EXP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) {
             raven_host::set_error("gemm (tiled): hipFuncSetAttribute failed: %s", hipGetErrorString(e));
             return (int)e;
@@ -391,13 +340,13 @@ static int launch_tiled(TiledArgs a, hipStream_t s) {
     const int64_t n_tiles = (int64_t)a.tiles_m * a.tiles_n;
     RAVEN_REQUIRE(n_tiles < (1 << 28), "gemm (tiled): too many tiles (M=%d N=%d)", a.M, a.N);
     const unsigned grid = (unsigned)((n_tiles + 7) / 8 * 8);
-    gemm_tiled_kernel<SWIGLU, TM, TN, EXP, PFD><<<dim3(grid), dim3(512), lds, s>>>(a);
+    gemm_tiled_kernel<SWIGLU, TM, TN, EXP><<<dim3(grid), dim3(512), lds, s>>>(a);
     return raven_host::check_launch("gemm (tiled MFMA)");
 }
 
 // Host entry for the other translation units: true when the shape is one the tiled kernel takes.
 bool tiled_gemm_fits(int M, int N, int K0, int K1, int dtype) {
-    return dtype == RAVEN_BF16 && M >= 1 && N % 8 == 0 && K0 % 8 == 0 && K1 % 8 == 0 && K0 > 0 && (int64_t)M * (K0 > K1 ? K0 : K1) < (1ll << 31) &&
+    return dtype == RAVEN_BF16 && M >= 1 && N % 8 == 0 && K0 % 8 == 0 && K0 > 0 && (K1 == 0 || K1 == K0) && (int64_t)M * (K0 > K1 ? K0 : K1) < (1ll << 31) &&
            (int64_t)N * 2 * (K0 + K1) < (1ll << 31);
 }
 
@@ -430,8 +379,6 @@ int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residu
             case 66: return launch_tiled<false, 4, 2, 66>(a, s);
             case 70: return launch_tiled<false, 4, 2, 70>(a, s);
             case 76: return launch_tiled<false, 4, 2, 76>(a, s);
-            case 103: return launch_tiled<false, 4, 2, 0, 3>(a, s);
-            case 167: return launch_tiled<false, 4, 2, 64, 3>(a, s);
         }
     }
     if (swiglu) return big ? launch_tiled<true, 4, 2>(a, s) : launch_tiled<true, 2, 1>(a, s);
