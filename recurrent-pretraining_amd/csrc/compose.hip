@@ -9,7 +9,9 @@
 //     mlp.fc), the residual adds ride in the proj / mlp.proj epilogues, bias + RoPE + cache append ride in
 //     the attention kernel; one closing norm_4 (+ ln_f) launch per call.
 //   several rows: the residual adds still ride in the GEMM epilogues, norm_2 + norm_3 are one launch, and
-//     inside an iteration norm_4 of one block and norm_1 of the next are one launch.
+//     inside an iteration norm_4 of one block and norm_1 of the next are one launch.  From 33 rows on the five
+//     products are tiles on the matrix cores (SwiGLU and the residual adds in their epilogues, the adapter's two
+//     operands as two K segments), and chunks of 16 or more rows per sequence attend through the MFMA kernel.
 
 #include "raven_common.h"
 
@@ -108,8 +110,13 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
     } else {       // a chunk of S tokens: every row's keys must be in the cache before any row attends
         if ((rc = raven_qkv_bias_rope_cache_append(s.qkv, w->qk_bias, freqs, s.q, cache, slot, B, S, pos0, pos_dev, d->n_heads,
                                                    d->head_dim, dt, stream))) return rc;
-        if ((rc = raven_decode_attention(s.q, s.ya, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, s.attn_ws,
-                                         s.attn_ws_bytes, stream))) return rc;
+        // chunks of 16 or more rows per sequence: 64 or 128 query rows of a head per workgroup on the matrix cores; a few
+        // rows per sequence (or a partially filled cache, which only that kernel looks up): one row at a time
+        const bool mfma = dt == RAVEN_BF16 && S >= 16 && (d->head_dim == 64 || d->head_dim == 96 || d->head_dim == 128) &&
+                          (cache->steps_present == nullptr || cache->lookup_mode == RAVEN_LOOKUP_NONE);
+        if (mfma) rc = raven_prefill_attention(s.q, s.ya, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, stream);
+        else rc = raven_decode_attention(s.q, s.ya, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream);
+        if (rc) return rc;
     }
     if ((rc = raven_linear(s.ya, nullptr, w->proj, x_in, s.x1, M, h, h, 0, 0, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
     if ((rc = raven_rmsnorm_residual(s.x1, nullptr, w->norm_2, s.x2, nullptr, w->norm_3, s.n3, M, h, d->eps, dt, stream))) return rc;

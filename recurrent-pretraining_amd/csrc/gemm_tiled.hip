@@ -5,23 +5,27 @@
 // float store (RMM:711), SwiGLU (RMM:507-508).  The concat of RMM:776 is two K segments of the X operand.
 //
 // Shape of the kernel (gfx950):
-//   * a workgroup of 8 waves owns a BN x BM tile of Y^T (BN weight rows x BM token rows, 256 x 256 in the main
-//     variant); wave (wm, wn) owns TN x TM MFMA tiles of 32 x 32 (v_mfma_f32_32x32x16_bf16, W rows as the A operand, X
-//     rows as B, so that a lane ends up with 4 neighbouring output columns of one token row);
-//   * K advances in steps of 32 through a ring of LDS stages.  A stage holds BN + BM rows of 64 bytes; it is filled by
-//     global -> LDS loads that never touch registers (16 bytes per lane, a wave instruction fills 1 KB = 16 rows).
-//     The 16-byte pieces of a row are stored in an order permuted by the row number ((row >> 2) & 3), chosen on the
-//     global side of the load, so that the 16 lanes of a quarter wave, which read the same piece of 16 neighbouring
-//     rows, hit all 64 banks;
-//   * the waves work in two groups of four (one wave of each group per SIMD) half a step apart: while one group
-//     multiplies the fragments it holds, the other issues its loads for three steps ahead and reads its fragments of
-//     the next step out of LDS; two workgroup barriers per step keep the groups in that rhythm.  The matrix pipe of a
-//     SIMD then always has one wave that does nothing but MFMAs;
+//   * a workgroup of 8 waves (2 along the token rows x 4 along the weight rows, two waves per SIMD) owns a BN x BM tile
+//     of Y^T (256 weight rows x 256 token rows in the main variant); a wave owns TN x TM MFMA tiles of 32 x 32
+//     (v_mfma_f32_32x32x16_bf16, W rows as the A operand, X rows as B, so that a lane ends up with 4 neighbouring output
+//     columns of one token row);
+//   * K advances in steps of 64 through two LDS stages of BN + BM rows of 128 bytes.  The 16-byte pieces of a row are
+//     kept at position piece ^ ((row >> 1) & 7), so that the 16 lanes of a quarter wave, which read the same piece of 16
+//     neighbouring rows, hit all 64 banks;
+//   * operands travel global -> registers -> LDS: 8 lanes fetch one whole 128-byte row step (the L1 address path
+//     serves full lines at twice the rate of half lines), a wave instruction 8 rows.  Every lane keeps one step of its
+//     pieces in registers; a piece is written to LDS one step after it was requested and its registers are reloaded at
+//     once, two pieces under the products of each k-slice, so that loads flow evenly and each has a whole step to land;
+//   * a step is four k-slices of 16; fragments of the next slice are read from LDS under the products of this one.  One
+//     workgroup barrier per step, between the products of slices 2 and 3;
+//   * the K loop is one basic block of plain loads, stores and MFMAs with the scheduler pinned between them: the
+//     compiler then counts the outstanding loads exactly and waits for one piece at a time;
 //   * workgroups are numbered so that the 32 that run together on one XCD (ids congruent modulo 8) cover 8 x 4
-//     neighbouring tiles and find each other's panels in that XCD's L2.
-//   * SwiGLU: a 32-row A tile holds 16 gate rows and the 16 matching up rows, so gate and up of one output element
-//     sit in the same lane, 8 accumulator registers apart.
-// M, N and the last tile: rows past the end are clamped on the load side and not stored.  K0 and K1 are multiples of 32.
+//     neighbouring tiles and find each other's panels in that XCD's L2;
+//   * SwiGLU: a 32-row A tile holds 16 gate rows and the 16 matching up rows, so gate and up of one output element sit
+//     in the same lane, 8 accumulator registers apart.
+// M, N and the last tile: rows past the end are clamped on the load side and not stored.  K0 and K1 are multiples of 8
+// (pieces past K come from a zero page); two segments share one row pitch (K1 == K0).
 
 #include <type_traits>
 #include <utility>
@@ -39,7 +43,6 @@ struct TiledArgs {
     int M, N, K0, K1;      // N = output columns (I for SwiGLU)
     int out_f32;
     int tiles_m, tiles_n;
-    unsigned long long* dbg;  // experiments only
 };
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -112,7 +115,7 @@ __device__ __forceinline__ void store_tiles(const TiledArgs& a, const f32x16 (&a
 
 __device__ __align__(16) unsigned int g_zero_piece[4];  // what a 16-byte piece past the end of K is loaded from
 
-template <bool SWIGLU, int TM, int TN, int EXP = 0>
+template <bool SWIGLU, int TM, int TN>
 __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
     constexpr int BM = 2 * TM * 32, BN = 4 * TN * 32;
     constexpr int ROWS = BN + BM;              // LDS rows of a stage: the W tile, then the X tile
@@ -191,12 +194,10 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
     u32x4 stg[LPW];
     auto load_piece = [&](const StepSrc& src, auto p_tag) {
         constexpr int p = decltype(p_tag)::value;
-        if (EXP & 2) return;
         stg[p] = *reinterpret_cast<const u32x4*>(src.base + (src.past ? 0u : goff[p]));
     };
     auto store_piece = [&](int kk, auto p_tag) {
         constexpr int p = decltype(p_tag)::value;
-        if (EXP & 2) return;
         *reinterpret_cast<lds_u32x4*>(wr_addr[p & 1] + (kk & 1) * STAGE_BYTES + p * 1024) = stg[p];
     };
     // Piece p of step j moves on: into stage j & 1; the registers take the piece of step j + 1 (source: next).
@@ -223,7 +224,6 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
     u32x4 fa[2][TN], fb[2][TM];
     auto read_frags = [&](auto ks_tag, int buf) {  // k-slice ks of stage buf into fragment set ks & 1
         constexpr int ks = decltype(ks_tag)::value;
-        if (EXP & 4) return;
         const unsigned off = buf * STAGE_BYTES + (pos0 ^ (32 * ks));
 #pragma unroll
         for (int t = 0; t < TN; ++t) fa[ks & 1][t] = *reinterpret_cast<const lds_u32x4*>(a_row + off + t * 4096);
@@ -234,8 +234,7 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
     auto products = [&](int set, auto&& after) {
         static_for<NM>([&](auto it) {
             constexpr int i = decltype(it)::value, tn = i / TM, tm = i % TM;
-            if (!(EXP & 8))
-                acc[tn][tm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[set][tn]),
+            acc[tn][tm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[set][tn]),
                                                                       __builtin_bit_cast(bf16x8, fb[set][tm]), acc[tn][tm], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             after(it);
@@ -265,21 +264,9 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
         static_for<LPW>([&](auto p) { move_piece(0, s1, p); });
         static_for<PPS>([&](auto p) { move_piece(1, s2, p); });  // as under slice 3 of a step in front of the first
     }
-    if (EXP & 4) {
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-#pragma unroll
-            for (int t = 0; t < TN; ++t) fa[ks][t] = u32x4{0, 0, 0, 0};
-#pragma unroll
-            for (int t = 0; t < TM; ++t) fb[ks][t] = u32x4{0, 0, 0, 0};
-        }
-    }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    unsigned long long dbg_vm = 0, dbg_bar = 0, dbg_t0 = 0;
-    unsigned long long dbg_r0 = 0;
-    if (EXP & 64) { dbg_t0 = __builtin_readcyclecounter(); dbg_r0 = __builtin_amdgcn_s_memrealtime(); }
     read_frags(ic0{}, 0);
     for (int k = 0; k < nk; ++k) {
         const int cur = k & 1;
@@ -291,44 +278,30 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
                 move_under(it, k + 1, src2, std::integral_constant<int, PPS * (ks + 1)>{});
             });
         });
-        unsigned long long t1 = 0, t2 = 0;
         // every LDS write of step k + 1 and every read of step k has completed in front of the barrier
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (EXP & 64) t1 = __builtin_readcyclecounter();
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("" ::: "memory");
-        if (EXP & 64) {
-            t2 = __builtin_readcyclecounter();
-            dbg_bar += t2 - t1;
-        }
         products(1, [&](auto it) {
             if (decltype(it)::value == 0) read_frags(ic0{}, cur ^ 1);  // behind the last step: zeros, not used
             move_under(it, k + 2, src3, ic0{});
         });
-    }
-    if ((EXP & 64) && a.dbg && lane == 0 && blockIdx.x < 64) {
-        unsigned long long* d = a.dbg + ((size_t)blockIdx.x * 8 + wave) * 4;
-        d[0] = __builtin_readcyclecounter() - dbg_t0;
-        d[1] = dbg_vm;
-        d[2] = dbg_bar;
-        d[3] = ((unsigned long long)nk << 32) | (unsigned)(__builtin_amdgcn_s_memrealtime() - dbg_r0);
     }
     store_tiles<SWIGLU, TM, TN>(a, acc, tile_m, tile_n, wm, wn, l32, hi);
 }
 
 int g_tiled_min_rows = 33;  // raven_set_tuning("gemm_tiled_min_rows"): fewest rows that take this kernel
 int g_tiled_variant = 0;    // raven_set_tuning("gemm_tiled_variant"): 0 = by shape, 1 = 256 x 256 tiles, 2 = 128 x 128 tiles
-int g_tiled_exp = 0;
 
-template <bool SWIGLU, int TM, int TN, int EXP = 0>
+template <bool SWIGLU, int TM, int TN>
 static int launch_tiled(TiledArgs a, hipStream_t s) {
     constexpr int BM = 2 * TM * 32, BN = 4 * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
     constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<SWIGLU, TM, TN, EXP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<SWIGLU, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) {
             raven_host::set_error("gemm (tiled): hipFuncSetAttribute failed: %s", hipGetErrorString(e));
             return (int)e;
@@ -340,12 +313,16 @@ static int launch_tiled(TiledArgs a, hipStream_t s) {
     const int64_t n_tiles = (int64_t)a.tiles_m * a.tiles_n;
     RAVEN_REQUIRE(n_tiles < (1 << 28), "gemm (tiled): too many tiles (M=%d N=%d)", a.M, a.N);
     const unsigned grid = (unsigned)((n_tiles + 7) / 8 * 8);
-    gemm_tiled_kernel<SWIGLU, TM, TN, EXP><<<dim3(grid), dim3(512), lds, s>>>(a);
+    gemm_tiled_kernel<SWIGLU, TM, TN><<<dim3(grid), dim3(512), lds, s>>>(a);
     return raven_host::check_launch("gemm (tiled MFMA)");
 }
 
-// Host entry for the other translation units: true when the shape is one the tiled kernel takes.
+// Host entry for the other translation units: true when the shape is one the tiled kernel takes and is the better choice
+// for.  Few token rows against a matrix with few rows give too few tiles to fill the chip (there is no K split here):
+// up to 160 rows those go to the skinny kernels, 32 rows per pass over the weights.
 bool tiled_gemm_fits(int M, int N, int K0, int K1, int dtype) {
+    const int64_t small_tiles = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
+    if (g_tiled_variant == 0 && M <= 160 && small_tiles < 128) return false;
     return dtype == RAVEN_BF16 && M >= 1 && N % 8 == 0 && K0 % 8 == 0 && K0 > 0 && (K1 == 0 || K1 == K0) && (int64_t)M * (K0 > K1 ? K0 : K1) < (1ll << 31) &&
            (int64_t)N * 2 * (K0 + K1) < (1ll << 31);
 }
@@ -363,24 +340,9 @@ int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residu
     a.residual = static_cast<const bf16*>(residual);
     a.y = y;
     a.M = M; a.N = N; a.K0 = K0; a.K1 = x1 ? K1 : 0; a.out_f32 = out_f32;
-    a.dbg = (g_tiled_exp & 64) ? static_cast<unsigned long long*>(const_cast<void*>(residual)) : nullptr;
-    if (a.dbg) a.residual = nullptr;
     // 256 x 256 tiles when they fill the chip at least once; 128 x 128 tiles otherwise
     const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + (swiglu ? 127 : 255)) / (swiglu ? 128 : 256));
     const bool big = g_tiled_variant == 1 || (g_tiled_variant == 0 && big_tiles >= 256);
-    if (!swiglu && big && g_tiled_exp) {
-        switch (g_tiled_exp) {
-            case 2: return launch_tiled<false, 4, 2, 2>(a, s);
-            case 4: return launch_tiled<false, 4, 2, 4>(a, s);
-            case 6: return launch_tiled<false, 4, 2, 6>(a, s);
-            case 8: return launch_tiled<false, 4, 2, 8>(a, s);
-            case 12: return launch_tiled<false, 4, 2, 12>(a, s);
-            case 64: return launch_tiled<false, 4, 2, 64>(a, s);
-            case 66: return launch_tiled<false, 4, 2, 66>(a, s);
-            case 70: return launch_tiled<false, 4, 2, 70>(a, s);
-            case 76: return launch_tiled<false, 4, 2, 76>(a, s);
-        }
-    }
     if (swiglu) return big ? launch_tiled<true, 4, 2>(a, s) : launch_tiled<true, 2, 1>(a, s);
     return big ? launch_tiled<false, 4, 2>(a, s) : launch_tiled<false, 2, 1>(a, s);
 }

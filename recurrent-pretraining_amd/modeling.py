@@ -353,68 +353,12 @@ class RavenForCausalLM(torch.nn.Module):
             return int(num_steps[0]) + int(num_steps[1])
         return int(num_steps)
 
-    # ---- many rows (prefill): library GEMMs for the five nn.Linear products, HIP kernels for the rest ----
-    # From this many token rows on the five nn.Linear products go to hipBLASLt via torch.matmul: the skinny kernels take
-    # at most 32 rows per pass over the weights, and from the second pass on the library is faster (33 rows: 1.25 ms per
-    # recurrence against 1.39; 56 rows: 1.25 against 1.60; 24 rows: 1.10 against 0.82).
-    WIDE_ROWS = 33
-
-    def _is_wide(self, M: int) -> bool:
-        return self.dtype == torch.bfloat16 and M >= self.WIDE_ROWS and self.config.head_dim in (64, 96, 128)
-
-    def _wide_block(self, blk: "SandwichBlock", x: torch.Tensor, kv, slot: int, B: int, S: int, pos0: int,
-                    n1: Optional[torch.Tensor] = None, tail_w: Optional[torch.Tensor] = None, pos_dev: Optional[torch.Tensor] = None):
-        """One SandwichBlock (RMM:525-536) on [B*S, h] rows.  Returns (block output, tail) where tail is one more
-        RMSNorm (weight tail_w: the next block's norm_1, or ln_f) of the output, fused into the closing norm launch."""
-        cfg, eps = self.config, self.config.norm_eps
-        freqs = self._natives()["freqs"]
-        if n1 is None:
-            n1 = hip.rmsnorm_residual(x, blk.norm_1.weight, eps)[0]
-        qkv = torch.matmul(n1, blk.attn.Wqkv.weight.t())
-        bias = blk.attn.qk_bias if hasattr(blk.attn, "qk_bias") else None
-        if S == 1:   # one new row per sequence: bias, RoPE, cache append and attention in one launch
-            ya = hip.qkv_attention_decode(qkv, bias, freqs, kv, slot, B, pos0, cfg.n_heads, cfg.head_dim, pos_dev=pos_dev)
-        else:
-            q = hip.qkv_bias_rope_cache_append(qkv, bias, freqs, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim, pos_dev=pos_dev)
-            if S >= 16:  # chunks: the MFMA kernel (64 query rows of one sequence per workgroup)
-                ya = hip.prefill_attention(q, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim, pos_dev=pos_dev)
-            else:        # many sequences with a few rows each: the per-row kernel
-                ya = hip.decode_attention(q, kv, slot, B, S, pos0, cfg.n_heads, cfg.head_dim, pos_dev=pos_dev)
-        a = torch.matmul(ya, blk.attn.proj.weight.t())
-        x2, _, n3 = hip.rmsnorm_residual(a, blk.norm_2.weight, eps, residual=x, weight2=blk.norm_3.weight)
-        g = hip.swiglu(torch.matmul(n3, blk.mlp.fc.weight.t()))
-        m = torch.matmul(g, blk.mlp.proj.weight.t())
-        y, _, tail = hip.rmsnorm_residual(m, blk.norm_4.weight, eps, residual=x2, weight2=tail_w)
-        return y, tail
-
-    def _wide_core(self, x: torch.Tensor, embeds: torch.Tensor, slots, kv, B: int, S: int, pos0: int, ln_f: bool,
-                   pos_dev: Optional[torch.Tensor] = None):
-        """One core_block_forward (RMM:764-781) on many rows."""
-        t = self.transformer
-        cur = torch.matmul(torch.cat([x, embeds], dim=-1), t.adapter.weight.t())
-        n1, out = None, cur
-        n_core = len(t.core_block)
-        for j, blk in enumerate(t.core_block):
-            last = j == n_core - 1
-            tail_w = (t.ln_f.weight if ln_f else None) if last else t.core_block[j + 1].norm_1.weight
-            cur, tail = self._wide_block(blk, cur, kv, slots[j], B, S, pos0, n1=n1, tail_w=tail_w, pos_dev=pos_dev)
-            n1 = None if last else tail
-            out = tail if (last and ln_f) else cur
-        if n_core == 0 and ln_f:
-            out = hip.rmsnorm_residual(cur, t.ln_f.weight, self.config.norm_eps)[0]
-        return out
-
     # ---- pieces of the forward --------------------------------------------------------------------
     def _run_block(self, which: str, i: int, step_idx: int, x: torch.Tensor, cache: HuginnDynamicCache, private: bool,
                    B: int, S: int, pos0: int, ln_f: bool = False) -> torch.Tensor:
         nat = self._natives()
         slot = 0 if private else cache.note_append(step_idx, S, pos0)
         kv = cache.native() if private else cache.native([step_idx], pos0)
-        if self._is_wide(B * S) and kv.steps_present is None:
-            blk = getattr(self.transformer, {"prelude": "prelude", "coda": "coda", "core": "core_block"}[which])[i]
-            y, tail = self._wide_block(blk, x, kv, slot, B, S, pos0,
-                                       tail_w=self.transformer.ln_f.weight if ln_f else None)
-            return tail if ln_f else y
         out = torch.empty_like(x)
         hip.sandwich_block(nat["dims"], nat[which][i], x, out, nat["freqs"], kv, slot, B, S, pos0,
                            self._workspace(B * S), ln_f=self.transformer.ln_f.weight if ln_f else None)
@@ -467,8 +411,6 @@ class RavenForCausalLM(torch.nn.Module):
         gaps = [False] * n_core if private else [cache.has_gap(s_, pos0) for s_ in steps]
         uniform = all(g == gaps[0] for g in gaps)
         kv = cache.native() if private or not uniform else cache.native(steps, pos0)
-        if self._is_wide(B * S) and uniform and kv.steps_present is None:
-            return self._wide_core(x, embeds, slots, kv, B, S, pos0, ln_f)
         out = torch.empty_like(x)
         ws = self._workspace(B * S)
         lnw = t.ln_f.weight if ln_f else None
@@ -476,7 +418,7 @@ class RavenForCausalLM(torch.nn.Module):
             hip.core_iteration(nat["dims"], t.adapter.weight, nat["core"], x, embeds, out, nat["freqs"], kv,
                                slots[0], B, S, pos0, ws, ln_f=lnw)
             return out
-        cur = hip.adapter_gemm_concat(x, embeds, t.adapter.weight)
+        cur = hip.linear(x, t.adapter.weight, x1=embeds, workspace=ws)  # the kernels raven_core_iteration would pick
         for j in range(n_core):
             last = j == n_core - 1
             nxt = out if last else torch.empty_like(x)
@@ -571,10 +513,7 @@ class RavenForCausalLM(torch.nn.Module):
         if n_coda == 0:
             x = hip.rmsnorm_residual(x, t.ln_f.weight, cfg.norm_eps)[0]
 
-        if self._is_wide(M):
-            logits = torch.matmul(x, self.lm_head.weight.t()).float().view(B, S, -1)
-        else:
-            logits = hip.gemm(x, self.lm_head.weight, out_f32=True).view(B, S, -1)
+        logits = hip.gemm(x, self.lm_head.weight, out_f32=True).view(B, S, -1)
         if labels is not None:
             loss = torch.nn.functional.cross_entropy(logits.view(-1, logits.shape[-1]), labels.view(-1), ignore_index=-100)
             log_ppl = loss.clone()
@@ -921,40 +860,10 @@ class DecodeRunner:
         coda = [c._slot(-(i + 1)) for i in range(n_coda)]
         return pre, core, coda
 
-    def _enqueue_wide(self):
-        """The same step for more sequences than the skinny kernels take in one pass over the weights: library GEMMs
-        around the norm / RoPE-append / attention / SwiGLU kernels (forward's path for many rows), position on the device."""
-        m, t = self.model, self.model.transformer
-        cfg, B = m.config, self.B
-        kv = self.cache.native()
-        hint = self.cache.t_max - 1
-        pre, core, coda = self._slots()
-        hip.embed(t.wte.weight, self.ids, m.emb_scale, out=self.embeds)
-        x = self.embeds
-        for i, slot in enumerate(pre):
-            x, _ = m._wide_block(t.prelude[i], x, kv, slot, B, 1, hint, pos_dev=self.pos)
-        embeds = x
-        x = self.state
-        for it in range(self.r):
-            x = m._wide_core(m._maybe_inject_noise(x, it), embeds, core[it], kv, B, 1, hint, ln_f=(it == self.r - 1), pos_dev=self.pos)
-        self.latents.copy_(x)
-        n_coda = len(coda)
-        for i, slot in enumerate(coda):
-            last = i == n_coda - 1
-            y, tail = m._wide_block(t.coda[i], x, kv, slot, B, 1, hint, tail_w=t.ln_f.weight if last else None, pos_dev=self.pos)
-            x = tail if last else y
-        if n_coda == 0:
-            x = hip.rmsnorm_residual(x, t.ln_f.weight, cfg.norm_eps)[0]
-        self.logits.copy_(torch.matmul(x, m.lm_head.weight.t()))
-        hip.argmax(self.logits, out=self.next_ids)
-        hip.advance_pos(self.pos, 1)
-
     def _enqueue(self):
         """Launches one token's kernels; reads the position from self.pos."""
         m, t = self.model, self.model.transformer
         nat, cfg, B = m._natives(), m.config, self.B
-        if m._is_wide(B) and self.r > 0 and len(t.core_block) > 0:
-            return self._enqueue_wide()
         kv = self.cache.native()
         hint = self.cache.t_max - 1  # sizes grids; the kernels take the true position from the device
         pre, core, coda = self._slots()

@@ -93,23 +93,21 @@ class PagedDecoder:
         return out
 
     # ------------------------------------------------------------------ rows of any sequences (prompt chunks, decode rows)
-    def _mm(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-        """x [T, K] times w [N, K] transposed: the library for many rows, the skinny kernels for few."""
-        return torch.matmul(x, w.t()) if x.shape[0] >= self.model.WIDE_ROWS else hip.gemm(x, w)
 
     def _token_block(self, blk, f: int, x: torch.Tensor, meta) -> torch.Tensor:
         """One SandwichBlock (vllm/raven_vllm.py:289-294 around its attention layer, :184-203) on flat rows, flat layer f."""
         eps = self.cfg.norm_eps
         positions, slots, table, lens, q_start, max_q = meta
         n1 = hip.rmsnorm_residual(x, blk.norm_1.weight, eps)[0]
-        qkv = self._mm(n1, blk.attn.Wqkv.weight)
+        qkv = hip.linear(n1, blk.attn.Wqkv.weight)
         bias = blk.attn.qk_bias if hasattr(blk.attn, "qk_bias") else None
         q = hip.paged_qkv_rope_append(qkv, bias, self.model._natives()["freqs"], positions, slots, self.k[f], self.v[f], layout=self.layout)
         ya = hip.paged_prefill_attention(q, self.k[f], self.v[f], table, lens, q_start, max_q, layout=self.layout)
-        a = self._mm(ya, blk.attn.proj.weight)
-        x2, _, n3 = hip.rmsnorm_residual(a, blk.norm_2.weight, eps, residual=x, weight2=blk.norm_3.weight)
-        m = self._mm(hip.swiglu(self._mm(n3, blk.mlp.fc.weight)), blk.mlp.proj.weight)
-        return hip.rmsnorm_residual(m, blk.norm_4.weight, eps, residual=x2)[0]
+        # the residual adds (RMM:534-535) and the SwiGLU (RMM:507-508) ride in the epilogues of the products
+        x1 = hip.linear(ya, blk.attn.proj.weight, residual=x)
+        x2, _, n3 = hip.rmsnorm_residual(x1, blk.norm_2.weight, eps, weight2=blk.norm_3.weight)
+        x3 = hip.linear(hip.linear(n3, blk.mlp.fc.weight, swiglu=True), blk.mlp.proj.weight, residual=x2)
+        return hip.rmsnorm_residual(x3, blk.norm_4.weight, eps)[0]
 
     @torch.no_grad()
     def forward_tokens(self, input_ids: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor, block_table: torch.Tensor,
@@ -140,7 +138,7 @@ class PagedDecoder:
         else:
             state = input_states.reshape(T, -1).to(dev, m.dtype)
         for _ in range(self.r):
-            state = self._mm(torch.cat([state, embeds], dim=-1), t.adapter.weight)
+            state = hip.linear(state, t.adapter.weight, x1=embeds)  # the concat of RMM:776 as two K segments
             for j in range(n_core):
                 state = self._token_block(t.core_block[j], n_pre + j, state, meta)
         latents = hip.rmsnorm_residual(state, t.ln_f.weight, cfg.norm_eps)[0]
@@ -148,7 +146,7 @@ class PagedDecoder:
         for i in range(cfg.n_layers_in_coda):
             x = self._token_block(t.coda[i], n_pre + n_core + i, x, meta)
         x = hip.rmsnorm_residual(x, t.ln_f.weight, cfg.norm_eps)[0]
-        logits = torch.matmul(x, m.lm_head.weight.t()).float() if T >= m.WIDE_ROWS else hip.gemm(x, m.lm_head.weight, out_f32=True)
+        logits = hip.gemm(x, m.lm_head.weight, out_f32=True)
         return logits, latents
 
     def prefill_paged(self, input_ids: torch.Tensor, table_row: Sequence[int], input_states: Optional[torch.Tensor] = None,

@@ -33,3 +33,25 @@ def oracle():
 def lib(pkg):
     """The loaded C-ABI library; GPU tests fail (not skip) when it is missing."""
     return pkg.hip.load()
+
+
+# defaults of the launch-shape knobs the tests change (raven_set_tuning); results never depend on them
+TUNING_DEFAULTS = {"linear_ks": 0, "gemm_four_tiles": 1, "attn_wide": 0, "gemm_tiled_min_rows": 33, "gemm_tiled_variant": 0}
+
+
+@pytest.fixture
+def tuned(pkg):
+    """tuned(key=value, ...) sets knobs for the rest of the test; all of them are back at their defaults afterwards, also
+    when the test fails."""
+    touched = set()
+
+    def set_knobs(**knobs):
+        for key, value in knobs.items():
+            touched.add(key)
+            pkg.hip.set_tuning(key, value)
+
+    try:
+        yield set_knobs
+    finally:
+        for key in touched:
+            pkg.hip.set_tuning(key, TUNING_DEFAULTS[key])

@@ -38,10 +38,12 @@ def _prompt(B, n=PROMPT, seed=1):
     return torch.randint(0, 65536, (B, n), generator=torch.Generator().manual_seed(seed)).cuda()
 
 
-def test_decode_is_deterministic_and_graph_replay_equals_eager(pkg, nebel):
-    """32 sequences, 512-token prompt: four decode steps from the same prefilled cache, three times (eager launches,
-    a captured HIP graph, a second captured graph): the same bits every time."""
-    B = 32
+@pytest.mark.parametrize("B", [1, 8, 32])
+def test_decode_is_deterministic_and_graph_replay_equals_eager(pkg, nebel, B):
+    """1, 8 and 32 sequences, 512-token prompt: four decode steps from the same prefilled cache, three times (eager
+    launches, a captured HIP graph, a second captured graph): the same bits every time.  One sequence takes the one-row
+    schedule (every norm in a GEMV prologue, all 32 recurrences in one raven_core_iterations call with the adapter split
+    by columns), 8 and 32 the multi-row one."""
     ids = _prompt(B)
     cache = pkg.HuginnDynamicCache(max_length=PROMPT + 8)
     h = nebel.config.n_embd
@@ -64,9 +66,38 @@ def test_decode_is_deterministic_and_graph_replay_equals_eager(pkg, nebel):
     for other in runs[1:]:
         for a, b in zip(runs[0], other):
             assert all(torch.equal(x, y) for x, y in zip(a, b))
-    again = [nebel(input_ids=ids[:2, :48].contiguous(), input_states=torch.zeros(2, 48, h, device="cuda", dtype=torch.bfloat16),
+    b2 = min(B, 2)
+    again = [nebel(input_ids=ids[:b2, :48].contiguous(), input_states=torch.zeros(b2, 48, h, device="cuda", dtype=torch.bfloat16),
                    num_steps=R).logits for _ in range(2)]
     assert torch.equal(again[0], again[1])
+
+
+@pytest.mark.parametrize("B", [1, 8])
+def test_full_token_decode_256_greedy_tokens(pkg, nebel, B):
+    """The full-token decode configuration at 1 and 8 sequences: 512-token random prompt, 256 greedy tokens at r = 32
+    (prefill through forward(), then one HIP-graph replay per token).  Zero initial states make the run reproducible:
+    the graph run and the eager run produce the same 256 tokens; all ids are inside the vocabulary; the cache holds
+    512 + 255 positions in all 132 step entries."""
+    ids = _prompt(B, seed=10 + B)
+    gc = pkg.GenerationSettings(max_new_tokens=256)
+    runs = []
+    for use_graph in (True, False):
+        out = nebel.generate_minimal(ids, gc, num_steps=R, init_scale=0.0, stop_tokens=set(), use_graph=use_graph)
+        assert out.shape == (B, PROMPT + 256)
+        assert torch.equal(out[:, :PROMPT], ids)
+        new = out[:, PROMPT:]
+        assert int(new.min()) >= 0 and int(new.max()) < 65536
+        runs.append(new.clone())
+    assert torch.equal(runs[0], runs[1]), "graph replay and eager launches must pick the same tokens"
+    # three tokens on a cache of the same capacity (how many workgroups split a sequence's positions follows from the
+    # capacity, and with it the order of the fp32 additions): the same first tokens
+    gc2 = pkg.GenerationSettings(max_new_tokens=3, return_dict_in_generate=True)
+    res = nebel.generate_minimal(ids, gc2, num_steps=R, init_scale=0.0, stop_tokens=set(),
+                                 past_key_values=pkg.HuginnDynamicCache(max_length=PROMPT + 256))
+    assert torch.equal(res.sequences[:, PROMPT:], runs[0][:, :3])
+    assert res.past_key_values.get_seq_length() == PROMPT + 2
+    for step in (0, 1, 2, 129, -1, -2):  # first and last of the 132 step entries hold every position
+        assert res.past_key_values.key_cache[step][PROMPT + 1].shape == (B, 55, 96)
 
 
 def _prefill_and_two_steps(pkg, model, ids, states, max_length):
@@ -84,20 +115,16 @@ def _prefill_and_two_steps(pkg, model, ids, states, max_length):
 
 
 def test_batch_permutation_and_cache_capacity_leave_every_bit_in_place(pkg, nebel):
-    """Through this library's own kernels only (the prompt goes through the skinny MFMA path in passes of 32 rows: a
-    library GEMM may choose its accumulation order by tile position, which a permutation changes)."""
+    """Every product's accumulation order is the same for every tile position in this library's kernels, so a permutation of
+    the sequences permutes the results bit for bit."""
     B, n = 32, 128
     ids = _prompt(B, n, seed=2)
     g = torch.Generator(device="cuda").manual_seed(3)
     states = (torch.randn(B, n + 2, nebel.config.n_embd, device="cuda", generator=g) * 0.632).to(torch.bfloat16)
-    nebel.WIDE_ROWS = 10 ** 9
-    try:
-        base, cache = _prefill_and_two_steps(pkg, nebel, ids, states, n + 2)
-        perm = torch.randperm(B, generator=torch.Generator().manual_seed(4)).cuda()
-        shuffled, cache_p = _prefill_and_two_steps(pkg, nebel, ids[perm].contiguous(), states[perm].contiguous(), n + 2)
-        roomy, cache_r = _prefill_and_two_steps(pkg, nebel, ids, states, 2 * n + 77)
-    finally:
-        del nebel.WIDE_ROWS  # back to the class default
+    base, cache = _prefill_and_two_steps(pkg, nebel, ids, states, n + 2)
+    perm = torch.randperm(B, generator=torch.Generator().manual_seed(4)).cuda()
+    shuffled, cache_p = _prefill_and_two_steps(pkg, nebel, ids[perm].contiguous(), states[perm].contiguous(), n + 2)
+    roomy, cache_r = _prefill_and_two_steps(pkg, nebel, ids, states, 2 * n + 77)
     for a, b, c in zip(base, shuffled, roomy):
         assert torch.equal(a.logits[perm], b.logits) and torch.equal(a.latent_states[perm], b.latent_states)
         assert torch.equal(a.logits, c.logits)

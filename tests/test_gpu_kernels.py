@@ -23,7 +23,6 @@ def close(got: torch.Tensor, want: torch.Tensor, what: str = ""):
     got, want = got.detach().float().cpu(), want.detach().float().cpu()
     assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
     assert torch.isfinite(got).all(), f"{what}: non-finite values"
-    bf = want.dtype == torch.bfloat16 or True
     max_abs = (got - want).abs().max().item()
     rel = ((got - want).norm() / want.norm().clamp_min(1e-30)).item()
     return max_abs, rel
@@ -145,11 +144,11 @@ def test_gemm_swiglu(pkg, dt, M, I, K):
 
 @pytest.mark.parametrize("M", [2, 3, 4, 5, 8, 16, 17, 32, 33, 34, 40])
 @pytest.mark.parametrize("ks", [0, 3])
-def test_linear_with_workspace_nebel_shapes(pkg, M, ks):
+def test_linear_with_workspace_nebel_shapes(pkg, tuned, M, ks):
     """raven_linear at the 3.5b shapes, every epilogue: with the library's own choice between its two MFMA
     kernels (ks = 0) and with the split-K, shared-X kernel forced to three K slices for every matrix."""
     dt, h, I = torch.bfloat16, 5280, 17920
-    pkg.hip.set_tuning("linear_ks", ks)
+    tuned(linear_ks=ks)
     ws = pkg.hip.linear_workspace(M, 2 * I, "cuda")
     x, xi, x1 = rnd((M, h), dt, 160 + M), rnd((M, I), dt, 161), rnd((M, h), dt, 162)
     res = rnd((M, h), dt, 163)
@@ -167,31 +166,29 @@ def test_linear_with_workspace_nebel_shapes(pkg, M, ks):
     a, b = pkg.hip.linear(dev(xi), dev(mlp), workspace=ws), pkg.hip.linear(dev(xi), dev(mlp), workspace=ws)
     assert torch.equal(a, b)
     check(pkg.hip.linear(dev(xi), dev(mlp)), lin(xi, mlp).to(dt), dt, "no workspace")
-    pkg.hip.set_tuning("linear_ks", 0)
 
 
-def test_linear_small_and_odd_shapes(pkg):
+def test_linear_small_and_odd_shapes(pkg, tuned):
     dt = torch.bfloat16
-    pkg.hip.set_tuning("linear_ks", 2)  # the split-K kernel for everything it accepts
+    tuned(linear_ks=2)  # the split-K kernel for everything it accepts
     for M, N, K in ((9, 48, 160), (32, 16, 128), (12, 528, 1056), (7, 32, 96), (6, 20, 64)):
         x, w = rnd((M, K), dt, 170), rnd((N, K), dt, 171, 0.05)
         ws = pkg.hip.linear_workspace(M, N, "cuda")
         check(pkg.hip.linear(x.cuda(), w.cuda(), workspace=ws), lin(x, w).to(dt), dt, f"linear {M}x{N}x{K}")
     x, w = rnd((3, 256), torch.float32, 172), rnd((64, 256), torch.float32, 173, 0.1)
     check(pkg.hip.linear(x.cuda(), w.cuda(), workspace=pkg.hip.linear_workspace(3, 64, "cuda")), lin(x, w), torch.float32, "fp32 falls through")
-    pkg.hip.set_tuning("linear_ks", 0)
 
 
 @pytest.mark.parametrize("M", [6, 20])
 @pytest.mark.parametrize("four", [1, 2])
-def test_mfma_gemm_row_alignment_cases(pkg, M, four):
+def test_mfma_gemm_row_alignment_cases(pkg, tuned, M, four):
     """Row pitches that are odd multiples of 64 bytes (tiles of one row parity, macro-steps shifted to the line
     boundary), with and without whole tile pairs, a second operand that starts mid-line, and a weight matrix
     whose base address is not line-aligned; both MFMA kernels (with and without a workspace)."""
     dt = torch.bfloat16
     ws = pkg.hip.linear_workspace(M, 4096, "cuda")
-    pkg.hip.set_tuning("gemm_four_tiles", four)  # 2: the four-tile, 64-wide-step variant wherever there is no workspace
-    pkg.hip.set_tuning("linear_ks", 2)  # with a workspace: the split-K kernel
+    # four = 2: the four-tile, 64-wide-step variant wherever there is no workspace; with a workspace: the split-K kernel
+    tuned(gemm_four_tiles=four, linear_ks=2)
     for N, K in ((32, 96), (64, 288), (64, 2336), (96, 416), (48, 416), (160, 1184), (64, 256)):
         x, w = rnd((M, K), dt, 180 + N), rnd((N, K), dt, 181 + K, 0.05)
         want = lin(x, w).to(dt)
@@ -212,14 +209,12 @@ def test_mfma_gemm_row_alignment_cases(pkg, M, four):
         for wsp in (None, ws):
             check(pkg.hip.linear(x0.cuda(), w.cuda(), x1=x1.cuda(), workspace=wsp), lin(torch.cat([x0, x1], -1), w).to(dt), dt,
                   f"two operands {M}x{N}x({K0}+{K1})")
-    pkg.hip.set_tuning("linear_ks", 0)
-    pkg.hip.set_tuning("gemm_four_tiles", 1)
 
 
 @pytest.mark.parametrize("M", [8, 32])
-def test_mfma_four_tile_variant_nebel_shapes(pkg, M):
+def test_mfma_four_tile_variant_nebel_shapes(pkg, tuned, M):
     dt, h, I = torch.bfloat16, 5280, 17920
-    pkg.hip.set_tuning("gemm_four_tiles", 2)
+    tuned(gemm_four_tiles=2)
     x, xi, res = rnd((M, h), dt, 230 + M), rnd((M, I), dt, 231), rnd((M, h), dt, 232)
     wqkv, fc, mlp = rnd((3 * h, h), dt, 233, 0.02), rnd((2 * I, h), dt, 234, 0.02), rnd((h, I), dt, 235, 0.02)
     check(pkg.hip.gemm(x.cuda(), wqkv.cuda()), lin(x, wqkv).to(dt), dt, "qkv")
@@ -228,7 +223,6 @@ def test_mfma_four_tile_variant_nebel_shapes(pkg, M):
     check(pkg.hip.gemm(xi.cuda(), mlp.cuda(), residual=res.cuda()), lin(xi, mlp).to(dt) + res, dt, "mlp.proj + residual")
     yf = pkg.hip.gemm(x.cuda(), wqkv.cuda(), out_f32=True)
     assert yf.dtype == torch.float32 and torch.equal(yf, pkg.hip.gemm(x.cuda(), wqkv.cuda()).float())
-    pkg.hip.set_tuning("gemm_four_tiles", 1)
 
 
 @pytest.mark.parametrize("dt,h,I", [(torch.bfloat16, 5280, 17920), (torch.float32, 256, 704), (torch.bfloat16, 64, 176)])

@@ -190,25 +190,24 @@ def test_forward_tiny_bf16_matches_oracle(tiny16):
 
 
 @pytest.mark.parametrize("B,S", [(1, 64), (2, 70), (1, 200)])
-def test_wide_prefill_path_bf16(pkg, tiny16, B, S):
-    """From 64 token rows on, the GEMMs go to the library and attention to the matrix-core chunk kernel:
-    same results as the oracle, and as the narrow path, then a decode token on top of the prefilled cache."""
+def test_wide_prefill_path_bf16(pkg, tiny16, tuned, B, S):
+    """From 33 token rows on, the five products go to the tiled MFMA kernel and chunks of 16 or more rows to the matrix-core
+    attention kernel: same results as the oracle, and as the skinny kernels in passes of 32 rows, then a decode token on
+    top of the prefilled cache."""
     s, w, model = tiny16
     g = torch.Generator().manual_seed(S)
     ids = torch.randint(0, s.vocab_size, (B, S + 1), generator=g)
     states = O.initialize_state(torch.empty(B, S + 1, s.n_embd), s, 1.0, g).to(torch.bfloat16)
-    assert model._is_wide(B * S)
+    assert B * S >= 33
     ref_cache, cache = O.DictCache(), pkg.HuginnDynamicCache()
     want = O.forward(w, s, input_ids=ids[:, :S], input_states=states[:, :S], past_key_values=ref_cache, use_cache=True)
     got = model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda(), past_key_values=cache, use_cache=True)
     check(got.latent_states, want.latent_states, torch.bfloat16, "wide latents")
     check(got.logits, want.logits, torch.bfloat16, "wide logits")
-    model.WIDE_ROWS = 1 << 30
-    try:
-        narrow = model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda())
-    finally:
-        model.WIDE_ROWS = type(model).WIDE_ROWS
-    check(got.logits, narrow.logits, torch.bfloat16, "wide vs narrow")
+    tuned(gemm_tiled_min_rows=1 << 30)
+    narrow = model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda())
+    tuned(gemm_tiled_min_rows=33)
+    check(got.logits, narrow.logits, torch.bfloat16, "tiled vs skinny")
     pos = torch.arange(S, S + 1)
     want1 = O.forward(w, s, input_ids=ids[:, S:], input_states=states[:, S:], past_key_values=ref_cache, use_cache=True, cache_position=pos)
     got1 = model(input_ids=ids[:, S:].cuda(), input_states=states[:, S:].cuda(), past_key_values=cache, use_cache=True,
@@ -219,12 +218,11 @@ def test_wide_prefill_path_bf16(pkg, tiny16, B, S):
 
 @pytest.mark.parametrize("use_graph", [False, True])
 def test_decode_runner_beyond_one_pass_of_rows_bf16(pkg, tiny16, use_graph):
-    """More sequences than the skinny kernels take per pass over the weights: the runner's step goes through the library
-    GEMMs with the position on the device.  Teacher-forced tokens; every step's logits against the oracle and against
-    forward() on the same cache contents; the graph is captured at the second step and replayed at the third."""
+    """More sequences than the skinny kernels take per pass over the weights, with the position on the device.
+    Teacher-forced tokens; every step's logits against the oracle and against forward() on the same cache contents; the
+    graph is captured at the second step and replayed at the third."""
     s, w, model = tiny16
     B, S, n_new = 40, 5, 3
-    assert model._is_wide(B)
     g = torch.Generator().manual_seed(77)
     ids = torch.randint(0, s.vocab_size, (B, S + n_new), generator=g)
     states = O.initialize_state(torch.empty(B, S + n_new, s.n_embd), s, 1.0, g).to(torch.bfloat16)
@@ -885,3 +883,141 @@ def test_core_iteration_nebel_bf16_config3(pkg, nebel_core, B):
     err_b = min(close(got, want_b)[1], close(got, alt_b)[1])
     print(f"block + ln_f B={B}: rel-L2 {err_b:.3e}, floor {floor_b:.3e}")
     assert err_b <= max(1.5 * floor_b, 1e-2) and err_b <= 3e-2
+
+
+# ----------------------------------------------------------------------------- the one-row, many-recurrences path at h = 5280
+def _nebel_cache(pkg, n_slots, B, T, dt, seed):
+    s = O.RavenShape.nebel()
+    kc, vc = rnd((n_slots, B, s.n_heads, T + 1, s.head_dim), dt, seed), rnd((n_slots, B, s.n_heads, T + 1, s.head_dim), dt, seed + 1)
+    kd, vd = kc.cuda(), vc.cuda()
+    return kc, vc, kd, vd, pkg.hip.make_cache(kd, vd)
+
+
+def test_adapter_column_split_over_recurrences_nebel(pkg, nebel_core):
+    """The launch sequence behind the decode benchmark's one-row step: raven_core_iterations with M = 1 and several
+    recurrences forms the embedding half of the adapter product once (a column block of the [5280, 10560] matrix with
+    row pitch 10560, unrounded fp32 sums), adds those sums to every recurrence's state half before the product's one
+    rounding, and folds each closing norm_4 into the next adapter product's prologue
+    (gemv_decode.hip gemv1_column_block; compose.hip iterations_impl).  To hold exactly those kernels to the per-kernel
+    bar, the block's four matrices are zero here: a block then returns norm_4(norm_2(x)) of the adapter output, and three
+    recurrences are three adapter products with two norms between them -- no chaotic amplification.  Oracle: the same
+    weights through core_block_forward three times (RMM:764-781)."""
+    s, w, dev = nebel_core
+    dt, h, T, r = torch.bfloat16, s.n_embd, 37, 3
+    ww = {k: v for k, v in w.items()}
+    p = "transformer.core_block.0"
+    for name in ("attn.Wqkv", "attn.proj", "mlp.fc", "mlp.proj"):
+        ww[f"{p}.{name}.weight"] = torch.zeros_like(w[f"{p}.{name}.weight"])
+    zdev = {k: (v.cuda() if k.startswith(p) else dev[k]) for k, v in ww.items()}
+    blocks = (pkg.hip.BlockWeights * 1)(_block_weights(pkg, zdev, p))
+    dims = pkg.hip.make_dims(h, s.n_heads, s.intermediate_size, s.norm_eps, dt)
+    g = torch.Generator().manual_seed(5)
+    state = O.initialize_state(torch.empty(1, 1, h), s, 1.0, g).to(dt)
+    embeds = torch.randn(1, 1, h, generator=g).to(dt)
+    table = O.rope_table(s.head_dim, s.block_size, s.rope_base).to(dt)
+    freqs = table.float().reshape(s.block_size, s.head_dim // 2, 2).contiguous().cuda()
+    kc, vc, kd, vd, cache = _nebel_cache(pkg, r, 1, T, dt, 900)
+    ws = pkg.hip.block_workspace(dims, 1, "cuda")
+    out = torch.empty(1, h, dtype=dt, device="cuda")
+    lnf = rnd((h,), dt, 902, 0.02, 1.0)
+    pkg.hip.core_iterations(dims, dev["transformer.adapter.weight"], blocks, state.view(1, h).cuda(), embeds.view(1, h).cuda(), out, freqs,
+                            cache, [[it] for it in range(r)], 1, 1, T, ws, ln_f=lnf.cuda())
+    # oracle: one core block per recurrence, its own cache entry per recurrence
+    x = state
+    for it in range(r):
+        rc = O.DictCache()  # step indices from 2 on: the core's entries (index 0 would advance the token count)
+        rc._seen_tokens = T + 1
+        rc.key_cache[2 + it] = {pp: kc[it, :, :, pp] for pp in range(T)}
+        rc.value_cache[2 + it] = {pp: vc[it, :, :, pp] for pp in range(T)}
+        x = O.linear(torch.cat([x, embeds], dim=-1), ww["transformer.adapter.weight"])
+        x = O.sandwich_block(x, ww, p, table[:, T:T + 1], 2 + it, rc, s)
+    want = O.rmsnorm(x, lnf, s.norm_eps).view(1, h)
+    check(out, want, dt, "three recurrences through the split adapter")
+    # the same three recurrences one call at a time take the unsplit two-operand product: agreement at the same bar
+    x_dev, one = state.view(1, h).cuda(), torch.empty(1, h, dtype=dt, device="cuda")
+    kc2, vc2, kd2, vd2, cache2 = _nebel_cache(pkg, r, 1, T, dt, 900)
+    for it in range(r):
+        pkg.hip.core_iteration(dims, dev["transformer.adapter.weight"], blocks, x_dev, embeds.view(1, h).cuda(), one, freqs, cache2, it, 1, 1, T,
+                               ws, ln_f=lnf.cuda() if it == r - 1 else None)
+        x_dev = one.clone()
+    check(out, one, dt, "core_iterations(3) vs three core_iteration calls")
+    check(kd, kd2, dt, "appended keys")
+
+
+def test_core_iterations_nebel_one_row_real_weights(pkg, nebel_core):
+    """The same call with the real (random-init) weights of all four core blocks, three recurrences, one row, 1024 cached
+    positions: against three raven_core_iteration calls.  The two launch sequences differ only in the order of fp32
+    additions inside the adapter product; four blocks per recurrence amplify such differences (the oracle differs from
+    itself by rel-L2 1.8e-2 per recurrence under a change of accumulation order), so the first recurrence's cache rows,
+    which sit in front of that amplification, carry the per-kernel bar and the final state a composed one."""
+    s, w, dev = nebel_core
+    dt, h, T, r = torch.bfloat16, s.n_embd, 1024, 3
+    blocks = (pkg.hip.BlockWeights * 4)(*[_block_weights(pkg, dev, f"transformer.core_block.{j}") for j in range(4)])
+    dims = pkg.hip.make_dims(h, s.n_heads, s.intermediate_size, s.norm_eps, dt)
+    g = torch.Generator().manual_seed(6)
+    state = O.initialize_state(torch.empty(1, 1, h), s, 1.0, g).to(dt).view(1, h).cuda()
+    embeds = torch.randn(1, h, generator=g).to(dt).cuda()
+    table = O.rope_table(s.head_dim, s.block_size, s.rope_base).to(dt)
+    freqs = table.float().reshape(s.block_size, s.head_dim // 2, 2).contiguous().cuda()
+    ws = pkg.hip.block_workspace(dims, 1, "cuda")
+    slots = [[it * 4 + j for j in range(4)] for it in range(r)]
+    _, _, kd, vd, cache = _nebel_cache(pkg, 4 * r, 1, T, dt, 910)
+    _, _, kd2, vd2, cache2 = _nebel_cache(pkg, 4 * r, 1, T, dt, 910)
+    many, one = torch.empty_like(state), torch.empty_like(state)
+    pkg.hip.core_iterations(dims, dev["transformer.adapter.weight"], blocks, state, embeds, many, freqs, cache, slots, 1, 1, T, ws)
+    x = state
+    for it in range(r):
+        pkg.hip.core_iteration(dims, dev["transformer.adapter.weight"], blocks, x, embeds, one, freqs, cache2, slots[it][0], 1, 1, T, ws)
+        x = one.clone()
+    check(kd[0, :, :, T], kd2[0, :, :, T], dt, "first recurrence, first block: appended K")
+    check(vd[0, :, :, T], vd2[0, :, :, T], dt, "first recurrence, first block: appended V")
+    err = close(many, one, "state after three recurrences")[1]
+    err2 = close(kd[4, :, :, T], kd2[4, :, :, T], "second recurrence, first block: appended K")[1]
+    print(f"core_iterations(3) vs 3 x core_iteration at h=5280, one row: rel-L2 {err:.3e} (K behind one recurrence: {err2:.3e})")
+    # behind one recurrence the rounding differences have grown about tenfold, behind three the two runs are related but
+    # no longer close (measured 0.2): the final state is only required to be finite and correlated
+    assert err2 <= 1e-1 and err <= 0.5 and torch.isfinite(many.float()).all()
+    assert torch.equal(kd[:, :, :, :T], kd2[:, :, :, :T]), "cached positions must be untouched"
+    # twice the same call: the same bits
+    _, _, kd3, vd3, cache3 = _nebel_cache(pkg, 4 * r, 1, T, dt, 910)
+    again = torch.empty_like(state)
+    pkg.hip.core_iterations(dims, dev["transformer.adapter.weight"], blocks, state, embeds, again, freqs, cache3, slots, 1, 1, T, ws)
+    assert torch.equal(again, many) and torch.equal(kd3, kd)
+
+
+def test_core_iteration_nebel_fp32_against_fp32_oracle(pkg):
+    """One recurrence at the 3.5b shape in fp32, one row, 1024 cached positions per step slot, against the fp32 oracle at
+    the fp32 bar (1e-4 / 1e-5): with rounding out of the picture this is a test of indexing at the real strides (5280-wide
+    rows, 55 heads of 96, the [5280, 10560] adapter, 17920-wide gate / up halves), RMM:764-781."""
+    s = O.RavenShape.nebel()
+    dt, h, nh, hd, T, B = torch.float32, s.n_embd, s.n_heads, s.head_dim, 1024, 1
+    w = O.make_weights(s, seed=0, dtype=dt, only_core=True)
+    dev = {k: v.cuda() for k, v in w.items()}
+    kc, vc = rnd((4, B, nh, T + 1, hd), dt, 920), rnd((4, B, nh, T + 1, hd), dt, 921)
+    kd, vd = kc.cuda(), vc.cuda()
+    cache = pkg.hip.make_cache(kd, vd)
+    g = torch.Generator().manual_seed(7)
+    state = O.initialize_state(torch.empty(B, 1, h), s, 1.0, g)
+    embeds = torch.randn(B, 1, h, generator=g)
+    table = O.rope_table(hd, s.block_size, s.rope_base)
+    freqs = table.reshape(s.block_size, hd // 2, 2).contiguous().cuda()
+    ref_cache = O.DictCache()
+    ref_cache._seen_tokens = T + 1
+    for j in range(4):
+        ref_cache.key_cache[2 + j] = {p: kc[j, :, :, p] for p in range(T)}
+        ref_cache.value_cache[2 + j] = {p: vc[j, :, :, p] for p in range(T)}
+    want, idx = O.core_block_forward(state, embeds, w, table[:, T:T + 1], ref_cache, 1, s)
+    assert idx == 5
+    dims = pkg.hip.make_dims(h, nh, s.intermediate_size, s.norm_eps, dt)
+    blocks = (pkg.hip.BlockWeights * 4)(*[_block_weights(pkg, dev, f"transformer.core_block.{j}") for j in range(4)])
+    ws = pkg.hip.block_workspace(dims, B, "cuda")
+    out = torch.empty(B, h, dtype=dt, device="cuda")
+    pkg.hip.core_iteration(dims, dev["transformer.adapter.weight"], blocks, state.view(B, h).cuda(), embeds.view(B, h).cuda(), out, freqs,
+                           cache, 0, B, 1, T, ws)
+    err = close(out, want.view(B, h), "fp32 core iteration")
+    print(f"fp32 core iteration at the 3.5b shape: max-abs {err[0]:.3e} rel-L2 {err[1]:.3e}")
+    check(out, want.view(B, h), dt, "fp32 core iteration at the 3.5b shape")
+    for j in range(4):
+        check(kd[j, :, :, T], ref_cache.key_cache[2 + j][T], dt, f"appended K, block {j}")
+        check(vd[j, :, :, T], ref_cache.value_cache[2 + j][T], dt, f"appended V, block {j}")
+    assert torch.equal(kd[:, :, :, :T].cpu(), kc[:, :, :, :T])

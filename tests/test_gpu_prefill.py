@@ -1,0 +1,244 @@
+"""GPU parity at the prefill configuration (core prefill at the 3.5b shape: 4 sequences x 4096 tokens, bf16) and of the
+tiled MFMA GEMM that serves every product with 33 or more token rows.
+
+All calls go through the C ABI (pkg.hip wrappers).  Reference values: fp32 `F.linear` on the same operands for the
+products (the library's GEMMs are row-independent, so a sample of rows is compared at full N), the CPU oracle's
+`sdpa` per head for attention, and the oracle's SandwichBlock on a sample of rows of one sequence for the composed block
+(attention needs all keys of that sequence, so its K / V rows are all computed by the oracle).
+Bars: per kernel max-abs <= 2e-2 (times max(1, |ref|max)) and rel-L2 <= 1e-2; the composed block as in test_gpu_model.py."""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import raven_oracle as O
+from test_gpu_kernels import check, close, rnd
+
+pytestmark = pytest.mark.gpu
+
+H, NH, HD, INTER = 5280, 55, 96, 17920
+
+
+def _rows(M, n=48, seed=0):
+    """Rows to compare: the first and last tile edges plus a random sample."""
+    g = torch.Generator().manual_seed(seed)
+    picks = [torch.arange(0, min(M, 8)), torch.arange(max(0, M - 8), M), torch.randint(0, M, (n,), generator=g)]
+    for edge in (255, 256, 257, 4095, 4096, 8191, 8192):
+        if edge < M:
+            picks.append(torch.tensor([edge]))
+    return torch.unique(torch.cat(picks))
+
+
+def _gpu_randn(shape, seed, std=1.0):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return (torch.randn(shape, device="cuda", generator=g) * std).to(torch.bfloat16)
+
+
+def _ref_rows(x, w, rows):
+    """fp32 product of the sampled rows with the whole matrix (a plain PyTorch fp32 reference of nn.Linear)."""
+    return F.linear(x[rows].float(), w.float())
+
+
+# ----------------------------------------------------------------------------- the five products at M = 16384
+@pytest.mark.parametrize("name", ["Wqkv", "attn.proj", "mlp.fc", "mlp.proj", "adapter", "lm_head"])
+def test_tiled_gemm_nebel_shapes_m16384(pkg, name):
+    """RMM:463, 493, 507-509, 776, 711 at 16384 token rows: the tiled kernel with each product's epilogue."""
+    dt, M = torch.bfloat16, 16384
+    rows = _rows(M).cuda()
+    if name == "Wqkv":
+        x, w = _gpu_randn((M, H), 1), _gpu_randn((3 * H, H), 2, 0.02)
+        got = pkg.hip.linear(x, w)
+        want = _ref_rows(x, w, rows).to(dt)
+    elif name == "attn.proj":
+        x, w, res = _gpu_randn((M, H), 3), _gpu_randn((H, H), 4, 0.02), _gpu_randn((M, H), 5)
+        got = pkg.hip.linear(x, w, residual=res)
+        want = (_ref_rows(x, w, rows).to(dt).float() + res[rows].float()).to(dt)
+    elif name == "mlp.fc":
+        x, w = _gpu_randn((M, H), 6), _gpu_randn((2 * INTER, H), 7, 0.02)
+        got = pkg.hip.linear(x, w, swiglu=True)
+        z = _ref_rows(x, w, rows).to(dt).float()
+        want = (F.silu(z[:, :INTER]).to(dt).float() * z[:, INTER:]).to(dt)
+        wrong = (F.silu(z[:, INTER:]).to(dt).float() * z[:, :INTER]).to(dt)
+        assert close(got[rows], wrong)[1] > 0.1, "the gate must be the first half of fc's output"
+    elif name == "mlp.proj":
+        x, w, res = _gpu_randn((M, INTER), 8), _gpu_randn((H, INTER), 9, 0.02), _gpu_randn((M, H), 10)
+        got = pkg.hip.linear(x, w, residual=res)
+        want = (_ref_rows(x, w, rows).to(dt).float() + res[rows].float()).to(dt)
+    elif name == "adapter":
+        x0, x1, w = _gpu_randn((M, H), 11), _gpu_randn((M, H), 12), _gpu_randn((H, 2 * H), 13, 0.02)
+        got = pkg.hip.linear(x0, w, x1=x1)
+        want = _ref_rows(torch.cat([x0[rows], x1[rows]], -1), w, torch.arange(rows.numel()).cuda()).to(dt)
+        swapped = _ref_rows(torch.cat([x1[rows], x0[rows]], -1), w, torch.arange(rows.numel()).cuda()).to(dt)
+        assert close(got[rows], swapped)[1] > 0.1, "the state is the first operand, the embedded input the second"
+    else:  # lm_head: a quarter of the rows is enough for a 65536-wide output (float logits)
+        M = 4096
+        rows = _rows(M).cuda()
+        x, w = _gpu_randn((M, H), 14), _gpu_randn((65536, H), 15, 0.02)
+        got = pkg.hip.gemm(x, w, out_f32=True)
+        assert got.dtype == torch.float32
+        want = _ref_rows(x, w, rows).to(dt).float()
+    check(got[rows], want, dt, f"{name} at {M} rows")
+    assert torch.isfinite(got.float()).all()
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("M,N,K", [(33, 64, 64), (64, 256, 256), (100, 264, 320), (257, 520, 96), (300, 5280, 5280), (513, 776, 1096)])
+def test_tiled_gemm_edges_against_oracle(pkg, tuned, variant, M, N, K):
+    """Both tile sizes (256 x 256 and 128 x 128) on shapes with partial tiles in M and N, K that is not a multiple of
+    the 64-wide step, every epilogue and the two-operand form, against the oracle's linear / SwiGLU / residual."""
+    dt = torch.bfloat16
+    tuned(gemm_tiled_variant=variant)
+    x, w, res = rnd((M, K), dt, 500 + M), rnd((N, K), dt, 501 + N, 0.05), rnd((M, N), dt, 502)
+    dev = lambda t: t.cuda()
+    lin = lambda a, b: F.linear(a.float(), b.float())
+    check(pkg.hip.linear(dev(x), dev(w)), lin(x, w).to(dt), dt, "plain")
+    check(pkg.hip.linear(dev(x), dev(w), residual=dev(res)), lin(x, w).to(dt) + res, dt, "+ residual")
+    yf = pkg.hip.linear(dev(x), dev(w), out_f32=True)
+    assert yf.dtype == torch.float32 and torch.equal(yf, pkg.hip.linear(dev(x), dev(w)).float())
+    if N % 16 == 0:
+        fc = rnd((2 * N, K), dt, 503, 0.05)
+        z = lin(x, fc).to(dt)
+        check(pkg.hip.linear(dev(x), dev(fc), swiglu=True), F.silu(z[:, :N]) * z[:, N:], dt, "SwiGLU")
+    x1, w2 = rnd((M, K), dt, 504), rnd((N, 2 * K), dt, 505, 0.05)
+    check(pkg.hip.linear(dev(x), dev(w2), x1=dev(x1)), lin(torch.cat([x, x1], -1), w2).to(dt), dt, "two operands")
+    # against the oracle's own statement of the products (nn.Linear in bf16 on the CPU; small shapes only: it is slow)
+    if M * N * K <= 2 * 10 ** 8:
+        check(pkg.hip.linear(dev(x), dev(w)), O.linear(x, w), dt, "oracle linear")
+    # the same call twice: the same bits; and the tile size does not change a bit either (one accumulation order)
+    a = pkg.hip.linear(dev(x), dev(w))
+    tuned(gemm_tiled_variant=3 - variant)
+    assert torch.equal(a, pkg.hip.linear(dev(x), dev(w)))
+
+
+# ----------------------------------------------------------------------------- attention at 4 x 4096
+def test_prefill_attention_config4(pkg):
+    """raven_prefill_attention at B=4, S=4096, 55 heads of 96: sampled (sequence, head) pairs against the oracle's sdpa,
+    all 4096 query rows of each (the causal case of RMM:484-491)."""
+    dt, B, S = torch.bfloat16, 4, 4096
+    q = _gpu_randn((B * S, H), 21)
+    k = _gpu_randn((1, B, NH, S, HD), 22)
+    v = _gpu_randn((1, B, NH, S, HD), 23)
+    cache = pkg.hip.make_cache(k, v)
+    y = pkg.hip.prefill_attention(q, cache, 0, B, S, 0, NH, HD)
+    torch.cuda.synchronize()
+    for b, head in ((0, 0), (1, 17), (2, 54), (3, 31), (3, 0)):
+        qh = q.view(B, S, NH, HD)[b, :, head].cpu()[None, None]
+        want = O.sdpa(qh, k[0, b, head].cpu()[None, None], v[0, b, head].cpu()[None, None])[0, 0]
+        check(y.view(B, S, NH, HD)[b, :, head], want, dt, f"sequence {b} head {head}")
+    # the chunk kernel and the per-row kernel agree on a sample of rows (two implementations of the same softmax)
+    rows = torch.tensor([0, 1, 63, 64, 127, 128, 2047, 2048, 4095])
+    for b in (0, 3):
+        for r in rows.tolist():
+            qr = q.view(B, S, H)[b, r].view(1, NH, 1, HD)
+            want = O.sdpa(qr.cpu(), k[0, b, :, :r + 1].cpu()[None], v[0, b, :, :r + 1].cpu()[None]).view(H)
+            check(y.view(B, S, H)[b, r], want, dt, f"row {r} of sequence {b}")
+
+
+# ----------------------------------------------------------------------------- one SandwichBlock at M = 16384
+def test_sandwich_block_config4_rows(pkg):
+    """raven_sandwich_block on 4 x 4096 rows at the 3.5b dims (tiled products, MFMA chunk attention, fused norms) against
+    the oracle's SandwichBlock (RMM:525-536) on sampled rows of one sequence.  The oracle projects K and V for all 4096
+    rows of that sequence (attention needs them) and everything else for the sampled rows only."""
+    dt, B, S = torch.bfloat16, 4, 4096
+    s = O.RavenShape.nebel()
+    g = torch.Generator().manual_seed(31)
+    prefix = "blk"
+    w = {f"{prefix}.norm_{i}.weight": (torch.randn(H, generator=g) * 0.02 + 1).to(dt) for i in (1, 2, 3, 4)}
+    w[f"{prefix}.attn.Wqkv.weight"] = (torch.randn(3 * H, H, generator=g) * 0.02).to(dt)
+    w[f"{prefix}.attn.qk_bias"] = (torch.randn(2, 1, NH, HD, generator=g) * 0.02).to(dt)
+    w[f"{prefix}.attn.proj.weight"] = (torch.randn(H, H, generator=g) * 0.02).to(dt)
+    w[f"{prefix}.mlp.fc.weight"] = (torch.randn(2 * INTER, H, generator=g) * 0.02).to(dt)
+    w[f"{prefix}.mlp.proj.weight"] = (torch.randn(H, INTER, generator=g) * 0.02).to(dt)
+    dev = {k_: v_.cuda() for k_, v_ in w.items()}
+    x = _gpu_randn((B * S, H), 32)
+    table = O.rope_table(HD, s.block_size, s.rope_base).to(dt)
+    freqs = table.float().reshape(s.block_size, HD // 2, 2).contiguous().cuda()
+    kd = torch.zeros(1, B, NH, S, HD, dtype=dt, device="cuda")
+    vd = torch.zeros_like(kd)
+    cache = pkg.hip.make_cache(kd, vd)
+    dims = pkg.hip.make_dims(H, NH, INTER, s.norm_eps, dt)
+    blk = pkg.hip.make_block_weights(dev[f"{prefix}.norm_1.weight"], dev[f"{prefix}.norm_2.weight"], dev[f"{prefix}.norm_3.weight"],
+                                     dev[f"{prefix}.norm_4.weight"], dev[f"{prefix}.attn.Wqkv.weight"], dev[f"{prefix}.attn.qk_bias"],
+                                     dev[f"{prefix}.attn.proj.weight"], dev[f"{prefix}.mlp.fc.weight"], dev[f"{prefix}.mlp.proj.weight"])
+    ws = pkg.hip.block_workspace(dims, B * S, "cuda")
+    out = pkg.hip.sandwich_block(dims, blk, x, torch.empty_like(x), freqs, cache, 0, B, S, 0, ws)
+    torch.cuda.synchronize()
+
+    # ---- the oracle, sequence b, fp32-accumulate linears (the same mathematics; the CPU's bf16 GEMM would take minutes)
+    b = 2
+    rows = torch.tensor([0, 1, 15, 16, 63, 64, 255, 256, 1023, 2048, 3071, 4094, 4095])
+    O.set_linear_mode("f32")
+    try:
+        xb = x.view(B, S, H)[b].cpu()
+        n1 = O.rmsnorm(xb, w[f"{prefix}.norm_1.weight"], s.norm_eps)
+        wqkv = w[f"{prefix}.attn.Wqkv.weight"]
+        kv = O.linear(n1, wqkv[H:])                                     # K and V of every row of the sequence
+        k_all, v_all = kv[:, :H].view(1, S, NH, HD), kv[:, H:].view(1, S, NH, HD)
+        q_s = O.linear(n1[rows], wqkv[:H]).view(1, -1, NH, HD)          # queries of the sampled rows
+        bias = w[f"{prefix}.attn.qk_bias"]
+        k_all = (k_all + bias[1:2]).to(dt)
+        q_s = (q_s + bias[0:1]).to(dt)
+        _, k_rot = O.apply_rope(k_all, k_all, table[:, :S])
+        q_rot, _ = O.apply_rope(q_s, q_s, table[:, rows])
+        ya = []
+        for i, r in enumerate(rows.tolist()):                           # row r attends to positions 0 .. r
+            qi = q_rot[:, i:i + 1].transpose(1, 2)
+            ya.append(O.sdpa(qi, k_rot[:, :r + 1].transpose(1, 2), v_all[:, :r + 1].transpose(1, 2)).transpose(1, 2).reshape(1, H))
+        ya = torch.cat(ya, 0)
+        a = O.linear(ya, w[f"{prefix}.attn.proj.weight"])
+        x2 = O.rmsnorm(a + xb[rows], w[f"{prefix}.norm_2.weight"], s.norm_eps)
+        m = O.gated_mlp(O.rmsnorm(x2, w[f"{prefix}.norm_3.weight"], s.norm_eps), w, prefix)
+        want = O.rmsnorm(m + x2, w[f"{prefix}.norm_4.weight"], s.norm_eps)
+    finally:
+        O.set_linear_mode("native")
+    got = out.view(B, S, H)[b][rows.cuda()]
+    # the cache rows the block appended: rotated keys and values of every position, one kernel chain deep
+    check(kd[0, b].transpose(0, 1), k_rot[0], dt, "appended K of the sequence")
+    check(vd[0, b].transpose(0, 1), v_all[0], dt, "appended V of the sequence")
+    err = close(got, want, "block output rows")
+    print(f"SandwichBlock at 4 x 4096: sampled rows max-abs {err[0]:.3e} rel-L2 {err[1]:.3e}")
+    # a chain of five products and four norms: the composed bar of test_gpu_model.py (per-kernel bars are applied kernel
+    # by kernel above and in test_gpu_kernels.py)
+    assert err[1] <= 3e-2, f"block output: rel-L2 {err[1]:.3e}"
+    scale = max(1.0, want.float().abs().max().item())
+    assert err[0] <= 2.5 * 2e-2 * scale, f"block output: max-abs {err[0]:.3e}"
+    # rows of other sequences are finite and differ from this one's (no row was skipped or written twice)
+    assert torch.isfinite(out.float()).all()
+    assert not torch.equal(out.view(B, S, H)[0], out.view(B, S, H)[b])
+
+
+def test_bench_prefill_iteration_runs_through_the_c_abi(pkg):
+    """One recurrence over 4 x 512 rows through raven_core_iteration (adapter with two K segments, four blocks, chunk
+    attention over a cache that already holds 512 positions): determinism, and the call equals adapter + four
+    raven_sandwich_block calls bit for bit (one composition of the block behind the C ABI)."""
+    dt, B, S, T = torch.bfloat16, 4, 512, 512
+    s = O.RavenShape.nebel()
+    w = O.make_weights(s, seed=0, dtype=dt, only_core=True)
+    dev = {k_: v_.cuda() for k_, v_ in w.items()}
+    from test_gpu_model import _block_weights
+    blocks = (pkg.hip.BlockWeights * 4)(*[_block_weights(pkg, dev, f"transformer.core_block.{j}") for j in range(4)])
+    dims = pkg.hip.make_dims(H, NH, INTER, s.norm_eps, dt)
+    table = O.rope_table(HD, s.block_size, s.rope_base).to(dt)
+    freqs = table.float().reshape(s.block_size, HD // 2, 2).contiguous().cuda()
+    state, embeds = _gpu_randn((B * S, H), 41, 0.632), _gpu_randn((B * S, H), 42)
+    k0, v0 = _gpu_randn((4, B, NH, T + S, HD), 43), _gpu_randn((4, B, NH, T + S, HD), 44)
+    ws = pkg.hip.block_workspace(dims, B * S, "cuda")
+    outs = []
+    for _ in range(2):
+        kd, vd = k0.clone(), v0.clone()
+        out = torch.empty_like(state)
+        pkg.hip.core_iteration(dims, dev["transformer.adapter.weight"], blocks, state, embeds, out, freqs, pkg.hip.make_cache(kd, vd), 0, B, S,
+                               T, ws)
+        outs.append((out, kd, vd))
+    assert all(torch.equal(a, b) for a, b in zip(outs[0], outs[1]))
+    kd, vd = k0.clone(), v0.clone()
+    cache = pkg.hip.make_cache(kd, vd)
+    cur = pkg.hip.linear(state, dev["transformer.adapter.weight"], x1=embeds)
+    for j in range(4):
+        nxt = torch.empty_like(cur)
+        pkg.hip.sandwich_block(dims, blocks[j], cur, nxt, freqs, cache, j, B, S, T, ws)
+        cur = nxt
+    assert torch.equal(cur, outs[0][0]) and torch.equal(kd, outs[0][1]) and torch.equal(vd, outs[0][2])
+    assert torch.isfinite(cur.float()).all()
