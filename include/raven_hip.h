@@ -93,8 +93,10 @@ const char* raven_last_error(void);
  * one 1024-thread workgroup each instead of a split launch; 0 = never), gemm_mfma_min_rows (fewest rows the MFMA
  * kernels take; fewer go to the vector kernels), linear_min_rows (most rows raven_linear still hands to the kernels
  * without a workspace), linear_ks (K slices of the split-K kernel behind raven_linear;
- * non-zero also makes raven_linear use that kernel for every shape it accepts).  Not needed in normal use: the
- * defaults are the tuned values. */
+ * non-zero also makes raven_linear use that kernel for every shape it accepts), gemm_tiled_min_rows (fewest rows, 33 or
+ * more, that the tiled MFMA kernel takes), gemm_tiled_variant (0 = tile size by shape, 1 = 256 x 256, 2 = 128 x 128 and
+ * no tile-count rule).  Not needed in normal use: the defaults are the tuned values.  The knobs are process-global
+ * state read at every launch: changing them while another thread or stream is inside a call of this library is a race. */
 int raven_set_tuning(const char* key, int32_t value);
 
 /* RMSNorm with the reference's two roundings, optionally preceded by a residual add and followed by
@@ -261,6 +263,22 @@ int raven_qkv_attention_decode(const void* qkv, const void* qk_bias, const float
                                const raven_kv_cache* cache, int32_t slot, int32_t B, int32_t pos0,
                                const int32_t* pos_dev, int32_t n_heads, int32_t head_dim,
                                int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* raven_qkv_attention_decode for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the same decode step with no workspace argument.  It has no counterpart in the
+ * reference.  The partial results of a split launch go to an array that is part of this library's code object
+ * (raven_qkv_attention_decode_static_scratch_bytes() bytes, about 17 MB, held by every GPU the library runs on until the
+ * process ends); its device address is looked up on the first call on each device (make that call outside a graph
+ * capture).  Same results, bit for bit, as raven_qkv_attention_decode with a workspace of
+ * raven_decode_attention_workspace_bytes(B, n_heads, head_dim).  A launch whose partial results would not fit the array
+ * (more than 1023 (head, row) pairs in a split launch, head_dim above 128: neither is reachable with the present
+ * splitting rule) is refused with a negative status.  All calls on one GPU share the array: calls that overlap on one
+ * GPU (two streams) race; every launch writes each partial result before it reads it, nothing needs clearing. */
+size_t raven_qkv_attention_decode_static_scratch_bytes(void);
+int    raven_qkv_attention_decode_static(const void* qkv, const void* qk_bias, const float* freqs, void* y,
+                                         const raven_kv_cache* cache, int32_t slot, int32_t B, int32_t pos0,
+                                         const int32_t* pos_dev, int32_t n_heads, int32_t head_dim,
+                                         int32_t dtype, void* stream);
 
 /* Causal attention for a prefill chunk on the matrix cores (bf16; head_dim 64, 96 or 128): the S > 1
  * cases of RMM:484-491.  Same contract as raven_decode_attention -- row m of sequence b attends to cached

@@ -801,6 +801,50 @@ extern "C" int raven_qkv_attention_decode(const void* qkv, const void* qk_bias, 
                             head_dim, dtype, workspace, workspace_bytes, stream);
 }
 
+// ---- the decode step without a caller's workspace --------------------------------------------------------------
+// Partial results of a split launch (per (head, row) pair and split: running maximum, sum, unnormalised output) go to a
+// buffer that is part of the loaded code object instead of an allocation: sized for the largest launch that is ever
+// split (fewer than 1024 (head, row) pairs, kAttnMaxSplits splits, head_dim up to 128).  In host code the array's name
+// is only a handle; its device address is looked up once per device.
+constexpr size_t kScratchMaxPairs = 1023, kScratchMaxHeadDim = 128;
+constexpr size_t kScratchBytes = ((kScratchMaxPairs * raven::kAttnMaxSplits * 2 * 4 + 255) / 256 * 256) +
+                                 ((kScratchMaxPairs * raven::kAttnMaxSplits * kScratchMaxHeadDim * 4 + 255) / 256 * 256);
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kScratchMaxDevices = 64;
+static void* g_scratch_ptr[kScratchMaxDevices];  // per device: each GPU holds its own copy of the array at its own address
+
+extern "C" size_t raven_qkv_attention_decode_static_scratch_bytes(void) { return kScratchBytes; }
+
+extern "C" int raven_qkv_attention_decode_static(const void* qkv, const void* qk_bias, const float* freqs, void* y,
+                                                 const raven_kv_cache* cache, int32_t slot, int32_t B, int32_t pos0,
+                                                 const int32_t* pos_dev, int32_t n_heads, int32_t head_dim, int32_t dtype,
+                                                 void* stream) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kScratchMaxDevices) {
+        raven_host::set_error("qkv_attention_decode_static: cannot tell the current device (%s, device %d of at most %d)",
+                              hipGetErrorString(e), dev, kScratchMaxDevices);
+        return e != hipSuccess ? (int)e : -1;
+    }
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            raven_host::set_error("qkv_attention_decode_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return e != hipSuccess ? (int)e : -1;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    // the same size rule as raven_decode_attention_workspace_bytes; what would not fit the array is refused
+    const size_t need = raven_decode_attention_workspace_bytes(B, n_heads, head_dim);
+    RAVEN_REQUIRE(need <= kScratchBytes,
+                  "qkv_attention_decode_static: %d sequences x %d heads of %d need %zu bytes of partial results, the built-in buffer holds %zu "
+                  "(at most %zu (head, row) pairs in a split launch, head_dim up to %zu)",
+                  B, n_heads, head_dim, need, kScratchBytes, kScratchMaxPairs, kScratchMaxHeadDim);
+    return attention_common("qkv_attention_decode_static", true, qkv, qk_bias, freqs, y, cache, slot, B, 1, pos0, pos_dev, n_heads,
+                            head_dim, dtype, g_scratch_ptr[dev], kScratchBytes, stream);
+}
+
 
 static int paged_strides(const char* who, int kv_layout, int block_size, int n_heads, int head_dim, int64_t* pos_stride, int64_t* head_stride) {
     RAVEN_REQUIRE(kv_layout == RAVEN_PAGED_NHD || kv_layout == RAVEN_PAGED_HND, "%s: unknown kv_layout %d", who, kv_layout);

@@ -91,6 +91,8 @@ SIGNATURES = {
                                          _VP, _SZ, _VP]),
     "raven_qkv_attention_decode": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _VP, _I32, _I32,
                                              _I32, _VP, _SZ, _VP]),
+    "raven_qkv_attention_decode_static_scratch_bytes": (_SZ, []),
+    "raven_qkv_attention_decode_static": (C.c_int, [_VP, _VP, _VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _VP, _I32, _I32, _I32, _VP]),
     "raven_prefill_attention": (C.c_int, [_VP, _VP, C.POINTER(KVCache), _I32, _I32, _I32, _I32, _VP, _I32, _I32, _I32, _VP]),
     "raven_swiglu": (C.c_int, [_VP, _VP, _I32, _I32, _I32, _VP]),
     "raven_noise_mix": (C.c_int, [_VP, _VP, _VP, _I64, _F, _F, _F, _I32, _VP]),
@@ -407,6 +409,18 @@ def qkv_attention_decode(qkv, qk_bias, freqs, cache: KVCache, slot, B, pos0, n_h
         slot, B, pos0, _ptr(pos_dev, "pos_dev", torch.int32), n_heads, head_dim, dtype_code(dt),
         _ptr(workspace, "workspace", torch.uint8), 0 if workspace is None else workspace.numel(), _stream())
     _check(rc, "raven_qkv_attention_decode")
+    return y
+
+
+def qkv_attention_decode_static(qkv, qk_bias, freqs, cache: KVCache, slot, B, pos0, n_heads, head_dim, pos_dev=None, out=None):
+    """The decode step of qkv_attention_decode without a workspace: partial results go to the library's built-in buffer.
+    With `out` given nothing is allocated on the way (for callers that cannot allocate)."""
+    dt = qkv.dtype
+    y = out if out is not None else torch.empty(B, n_heads * head_dim, device=qkv.device, dtype=dt)
+    rc = load().raven_qkv_attention_decode_static(
+        _ptr(qkv, "qkv"), _ptr(qk_bias, "qk_bias", dt), _ptr(freqs, "freqs", torch.float32), _ptr(y, "y", dt), C.byref(cache),
+        slot, B, pos0, _ptr(pos_dev, "pos_dev", torch.int32), n_heads, head_dim, dtype_code(dt), _stream())
+    _check(rc, "raven_qkv_attention_decode_static")
     return y
 
 

@@ -239,7 +239,9 @@ def test_decode_runner_beyond_one_pass_of_rows_bf16(pkg, tiny16, use_graph):
         logits, nxt, lat = runner.step(tok.cuda(), st.cuda())
         check(logits, want.logits[:, 0], torch.bfloat16, f"runner logits, token {i}")
         check(lat, want.latent_states[:, 0], torch.bfloat16, f"runner latents, token {i}")
-        assert torch.equal(logits, fwd.logits[:, 0]), f"token {i}: runner and forward() launch the same kernels"
+        # the same kernels as forward(); only the number of workgroups that share a sequence's positions follows the
+        # cache capacity in the runner (its launch shapes must serve every later token) and the position in forward()
+        check(logits, fwd.logits[:, 0], torch.bfloat16, f"token {i}: runner against forward()")
         assert torch.equal(nxt.cpu(), logits.argmax(-1).cpu())
     assert cache.get_seq_length() == ref_cache.get_seq_length() == S + n_new
     assert (runner.graph is not None) == use_graph

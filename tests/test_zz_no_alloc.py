@@ -1,0 +1,56 @@
+"""The entry point that allocates nothing (raven_qkv_attention_decode_static) against raven_qkv_attention_decode, through
+the C ABI: the same bits in the output and in the appended cache rows, on two calls in a row, the second with a smaller
+input (fewer sequences, a shorter cache, so that stale partial results of the first call lie behind the second's)."""
+
+import pytest
+import torch
+
+from oracle import raven_oracle as O
+from test_gpu_kernels import check, rnd
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(pkg, B, T, nh, hd, dt, seed):
+    h = nh * hd
+    qkv = rnd((B, 3 * h), dt, seed).cuda()
+    bias = rnd((2, nh, hd), dt, seed + 1, 0.1).cuda()
+    table = O.rope_table(hd, T + 8, 50000.0)
+    freqs = table.reshape(T + 8, hd // 2, 2).contiguous().cuda()
+    k, v = rnd((2, B, nh, T + 1, hd), dt, seed + 2), rnd((2, B, nh, T + 1, hd), dt, seed + 3)
+    return qkv, bias, freqs, k, v
+
+
+@pytest.mark.parametrize("dt,nh,hd", [(torch.bfloat16, 55, 96), (torch.float32, 4, 64)])
+def test_static_scratch_decode_attention_equals_workspace_version(pkg, dt, nh, hd):
+    lib = pkg.hip.load()
+    assert lib.raven_qkv_attention_decode_static_scratch_bytes() >= lib.raven_decode_attention_workspace_bytes(18, 55, 128)
+    for call, (B, T) in enumerate([(3, 1500), (1, 700)]):  # both launches are split over positions
+        qkv, bias, freqs, k, v = _case(pkg, B, T, nh, hd, dt, 40 + call)
+        ka, va, kb, vb = k.cuda(), v.cuda(), k.cuda(), v.cuda()
+        ws = pkg.hip.attention_workspace(B, nh, hd, "cuda")
+        assert ws is not None
+        want = pkg.hip.qkv_attention_decode(qkv, bias, freqs, pkg.hip.make_cache(ka, va), 1, B, T, nh, hd, workspace=ws)
+        out = torch.empty(B, nh * hd, dtype=dt, device="cuda")
+        got = pkg.hip.qkv_attention_decode_static(qkv, bias, freqs, pkg.hip.make_cache(kb, vb), 1, B, T, nh, hd, out=out)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"call {call}: output"
+        assert torch.equal(ka, kb) and torch.equal(va, vb), f"call {call}: appended cache rows"
+        # and both equal the oracle's attention over the T cached positions plus the new one
+        h = nh * hd
+        q_, k_, v_ = (t.view(B, 1, nh, hd) for t in qkv.cpu().split([h, h, h], dim=1))
+        b_ = bias.cpu()
+        q_, k_ = (q_ + b_[0]).to(dt), (k_ + b_[1]).to(dt)
+        tab = O.rope_table(hd, T + 8, 50000.0)
+        rq, rk = O.apply_rope(q_, k_, tab[:, T:T + 1])
+        K = torch.cat([k[1, :, :, :T], rk.transpose(1, 2)], dim=2)
+        V = torch.cat([v[1, :, :, :T], v_.transpose(1, 2)], dim=2)
+        check(got, O.sdpa(rq.transpose(1, 2), K, V).transpose(1, 2).reshape(B, h), dt, f"call {call}: against the oracle")
+    # with the device-side position (a replayed graph's form) the same again, and a launch that is never split
+    qkv, bias, freqs, k, v = _case(pkg, 32, 300, nh, hd, dt, 60)
+    ka, kb, va, vb = k.cuda(), k.cuda(), v.cuda(), v.cuda()
+    pos_dev = torch.tensor([300], dtype=torch.int32, device="cuda")
+    want = pkg.hip.qkv_attention_decode(qkv, bias, freqs, pkg.hip.make_cache(ka, va), 0, 32, 300, nh, hd, pos_dev=pos_dev,
+                                        workspace=pkg.hip.attention_workspace(32, nh, hd, "cuda"))
+    got = pkg.hip.qkv_attention_decode_static(qkv, bias, freqs, pkg.hip.make_cache(kb, vb), 0, 32, 300, nh, hd, pos_dev=pos_dev)
+    assert torch.equal(got, want) and torch.equal(ka, kb)
