@@ -475,13 +475,26 @@ def forward(w, s: RavenShape, input_ids=None, input_embeds=None, input_states=No
     return OracleOutput(logits=logits, latent_states=latents, past_key_values=cache, hidden_states=x)
 
 
+def repetition_penalty(logits: torch.Tensor, ids: torch.Tensor, penalty: float) -> torch.Tensor:
+    """The standard penalty of RMM:2047-2061 on [B, V] logits: every token that occurs in the row's sequence so far has
+    its logit divided by the penalty when positive and multiplied when negative."""
+    out = logits.to(copy=True, dtype=torch.float32)
+    for b in range(out.shape[0]):
+        seen = torch.unique(ids[b])
+        vals = out[b, seen]
+        out[b, seen] = torch.where(vals < 0, vals * penalty, vals / penalty)
+    return out
+
+
 def greedy_generate(w, s: RavenShape, input_ids: torch.Tensor, max_new_tokens: int, num_steps=None,
-                    state_fn=None, stop_tokens=(), record: Optional[dict] = None) -> torch.Tensor:
+                    state_fn=None, stop_tokens=(), record: Optional[dict] = None,
+                    penalty: Optional[float] = None) -> torch.Tensor:
     """The greedy branch of generate_minimal (RMM:1165-1232, argmax at RMM:1988-1989).
 
     `state_fn(call_index, embeds_shape)` supplies the latent state injected into each forward (the
     reference draws it from the global RNG on every call, RMM:738; parity runs inject it instead).
     `record`, if given, receives per-token top-2 logit margins and the cache object.
+    `penalty`: generation_config.repetition_penalty (RMM:1946-1947, 2047-2061).
     """
     cache = DictCache()
     ids = input_ids.clone()
@@ -496,6 +509,8 @@ def greedy_generate(w, s: RavenShape, input_ids: torch.Tensor, max_new_tokens: i
                       past_key_values=cache, use_cache=True, cache_position=pos,
                       init_scale=0.0 if state_fn is None else 1.0)
         last = out.logits[:, -1, :].float()
+        if penalty is not None and penalty != 1.0:  # RMM:1946-1947: over the whole sequence so far, on every step
+            last = repetition_penalty(last, ids, penalty)
         top2 = last.topk(2, dim=-1).values
         margins.append((top2[:, 0] - top2[:, 1]).tolist())
         nxt = last.argmax(dim=-1, keepdim=True)

@@ -7,8 +7,8 @@ state dict loads with `load_state_dict` unchanged.
 
 What differs from the reference on purpose:
   * token rows are processed as [B*S, h]; K/V live in one contiguous step-indexed buffer;
-  * positions must be contiguous and, when a cache is given, continue the cache
-    (position == cache index); anything else raises NotImplementedError;
+  * positions are one 1-D list shared by the batch, as in the reference (RMM:660-665); when they are not the tokens'
+    cache indices the call rotates with a table gathered for it;
   * `attention_mask` is accepted and ignored, as in the reference (RMM:676);
   * only inference: no autograd, no labels-driven backward (a loss value is still returned).
 """
@@ -156,6 +156,7 @@ class RavenForCausalLM(torch.nn.Module):
         self.noise_source = None  # test-time noise draws: an object with normal(x) and uniform(x); None = torch's generator
         self._native_key = None
         self._native: dict = {}
+        self._rope_override: Optional[torch.Tensor] = None  # a forward with positions that are not the cache's (see _rope_table_for)
         self._scratch: dict = {}
         self.eval()
 
@@ -331,17 +332,33 @@ class RavenForCausalLM(torch.nn.Module):
             self._scratch[key] = c
         return c
 
-    def _positions(self, n_tokens: int, position_ids, cache_position) -> int:
-        """First RoPE position of this call (RMM:660-665); positions must be contiguous."""
+    def _rope_positions(self, n_tokens: int, position_ids, cache_position) -> list:
+        """The RoPE positions of this call's tokens, shared by the batch (RMM:660-665): `position_ids` squeezed to one
+        dimension, else `cache_position`, else 0 .. S-1.  Any values inside the table are allowed; they only pick rows of
+        the RoPE table, the cache index of a token is the number of tokens the cache has seen."""
         src = position_ids if position_ids is not None else cache_position
         if src is None:
-            return 0
-        pos = src.reshape(-1)[-n_tokens:].tolist() if src.numel() >= n_tokens else src.reshape(-1).tolist()
-        if len(pos) != n_tokens or any(pos[i] != pos[0] + i for i in range(n_tokens)):
-            raise NotImplementedError("positions must be one contiguous range shared by the batch")
-        if pos[0] + n_tokens > self.config.block_size:
-            raise ValueError(f"positions up to {pos[0] + n_tokens - 1} exceed block_size {self.config.block_size}")
-        return int(pos[0])
+            return list(range(n_tokens))
+        pos = [int(v) for v in src.reshape(-1).tolist()]
+        if len(pos) != n_tokens:
+            raise ValueError(f"{len(pos)} positions for {n_tokens} tokens: positions are one 1-D list shared by the batch")
+        if min(pos) < 0 or max(pos) >= self.config.block_size:
+            raise IndexError(f"positions {min(pos)} .. {max(pos)} outside the RoPE table of {self.config.block_size} rows")
+        return pos
+
+    def _rope_table_for(self, rope_pos: list, cache_pos0: int) -> Optional[torch.Tensor]:
+        """None when the tokens' RoPE positions are their cache positions (cache_pos0, cache_pos0 + 1, ...): the kernels
+        then read the model's table.  Otherwise a table for this call whose rows cache_pos0 + i hold the model's rows
+        rope_pos[i] (the kernels rotate the token at cache index p with row p)."""
+        if all(p == cache_pos0 + i for i, p in enumerate(rope_pos)):
+            return None
+        full = self._natives()["freqs"]
+        table = torch.zeros(cache_pos0 + len(rope_pos), full.shape[1], 2, dtype=full.dtype, device=full.device)
+        table[cache_pos0:] = full[torch.as_tensor(rope_pos, device=full.device)]
+        return table
+
+    def _freqs(self) -> torch.Tensor:
+        return self._rope_override if self._rope_override is not None else self._natives()["freqs"]
 
     def _split_steps(self, num_steps) -> int:
         """Total recurrences (RMM:739-744; eval sampler RMM:799-802)."""
@@ -360,7 +377,7 @@ class RavenForCausalLM(torch.nn.Module):
         slot = 0 if private else cache.note_append(step_idx, S, pos0)
         kv = cache.native() if private else cache.native([step_idx], pos0)
         out = torch.empty_like(x)
-        hip.sandwich_block(nat["dims"], nat[which][i], x, out, nat["freqs"], kv, slot, B, S, pos0,
+        hip.sandwich_block(nat["dims"], nat[which][i], x, out, self._freqs(), kv, slot, B, S, pos0,
                            self._workspace(B * S), ln_f=self.transformer.ln_f.weight if ln_f else None)
         return out
 
@@ -415,7 +432,7 @@ class RavenForCausalLM(torch.nn.Module):
         ws = self._workspace(B * S)
         lnw = t.ln_f.weight if ln_f else None
         if not private and uniform and n_core > 0 and all(slots[j] == slots[0] + j for j in range(n_core)):
-            hip.core_iteration(nat["dims"], t.adapter.weight, nat["core"], x, embeds, out, nat["freqs"], kv,
+            hip.core_iteration(nat["dims"], t.adapter.weight, nat["core"], x, embeds, out, self._freqs(), kv,
                                slots[0], B, S, pos0, ws, ln_f=lnw)
             return out
         cur = hip.linear(x, t.adapter.weight, x1=embeds, workspace=ws)  # the kernels raven_core_iteration would pick
@@ -423,7 +440,7 @@ class RavenForCausalLM(torch.nn.Module):
             last = j == n_core - 1
             nxt = out if last else torch.empty_like(x)
             kv_j = kv if uniform else cache.native([steps[j]], pos0)
-            hip.sandwich_block(nat["dims"], nat["core"][j], cur, nxt, nat["freqs"], kv_j, slots[j], B, S, pos0, ws,
+            hip.sandwich_block(nat["dims"], nat["core"][j], cur, nxt, self._freqs(), kv_j, slots[j], B, S, pos0, ws,
                                ln_f=lnw if last else None)
             cur = nxt
         if n_core == 0:
@@ -481,13 +498,22 @@ class RavenForCausalLM(torch.nn.Module):
         src = input_ids if input_embeds is None else input_embeds
         B, S = src.shape[0], src.shape[1]
         M, h = B * S, cfg.n_embd
-        rope_pos0 = self._positions(S, position_ids, cache_position)
+        rope_pos = self._rope_positions(S, position_ids, cache_position)
         r = self._split_steps(num_steps)
         cache, private, pos0 = self._prepare_cache(past_key_values, use_cache, B, S, r)
-        if rope_pos0 != pos0 and not (private and position_ids is None and cache_position is None):
-            raise NotImplementedError(f"positions start at {rope_pos0} but the cache holds {pos0} tokens")
+        override = self._rope_table_for(rope_pos, pos0)
         if not private:
             cache._seen_tokens += S  # what the step-0 update does in the reference (RMM:188-189)
+        self._rope_override = override
+        try:
+            return self._forward_rows(input_ids, input_embeds, input_states, labels, output_details, init_scale, cache, private, pos0,
+                                      B, S, r)
+        finally:
+            self._rope_override = None
+
+    def _forward_rows(self, input_ids, input_embeds, input_states, labels, output_details, init_scale, cache, private, pos0, B, S, r):
+        cfg, t = self.config, self.transformer
+        M, h = B * S, cfg.n_embd
 
         if input_embeds is None:
             x = hip.embed(t.wte.weight, input_ids.reshape(-1).to(torch.int64).contiguous(), self.emb_scale)
@@ -612,17 +638,19 @@ class RavenForCausalLM(torch.nn.Module):
         """RMM:902-934: embedding times sqrt(h), then the prelude; returns (embeds, block_idx)."""
         cfg, t = self.config, self.transformer
         B, S = input_ids.shape
-        rope_pos0 = self._positions(S, position_ids, cache_position)
+        rope_pos = self._rope_positions(S, position_ids, cache_position)
         cache, private, pos0 = self._prepare_cache(past_key_values, use_cache, B, S, 0)
-        if rope_pos0 != pos0 and not (private and position_ids is None and cache_position is None):
-            raise NotImplementedError(f"positions start at {rope_pos0} but the cache holds {pos0} tokens")
+        self._rope_override = self._rope_table_for(rope_pos, pos0)
         if not private:
             cache._seen_tokens += S
-        x = hip.embed(t.wte.weight, input_ids.reshape(-1).to(torch.int64).contiguous(), self.emb_scale)
-        block_idx = -1
-        for i in range(len(t.prelude)):
-            block_idx += 1
-            x = self._run_block("prelude", i, block_idx, x, cache, private, B, S, pos0)
+        try:
+            x = hip.embed(t.wte.weight, input_ids.reshape(-1).to(torch.int64).contiguous(), self.emb_scale)
+            block_idx = -1
+            for i in range(len(t.prelude)):
+                block_idx += 1
+                x = self._run_block("prelude", i, block_idx, x, cache, private, B, S, pos0)
+        finally:
+            self._rope_override = None
         return x.view(B, S, cfg.n_embd), torch.tensor(block_idx, dtype=torch.long)
 
     # ---- generation --------------------------------------------------------------------------------
@@ -799,14 +827,20 @@ class RavenForCausalLM(torch.nn.Module):
 
         runner = None
         call = 1
+        # the penalties look at the growing sequence on every step (RMM:1198-1201, 1946-1947); with one configured the
+        # pick is made from the penalised logits on the greedy path too
+        penalised = getattr(gc, "repetition_penalty", None) is not None and gc.repetition_penalty != 1.0
+        pick_on_host = bool(getattr(gc, "do_sample", False)) or penalised
+        all_ids = torch.cat([input_ids, next_tok], dim=-1) if pick_on_host else None
         while len(tokens) < max_new and update_alive(tokens[-1]) and cache.get_seq_length() + 1 <= total:
             if runner is None:
                 runner = DecodeRunner(self, cache, B, self._split_steps(num_steps), greedy=not getattr(gc, "do_sample", False),
                                       use_graph=use_graph)
             state = carried if continuous_compute else state_for(call, 1)
             logits, nxt, latents = runner.step(tokens[-1].view(-1), state, init_scale)
-            if getattr(gc, "do_sample", False):
-                nxt = self._sample_next_token(logits, input_ids, gc).view(-1)
+            if pick_on_host:
+                nxt = self._sample_next_token(logits, all_ids, gc).view(-1)
+                all_ids = torch.cat([all_ids, nxt.view(B, 1)], dim=-1)
             tokens.append(nxt.view(B, 1).clone())
             if continuous_compute:
                 carried = latents.view(B, 1, -1).clone()
@@ -848,7 +882,7 @@ class DecodeRunner:
         self.ws = hip.block_workspace(model._natives()["dims"], batch, dev)
         self.use_graph = use_graph and cfg.test_time_noise <= 0  # the noise draws are not part of a replayable launch sequence
         self.graph: Optional[torch.cuda.CUDAGraph] = None
-        self._graph_t_max = None
+        self._graph_key = None
         self._warm = False
 
     def _slots(self):
@@ -913,6 +947,8 @@ class DecodeRunner:
         The returned tensors are the runner's own buffers: copy what must outlive the next step."""
         m, c = self.model, self.cache
         pos0 = c._seen_tokens
+        if pos0 + 1 > m.config.block_size:
+            raise ValueError(f"position {pos0} lies past the RoPE table (block_size {m.config.block_size})")
         last_step = m.config.n_layers_in_prelude + m.config.n_layers_in_recurrent_block * self.r - 1
         if c.has_gap(last_step, pos0):
             raise NotImplementedError("the decode runner's fixed launch sequence needs a cache whose earlier tokens were all "
@@ -930,11 +966,14 @@ class DecodeRunner:
         else:
             self.state.copy_(state.reshape(self.B, -1))
         if self.use_graph and self._warm:
-            if self.graph is None or self._graph_t_max != c.t_max:
+            # the captured launches hold the cache's pointers, slot numbers and capacity: any reallocation (more
+            # positions, more step slots) makes them stale
+            key = (c._k.data_ptr(), c._v.data_ptr(), tuple(c._k.shape), c._neg_slots)
+            if self.graph is None or self._graph_key != key:
                 self.graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(self.graph):
                     self._enqueue()
-                self._graph_t_max = c.t_max
+                self._graph_key = key
                 self.pos.fill_(pos0)  # capture does not execute; make sure the counter is what this step needs
             self.graph.replay()
         else:

@@ -112,7 +112,7 @@ class PagedDecoder:
     @torch.no_grad()
     def forward_tokens(self, input_ids: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor, block_table: torch.Tensor,
                        seq_lens: torch.Tensor, query_start_loc: torch.Tensor, max_query_len: int,
-                       input_states: Optional[torch.Tensor] = None, init_scale: float = 1.0):
+                       input_states: Optional[torch.Tensor] = None, init_scale: float = 1.0, check_bounds: bool = True):
         """What the plugin's model computes for one scheduler step (RavenModel.forward, vllm/raven_vllm.py:374-411), straight on
         the pages: input_ids [T] are the new rows of B sequences, flattened (prompt chunks of any length and decode rows
         together); positions [T] and slot_mapping [T] (int64) say where each row sits; sequence b owns rows
@@ -125,6 +125,8 @@ class PagedDecoder:
         B = seq_lens.shape[0]
         if positions.shape != (T,) or slot_mapping.shape != (T,) or query_start_loc.shape != (B + 1,) or block_table.shape[0] != B:
             raise ValueError("positions [T], slot_mapping [T], block_table [B, max_blocks], seq_lens [B], query_start_loc [B + 1]")
+        if check_bounds:
+            self._check_pages(block_table, seq_lens, positions, slot_mapping)
         dev = m.device
         meta = (positions.to(dev, torch.int64), slot_mapping.to(dev, torch.int64), block_table.to(dev, torch.int32).contiguous(),
                 seq_lens.to(dev, torch.int32), query_start_loc.to(dev, torch.int32), int(max_query_len))
@@ -211,15 +213,46 @@ class PagedDecoder:
                                    cfg.padded_vocab_size, cfg.n_embd, hip.dtype_code(m.dtype), 1, hip._stream())
         hip._check(rc, "raven_gemm")
 
+    def _check_pages(self, block_table: torch.Tensor, seq_lens: torch.Tensor, positions: Optional[torch.Tensor] = None,
+                     slot_mapping: Optional[torch.Tensor] = None) -> None:
+        """The kernels index the RoPE table by position and the pages through the block table without looking: whatever
+        they will dereference is checked here, on host copies (one device-to-host read when the tensors live on the GPU)."""
+        lens = seq_lens.detach().to("cpu", torch.int64)
+        table = block_table.detach().to("cpu", torch.int64)
+        n_pos = self.cfg.block_size  # rows of the RoPE table
+        if lens.numel() and (int(lens.min()) < 0 or int(lens.max()) > n_pos):
+            raise ValueError(f"seq_lens must lie in [0, {n_pos}] (the RoPE table has {n_pos} positions); got up to {int(lens.max())}")
+        if lens.numel() and int(lens.max()) > table.shape[1] * self.block_size:
+            raise ValueError(f"a sequence of {int(lens.max())} positions does not fit {table.shape[1]} blocks of {self.block_size}")
+        used = (lens + self.block_size - 1) // self.block_size
+        mask = torch.arange(table.shape[1])[None, :] < used[:, None]
+        if mask.any():
+            ids = table[mask]
+            if int(ids.min()) < 0 or int(ids.max()) >= self.num_blocks:
+                raise ValueError(f"block_table names block {int(ids.max() if ids.max() >= self.num_blocks else ids.min())}; "
+                                 f"the caches have {self.num_blocks}")
+        if positions is not None and positions.numel():
+            pos = positions.detach().to("cpu", torch.int64)
+            if int(pos.min()) < 0 or int(pos.max()) >= n_pos:
+                raise ValueError(f"positions must lie in [0, {n_pos}); got {int(pos.min())} .. {int(pos.max())}")
+        if slot_mapping is not None and slot_mapping.numel():
+            slots = slot_mapping.detach().to("cpu", torch.int64)
+            if int(slots.max()) >= self.num_blocks * self.block_size:
+                raise ValueError(f"slot_mapping names slot {int(slots.max())}; the caches have {self.num_blocks * self.block_size}")
+
     def step(self, ids: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor, input_states: Optional[torch.Tensor] = None,
-             init_scale: float = 1.0):
+             init_scale: float = 1.0, check_bounds: bool = True):
         """One new token per sequence.  ids [B]; block_table [B, max_blocks] int32; seq_lens [B] int32 = each sequence's
         length INCLUDING the new token (its position is seq_lens - 1; the page for it must be in the table).
-        Returns (logits [B, V] float32, latents [B, h]); both are buffers reused by the next step of the same batch size."""
+        Returns (logits [B, V] float32, latents [B, h]); both are buffers reused by the next step of the same batch size.
+        check_bounds=False skips the host-side validation of seq_lens / block_table (a caller that builds them itself and
+        keeps them on the GPU saves one device-to-host read per step)."""
         m = self.model
         B = ids.shape[0]
         if block_table.dim() != 2 or block_table.shape[0] != B or seq_lens.shape != (B,):
             raise ValueError("block_table [B, max_blocks] and seq_lens [B] must match ids [B]")
+        if check_bounds:
+            self._check_pages(block_table, seq_lens)
         buf = self._buffers(B, block_table.shape[1])
         buf["ids"].copy_(ids.view(-1))
         buf["table"].copy_(block_table)

@@ -3,10 +3,9 @@ small number of recurrences, drops them from the cache, and verifies all of them
 number of recurrences -- a chunk of `lookahead_for_draft` rows through the same kernels a prefill uses.
 
 The loop is the reference's, tensor operation by tensor operation (including what it does to batches: sequences
-that accept fewer tokens are padded with `pad_id` and the cache is rolled back to the shortest accepted prefix).
-One difference follows from the package's forward: once the sequences of a batch have accepted different numbers of
-tokens, the reference goes on with RoPE positions that differ from the cache positions; forward() raises
-NotImplementedError for such calls, so batches run as long as their sequences accept in step (always for B = 1)."""
+that accept fewer tokens are padded with `pad_id` and the cache is rolled back to the shortest accepted prefix; once
+the sequences of a batch have accepted different numbers of tokens the loop goes on, as the reference's does, with
+RoPE positions that differ from the cache positions -- forward() rotates by the positions it is given)."""
 
 from __future__ import annotations
 

@@ -98,8 +98,28 @@ def test_forward_with_cache_prefill_then_decode_and_cache_contents(pkg, tiny32):
     again = model(input_ids=ids[:, 5:7].cuda(), input_states=states[:, 5:7].cuda(), past_key_values=cache, use_cache=True,
                   cache_position=torch.arange(5, 7).cuda())
     check(again.logits[:, -1], got.logits[:, -1], torch.float32, "after clear_last_k_entries")
-    with pytest.raises(NotImplementedError):
-        model(input_ids=ids[:, :2].cuda(), past_key_values=cache, use_cache=True, cache_position=torch.arange(0, 2).cuda())
+    # any 1-D positions shared by the batch pick the RoPE rows (RMM:660-665); the cache index of the new tokens is the
+    # number of tokens seen.  Non-contiguous positions through cache_position, then through position_ids, then none at all
+    # (rows 0 .. S-1) on top of the cached tokens; the oracle's dict cache goes through the same calls.
+    O.forward(w, s, input_ids=ids[:, 5:7], input_states=states[:, 5:7], past_key_values=ref_cache, use_cache=True,
+              cache_position=torch.arange(5, 7))  # the oracle's cache redoes the two tokens too
+    g2 = torch.Generator().manual_seed(55)
+    for kind, pos in (("cache_position", torch.tensor([3, 9])), ("position_ids", torch.tensor([[11, 2]])), ("none", None)):
+        tok = torch.randint(0, s.vocab_size, (2, 2), generator=g2)
+        st = O.initialize_state(torch.empty(2, 2, s.n_embd), s, 1.0, g2)
+        kw_ref = {} if pos is None else {kind: pos}
+        kw = {} if pos is None else {kind: pos.cuda()}
+        want_p = O.forward(w, s, input_ids=tok, input_states=st, past_key_values=ref_cache, use_cache=True, **kw_ref)
+        got_p = model(input_ids=tok.cuda(), input_states=st.cuda(), past_key_values=cache, use_cache=True, **kw)
+        check(got_p.logits, want_p.logits, torch.float32, f"positions through {kind}")
+        assert cache.get_seq_length() == ref_cache.get_seq_length()
+    n_seen = cache.get_seq_length()
+    for step in (0, 2, -1):
+        check(cache.key_cache[step][n_seen - 1], ref_cache.key_cache[step][n_seen - 1], torch.float32, f"K[{step}] under free positions")
+    with pytest.raises(IndexError):
+        model(input_ids=ids[:, :2].cuda(), past_key_values=cache, use_cache=True, cache_position=torch.tensor([0, s.block_size]).cuda())
+    with pytest.raises(ValueError):
+        model(input_ids=ids[:, :2].cuda(), past_key_values=cache, use_cache=True, cache_position=torch.arange(3).cuda())
 
 
 @pytest.mark.parametrize("use_graph", [False, True])
@@ -129,6 +149,39 @@ def test_greedy_batch_and_zero_state_and_stop(tiny32):
     want_s = O.greedy_generate(w, s, prompt[:1], 12, stop_tokens={stop})
     got_s = model.generate(prompt[:1].cuda(), max_new_tokens=12, init_scale=0.0, stop_tokens={stop})
     assert torch.equal(got_s.cpu(), want_s) and got_s.shape[1] < 17
+
+
+def test_repetition_penalty_follows_the_growing_sequence(pkg, tiny32):
+    """generate_minimal penalises the tokens of the prompt AND of everything generated so far, on every step
+    (RMM:1198-1201, 1946-1947, 2047-2061), also when it picks greedily.  A prompt whose plain greedy stream repeats one of
+    its own generated tokens is searched for with the oracle; the penalised stream must then equal the oracle's penalised
+    stream (which differs from the plain one exactly because generated tokens are penalised too)."""
+    s, w, model = tiny32
+    found = None
+    for seed in range(40):
+        prompt = torch.randint(0, s.vocab_size, (1, 6), generator=torch.Generator().manual_seed(1000 + seed))
+        plain = O.greedy_generate(w, s, prompt, 14)[0, 6:].tolist()
+        if len(set(plain)) == len(plain):
+            continue  # no generated token repeats: the penalty on generated tokens would not show
+        pen = O.greedy_generate(w, s, prompt, 14, penalty=1.6)
+        prompt_only = prompt.clone()
+        # what a loop that forgets to extend the sequence would produce: the prompt's tokens penalised, nothing else
+        ids, cache = prompt.clone(), O.DictCache()
+        for call in range(14):
+            pos = torch.arange(cache.get_seq_length(), ids.shape[1])
+            out = O.forward(w, s, input_ids=ids[:, pos], past_key_values=cache, use_cache=True, cache_position=pos, init_scale=0.0)
+            nxt = O.repetition_penalty(out.logits[:, -1].float(), prompt_only, 1.6).argmax(-1, keepdim=True)
+            ids = torch.cat([ids, nxt], dim=-1)
+        if not torch.equal(ids, pen):
+            found = (prompt, pen, ids)
+            break
+    assert found is not None, "no prompt with a repeating greedy stream among the seeds"
+    prompt, want, stale = found
+    gc = pkg.GenerationSettings(repetition_penalty=1.6)
+    for use_graph in (True, False):
+        got = model.generate(prompt.cuda(), gc, max_new_tokens=14, init_scale=0.0, stop_tokens=set(), use_graph=use_graph)
+        assert torch.equal(got.cpu(), want), "the penalty must see the generated tokens"
+        assert not torch.equal(got.cpu(), stale)
 
 
 def test_generate_options(pkg, tiny32):
@@ -1023,3 +1076,34 @@ def test_core_iteration_nebel_fp32_against_fp32_oracle(pkg):
         check(kd[j, :, :, T], ref_cache.key_cache[2 + j][T], dt, f"appended K, block {j}")
         check(vd[j, :, :, T], ref_cache.value_cache[2 + j][T], dt, f"appended V, block {j}")
     assert torch.equal(kd[:, :, :, :T].cpu(), kc[:, :, :, :T])
+
+
+def test_positions_and_pages_are_bounded_on_the_host(pkg, small242):
+    """The kernels index the RoPE table by position and the pages through the block table without looking, so the host
+    refuses what would run past them: a decode step beyond block_size positions, sequence lengths beyond the table or the
+    RoPE table, block ids and slots outside the caches, positions outside the RoPE table."""
+    s, w, model = small242
+    dec = pkg.PagedDecoder(model, num_blocks=8, block_size=16, num_steps=2)
+    table = torch.arange(8, dtype=torch.int32).view(2, 4)
+    ids = torch.zeros(2, dtype=torch.int64, device="cuda")
+    with pytest.raises(ValueError, match="does not fit"):
+        dec.step(ids, table.cuda(), torch.tensor([65, 3], dtype=torch.int32).cuda())
+    with pytest.raises(ValueError, match="block_table names block"):
+        dec.step(ids, (table + 5).cuda(), torch.tensor([40, 3], dtype=torch.int32).cuda())
+    with pytest.raises(ValueError, match="RoPE table"):
+        big = pkg.PagedDecoder(model, num_blocks=2, block_size=model.config.block_size + 16, num_steps=2)
+        big.step(ids[:1], torch.zeros(1, 1, dtype=torch.int32).cuda(), torch.tensor([model.config.block_size + 1], dtype=torch.int32).cuda())
+    T = 3
+    args = (torch.zeros(T, dtype=torch.int64), torch.tensor([0, 1, model.config.block_size]), torch.tensor([0, 1, 2]), table[:1],
+            torch.tensor([3], dtype=torch.int32), torch.tensor([0, 3], dtype=torch.int32), 3)
+    if model.dtype == torch.bfloat16:
+        with pytest.raises(ValueError, match="positions must lie"):
+            dec.forward_tokens(*args)
+    # the padding entries of a table (beyond a sequence's blocks) may hold anything
+    dec.step(ids, torch.tensor([[0, 1, -1, -1], [2, -1, -1, -1]], dtype=torch.int32).cuda(), torch.tensor([20, 3], dtype=torch.int32).cuda())
+    # the decode runner refuses a position past the RoPE table
+    cache = pkg.HuginnDynamicCache()
+    runner = pkg.DecodeRunner(model, cache, 1, 2)
+    cache._seen_tokens = model.config.block_size
+    with pytest.raises(ValueError, match="RoPE table"):
+        runner.step(torch.zeros(1, dtype=torch.int64, device="cuda"), None, 0.0)
