@@ -10,6 +10,9 @@ token ids).  Prints ONE JSON line:
                    token's bytes): algorithmic bytes per launch / its mean duration (HIP events on the
                    launch stream)
   core_iteration   one recurrence iteration (the unit the 70 %-of-HBM target is stated on)
+  bs8, bs32        the same decode at 8 and 32 sequences, each with the roofline of its own mlp.fc kernel
+  prefill          the recurrent core over 4 x 4096 prompt rows (the MFMA-bound regime): a few iterations, with the
+                   roofline of its dominant kernel, the tiled mlp.fc GEMM, and of the whole iteration
   cpu_baseline     the CPU oracle on this box's host cores, on a bounded sample, scaled to tokens/s
 """
 
@@ -36,7 +39,10 @@ def parse():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-iters", type=int, default=3)
-    ap.add_argument("--also-batch", type=int, default=32, help="second batch size reported under 'also' (0 = skip)")
+    ap.add_argument("--also-batch", type=int, action="append", default=None, metavar="B",
+                    help="further batch sizes reported as sub-records bs<B> (default 8 and 32; 0 = none)")
+    ap.add_argument("--prefill-iters", type=int, default=8,
+                    help="core iterations timed for the 'prefill' sub-record of the default line (0 = skip)")
     ap.add_argument("--adaptive", action="store_true",
                     help="per-token adaptive compute at bs=1 with a fixed cycle of recurrences per token (a next-row measurement)")
     ap.add_argument("--paged", action="store_true",
@@ -58,19 +64,28 @@ def parse():
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
-def prefill(args):
+def core_iteration_bytes(cfg, batch, t_cached, elt=2):
+    """Algorithmic HBM bytes of one recurrence iteration of a decode step: every weight of the adapter and the core blocks
+    once (Wqkv 3h*h, attn.proj h*h, mlp.fc 2*inter*h, mlp.proj h*inter, four norm weights, the q/k bias; adapter 2h*h),
+    the cached keys and values of `t_cached` positions read once per block, and the new position's K and V written."""
+    h, inter, nb = cfg.n_embd, cfg.intermediate_size, cfg.n_layers_in_recurrent_block
+    per_block = (3 * h * h + h * h + 2 * inter * h + h * inter + 4 * h + (2 * h if cfg.qk_bias else 0)) * elt
+    weights = nb * per_block + 2 * h * h * elt
+    kv_read = batch * nb * 2 * h * t_cached * elt
+    kv_write = batch * nb * 2 * h * elt
+    return {"weights": weights, "kv_read": kv_read, "kv_write": kv_write, "total": weights + kv_read + kv_write}
+
+
+def prefill_record(pkg, model, B, S, r):
     """BASELINE.json configs[4]: the recurrent core over a full prompt.  Token ids uniform over the vocabulary from seed 1,
-    random-init weights; the prelude runs once (untimed), then r core iterations over all B x S rows are timed.
-    FLOPs per iteration: GEMMs 2*M*(params of adapter + 4 blocks) + causal attention 4 * 2*B*nh*hd*S*(S+1)/2 * 2."""
+    random-init weights; the prelude runs once (untimed), then r core iterations over all B x S rows are timed (an
+    iteration costs the same whatever r is: every iteration attends over its own S keys).
+    FLOPs per iteration: GEMMs 2*M*(params of adapter + 4 blocks) + causal attention 4 * 2*B*nh*hd*S*(S+1)/2 * 2.
+    The dominant kernel, the tiled GEMM of mlp.fc with its SwiGLU epilogue (41 % of an iteration's FLOPs), is then
+    timed alone with HIP events on the launch stream, rotating over the four core blocks' matrices."""
     import torch
-    import __graft_entry__ as entry
-    pkg = entry.import_package()
-    pkg.hip.load()
     dev = torch.device("cuda:0")
-    cfg = pkg.RavenConfig()
-    r, B, S = args.recurrence, args.prefill_batch, args.prefill_len
-    model = pkg.RavenForCausalLM(cfg, device=dev, dtype=torch.bfloat16)
-    fill_synthetic(model, 0)
+    cfg = model.config
     ids = torch.randint(0, cfg.vocab_size, (B, S), generator=torch.Generator().manual_seed(1)).cuda()
     cache = pkg.HuginnDynamicCache(max_length=S)
     cache.ensure(cfg.n_layers_in_prelude + cfg.n_layers_in_recurrent_block * r, cfg.n_layers_in_coda, B, cfg.n_heads, cfg.head_dim, S,
@@ -95,17 +110,52 @@ def prefill(args):
     b.record()
     torch.cuda.synchronize()
     ms = a.elapsed_time(b)
+    del cache, embeds, state
+    torch.cuda.empty_cache()
     tflops = (gemm_flops + attn_flops) * r / (ms * 1e-3) / 1e12
-    line = {
-        "metric": "core prefill tokens*iterations/s, raven-3.5b shape bf16; MFMA utilisation",
-        "value": round(M * r / (ms * 1e-3), 1), "unit": "tokens*iterations/s", "n_gpus": 1, "steps": r, "warmup": 1,
-        "ms_per_step": round(ms / r, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic",
-        "config": {"workload": f"recurrent-core prefill, nebel-raven-3.5b shape, bs={B} x {S} tokens, r={r} (BASELINE.json configs[4])",
-                   "batch": B, "seq_len": S, "recurrence": r, "gemm": "hipBLASLt via torch.matmul", "attention": "attention_prefill_kernel"},
-        "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tflops / MFMA_PEAK_TFLOPS, 4), "flops_per_iteration": gemm_flops + attn_flops, "traffic": None},
+    # the dominant kernel alone
+    lib = pkg.hip.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    blocks = model.transformer.core_block
+    x = torch.randn(M, h, device=dev, dtype=torch.bfloat16)
+    gate = torch.empty(M, inter, device=dev, dtype=torch.bfloat16)
+
+    def fc_launch(i=[0]):
+        blk = blocks[i[0] % len(blocks)]
+        i[0] += 1
+        lib.raven_gemm_swiglu(x.data_ptr(), blk.mlp.fc.weight.data_ptr(), gate.data_ptr(), M, inter, h, pkg.hip.BF16, stream)
+
+    fc_ms = event_time_ms(fc_launch, 8, warm=2)
+    fc_flops = 2.0 * M * 2 * inter * h
+    fc_tflops = fc_flops / (fc_ms * 1e-3) / 1e12
+    return {
+        "value": round(M * r / (ms * 1e-3), 1), "unit": "tokens*iterations/s", "steps": r, "warmup": 1, "ms_per_step": round(ms / r, 3),
+        "config": {"workload": f"recurrent-core prefill, nebel-raven-3.5b shape, bs={B} x {S} tokens, {r} timed iterations "
+                               f"(BASELINE.json configs[4])",
+                   "batch": B, "seq_len": S, "iterations": r, "gemm": "gemm_tiled_kernel (hand-written MFMA, 256 x 256 tiles)",
+                   "attention": "attention_prefill_kernel"},
+        "roofline": {"bound": "mfma", "kernel": f"gemm_tiled_kernel<SwiGLU, 256x256> (mlp.fc {2 * inter}x{h}, M={M})",
+                     "achieved": round(fc_tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(fc_tflops / MFMA_PEAK_TFLOPS, 4), "flops_per_launch": fc_flops, "avg_us": round(fc_ms * 1e3, 1),
+                     "traffic": None},
+        "iteration_roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                               "frac": round(tflops / MFMA_PEAK_TFLOPS, 4), "flops_per_iteration": gemm_flops + attn_flops},
     }
+
+
+def prefill(args):
+    """The configs[4] measurement as a line of its own: --recurrence iterations (32) instead of the default line's few."""
+    import torch
+    import __graft_entry__ as entry
+    pkg = entry.import_package()
+    pkg.hip.load()
+    model = pkg.RavenForCausalLM(pkg.RavenConfig(), device=torch.device("cuda:0"), dtype=torch.bfloat16)
+    fill_synthetic(model, 0)
+    rec = prefill_record(pkg, model, args.prefill_batch, args.prefill_len, args.recurrence)
+    line = {"metric": "core prefill tokens*iterations/s, raven-3.5b shape bf16; MFMA utilisation", "value": rec["value"],
+            "unit": rec["unit"], "n_gpus": 1, "steps": rec["steps"], "warmup": rec["warmup"], "ms_per_step": rec["ms_per_step"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": rec["config"], "roofline": rec["roofline"], "iteration_roofline": rec["iteration_roofline"]}
     print(json.dumps(line))
 
 
@@ -364,31 +414,116 @@ def main():
         sys.exit(2)
     import torch
     import __graft_entry__ as entry
-    from oracle import raven_oracle as O
 
     pkg = entry.import_package()
     pkg.hip.load()
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    shape = O.RavenShape.nebel()
     cfg = pkg.RavenConfig()
     r = args.recurrence
     model = pkg.RavenForCausalLM(cfg, device=dev, dtype=torch.bfloat16)
     fill_synthetic(model, 0)
     use_graph = not args.no_graph
+    h = cfg.n_embd
+    lib = pkg.hip.load()
+    stream = torch.cuda.current_stream().cuda_stream
 
-    tok_s, ms_step, prefill_s, cache = decode_tokens_per_s(pkg, model, args.batch, args.prompt, args.steps, args.warmup, r, use_graph)
-    mean_t = args.prompt + args.warmup + args.steps / 2.0
-    blocks_bytes = O.core_iteration_bytes(shape, args.batch, int(mean_t))
-    per_block_w = (blocks_bytes["weights"] - 2 * shape.n_embd * shape.n_embd * 2) // 4
-    token_bytes = (r * blocks_bytes["total"] + 4 * (per_block_w + (blocks_bytes["kv_read"] + blocks_bytes["kv_write"]) // 4)
-                   + shape.vocab_size * shape.n_embd * 2)
+    head = decode_record(pkg, model, args.batch, args.prompt, args.steps, args.warmup, r, use_graph)
+    tok_s, ms_step = head["tokens_per_s"], head["ms_per_step"]
+
+    # ---- device copy bandwidth, for context next to the published peak ----
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    copy_ms = event_time_ms(lambda: dst.copy_(src), 10)
+    copy_gbs = 2 * src.numel() / (copy_ms * 1e-3) / 1e9
+    del src, dst
+
+    # ---- the isolated norm kernel (BASELINE.json configs[1]): x + residual -> RMSNorm, [T, 5280] bf16, 31,680 B per row ----
+    norm_w = model.transformer.core_block[0].norm_1.weight
+    norm_cfg2 = {}
+    for T_rows in (1, 32, 4096):
+        xs = [torch.randn(T_rows, h, device=dev, dtype=torch.bfloat16) for _ in range(8)]  # rotate: 8 x 43 MB at T = 4096
+        rs = torch.randn(T_rows, h, device=dev, dtype=torch.bfloat16)
+        yo = torch.empty_like(rs)
+
+        def norm_launch(i=[0]):
+            i[0] += 1
+            lib.raven_rmsnorm_residual(xs[i[0] % 8].data_ptr(), rs.data_ptr(), norm_w.data_ptr(), yo.data_ptr(), None, None, None, T_rows, h,
+                                       cfg.norm_eps, pkg.hip.BF16, stream)
+
+        t_ms = event_time_ms(norm_launch, 100, warm=10)
+        norm_cfg2[f"T={T_rows}"] = {"us": round(t_ms * 1e3, 2), "GBs": round(T_rows * 3 * h * 2 / (t_ms * 1e-3) / 1e9, 1)}
+        del xs, rs, yo
+
+    subs = {}
+    for b2 in ([8, 32] if args.also_batch is None else args.also_batch):
+        if b2 and b2 != args.batch:
+            torch.cuda.empty_cache()
+            subs[f"bs{b2}"] = decode_record(pkg, model, b2, args.prompt, max(8, args.steps // 4), 2, r, use_graph)
+
+    pre = None
+    if args.prefill_iters:
+        torch.cuda.empty_cache()
+        pre = prefill_record(pkg, model, args.prefill_batch, args.prefill_len, args.prefill_iters)
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(model, args.cpu_iters, r)
+
+    line = {
+        "metric": "decode tokens/s at r=32, raven-3.5b shape bf16 bs=1/32; % HBM roofline",
+        "value": round(tok_s, 3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"full-token greedy decode, nebel-raven-3.5b shape, r={r}, bs={args.batch}, "
+                               f"{args.prompt}-token random prompt, {args.steps} timed tokens (BASELINE.json configs[3])",
+                   "batch": args.batch, "recurrence": r, "prompt": args.prompt, "hip_graph": use_graph},
+        "recurrence_steps_per_s": head["recurrence_steps_per_s"],
+        "token_roofline": head["token_roofline"],
+        "roofline": head["roofline"],
+        "core_iteration": head["core_iteration"],
+        "rmsnorm_residual_5280": norm_cfg2,
+        "device_copy_GBs": round(copy_gbs, 1),
+        "prefill_s": head["prefill_s"],
+        **subs,
+        "prefill": pre,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+# HBM bytes per launch of the bs=1 mlp.fc kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy: a
+# profiler figure, so a constant here, with the file that holds the readings
+FC_BS1_TRAFFIC = {"bytes": 386061876, "source": "profiles/mlp_fc_gemv_bs1_hbm_traffic.txt"}
+
+
+def decode_record(pkg, model, B, prompt_len, steps, warmup, r, use_graph):
+    """Full-token decode at B sequences with what bounds it: tokens/s over `steps` greedy tokens, one recurrence
+    iteration at 1024 cached positions (eager launches and a replayed graph of eight), and the dominant kernel -- the
+    mlp.fc product with its norm prologue and SwiGLU epilogue, 47 % of a token's bytes -- alone, timed with HIP events on
+    the launch stream exactly as the decode loop launches it, rotating over the four core blocks' fc matrices (1.5 GB)
+    so that no cache level can keep a matrix between launches."""
+    import torch
+    cfg = model.config
+    dev = model.device
+    tok_s, ms_step, prefill_s, cache = decode_tokens_per_s(pkg, model, B, prompt_len, steps, warmup, r, use_graph)
     del cache
     torch.cuda.empty_cache()
+    mean_t = prompt_len + warmup + steps / 2.0
+    bb = core_iteration_bytes(cfg, B, int(mean_t))
+    per_block_w = (bb["weights"] - 2 * cfg.n_embd * cfg.n_embd * 2) // 4
+    token_bytes = (r * bb["total"] + 4 * (per_block_w + (bb["kv_read"] + bb["kv_write"]) // 4) + cfg.vocab_size * cfg.n_embd * 2)
 
     # ---- one recurrence iteration at T = 1024 (the unit of the roofline target) ----
-    B = args.batch
     h, nh, hd, T = cfg.n_embd, cfg.n_heads, cfg.head_dim, 1024
     nat = model._natives()
     kc = torch.randn(4, B, nh, T + 1, hd, device=dev, dtype=torch.bfloat16)
@@ -413,12 +548,11 @@ def main():
     with torch.cuda.graph(graph):
         eight_iters()
     iter_graph_ms = event_time_ms(graph.replay, 10) / 8
-    it_bytes = O.core_iteration_bytes(shape, B, T)["total"]
+    it_bytes = core_iteration_bytes(cfg, B, T)["total"]
     iter_ms = min(iter_eager_ms, iter_graph_ms)
+    del graph, kc, vc, kv
 
-    # ---- dominant kernel: mlp.fc GEMV with its norm_2/norm_3 prologue and SwiGLU epilogue ----
-    # (47 % of a token's bytes).  Timed exactly as the decode loop launches it, rotating over the four
-    # core blocks' fc matrices (1.5 GB) so that no cache level can keep a matrix between launches.
+    # ---- dominant kernel ----
     blocks = model.transformer.core_block
     xin = torch.randn(B, h, device=dev, dtype=torch.bfloat16)
     x2 = torch.empty_like(xin)
@@ -444,88 +578,32 @@ def main():
                                   pkg.hip.BF16, stream)
 
     fc_ms = event_time_ms(fc_launch, 200, warm=10)
-    fc_w = blocks[0].mlp.fc.weight
-    fc_bytes = fc_w.numel() * 2 + B * h * 2 + B * cfg.intermediate_size * 2
+    fc_bytes = blocks[0].mlp.fc.weight.numel() * 2 + B * h * 2 + B * cfg.intermediate_size * 2
     fc_gbs = fc_bytes / (fc_ms * 1e-3) / 1e9
-
-    # ---- device copy bandwidth, for context next to the published peak ----
-    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-    dst = torch.empty_like(src)
-    copy_ms = event_time_ms(lambda: dst.copy_(src), 10)
-    copy_gbs = 2 * src.numel() / (copy_ms * 1e-3) / 1e9
-    del src, dst, kc, vc
-
-    # ---- the isolated norm kernel (BASELINE.json configs[1]): x + residual -> RMSNorm, [T, 5280] bf16, 31,680 B per row ----
-    norm_w = model.transformer.core_block[0].norm_1.weight
-    norm_cfg2 = {}
-    for T_rows in (1, 32, 4096):
-        xs = [torch.randn(T_rows, h, device=dev, dtype=torch.bfloat16) for _ in range(8)]  # rotate: 8 x 43 MB at T = 4096
-        rs = torch.randn(T_rows, h, device=dev, dtype=torch.bfloat16)
-        yo = torch.empty_like(rs)
-
-        def norm_launch(i=[0]):
-            i[0] += 1
-            lib.raven_rmsnorm_residual(xs[i[0] % 8].data_ptr(), rs.data_ptr(), norm_w.data_ptr(), yo.data_ptr(), None, None, None, T_rows, h,
-                                       cfg.norm_eps, pkg.hip.BF16, stream)
-
-        t_ms = event_time_ms(norm_launch, 100, warm=10)
-        norm_cfg2[f"T={T_rows}"] = {"us": round(t_ms * 1e3, 2), "GBs": round(T_rows * 3 * h * 2 / (t_ms * 1e-3) / 1e9, 1)}
-        del xs, rs, yo
-
-    also = None
-    if args.also_batch and args.also_batch != args.batch:
-        torch.cuda.empty_cache()
-        steps2 = max(8, args.steps // 4)
-        t2, ms2, _, c2 = decode_tokens_per_s(pkg, model, args.also_batch, args.prompt, steps2, 2, r, use_graph)
-        also = {"batch": args.also_batch, "tokens_per_s": round(t2, 2), "ms_per_step": round(ms2, 3), "steps": steps2}
-        del c2
-
-    cpu = None
-    if not args.no_cpu_baseline:
-        cpu = cpu_baseline(O, shape, model, args.cpu_iters, r)
-
-    line = {
-        "metric": "decode tokens/s at r=32, raven-3.5b shape bf16 bs=1/32; % HBM roofline",
-        "value": round(tok_s, 3),
-        "unit": "tokens/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms_step, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
-        "config": {"workload": f"full-token greedy decode, nebel-raven-3.5b shape, r={r}, bs={args.batch}, "
-                               f"{args.prompt}-token random prompt, {args.steps} timed tokens (BASELINE.json configs[3])",
-                   "batch": args.batch, "recurrence": r, "prompt": args.prompt, "hip_graph": use_graph},
-        "recurrence_steps_per_s": round(tok_s * r / args.batch, 2),
-        "token_roofline": {"bytes_per_token": int(token_bytes), "achieved_GBs": round(token_bytes * (tok_s / args.batch) / 1e9, 1),
-                           "frac": round(token_bytes * (tok_s / args.batch) / 1e9 / HBM_PEAK_GBS, 4)},
+    return {
+        "batch": B, "tokens_per_s": round(tok_s, 3), "ms_per_step": round(ms_step, 4), "steps": steps, "prefill_s": round(prefill_s, 3),
+        "recurrence_steps_per_s": round(tok_s * r / B, 2),
+        "token_roofline": {"bytes_per_token": int(token_bytes), "achieved_GBs": round(token_bytes * (tok_s / B) / 1e9, 1),
+                           "frac": round(token_bytes * (tok_s / B) / 1e9 / HBM_PEAK_GBS, 4)},
         "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": round(fc_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(fc_gbs / HBM_PEAK_GBS, 4),
                      "bytes_per_launch": int(fc_bytes), "avg_us": round(fc_ms * 1e3, 2),
-                     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy
-                     # (profiles/mlp_fc_gemv_bs1_hbm_traffic.txt); a profiler figure, so a constant here
-                     "traffic": 386061876 if B == 1 else None},
+                     "traffic": FC_BS1_TRAFFIC["bytes"] if B == 1 else None,
+                     "traffic_source": FC_BS1_TRAFFIC["source"] if B == 1 else None},
         "core_iteration": {"T": T, "batch": B, "bytes": int(it_bytes), "ms_eager": round(iter_eager_ms, 4),
                            "ms_graph": round(iter_graph_ms, 4), "achieved_GBs": round(it_bytes / (iter_ms * 1e-3) / 1e9, 1),
                            "frac": round(it_bytes / (iter_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
-        "rmsnorm_residual_5280": norm_cfg2,
-        "device_copy_GBs": round(copy_gbs, 1),
-        "prefill_s": round(prefill_s, 3),
-        "also": also,
-        "cpu_baseline": cpu,
     }
-    print(json.dumps(line))
 
 
-def cpu_baseline(O, shape, model, n_iters, r):
+def cpu_baseline(model, n_iters, r):
     """The CPU oracle (a port of the reference's CPU path) on the host cores: a few recurrence
     iterations plus one LM-head product at the nebel shape, bs=1, 512 cached positions, scaled to
-    tokens/s as 1 / ((r + 1) * t_iteration + t_head) -- the 4 prelude/coda blocks cost one iteration."""
+    tokens/s as 1 / ((r + 1) * t_iteration + t_head) -- the 4 prelude/coda blocks cost one iteration.
+    The only part of this file that touches the oracle."""
     import torch
+    from oracle import raven_oracle as O
+    shape = O.RavenShape.nebel()
     T = 512
     w = {}
     for name, p in model.state_dict().items():

@@ -220,7 +220,7 @@ def generate_with_adaptive_compute(model, input_ids: torch.Tensor, generation_co
     elif getattr(gc, "max_new_tokens", None):
         max_new = gc.max_new_tokens
     else:
-        max_new = model_kwargs.get("max_length", gc.max_length) - prompt_len
+        max_new = model_kwargs.get("max_length", model._default_max_length(gc)) - prompt_len
     max_steps = model_kwargs.get("num_steps", model.config.mean_recurrence)
     stops = model._get_stops(gc) if stop_tokens is None else set(stop_tokens)
     dev = model.device

@@ -188,6 +188,8 @@ class HuginnDynamicCache:
     graph needs); without it the storage grows geometrically as tokens arrive.
     """
 
+    is_compileable = False  # what transformers' generation loop asks a cache before it considers compiling the forward
+
     def __init__(self, lookup_strategy: str = "full", max_length: Optional[int] = None):
         self._seen_tokens = 0
         self.lookup_strategy = lookup_strategy

@@ -54,7 +54,7 @@ def generate_diffusion_style(model, input_ids: torch.Tensor, generation_config=N
     elif getattr(gc, "max_new_tokens", None):
         max_new = gc.max_new_tokens
     else:
-        max_new = model_kwargs.get("max_length", gc.max_length) - n_prompt
+        max_new = model_kwargs.get("max_length", model._default_max_length(gc)) - n_prompt
     stops = model._get_stops(gc) if stop_tokens is None else set(stop_tokens)
     cache = model._generation_cache(model_kwargs, cache_lookup_strategy, 1)
     draws = [0]

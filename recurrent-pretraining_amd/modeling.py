@@ -3,7 +3,10 @@ reference's RavenForCausalLM (recpre/raven_modeling_minimal.py, "RMM": forward 6
 iterate_forward 726-762, core_block_forward 764-781, iterate_one_step 841-868, predict_from_latents
 870-900, embed_inputs 902-934, generate_minimal 1165-1232) whose arithmetic runs in the HIP kernels
 of libraven_hip.so.  torch.nn modules are used only as named parameter containers, so a reference
-state dict loads with `load_state_dict` unchanged.
+state dict loads with `load_state_dict` unchanged.  The class is a transformers `PreTrainedModel` with
+`GenerationMixin` (RMM:36-112, 326), registered for `AutoConfig` / `AutoModel` / `AutoModelForCausalLM` under
+the model type `huginn_raven` (RMM:2312-2323): a generate() call with none of the reference's own loop
+keywords runs transformers' generation loop over this forward, as in the reference (RMM:1112-1127).
 
 What differs from the reference on purpose:
   * token rows are processed as [B*S, h]; K/V live in one contiguous step-indexed buffer;
@@ -20,6 +23,8 @@ from dataclasses import dataclass
 from typing import Any, Callable, Optional, Union
 
 import torch
+from transformers import AutoConfig, AutoModel, AutoModelForCausalLM, GenerationMixin, PreTrainedModel
+from transformers.utils import ModelOutput
 
 from . import hip
 from .cache import HuginnDynamicCache, HuginnStaticCache, remap_step
@@ -27,7 +32,7 @@ from .config import RavenConfig
 
 
 @dataclass
-class CausalLMOutputRecurrentLatents:  # RMM:113-123
+class CausalLMOutputRecurrentLatents(ModelOutput):  # RMM:113-123
     loss: Optional[torch.Tensor] = None
     log_ppl: Optional[torch.Tensor] = None
     logits: Optional[torch.Tensor] = None
@@ -36,9 +41,6 @@ class CausalLMOutputRecurrentLatents:  # RMM:113-123
     hidden_states: Optional[torch.Tensor] = None
     attention_maps: Optional[dict] = None
     stats: Optional[dict] = None
-
-    def __getitem__(self, k):
-        return getattr(self, k)
 
 
 @dataclass
@@ -128,13 +130,65 @@ def _as_int(v) -> int:
     return int(v.item()) if isinstance(v, torch.Tensor) else int(v)
 
 
-class RavenForCausalLM(torch.nn.Module):
+class RavenPreTrainedModel(PreTrainedModel):
+    """What transformers needs to know about the model family (RMM:36-112): the configuration class, the tied head, and
+    the reference's weight initialisation for a model built from a configuration alone."""
     config_class = RavenConfig
+    base_model_prefix = "model"
+    supports_gradient_checkpointing = False  # inference only
+    _no_split_modules = ["SandwichBlock"]
+    _skip_keys_device_placement = ["past_key_values"]
+    _tied_weights_keys = {"lm_head.weight": "transformer.wte.weight"}
+    _supports_flash_attn = True
+    _supports_sdpa = True
+    _supports_attention_backend = True
+    _tp_plan = {}
 
-    def __init__(self, config: RavenConfig, device: Union[str, torch.device] = "cuda", dtype: Optional[torch.dtype] = None):
-        super().__init__()
-        self.config = config
-        dtype = dtype if dtype is not None else getattr(torch, config.torch_dtype)
+    @property
+    def emb_scale(self) -> float:  # RMM:50-52
+        return self.config.init_values["embed_scale"]
+
+    @torch.no_grad()
+    def _init_weights(self, module) -> None:
+        """RMM:57-110 ("takase" scheme): truncated normals at +-3 std; Q, K, V and the two halves of fc drawn apart;
+        output projections scaled down by the expected depth; norm weights one."""
+        iv = self.config.init_values
+
+        def normal(t, std):
+            return torch.nn.init.trunc_normal_(t, mean=0.0, std=std, a=-3 * std, b=3 * std)
+
+        names = getattr(self, "_module_names", None)
+        if names is None:
+            names = self._module_names = {id(m): n for n, m in self.named_modules()}
+        name = names.get(id(module), "")
+        if isinstance(module, RMSNorm):
+            torch.nn.init.ones_(module.weight)
+        elif isinstance(module, torch.nn.Embedding):
+            normal(module.weight, iv["embedding"])
+        elif isinstance(module, torch.nn.Linear):  # transformers visits the modules that own parameters
+            if name.endswith("Wqkv"):
+                for part in module.weight.split(self.config.n_embd, dim=0):  # n_kv_heads == n_heads: three h x h pieces
+                    normal(part, iv["std"])
+            elif name.endswith("mlp.fc"):
+                gate, up = module.weight.chunk(2, dim=0)
+                normal(gate, iv["std"])
+                normal(up, iv["out_proj"])
+            elif name.endswith("mlp.proj") or name.endswith("attn.proj"):
+                normal(module.weight, iv["out_proj"])
+            elif name.endswith("adapter") or (name == "lm_head" and not self.config.tie_embeddings):
+                normal(module.weight, iv["std"])
+
+
+class RavenForCausalLM(RavenPreTrainedModel, GenerationMixin):
+    def __init__(self, config: RavenConfig, device: Union[str, torch.device, None] = None, dtype: Optional[torch.dtype] = None):
+        """`device` None: wherever torch currently creates tensors (a `with torch.device(...)` block, transformers'
+        loaders), else the GPU when there is one.  The parameters may live on the CPU; the forward needs them on the GPU."""
+        super().__init__(config)
+        if device is None:
+            device = torch.get_default_device()
+            if device.type == "cpu" and torch.cuda.is_available():
+                device = torch.device("cuda")
+        dtype = dtype if dtype is not None else (config.dtype if isinstance(config.dtype, torch.dtype) else torch.bfloat16)
         with torch.device(device):
             prelude = torch.nn.ModuleList(SandwichBlock(config, i) for i in range(config.n_layers_in_prelude))
             adapter = _linear(2 * config.n_embd, config.n_embd)
@@ -152,7 +206,7 @@ class RavenForCausalLM(torch.nn.Module):
             table = precompute_freqs_cis(config.head_dim, config.block_size, config.rope_base)
             self.register_buffer("freqs_cis", table.to(device), persistent=True)
         self.to(dtype)  # casts the RoPE table too, as nn.Module.to does for the reference (RMM:577)
-        self.generation_config = GenerationSettings()
+        self.post_init()
         self.noise_source = None  # test-time noise draws: an object with normal(x) and uniform(x); None = torch's generator
         self._native_key = None
         self._native: dict = {}
@@ -161,10 +215,6 @@ class RavenForCausalLM(torch.nn.Module):
         self.eval()
 
     # ---- small helpers -------------------------------------------------------------------------
-    @property
-    def emb_scale(self) -> float:  # RMM:50-52
-        return self.config.init_values["embed_scale"]
-
     @property
     def dtype(self) -> torch.dtype:
         return self.transformer.wte.weight.dtype
@@ -198,9 +248,12 @@ class RavenForCausalLM(torch.nn.Module):
         return names
 
     @torch.no_grad()
-    def init_weights(self, seed: int = 0, std: float = 0.02) -> None:
-        """Synthetic weights: every tensor ~ N(0, std) (norm weights ~ N(1, std)), drawn on the CPU in
-        synthetic_weight_order() from one seeded generator and cast, so that any host reproduces them."""
+    def init_weights(self, seed: Optional[int] = None, std: float = 0.02) -> None:
+        """With a seed, synthetic weights: every tensor ~ N(0, std) (norm weights ~ N(1, std)), drawn on the CPU in
+        synthetic_weight_order() from one seeded generator and cast, so that any host reproduces them.  Without one,
+        what transformers calls at the end of construction: the reference's initialisation (_init_weights) and the tie."""
+        if seed is None:
+            return super().init_weights()
         g = torch.Generator(device="cpu").manual_seed(seed)
         sd = self.state_dict()
         for name in self.synthetic_weight_order():
@@ -209,19 +262,48 @@ class RavenForCausalLM(torch.nn.Module):
             p.copy_(torch.empty(p.shape, dtype=torch.float32).normal_(mean, std, generator=g).to(p.dtype))
 
     # ---- checkpoints -----------------------------------------------------------------------------
+    _LOADER_KWARGS = ("trust_remote_code", "revision", "cache_dir", "token", "local_files_only", "force_download", "proxies",
+                      "subfolder", "use_safetensors", "low_cpu_mem_usage", "attn_implementation", "code_revision", "adapter_kwargs",
+                      "weights_only", "_from_auto", "_commit_hash", "use_auth_token", "resume_download", "state_dict", "variant")
+
     @classmethod
-    def from_pretrained(cls, path: str, device: Union[str, torch.device] = "cuda", dtype: Optional[torch.dtype] = None,
-                        **config_overrides) -> "RavenForCausalLM":
+    def from_pretrained(cls, path: str, *model_args, device: Union[str, torch.device, None] = None,
+                        dtype: Optional[torch.dtype] = None, config: Optional[RavenConfig] = None,
+                        **kwargs) -> "RavenForCausalLM":
         """Builds the model from a LOCAL directory laid out like the reference's published checkpoints (what
         `AutoModelForCausalLM.from_pretrained(..., trust_remote_code=True)` reads for raven_modeling_minimal.py:2312-2323):
         `config.json` plus `model.safetensors`, or sharded `model-XXXXX-of-YYYYY.safetensors` with
         `model.safetensors.index.json`, or `pytorch_model.bin` (read with weights_only=True).  Nothing is downloaded.
-        The parameter names are the reference's, so the tensors load unchanged; a tied head may be absent from the file."""
+        The parameter names are the reference's, so the tensors load unchanged; a tied head may be absent from the file.
+        Replaces transformers' loader (one shard in host memory at a time, straight into the parameters) and takes its
+        call shape: `config=` from an Auto class, `torch_dtype` / `dtype`, `device_map` as one device; the other loader
+        keywords are accepted and have nothing to act on; any remaining keyword overrides a configuration field."""
         import json
         import os
+        if dtype is None:
+            dtype = kwargs.pop("torch_dtype", None)
+        else:
+            kwargs.pop("torch_dtype", None)
+        if isinstance(dtype, str):
+            dtype = None if dtype == "auto" else getattr(torch, dtype)
+        device_map = kwargs.pop("device_map", None)
+        if device is None and device_map is not None:
+            if isinstance(device_map, dict):
+                places = set(device_map.values())
+                if len(places) != 1:
+                    raise ValueError("the model lives on one device: device_map must name exactly one")
+                device_map = places.pop()
+            device = "cuda" if device_map == "auto" else device_map
+        for k in cls._LOADER_KWARGS:
+            kwargs.pop(k, None)
+        path = str(path)
+        if not os.path.isdir(path):
+            raise FileNotFoundError(f"{path} is not a local directory (nothing is downloaded)")
         with open(os.path.join(path, "config.json")) as f:
             cfg_dict = json.load(f)
-        cfg_dict.update(config_overrides)
+        if config is not None:
+            cfg_dict = config.to_dict()
+        cfg_dict.update(kwargs)
         config = RavenConfig(**cfg_dict)
         model = cls(config, device=device, dtype=dtype)
         index = os.path.join(path, "model.safetensors.index.json")
@@ -263,15 +345,19 @@ class RavenForCausalLM(torch.nn.Module):
         model._native_key = None
         return model
 
-    def save_pretrained(self, path: str, max_shard_bytes: int = 5 * 2 ** 30) -> None:
+    def save_pretrained(self, path: str, max_shard_bytes: int = 5 * 2 ** 30, **unused) -> None:
         """Writes `config.json` and safetensors shards (with an index when there are several) that from_pretrained and
         the reference's loader read.  The tied head is stored once, under the embedding's name."""
         import json
         import os
         from safetensors.torch import save_file
+        path = str(path)
         os.makedirs(path, exist_ok=True)
+        cfg = self.config.to_dict()
+        cfg.update(architectures=["RavenForCausalLM"], torch_dtype=str(self.dtype).replace("torch.", ""))
+        cfg["dtype"] = cfg["torch_dtype"]
         with open(os.path.join(path, "config.json"), "w") as f:
-            json.dump({**self.config.to_dict(), "architectures": ["RavenForCausalLM"]}, f, indent=1)
+            json.dump(cfg, f, indent=1, sort_keys=True)
         sd = {k: v.detach().to("cpu").contiguous() for k, v in self.state_dict().items()
               if not (self.config.tie_embeddings and k == "lm_head.weight")}
         shards, cur, size = [], {}, 0
@@ -339,6 +425,11 @@ class RavenForCausalLM(torch.nn.Module):
         src = position_ids if position_ids is not None else cache_position
         if src is None:
             return list(range(n_tokens))
+        if src.dim() == 2 and src.shape[0] > 1:  # one row per sequence, as transformers' generate() builds them
+            if not bool((src == src[:1]).all()):
+                raise ValueError("positions differ between the sequences of the batch: they are one list shared by the batch "
+                                 "(a left-padded batch cannot be rotated row by row, RMM:660-665)")
+            src = src[0]
         pos = [int(v) for v in src.reshape(-1).tolist()]
         if len(pos) != n_tokens:
             raise ValueError(f"{len(pos)} positions for {n_tokens} tokens: positions are one 1-D list shared by the batch")
@@ -654,18 +745,45 @@ class RavenForCausalLM(torch.nn.Module):
         return x.view(B, S, cfg.n_embd), torch.tensor(block_idx, dtype=torch.long)
 
     # ---- generation --------------------------------------------------------------------------------
-    def prepare_inputs_for_generation(self, input_ids, past_key_values=None, attention_mask=None, inputs_embeds=None,
-                                      cache_position=None, cache_lookup_strategy: str = "full", **kwargs):
-        """RMM:1066-1110, without the HF cache swapping: feeds the tokens the cache has not seen."""
+    @classmethod
+    def _supports_default_dynamic_cache(cls) -> bool:
+        """transformers' generate() must not build its own per-layer cache: the forward makes a HuginnDynamicCache."""
+        return False
+
+    def prepare_inputs_for_generation(self, input_ids, next_sequence_length=None, past_key_values=None, attention_mask=None,
+                                      inputs_embeds=None, is_first_iteration=False, cache_position=None,
+                                      cache_lookup_strategy: str = "full", **kwargs):
+        """What transformers' generation loop calls before every forward (RMM:1066-1110).  It selects the tokens to feed:
+        `input_ids[:, cache_position]` when the loop tracks cache positions (transformers 4.x, as in the reference), else
+        the last `next_sequence_length` tokens (5.x), else all of them.  A cache of another class (the loop's own
+        default) must be empty and is replaced by this package's, as the reference does; `attention_mask` is accepted
+        and not forwarded (the forward ignores it, RMM:676)."""
         model_inputs = {}
-        seen = past_key_values.get_seq_length() if past_key_values is not None else 0
-        if cache_position is None:
-            cache_position = torch.arange(seen, input_ids.shape[1], device=input_ids.device)
-        model_inputs["cache_position"] = cache_position
-        model_inputs["past_key_values"] = past_key_values if kwargs.get("use_cache", True) else None
-        model_inputs["input_ids"] = input_ids[:, cache_position].contiguous()
+        if past_key_values is not None and not isinstance(past_key_values, HuginnDynamicCache):
+            if past_key_values.get_seq_length() != 0:
+                raise ValueError("only an empty cache of another class can be replaced by a HuginnDynamicCache")
+            if type(past_key_values).__name__ == "StaticCache":
+                cfg = self.config
+                past_key_values = HuginnStaticCache(
+                    max_length=min(getattr(self.generation_config, "max_length", None) or cfg.block_size, cfg.block_size),
+                    max_num_steps=4 + kwargs.get("num_steps", cfg.mean_recurrence) * 4, num_heads=cfg.num_key_value_heads,
+                    hidden_dim=cfg.head_dim, batch_size=input_ids.shape[0], device=self.device, dtype=self.dtype,
+                    lookup_strategy=cache_lookup_strategy)
+            else:
+                past_key_values = HuginnDynamicCache(cache_lookup_strategy)
+        use_cache = kwargs.get("use_cache", True)
+        model_inputs["past_key_values"] = past_key_values if use_cache else None
+        if cache_position is not None:
+            model_inputs["cache_position"] = cache_position
+            input_ids = input_ids[:, cache_position]
+        elif next_sequence_length is not None:
+            input_ids = input_ids[:, -next_sequence_length:]
+        model_inputs["input_ids"] = input_ids.clone(memory_format=torch.contiguous_format)
+        position_ids = kwargs.pop("position_ids", None)
+        if position_ids is not None and cache_position is None:
+            model_inputs["position_ids"] = position_ids[..., -input_ids.shape[1]:].clone(memory_format=torch.contiguous_format)
         for key, value in kwargs.items():
-            if key not in model_inputs:
+            if key not in model_inputs and key not in ("labels", "next_sequence_length"):
                 model_inputs[key] = value
         return model_inputs
 
@@ -704,6 +822,13 @@ class RavenForCausalLM(torch.nn.Module):
         probs = probs / probs.sum(dim=-1, keepdim=True).clamp(min=1e-10)
         return torch.multinomial(probs, num_samples=1)
 
+    def _default_max_length(self, gc) -> int:
+        """`max_length` of the generation settings; transformers 5 leaves it unset by default, then the RoPE table's length."""
+        for src in (gc, self.generation_config):
+            if getattr(src, "max_length", None):
+                return src.max_length
+        return self.config.block_size
+
     def _generation_cache(self, model_kwargs: dict, cache_lookup_strategy: str, batch: int, max_length: Optional[int] = None):
         """The cache a generate loop works on (RMM:1146-1160): the caller's `past_key_values`, or a new one --
         HuginnStaticCache when `cache_implementation="static"` is asked for, else HuginnDynamicCache."""
@@ -712,7 +837,7 @@ class RavenForCausalLM(torch.nn.Module):
             return given
         if model_kwargs.get("cache_implementation", "dynamic") == "static":
             cfg = self.config
-            length = max_length if max_length is not None else model_kwargs.get("max_length", self.generation_config.max_length)
+            length = max_length if max_length is not None else model_kwargs.get("max_length", self._default_max_length(None))
             steps = 4 + model_kwargs.get("num_steps", cfg.mean_recurrence) * 4
             return HuginnStaticCache(max_length=min(length, cfg.block_size), max_num_steps=steps, num_heads=cfg.num_key_value_heads,
                                      hidden_dim=cfg.head_dim, batch_size=batch, device=self.device, dtype=self.dtype,
@@ -732,19 +857,26 @@ class RavenForCausalLM(torch.nn.Module):
                 "rel_residual": residual_diff / latent_states.norm(dim=-1), "num_steps_no_grad": num_steps_no_grad,
                 "num_steps_with_grad": num_steps_with_grad}
 
+    _MINIMAL_LOOP_KEYS = ("continuous_compute", "input_states_fn", "stop_tokens", "use_graph")
+
     @torch.no_grad()
-    def generate(self, input_ids: torch.Tensor, generation_config=None, **kwargs):
+    def generate(self, input_ids: Optional[torch.Tensor] = None, generation_config=None, **kwargs):
         """Dispatcher of RMM:1112-1127: `criterion` / `exit_threshold` / `exit_evaluator` select the adaptive-compute
         loop, `draft_steps` / `lookahead_for_draft` / `verification_threshold` the self-speculative one, `headway` /
-        `state_noise_mixing` / `inner_recurrence` / `freeze_strategy` the diffusion-style one; everything else goes to
-        generate_minimal (the reference hands those calls to transformers' GenerationMixin)."""
+        `state_noise_mixing` / `inner_recurrence` / `freeze_strategy` the diffusion-style one, `continuous_compute` (and
+        this package's own `input_states_fn` / `stop_tokens` / `use_graph`, or a GenerationSettings) generate_minimal;
+        every other call is transformers' GenerationMixin.generate over this model's forward."""
         if any(k in kwargs for k in ("criterion", "exit_threshold", "exit_evaluator")):
             return self.generate_with_adaptive_compute(input_ids, generation_config, **kwargs)
         if any(k in kwargs for k in ("draft_steps", "lookahead_for_draft", "verification_threshold")):
             return self.generate_speculative(input_ids, generation_config, **kwargs)
         if any(k in kwargs for k in ("headway", "state_noise_mixing", "inner_recurrence", "freeze_strategy")):
             return self.generate_diffusion_style(input_ids, generation_config, **kwargs)
-        return self.generate_minimal(input_ids, generation_config, **kwargs)
+        if any(k in kwargs for k in self._MINIMAL_LOOP_KEYS) or isinstance(generation_config, GenerationSettings):
+            return self.generate_minimal(input_ids, generation_config, **kwargs)
+        if generation_config is not None:
+            kwargs["generation_config"] = generation_config
+        return super().generate(input_ids, **kwargs)
 
     def generate_diffusion_style(self, input_ids: torch.Tensor, generation_config=None, **kwargs):
         """RMM:1234-1549; see diffusion.generate_diffusion_style."""
@@ -792,7 +924,7 @@ class RavenForCausalLM(torch.nn.Module):
         elif getattr(gc, "max_new_tokens", None):
             max_new = gc.max_new_tokens
         else:
-            max_new = model_kwargs.get("max_length", gc.max_length) - prompt_len
+            max_new = model_kwargs.get("max_length", self._default_max_length(gc)) - prompt_len
         num_steps = model_kwargs.get("num_steps", None)
         stops = self._get_stops(gc) if stop_tokens is None else set(stop_tokens)
         input_ids = input_ids.to(self.device)
@@ -986,3 +1118,13 @@ class DecodeRunner:
         for s in list(range(n_steps)) + [-(i + 1) for i in range(cfg.n_layers_in_coda)]:
             c.note_append(s, 1, pos0)
         return self.logits, self.next_ids, self.latents
+
+
+
+# ---- transformers registration (RMM:2312-2323) -----------------------------------------------------
+RavenConfig.register_for_auto_class()
+RavenForCausalLM.register_for_auto_class("AutoModel")
+RavenForCausalLM.register_for_auto_class("AutoModelForCausalLM")
+AutoConfig.register("huginn_raven", RavenConfig, exist_ok=True)
+AutoModel.register(RavenConfig, RavenForCausalLM, exist_ok=True)
+AutoModelForCausalLM.register(RavenConfig, RavenForCausalLM, exist_ok=True)

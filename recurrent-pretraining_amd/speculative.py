@@ -38,7 +38,7 @@ def generate_speculative(model, input_ids: torch.Tensor, generation_config=None,
     elif getattr(gc, "max_new_tokens", None):
         max_new = gc.max_new_tokens
     else:
-        max_new = model_kwargs.get("max_length", gc.max_length) - prompt_len
+        max_new = model_kwargs.get("max_length", model._default_max_length(gc)) - prompt_len
     stops = model._get_stops(gc) if stop_tokens is None else set(stop_tokens)
     dev, h = model.device, model.config.n_embd
     input_ids = input_ids.to(dev)

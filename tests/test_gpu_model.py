@@ -151,6 +151,32 @@ def test_greedy_batch_and_zero_state_and_stop(tiny32):
     assert torch.equal(got_s.cpu(), want_s) and got_s.shape[1] < 17
 
 
+def test_transformers_generate_equals_generate_minimal_and_the_oracle(pkg, tiny32):
+    """A generate() call without any of the reference's own loop keywords is transformers' GenerationMixin loop over this
+    forward (RMM:1126-1127).  Greedy, with the zero initial state, it must emit the oracle's tokens, and so the tokens of
+    generate_minimal; repetition_penalty then goes through transformers' own logits processor."""
+    from transformers import AutoModelForCausalLM, GenerationConfig
+    s, w, model = tiny32
+    prompt = torch.randint(0, s.vocab_size, (3, 5), generator=torch.Generator().manual_seed(9))
+    want = O.greedy_generate(w, s, prompt, 12)
+    hf = model.generate(prompt.cuda(), max_new_tokens=12, do_sample=False, init_scale=0.0)
+    assert torch.equal(hf.cpu(), want)
+    own = model.generate(prompt.cuda(), max_new_tokens=12, init_scale=0.0, stop_tokens=set())
+    assert torch.equal(hf, own)
+    # a GenerationConfig object, fewer recurrences, the cache handed back
+    out = model.generate(prompt.cuda(), GenerationConfig(max_new_tokens=6, do_sample=False, return_dict_in_generate=True),
+                         init_scale=0.0, num_steps=2)
+    assert torch.equal(out.sequences.cpu(), O.greedy_generate(w, s, prompt, 6, num_steps=2))
+    assert isinstance(out.past_key_values, pkg.HuginnDynamicCache) and out.past_key_values.get_seq_length() == 5 + 6 - 1
+    # the penalty of transformers' processor is the reference's rule (RMM:2047-2061) over prompt and generated tokens
+    pen = model.generate(prompt.cuda(), max_new_tokens=10, do_sample=False, init_scale=0.0, repetition_penalty=1.5)
+    assert torch.equal(pen.cpu(), O.greedy_generate(w, s, prompt, 10, penalty=1.5))
+    # a model built through the Auto class from the configuration alone, given the same weights, is the same model
+    auto = AutoModelForCausalLM.from_config(pkg.RavenConfig.tiny(), dtype=torch.float32).to("cuda:0")
+    auto.load_state_dict(w, strict=True)
+    assert torch.equal(auto.generate(prompt.cuda(), max_new_tokens=12, do_sample=False, init_scale=0.0), hf)
+
+
 def test_repetition_penalty_follows_the_growing_sequence(pkg, tiny32):
     """generate_minimal penalises the tokens of the prompt AND of everything generated so far, on every step
     (RMM:1198-1201, 1946-1947, 2047-2061), also when it picks greedily.  A prompt whose plain greedy stream repeats one of

@@ -298,7 +298,9 @@ def test_checkpoint_directory_round_trip(pkg, tmp_path):
     assert len(set(index["weight_map"].values())) > 2 and "lm_head.weight" not in index["weight_map"]
     for d in (one, many):
         got = pkg.RavenForCausalLM.from_pretrained(str(d), device="cpu", dtype=torch.float32)
-        assert {k: v for k, v in got.config.to_dict().items() if k != "architectures"} == cfg.to_dict()
+        skip = ("architectures", "dtype", "torch_dtype")  # the file names the class and the dtype the weights were saved in
+        assert {k: v for k, v in got.config.to_dict().items() if k not in skip} == {k: v for k, v in cfg.to_dict().items() if k not in skip}
+        assert got.config.to_dict()["dtype"] == "float32" and got.config.architectures == ["RavenForCausalLM"]
         sd = got.state_dict()
         assert sd.keys() == want.keys() and all(torch.equal(sd[k], want[k]) for k in want)
         assert got.lm_head.weight.data_ptr() == got.transformer.wte.weight.data_ptr()          # still tied
@@ -386,3 +388,124 @@ def test_repetition_penalties_against_the_reference_loops(pkg):
     assert cfg.to_dict()["test_time_noise"] == 0.1 and cfg.to_dict()["test_time_noise_type"] == "geom"
     with pytest.raises(ValueError):
         pkg.RavenConfig(test_time_noise=0.1, test_time_noise_type="pink")
+
+
+# ---- the transformers surface (RMM:36-112, 1066-1127, 2312-2323) --------------------------------------------------
+TINY_KEYS = ("n_embd", "n_heads", "n_layers", "n_layers_in_prelude", "n_layers_in_recurrent_block", "n_layers_in_coda",
+             "intermediate_size", "vocab_size", "mean_recurrence")
+
+
+def test_auto_classes_resolve_huginn_raven_and_build_from_a_config(pkg, tmp_path):
+    from transformers import AutoConfig, AutoModel, AutoModelForCausalLM, GenerationMixin, PretrainedConfig, PreTrainedModel
+    tiny = pkg.RavenConfig.tiny()
+    cfg = AutoConfig.for_model("huginn_raven", **{k: getattr(tiny, k) for k in TINY_KEYS})
+    assert type(cfg) is pkg.RavenConfig and isinstance(cfg, PretrainedConfig)
+    assert (cfg.hidden_size, cfg.num_attention_heads, cfg.num_hidden_layers) == (256, 4, 4)      # raven_config_minimal.py:10
+    assert cfg.tie_word_embeddings is True and cfg.dtype == torch.bfloat16
+    model = AutoModelForCausalLM.from_config(cfg)
+    assert type(model) is pkg.RavenForCausalLM and isinstance(model, PreTrainedModel) and isinstance(model, GenerationMixin)
+    assert type(AutoModel.from_config(cfg)) is pkg.RavenForCausalLM
+    assert model._tied_weights_keys == {"lm_head.weight": "transformer.wte.weight"}
+    assert model.lm_head.weight.data_ptr() == model.transformer.wte.weight.data_ptr()
+    assert model.dtype == torch.bfloat16 and not model.training
+    # the reference's initialisation (RMM:73-110): truncated at 3 std, output projections scaled down, norms one
+    iv, sd = cfg.init_values, model.state_dict()
+    fc = sd["transformer.core_block.0.mlp.fc.weight"].float()
+    for t, std in ((sd["transformer.wte.weight"], iv["embedding"]), (sd["transformer.adapter.weight"], iv["std"]),
+                   (sd["transformer.prelude.0.attn.Wqkv.weight"], iv["std"]), (fc[: fc.shape[0] // 2], iv["std"]),
+                   (fc[fc.shape[0] // 2:], iv["out_proj"]), (sd["transformer.coda.0.mlp.proj.weight"], iv["out_proj"]),
+                   (sd["transformer.core_block.1.attn.proj.weight"], iv["out_proj"])):
+        t = t.float()
+        assert abs(t.std().item() / std - 1) < 0.08 and t.abs().max().item() <= 3.02 * std and abs(t.mean().item()) < 0.1 * std
+    assert torch.all(sd["transformer.ln_f.weight"] == 1) and torch.all(sd["transformer.core_block.0.attn.qk_bias"] == 0)
+    # a saved directory comes back through the Auto classes with the same tensors
+    model.save_pretrained(tmp_path / "ckpt")
+    assert AutoConfig.from_pretrained(str(tmp_path / "ckpt")).to_dict()["n_embd"] == 256
+    back = AutoModelForCausalLM.from_pretrained(str(tmp_path / "ckpt"), device_map="cpu", torch_dtype=torch.bfloat16, trust_remote_code=True)
+    assert type(back) is pkg.RavenForCausalLM
+    assert all(torch.equal(v, back.state_dict()[k]) for k, v in sd.items())
+    # the forward needs the GPU library and says so instead of computing anything on the CPU
+    with pytest.raises((pkg.hip.RavenHipError, RuntimeError)):
+        model(input_ids=torch.zeros(1, 2, dtype=torch.long))
+
+
+def _with_counting_forward(pkg, model, calls):
+    """Replaces the forward by a stand-in that only does the cache bookkeeping and makes token (seen + S) % 7 win."""
+    def forward(input_ids=None, past_key_values=None, use_cache=False, position_ids=None, num_steps=None, **kw):
+        B, S = input_ids.shape
+        if use_cache and past_key_values is None:
+            past_key_values = pkg.HuginnDynamicCache()
+        seen = past_key_values._seen_tokens if past_key_values is not None else 0
+        calls.append((S, seen, None if position_ids is None else position_ids.reshape(-1)[-S:].tolist(), num_steps))
+        if past_key_values is not None:
+            past_key_values._seen_tokens += S
+        logits = torch.zeros(B, S, model.config.vocab_size)
+        logits[:, :, (seen + S) % 7] = 1.0
+        return pkg.CausalLMOutputRecurrentLatents(logits=logits, past_key_values=past_key_values)
+    model.forward = forward
+
+
+def test_transformers_generate_drives_the_forward_one_token_at_a_time(pkg):
+    """The plain generate() call is transformers' loop (RMM:1126-1127): prompt once, then one token per forward on the
+    cache the forward returned, positions following the cache, keyword arguments of the forward passed through."""
+    from transformers import DynamicCache
+    model = pkg.RavenForCausalLM(pkg.RavenConfig.tiny(), device="cpu")
+    calls = []
+    _with_counting_forward(pkg, model, calls)
+    ids = torch.tensor([[5, 6, 7], [8, 9, 10]])
+    out = model.generate(ids, max_new_tokens=4, do_sample=False, num_steps=3)
+    assert out.tolist() == [[5, 6, 7, 3, 4, 5, 6], [8, 9, 10, 3, 4, 5, 6]]
+    assert calls == [(3, 0, [0, 1, 2], 3), (1, 3, [3], 3), (1, 4, [4], 3), (1, 5, [5], 3)]
+    # an empty cache of transformers' own class is swapped for this package's; one that holds tokens is refused
+    calls.clear()
+    out = model.generate(ids, max_new_tokens=2, do_sample=False, past_key_values=DynamicCache(config=model.config))
+    assert out.shape == (2, 5) and [c[:2] for c in calls] == [(3, 0), (1, 3)]
+
+    class Used:
+        def get_seq_length(self):
+            return 2
+    with pytest.raises(ValueError, match="empty"):
+        model.prepare_inputs_for_generation(ids, past_key_values=Used(), use_cache=True)
+
+
+def test_prepare_inputs_for_generation_selects_the_new_tokens(pkg):
+    model = pkg.RavenForCausalLM(pkg.RavenConfig.tiny(), device="cpu")
+    ids = torch.arange(10).view(2, 5)
+    cache = pkg.HuginnDynamicCache()
+    # transformers 4.x: the loop hands over cache positions (RMM:1100)
+    got = model.prepare_inputs_for_generation(ids, past_key_values=cache, cache_position=torch.tensor([3, 4]), use_cache=True, num_steps=2)
+    assert got["input_ids"].tolist() == [[3, 4], [8, 9]] and got["past_key_values"] is cache and got["num_steps"] == 2
+    assert got["cache_position"].tolist() == [3, 4] and "position_ids" not in got and "attention_mask" not in got
+    # transformers 5.x: the number of new tokens, and positions the loop keeps for the whole sequence
+    pos = torch.arange(5).view(1, 5)
+    got = model.prepare_inputs_for_generation(ids, next_sequence_length=1, past_key_values=cache, position_ids=pos, use_cache=True,
+                                              attention_mask=torch.ones(2, 5))
+    assert got["input_ids"].tolist() == [[4], [9]] and got["position_ids"].tolist() == [[4]] and "attention_mask" not in got
+    assert got["input_ids"].is_contiguous()
+    # neither: all tokens; without use_cache no cache reaches the forward
+    got = model.prepare_inputs_for_generation(ids, past_key_values=cache, use_cache=False)
+    assert got["input_ids"].shape == (2, 5) and got["past_key_values"] is None
+    # positions given per sequence must agree between the sequences (RMM:660-665 rotates the batch with one list)
+    assert model._rope_positions(3, torch.tensor([[2, 3, 4], [2, 3, 4]]), None) == [2, 3, 4]
+    with pytest.raises(ValueError, match="shared"):
+        model._rope_positions(3, torch.tensor([[2, 3, 4], [0, 1, 2]]), None)
+
+
+def test_generate_dispatch_follows_the_reference_keywords(pkg, monkeypatch):
+    """RMM:1112-1127."""
+    model = pkg.RavenForCausalLM(pkg.RavenConfig.tiny(), device="cpu")
+    seen = []
+    for name in ("generate_with_adaptive_compute", "generate_speculative", "generate_diffusion_style", "generate_minimal"):
+        monkeypatch.setattr(model, name, lambda *a, _n=name, **k: seen.append(_n))
+    from transformers import GenerationMixin
+    monkeypatch.setattr(GenerationMixin, "generate", lambda self, *a, **k: seen.append("transformers"))
+    ids = torch.zeros(1, 2, dtype=torch.long)
+    model.generate(ids, criterion="entropy-diff")
+    model.generate(ids, draft_steps=2)
+    model.generate(ids, headway=1)
+    model.generate(ids, continuous_compute=True)
+    model.generate(ids, stop_tokens=set())
+    model.generate(ids, pkg.GenerationSettings(max_new_tokens=2))
+    model.generate(ids, max_new_tokens=2)
+    assert seen == ["generate_with_adaptive_compute", "generate_speculative", "generate_diffusion_style", "generate_minimal",
+                    "generate_minimal", "generate_minimal", "transformers"]

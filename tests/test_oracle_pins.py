@@ -748,3 +748,21 @@ def test_line_noise_replaces_the_state_at_step_zero_inside_forward():
     out_c = O.forward(w, s2, input_ids=ids, input_states=a, noise_draws=_Draws(seed=9))
     out_d = O.forward(w, s2, input_ids=ids, input_states=b, noise_draws=_Draws(seed=9))
     assert not torch.equal(out_c.logits, out_d.logits)
+
+
+def test_bench_counts_the_same_bytes_and_keeps_the_oracle_to_its_cpu_leg(pkg):
+    """bench.py carries its own statement of an iteration's algorithmic bytes (the product side may not import the
+    oracle); it must agree with the pinned count above, and the oracle import must sit inside cpu_baseline only."""
+    import ast
+    import os
+    import bench
+    s = O.RavenShape.nebel()
+    for B, T in ((1, 1024), (8, 640), (32, 1024)):
+        assert bench.core_iteration_bytes(pkg.RavenConfig(), B, T) == O.core_iteration_bytes(s, B, T)
+    tree = ast.parse(open(os.path.join(os.path.dirname(bench.__file__), "bench.py")).read())
+    holders = [fn.name for fn in ast.walk(tree) if isinstance(fn, ast.FunctionDef)
+               for node in ast.walk(fn) if isinstance(node, (ast.Import, ast.ImportFrom))
+               and "oracle" in (getattr(node, "module", None) or " ".join(a.name for a in node.names))]
+    top = [node for node in tree.body if isinstance(node, (ast.Import, ast.ImportFrom))
+           and "oracle" in (getattr(node, "module", None) or " ".join(a.name for a in node.names))]
+    assert holders == ["cpu_baseline"] and not top
