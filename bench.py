@@ -56,6 +56,8 @@ def parse():
                     help="launch-shape override passed to raven_set_tuning before the run (experiments only)")
     ap.add_argument("--attention-only", type=int, default=0, metavar="N",
                     help="with --prefill: run only N launches of the chunk attention kernel at that shape (for rocprofv3 --pmc runs)")
+    ap.add_argument("--gemm-only", type=int, default=0, metavar="N",
+                    help="with --prefill: launch each of the five products of a core iteration N times at the prefill shape and time it")
     ap.add_argument("--kernel-only", type=int, default=0, metavar="N",
                     help="run only N launches of the dominant kernel plus one 256 MiB device copy (for rocprofv3 --pmc runs)")
     return ap.parse_args()
@@ -301,6 +303,47 @@ def attention_only(args):
                       "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4)}))
 
 
+def gemm_only(args):
+    """The five products of one core iteration alone at the prefill shape (--prefill-batch x --prefill-len token rows):
+    synthetic operands, HIP events around --gemm-only launches of each, the four core blocks' worth of weights rotated so
+    that no launch finds its matrix in a cache."""
+    import torch
+    import __graft_entry__ as entry
+    pkg = entry.import_package()
+    pkg.hip.load()
+    cfg = pkg.RavenConfig()
+    dev = torch.device("cuda:0")
+    M, h, inter = args.prefill_batch * args.prefill_len, cfg.n_embd, cfg.intermediate_size
+    torch.manual_seed(0)
+
+    def mats(n, k):
+        return [torch.randn(n, k, device=dev, dtype=torch.bfloat16) * 0.02 for _ in range(4)]
+
+    x, e, res = (torch.randn(M, h, device=dev, dtype=torch.bfloat16) for _ in range(3))
+    g = torch.randn(M, inter, device=dev, dtype=torch.bfloat16)
+    cases = [("mlp.fc + SwiGLU", mats(2 * inter, h), dict(x=x, swiglu=True)), ("attn.Wqkv", mats(3 * h, h), dict(x=x)),
+             ("attn.proj + residual", mats(h, h), dict(x=x, residual=res)), ("mlp.proj + residual", mats(h, inter), dict(x=g, residual=res)),
+             ("adapter (two K segments)", mats(h, 2 * h), dict(x=x, x1=e))]
+    out = {"gemm_only": args.gemm_only, "kernel": "gemm_tiled_kernel", "rows": M, "products": {}}
+    total_ms, total_flops = 0.0, 0.0
+    for name, ws, kw in cases:
+        xin = kw.pop("x")
+
+        def launch(i=[0]):
+            i[0] += 1
+            pkg.hip.linear(xin, ws[i[0] % 4], **kw)
+
+        ms = event_time_ms(launch, args.gemm_only, warm=2)
+        flops = 2.0 * M * ws[0].shape[0] * ws[0].shape[1]
+        n_iter = 1 if name.startswith("adapter") else 4
+        total_ms += n_iter * ms
+        total_flops += n_iter * flops
+        out["products"][name] = {"N": ws[0].shape[0], "K": ws[0].shape[1], "ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
+                                 "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4)}
+    out["per_iteration"] = {"ms": round(total_ms, 3), "TFLOP/s": round(total_flops / total_ms / 1e9, 1)}
+    print(json.dumps(out))
+
+
 def kernel_only(n_launches):
     """The dominant kernel alone, as the decode loop launches it, on four rotating fc matrices, followed by
     one device copy of known size (the yardstick that scales FETCH_SIZE / WRITE_SIZE readings)."""
@@ -399,6 +442,9 @@ def main():
         return
     if args.prefill and args.attention_only:
         attention_only(args)
+        return
+    if args.prefill and args.gemm_only:
+        gemm_only(args)
         return
     if args.prefill:
         prefill(args)

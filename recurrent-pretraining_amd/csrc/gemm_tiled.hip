@@ -113,6 +113,78 @@ __device__ __forceinline__ void store_tiles(const TiledArgs& a, const f32x16 (&a
     }
 }
 
+// Epilogue through LDS for the bf16 outputs: the accumulators (a lane: 4 columns of 32 different token rows per store)
+// are laid down as the output tile, rows of BN_OUT columns, and read back so that a wave instruction stores two whole
+// tile rows, 16 bytes per lane: full 128-byte lines instead of 32 pieces of 16 bytes.  The residual is fetched the same
+// way, before the tile is laid down, so that its latency hides behind the transposition.  16-byte unit u of tile row r
+// sits at position u ^ (r mod units per row): the 32 rows a store instruction spreads over then fall on different banks.
+template <bool SWIGLU, int TM, int TN>
+__device__ __forceinline__ void store_tiles_lds(const TiledArgs& a, const f32x16 (&acc)[TN][TM], int tile_m, int tile_n, int wave, int lane,
+                                                unsigned lds_base) {
+    constexpr int BM = 2 * TM * 32, BN = 4 * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
+    constexpr int RB = BN_OUT * 2, U = RB / 16;      // bytes and 16-byte units per tile row
+    constexpr int ITERS = BM * U / 512;              // 16-byte units per lane
+    const int wn = wave & 3, wm = wave >> 2, l32 = lane & 31, hi = lane >> 5;
+    bf16* const y = static_cast<bf16*>(a.y);
+    int64_t goff[ITERS];                             // element offset of this lane's unit in y / residual, -1: outside
+    u32x4 res[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int idx = (wave * ITERS + it) * 64 + lane;
+        const int m = tile_m * BM + idx / U, n = tile_n * BN_OUT + (idx % U) * 8;
+        goff[it] = (m < a.M && n < a.N) ? (int64_t)m * a.N + n : -1;
+        res[it] = u32x4{0, 0, 0, 0};
+        if (!SWIGLU && a.residual && goff[it] >= 0) res[it] = *reinterpret_cast<const u32x4*>(a.residual + goff[it]);
+    }
+    // every wave has its last fragments; the stages are free
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+        const int row = (wm * TM + tm) * 32 + l32;
+        const unsigned row_addr = lds_base + row * RB + hi * 8;
+        const int sw = row & (U - 1);
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+            const int t32 = wn * TN + tn;
+#pragma unroll
+            for (int j = 0; j < (SWIGLU ? 2 : 4); ++j) {
+                bf16 o[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (SWIGLU) {
+                        const float g = round_to<bf16>(acc[tn][tm][4 * j + i]), u = round_to<bf16>(acc[tn][tm][8 + 4 * j + i]);
+                        o[i] = from_f32<bf16>(round_to<bf16>(silu_f32(g)) * u);
+                    } else {
+                        o[i] = from_f32<bf16>(acc[tn][tm][4 * j + i]);
+                    }
+                }
+                const int unit = t32 * (SWIGLU ? 2 : 4) + j;
+                *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(row_addr + ((unit ^ sw) * 16)) = *reinterpret_cast<const u32x2*>(o);
+            }
+        }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int idx = (wave * ITERS + it) * 64 + lane;
+        const int row = idx / U, unit = idx % U;
+        u32x4 v = *reinterpret_cast<const lds_u32x4*>(lds_base + row * RB + ((unit ^ (row & (U - 1))) * 16));
+        if (!SWIGLU && a.residual) {
+            bf16 o[8], r[8];
+            *reinterpret_cast<u32x4*>(o) = v;
+            *reinterpret_cast<u32x4*>(r) = res[it];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = from_f32<bf16>(to_f32(o[i]) + to_f32(r[i]));
+            v = *reinterpret_cast<const u32x4*>(o);
+        }
+        if (goff[it] >= 0) *reinterpret_cast<u32x4*>(y + goff[it]) = v;
+    }
+}
+
 __device__ __align__(16) unsigned int g_zero_piece[4];  // what a 16-byte piece past the end of K is loaded from
 
 template <bool SWIGLU, int TM, int TN>
@@ -289,7 +361,8 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
             move_under(it, k + 2, src3, ic0{});
         });
     }
-    store_tiles<SWIGLU, TM, TN>(a, acc, tile_m, tile_n, wm, wn, l32, hi);
+    if (a.out_f32) store_tiles<SWIGLU, TM, TN>(a, acc, tile_m, tile_n, wm, wn, l32, hi);
+    else store_tiles_lds<SWIGLU, TM, TN>(a, acc, tile_m, tile_n, wave, lane, lds_base);
 }
 
 int g_tiled_min_rows = 33;  // raven_set_tuning("gemm_tiled_min_rows"): fewest rows that take this kernel
@@ -332,7 +405,7 @@ int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residu
     RAVEN_REQUIRE(tiled_gemm_fits(M, N, K0, K1, RAVEN_BF16), "gemm (tiled): unsupported shape M=%d N=%d K0=%d K1=%d", M, N, K0, K1);
     RAVEN_REQUIRE(!(swiglu && (residual || out_f32)), "gemm (tiled): the SwiGLU epilogue has no residual and stores bf16");
     RAVEN_REQUIRE(((uintptr_t)x0 & 15) == 0 && ((uintptr_t)x1 & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)y & 15) == 0 &&
-                      ((uintptr_t)residual & 7) == 0, "gemm (tiled): operands must be 16-byte aligned");
+                      ((uintptr_t)residual & 15) == 0, "gemm (tiled): operands must be 16-byte aligned");
     TiledArgs a{};
     a.w = static_cast<const bf16*>(w);
     a.x0 = static_cast<const bf16*>(x0);
@@ -341,10 +414,15 @@ int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residu
     a.y = y;
     a.M = M; a.N = N; a.K0 = K0; a.K1 = x1 ? K1 : 0; a.out_f32 = out_f32;
     // 256 x 256 tiles when they fill the chip at least once; 128 x 128 tiles otherwise
-    const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + (swiglu ? 127 : 255)) / (swiglu ? 128 : 256));
+    const int bn_out = swiglu ? 128 : 256;
+    const int64_t tiles_n = (N + bn_out - 1) / bn_out, tiles_m = (M + 255) / 256;
+    const int64_t big_tiles = tiles_m * tiles_n;
     const bool big = g_tiled_variant == 1 || (g_tiled_variant == 0 && big_tiles >= 256);
-    if (swiglu) return big ? launch_tiled<true, 4, 2>(a, s) : launch_tiled<true, 2, 1>(a, s);
-    return big ? launch_tiled<false, 4, 2>(a, s) : launch_tiled<false, 2, 1>(a, s);
+    auto launch = [&](const TiledArgs& t, bool as_big) {
+        if (swiglu) return as_big ? launch_tiled<true, 4, 2>(t, s) : launch_tiled<true, 2, 1>(t, s);
+        return as_big ? launch_tiled<false, 4, 2>(t, s) : launch_tiled<false, 2, 1>(t, s);
+    };
+    return launch(a, big);
 }
 
 }  // namespace raven
