@@ -344,9 +344,9 @@ def gemm_only(args):
     print(json.dumps(out))
 
 
-def kernel_only(n_launches):
-    """The dominant kernel alone, as the decode loop launches it, on four rotating fc matrices, followed by
-    one device copy of known size (the yardstick that scales FETCH_SIZE / WRITE_SIZE readings)."""
+def kernel_only(n_launches, batch=1):
+    """The dominant kernel alone, as the decode loop launches it at `batch` sequences, on four rotating fc matrices,
+    followed by one device copy of known size (the yardstick that scales FETCH_SIZE / WRITE_SIZE readings)."""
     import torch
     import __graft_entry__ as entry
     pkg = entry.import_package()
@@ -357,18 +357,21 @@ def kernel_only(n_launches):
     torch.manual_seed(0)
     fcs = [torch.randn(2 * inter, h, device=dev, dtype=torch.bfloat16) * 0.02 for _ in range(4)]
     na, nb = (torch.ones(h, device=dev, dtype=torch.bfloat16) for _ in range(2))
-    x = torch.randn(h, device=dev, dtype=torch.bfloat16)
-    x2, g = torch.empty_like(x), torch.empty(inter, device=dev, dtype=torch.bfloat16)
+    x = torch.randn(batch, h, device=dev, dtype=torch.bfloat16)
+    x2, g = torch.empty_like(x), torch.empty(batch, inter, device=dev, dtype=torch.bfloat16)
     stream = torch.cuda.current_stream().cuda_stream
     for i in range(n_launches):
-        lib.raven_gemv_fused(x.data_ptr(), None, na.data_ptr(), nb.data_ptr(), x2.data_ptr(), fcs[i % 4].data_ptr(), None,
-                             g.data_ptr(), inter, h, 0, cfg.norm_eps, 1, 0, pkg.hip.BF16, stream)
+        if batch == 1:
+            lib.raven_gemv_fused(x.data_ptr(), None, na.data_ptr(), nb.data_ptr(), x2.data_ptr(), fcs[i % 4].data_ptr(), None,
+                                 g.data_ptr(), inter, h, 0, cfg.norm_eps, 1, 0, pkg.hip.BF16, stream)
+        else:
+            lib.raven_gemm_swiglu(x.data_ptr(), fcs[i % 4].data_ptr(), g.data_ptr(), batch, inter, h, pkg.hip.BF16, stream)
     torch.cuda.synchronize()
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
     dst = torch.empty_like(src)
     dst.copy_(src)
     torch.cuda.synchronize()
-    print(json.dumps({"kernel_only": n_launches, "bytes_per_launch": 2 * inter * h * 2 + h * 2 + inter * 2,
+    print(json.dumps({"kernel_only": n_launches, "batch": batch, "bytes_per_launch": 2 * inter * h * 2 + batch * h * 2 + batch * inter * 2,
                       "copy_bytes": src.numel()}))
 
 
@@ -438,7 +441,7 @@ def main():
     args = parse()
     apply_tuning(args)
     if args.kernel_only:
-        kernel_only(args.kernel_only)
+        kernel_only(args.kernel_only, args.batch)
         return
     if args.prefill and args.attention_only:
         attention_only(args)

@@ -273,7 +273,9 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
             if (shift > seg_len) shift = 0;
         }
         const int n_macro = (seg_len - shift) / KM;
-        const int mb = (int)((int64_t)n_macro * wave / 4), me = (int)((int64_t)n_macro * (wave + 1) / 4);
+        // the four waves take the macro-steps in turn, so that the workgroup as a whole walks its rows in pieces of
+        // 4 * KM contiguous elements (DRAM pages are then read in longer runs than one wave's 256 bytes)
+        const int mb = wave, me = n_macro;
 
         auto fetch = [&](int mac, Staged& st) {  // global -> registers, row-contiguous lanes
             const int k = shift + mac * KM + lc;
@@ -326,10 +328,10 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
         // one register set: its loads for macro-step s+1 are in flight while step s is multiplied out of LDS
         Staged st;
         if (mb < me) fetch(mb, st);
-        for (int mac = mb; mac < me; ++mac) {
+        for (int mac = mb; mac < me; mac += 4) {
             park(st);
             wave_sync();
-            if (mac + 1 < me) fetch(mac + 1, st);
+            if (mac + 4 < me) fetch(mac + 4, st);
             multiply();
             wave_sync();
         }
