@@ -32,12 +32,13 @@ How each function is pinned (tests/test_oracle_pins.py), without running the ref
   embed_inputs / iterate_one_step / predict_from_latents / generate_with_adaptive_compute
                      pieces compose to forward(); criterion "none" equals greedy_generate;
                      num-steps evaluator equals forward(num_steps=k) token by token -> pinned
-  generate_diffusion_style   the first position of the wave followed by hand (its embedding average, noise
-                     mixing and recurrences over several steps, on a private copy of the prompt cache)
-                     gives the token the loop freezes there; schedule / counter closed forms for the
-                     "fixed" strategy and for exit thresholds 0 and infinity.  The later positions' tokens
-                     (whose inputs change from step to step) have no independent check: parity unpinned
-                     beyond that                                                     -> partly pinned
+  generate_diffusion_style   every position of the wave recomputed one position at a time, without a step-indexed
+                     cache, roll-back or batching (each position keeps the key/value rows of its own last
+                     computation; tokens, embedding averages, noise damping and the freeze rule restated per
+                     position): states and logits of all wave positions after every step and the frozen text, for
+                     "fixed" and for "latent-diff" at two thresholds with waves up to 12 wide; the leftmost
+                     position also by hand on a copy of the prompt cache; schedule / counter closed forms for
+                     "fixed" and for exit thresholds 0 and infinity                  -> pinned
   inject_noise       amplitude n = t * sqrt(2/5) and the per-type coefficients (n/(k+1), n/sqrt(k+1), max(n, (r-k)/r),
                      2un) by closed form on x = 0 / noise = 1; zero noise leaves norm_4(x) (scale invariance);
                      "line" at step 0 replaces the state, so forward() no longer depends on input_states;
@@ -931,6 +932,7 @@ def generate_diffusion_style(w, s: RavenShape, input_ids: torch.Tensor, max_new_
             passes, tokens_forward = passes + 1, tokens_forward + n_wave
         logits = predict_from_latents(w, s, states, cache=cache, cache_position=pos).logits
         first_state, first_logits = states[0, 0].clone(), logits[0, 0].clone()  # of the wave's leftmost position, for the record
+        wave_states = states[0].clone()                                         # of every position of the wave
         # positions whose prediction is not frozen yet: from the last frozen token on (RMM:1366-1369)
         new_tokens = logits[0, max(frozen.shape[1] - 1 - ci, 0):, :].argmax(-1, keepdim=True).T
         guess = torch.cat([frozen, new_tokens[:, :-1]], dim=1)
@@ -1011,7 +1013,7 @@ def generate_diffusion_style(w, s: RavenShape, input_ids: torch.Tensor, max_new_
         else:
             raise ValueError(f"Invalid freeze strategy {freeze_strategy}")
         log.append(dict(step=step, cache_index=ci, wave=n_wave, frozen=frozen.shape[1], current=current[0].tolist(),
-                        first_state=first_state, first_logits=first_logits))
+                        first_state=first_state, first_logits=first_logits, wave_states=wave_states, wave_logits=logits[0].clone()))
 
         if step > num_steps:                                               # RMM:1478-1492
             seen = frozen[0, old_k:k].tolist() if latent else frozen[0, -headway:].tolist()

@@ -766,3 +766,168 @@ def test_bench_counts_the_same_bytes_and_keeps_the_oracle_to_its_cpu_leg(pkg):
     top = [node for node in tree.body if isinstance(node, (ast.Import, ast.ImportFrom))
            and "oracle" in (getattr(node, "module", None) or " ".join(a.name for a in node.names))]
     assert holders == ["cpu_baseline"] and not top
+
+
+# ----------------------------------------------------------------------------- diffusion sampler, every wave position
+class _RowContext:
+    """What one position sees, kept position by position instead of in a step-indexed cache: `done[q][step_idx]` holds the
+    key/value row that position q wrote at block `step_idx` the last time it was computed.  The position being computed
+    reads, at block `step_idx`, the rows of all positions to its left -- from the same block of the same recurrence when
+    that position was computed earlier in this pass (it is part of the same wave), else from that position's last pass:
+    its last recurrence for a core block (which is what a cache that keeps one slot per core block holds)."""
+
+    def __init__(self, shape):
+        self.s = shape
+        self.done = {}      # position -> {step_idx: (k, v)} of its last complete pass
+        self.pass_rows = {}  # position -> {step_idx: (k, v)} of the pass in progress (all positions of the current wave)
+        self.pos = None
+        self.write = True
+
+    def core_class(self, step_idx):
+        n_pre, n_core = self.s.n_layers_in_prelude, self.s.n_layers_in_recurrent_block
+        return None if step_idx < n_pre else (step_idx - n_pre) % n_core   # coda blocks (negative) never get here
+
+    def rows_of(self, q, step_idx):
+        if q in self.pass_rows and step_idx in self.pass_rows[q]:
+            return self.pass_rows[q][step_idx]
+        rows = self.done[q]                       # a position from an earlier pass
+        cls = self.core_class(step_idx)
+        if step_idx < 0 or cls is None:           # prelude and coda blocks run once per pass
+            return rows[step_idx]
+        last = max(i for i in rows if i >= self.s.n_layers_in_prelude and self.core_class(i) == cls)
+        return rows[last]                         # its last recurrence of that core block
+
+    def update(self, k, v, step_idx, lookup_strategy=None):
+        left = [self.rows_of(q, step_idx) for q in range(self.pos)]
+        if self.write:
+            self.pass_rows.setdefault(self.pos, {})[step_idx] = (k, v)
+        ks = torch.cat([r[0] for r in left] + [k], dim=2)
+        vs = torch.cat([r[1] for r in left] + [v], dim=2)
+        return ks, vs
+
+    def end_pass(self):
+        self.done.update(self.pass_rows)
+        self.pass_rows = {}
+
+
+def _one_position(s, w, ctx, p, token, state, n_rec, embed_mix=None, write=True):
+    """Prelude, n_rec recurrences and coda for position p alone; returns (embedding used, state, logits)."""
+    ctx.pos, ctx.write = p, write
+    cp = torch.tensor([p])
+    e, block_idx = O.embed_inputs(w, s, token.view(1, 1), cache=ctx, cache_position=cp)
+    if embed_mix is not None:
+        e = embed_mix(e)
+    for _ in range(n_rec):
+        state, block_idx = O.iterate_one_step(w, s, e, state, block_idx, cache=ctx, cache_position=cp)
+    logits = O.predict_from_latents(w, s, state, cache=ctx, cache_position=cp).logits[0, 0] if n_rec else None
+    return e, state, logits
+
+
+@pytest.mark.parametrize("strategy,exit_t", [("fixed", None), ("latent-diff", 0.35), ("latent-diff", 0.2)])
+def test_diffusion_sampler_every_wave_position_followed_position_by_position(strategy, exit_t):
+    """The sampler advances a wave of positions together, over a cache with one slot per core block whose wave part is
+    rolled back after every step.  Here the same text is produced one position at a time, with no step-indexed cache,
+    no roll-back and no batching: every position keeps the key/value rows of its own last computation, and a position
+    reads its left neighbours row by row (_RowContext).  The bookkeeping is restated per position as well: a position's
+    token is the frozen one or the previous step's prediction of its left neighbour; its embedding is averaged with its
+    own previous one; its state is mixed with noise damped by its own recurrence count; "fixed" freezes the leftmost
+    wave position from step num_steps // inner + 1 on, "latent-diff" everything up to the rightmost position whose state
+    moved by less than exit_t since the previous step.  States and logits of EVERY wave position must agree after every
+    step, and the frozen text at the end -- so a wrong wave offset, roll-back count, slot, guess alignment or damping
+    count for any position, not only the leftmost, shows."""
+    s, w, ids, sf = _diffusion_model()
+    n, h = ids.shape[1], s.n_embd
+    num_steps, inner, a, m, max_new = 4, 2, 0.1, 0.5, 5
+    rec = {}
+    kw = dict(freeze_strategy=strategy) if exit_t is None else dict(freeze_strategy=strategy, exit_t=exit_t)
+    got = O.generate_diffusion_style(w, s, ids, max_new, num_steps=num_steps, inner_recurrence=inner, ema_embeds=a, state_noise_mixing=m,
+                                     state_fn=sf, record=rec, **kw)
+    # ---- position by position
+    ctx = _RowContext(s)
+    x0 = sf(0, (1, n, h))
+    for p in range(n):                                             # the prompt, num_steps recurrences per position
+        _, _, logits = _one_position(s, w, ctx, p, ids[0, p], x0[:, p:p + 1], num_steps)
+    ctx.end_pass()
+    text = ids[0].tolist() + [int(logits.argmax())]                # frozen tokens
+    n_frozen = n + 1
+    guess = {}                                                     # position -> predicted token, for positions not frozen yet
+    state = {n: sf(1, (1, 1, h))}
+    count = {n: num_steps}                                         # recurrences a position has had (the prefill counts for n)
+    old_e = {n: _one_position(s, w, ctx, n, torch.tensor(text[n]), None, 0, write=False)[0]}
+    prev_state = None
+    hold = num_steps // inner
+    draws, t = 2, 0
+    while n_frozen - n < max_new:
+        first = n_frozen - 1                                       # the newest frozen token is the wave's leftmost position
+        wave = sorted(state)
+        assert wave == list(range(first, first + len(wave)))
+        entry = rec["log"][t]
+        assert (entry["cache_index"], entry["wave"]) == (first, len(wave)), t
+        noise = sf(draws, (1, len(wave), h))
+        after, logit_of = {}, {}
+        for i, p in enumerate(wave):
+            tok = text[p] if p < n_frozen else guess[p]
+            x = state[p]
+            mix = m / (1 + count.get(p, 0))
+            x = x * (1 - mix) + mix * noise[:, i:i + 1]
+            carry = old_e.get(p)
+            e, x, lg = _one_position(s, w, ctx, p, torch.tensor(tok), x, inner,
+                                     embed_mix=lambda new, c=carry: new * (1 - a) + (c * a if c is not None else 0))
+            old_e[p], after[p], logit_of[p] = e, x, lg
+            count[p] = count.get(p, 0) + inner
+            assert torch.allclose(entry["wave_states"][i], x[0, 0], rtol=1e-4, atol=1e-5), (t, p)
+            assert torch.allclose(entry["wave_logits"][i], lg, rtol=1e-4, atol=1e-5), (t, p)
+        ctx.end_pass()
+        for p in wave:                                             # predictions for the positions behind the frozen text
+            if p + 1 >= n_frozen:
+                guess[p + 1] = int(logit_of[p].argmax())
+        new_pos = wave[-1] + 1
+        after[new_pos] = sf(draws + 1, (1, 1, h)).to(torch.bfloat16).to(x0.dtype)
+        draws += 2
+        if strategy == "fixed":
+            new_frozen = n_frozen + (1 if t > hold else 0)
+        else:
+            new_frozen = n_frozen
+            if prev_state is not None:
+                moved = {p: float((after[p] - prev_state[p]).norm() / after[p].norm()) for p in after if p in prev_state}
+                settled = [p for p, v in moved.items() if v < exit_t]
+                if settled:
+                    new_frozen = max(settled) + 1
+        for p in range(n_frozen, new_frozen):
+            text.append(guess[p])
+        n_frozen = new_frozen
+        state = {p: x for p, x in after.items() if p >= n_frozen - 1}
+        old_e = {p: e for p, e in old_e.items() if p >= n_frozen - 1}
+        prev_state = dict(state)
+        assert entry["frozen"] == n_frozen, t
+        t += 1
+    assert got[0].tolist() == text[:got.shape[1]] and got.shape[1] == n_frozen
+    assert t == rec["diffusion_steps"]
+
+
+def test_repetition_penalty_by_hand_and_against_the_library_processor():
+    """RMM:2047-2061 is the rule of transformers' RepetitionPenaltyLogitsProcessor: seen tokens' logits are divided by the
+    penalty when positive and multiplied when negative; a token seen twice is penalised once; unseen tokens stay."""
+    from transformers import RepetitionPenaltyLogitsProcessor
+    logits = torch.tensor([[2.0, -3.0, 0.5, 4.0], [1.0, 1.0, -1.0, 0.0]])
+    ids = torch.tensor([[0, 1, 1], [2, 2, 3]])
+    got = O.repetition_penalty(logits, ids, 2.0)
+    assert got.tolist() == [[1.0, -6.0, 0.5, 4.0], [1.0, 1.0, -2.0, 0.0]]
+    g = torch.Generator().manual_seed(5)
+    big, seq = torch.randn(3, 50, generator=g), torch.randint(0, 50, (3, 12), generator=g)
+    assert torch.equal(O.repetition_penalty(big, seq, 1.3), RepetitionPenaltyLogitsProcessor(1.3)(seq, big.clone()))
+    # greedy_generate with a penalty = the plain loop with the library's processor applied to the growing sequence
+    s = O.RavenShape.tiny()
+    w = O.make_weights(s, seed=0, dtype=torch.float32)
+    proc = RepetitionPenaltyLogitsProcessor(1.6)
+    changed = 0
+    for seed in range(1000, 1012):
+        prompt = torch.randint(0, s.vocab_size, (1, 6), generator=torch.Generator().manual_seed(seed))
+        seq, cache = prompt.clone(), O.DictCache()
+        for _ in range(14):
+            pos = torch.arange(cache.get_seq_length(), seq.shape[1])
+            out = O.forward(w, s, input_ids=seq[:, pos], past_key_values=cache, use_cache=True, cache_position=pos, init_scale=0.0)
+            seq = torch.cat([seq, proc(seq, out.logits[:, -1].float().clone()).argmax(-1, keepdim=True)], dim=-1)
+        assert torch.equal(O.greedy_generate(w, s, prompt, 14, penalty=1.6), seq), seed
+        changed += not torch.equal(O.greedy_generate(w, s, prompt, 14), seq)
+    assert changed >= 1                                                   # some of these streams repeat without the penalty
