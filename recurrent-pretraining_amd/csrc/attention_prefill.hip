@@ -64,18 +64,23 @@ __device__ __forceinline__ float max_over_quarters(float x) {
     return fmaxf(__builtin_bit_cast(float, q[0]), __builtin_bit_cast(float, q[1]));
 }
 
-template <int HD, int RG, bool PAGED = false>
-__global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a) {
+template <int HD, int RG, bool PAGED = false, int NW = 4>
+__global__ __launch_bounds__(NW * 64, NW == 6 ? 3 : 2) void attention_prefill_kernel(PrefillArgs a) {
+    constexpr int NTH = NW * 64;     // threads; NW waves, each with its own query rows
     constexpr int KS = HD / 32;      // k-steps of the score MFMA
     constexpr int NT = HD / 16;      // 16-wide output tiles of O; tile NT holds the row sums
     constexpr int KP = HD + 8;       // K tile row pitch (elements): (HD*2+16) bytes, 16-byte aligned rows
     constexpr int WR = 16 * RG;      // query rows per wave
-    constexpr int ROWS = 4 * WR;     // query rows per workgroup
-    __shared__ __align__(16) bf16 sk[2][kPfKeys][KP];
+    constexpr int ROWS = NW * WR;    // query rows per workgroup
+    constexpr int kVPitch = HD + 16;
+    // one block of LDS: the two K buffers, then the two V buffers; the output pass at the end reuses all of it
+    constexpr int SK_ELEMS = 2 * kPfKeys * KP, SV_ELEMS = 2 * kPfKeys * kVPitch;
+    static_assert(SK_ELEMS + SV_ELEMS >= NW * (RG == 1 ? 16 : 32) * KP, "the output pass fits the staging buffers");
+    __shared__ __align__(16) bf16 smem_kv[SK_ELEMS + SV_ELEMS];
+    bf16(*sk)[kPfKeys][KP] = reinterpret_cast<bf16(*)[kPfKeys][KP]>(smem_kv);
     // bf16 elements per V row in LDS: HD + 16, i.e. 40 / 56 / 72 banks -- an odd multiple of 8, so that the 8 key rows that
     // 32 lanes read transposed (8 banks each) hit 64 different banks
-    constexpr int kVPitch = HD + 16;
-    __shared__ __align__(16) bf16 sv[2][kPfKeys][kVPitch];
+    bf16(*sv)[kPfKeys][kVPitch] = reinterpret_cast<bf16(*)[kPfKeys][kVPitch]>(smem_kv + SK_ELEMS);
 
     const int qb = gridDim.x - 1 - blockIdx.x;  // the blocks with the most keys start first
     const int head = blockIdx.y, b = blockIdx.z;
@@ -94,7 +99,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
         t_lim = a.seq_lens[b];
         pos0 = t_lim - n_rows;
         table_row = a.block_table + (int64_t)b * a.max_blocks;
-        if (n_rows <= 0 || pos0 < 0 || qb * (64 * RG) >= n_rows) return;  // the grid is sized for the longest sequence
+        if (n_rows <= 0 || pos0 < 0 || qb * ROWS >= n_rows) return;  // the grid is sized for the longest sequence
     } else {
         q_row0 = (int64_t)b * a.S;
         n_rows = a.S;
@@ -143,8 +148,8 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
     // K and V tiles are contiguous pieces of the cache (or gathered page rows), moved as 16-byte chunks of key rows; V
     // stays row-major in LDS and is read through ds_read_b64_tr_b16, which hands a lane four keys of one column.
     constexpr int CPR = HD / 8;                     // chunks per key row
-    constexpr int KCH = kPfKeys * CPR / 256;        // chunks per thread, of K and of V
-    static_assert(kPfKeys * CPR % 256 == 0, "staging shape");
+    constexpr int KCH = kPfKeys * CPR / NTH;        // chunks per thread, of K and of V
+    static_assert(kPfKeys * CPR % NTH == 0, "staging shape");
     u32x4 kreg[KCH];
     u32x4 vreg[KCH];
     const bf16* k_src = Kb + threadIdx.x * 8;
@@ -152,7 +157,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
     int k_dst[KCH], v_dst[KCH];  // element offsets inside one buffer
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
-        const int c = threadIdx.x + 256 * i;
+        const int c = threadIdx.x + NTH * i;
         k_dst[i] = (c / CPR) * KP + (c % CPR) * 8;
         v_dst[i] = (c / CPR) * kVPitch + (c % CPR) * 8;
     }
@@ -176,7 +181,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
                 };
 #pragma unroll
                 for (int i = 0; i < KCH; ++i) {
-                    const int c = threadIdx.x + 256 * i;
+                    const int c = threadIdx.x + NTH * i;
                     const int key = c / CPR, dc = c - key * CPR;
                     const int64_t o = off(kt + key);
                     kreg[i] = *reinterpret_cast<const u32x4*>(Kb + o + dc * 8);
@@ -185,7 +190,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
             } else {
 #pragma unroll
                 for (int i = 0; i < KCH; ++i) {
-                    const int c = threadIdx.x + 256 * i;
+                    const int c = threadIdx.x + NTH * i;
                     const int key = c / CPR, dc = c - key * CPR;
                     const int64_t o = paged_off(kt + key);
                     kreg[i] = *reinterpret_cast<const u32x4*>(Kb + o + dc * 8);
@@ -194,13 +199,13 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
             }
         } else if (kt + kPfKeys <= a.t_max) {
 #pragma unroll
-            for (int i = 0; i < KCH; ++i) kreg[i] = *reinterpret_cast<const u32x4*>(k_src + (int64_t)kt * HD + 2048 * i);
+            for (int i = 0; i < KCH; ++i) kreg[i] = *reinterpret_cast<const u32x4*>(k_src + (int64_t)kt * HD + NTH * 8 * i);
 #pragma unroll
-            for (int i = 0; i < KCH; ++i) vreg[i] = *reinterpret_cast<const u32x4*>(v_src + (int64_t)kt * HD + 2048 * i);
+            for (int i = 0; i < KCH; ++i) vreg[i] = *reinterpret_cast<const u32x4*>(v_src + (int64_t)kt * HD + NTH * 8 * i);
         } else {  // the cache ends inside this tile: rows past it are masked below, their loads stay in bounds
 #pragma unroll
             for (int i = 0; i < KCH; ++i) {
-                const int c = threadIdx.x + 256 * i;
+                const int c = threadIdx.x + NTH * i;
                 const int key = c / CPR, dc = c - key * CPR;
                 const int64_t o = (int64_t)min(kt + key, a.t_max - 1) * HD + dc * 8;
                 kreg[i] = *reinterpret_cast<const u32x4*>(Kb + o);
@@ -336,7 +341,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
 
     if constexpr (PAGED) {
         const int n_pages = min((n_keys + a.block_size - 1) / a.block_size, kPfTable);
-        for (int i = threadIdx.x; i < n_pages; i += 256) tbl[i] = table_row[i];
+        for (int i = threadIdx.x; i < n_pages; i += NTH) tbl[i] = table_row[i];
         __syncthreads();
     }
     if (n_keys > 0) {
@@ -371,7 +376,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
     // rows round through LDS (the K buffers are free after the last barrier; each wave has its own WR x KP piece) and
     // writes 16-byte pieces of whole rows.
     constexpr int ER = RG == 1 ? 16 : 32;  // rows per pass
-    bf16* ot = &sk[0][0][0] + wave * (ER * KP);
+    bf16* ot = smem_kv + wave * (ER * KP);
 #pragma unroll
     for (int g0 = 0; g0 < RG; g0 += ER / 16) {
 #pragma unroll
@@ -397,6 +402,10 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(PrefillArgs a
 }
 
 }  // namespace raven
+
+namespace raven {
+int g_prefill_waves = 0;  // raven_set_tuning("prefill_waves"): 0 = by shape, 4 or 6 = waves per workgroup where the shape allows both
+}
 
 extern "C" int raven_prefill_attention(const void* q, void* y, const raven_kv_cache* cache, int32_t slot, int32_t B, int32_t S,
                                        int32_t pos0, const int32_t* pos_dev, int32_t n_heads, int32_t head_dim, int32_t dtype,
@@ -426,12 +435,17 @@ extern "C" int raven_prefill_attention(const void* q, void* y, const raven_kv_ca
     // launches keep 64 rows per workgroup so that there are more workgroups than compute units.
     const int64_t wgs128 = (int64_t)((S + 127) / 128) * n_heads * B;
     const int rg = wgs128 >= 512 ? 2 : 1;
-    const int rows = 64 * rg;
+    // head_dim 96, long launches: six waves (192 query rows) per workgroup.  Two such workgroups fit a CU's LDS, which
+    // puts three waves on every SIMD instead of two, and each staged K / V tile serves half as many rows again.
+    const bool six = head_dim == 96 && rg == 2 && g_prefill_waves != 4 &&
+                     (g_prefill_waves == 6 || (int64_t)((S + 191) / 192) * n_heads * B >= 512);
+    const int rows = six ? 192 : 64 * rg;
     const dim3 grid((S + rows - 1) / rows, n_heads, B);
 #define RAVEN_PREFILL(HD)                                                                  \
     if (rg == 2) attention_prefill_kernel<HD, 2><<<grid, dim3(256), 0, s>>>(a);            \
     else attention_prefill_kernel<HD, 1><<<grid, dim3(256), 0, s>>>(a)
-    if (head_dim == 64) { RAVEN_PREFILL(64); }
+    if (six) attention_prefill_kernel<96, 2, false, 6><<<grid, dim3(384), 0, s>>>(a);
+    else if (head_dim == 64) { RAVEN_PREFILL(64); }
     else if (head_dim == 96) { RAVEN_PREFILL(96); }
     else { RAVEN_PREFILL(128); }
 #undef RAVEN_PREFILL
