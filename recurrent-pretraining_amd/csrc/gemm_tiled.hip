@@ -61,10 +61,10 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 // Epilogue of both kernels.  A lane holds, for token row m = .. + l32, output columns 8 j + 4 hi + (0 .. 3) of each
 // 32-row A tile (SwiGLU: gate columns in registers 0 .. 7, the matching up columns in 8 .. 15).
-template <bool SWIGLU, int TM, int TN>
+template <bool SWIGLU, int TM, int TN, int WM = 2, int WN = 4>
 __device__ __forceinline__ void store_tiles(const TiledArgs& a, const f32x16 (&acc)[TN][TM], int tile_m, int tile_n, int wm, int wn,
                                             int l32, int hi) {
-    constexpr int BM = 2 * TM * 32, BN = 4 * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
         const int m = tile_m * BM + (wm * TM + tm) * 32 + l32;
@@ -118,13 +118,13 @@ __device__ __forceinline__ void store_tiles(const TiledArgs& a, const f32x16 (&a
 // tile rows, 16 bytes per lane: full 128-byte lines instead of 32 pieces of 16 bytes.  The residual is fetched the same
 // way, before the tile is laid down, so that its latency hides behind the transposition.  16-byte unit u of tile row r
 // sits at position u ^ (r mod units per row): the 32 rows a store instruction spreads over then fall on different banks.
-template <bool SWIGLU, int TM, int TN>
+template <bool SWIGLU, int TM, int TN, int WM = 2, int WN = 4>
 __device__ __forceinline__ void store_tiles_lds(const TiledArgs& a, const f32x16 (&acc)[TN][TM], int tile_m, int tile_n, int wave, int lane,
                                                 unsigned lds_base) {
-    constexpr int BM = 2 * TM * 32, BN = 4 * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
     constexpr int RB = BN_OUT * 2, U = RB / 16;      // bytes and 16-byte units per tile row
-    constexpr int ITERS = BM * U / 512;              // 16-byte units per lane
-    const int wn = wave & 3, wm = wave >> 2, l32 = lane & 31, hi = lane >> 5;
+    constexpr int ITERS = BM * U / (64 * WM * WN);    // 16-byte units per lane
+    const int wn = wave % WN, wm = wave / WN, l32 = lane & 31, hi = lane >> 5;
     bf16* const y = static_cast<bf16*>(a.y);
     int64_t goff[ITERS];                             // element offset of this lane's unit in y / residual, -1: outside
     u32x4 res[ITERS];
@@ -187,13 +187,14 @@ __device__ __forceinline__ void store_tiles_lds(const TiledArgs& a, const f32x16
 
 __device__ __align__(16) unsigned int g_zero_piece[4];  // what a 16-byte piece past the end of K is loaded from
 
-template <bool SWIGLU, int TM, int TN>
-__global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
-    constexpr int BM = 2 * TM * 32, BN = 4 * TN * 32;
+template <bool SWIGLU, int TM, int TN, int WM = 2, int WN = 4>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(TiledArgs a) {
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    constexpr int NWAVES = WM * WN;
     constexpr int ROWS = BN + BM;              // LDS rows of a stage: the W tile, then the X tile
     constexpr int STAGE_BYTES = ROWS * 128;
-    constexpr int LPW = ROWS / 8 / 8;          // 16-byte pieces per lane and step: piece p of a wave = 8 rows x 128 bytes
-    static_assert(ROWS % 256 == 0 && (BN / 8) % LPW == 0, "a wave loads rows of one operand only, the same number under every k-slice");
+    constexpr int LPW = ROWS / 8 / NWAVES;     // 16-byte pieces per lane and step: piece p of a wave = 8 rows x 128 bytes
+    static_assert(ROWS % (32 * NWAVES) == 0 && (BN / 8) % LPW == 0, "a wave loads rows of one operand only, the same number under every k-slice");
     constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
     constexpr int NM = TN * TM;                // MFMAs per k-slice
     constexpr int PPS = LPW / 4;               // pieces handled under the products of one k-slice
@@ -214,7 +215,7 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int wn = wave & 3, wm = wave >> 2;
+    const int wn = wave % WN, wm = wave / WN;
     const int K = a.K0 + a.K1;
     const int nk = (K + 63) >> 6;
 
@@ -361,20 +362,20 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(TiledArgs a) {
             move_under(it, k + 2, src3, ic0{});
         });
     }
-    if (a.out_f32) store_tiles<SWIGLU, TM, TN>(a, acc, tile_m, tile_n, wm, wn, l32, hi);
-    else store_tiles_lds<SWIGLU, TM, TN>(a, acc, tile_m, tile_n, wave, lane, lds_base);
+    if (a.out_f32) store_tiles<SWIGLU, TM, TN, WM, WN>(a, acc, tile_m, tile_n, wm, wn, l32, hi);
+    else store_tiles_lds<SWIGLU, TM, TN, WM, WN>(a, acc, tile_m, tile_n, wave, lane, lds_base);
 }
 
 int g_tiled_min_rows = 33;  // raven_set_tuning("gemm_tiled_min_rows"): fewest rows that take this kernel
 int g_tiled_variant = 0;    // raven_set_tuning("gemm_tiled_variant"): 0 = by shape, 1 = 256 x 256 tiles, 2 = 128 x 128 tiles
 
-template <bool SWIGLU, int TM, int TN>
+template <bool SWIGLU, int TM, int TN, int WM = 2, int WN = 4>
 static int launch_tiled(TiledArgs a, hipStream_t s) {
-    constexpr int BM = 2 * TM * 32, BN = 4 * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
     constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<SWIGLU, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<SWIGLU, TM, TN, WM, WN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) {
             raven_host::set_error("gemm (tiled): hipFuncSetAttribute failed: %s", hipGetErrorString(e));
             return (int)e;
@@ -386,7 +387,7 @@ static int launch_tiled(TiledArgs a, hipStream_t s) {
     const int64_t n_tiles = (int64_t)a.tiles_m * a.tiles_n;
     RAVEN_REQUIRE(n_tiles < (1 << 28), "gemm (tiled): too many tiles (M=%d N=%d)", a.M, a.N);
     const unsigned grid = (unsigned)((n_tiles + 7) / 8 * 8);
-    gemm_tiled_kernel<SWIGLU, TM, TN><<<dim3(grid), dim3(512), lds, s>>>(a);
+    gemm_tiled_kernel<SWIGLU, TM, TN, WM, WN><<<dim3(grid), dim3(64 * WM * WN), lds, s>>>(a);
     return raven_host::check_launch("gemm (tiled MFMA)");
 }
 
