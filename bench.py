@@ -550,9 +550,10 @@ def main():
     print(json.dumps(line))
 
 
-# HBM bytes per launch of the bs=1 mlp.fc kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy: a
-# profiler figure, so a constant here, with the file that holds the readings
-FC_BS1_TRAFFIC = {"bytes": 386061876, "source": "profiles/mlp_fc_gemv_bs1_hbm_traffic.txt"}
+# HBM bytes per launch of the mlp.fc kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy: profiler
+# figures, so constants here, with the file that holds the readings
+FC_TRAFFIC = {1: 386113760, 32: 385933770}
+FC_TRAFFIC_SOURCE = "profiles/mlp_fc_decode_hbm_traffic.txt"
 
 
 def decode_record(pkg, model, B, prompt_len, steps, warmup, r, use_graph):
@@ -637,8 +638,7 @@ def decode_record(pkg, model, B, prompt_len, steps, warmup, r, use_graph):
         "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": round(fc_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(fc_gbs / HBM_PEAK_GBS, 4),
                      "bytes_per_launch": int(fc_bytes), "avg_us": round(fc_ms * 1e3, 2),
-                     "traffic": FC_BS1_TRAFFIC["bytes"] if B == 1 else None,
-                     "traffic_source": FC_BS1_TRAFFIC["source"] if B == 1 else None},
+                     "traffic": FC_TRAFFIC.get(B), "traffic_source": FC_TRAFFIC_SOURCE if B in FC_TRAFFIC else None},
         "core_iteration": {"T": T, "batch": B, "bytes": int(it_bytes), "ms_eager": round(iter_eager_ms, 4),
                            "ms_graph": round(iter_graph_ms, 4), "achieved_GBs": round(it_bytes / (iter_ms * 1e-3) / 1e9, 1),
                            "frac": round(it_bytes / (iter_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},

@@ -525,18 +525,20 @@ def test_forward_with_adaptive_compute_token_by_token(pkg, small242):
     check(got, want, torch.float32, "kl exits, token by token")
 
 
-@pytest.mark.parametrize("B,draft_steps,L,vt", [(1, 1, 3, 1), (1, 2, 4, 1), (2, 4, 3, 1), (1, 4, 3, 1), (1, 2, 3, 0.5)])
-def test_generate_speculative_matches_oracle(pkg, small242, B, draft_steps, L, vt):
+@pytest.mark.parametrize("B,draft_steps,L,vt,in_step", [(1, 1, 3, 1, True), (1, 2, 4, 1, True), (2, 4, 3, 1, True), (1, 4, 3, 1, True),
+                                                        (1, 2, 3, 0.5, True), (2, 1, 3, 1, False), (2, 2, 3, 1, False)])
+def test_generate_speculative_matches_oracle(pkg, small242, B, draft_steps, L, vt, in_step):
     """Self-speculative decoding: drafts with few recurrences, rollback, one verifying chunk with all of them.
     Same sequences and the same accepted counts per round as the oracle's restatement of the loop; for one
     sequence with zero initial states it also equals plain greedy decoding (what speculation must preserve).
-    Batches are covered where all sequences accept the same number of tokens: once they differ, the reference feeds
-    RoPE positions that no longer equal the cache positions, which this package's forward refuses."""
+    Batches: in step (all sequences accept the same number of tokens), and out of step -- the sequences of the last
+    two cases accept 3 and 1 tokens in the first round; the reference then goes on with RoPE positions that differ
+    from the cache positions (RMM:1860-1900), and so does forward() here."""
     s, w, model = small242
     g = torch.Generator().manual_seed(40 + B)
     ids = torch.randint(0, s.vocab_size, (B, 5), generator=g)
     sf = lambda c, sh: O.initialize_state(torch.empty(sh), s, 1.0, torch.Generator().manual_seed(500 + c))
-    if B > 1:   # zero states and a draft as deep as the verifier: every token is accepted, the batch stays in step
+    if B > 1 and in_step:   # zero states and a draft as deep as the verifier: every token is accepted, the batch stays in step
         sf = lambda c, sh: torch.zeros(sh)
     rec = {}
     want = O.generate_speculative(w, s, ids, 9, draft_steps=draft_steps, lookahead_for_draft=L, num_steps=4,
@@ -546,6 +548,8 @@ def test_generate_speculative_matches_oracle(pkg, small242, B, draft_steps, L, v
                          input_states_fn=sf, stop_tokens=set(), pad_id=s.vocab_size - 1)
     assert out.scores["accepted_tokens"] == rec["accepted"], (out.scores["accepted_tokens"], rec["accepted"])
     assert torch.equal(out.sequences.cpu(), want)
+    if not in_step:
+        assert any(len(set(a)) > 1 for a in rec["accepted"])
     assert out.past_key_values.get_seq_length() == rec["cache"].get_seq_length()
     if B == 1:
         plain = model.generate_minimal(ids.cuda(), pkg.GenerationSettings(max_new_tokens=9), num_steps=4, init_scale=0.0,
