@@ -136,6 +136,27 @@ def test_prefill_attention_config4(pkg):
             check(y.view(B, S, H)[b, r], want, dt, f"row {r} of sequence {b}")
 
 
+def test_prefill_attention_wave_variants_agree(pkg, tuned):
+    """head_dim 96 has two workgroup shapes (four waves = 128 query rows, six waves = 192): a row's arithmetic is the same
+    in both, so the outputs must be the same bits -- with a chunk length that is no multiple of either, behind cached
+    positions, and at the oracle's values on sampled rows."""
+    dt, B, S, T0 = torch.bfloat16, 2, 1000, 24
+    q = _gpu_randn((B * S, H), 61)
+    k = _gpu_randn((1, B, NH, T0 + S, HD), 62)
+    v = _gpu_randn((1, B, NH, T0 + S, HD), 63)
+    cache = pkg.hip.make_cache(k, v)
+    outs = {}
+    for waves in (4, 6):
+        tuned(prefill_waves=waves)
+        outs[waves] = pkg.hip.prefill_attention(q, cache, 0, B, S, T0, NH, HD)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[4], outs[6])
+    for b, r in ((0, 0), (0, 191), (0, 192), (1, 575), (1, 999)):
+        qr = q.view(B, S, H)[b, r].view(1, NH, 1, HD)
+        want = O.sdpa(qr.cpu(), k[0, b, :, :T0 + r + 1].cpu()[None], v[0, b, :, :T0 + r + 1].cpu()[None]).view(H)
+        check(outs[6].view(B, S, H)[b, r], want, dt, f"row {r} of sequence {b}")
+
+
 # ----------------------------------------------------------------------------- one SandwichBlock at M = 16384
 def test_sandwich_block_config4_rows(pkg):
     """raven_sandwich_block on 4 x 4096 rows at the 3.5b dims (tiled products, MFMA chunk attention, fused norms) against
