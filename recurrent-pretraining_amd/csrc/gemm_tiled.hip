@@ -6,24 +6,32 @@
 //
 // Shape of the kernel (gfx950):
 //   * a workgroup of 8 waves (2 along the token rows x 4 along the weight rows, two waves per SIMD) owns a BN x BM tile
-//     of Y^T (256 weight rows x 256 token rows in the main variant); a wave owns TN x TM MFMA tiles of 32 x 32
-//     (v_mfma_f32_32x32x16_bf16, W rows as the A operand, X rows as B, so that a lane ends up with 4 neighbouring output
-//     columns of one token row);
+//     of Y^T (256 weight rows x 256 token rows in the main variant); a wave owns 2 TN x 2 TM MFMA tiles of 16 x 16
+//     (v_mfma_f32_16x16x32_bf16, W rows as the A operand, X rows as B, so that a lane ends up with 4 neighbouring output
+//     columns of one token row).  The 16 x 16 x 32 instruction has the same rate per product as 32 x 32 x 16 and needs
+//     the same LDS traffic here; measured, it runs the main variant 1 % to 5 % faster at the model's shapes;
 //   * K advances in steps of 64 through two LDS stages of BN + BM rows of 128 bytes.  The 16-byte pieces of a row are
 //     kept at position piece ^ ((row >> 1) & 7), so that the 16 lanes of a quarter wave, which read the same piece of 16
 //     neighbouring rows, hit all 64 banks;
 //   * operands travel global -> registers -> LDS: 8 lanes fetch one whole 128-byte row step (the L1 address path
 //     serves full lines at twice the rate of half lines), a wave instruction 8 rows.  Every lane keeps one step of its
 //     pieces in registers; a piece is written to LDS one step after it was requested and its registers are reloaded at
-//     once, two pieces under the products of each k-slice, so that loads flow evenly and each has a whole step to land;
-//   * a step is four k-slices of 16; fragments of the next slice are read from LDS under the products of this one.  One
-//     workgroup barrier per step, between the products of slices 2 and 3;
-//   * the K loop is one basic block of plain loads, stores and MFMAs with the scheduler pinned between them: the
-//     compiler then counts the outstanding loads exactly and waits for one piece at a time;
+//     once, two pieces under the products of each quarter step, so that loads flow evenly and each has a whole step to land;
+//   * a step is two k-slices of 32 and a slice two quarter steps, each all weight tiles of the wave against half of its
+//     token tiles.  A token fragment is replaced in place, as soon as its products are issued, by the one the next
+//     quarter needs; the weight fragments of the next slice go into a second register set.  One workgroup barrier per
+//     step, in front of the last quarter;
+//   * a loop over K steps is one basic block of plain loads, stores and MFMAs with the scheduler pinned between them:
+//     the compiler then counts the outstanding loads exactly and waits for one piece at a time.  Besides the MFMAs it
+//     holds little vector arithmetic (one 64-bit add per piece, six address updates per step): steps whose 64 columns
+//     lie in one segment and below K take their pieces from a scalar base, and the LDS addresses that alternate
+//     between the stages live in registers.  Steps near a segment boundary or the end of K run in loops of their own
+//     with a per-lane source; every lambda of the loops is forced inline, or the compiler keeps one shared copy with
+//     the accumulators in memory;
 //   * workgroups are numbered so that the 32 that run together on one XCD (ids congruent modulo 8) cover 8 x 4
 //     neighbouring tiles and find each other's panels in that XCD's L2;
-//   * SwiGLU: a 32-row A tile holds 16 gate rows and the 16 matching up rows, so gate and up of one output element sit
-//     in the same lane, 8 accumulator registers apart.
+//   * SwiGLU: 32 weight rows of the tile are 16 gate rows and the 16 matching up rows, so gate and up of one output
+//     element sit in the same lane, in neighbouring accumulator tiles.
 // M, N and the last tile: rows past the end are clamped on the load side and not stored.  K0 and K1 are multiples of 8
 // (pieces past K come from a zero page); two segments share one row pitch (K1 == K0).
 
@@ -59,72 +67,67 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
 }
 
-// Epilogue of both kernels.  A lane holds, for token row m = .. + l32, output columns 8 j + 4 hi + (0 .. 3) of each
-// 32-row A tile (SwiGLU: gate columns in registers 0 .. 7, the matching up columns in 8 .. 15).
+// Epilogue of both kernels.  Accumulator tile [ta][tb] (16 weight rows x 16 token rows) leaves a lane with token row
+// 16 tb + l16 and output columns 16 ta + 4 q4 + (0 .. 3); under SwiGLU tile 2 t holds gate columns and 2 t + 1 the
+// matching up columns.
 template <bool SWIGLU, int TM, int TN, int WM = 2, int WN = 4>
-__device__ __forceinline__ void store_tiles(const TiledArgs& a, const f32x16 (&acc)[TN][TM], int tile_m, int tile_n, int wm, int wn,
-                                            int l32, int hi) {
+__device__ __forceinline__ void store_tiles(const TiledArgs& a, const f32x4 (&acc)[2 * TN][2 * TM], int tile_m, int tile_n, int wm, int wn,
+                                            int l16, int q4) {
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
+    constexpr int NA = 2 * TN, NB = 2 * TM, NT = SWIGLU ? TN : NA;
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm) {
-        const int m = tile_m * BM + (wm * TM + tm) * 32 + l32;
+    for (int tb = 0; tb < NB; ++tb) {
+        const int m = tile_m * BM + (wm * NB + tb) * 16 + l16;
         if (m >= a.M) continue;
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn) {
-            const int t32 = wn * TN + tn;
+        for (int t = 0; t < NT; ++t) {
+            const int n = tile_n * BN_OUT + (wn * NT + t) * 16 + 4 * q4;
+            if (n >= a.N) continue;
             if (SWIGLU) {
+                bf16 o[4];
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int n = tile_n * BN_OUT + t32 * 16 + 8 * j + 4 * hi;
-                    if (n >= a.N) continue;
+                for (int i = 0; i < 4; ++i) {
+                    const float g = round_to<bf16>(acc[2 * t][tb][i]), u = round_to<bf16>(acc[2 * t + 1][tb][i]);
+                    o[i] = from_f32<bf16>(round_to<bf16>(silu_f32(g)) * u);
+                }
+                *reinterpret_cast<u32x2*>(static_cast<bf16*>(a.y) + (int64_t)m * a.N + n) = *reinterpret_cast<const u32x2*>(o);
+            } else {
+                float r[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) r[i] = round_to<bf16>(acc[t][tb][i]);
+                if (a.residual) {
+                    bf16 res[4];
+                    *reinterpret_cast<u32x2*>(res) = *reinterpret_cast<const u32x2*>(a.residual + (int64_t)m * a.N + n);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) r[i] = round_to<bf16>(r[i] + to_f32(res[i]));
+                }
+                if (a.out_f32) {
+                    *reinterpret_cast<f32x4*>(static_cast<float*>(a.y) + (int64_t)m * a.N + n) = f32x4{r[0], r[1], r[2], r[3]};
+                } else {
                     bf16 o[4];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float g = round_to<bf16>(acc[tn][tm][4 * j + i]), u = round_to<bf16>(acc[tn][tm][8 + 4 * j + i]);
-                        o[i] = from_f32<bf16>(round_to<bf16>(silu_f32(g)) * u);
-                    }
+                    for (int i = 0; i < 4; ++i) o[i] = from_f32<bf16>(r[i]);
                     *reinterpret_cast<u32x2*>(static_cast<bf16*>(a.y) + (int64_t)m * a.N + n) = *reinterpret_cast<const u32x2*>(o);
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int n = tile_n * BN + t32 * 32 + 8 * j + 4 * hi;
-                    if (n >= a.N) continue;
-                    float r[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) r[i] = round_to<bf16>(acc[tn][tm][4 * j + i]);
-                    if (a.residual) {
-                        bf16 res[4];
-                        *reinterpret_cast<u32x2*>(res) = *reinterpret_cast<const u32x2*>(a.residual + (int64_t)m * a.N + n);
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) r[i] = round_to<bf16>(r[i] + to_f32(res[i]));
-                    }
-                    if (a.out_f32) {
-                        *reinterpret_cast<f32x4*>(static_cast<float*>(a.y) + (int64_t)m * a.N + n) = f32x4{r[0], r[1], r[2], r[3]};
-                    } else {
-                        bf16 o[4];
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) o[i] = from_f32<bf16>(r[i]);
-                        *reinterpret_cast<u32x2*>(static_cast<bf16*>(a.y) + (int64_t)m * a.N + n) = *reinterpret_cast<const u32x2*>(o);
-                    }
                 }
             }
         }
     }
 }
 
-// Epilogue through LDS for the bf16 outputs: the accumulators (a lane: 4 columns of 32 different token rows per store)
-// are laid down as the output tile, rows of BN_OUT columns, and read back so that a wave instruction stores two whole
-// tile rows, 16 bytes per lane: full 128-byte lines instead of 32 pieces of 16 bytes.  The residual is fetched the same
-// way, before the tile is laid down, so that its latency hides behind the transposition.  16-byte unit u of tile row r
-// sits at position u ^ (r mod units per row): the 32 rows a store instruction spreads over then fall on different banks.
+// Epilogue through LDS for the bf16 outputs: the accumulators (a lane: 4 columns of one token row per store, a wave
+// instruction 16 token rows) are laid down as the output tile, rows of BN_OUT columns, and read back so that a wave
+// instruction stores two whole tile rows, 16 bytes per lane: full 128-byte lines instead of pieces of 8 bytes.  The
+// residual is fetched the same way, before the tile is laid down, so that its latency hides behind the transposition.
+// 16-byte unit u of tile row r sits at position u ^ (r mod units per row): the 16 rows a store instruction spreads over
+// then fall on different banks.
 template <bool SWIGLU, int TM, int TN, int WM = 2, int WN = 4>
-__device__ __forceinline__ void store_tiles_lds(const TiledArgs& a, const f32x16 (&acc)[TN][TM], int tile_m, int tile_n, int wave, int lane,
-                                                unsigned lds_base) {
+__device__ __forceinline__ void store_tiles_lds(const TiledArgs& a, const f32x4 (&acc)[2 * TN][2 * TM], int tile_m, int tile_n, int wave,
+                                                int lane, unsigned lds_base) {
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
+    constexpr int NA = 2 * TN, NB = 2 * TM, NT = SWIGLU ? TN : NA;
     constexpr int RB = BN_OUT * 2, U = RB / 16;      // bytes and 16-byte units per tile row
     constexpr int ITERS = BM * U / (64 * WM * WN);    // 16-byte units per lane
-    const int wn = wave % WN, wm = wave / WN, l32 = lane & 31, hi = lane >> 5;
+    const int wn = wave % WN, wm = wave / WN, l16 = lane & 15, q4 = lane >> 4;
     bf16* const y = static_cast<bf16*>(a.y);
     int64_t goff[ITERS];                             // element offset of this lane's unit in y / residual, -1: outside
     u32x4 res[ITERS];
@@ -141,28 +144,24 @@ __device__ __forceinline__ void store_tiles_lds(const TiledArgs& a, const f32x16
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm) {
-        const int row = (wm * TM + tm) * 32 + l32;
-        const unsigned row_addr = lds_base + row * RB + hi * 8;
+    for (int tb = 0; tb < NB; ++tb) {
+        const int row = (wm * NB + tb) * 16 + l16;
+        const unsigned row_addr = lds_base + row * RB + (q4 & 1) * 8;
         const int sw = row & (U - 1);
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn) {
-            const int t32 = wn * TN + tn;
+        for (int t = 0; t < NT; ++t) {
+            bf16 o[4];
 #pragma unroll
-            for (int j = 0; j < (SWIGLU ? 2 : 4); ++j) {
-                bf16 o[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    if (SWIGLU) {
-                        const float g = round_to<bf16>(acc[tn][tm][4 * j + i]), u = round_to<bf16>(acc[tn][tm][8 + 4 * j + i]);
-                        o[i] = from_f32<bf16>(round_to<bf16>(silu_f32(g)) * u);
-                    } else {
-                        o[i] = from_f32<bf16>(acc[tn][tm][4 * j + i]);
-                    }
+            for (int i = 0; i < 4; ++i) {
+                if (SWIGLU) {
+                    const float g = round_to<bf16>(acc[2 * t][tb][i]), u = round_to<bf16>(acc[2 * t + 1][tb][i]);
+                    o[i] = from_f32<bf16>(round_to<bf16>(silu_f32(g)) * u);
+                } else {
+                    o[i] = from_f32<bf16>(acc[t][tb][i]);
                 }
-                const int unit = t32 * (SWIGLU ? 2 : 4) + j;
-                *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(row_addr + ((unit ^ sw) * 16)) = *reinterpret_cast<const u32x2*>(o);
             }
+            const int unit = (wn * NT + t) * 2 + (q4 >> 1);
+            *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(row_addr + ((unit ^ sw) * 16)) = *reinterpret_cast<const u32x2*>(o);
         }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -196,8 +195,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(TiledArgs a) {
     constexpr int LPW = ROWS / 8 / NWAVES;     // 16-byte pieces per lane and step: piece p of a wave = 8 rows x 128 bytes
     static_assert(ROWS % (32 * NWAVES) == 0 && (BN / 8) % LPW == 0, "a wave loads rows of one operand only, the same number under every k-slice");
     constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
-    constexpr int NM = TN * TM;                // MFMAs per k-slice
-    constexpr int PPS = LPW / 4;               // pieces handled under the products of one k-slice
+    constexpr int NA = 2 * TN, NB = 2 * TM;   // 16-row MFMA tiles of a wave along the weight rows / the token rows
+    constexpr int HB = NB / 2;                 // token tiles of a quarter step
+    static_assert(NA == HB, "one weight fragment is fetched behind each group of a quarter step");
+    constexpr int NM = NA * HB;                // MFMAs per quarter step
+    constexpr int PPS = LPW / 4;               // pieces handled under the products of one quarter step
     extern __shared__ __align__(1024) unsigned char smem[];
 
     // ---- which tile -----------------------------------------------------------------------------------------------
@@ -249,120 +251,165 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(TiledArgs a) {
     const char* const seg1 = reinterpret_cast<const char*>(a.x1) - 2 * (int64_t)a.K0;  // column c >= K0 of the token rows
     const int k_split = loads_w ? K : a.K0;    // columns from here on come from the second segment
 
-    // Plain loads and stores, and no branch inside the K loop: the compiler then knows the order of all outstanding loads
-    // and waits, in front of the LDS write of a piece, for exactly that piece's load (issued one step earlier).
+    // Plain loads and stores inside a step: the compiler then knows the order of all outstanding loads and waits, in
+    // front of the LDS write of a piece, for exactly that piece's load (issued one step earlier).
     // Where this lane's 16 bytes of step kk come from: its segment's pointer (rebased so that the piece's offset is
     // goff[p] + 2 * 64 kk), or the zero page for columns past K -- which is every column of a step past the last one.
+    // A step whose 64 columns lie in one segment and below K has one source for the whole wave (WHOLE): a scalar base
+    // plus the lane's 32-bit offset, no vector arithmetic per piece.
     struct StepSrc {
         const char* base;
         bool past;  // this lane's column lies past K
     };
-    auto step_src = [&](int kk) {
+    auto step_src = [&](int kk) __attribute__((always_inline)) {
         const int col = (kk << 6) + col8;
         StepSrc s;
         s.past = col >= K;
         s.base = s.past ? zero : (col < k_split ? seg0 : seg1) + 2 * (kk << 6);
         return s;
     };
-    u32x4 stg[LPW];
-    auto load_piece = [&](const StepSrc& src, auto p_tag) {
-        constexpr int p = decltype(p_tag)::value;
-        stg[p] = *reinterpret_cast<const u32x4*>(src.base + (src.past ? 0u : goff[p]));
+    auto whole_step = [&](int kk) __attribute__((always_inline)) {  // wave-uniform
+        const int c0 = kk << 6;
+        return c0 + 64 <= k_split || (c0 >= k_split && c0 + 64 <= K);
     };
-    auto store_piece = [&](int kk, auto p_tag) {
+    auto whole_src = [&](int kk) __attribute__((always_inline)) {   // wave-uniform
+        const int c0 = kk << 6;
+        StepSrc s;
+        s.past = false;
+        s.base = (c0 < k_split ? seg0 : seg1) + 2 * c0;
+        return s;
+    };
+    u32x4 stg[LPW];
+    auto load_piece = [&](const StepSrc& src, auto p_tag, auto whole_tag) __attribute__((always_inline)) {
+        constexpr int p = decltype(p_tag)::value;
+        if constexpr (decltype(whole_tag)::value) stg[p] = *reinterpret_cast<const u32x4*>(src.base + goff[p]);
+        else stg[p] = *reinterpret_cast<const u32x4*>(src.base + (src.past ? 0u : goff[p]));
+    };
+    // LDS addresses that alternate between the two stages are kept in registers and advanced once per step
+    unsigned wr_cur[2] = {wr_addr[0] + STAGE_BYTES, wr_addr[1] + STAGE_BYTES};  // the first step of the loop writes stage 1
+    auto store_piece_at = [&](int kk, auto p_tag) __attribute__((always_inline)) {  // in front of the loops
         constexpr int p = decltype(p_tag)::value;
         *reinterpret_cast<lds_u32x4*>(wr_addr[p & 1] + (kk & 1) * STAGE_BYTES + p * 1024) = stg[p];
     };
-    // Piece p of step j moves on: into stage j & 1; the registers take the piece of step j + 1 (source: next).
-    auto move_piece = [&](int j, const StepSrc& next, auto p_tag) {
-        store_piece(j, p_tag);
-        load_piece(next, p_tag);
+    // Piece p moves on into the stage wr_cur points at; the registers take the piece of the step after (source: next).
+    auto move_piece = [&](const StepSrc& next, auto p_tag, auto whole_tag) __attribute__((always_inline)) {
+        constexpr int p = decltype(p_tag)::value;
+        *reinterpret_cast<lds_u32x4*>(wr_cur[p & 1] + p * 1024) = stg[p];
+        load_piece(next, p_tag, whole_tag);
     };
 
     // ---- LDS -> registers -------------------------------------------------------------------------------------------
-    const int l32 = lane & 31, hi = lane >> 5;
-    const int swz = (l32 >> 1) & 7;
-    const unsigned a_row = lds_base + (wn * TN * 32 + l32) * 128;
-    const unsigned b_row = lds_base + (BN + wm * TM * 32 + l32) * 128;
-    const unsigned pos0 = (hi ^ swz) * 16;     // position of k-slice ks: pos0 ^ (32 ks)
+    // v_mfma_f32_16x16x32_bf16: lane l supplies row l & 15 of its tile, columns 8 (l >> 4) ..+7 of a 32-column k-slice.
+    const int l16 = lane & 15, q4 = lane >> 4;
+    const int swz = (l16 >> 1) & 7;
+    const unsigned a_row = lds_base + (wn * TN * 32 + l16) * 128;
+    const unsigned b_row = lds_base + (BN + wm * TM * 32 + l16) * 128;
+    const unsigned pos0 = (q4 ^ swz) * 16;     // position of k-slice s: pos0 ^ (64 s)
 
-    f32x16 acc[TN][TM];
+    f32x4 acc[NA][NB];
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn)
+    for (int ta = 0; ta < NA; ++ta)
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[tn][tm][e] = 0.f;
+        for (int tb = 0; tb < NB; ++tb) acc[ta][tb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    u32x4 fa[2][TN], fb[2][TM];
-    auto read_frags = [&](auto ks_tag, int buf) {  // k-slice ks of stage buf into fragment set ks & 1
-        constexpr int ks = decltype(ks_tag)::value;
-        const unsigned off = buf * STAGE_BYTES + (pos0 ^ (32 * ks));
-#pragma unroll
-        for (int t = 0; t < TN; ++t) fa[ks & 1][t] = *reinterpret_cast<const lds_u32x4*>(a_row + off + t * 4096);
-#pragma unroll
-        for (int t = 0; t < TM; ++t) fb[ks & 1][t] = *reinterpret_cast<const lds_u32x4*>(b_row + off + t * 4096);
+    // A step is two k-slices of 32, a slice two quarter steps: the NA weight tiles against one half of the token tiles
+    // (HB of them), token tile by token tile.  The weight fragments of a slice live through both its quarters and
+    // have a second register set, filled under the slice before; a token fragment is replaced by the one the next
+    // quarter needs in the same place as soon as its NA products are issued -- 3/4 of a quarter ahead of its use.
+    u32x4 fa[2][NA], fb[HB];
+    unsigned ra[2] = {a_row + pos0, a_row + (pos0 ^ 64)}, rb[2] = {b_row + pos0, b_row + (pos0 ^ 64)};  // slice 0 / 1, stage 0
+    auto read_a = [&](auto set_tag, auto t_tag) __attribute__((always_inline)) {  // weight tile t of slice `set` into fragment set `set`
+        constexpr int set = decltype(set_tag)::value, t = decltype(t_tag)::value;
+        fa[set][t] = *reinterpret_cast<const lds_u32x4*>(ra[set] + t * 2048);
     };
-    // the NM products of one k-slice; after(i) is called behind product i
-    auto products = [&](int set, auto&& after) {
+    auto read_b = [&](auto slice_tag, auto half_tag, auto j_tag) __attribute__((always_inline)) {
+        constexpr int slice = decltype(slice_tag)::value, half = decltype(half_tag)::value, j = decltype(j_tag)::value;
+        fb[j] = *reinterpret_cast<const lds_u32x4*>(rb[slice] + (half * HB + j) * 2048);
+    };
+    // Quarter q of a step: slice q >> 1, token half q & 1.  Behind the first NA products of a second half the weight
+    // fragments of the next slice are requested (for q = 3: of the next step; ra[0] and rb[0] point there by then).
+    auto quarter = [&](auto q_tag, auto&& extra) __attribute__((always_inline)) {
+        constexpr int q = decltype(q_tag)::value, s = q >> 1, h = q & 1;
+        constexpr int sn = ((q + 1) & 3) >> 1, hn = (q + 1) & 1;
         static_for<NM>([&](auto it) {
-            constexpr int i = decltype(it)::value, tn = i / TM, tm = i % TM;
-            acc[tn][tm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[set][tn]),
-                                                                      __builtin_bit_cast(bf16x8, fb[set][tm]), acc[tn][tm], 0, 0, 0);
+            constexpr int i = decltype(it)::value, j = i / NA, ta = i % NA;
+            acc[ta][h * HB + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, fa[s][ta]),
+                                                                           __builtin_bit_cast(bf16x8, fb[j]), acc[ta][h * HB + j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            after(it);
+            if (h == 1 && i < NA) read_a(std::integral_constant<int, s ^ 1>{}, std::integral_constant<int, (i < NA ? i : 0)>{});
+            if (ta == NA - 1) read_b(std::integral_constant<int, sn>{}, std::integral_constant<int, hn>{}, std::integral_constant<int, j>{});
+            extra(it);
             __builtin_amdgcn_sched_barrier(0);
         });
     };
-    // pieces FIRST .. FIRST + PPS - 1 of step j, behind products 1, 1 + NM / PPS, ... of a slice
-    auto move_under = [&](auto it, int j, const StepSrc& next, auto first_tag) {
+    // pieces FIRST .. FIRST + PPS - 1, spread over the products of a quarter
+    auto move_under = [&](auto it, const StepSrc& next, auto first_tag, auto whole_tag) __attribute__((always_inline)) {
         constexpr int i = decltype(it)::value, FIRST = decltype(first_tag)::value;
-        static_for<PPS>([&](auto q) {
-            constexpr int slot = 1 + decltype(q)::value * (NM / PPS) < NM - 1 ? 1 + decltype(q)::value * (NM / PPS) : NM - 1;
-            if (slot == i) move_piece(j, next, std::integral_constant<int, FIRST + decltype(q)::value>{});
+        static_for<PPS>([&](auto qq) {
+            constexpr int want = NA + 1 + decltype(qq)::value * (NM / PPS);
+            constexpr int slot = want < NM - 1 ? want : NM - 1;
+            if (slot == i) move_piece(next, std::integral_constant<int, FIRST + decltype(qq)::value>{}, whole_tag);
         });
     };
     using ic0 = std::integral_constant<int, 0>;
 
     // ---- the K loop: two LDS stages and one set of staging registers, one barrier per step --------------------------
-    // Step k is multiplied out of stage k & 1 in four k-slices of 16.  The barrier of step k sits between the products of
-    // slices 2 and 3: in front of it every wave has all fragments of step k in registers and has written its pieces of
-    // step k + 1; behind it stage k & 1 is free for step k + 2 and stage (k + 1) & 1 may be read.  Every piece goes round
-    // once per step: under slice 3 of step k the pieces 0 .. PPS - 1 of step k + 2 are written and reloaded for step
-    // k + 3, under slices 0 .. 2 of the next step the others -- each load has a whole step to land and the loads flow
-    // evenly.
+    // Step k is multiplied out of stage k & 1 in four quarters.  The barrier of step k sits between quarters 2 and 3:
+    // in front of it every wave has requested all it needs of stage k & 1 and has written its pieces of step k + 1;
+    // behind it stage k & 1 is free for step k + 2 and stage (k + 1) & 1 may be read.  Every piece goes round once per
+    // step: under quarter 3 of step k the pieces 0 .. PPS - 1 of step k + 2 are written and reloaded for step k + 3,
+    // under quarters 0 .. 2 of the next step the others -- each load has a whole step to land and the loads flow evenly.
     {
         const StepSrc s0 = step_src(0), s1 = step_src(1), s2 = step_src(2);
-        static_for<LPW>([&](auto p) { load_piece(s0, p); });
-        static_for<LPW>([&](auto p) { move_piece(0, s1, p); });
-        static_for<PPS>([&](auto p) { move_piece(1, s2, p); });  // as under slice 3 of a step in front of the first
+        static_for<LPW>([&](auto p) { load_piece(s0, p, std::false_type{}); });
+        static_for<LPW>([&](auto p) { store_piece_at(0, p); load_piece(s1, p, std::false_type{}); });
+        static_for<PPS>([&](auto p) { store_piece_at(1, p); load_piece(s2, p, std::false_type{}); });  // as under quarter 3 of a step before
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    read_frags(ic0{}, 0);
-    for (int k = 0; k < nk; ++k) {
-        const int cur = k & 1;
-        const StepSrc src2 = step_src(k + 2), src3 = step_src(k + 3);
-        static_for<3>([&](auto ks_tag) {
-            constexpr int ks = decltype(ks_tag)::value;
-            products(ks & 1, [&](auto it) {
-                if (decltype(it)::value == 0) read_frags(std::integral_constant<int, ks + 1>{}, cur);
-                move_under(it, k + 1, src2, std::integral_constant<int, PPS * (ks + 1)>{});
-            });
+    static_for<NA>([&](auto t) { read_a(ic0{}, t); });
+    static_for<HB>([&](auto j) { read_b(ic0{}, ic0{}, j); });
+    // One step; src2 / src3: where steps k + 2 / k + 3 come from.  flip = +-STAGE_BYTES: from this step's stage to the other.
+    auto step = [&](const StepSrc& src2, const StepSrc& src3, int flip, auto whole_tag) __attribute__((always_inline)) {
+        static_for<3>([&](auto q_tag) {
+            constexpr int q = decltype(q_tag)::value;
+            quarter(q_tag, [&](auto it) { move_under(it, src2, std::integral_constant<int, PPS * (q + 1)>{}, whole_tag); });
         });
-        // every LDS write of step k + 1 and every read of step k has completed in front of the barrier
+        // every LDS write of step k + 1 and every read of stage k & 1 has completed in front of the barrier
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("" ::: "memory");
-        products(1, [&](auto it) {
-            if (decltype(it)::value == 0) read_frags(ic0{}, cur ^ 1);  // behind the last step: zeros, not used
-            move_under(it, k + 2, src3, ic0{});
-        });
-    }
-    if (a.out_f32) store_tiles<SWIGLU, TM, TN, WM, WN>(a, acc, tile_m, tile_n, wm, wn, l32, hi);
+        // from here on: fragments of the next step out of the other stage, pieces of step k + 2 into this one
+        ra[0] += flip; ra[1] += flip; rb[0] += flip; rb[1] += flip;
+        wr_cur[0] -= flip; wr_cur[1] -= flip;
+        // behind the last step the fragments requested here are zeros and not used
+        quarter(std::integral_constant<int, 3>{}, [&](auto it) { move_under(it, src3, ic0{}, whole_tag); });
+    };
+    // Runs of steps that take their pieces from whole steps alternate with runs that do not (around the boundary
+    // between two segments when it is not a multiple of 64, and at the end of K); each run is a loop of its own, so
+    // that a loop body stays one basic block.
+    auto whole_ok = [&](int k) __attribute__((always_inline)) { return whole_step(k + 2) && whole_step(k + 3); };
+    auto run = [&](int k, int k_end, auto whole_tag) __attribute__((always_inline)) {
+        for (; k < k_end; ++k) {
+            const int flip = (k & 1) ? -STAGE_BYTES : STAGE_BYTES;
+            if constexpr (decltype(whole_tag)::value) step(whole_src(k + 2), whole_src(k + 3), flip, whole_tag);
+            else step(step_src(k + 2), step_src(k + 3), flip, whole_tag);
+        }
+    };
+    int e1 = 0, e2, e3;
+    while (e1 < nk && whole_ok(e1)) ++e1;
+    e2 = e1;
+    while (e2 < nk && !whole_ok(e2)) ++e2;
+    e3 = e2;
+    while (e3 < nk && whole_ok(e3)) ++e3;
+    run(0, e1, std::true_type{});
+    run(e1, e2, std::false_type{});
+    run(e2, e3, std::true_type{});
+    run(e3, nk, std::false_type{});
+    if (a.out_f32) store_tiles<SWIGLU, TM, TN, WM, WN>(a, acc, tile_m, tile_n, wm, wn, l16, q4);
     else store_tiles_lds<SWIGLU, TM, TN, WM, WN>(a, acc, tile_m, tile_n, wave, lane, lds_base);
 }
 
