@@ -25,7 +25,7 @@ namespace raven {
 
 int set_gemv1_tuning(const char* key, int value);
 extern int g_linear_ks;
-extern int g_tiled_min_rows, g_tiled_variant;
+extern int g_tiled_min_rows, g_tiled_variant, g_tiled_split_tail;
 bool tiled_gemm_fits(int M, int N, int K0, int K1, int dtype);
 int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residual, void* y, int M, int N, int K0, int K1, int swiglu,
                int out_f32, hipStream_t s);
@@ -573,6 +573,7 @@ extern "C" int raven_set_tuning(const char* key, int32_t value) {
     else if (k == "linear_min_rows" && value >= 1) g_linear_min_rows = value;
     else if (k == "gemm_tiled_min_rows" && value >= 33) g_tiled_min_rows = value;
     else if (k == "gemm_tiled_variant" && value >= 0 && value <= 2) g_tiled_variant = value;
+    else if (k == "gemm_tiled_split_tail" && (value == 0 || value == 1)) g_tiled_split_tail = value;
     else RAVEN_REQUIRE(set_gemv1_tuning(key, value) == 0, "set_tuning: unknown key %s", key);
     return 0;
 }

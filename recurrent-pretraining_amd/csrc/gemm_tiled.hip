@@ -48,7 +48,8 @@ struct TiledArgs {
     const bf16* x1;        // [M, K1] or null
     const bf16* residual;  // [M, N] or null
     void* y;               // [M, N] bf16, or float when out_f32
-    int M, N, K0, K1;      // N = output columns (I for SwiGLU)
+    int M, N, K0, K1;      // N = output columns of this launch (I for SwiGLU)
+    int ldy;               // row pitch of y and residual in elements (>= N: a launch may cover a range of columns)
     int out_f32;
     int tiles_m, tiles_n;
 };
@@ -90,24 +91,24 @@ __device__ __forceinline__ void store_tiles(const TiledArgs& a, const f32x4 (&ac
                     const float g = round_to<bf16>(acc[2 * t][tb][i]), u = round_to<bf16>(acc[2 * t + 1][tb][i]);
                     o[i] = from_f32<bf16>(round_to<bf16>(silu_f32(g)) * u);
                 }
-                *reinterpret_cast<u32x2*>(static_cast<bf16*>(a.y) + (int64_t)m * a.N + n) = *reinterpret_cast<const u32x2*>(o);
+                *reinterpret_cast<u32x2*>(static_cast<bf16*>(a.y) + (int64_t)m * a.ldy + n) = *reinterpret_cast<const u32x2*>(o);
             } else {
                 float r[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) r[i] = round_to<bf16>(acc[t][tb][i]);
                 if (a.residual) {
                     bf16 res[4];
-                    *reinterpret_cast<u32x2*>(res) = *reinterpret_cast<const u32x2*>(a.residual + (int64_t)m * a.N + n);
+                    *reinterpret_cast<u32x2*>(res) = *reinterpret_cast<const u32x2*>(a.residual + (int64_t)m * a.ldy + n);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) r[i] = round_to<bf16>(r[i] + to_f32(res[i]));
                 }
                 if (a.out_f32) {
-                    *reinterpret_cast<f32x4*>(static_cast<float*>(a.y) + (int64_t)m * a.N + n) = f32x4{r[0], r[1], r[2], r[3]};
+                    *reinterpret_cast<f32x4*>(static_cast<float*>(a.y) + (int64_t)m * a.ldy + n) = f32x4{r[0], r[1], r[2], r[3]};
                 } else {
                     bf16 o[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) o[i] = from_f32<bf16>(r[i]);
-                    *reinterpret_cast<u32x2*>(static_cast<bf16*>(a.y) + (int64_t)m * a.N + n) = *reinterpret_cast<const u32x2*>(o);
+                    *reinterpret_cast<u32x2*>(static_cast<bf16*>(a.y) + (int64_t)m * a.ldy + n) = *reinterpret_cast<const u32x2*>(o);
                 }
             }
         }
@@ -135,7 +136,7 @@ __device__ __forceinline__ void store_tiles_lds(const TiledArgs& a, const f32x4 
     for (int it = 0; it < ITERS; ++it) {
         const int idx = (wave * ITERS + it) * 64 + lane;
         const int m = tile_m * BM + idx / U, n = tile_n * BN_OUT + (idx % U) * 8;
-        goff[it] = (m < a.M && n < a.N) ? (int64_t)m * a.N + n : -1;
+        goff[it] = (m < a.M && n < a.N) ? (int64_t)m * a.ldy + n : -1;
         res[it] = u32x4{0, 0, 0, 0};
         if (!SWIGLU && a.residual && goff[it] >= 0) res[it] = *reinterpret_cast<const u32x4*>(a.residual + goff[it]);
     }
@@ -415,6 +416,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(TiledArgs a) {
 
 int g_tiled_min_rows = 33;  // raven_set_tuning("gemm_tiled_min_rows"): fewest rows that take this kernel
 int g_tiled_variant = 0;    // raven_set_tuning("gemm_tiled_variant"): 0 = by shape, 1 = 256 x 256 tiles, 2 = 128 x 128 tiles
+int g_tiled_split_tail = 1; // raven_set_tuning("gemm_tiled_split_tail"): 0 = never hand the last round's tile columns to 128 x 128 tiles
 
 template <bool SWIGLU, int TM, int TN, int WM = 2, int WN = 4>
 static int launch_tiled(TiledArgs a, hipStream_t s) {
@@ -461,6 +463,7 @@ int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residu
     a.residual = static_cast<const bf16*>(residual);
     a.y = y;
     a.M = M; a.N = N; a.K0 = K0; a.K1 = x1 ? K1 : 0; a.out_f32 = out_f32;
+    a.ldy = N;
     // 256 x 256 tiles when they fill the chip at least once; 128 x 128 tiles otherwise
     const int bn_out = swiglu ? 128 : 256;
     const int64_t tiles_n = (N + bn_out - 1) / bn_out, tiles_m = (M + 255) / 256;
@@ -470,6 +473,22 @@ int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residu
         if (swiglu) return as_big ? launch_tiled<true, 4, 2>(t, s) : launch_tiled<true, 2, 1>(t, s);
         return as_big ? launch_tiled<false, 4, 2>(t, s) : launch_tiled<false, 2, 1>(t, s);
     };
+    // The last round of 256 x 256 tiles: when it would fill at most half of the 256 CUs and is whole tile columns, those
+    // columns are multiplied as 128 x 128 tiles instead -- four times as many workgroups, a quarter of the time each
+    // (5.25 rounds of work then take about 5.4 rounds instead of 6: the N = 5280 products of the model at 16384 rows).
+    const int64_t rest = big_tiles % 256;
+    if (big && g_tiled_variant == 0 && g_tiled_split_tail && !swiglu && big_tiles > 256 && rest > 0 && rest <= 128 && rest % tiles_m == 0) {
+        const int cols = (int)(rest / tiles_m);              // trailing tile columns
+        const int n_big = (int)(tiles_n - cols) * 256;       // output columns of the first launch
+        TiledArgs head = a, tail = a;
+        head.N = n_big;
+        tail.N = N - n_big;
+        tail.w = a.w + (int64_t)n_big * (K0 + a.K1);
+        tail.residual = a.residual ? a.residual + n_big : nullptr;
+        tail.y = out_f32 ? static_cast<void*>(static_cast<float*>(y) + n_big) : static_cast<void*>(static_cast<bf16*>(y) + n_big);
+        const int rc = launch(head, true);
+        return rc ? rc : launch(tail, false);
+    }
     return launch(a, big);
 }
 

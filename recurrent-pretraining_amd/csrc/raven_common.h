@@ -110,7 +110,9 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + __expf(-x)); }
+// x * sigmoid(x).  The reciprocal is the hardware's (1 ulp): its error vanishes in the bf16 rounding that follows and stays
+// inside the fp32 bar, and a true division costs five times the instructions in the SwiGLU epilogue of a 256 x 256 tile.
+__device__ __forceinline__ float silu_f32(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
 }  // namespace raven
 

@@ -112,6 +112,28 @@ def test_tiled_gemm_edges_against_oracle(pkg, tuned, variant, M, N, K):
     assert torch.equal(a, pkg.hip.linear(dev(x), dev(w)))
 
 
+@pytest.mark.parametrize("N", [16640, 16544])
+def test_tiled_gemm_last_round_as_small_tiles_changes_no_bit(pkg, tuned, N):
+    """4 x 65 tiles of 256 x 256: the 4 tiles of the last, nearly empty round (the last tile column, whole or 160 wide)
+    are multiplied as 128 x 128 tiles by a second launch over that column range.  Same bits as one launch, for every
+    epilogue that takes the split, and right against the fp32 product on sampled columns of both ranges."""
+    dt, M, K = torch.bfloat16, 1024, 192
+    x, x1 = _gpu_randn((M, K), 600), _gpu_randn((M, K), 601)
+    w, w2, res = _gpu_randn((N, K), 602, 0.05), _gpu_randn((N, 2 * K), 603, 0.05), _gpu_randn((M, N), 604)
+    calls = {"plain": lambda: pkg.hip.linear(x, w), "+ residual": lambda: pkg.hip.linear(x, w, residual=res),
+             "float": lambda: pkg.hip.linear(x, w, out_f32=True), "two operands": lambda: pkg.hip.linear(x, w2, x1=x1)}
+    for name, call in calls.items():
+        tuned(gemm_tiled_split_tail=1)
+        split = call()
+        tuned(gemm_tiled_split_tail=0)
+        whole = call()
+        assert torch.equal(split, whole), name
+    cols = torch.tensor([0, 255, 256, 8191, 16383, 16384, 16385, 16511, 16512, N - 1]).cuda()
+    tuned(gemm_tiled_split_tail=1)
+    want = (x.float() @ w[cols].float().T).to(dt).float() + res[:, cols].float()
+    check(pkg.hip.linear(x, w, residual=res)[:, cols], want.to(dt), dt, "sampled columns")
+
+
 # ----------------------------------------------------------------------------- attention at 4 x 4096
 def test_prefill_attention_config4(pkg):
     """raven_prefill_attention at B=4, S=4096, 55 heads of 96: sampled (sequence, head) pairs against the oracle's sdpa,
