@@ -403,7 +403,7 @@ def test_published_cache_sizes():
     assert 132 * 55 * 1024 * 96 * 2 * 2 / 2**20 == 2722.5
 
 
-def test_core_iteration_byte_count_matches_survey():
+def test_core_iteration_byte_count_at_the_3_5b_shape():
     s = O.RavenShape.nebel()
     b1 = O.core_iteration_bytes(s, 1, 1024)
     assert b1["weights"] == 3_274_698_240 and b1["kv_read"] == 86_507_520 and b1["kv_write"] == 84_480
