@@ -114,14 +114,16 @@ def test_tiled_gemm_edges_against_oracle(pkg, tuned, variant, M, N, K):
 
 @pytest.mark.parametrize("N", [16640, 16544])
 def test_tiled_gemm_last_round_as_small_tiles_changes_no_bit(pkg, tuned, N):
-    """4 x 65 tiles of 256 x 256: the 4 tiles of the last, nearly empty round (the last tile column, whole or 160 wide)
-    are multiplied as 128 x 128 tiles by a second launch over that column range.  Same bits as one launch, for every
-    epilogue that takes the split, and right against the fp32 product on sampled columns of both ranges."""
+    """4 x 65 tiles of 256 x 256 (4 x 130 under SwiGLU): the tiles of the last, nearly empty round (the last tile
+    columns, whole or partly filled) are multiplied as 128 x 128 tiles by a second launch over that column range.  Same
+    bits as one launch, for every epilogue, and right against the fp32 product on sampled columns of both ranges."""
     dt, M, K = torch.bfloat16, 1024, 192
     x, x1 = _gpu_randn((M, K), 600), _gpu_randn((M, K), 601)
     w, w2, res = _gpu_randn((N, K), 602, 0.05), _gpu_randn((N, 2 * K), 603, 0.05), _gpu_randn((M, N), 604)
+    fc = _gpu_randn((2 * N, K), 605, 0.05)
     calls = {"plain": lambda: pkg.hip.linear(x, w), "+ residual": lambda: pkg.hip.linear(x, w, residual=res),
-             "float": lambda: pkg.hip.linear(x, w, out_f32=True), "two operands": lambda: pkg.hip.linear(x, w2, x1=x1)}
+             "float": lambda: pkg.hip.linear(x, w, out_f32=True), "two operands": lambda: pkg.hip.linear(x, w2, x1=x1),
+             "SwiGLU": lambda: pkg.hip.linear(x, fc, swiglu=True)}
     for name, call in calls.items():
         tuned(gemm_tiled_split_tail=1)
         split = call()
@@ -132,6 +134,9 @@ def test_tiled_gemm_last_round_as_small_tiles_changes_no_bit(pkg, tuned, N):
     tuned(gemm_tiled_split_tail=1)
     want = (x.float() @ w[cols].float().T).to(dt).float() + res[:, cols].float()
     check(pkg.hip.linear(x, w, residual=res)[:, cols], want.to(dt), dt, "sampled columns")
+    z = (x.float() @ torch.cat([fc[cols], fc[N + cols]]).float().T).to(dt).float()
+    want = (F.silu(z[:, :cols.numel()]).to(dt).float() * z[:, cols.numel():]).to(dt)
+    check(pkg.hip.linear(x, fc, swiglu=True)[:, cols], want, dt, "sampled columns, SwiGLU")
 
 
 # ----------------------------------------------------------------------------- attention at 4 x 4096
