@@ -443,10 +443,13 @@ static int launch_tiled(TiledArgs a, hipStream_t s) {
 
 // Host entry for the other translation units: true when the shape is one the tiled kernel takes and is the better choice
 // for.  Few token rows against a matrix with few rows give too few tiles to fill the chip (there is no K split here):
-// up to 160 rows those go to the skinny kernels, 32 rows per pass over the weights.
+// those go to the skinny kernels, 32 rows per pass over the weights -- up to two passes at K = 5280, four at 10560 and
+// five (160 rows) at 17920, where the passes' split over K still beats one round of 128 x 128 tiles walking the whole of K
+// (measured at 33 .. 160 rows: Wqkv 98 / 130 us in three / four passes against 75 / 81 tiled, mlp.proj 172 against 199).
 bool tiled_gemm_fits(int M, int N, int K0, int K1, int dtype) {
     const int64_t small_tiles = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
-    if (g_tiled_variant == 0 && M <= 160 && small_tiles < 128) return false;
+    const int passes = (K0 + K1 + 3499) / 3500;
+    if (g_tiled_variant == 0 && small_tiles < 128 && M <= 160 && M <= 32 * passes) return false;
     return dtype == RAVEN_BF16 && M >= 1 && N % 8 == 0 && K0 % 8 == 0 && K0 > 0 && (K1 == 0 || K1 == K0) && (int64_t)M * (K0 > K1 ? K0 : K1) < (1ll << 31) &&
            (int64_t)N * 2 * (K0 + K1) < (1ll << 31);
 }
