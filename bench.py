@@ -66,16 +66,34 @@ def parse():
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
-def core_iteration_bytes(cfg, batch, t_cached, elt=2):
+def core_iteration_bytes(cfg, batch, t_cached, elt=2, adapter_split=False):
     """Algorithmic HBM bytes of one recurrence iteration of a decode step: every weight of the adapter and the core blocks
     once (Wqkv 3h*h, attn.proj h*h, mlp.fc 2*inter*h, mlp.proj h*inter, four norm weights, the q/k bias; adapter 2h*h),
-    the cached keys and values of `t_cached` positions read once per block, and the new position's K and V written."""
+    the cached keys and values of `t_cached` positions read once per block, and the new position's K and V written.
+    adapter_split: the schedule of a call with two or more recurrences, which streams only the state half of the adapter
+    (h*h) per recurrence plus the fp32 sums of the embedding half (batch*h*4); the embedding half itself is read once per
+    call and is counted by the caller (`adapter_once_bytes`)."""
     h, inter, nb = cfg.n_embd, cfg.intermediate_size, cfg.n_layers_in_recurrent_block
     per_block = (3 * h * h + h * h + 2 * inter * h + h * inter + 4 * h + (2 * h if cfg.qk_bias else 0)) * elt
-    weights = nb * per_block + 2 * h * h * elt
+    adapter = (h * h * elt + batch * h * 4) if adapter_split else 2 * h * h * elt
+    weights = nb * per_block + adapter
     kv_read = batch * nb * 2 * h * t_cached * elt
     kv_write = batch * nb * 2 * h * elt
-    return {"weights": weights, "kv_read": kv_read, "kv_write": kv_write, "total": weights + kv_read + kv_write}
+    return {"weights": weights, "adapter": adapter, "kv_read": kv_read, "kv_write": kv_write, "total": weights + kv_read + kv_write}
+
+
+def adapter_once_bytes(cfg, batch, elt=2):
+    """What a call with the adapter split by columns reads and writes once, whatever its number of recurrences: the
+    embedding half of the matrix and the fp32 sums it leaves."""
+    h = cfg.n_embd
+    return h * h * elt + batch * h * 4
+
+
+# HBM-side bytes per launch of the tiled mlp.fc GEMM at M = 16384 from rocprofv3 --pmc (FETCH_SIZE 4,445,529 KiB x 1.99974 +
+# WRITE_SIZE 573,440 KiB x 1.0, both scaled by a 256 MiB copy): 8 x the 1.14 GB of operands + output, the panel re-reads
+# of 256 x 256 tiles in 8 x 4 groups per XCD.  Profiler figures, so constants, with the file that holds the readings.
+TILED_FC_TRAFFIC = int(4445529 * 1024 * 1.99974 + 573440 * 1024)
+TILED_FC_TRAFFIC_SOURCE = "profiles/gemm_tiled_bs4x4096_counters.txt"
 
 
 def prefill_record(pkg, model, B, S, r):
@@ -139,7 +157,7 @@ def prefill_record(pkg, model, B, S, r):
         "roofline": {"bound": "mfma", "kernel": f"gemm_tiled_kernel<SwiGLU, 256x256> (mlp.fc {2 * inter}x{h}, M={M})",
                      "achieved": round(fc_tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(fc_tflops / MFMA_PEAK_TFLOPS, 4), "flops_per_launch": fc_flops, "avg_us": round(fc_ms * 1e3, 1),
-                     "traffic": None},
+                     "traffic": TILED_FC_TRAFFIC, "traffic_source": TILED_FC_TRAFFIC_SOURCE},
         "iteration_roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                                "frac": round(tflops / MFMA_PEAK_TFLOPS, 4), "flops_per_iteration": gemm_flops + attn_flops},
     }
@@ -558,7 +576,8 @@ FC_TRAFFIC_SOURCE = "profiles/mlp_fc_decode_hbm_traffic.txt"
 
 def decode_record(pkg, model, B, prompt_len, steps, warmup, r, use_graph):
     """Full-token decode at B sequences with what bounds it: tokens/s over `steps` greedy tokens, one recurrence
-    iteration at 1024 cached positions (eager launches and a replayed graph of eight), and the dominant kernel -- the
+    iteration at 1024 cached positions (single eager calls, and a replayed graph of a token's worth of them, each leg over
+    the bytes its own schedule streams and over distinct K/V slots), and the dominant kernel -- the
     mlp.fc product with its norm prologue and SwiGLU epilogue, 47 % of a token's bytes -- alone, timed with HIP events on
     the launch stream exactly as the decode loop launches it, rotating over the four core blocks' fc matrices (1.5 GB)
     so that no cache level can keep a matrix between launches."""
@@ -569,15 +588,25 @@ def decode_record(pkg, model, B, prompt_len, steps, warmup, r, use_graph):
     del cache
     torch.cuda.empty_cache()
     mean_t = prompt_len + warmup + steps / 2.0
-    bb = core_iteration_bytes(cfg, B, int(mean_t))
-    per_block_w = (bb["weights"] - 2 * cfg.n_embd * cfg.n_embd * 2) // 4
-    token_bytes = (r * bb["total"] + 4 * (per_block_w + (bb["kv_read"] + bb["kv_write"]) // 4) + cfg.vocab_size * cfg.n_embd * 2)
+    # a token's r recurrences are one library call, which splits the adapter by columns (state half per recurrence, embedding
+    # half once per token) whenever r >= 2: count what that schedule streams
+    split = r >= 2
+    bb = core_iteration_bytes(cfg, B, int(mean_t), adapter_split=split)
+    per_block_w = (bb["weights"] - bb["adapter"]) // 4
+    token_bytes = (r * bb["total"] + (adapter_once_bytes(cfg, B) if split else 0)
+                   + 4 * (per_block_w + (bb["kv_read"] + bb["kv_write"]) // 4) + cfg.vocab_size * cfg.n_embd * 2)
 
     # ---- one recurrence iteration at T = 1024 (the unit of the roofline target) ----
+    # Two legs, each with the bytes its own schedule streams: (1) single raven_core_iteration launches (whole adapter per
+    # iteration); (2) a replayed HIP graph of one raven_core_iterations call of n_it recurrences, as the decode loop
+    # issues them (adapter split by columns, its embedding half read once per call).  Both walk distinct K/V slots, as a
+    # token's recurrences do: 128 slots (2.8 GB) for one sequence, 32 slots for more.
     h, nh, hd, T = cfg.n_embd, cfg.n_heads, cfg.head_dim, 1024
     nat = model._natives()
-    kc = torch.randn(4, B, nh, T + 1, hd, device=dev, dtype=torch.bfloat16)
-    vc = torch.randn(4, B, nh, T + 1, hd, device=dev, dtype=torch.bfloat16)
+    n_slots = 128 if B == 1 else 32
+    n_it = n_slots // 4
+    kc = torch.empty(n_slots, B, nh, T + 1, hd, device=dev, dtype=torch.bfloat16).normal_()
+    vc = torch.empty(n_slots, B, nh, T + 1, hd, device=dev, dtype=torch.bfloat16).normal_()
     kv = pkg.hip.make_cache(kc, vc)
     ws = pkg.hip.block_workspace(nat["dims"], B, dev)
     state = torch.randn(B, h, device=dev, dtype=torch.bfloat16)
@@ -585,21 +614,25 @@ def decode_record(pkg, model, B, prompt_len, steps, warmup, r, use_graph):
     outb = torch.empty_like(state)
     adapter_w = model.transformer.adapter.weight
 
-    def one_iter():
-        pkg.hip.core_iteration(nat["dims"], adapter_w, nat["core"], state, emb, outb, nat["freqs"], kv, 0, B, 1, T, ws)
+    def one_iter(i=[0]):
+        i[0] += 1
+        pkg.hip.core_iteration(nat["dims"], adapter_w, nat["core"], state, emb, outb, nat["freqs"], kv, 4 * (i[0] % n_it), B, 1, T, ws)
 
-    def eight_iters():  # as the decode loop runs them: one call, the same four slots every time
-        pkg.hip.core_iterations(nat["dims"], adapter_w, nat["core"], state, emb, outb, nat["freqs"], kv, [[0, 1, 2, 3]] * 8, B, 1, T, ws)
+    def many_iters():
+        pkg.hip.core_iterations(nat["dims"], adapter_w, nat["core"], state, emb, outb, nat["freqs"], kv,
+                                [[4 * it + j for j in range(4)] for it in range(n_it)], B, 1, T, ws)
 
-    iter_eager_ms = event_time_ms(one_iter, 20)
-    eight_iters()
+    iter_eager_ms = event_time_ms(one_iter, 2 * n_it, warm=n_it)
+    many_iters()
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        eight_iters()
-    iter_graph_ms = event_time_ms(graph.replay, 10) / 8
-    it_bytes = core_iteration_bytes(cfg, B, T)["total"]
-    iter_ms = min(iter_eager_ms, iter_graph_ms)
+        many_iters()
+    iter_graph_ms = event_time_ms(graph.replay, 6, warm=2) / n_it
+    eager_bytes = core_iteration_bytes(cfg, B, T)["total"]
+    graph_bytes = core_iteration_bytes(cfg, B, T, adapter_split=True)["total"] + adapter_once_bytes(cfg, B) / n_it
+    eager_gbs = eager_bytes / (iter_eager_ms * 1e-3) / 1e9
+    graph_gbs = graph_bytes / (iter_graph_ms * 1e-3) / 1e9
     del graph, kc, vc, kv
 
     # ---- dominant kernel ----
@@ -633,15 +666,22 @@ def decode_record(pkg, model, B, prompt_len, steps, warmup, r, use_graph):
     return {
         "batch": B, "tokens_per_s": round(tok_s, 3), "ms_per_step": round(ms_step, 4), "steps": steps, "prefill_s": round(prefill_s, 3),
         "recurrence_steps_per_s": round(tok_s * r / B, 2),
-        "token_roofline": {"bytes_per_token": int(token_bytes), "achieved_GBs": round(token_bytes * (tok_s / B) / 1e9, 1),
+        "token_roofline": {"bytes_per_token": int(token_bytes), "adapter_split": split, "achieved_GBs": round(token_bytes * (tok_s / B) / 1e9, 1),
                            "frac": round(token_bytes * (tok_s / B) / 1e9 / HBM_PEAK_GBS, 4)},
         "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": round(fc_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(fc_gbs / HBM_PEAK_GBS, 4),
                      "bytes_per_launch": int(fc_bytes), "avg_us": round(fc_ms * 1e3, 2),
                      "traffic": FC_TRAFFIC.get(B), "traffic_source": FC_TRAFFIC_SOURCE if B in FC_TRAFFIC else None},
-        "core_iteration": {"T": T, "batch": B, "bytes": int(it_bytes), "ms_eager": round(iter_eager_ms, 4),
-                           "ms_graph": round(iter_graph_ms, 4), "achieved_GBs": round(it_bytes / (iter_ms * 1e-3) / 1e9, 1),
-                           "frac": round(it_bytes / (iter_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+        # frac is the graph leg's: the schedule the decode loop runs, over the bytes that schedule streams
+        "core_iteration": {"T": T, "batch": B, "kv_slots_walked": n_slots,
+                           "eager_single_call": {"bytes": int(eager_bytes), "ms": round(iter_eager_ms, 4), "achieved_GBs": round(eager_gbs, 1),
+                                                 "frac": round(eager_gbs / HBM_PEAK_GBS, 4), "adapter": "whole (2h x h) per iteration"},
+                           "graph": {"iterations_per_replay": n_it, "bytes_per_iteration": int(graph_bytes),
+                                     "ms_per_iteration": round(iter_graph_ms, 4), "achieved_GBs": round(graph_gbs, 1),
+                                     "frac": round(graph_gbs / HBM_PEAK_GBS, 4),
+                                     "adapter": "state half (h x h) per iteration, embedding half once per replay"},
+                           "bytes": int(graph_bytes), "ms": round(iter_graph_ms, 4), "achieved_GBs": round(graph_gbs, 1),
+                           "frac": round(graph_gbs / HBM_PEAK_GBS, 4)},
     }
 
 

@@ -757,8 +757,15 @@ def test_bench_counts_the_same_bytes_and_keeps_the_oracle_to_its_cpu_leg(pkg):
     import os
     import bench
     s = O.RavenShape.nebel()
+    cfg = pkg.RavenConfig()
     for B, T in ((1, 1024), (8, 640), (32, 1024)):
-        assert bench.core_iteration_bytes(pkg.RavenConfig(), B, T) == O.core_iteration_bytes(s, B, T)
+        mine, pinned = bench.core_iteration_bytes(cfg, B, T), O.core_iteration_bytes(s, B, T)
+        assert {k: mine[k] for k in pinned} == pinned
+        # the schedule of a call with several recurrences: the embedding half of the adapter (5280 x 5280 bf16) leaves the
+        # per-iteration count, its fp32 sums (B x 5280) enter it; that half and the sums are counted once per call
+        split = bench.core_iteration_bytes(cfg, B, T, adapter_split=True)
+        assert split["total"] == pinned["total"] - 5280 * 5280 * 2 + B * 5280 * 4
+        assert bench.adapter_once_bytes(cfg, B) == 5280 * 5280 * 2 + B * 5280 * 4
     tree = ast.parse(open(os.path.join(os.path.dirname(bench.__file__), "bench.py")).read())
     holders = [fn.name for fn in ast.walk(tree) if isinstance(fn, ast.FunctionDef)
                for node in ast.walk(fn) if isinstance(node, (ast.Import, ast.ImportFrom))
