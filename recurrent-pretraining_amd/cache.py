@@ -55,13 +55,14 @@ class _CoreSteps:
         self.runs.insert(i + 1, [pos, en, mask])
         return i + 1
 
-    def add(self, bit: int, first: int, n: int) -> None:
-        """Positions first .. first+n-1 now hold core step `bit`; a second write of the same entry is an error."""
+    def add(self, bit: int, first: int, n: int, overwrite: bool = False) -> None:
+        """Positions first .. first+n-1 now hold core step `bit`; a second write of the same entry is an error unless
+        the steps share entries (the compress-* strategies)."""
         if len(self) < first + n:
             self.runs.append([len(self), first + n, 0])
         i, j = self._split(first), self._split(first + n)
         for r in self.runs[i:j]:
-            assert not (r[2] >> bit) & 1, "overwrite of a cached position"  # RMM:192-193
+            assert overwrite or not (r[2] >> bit) & 1, "overwrite of a cached position"  # RMM:192-193
             r[2] |= 1 << bit
         for k in range(min(j, len(self.runs) - 1), max(i - 1, 0) - 1, -1):  # re-join equal neighbours
             if k + 1 < len(self.runs) and self.runs[k][2] == self.runs[k + 1][2]:
@@ -198,16 +199,26 @@ class HuginnDynamicCache:
         self._v: Optional[torch.Tensor] = None
         self._neg_slots = 0          # slots reserved for negative (coda) step indices
         self._filled: dict[int, int] = {}  # step -> 1 + highest position present (first-touch order)
-        # Tokens computed with different numbers of recurrences leave gaps at the deeper core steps.  Kept while no
-        # compress-* remap is in use (those strategies overwrite a few shared steps instead).  A token runs its core
-        # steps in order, so for the kernels "how many of the steps 2, 3, 4, ... are cached" per position says it all.
+        # Tokens computed with different numbers of recurrences leave gaps at the deeper core steps.  A token runs its
+        # core steps in order, so for the kernels "how many of the steps 2, 3, 4, ... are cached" per position says it
+        # all.  Under a compress-* remap the same holds for the shared entries: every one of the reference's remaps sends
+        # the steps 2, 3, 4, ... of a token to entries 2, 3, 4, ... without skipping one (RMM:169-182), later steps
+        # overwriting earlier ones.
         self._core = _CoreSteps()
         self._sp_dev: Optional[torch.Tensor] = None   # device copy of the per-position depths, built on demand
         self._sp_valid = 0                            # positions of _sp_dev that are up to date
         self._min_memo = (0, 0)                       # (n, smallest depth below n): older positions never change
-        self.key_cache = _StepView(self, "_k")
-        self.value_cache = _StepView(self, "_v")
         self._struct: Optional[hip.KVCache] = None
+
+    # views made on access: a view stored on the cache would tie it into a reference cycle, and its tens of GB would
+    # then stay allocated until the garbage collector happens to run
+    @property
+    def key_cache(self) -> _StepView:
+        return _StepView(self, "_k")
+
+    @property
+    def value_cache(self) -> _StepView:
+        return _StepView(self, "_v")
 
     # ---- storage ---------------------------------------------------------------------------
     def _slot(self, step: int) -> int:
@@ -266,6 +277,9 @@ class HuginnDynamicCache:
         if not all(self.has_gap(s, first_pos) for s in steps):
             raise ValueError("steps of one launch must agree on whether older positions are missing")
         mode = lookup_mode(self.lookup_strategy)
+        if mode == hip.LOOKUP_ALWAYS_LAST and "compress-" in self.lookup_strategy:
+            # the reference then also looks up the new rows themselves, among entries their own earlier recurrences left
+            raise NotImplementedError("always-last-m4 lookups over shared (compress-*) entries with missing positions are not built")
         if self._core.holes(first_pos):
             raise NotImplementedError("lookups need positions that hold the core steps 2, 3, ... without holes")
         if mode != hip.LOOKUP_SKIP and self._min_core(first_pos) <= max((remap_step(int(s), self.lookup_strategy) - 2) % 4 for s in steps):
@@ -278,8 +292,9 @@ class HuginnDynamicCache:
             self._sp_valid = first_pos
         return hip.make_cache(self._k, self._v, self._sp_dev, mode, self._slot(2))
 
-    def _tracks_core(self, step: int) -> bool:
-        return step >= 2 and "compress-" not in self.lookup_strategy
+    @staticmethod
+    def _tracks_core(step: int) -> bool:
+        return step >= 2
 
     def _present(self, step: int, pos: int) -> bool:
         if not 0 <= pos < self._filled.get(step, 0):
@@ -296,9 +311,7 @@ class HuginnDynamicCache:
         if first_pos <= 0:
             return False
         if not self._tracks_core(step):
-            if self._filled.get(step, 0) < first_pos:
-                raise NotImplementedError(f"positions missing at step {step} under lookup strategy {self.lookup_strategy!r}")
-            return False
+            return False  # the prelude and coda entries: every token passes through them
         return self._min_core(first_pos) <= step - 2
 
     def _min_core(self, n: int) -> int:
@@ -309,9 +322,10 @@ class HuginnDynamicCache:
     def note_append(self, step_idx: int, n_new: int, first_pos: int) -> int:
         """Bookkeeping for positions the kernels wrote at `step_idx`; returns the slot used."""
         step = remap_step(int(step_idx), self.lookup_strategy)
+        shared = "compress-" in self.lookup_strategy
         if self._tracks_core(step):
-            self._core.add(step - 2, first_pos, n_new)
-        elif "compress-" not in self.lookup_strategy:  # RMM:192-193: no overwrite except for the coda
+            self._core.add(step - 2, first_pos, n_new, overwrite=shared)
+        elif not shared:  # RMM:192-193: no overwrite except for the coda
             assert step < 0 or self._filled.get(step, 0) <= first_pos, "overwrite of a cached position"
         self._filled[step] = max(self._filled.get(step, 0), first_pos + n_new)
         return self._slot(step)
@@ -338,6 +352,8 @@ class HuginnDynamicCache:
         # some positions were never computed at this step: gather per position, as RMM:199-253 does
         lookup = self.lookup_strategy if lookup_strategy is None else lookup_strategy
         mode = hip.LOOKUP_SKIP if self.lookup_strategy == "full" else lookup_mode(lookup)
+        if mode == hip.LOOKUP_ALWAYS_LAST and "compress-" in self.lookup_strategy:
+            raise NotImplementedError("always-last-m4 lookups over shared (compress-*) entries with missing positions are not built")
         if self._core.holes(first):
             raise NotImplementedError("lookups need positions that hold the core steps 2, 3, ... without holes")
         depths = self._core.depths(first) if self._tracks_core(mapped) else []

@@ -45,6 +45,7 @@ struct GemmArgs {
     int interleave;        // gemv: unit = u * total_waves + wave (1) or wave * units_per_wave + u (0)
     int row_stride;        // mfma: 1 = a tile is 16 neighbouring weight rows, 2 = every second row (see mfma_kernel)
     int line_aligned;      // mfma: the rows of a tile all start at the same offset inside a 128-byte line
+    int rows_per_unit;     // mfma, ragged variants: weight rows (per side for SwiGLU) a workgroup owns; its last tile is partly empty
 };
 
 // Launch-shape knobs (raven_set_tuning); 0 = automatic.
@@ -55,6 +56,7 @@ struct Tuning {
     int gemv_wgs_per_cu = 4;
     int gemm_four_tiles = 1;
     int gemm_mfma_min_rows = 2;  // fewer rows go to the vector kernels (one row: the K-split GEMV)
+    int gemm_ragged = 1;         // 0 never, 1 = one workgroup per resident slot with partly empty last tiles where the shape divides so
 };
 static Tuning g_tuning;
 
@@ -203,7 +205,12 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemmArgs a) {
 // KM = k-values per macro-step: 128, or 64 for the variants with four weight tiles per workgroup (the same
 // bytes per macro-step; a quarter-wave then reads two rows of 128 bytes).  LDS rows are KM + 8 elements long
 // (272 or 144 bytes: both spread 16 rows over the 64 banks without conflicts for 16-byte reads).
-template <int MT, int NT, int EPI, int KM = 128>
+//
+// RAG: a workgroup owns a.rows_per_unit rows (per side for SwiGLU) instead of 16 per tile slot: its tile slots cover them
+// 16 at a time and the last slot is partly empty (its missing rows are neither loaded nor stored).  This lets the host cut
+// a matrix into exactly as many workgroups as the chip holds at once (17920 gate rows = 512 x 35), where whole tiles
+// would leave a partly filled last round.
+template <int MT, int NT, int EPI, int KM = 128, bool RAG = false>
 __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
     constexpr int ROWS = 16 * (NT + MT);
     constexpr int kPitch = KM + 8;
@@ -225,19 +232,16 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
     int tile_row0[NT];  // first weight row of each tile; row i of the tile is tile_row0 + i * rs
     int tile_out0[NT];  // output column of that row
     bool tile_ok[NT];
+    int tile_rows[NT];  // RAG: rows of the tile that exist (1..16 where tile_ok); 16 otherwise
+    const int rpu = RAG ? a.rows_per_unit : 16 * NG;  // rows a unit owns per side
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        if (EPI == EPI_SWIGLU) {
-            const int first = (group * NG + t % NG) * 16 * rs;
-            tile_ok[t] = first < a.N;
-            tile_out0[t] = (tile_ok[t] ? first : group * NG * 16 * rs) + parity;
-            tile_row0[t] = tile_out0[t] + (t / NG) * a.N;  // the first NG tiles are gate tiles, the others their up tiles
-        } else {
-            const int first = (group * NT + t) * 16 * rs;
-            tile_ok[t] = first < a.N;
-            tile_out0[t] = (tile_ok[t] ? first : group * NT * 16 * rs) + parity;
-            tile_row0[t] = tile_out0[t];
-        }
+        const int first = (group * rpu + (t % NG) * 16) * rs;   // SwiGLU: the first NG tiles are gate tiles, the others their up tiles
+        tile_ok[t] = first < a.N && (!RAG || (t % NG) * 16 < rpu);
+        tile_rows[t] = RAG ? min(16, rpu - (t % NG) * 16) : 16;
+        tile_out0[t] = (tile_ok[t] ? first : group * rpu * rs) + parity;
+        tile_row0[t] = tile_out0[t] + (EPI == EPI_SWIGLU ? (t / NG) * a.N : 0);
+        if (RAG && !tile_ok[t]) tile_rows[t] = 1;  // reads row 0 of the unit's first tile, stores nothing
     }
 
     f32x4 acc[NT][MT];
@@ -289,8 +293,10 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
 #pragma unroll
             for (int t = 0; t < NT; ++t)
 #pragma unroll
-                for (int i = 0; i < IPT; ++i)
+                for (int i = 0; i < IPT; ++i) {
+                    if (RAG && RPI * i + lr >= tile_rows[t]) continue;  // rows the tile does not have: their products are never stored
                     st.w[t][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(W + (int64_t)(tile_row0[t] + (RPI * i + lr) * rs) * K + wk0 + k));
+                }
         };
         auto park = [&](const Staged& st) {  // registers -> this wave's LDS tile
 #pragma unroll
@@ -326,7 +332,7 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         };
         // one register set: its loads for macro-step s+1 are in flight while step s is multiplied out of LDS
-        Staged st;
+        Staged st{};
         if (mb < me) fetch(mb, st);
         for (int mac = mb; mac < me; mac += 4) {
             park(st);
@@ -341,7 +347,8 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
             for (int k = kb; k < ke; k += 32) {
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    const bf16x8 wv = *reinterpret_cast<const bf16x8*>(W + (int64_t)(tile_row0[t] + ln * rs) * K + wk0 + k + kq * 8);
+                    const int wr = RAG ? min(ln, tile_rows[t] - 1) : ln;  // a partly empty tile repeats its last row
+                    const bf16x8 wv = *reinterpret_cast<const bf16x8*>(W + (int64_t)(tile_row0[t] + wr * rs) * K + wk0 + k + kq * 8);
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt) {
                         const int m = min(mt * 16 + ln, a.M - 1);
@@ -384,6 +391,7 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
                 if (!tile_ok[g]) continue;
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
+                    if (RAG && kq * 4 + v >= tile_rows[g]) continue;
                     const int n = tile_out0[g] + (kq * 4 + v) * rs;
                     static_cast<bf16*>(a.y)[(int64_t)m * a.N + n] = from_f32<bf16>(swiglu<bf16>(acc[g][mt][v], acc[NG + g][mt][v]));
                 }
@@ -393,7 +401,8 @@ __global__ __launch_bounds__(256) void mfma_kernel(GemmArgs a) {
             for (int t = 0; t < NT; ++t) {
                 if (!tile_ok[t]) continue;
 #pragma unroll
-                for (int v = 0; v < 4; ++v) store_out<bf16>(a, m, tile_out0[t] + (kq * 4 + v) * rs, acc[t][mt][v]);
+                for (int v = 0; v < 4; ++v)
+                    if (!RAG || kq * 4 + v < tile_rows[t]) store_out<bf16>(a, m, tile_out0[t] + (kq * 4 + v) * rs, acc[t][mt][v]);
             }
         }
     }
@@ -473,7 +482,19 @@ static int dispatch_mfma(GemmArgs a, hipStream_t s) {
     const bool four = g_tuning.gemm_four_tiles == 2 ||
                       (g_tuning.gemm_four_tiles == 1 && a.M > 16 && g4 >= n_cus() / 2 && (g4 <= n_cus() || g4 >= 8 * n_cus()));
     if constexpr (EPI == EPI_SWIGLU) {
-        if (four) {
+        // A matrix that divides into one workgroup per resident slot (two per CU) of 33..48 gate rows: three tile slots
+        // per side, the last one partly empty -- one full round instead of a partly filled last one, and the X tile is
+        // fetched once per 70 weight rows instead of once per 32.  mlp.fc of the 3.5b shape (17920 = 512 x 35), us per
+        // launch against the whole-tile variants: 32 rows 67.7 / 79.1, 16 rows 60.2 / 66.2, 8 rows 58.9 / 61.7
+        int rpu = 0;
+        if (g_tuning.gemm_ragged)
+            for (int r = 33; r <= 48 && !rpu; ++r)
+                if (a.N % (r * rs) == 0 && a.N / r <= 2 * n_cus() && a.N / r >= 2 * n_cus() - n_cus() / 4) rpu = r;
+        if (rpu) {
+            a.rows_per_unit = rpu;
+            if (a.M <= 16) mfma_kernel<1, 6, EPI, 64, true><<<dim3(a.N / rpu), dim3(256), 0, s>>>(a);
+            else           mfma_kernel<2, 6, EPI, 64, true><<<dim3(a.N / rpu), dim3(256), 0, s>>>(a);
+        } else if (four) {
             if (a.M <= 16) mfma_kernel<1, 4, EPI, 64><<<dim3(groups2), dim3(256), 0, s>>>(a);
             else           mfma_kernel<2, 4, EPI, 64><<<dim3(groups2), dim3(256), 0, s>>>(a);
         } else if (a.M <= 16)
@@ -563,6 +584,7 @@ extern "C" int raven_set_tuning(const char* key, int32_t value) {
     else if (k == "gemv_wgs_per_cu") g_tuning.gemv_wgs_per_cu = value;
     else if (k == "linear_ks") g_linear_ks = value;
     else if (k == "gemm_four_tiles") g_tuning.gemm_four_tiles = value;
+    else if (k == "gemm_ragged") g_tuning.gemm_ragged = value;
     else if (k == "gemm_mfma_min_rows" && value >= 2) g_tuning.gemm_mfma_min_rows = value;
     else if (k == "attn_split_target" && value > 0) g_attn_split_target = value;
     else if (k == "attn_big_grid" && value > 0) g_attn_big_grid = value;

@@ -14,6 +14,16 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+def pytest_terminal_summary(terminalreporter):
+    """The largest unscaled max-abs and rel-L2 each GPU parity test saw in its check() calls."""
+    log = getattr(sys.modules.get("test_gpu_kernels"), "PARITY_LOG", None)
+    if not log:
+        return
+    terminalreporter.write_sep("-", "parity: largest max-abs / rel-L2 per test (unscaled)")
+    for test, (max_abs, rel, n) in log.items():
+        terminalreporter.write_line(f"{max_abs:.3e}  {rel:.3e}  {n:4d} checks  {test}")
+
+
 @pytest.fixture(scope="session")
 def pkg():
     """The product package (its directory name has a hyphen, so it is imported through the entry module)."""
@@ -36,7 +46,7 @@ def lib(pkg):
 
 
 # defaults of the launch-shape knobs the tests change (raven_set_tuning); results never depend on them
-TUNING_DEFAULTS = {"linear_ks": 0, "gemm_four_tiles": 1, "attn_wide": 0, "gemm_tiled_min_rows": 33, "gemm_tiled_variant": 0, "gemm_tiled_split_tail": 1, "prefill_waves": 0}
+TUNING_DEFAULTS = {"linear_ks": 0, "gemm_four_tiles": 1, "attn_wide": 0, "gemm_tiled_min_rows": 33, "gemm_tiled_variant": 0, "gemm_tiled_split_tail": 1, "prefill_waves": 0, "gemm_ragged": 1, "norm_early": -1}
 
 
 @pytest.fixture

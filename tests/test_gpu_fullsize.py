@@ -1,5 +1,7 @@
 """Full-size checks at the 3.5b shape (bf16, 512-token prompts, 32 recurrences, up to 32 sequences), where the CPU
-oracle would take minutes per call: properties that hold independently of the size and need no reference values.
+oracle would take minutes per call: properties that hold independently of the size and need no reference values, and
+one whole forward in fp32 against the fp32 oracle (short prompt, two recurrences), which pins the indexing of every
+part of the model at its real strides.
 
   * determinism: the same call twice gives the same bits; a HIP-graph replay gives the bits of the eager launches;
   * permutation equivariance: shuffling the sequences of a batch shuffles logits, latents and cache rows, bit for bit
@@ -20,6 +22,15 @@ import torch
 pytestmark = pytest.mark.gpu
 
 PROMPT, R = 512, 32
+
+
+@pytest.fixture(autouse=True)
+def _release_device_memory():
+    """The caches of these tests are tens of GB each: give them back before the next test allocates its own."""
+    yield
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
 
 
 @pytest.fixture(scope="module")
@@ -72,9 +83,9 @@ def test_decode_is_deterministic_and_graph_replay_equals_eager(pkg, nebel, B):
     assert torch.equal(again[0], again[1])
 
 
-@pytest.mark.parametrize("B", [1, 8])
+@pytest.mark.parametrize("B", [1, 8, 32])
 def test_full_token_decode_256_greedy_tokens(pkg, nebel, B):
-    """The full-token decode configuration at 1 and 8 sequences: 512-token random prompt, 256 greedy tokens at r = 32
+    """The full-token decode configuration at 1, 8 and 32 sequences: 512-token random prompt, 256 greedy tokens at r = 32
     (prefill through forward(), then one HIP-graph replay per token).  Zero initial states make the run reproducible:
     the graph run and the eager run produce the same 256 tokens; all ids are inside the vocabulary; the cache holds
     512 + 255 positions in all 132 step entries."""
@@ -165,3 +176,54 @@ def test_fp32_model_at_the_3_5b_shape_cache_equivalence(pkg):
     out = model.generate_minimal(ids[:1, :n].contiguous(), pkg.GenerationSettings(max_new_tokens=3), num_steps=2, init_scale=0.0,
                                  stop_tokens=set())
     assert out.shape == (1, n + 3)
+
+
+def test_fp32_whole_forward_at_the_3_5b_shape_against_the_fp32_oracle(pkg):
+    """Embedding (65536 x 5280, scaled), two prelude blocks, two recurrences of adapter + four core blocks, two coda
+    blocks, ln_f on the latents and again on the coda output, tied LM head: an 8-token prompt through the cache and one
+    decode step, in fp32 against the fp32 oracle (RMM:638-724) -- logits, latent states, and the key / value rows of the
+    step entries 0, 1 (prelude), 2 and 9 (first and last core step), -1 and -2 (coda).  In fp32 a wrong slot, stride,
+    head or column shows as an O(1) difference, while rounding differences stay small: per kernel they are 1e-6, and the
+    recurrent block amplifies them by about an order of magnitude per recurrence with random weights, hence the bars
+    below for what sits behind two recurrences (the first block's rows are held to the per-kernel fp32 bar)."""
+    from oracle import raven_oracle as O
+    from test_gpu_kernels import check, close
+    s = O.RavenShape.nebel()
+    model = pkg.RavenForCausalLM(pkg.RavenConfig(), device="cuda:0", dtype=torch.float32)
+    torch.manual_seed(0)
+    with torch.no_grad():
+        for name, p in model.state_dict().items():
+            if name == "freqs_cis" or name == "lm_head.weight":
+                continue
+            p.normal_(1.0 if p.dim() == 1 else 0.0, 0.02)
+    w = {k: v.detach().cpu() for k, v in model.state_dict().items() if k != "freqs_cis"}
+    w["lm_head.weight"] = w["transformer.wte.weight"]
+    w["freqs_cis"] = O.rope_table(s.head_dim, s.block_size, s.rope_base)
+    B, n, h, r = 2, 8, s.n_embd, 2
+    g = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, s.vocab_size, (B, n + 1), generator=g)
+    ids[0, 0], ids[1, 0], ids[0, n] = 0, s.vocab_size - 1, s.vocab_size - 1   # first and last row of the embedding table
+    states = O.initialize_state(torch.empty(B, n + 1, h), s, 1.0, g)
+    ref_cache, cache = O.DictCache(), pkg.HuginnDynamicCache()
+    steps = [(ids[:, :n], states[:, :n], torch.arange(n)), (ids[:, n:], states[:, n:], torch.tensor([n]))]
+    for i, (tok, st, cp) in enumerate(steps):
+        want = O.forward(w, s, input_ids=tok, input_states=st, past_key_values=ref_cache, use_cache=True, cache_position=cp, num_steps=r)
+        got = model(input_ids=tok.cuda(), input_states=st.cuda(), past_key_values=cache, use_cache=True, cache_position=cp.cuda(),
+                    num_steps=r)
+        e_lat, e_log = close(got.latent_states, want.latent_states, "latents"), close(got.logits, want.logits, "logits")
+        print(f"fp32 whole forward at the 3.5b shape, call {i}: latents max-abs {e_lat[0]:.3e} rel-L2 {e_lat[1]:.3e}; "
+              f"logits max-abs {e_log[0]:.3e} rel-L2 {e_log[1]:.3e} (|logit|max {want.logits.abs().max():.2f})")
+        assert got.logits.shape == (B, tok.shape[1], 65536) and got.logits.dtype == torch.float32
+        assert e_lat[1] <= 5e-4 and e_log[1] <= 5e-4, (e_lat, e_log)   # seen: 9e-5 and 1.5e-4
+        assert torch.equal(got.logits[:, -1].argmax(-1).cpu(), want.logits[:, -1].argmax(-1))
+    assert cache.get_seq_length() == ref_cache.get_seq_length() == n + 1
+    assert sorted(cache.key_cache.keys()) == sorted(ref_cache.key_cache.keys()) == [-2, -1] + list(range(10))
+    for step in (0, 1, 2, 9, -1, -2):
+        for pos in (0, n - 1, n):
+            ek = close(cache.key_cache[step][pos], ref_cache.key_cache[step][pos], f"K[{step}][{pos}]")
+            ev = close(cache.value_cache[step][pos], ref_cache.value_cache[step][pos], f"V[{step}][{pos}]")
+            print(f"  step {step:2d} pos {pos}: K rel-L2 {ek[1]:.3e}  V rel-L2 {ev[1]:.3e}")
+            if step in (0, 1, 2):   # in front of the recurrence's amplification: the per-kernel fp32 bar (seen: 3e-7 .. 4e-6)
+                check(cache.key_cache[step][pos], ref_cache.key_cache[step][pos], torch.float32, f"K[{step}][{pos}]")
+                check(cache.value_cache[step][pos], ref_cache.value_cache[step][pos], torch.float32, f"V[{step}][{pos}]")
+            assert ek[1] <= 5e-4 and ev[1] <= 5e-4, (step, pos, ek, ev)   # seen behind two recurrences: 1e-5 .. 1.2e-4

@@ -2,8 +2,10 @@
 against the CPU oracle on identical seeded inputs.
 
 Tolerances: bf16 results must satisfy max-abs <= 2e-2 and rel-L2 <= 1e-2 against the oracle
-(the bar the build's target states for per-kernel outputs); fp32 results 1e-4 / 1e-5; integer
-outputs (argmax ids, cache positions) bit-exact."""
+(the bar the build's target states for per-kernel outputs), element by element; an element whose
+reference value is 4 or larger, where one step of bf16 is already 0.031, may instead be one step off.
+fp32 results 1e-4 / 1e-5; integer outputs (argmax ids, cache positions) bit-exact.  The largest
+max-abs and rel-L2 every test saw are printed at the end of the run."""
 
 import math
 
@@ -28,11 +30,50 @@ def close(got: torch.Tensor, want: torch.Tensor, what: str = ""):
     return max_abs, rel
 
 
-def check(got, want, dtype, what=""):
+PARITY_LOG = {}  # test id -> [largest max-abs, largest rel-L2, checks]; printed by conftest's terminal summary
+
+
+def bf16_spacing(t: torch.Tensor) -> torch.Tensor:
+    """Distance between neighbouring bf16 values at each element's magnitude (8 significant bits)."""
+    a = t.detach().float().abs().clamp_min(2.0 ** -126)
+    return torch.exp2(torch.floor(torch.log2(a)) - 7)
+
+
+ULPS_SWIGLU = 3    # silu(gate) * up: two rounded factors, each of which may land one step off, and the product's own rounding
+# round(round(product) + residual): sums of bf16 products land on exact ties of the bf16 grid often; when the product is a
+# tie the two implementations' fp32 sums may break it differently (one step), and the sum with the residual is then a tie
+# again whose two break directions lie one more step apart (seen: -6.140625 -> -6.125 / -6.15625, + 1.671875 -> -4.4375 / -4.5)
+ULPS_RESIDUAL = 2
+# results behind several kernels in a row (a block, a small model's forward): an element's error no longer scales with the
+# element but with the sums it came from, so the step is taken at the largest magnitude of the element's row; four such
+# steps (largest seen: three, in the small bf16 models' latents behind 6 to 14 blocks)
+ULPS_COMPOSED = "4 steps at the row's largest magnitude"
+
+
+def check(got, want, dtype, what="", ulps=1, mag=None):
+    """bf16: every element within 2e-2 of the reference element or, where the reference element is so large that bf16
+    cannot resolve 2e-2 (|ref| >= 4: one step of the format is 0.031), within `ulps` steps of the format there; and
+    rel-L2 <= 1e-2.  `mag`: an intermediate that was rounded to bf16 on the way (the product in front of a residual add,
+    RMM:534-535); the step is then taken at the larger of the two magnitudes, since a one-step flip of the product
+    survives a cancelling add.  fp32: max-abs 1e-4 (times the largest reference magnitude when that exceeds 1), rel-L2 1e-5."""
     max_abs, rel = close(got, want, what)
-    lim_a, lim_r = (BF16_MAXABS, BF16_RELL2) if dtype == torch.bfloat16 else (F32_MAXABS, F32_RELL2)
-    scale = max(1.0, want.detach().float().abs().max().item())
-    assert max_abs <= lim_a * scale and rel <= lim_r, f"{what}: max-abs {max_abs:.3e} (scale {scale:.2f}), rel-L2 {rel:.3e}"
+    import os
+    rec = PARITY_LOG.setdefault(os.environ.get("PYTEST_CURRENT_TEST", "?").split(" ")[0], [0.0, 0.0, 0])
+    rec[0], rec[1], rec[2] = max(rec[0], max_abs), max(rec[1], rel), rec[2] + 1
+    if dtype == torch.bfloat16:
+        g, w = got.detach().float().cpu(), want.detach().float().cpu()
+        if ulps == ULPS_COMPOSED:
+            ulps, at = 4, w.abs().amax(dim=-1, keepdim=True).expand_as(w)
+        else:
+            at = w if mag is None else torch.maximum(w.abs(), mag.detach().float().cpu().abs())
+        bar = (ulps * bf16_spacing(at)).clamp_min(BF16_MAXABS)
+        over = (g - w).abs() > bar
+        worst = ((g - w).abs() / bar).max().item() if g.numel() else 0.0
+        assert not over.any() and rel <= BF16_RELL2, \
+            f"{what}: max-abs {max_abs:.3e}, {int(over.sum())} elements beyond max(2e-2, {ulps} bf16 ulp) (worst {worst:.2f} x the bar), rel-L2 {rel:.3e}"
+    else:
+        scale = max(1.0, want.detach().float().abs().max().item())
+        assert max_abs <= F32_MAXABS * scale and rel <= F32_RELL2, f"{what}: max-abs {max_abs:.3e} (scale {scale:.2f}), rel-L2 {rel:.3e}"
 
 
 def rnd(shape, dtype, seed, std=1.0, mean=0.0):
@@ -93,7 +134,7 @@ def test_gemm_bf16_all_row_counts(pkg, M):
     y = pkg.hip.gemm(x.cuda(), w.cuda())
     check(y, lin(x, w).to(dt), dt, f"gemm M={M}")
     yr = pkg.hip.gemm(x.cuda(), w.cuda(), residual=res.cuda())
-    check(yr, (lin(x, w).to(dt) + res), dt, f"gemm+residual M={M}")
+    check(yr, (lin(x, w).to(dt) + res), dt, f"gemm+residual M={M}", mag=lin(x, w), ulps=ULPS_RESIDUAL)
     yf = pkg.hip.gemm(x.cuda(), w.cuda(), out_f32=True)
     assert yf.dtype == torch.float32
     assert torch.equal(yf.cpu(), y.float().cpu()), "float store must be the upcast of the rounded result"
@@ -106,6 +147,41 @@ def test_gemm_bf16_nebel_shapes(pkg, M, N, K):
     x, w = rnd((M, K), dt, 40 + M), rnd((N, K), dt, 41, 0.02)
     y = pkg.hip.gemm(x.cuda(), w.cuda())
     check(y, lin(x, w).to(dt), dt, f"gemm {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("M", [1, 8, 32])
+def test_lm_head_product_at_decode_row_counts(pkg, M):
+    """The LM head of a decode step: [M, 5280] x [65536, 5280]^T with the float store (logits stay fp32, RMM:712-714),
+    at 1, 8 and 32 rows -- the widest product of a token (692 MB of weights, 32768 workgroups of the one-row kernel).
+    Against fp32 F.linear on the first and last 1024 vocabulary rows and 2048 rows in between."""
+    dt, N, K = torch.bfloat16, 65536, 5280
+    x = rnd((M, K), dt, 60 + M)
+    wd = torch.empty(N, K, dtype=dt, device="cuda").normal_(0.0, 0.02, generator=torch.Generator(device="cuda").manual_seed(61))
+    y = pkg.hip.gemm(x.cuda(), wd, out_f32=True)
+    assert y.dtype == torch.float32 and y.shape == (M, N)
+    cols = torch.cat([torch.arange(1024), torch.randperm(N - 2048, generator=torch.Generator().manual_seed(62))[:2048] + 1024,
+                      torch.arange(N - 1024, N)])
+    want = lin(x, wd[cols.cuda()].cpu()).to(dt)
+    check(y[:, cols.cuda()], want, dt, f"LM head M={M}")
+    assert torch.equal(y, y.to(dt).float()), "the float store holds the bf16-rounded product"
+    # every vocabulary row was written: the product against the device's own fp32 matmul over all 65536 columns
+    full = (x.cuda().float() @ wd.float().t()).to(dt)
+    check(y, full, dt, f"LM head M={M}, all columns")
+
+
+def test_embedding_at_the_full_vocabulary(pkg):
+    """raven_embed over the 65536 x 5280 table: first, last and random rows, scaled by sqrt(5280) in the table's dtype
+    (one rounding, RMM:672-675)."""
+    dt, V, h = torch.bfloat16, 65536, 5280
+    wd = torch.empty(V, h, dtype=dt, device="cuda").normal_(0.0, 0.02, generator=torch.Generator(device="cuda").manual_seed(63))
+    ids = torch.cat([torch.tensor([0, V - 1, 1, V - 2, 32768]), torch.randint(0, V, (59,), generator=torch.Generator().manual_seed(64))])
+    scale = math.sqrt(h)
+    got = pkg.hip.embed(wd, ids.cuda(), scale)
+    want = (wd[ids.cuda()].cpu() * scale)   # a bf16 tensor times a Python float: computed in fp32, rounded once
+    assert got.shape == (64, h) and torch.equal(got.cpu(), want)
+    wf = wd[:4096].float()
+    gf = pkg.hip.embed(wf, torch.tensor([0, 4095, 17]).cuda(), scale)
+    assert torch.equal(gf.cpu(), (wf[[0, 4095, 17]].cpu() * scale))
 
 
 @pytest.mark.parametrize("M", [1, 3, 8, 9, 40])
@@ -137,7 +213,7 @@ def test_gemm_swiglu(pkg, dt, M, I, K):
     z = lin(x, fc).to(dt)
     gate, up = z[:, :I], z[:, I:]
     want = F.silu(gate) * up
-    check(y, want, dt, "swiglu")
+    check(y, want, dt, "swiglu", ulps=ULPS_SWIGLU)
     wrong = F.silu(up) * gate
     assert close(y, wrong)[1] > 0.1, "the gate must be the first half"
 
@@ -155,10 +231,10 @@ def test_linear_with_workspace_nebel_shapes(pkg, tuned, M, ks):
     wqkv, proj, fc, mlp, ada = (rnd(sh, dt, 164 + i, 0.02) for i, sh in enumerate(((3 * h, h), (h, h), (2 * I, h), (h, I), (h, 2 * h))))
     dev = lambda t: t.cuda()
     check(pkg.hip.linear(dev(x), dev(wqkv), workspace=ws), lin(x, wqkv).to(dt), dt, "qkv")
-    check(pkg.hip.linear(dev(x), dev(proj), residual=dev(res), workspace=ws), lin(x, proj).to(dt) + res, dt, "proj + residual")
+    check(pkg.hip.linear(dev(x), dev(proj), residual=dev(res), workspace=ws), lin(x, proj).to(dt) + res, dt, "proj + residual", mag=lin(x, proj), ulps=ULPS_RESIDUAL)
     z = lin(x, fc).to(dt)
-    check(pkg.hip.linear(dev(x), dev(fc), swiglu=True, workspace=ws), F.silu(z[:, :I]) * z[:, I:], dt, "fc + swiglu")
-    check(pkg.hip.linear(dev(xi), dev(mlp), residual=dev(res), workspace=ws), lin(xi, mlp).to(dt) + res, dt, "mlp.proj + residual")
+    check(pkg.hip.linear(dev(x), dev(fc), swiglu=True, workspace=ws), F.silu(z[:, :I]) * z[:, I:], dt, "fc + swiglu", ulps=ULPS_SWIGLU)
+    check(pkg.hip.linear(dev(xi), dev(mlp), residual=dev(res), workspace=ws), lin(xi, mlp).to(dt) + res, dt, "mlp.proj + residual", mag=lin(xi, mlp), ulps=ULPS_RESIDUAL)
     check(pkg.hip.linear(dev(x), dev(ada), x1=dev(x1), workspace=ws), lin(torch.cat([x, x1], -1), ada).to(dt), dt, "adapter")
     yf = pkg.hip.linear(dev(x), dev(proj), out_f32=True, workspace=ws)
     assert yf.dtype == torch.float32 and torch.equal(yf, pkg.hip.linear(dev(x), dev(proj), workspace=ws).float())
@@ -203,7 +279,7 @@ def test_mfma_gemm_row_alignment_cases(pkg, tuned, M, four):
         x, fc = rnd((M, K), dt, 190), rnd((2 * I, K), dt, 191 + I, 0.05)
         z = lin(x, fc).to(dt)
         for wsp in (None, ws):
-            check(pkg.hip.linear(x.cuda(), fc.cuda(), swiglu=True, workspace=wsp), F.silu(z[:, :I]) * z[:, I:], dt, f"swiglu {M}x{I}x{K}")
+            check(pkg.hip.linear(x.cuda(), fc.cuda(), swiglu=True, workspace=wsp), F.silu(z[:, :I]) * z[:, I:], dt, f"swiglu {M}x{I}x{K}", ulps=ULPS_SWIGLU)
     for N, K0, K1 in ((64, 160, 160), (32, 288, 160), (64, 416, 416)):
         x0, x1, w = rnd((M, K0), dt, 195), rnd((M, K1), dt, 196), rnd((N, K0 + K1), dt, 197 + N, 0.05)
         for wsp in (None, ws):
@@ -219,8 +295,8 @@ def test_mfma_four_tile_variant_nebel_shapes(pkg, tuned, M):
     wqkv, fc, mlp = rnd((3 * h, h), dt, 233, 0.02), rnd((2 * I, h), dt, 234, 0.02), rnd((h, I), dt, 235, 0.02)
     check(pkg.hip.gemm(x.cuda(), wqkv.cuda()), lin(x, wqkv).to(dt), dt, "qkv")
     z = lin(x, fc).to(dt)
-    check(pkg.hip.gemm_swiglu(x.cuda(), fc.cuda()), F.silu(z[:, :I]) * z[:, I:], dt, "fc + swiglu")
-    check(pkg.hip.gemm(xi.cuda(), mlp.cuda(), residual=res.cuda()), lin(xi, mlp).to(dt) + res, dt, "mlp.proj + residual")
+    check(pkg.hip.gemm_swiglu(x.cuda(), fc.cuda()), F.silu(z[:, :I]) * z[:, I:], dt, "fc + swiglu", ulps=ULPS_SWIGLU)
+    check(pkg.hip.gemm(xi.cuda(), mlp.cuda(), residual=res.cuda()), lin(xi, mlp).to(dt) + res, dt, "mlp.proj + residual", mag=lin(xi, mlp), ulps=ULPS_RESIDUAL)
     yf = pkg.hip.gemm(x.cuda(), wqkv.cuda(), out_f32=True)
     assert yf.dtype == torch.float32 and torch.equal(yf, pkg.hip.gemm(x.cuda(), wqkv.cuda()).float())
 
@@ -246,11 +322,11 @@ def test_gemv_fused_one_row(pkg, dt, h, I):
     # norm_2 -> norm_3 -> fc with SwiGLU
     y, xa = pkg.hip.gemv_fused(dev(x), dev(fc), norm_a=dev(wa), norm_b=dev(wb), want_xa=True, swiglu=True)
     z = lin(xb_want, fc).to(dt)
-    check(y[None], F.silu(z[:, :I]) * z[:, I:], dt, "double norm + fc + swiglu")
+    check(y[None], F.silu(z[:, :I]) * z[:, I:], dt, "double norm + fc + swiglu", ulps=ULPS_SWIGLU)
     # long K with residual (mlp.proj) and the adapter's two operands
     g = rnd((I,), dt, 129)
     y, _ = pkg.hip.gemv_fused(dev(g), dev(mlp), residual=dev(res))
-    check(y[None], lin(g[None], mlp).to(dt) + res, dt, "mlp.proj + residual")
+    check(y[None], lin(g[None], mlp).to(dt) + res, dt, "mlp.proj + residual", mag=lin(g[None], mlp), ulps=ULPS_RESIDUAL)
     y, _ = pkg.hip.gemv_fused(dev(x), dev(ada), x1=dev(x1))
     check(y[None], lin(torch.cat([x, x1])[None], ada).to(dt), dt, "adapter")
     y, _ = pkg.hip.gemv_fused(dev(x), dev(ada), x1=dev(x1), norm_a=dev(wa))
@@ -415,7 +491,7 @@ def test_swiglu_elementwise(pkg):
     for dt, M, I in ((torch.bfloat16, 5, 17920), (torch.float32, 3, 704), (torch.bfloat16, 1, 8)):
         z = rnd((M, 2 * I), dt, 140)
         got = pkg.hip.swiglu(z.cuda())
-        check(got, F.silu(z[:, :I]) * z[:, I:], dt, "swiglu")
+        check(got, F.silu(z[:, :I]) * z[:, I:], dt, "swiglu", ulps=ULPS_SWIGLU)
         if dt == torch.bfloat16:
             assert bool((got.cpu() == F.silu(z[:, :I]) * z[:, I:]).float().mean() > 0.99)
 

@@ -1,7 +1,7 @@
 """GPU parity tests of the composed path: SandwichBlock, one recurrence iteration, the full forward and
 greedy decode, against the CPU oracle on identical seeded weights and injected latent states.
 
-Tolerances as in test_gpu_kernels.py (bf16: max-abs <= 2e-2 * max(1, |ref|_max), rel-L2 <= 1e-2) for
+Tolerances as in test_gpu_kernels.py (bf16: every element within max(2e-2, 1 bf16 ulp of the reference element), rel-L2 <= 1e-2) for
 single kernels and the tiny model; token ids and cache indexing bit-exact; fp32 greedy streams identical
 over 64 tokens.  A chain of several bf16 blocks amplifies 1-ulp rounding flips, so at the 3.5b shape the
 composed results are held to the oracle's own sensitivity to a change of accumulation order (the oracle
@@ -13,7 +13,7 @@ import pytest
 import torch
 
 from oracle import raven_oracle as O
-from test_gpu_kernels import check, close, rnd
+from test_gpu_kernels import ULPS_COMPOSED, check, close, rnd
 
 pytestmark = pytest.mark.gpu
 
@@ -264,7 +264,7 @@ def test_forward_tiny_bf16_matches_oracle(tiny16):
     states = O.initialize_state(torch.empty(2, 6, s.n_embd), s, 1.0, g).to(torch.bfloat16)
     want = O.forward(w, s, input_ids=ids, input_states=states)
     got = model(input_ids=ids.cuda(), input_states=states.cuda())
-    check(got.latent_states, want.latent_states, torch.bfloat16, "bf16 latents")
+    check(got.latent_states, want.latent_states, torch.bfloat16, "bf16 latents", ulps=ULPS_COMPOSED)
     check(got.logits, want.logits, torch.bfloat16, "bf16 logits")
 
 
@@ -281,7 +281,7 @@ def test_wide_prefill_path_bf16(pkg, tiny16, tuned, B, S):
     ref_cache, cache = O.DictCache(), pkg.HuginnDynamicCache()
     want = O.forward(w, s, input_ids=ids[:, :S], input_states=states[:, :S], past_key_values=ref_cache, use_cache=True)
     got = model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda(), past_key_values=cache, use_cache=True)
-    check(got.latent_states, want.latent_states, torch.bfloat16, "wide latents")
+    check(got.latent_states, want.latent_states, torch.bfloat16, "wide latents", ulps=ULPS_COMPOSED)
     check(got.logits, want.logits, torch.bfloat16, "wide logits")
     tuned(gemm_tiled_min_rows=1 << 30)
     narrow = model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda())
@@ -317,7 +317,7 @@ def test_decode_runner_beyond_one_pass_of_rows_bf16(pkg, tiny16, use_graph):
         fwd = model(input_ids=tok.cuda(), input_states=st.cuda(), past_key_values=cache2, use_cache=True, cache_position=pos.cuda())
         logits, nxt, lat = runner.step(tok.cuda(), st.cuda())
         check(logits, want.logits[:, 0], torch.bfloat16, f"runner logits, token {i}")
-        check(lat, want.latent_states[:, 0], torch.bfloat16, f"runner latents, token {i}")
+        check(lat, want.latent_states[:, 0], torch.bfloat16, f"runner latents, token {i}", ulps=ULPS_COMPOSED)
         # the same kernels as forward(); only the number of workgroups that share a sequence's positions follows the
         # cache capacity in the runner (its launch shapes must serve every later token) and the position in forward()
         check(logits, fwd.logits[:, 0], torch.bfloat16, f"token {i}: runner against forward()")
@@ -363,7 +363,7 @@ def test_forward_and_decode_with_test_time_noise(pkg, kind, dt):
     want = O.forward(w, s, input_ids=ids[:, :S], input_states=states[:, :S], past_key_values=ref_cache, use_cache=True,
                      noise_draws=ref_draws)
     got = model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda(), past_key_values=cache, use_cache=True)
-    check(got.latent_states, want.latent_states, dt, f"{kind} latents")
+    check(got.latent_states, want.latent_states, dt, f"{kind} latents", ulps=ULPS_COMPOSED)
     check(got.logits, want.logits, dt, f"{kind} logits")
     runner = pkg.DecodeRunner(model, cache, B, s.mean_recurrence, use_graph=True)
     assert not runner.use_graph
@@ -374,7 +374,7 @@ def test_forward_and_decode_with_test_time_noise(pkg, kind, dt):
                          noise_draws=ref_draws)
         logits, _, lat = runner.step(tok.cuda(), st.cuda())
         check(logits, want.logits[:, 0], dt, f"{kind} runner logits, token {i}")
-        check(lat, want.latent_states[:, 0], dt, f"{kind} runner latents, token {i}")
+        check(lat, want.latent_states[:, 0], dt, f"{kind} runner latents, token {i}", ulps=ULPS_COMPOSED)
     # without the noise the same model gives something else: the option is not silently ignored
     model.config.test_time_noise = 0.0
     plain = model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda())
@@ -395,10 +395,13 @@ def small242(pkg):
     return s, w, build_model(pkg, cfg, w, torch.float32)
 
 
-@pytest.mark.parametrize("strategy", ["full", "skip", "latest-m4", "available-m4", "always-last-m4", "latest-m4-compress-s4"])
+@pytest.mark.parametrize("strategy", ["full", "skip", "latest-m4", "available-m4", "always-last-m4", "latest-m4-compress-s4",
+                                      "latest-m4-compress-s16", "available-m4-compress-s8", "skip-compress-s8", "skip-compress-r4"])
 def test_partially_filled_cache_lookups_in_the_attention_kernels(pkg, small242, strategy):
     """Tokens computed with different numbers of recurrences (what per-token adaptive compute leaves behind): the
-    attention kernels resolve positions that are not cached at a step as HuginnDynamicCache.update does (RMM:199-253)."""
+    attention kernels resolve positions that are not cached at a step as HuginnDynamicCache.update does (RMM:199-253),
+    also when the steps share entries (compress-* remaps, RMM:169-182): a deeper token is then the first to reach some
+    shared entries, and recurrences past the remap's period overwrite the entries of earlier ones."""
     s, w, model = small242
     g = torch.Generator().manual_seed(11)
     B = 2
@@ -420,6 +423,63 @@ def test_partially_filled_cache_lookups_in_the_attention_kernels(pkg, small242, 
         assert sorted(cache.key_cache[step].keys()) == sorted(ref_cache.key_cache[step].keys()), step
         for p, kref in ref_cache.key_cache[step].items():
             check(cache.key_cache[step][p], kref, torch.float32, f"{strategy}: K[{step}][{p}]")
+    assert cache.get_memory_usage() == ref_cache.get_memory_usage()
+
+
+SHARED_ENTRIES = {"compress-s16": 16, "latest-m4-compress-s16": 16, "compress-r4": 10, "compress-anchor": 36}
+
+
+@pytest.mark.parametrize("runner", [False, True])
+@pytest.mark.parametrize("strategy", list(SHARED_ENTRIES))
+def test_cache_sharing_remaps_through_the_forward_and_the_decode_runner(pkg, small242, strategy, runner):
+    """The reference's cache-sharing strategies (RMM:169-182) through the HIP forward, ten recurrences so that every remap
+    differs from `full`: compress-s16 walks its 16 shared entries two and a half times, compress-r4 folds the four blocks
+    of a recurrence into one entry (each block overwrites and then reads what the block before it left there for the older
+    positions), compress-anchor keeps eight recurrences apart and shares four entries among the rest.  A 6-token prompt,
+    then single tokens (through forward(), or through the decode runner's fixed launch sequence) against the oracle's dict
+    cache with the same strategy: logits, greedy ids, which entries exist, what they hold, and the cache size."""
+    s, w, model = small242
+    g = torch.Generator().manual_seed(31)
+    B, n0, r, h = 2, 6, 10, s.n_embd
+    ref_cache, cache = O.DictCache(strategy), pkg.HuginnDynamicCache(strategy, max_length=16)
+    ids = torch.randint(0, s.vocab_size, (B, n0), generator=g)
+    states = O.initialize_state(torch.empty(B, n0, h), s, 1.0, g)
+    want = O.forward(w, s, input_ids=ids, input_states=states, past_key_values=ref_cache, use_cache=True, cache_position=torch.arange(n0),
+                     num_steps=r)
+    got = model(input_ids=ids.cuda(), input_states=states.cuda(), past_key_values=cache, use_cache=True,
+                cache_position=torch.arange(n0).cuda(), num_steps=r)
+    err = close(got.logits, want.logits, f"{strategy}: prompt logits")
+    assert err[0] <= 1e-4 and err[1] <= 5e-5, (strategy, err)
+    dr = pkg.DecodeRunner(model, cache, B, r, greedy=True, use_graph=False) if runner else None
+    tok = want.logits[:, -1].argmax(-1)
+    for i in range(4):
+        st = O.initialize_state(torch.empty(B, 1, h), s, 1.0, g)
+        cp = torch.tensor([n0 + i])
+        want = O.forward(w, s, input_ids=tok[:, None], input_states=st, past_key_values=ref_cache, use_cache=True, cache_position=cp,
+                         num_steps=r)
+        if runner:
+            logits, nxt, lat = dr.step(tok.cuda(), st.view(B, h).cuda())
+            err = close(lat, want.latent_states[:, 0], f"{strategy}: runner latents, token {i}")
+            assert err[0] <= 1e-4 and err[1] <= 5e-5, (strategy, i, err)
+        else:
+            out = model(input_ids=tok[:, None].cuda(), input_states=st.cuda(), past_key_values=cache, use_cache=True,
+                        cache_position=cp.cuda(), num_steps=r)
+            logits, nxt = out.logits[:, -1], out.logits[:, -1].argmax(-1)
+        # behind ten recurrences (42 blocks): the per-kernel fp32 differences (1e-6) have grown by an order of magnitude
+        err = close(logits, want.logits[:, -1], f"{strategy}: logits of token {i}")
+        assert err[0] <= 1e-4 and err[1] <= 5e-5, (strategy, i, err)
+        tok = want.logits[:, -1].argmax(-1)
+        assert torch.equal(nxt.cpu(), tok)
+    assert cache.get_seq_length() == ref_cache.get_seq_length() == n0 + 4
+    core_entries = [k for k in ref_cache.key_cache if k >= 2]
+    assert len(core_entries) == SHARED_ENTRIES[strategy] < 4 * r     # the remap really shares entries
+    assert sorted(cache.key_cache.keys()) == sorted(ref_cache.key_cache.keys())
+    for step in ref_cache.key_cache:
+        assert sorted(cache.key_cache[step].keys()) == sorted(ref_cache.key_cache[step].keys()), step
+        for p, kref in ref_cache.key_cache[step].items():
+            for got_e, want_e in ((cache.key_cache[step][p], kref), (cache.value_cache[step][p], ref_cache.value_cache[step][p])):
+                err = close(got_e, want_e, f"{strategy}: entry [{step}][{p}]")
+                assert err[0] <= 1e-4 * max(1.0, want_e.abs().max().item()) and err[1] <= 5e-5, (strategy, step, p, err)
     assert cache.get_memory_usage() == ref_cache.get_memory_usage()
 
 
@@ -709,7 +769,7 @@ def test_paged_forward_tokens_prompt_chunks_and_decode_rows_together(pkg, layout
     one = pkg.PagedDecoder(model, num_blocks=n_blocks, block_size=bs, num_steps=1, layout=layout)
     want = O.forward(w, s, input_ids=prompts[2], input_states=states[2][:, :lens[2]], num_steps=1)
     logits, latents = one.prefill_paged(prompts[2].cuda(), table[2].tolist(), input_states=states[2][:, :lens[2]].cuda())
-    check(latents, want.latent_states[0], dt, "one recurrence, latents")
+    check(latents, want.latent_states[0], dt, "one recurrence, latents", ulps=ULPS_COMPOSED)
     check(logits, want.logits[0], dt, "one recurrence, logits")
 
     # (2) a mixed step on fresh pages: sequence 0 has its prompt cached and decodes one row, sequence 1 has 20 rows cached

@@ -14,7 +14,7 @@ import torch
 import torch.nn.functional as F
 
 from oracle import raven_oracle as O
-from test_gpu_kernels import check, close, rnd
+from test_gpu_kernels import ULPS_COMPOSED, ULPS_RESIDUAL, ULPS_SWIGLU, check, close, rnd
 
 pytestmark = pytest.mark.gpu
 
@@ -47,6 +47,7 @@ def test_tiled_gemm_nebel_shapes_m16384(pkg, name):
     """RMM:463, 493, 507-509, 776, 711 at 16384 token rows: the tiled kernel with each product's epilogue."""
     dt, M = torch.bfloat16, 16384
     rows = _rows(M).cuda()
+    kw = {}
     if name == "Wqkv":
         x, w = _gpu_randn((M, H), 1), _gpu_randn((3 * H, H), 2, 0.02)
         got = pkg.hip.linear(x, w)
@@ -55,6 +56,7 @@ def test_tiled_gemm_nebel_shapes_m16384(pkg, name):
         x, w, res = _gpu_randn((M, H), 3), _gpu_randn((H, H), 4, 0.02), _gpu_randn((M, H), 5)
         got = pkg.hip.linear(x, w, residual=res)
         want = (_ref_rows(x, w, rows).to(dt).float() + res[rows].float()).to(dt)
+        kw = dict(mag=_ref_rows(x, w, rows), ulps=ULPS_RESIDUAL)
     elif name == "mlp.fc":
         x, w = _gpu_randn((M, H), 6), _gpu_randn((2 * INTER, H), 7, 0.02)
         got = pkg.hip.linear(x, w, swiglu=True)
@@ -62,10 +64,12 @@ def test_tiled_gemm_nebel_shapes_m16384(pkg, name):
         want = (F.silu(z[:, :INTER]).to(dt).float() * z[:, INTER:]).to(dt)
         wrong = (F.silu(z[:, INTER:]).to(dt).float() * z[:, :INTER]).to(dt)
         assert close(got[rows], wrong)[1] > 0.1, "the gate must be the first half of fc's output"
+        kw = dict(ulps=ULPS_SWIGLU)
     elif name == "mlp.proj":
         x, w, res = _gpu_randn((M, INTER), 8), _gpu_randn((H, INTER), 9, 0.02), _gpu_randn((M, H), 10)
         got = pkg.hip.linear(x, w, residual=res)
         want = (_ref_rows(x, w, rows).to(dt).float() + res[rows].float()).to(dt)
+        kw = dict(mag=_ref_rows(x, w, rows), ulps=ULPS_RESIDUAL)
     elif name == "adapter":
         x0, x1, w = _gpu_randn((M, H), 11), _gpu_randn((M, H), 12), _gpu_randn((H, 2 * H), 13, 0.02)
         got = pkg.hip.linear(x0, w, x1=x1)
@@ -79,7 +83,7 @@ def test_tiled_gemm_nebel_shapes_m16384(pkg, name):
         got = pkg.hip.gemm(x, w, out_f32=True)
         assert got.dtype == torch.float32
         want = _ref_rows(x, w, rows).to(dt).float()
-    check(got[rows], want, dt, f"{name} at {M} rows")
+    check(got[rows], want, dt, f"{name} at {M} rows", **kw)
     assert torch.isfinite(got.float()).all()
 
 
@@ -94,13 +98,13 @@ def test_tiled_gemm_edges_against_oracle(pkg, tuned, variant, M, N, K):
     dev = lambda t: t.cuda()
     lin = lambda a, b: F.linear(a.float(), b.float())
     check(pkg.hip.linear(dev(x), dev(w)), lin(x, w).to(dt), dt, "plain")
-    check(pkg.hip.linear(dev(x), dev(w), residual=dev(res)), lin(x, w).to(dt) + res, dt, "+ residual")
+    check(pkg.hip.linear(dev(x), dev(w), residual=dev(res)), lin(x, w).to(dt) + res, dt, "+ residual", mag=lin(x, w), ulps=ULPS_RESIDUAL)
     yf = pkg.hip.linear(dev(x), dev(w), out_f32=True)
     assert yf.dtype == torch.float32 and torch.equal(yf, pkg.hip.linear(dev(x), dev(w)).float())
     if N % 16 == 0:
         fc = rnd((2 * N, K), dt, 503, 0.05)
         z = lin(x, fc).to(dt)
-        check(pkg.hip.linear(dev(x), dev(fc), swiglu=True), F.silu(z[:, :N]) * z[:, N:], dt, "SwiGLU")
+        check(pkg.hip.linear(dev(x), dev(fc), swiglu=True), F.silu(z[:, :N]) * z[:, N:], dt, "SwiGLU", ulps=ULPS_SWIGLU)
     x1, w2 = rnd((M, K), dt, 504), rnd((N, 2 * K), dt, 505, 0.05)
     check(pkg.hip.linear(dev(x), dev(w2), x1=dev(x1)), lin(torch.cat([x, x1], -1), w2).to(dt), dt, "two operands")
     # against the oracle's own statement of the products (nn.Linear in bf16 on the CPU; small shapes only: it is slow)
@@ -243,7 +247,7 @@ def test_sandwich_block_config4_rows(pkg):
         O.set_linear_mode("native")
     got = out.view(B, S, H)[b][rows.cuda()]
     # the cache rows the block appended: rotated keys and values of every position, one kernel chain deep
-    check(kd[0, b].transpose(0, 1), k_rot[0], dt, "appended K of the sequence")
+    check(kd[0, b].transpose(0, 1), k_rot[0], dt, "appended K of the sequence", ulps=ULPS_COMPOSED)
     check(vd[0, b].transpose(0, 1), v_all[0], dt, "appended V of the sequence")
     err = close(got, want, "block output rows")
     print(f"SandwichBlock at 4 x 4096: sampled rows max-abs {err[0]:.3e} rel-L2 {err[1]:.3e}")

@@ -149,17 +149,33 @@ def test_static_cache_known_answer_and_interface(pkg):
     assert s16.max_num_steps == 20
 
 
-@pytest.mark.parametrize("strategy", ["full", "skip", "latest-m4", "available-m4", "always-last-m4", "latest-m4-compress-s4"])
+@pytest.mark.parametrize("strategy", ["full", "skip", "latest-m4", "available-m4", "always-last-m4", "latest-m4-compress-s4",
+                                      "latest-m4-compress-s16", "available-m4-compress-s8", "skip-compress-r4", "latest-m4-compress-r2",
+                                      "available-m4-compress-r4", "latest-m4-compress-anchor", "skip-compress-anchor"])
 def test_cache_lookups_with_partially_filled_steps_match_dict_model(pkg, strategy):
     """Tokens computed with different numbers of recurrences: every update of the contiguous cache returns what the
-    brute-force dict model of the reference's cache returns (RMM:199-253)."""
+    brute-force dict model of the reference's cache returns (RMM:199-253), also when steps share entries (the
+    compress-* remaps, RMM:169-182: a deeper token then finds shallower tokens missing at the shared entries it is
+    the first to reach, and later recurrences overwrite the entries of earlier ones)."""
     g = torch.Generator().manual_seed(5)
     ours, ref = pkg.HuginnDynamicCache(strategy), O.DictCache(strategy)
-    # (new tokens, recurrences): a prefill, then single tokens that stop earlier or go deeper
-    for n_new, r in ((5, 3), (1, 1), (1, 4), (2, 2), (1, 6), (1, 3)):
+    # (new tokens, recurrences): a prefill, then single tokens that stop earlier or go deeper; 9 and 11 recurrences reach
+    # past the 8 recurrences compress-anchor keeps apart
+    schedule = ((5, 3), (1, 1), (1, 4), (2, 2), (1, 6), (1, 3))
+    if "anchor" in strategy or "compress-s16" in strategy:
+        schedule += ((1, 9), (2, 5), (1, 11), (1, 8))
+    for n_new, r in schedule:
         for step in [0, 1] + list(range(2, 2 + 4 * r)) + [-1, -2]:
             k, v = torch.randn(2, 3, n_new, 8, generator=g), torch.randn(2, 3, n_new, 8, generator=g)
-            got, want = ours.update(k, v, step), ref.update(k, v, step)
+            try:
+                want = ref.update(k, v, step)
+            except ValueError:
+                # the reference's max() over an empty list: an older position holds no entry of this block at all (the
+                # compress-r remaps put whole recurrences into single entries); the contiguous cache refuses it too
+                with pytest.raises(ValueError):
+                    ours.update(k, v, step)
+                return
+            got = ours.update(k, v, step)
             assert got[0].shape == want[0].shape, (strategy, step, got[0].shape, want[0].shape)
             assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]), (strategy, step)
         assert ours.get_seq_length() == ref.get_seq_length()
