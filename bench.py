@@ -124,6 +124,7 @@ def prefill_record(pkg, model, B, S, r):
     model.iterate_forward(embeds, state, block_idx=block_idx, past_key_values=cache, num_steps=1)
     cache.lookup_strategy = "full"
     cache._filled = {k: v for k, v in cache._filled.items() if k < cfg.n_layers_in_prelude}
+    cache._core = type(cache._core)()   # forget the warm-up's core steps: the timed run writes them again
     torch.cuda.synchronize()
     a.record()
     model.iterate_forward(embeds, state, block_idx=block_idx, past_key_values=cache, num_steps=r)

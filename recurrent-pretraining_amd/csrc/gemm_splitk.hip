@@ -97,7 +97,9 @@ __global__ __launch_bounds__(256) void mfma_ns_kernel(NsArgs a) {
     // macro-steps of 128 k-values over the (up to two) X segments; this workgroup's share of them
     const int mac0 = (a.k0 - shift0) / 128, mac1 = (a.k1 - shift1) / 128;
     const int n_mac = mac0 + mac1;
-    const int mb = (int)((int64_t)n_mac * blockIdx.y / a.ks), me = (int)((int64_t)n_mac * (blockIdx.y + 1) / a.ks);
+    // (the division runs on the vector unit: readfirstlane tells the compiler that the result is the same in every lane)
+    const int mb = __builtin_amdgcn_readfirstlane((int)((int64_t)n_mac * blockIdx.y / a.ks));
+    const int me = __builtin_amdgcn_readfirstlane((int)((int64_t)n_mac * (blockIdx.y + 1) / a.ks));
 
     f32x4 acc[NT][MT];
 #pragma unroll
@@ -105,38 +107,52 @@ __global__ __launch_bounds__(256) void mfma_ns_kernel(NsArgs a) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const bf16* wrow[NT][4];  // this lane's chunk column in each of the rows it loads
+    int64_t wrow[NT][4];  // element offset of this lane's chunk column in each of the rows it loads
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) wrow[t][i] = a.w + (int64_t)(tile_row0[t] + (4 * i + lr) * rs) * K + lc;
-    u32x4 xr[MT], wr[NT][4];
-    auto fetch = [&](int mac) {  // global -> registers
+        for (int i = 0; i < 4; ++i) wrow[t][i] = (int64_t)(tile_row0[t] + (4 * i + lr) * rs) * K + lc;
+    // D register sets: the loads of D macro-steps are in flight per wave.  A K slice is short (5 macro-steps for attn.proj of
+    // the 3.5b shape with 8 slices), so with one set in flight a workgroup's life was one memory latency per step.
+    constexpr int D = SWIGLU ? 2 : 4;
+    struct Set {
+        u32x4 x[MT], w[NT][4];
+    };
+    Set st[D];
+    const int n_steps = me - mb;
+    const int xrow = threadIdx.x >> 4, xc = (threadIdx.x & 15) * 8;
+    // global -> registers.  Steps past the end of the slice load the first elements of X and W instead, which every
+    // workgroup keeps hitting in the cache: the offsets are selected, not the loads, so that the loop body has no branch
+    // around a load and the waits the compiler inserts count only the loads of the set being parked
+    auto fetch = [&](int step, Set& set) {
+        const bool live = step < n_steps;
+        const int mac = mb + (live ? step : 0);
         const bool s1 = mac >= mac0;
         const bf16* X = s1 ? a.x1 : a.x0;
         const int ldx = s1 ? a.k1 : a.k0;
         const int kx = s1 ? shift1 + (mac - mac0) * 128 : shift0 + mac * 128;  // column inside the segment
         const int kw = (s1 ? a.k0 : 0) + kx;            // column of W
-        const int xrow = threadIdx.x >> 4, xc = (threadIdx.x & 15) * 8;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int m = min(mt * 16 + xrow, a.M - 1);  // rows past M repeat the last one; never stored
-            xr[mt] = *reinterpret_cast<const u32x4*>(X + (int64_t)m * ldx + kx + xc);
+            const int64_t off = live ? (int64_t)m * ldx + kx + xc : (int64_t)(xc + 128 * mt);  // distinct, or the compiler merges the idle loads and branches
+            set.x[mt] = *reinterpret_cast<const u32x4*>(X + off);
         }
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                wr[t][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[t][i] + kw));
+            for (int i = 0; i < 4; ++i) {
+                const int64_t off = live ? wrow[t][i] + kw : (int64_t)(lc + 128 * (4 * t + i));
+                set.w[t][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.w + off));
+            }
     };
-    auto park = [&](int buf) {  // registers -> LDS
-        const int xrow = threadIdx.x >> 4, xc = (threadIdx.x & 15) * 8;
+    auto park = [&](const Set& set, int buf) {  // registers -> LDS
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<u32x4*>(&xs[buf][mt * 16 + xrow][xc]) = xr[mt];
+        for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<u32x4*>(&xs[buf][mt * 16 + xrow][xc]) = set.x[mt];
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&wsm[wave][t * 16 + 4 * i + lr][lc]) = wr[t][i];
+            for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&wsm[wave][t * 16 + 4 * i + lr][lc]) = set.w[t][i];
     };
     auto multiply = [&](int buf) {
 #pragma unroll
@@ -161,18 +177,23 @@ __global__ __launch_bounds__(256) void mfma_ns_kernel(NsArgs a) {
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     };
-    if (mb < me) {
-        fetch(mb);
-        park(0);
+    if (n_steps > 0) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) fetch(d, st[d]);
     }
-    __syncthreads();
-    for (int mac = mb; mac < me; ++mac) {
-        const int buf = (mac - mb) & 1;
-        if (mac + 1 < me) fetch(mac + 1);  // in flight while this step is multiplied
-        multiply(buf);
-        wave_sync();                       // this wave is done with its own weight tile
-        if (mac + 1 < me) park(buf ^ 1);   // xs[buf ^ 1] was last read before the previous barrier
-        __syncthreads();                   // the new X tile is visible; nobody still reads xs[buf]
+    // step s parks into xs[s & 1] before its barrier and multiplies out of it behind the barrier; the buffer it overwrites
+    // was last read in step s - 2, which every wave has left when it passed the barrier of step s - 1.  The loop runs in
+    // rounds of D steps; the steps of the last round that lie past the slice park their idle loads and skip the products,
+    // so that every round issues the same loads in the same order (and the compiler's wait counts stay exact)
+    for (int s0 = 0; s0 < n_steps; s0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            park(st[d], d & 1);         // D is even: step s0 + d has the parity of d
+            fetch(s0 + d + D, st[d]);
+            __syncthreads();
+            if (s0 + d < n_steps) multiply(d & 1);
+            wave_sync();                // this wave is done with its own weight tile
+        }
     }
 
     // k-values in front of the first and behind the last full macro-step of each segment (32 for K = 5280):
@@ -264,8 +285,11 @@ static int launch_ns(NsArgs a, void* workspace, size_t workspace_bytes, hipStrea
     const int blocks = (a.N / 16 + 4 * rs - 1) / (4 * rs) * rs;
     const int n_mac = a.k0 / 128 + a.k1 / 128;
     const int n_total = SWIGLU ? 2 * a.N : a.N;
-    // enough workgroups for every CU to hold two or three, at least four macro-steps per slice
-    int ks = g_linear_ks > 0 ? g_linear_ks : (ns_cus() * 5 / 2 + blocks - 1) / blocks;
+    // As few K slices as give every CU a workgroup (84 tile groups x 3 slices = 252 for the 5280-row products of the 3.5b
+    // shape), at least four macro-steps per slice.  With four macro-steps of loads in flight per wave one workgroup keeps
+    // a CU's memory pipe busy, and the launch then ends in one round: us per product (both launches) at 32 rows with
+    // 2 / 3 / 5 / 6 / 8 slices: attn.proj 20.6 / 18.6 / 22.6 / 21.7 / 25.8, mlp.proj 45.2 / 37.4 / 43.2 / 41.7 / 45.9
+    int ks = g_linear_ks > 0 ? g_linear_ks : (ns_cus() * 9 / 10 + blocks - 1) / blocks;
     if (ks > n_mac / 4) ks = n_mac / 4;
     if (ks > 8) ks = 8;
     if (ks < 1) ks = 1;

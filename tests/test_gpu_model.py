@@ -995,8 +995,8 @@ def test_core_iteration_nebel_bf16_config3(pkg, nebel_core, B):
     assert min(err, err_alt) <= max(1.5 * floor, 1e-2) and err <= 5e-2
     # the new key/value rows landed at position T of each slot; slot 0 is one kernel chain deep and is
     # held to the per-kernel bar, the later slots sit behind 1-3 whole blocks (see the note on chains above)
-    check(kd[0, :, :, T], ref_cache.key_cache[2][T], dt, "appended K slot 0")
-    check(vd[0, :, :, T], ref_cache.value_cache[2][T], dt, "appended V slot 0")
+    check(kd[0, :, :, T], ref_cache.key_cache[2][T], dt, "appended K slot 0", ulps=ULPS_COMPOSED)   # adapter -> norm_1 -> Wqkv -> bias, RoPE
+    check(vd[0, :, :, T], ref_cache.value_cache[2][T], dt, "appended V slot 0", ulps=ULPS_COMPOSED)
     for j in range(1, 4):
         assert close(kd[j, :, :, T], ref_cache.key_cache[2 + j][T])[1] <= 5e-2, f"appended K slot {j}"
         assert close(vd[j, :, :, T], ref_cache.value_cache[2 + j][T])[1] <= 5e-2, f"appended V slot {j}"
@@ -1114,8 +1114,8 @@ def test_core_iterations_nebel_one_row_real_weights(pkg, nebel_core):
     for it in range(r):
         pkg.hip.core_iteration(dims, dev["transformer.adapter.weight"], blocks, x, embeds, one, freqs, cache2, slots[it][0], 1, 1, T, ws)
         x = one.clone()
-    check(kd[0, :, :, T], kd2[0, :, :, T], dt, "first recurrence, first block: appended K")
-    check(vd[0, :, :, T], vd2[0, :, :, T], dt, "first recurrence, first block: appended V")
+    check(kd[0, :, :, T], kd2[0, :, :, T], dt, "first recurrence, first block: appended K", ulps=ULPS_COMPOSED)
+    check(vd[0, :, :, T], vd2[0, :, :, T], dt, "first recurrence, first block: appended V", ulps=ULPS_COMPOSED)
     err = close(many, one, "state after three recurrences")[1]
     err2 = close(kd[4, :, :, T], kd2[4, :, :, T], "second recurrence, first block: appended K")[1]
     print(f"core_iterations(3) vs 3 x core_iteration at h=5280, one row: rel-L2 {err:.3e} (K behind one recurrence: {err2:.3e})")
