@@ -27,6 +27,23 @@ int gemv1_column_block(const void* x, const void* norm_a, const void* w_block, i
 int linear_column_block(const void* x, const void* w_block, int ldw, const float* extra, void* y, int raw_out, int M, int N, int K,
                         void* workspace, size_t workspace_bytes, hipStream_t s);
 
+int linear_leave_sums(const void* x0, const void* x1, const void* w, int ldw, const float* extra, const void* residual, void* y, int M,
+                      int N, int K0, int K1, int dtype, void* workspace, size_t workspace_bytes, hipStream_t s, int* ks_left);
+
+int splitk_sums_then_norm(const float* partial, int ks, const float* extra, const void* residual, void* sum_out, const void* weight,
+                          void* y, const void* weight2, void* y2, int rows, int dim, float eps, hipStream_t s);
+
+// y = round(round(x W^T) + residual), then RMSNorm(weight) -> out1 and RMSNorm(weight2) of that -> out2 (either may be
+// null): two launches where the product is K-split (the norm launch adds the slices), three otherwise
+static int linear_then_norm(const void* x, const void* w, const void* residual, void* y, const void* weight, void* out1,
+                            const void* weight2, void* out2, int M, int N, int K, float eps, int dtype, void* ws, size_t ws_bytes,
+                            hipStream_t s) {
+    int ks = 0;
+    if (int rc = linear_leave_sums(x, nullptr, w, 0, nullptr, residual, y, M, N, K, 0, dtype, ws, ws_bytes, s, &ks)) return rc;
+    if (ks) return splitk_sums_then_norm(static_cast<const float*>(ws), ks, nullptr, residual, nullptr, weight, out1, weight2, out2, M, N, eps, s);
+    return raven_rmsnorm_residual(y, nullptr, weight, out1, nullptr, weight2, out2, M, N, eps, dtype, s);
+}
+
 struct BlockScratch {
     char *n1, *qkv, *q, *ya, *x1, *x2, *n3, *g, *x3, *xa, *xr;
     float* e_sums;  // up to 32 rows: fp32 sums of the adapter's embedding half, computed once for all recurrences
@@ -118,11 +135,10 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
         else rc = raven_decode_attention(s.q, s.ya, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream);
         if (rc) return rc;
     }
-    if ((rc = raven_linear(s.ya, nullptr, w->proj, x_in, s.x1, M, h, h, 0, 0, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
-    if ((rc = raven_rmsnorm_residual(s.x1, nullptr, w->norm_2, s.x2, nullptr, w->norm_3, s.n3, M, h, d->eps, dt, stream))) return rc;
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    if ((rc = linear_then_norm(s.ya, w->proj, x_in, s.x1, w->norm_2, s.x2, w->norm_3, s.n3, M, h, h, d->eps, dt, s.lin_ws, s.lin_ws_bytes, hs))) return rc;
     if ((rc = raven_linear(s.n3, nullptr, w->fc, nullptr, s.g, M, I, h, 0, 1, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
-    if ((rc = raven_linear(s.g, nullptr, w->mlp_proj, s.x2, s.x3, M, h, I, 0, 0, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
-    return raven_rmsnorm_residual(s.x3, nullptr, w->norm_4, y_out, nullptr, tail_w, tail_out, M, h, d->eps, dt, stream);
+    return linear_then_norm(s.g, w->mlp_proj, s.x2, s.x3, w->norm_4, y_out, tail_w, tail_out, M, h, I, d->eps, dt, s.lin_ws, s.lin_ws_bytes, hs);
 }
 
 // One row.  x_raw is the block input before `pre_norm` (the previous block's norm_4, or null when x_raw is
@@ -259,10 +275,18 @@ static int iterations_impl(const char* who, const raven_dims* dims, const void* 
         const bool last_it = it == n_iterations - 1;
         // the adapter product consumes the state before the last block of this iteration overwrites state_out
         const void* st = it == 0 ? state_in : state_out;
+        bool n1_ready = false;  // scratch.n1 holds norm_1 of the first block's input
         if (adapter_w) {
-            if (split) rc = linear_column_block(st, adapter_w, 2 * h, s.e_sums, s.xa, 0, M, h, h, s.lin_ws, s.lin_ws_bytes, hs);
-            else rc = raven_linear(st, embeds, adapter_w, nullptr, s.xa, M, h, h, h, 0, 0, dims->dtype, s.lin_ws, s.lin_ws_bytes, stream);
+            // where the product is K-split, the launch that adds its slices also applies the first block's norm_1
+            int ks = 0;
+            if (split) rc = linear_leave_sums(st, nullptr, adapter_w, 2 * h, s.e_sums, nullptr, s.xa, M, h, h, 0, dims->dtype, s.lin_ws, s.lin_ws_bytes, hs, &ks);
+            else rc = linear_leave_sums(st, embeds, adapter_w, 0, nullptr, nullptr, s.xa, M, h, h, h, dims->dtype, s.lin_ws, s.lin_ws_bytes, hs, &ks);
             if (rc) return rc;
+            if (ks) {
+                if ((rc = splitk_sums_then_norm(static_cast<const float*>(s.lin_ws), ks, split ? s.e_sums : nullptr, nullptr, s.xa, blocks[0].norm_1,
+                                                s.n1, nullptr, nullptr, M, h, dims->eps, hs))) return rc;
+                n1_ready = true;
+            }
         }
         const void* lnw = last_it ? ln_f : nullptr;
         for (int j = 0; j < n_blocks; ++j) {
@@ -271,7 +295,7 @@ static int iterations_impl(const char* who, const raven_dims* dims, const void* 
             void* y_out = last ? (lnw ? nullptr : state_out) : s.xa;
             const void* tail_w = last ? lnw : blocks[j + 1].norm_1;
             void* tail_out = last ? (lnw ? state_out : nullptr) : s.n1;
-            if ((rc = run_block(dims, &blocks[j], s, j > 0, x_in, y_out, tail_w, tail_out, freqs, cache, sl ? sl[j] : 0, B, S, pos0,
+            if ((rc = run_block(dims, &blocks[j], s, j > 0 || n1_ready, x_in, y_out, tail_w, tail_out, freqs, cache, sl ? sl[j] : 0, B, S, pos0,
                                 pos_dev, stream, paged, j))) return rc;
         }
     }

@@ -275,8 +275,10 @@ static int ns_cus() {
 int g_linear_min_rows = 1;  // raven_set_tuning("linear_min_rows"): up to this many rows go to the kernels without a workspace
 int g_linear_ks = 0;  // raven_set_tuning("linear_ks"): K slices per weight tile, 0 = choose from the grid size
 
+// ks_left (may be null): the caller adds the K slices itself (rmsnorm.hip, splitk_sums_then_norm); receives their number,
+// 0 when the product was finished here
 template <bool SWIGLU>
-static int launch_ns(NsArgs a, void* workspace, size_t workspace_bytes, hipStream_t s) {
+static int launch_ns(NsArgs a, void* workspace, size_t workspace_bytes, hipStream_t s, int* ks_left = nullptr) {
     // tiles of one row parity when the row pitch is an odd multiple of 64 bytes (needs whole pairs of tiles)
     if (a.ldw == 0) a.ldw = a.K;
     a.row_stride = ((a.ldw * 2) % 128 == 64 && a.N % 32 == 0) ? 2 : 1;
@@ -306,7 +308,8 @@ static int launch_ns(NsArgs a, void* workspace, size_t workspace_bytes, hipStrea
     const dim3 grid(blocks, ks);
     if (a.M <= 16) mfma_ns_kernel<1, SWIGLU><<<grid, dim3(256), 0, s>>>(a);
     else mfma_ns_kernel<2, SWIGLU><<<grid, dim3(256), 0, s>>>(a);
-    if (ks > 1) {
+    if (ks_left) *ks_left = ks > 1 ? ks : 0;
+    if (ks > 1 && !ks_left) {
         const int64_t n_out = (int64_t)a.M * a.N;
         splitk_finalize_kernel<SWIGLU><<<dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s>>>(a);
     }
@@ -329,6 +332,33 @@ int linear_column_block(const void* x, const void* w_block, int ldw, const float
     a.y = y;
     a.M = M; a.N = N; a.K = K; a.k0 = K; a.k1 = 0; a.ldw = ldw; a.extra = extra; a.raw_out = raw_out;
     return launch_ns<false>(a, workspace, workspace_bytes, s);
+}
+
+int g_fuse_sums_norm = 1;  // raven_set_tuning("fuse_sums_norm"): 0 = a K-split product always adds its slices in a launch of its own
+
+// A product whose result goes straight into an RMSNorm launch: y = round(round(x W^T [+ extra]) + residual) for at most 32
+// bf16 rows, W either a whole [N, K0 + K1] matrix (ldw = 0) or a column block with row pitch ldw (K1 = 0).  When the product
+// takes the K-split kernel, its slices are left in the workspace un-added (*ks_left slices, to be handed to
+// splitk_sums_then_norm before anything else uses the workspace) and y is not written; otherwise the product is finished
+// into y and *ks_left is 0.
+int linear_leave_sums(const void* x0, const void* x1, const void* w, int ldw, const float* extra, const void* residual, void* y, int M,
+                      int N, int K0, int K1, int dtype, void* workspace, size_t workspace_bytes, hipStream_t s, int* ks_left) {
+    *ks_left = 0;
+    bool split = g_fuse_sums_norm && dtype == RAVEN_BF16 && M >= 2 && M <= 32 && N % 16 == 0 && N <= 8192 && K0 % 32 == 0 && K1 % 32 == 0 &&
+                 workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && K0 / 128 + K1 / 128 >= 8 && M > g_linear_min_rows;
+    if (split && !ldw && g_linear_ks == 0) split = N / 16 < 2 * ns_cus() && (M > 16 || K0 + K1 >= 8192);  // raven_linear's rule
+    if (!split) {
+        if (ldw) return linear_column_block(x0, w, ldw, extra, y, 0, M, N, K0, workspace, workspace_bytes, s);
+        return raven_linear(x0, x1, w, residual, y, M, N, K0, K1, 0, 0, dtype, workspace, workspace_bytes, s);
+    }
+    NsArgs a{};
+    a.w = static_cast<const bf16*>(w);
+    a.x0 = static_cast<const bf16*>(x0);
+    a.x1 = static_cast<const bf16*>(x1);
+    a.residual = static_cast<const bf16*>(residual);
+    a.y = y;
+    a.M = M; a.N = N; a.K = K0 + K1; a.k0 = K0; a.k1 = K1; a.ldw = ldw; a.extra = extra;
+    return launch_ns<false>(a, workspace, workspace_bytes, s, ks_left);
 }
 
 }  // namespace raven

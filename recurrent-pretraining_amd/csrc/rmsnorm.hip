@@ -25,10 +25,21 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
 // measured at 5280 columns it is worth 0.1 us of a 3.6 us launch at best, the weights being cache hits).  Otherwise
 // each weight chunk is fetched where it is used, which keeps 32 registers free and more rows in flight per CU: from
 // 1024 rows on the early form is 3-20 % slower (4096 rows: 25.7 against 23.7 us, two norms 31.9 against 26.7).
-template <typename T, int MC, bool EARLY>
+//
+// SPLIT: the row is not read from x but formed from the fp32 partial sums a K-split product left behind (gemm_splitk.hip):
+// extra + slice 0 + slice 1 + ... in this order, rounded to T, plus the residual, rounded again -- the arithmetic of that
+// file's second launch, which this launch then replaces.
+struct SplitSums {
+    const float* partial;  // [ks][rows][dim]
+    const float* extra;    // [rows][dim] or null
+    int ks;
+    int64_t slice_stride;  // rows * dim
+};
+
+template <typename T, int MC, bool EARLY, bool SPLIT>
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
     const T* __restrict__ x, const T* __restrict__ residual, const T* __restrict__ weight, T* __restrict__ y,
-    T* __restrict__ sum_out, const T* __restrict__ weight2, T* __restrict__ y2, int dim, float eps) {
+    T* __restrict__ sum_out, const T* __restrict__ weight2, T* __restrict__ y2, int dim, float eps, SplitSums sp) {
     constexpr int E = Chunk<T>::N;
     __shared__ float red[4];
     const int64_t row = blockIdx.x;
@@ -54,13 +65,35 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
     for (int i = 0; i < MC; ++i) {
         const int c = threadIdx.x + i * kNormThreads;
         if (c < n_chunks) {
-            Chunk<T> cx = load_chunk(xr + c * E);
+            Chunk<T> cx;
+            if constexpr (SPLIT) {
+                float acc[E];
+                const int64_t at = row * dim + c * E;
+#pragma unroll
+                for (int q = 0; q < E / 4; ++q) {
+                    const f32x4 ex = sp.extra ? *reinterpret_cast<const f32x4*>(sp.extra + at + 4 * q) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[4 * q + e] = ex[e];
+                }
+                for (int sl = 0; sl < sp.ks; ++sl) {
+#pragma unroll
+                    for (int q = 0; q < E / 4; ++q) {
+                        const f32x4 pv = *reinterpret_cast<const f32x4*>(sp.partial + sl * sp.slice_stride + at + 4 * q);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[4 * q + e] += pv[e];
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < E; ++e) cx.v[e] = from_f32<T>(acc[e]);
+            } else {
+                cx = load_chunk(xr + c * E);
+            }
             if (rr) {
                 Chunk<T> cr = load_chunk(rr + c * E);
 #pragma unroll
                 for (int e = 0; e < E; ++e) cx.v[e] = from_f32<T>(to_f32(cx.v[e]) + to_f32(cr.v[e]));
-                if (sum_out) store_chunk(sum_out + row * dim + c * E, cx);
             }
+            if (sum_out && (rr || SPLIT)) store_chunk(sum_out + row * dim + c * E, cx);
 #pragma unroll
             for (int e = 0; e < E; ++e) {
                 v[i][e] = to_f32(cx.v[e]);
@@ -104,6 +137,19 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
 
 int g_norm_early = -1;  // raven_set_tuning("norm_early"): -1 = by row count, 0 / 1 = weights fetched late / early
 
+// The second launch of a K-split product (its slices added in order, rounded, plus the residual) and the RMSNorm(s) that
+// consume the result, as one launch: bf16, up to 32 rows of at most 8192 columns.  sum_out (may be null) receives the
+// product's value, y (may be null) the first norm's, y2 the second's when weight2 is given.
+int splitk_sums_then_norm(const float* partial, int ks, const float* extra, const void* residual, void* sum_out, const void* weight,
+                          void* y, const void* weight2, void* y2, int rows, int dim, float eps, hipStream_t s) {
+    RAVEN_REQUIRE(partial && ks >= 1 && weight && (y || y2) && (weight2 == nullptr) == (y2 == nullptr), "splitk_sums_then_norm: bad arguments");
+    RAVEN_REQUIRE(rows >= 1 && dim % 8 == 0 && dim / 8 <= kNormThreads * 4, "splitk_sums_then_norm: unsupported shape %d x %d", rows, dim);
+    SplitSums sp{partial, extra, ks, (int64_t)rows * dim};
+    rmsnorm_kernel<bf16, 4, true, true><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(
+        nullptr, (const bf16*)residual, (const bf16*)weight, (bf16*)y, (bf16*)sum_out, (const bf16*)weight2, (bf16*)y2, dim, eps, sp);
+    return raven_host::check_launch("split-K sums + rmsnorm");
+}
+
 }  // namespace raven
 
 extern "C" int raven_rmsnorm_residual(const void* x, const void* residual, const void* weight, void* y,
@@ -123,14 +169,15 @@ extern "C" int raven_rmsnorm_residual(const void* x, const void* residual, const
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int per_thread = (dim / elts + kNormThreads - 1) / kNormThreads;
     const bool early = g_norm_early >= 0 ? g_norm_early != 0 : rows <= 64;
+    const SplitSums none{};
 #define RAVEN_NORM_LAUNCH(T_, MC_)                                                                                           \
     do {                                                                                                                     \
         if (early)                                                                                                           \
-            rmsnorm_kernel<T_, MC_, true><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                               \
-                (const T_*)x, (const T_*)residual, (const T_*)weight, (T_*)y, (T_*)sum_out, (const T_*)weight2, (T_*)y2, dim, eps); \
+            rmsnorm_kernel<T_, MC_, true, false><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                        \
+                (const T_*)x, (const T_*)residual, (const T_*)weight, (T_*)y, (T_*)sum_out, (const T_*)weight2, (T_*)y2, dim, eps, none); \
         else                                                                                                                 \
-            rmsnorm_kernel<T_, MC_, false><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                              \
-                (const T_*)x, (const T_*)residual, (const T_*)weight, (T_*)y, (T_*)sum_out, (const T_*)weight2, (T_*)y2, dim, eps); \
+            rmsnorm_kernel<T_, MC_, false, false><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                       \
+                (const T_*)x, (const T_*)residual, (const T_*)weight, (T_*)y, (T_*)sum_out, (const T_*)weight2, (T_*)y2, dim, eps, none); \
     } while (0)
     if (dtype == RAVEN_BF16) {
         if (per_thread <= 4) RAVEN_NORM_LAUNCH(bf16, 4);

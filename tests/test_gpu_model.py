@@ -1130,6 +1130,39 @@ def test_core_iterations_nebel_one_row_real_weights(pkg, nebel_core):
     assert torch.equal(again, many) and torch.equal(kd3, kd)
 
 
+@pytest.mark.parametrize("B", [5, 8, 32])
+def test_slice_sums_folded_into_the_norm_launch_change_no_bit(pkg, nebel_core, tuned, B):
+    """For 2..32 rows the 5280-row products (attn.proj, mlp.proj, the adapter) are K-split; the launch that applies the
+    RMSNorms behind them also adds their slices (slice order, one rounding, residual, second rounding: the arithmetic
+    of the product's own second launch, gemm_splitk.hip / rmsnorm.hip).  Two recurrences at the 3.5b shape with that
+    folding on and off: the same bits in the state and in every appended cache row."""
+    s, w, dev = nebel_core
+    dt, h, T, r = torch.bfloat16, s.n_embd, 300, 2
+    blocks = (pkg.hip.BlockWeights * 4)(*[_block_weights(pkg, dev, f"transformer.core_block.{j}") for j in range(4)])
+    dims = pkg.hip.make_dims(h, s.n_heads, s.intermediate_size, s.norm_eps, dt)
+    g = torch.Generator().manual_seed(40 + B)
+    state = O.initialize_state(torch.empty(B, 1, h), s, 1.0, g).to(dt).view(B, h).cuda()
+    embeds = torch.randn(B, h, generator=g).to(dt).cuda()
+    table = O.rope_table(s.head_dim, s.block_size, s.rope_base).to(dt)
+    freqs = table.float().reshape(s.block_size, s.head_dim // 2, 2).contiguous().cuda()
+    ws = pkg.hip.block_workspace(dims, B, "cuda")
+    slots = [[it * 4 + j for j in range(4)] for it in range(r)]
+    lnf = rnd((h,), dt, 41, 0.02, 1.0).cuda()
+    outs = []
+    for fold in (1, 0):
+        tuned(fuse_sums_norm=fold)
+        _, _, kd, vd, cache = _nebel_cache(pkg, 4 * r, B, T, dt, 930)
+        out = torch.empty_like(state)
+        pkg.hip.core_iterations(dims, dev["transformer.adapter.weight"], blocks, state, embeds, out, freqs, cache, slots, B, 1, T, ws, ln_f=lnf)
+        one = torch.empty_like(state)   # a single recurrence takes the two-operand adapter product
+        _, _, kd1, vd1, cache1 = _nebel_cache(pkg, 4, B, T, dt, 930)
+        pkg.hip.core_iteration(dims, dev["transformer.adapter.weight"], blocks, state, embeds, one, freqs, cache1, 0, B, 1, T, ws)
+        outs.append((out, kd[:, :, :, T].clone(), vd[:, :, :, T].clone(), one, kd1[:, :, :, T].clone()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    assert torch.isfinite(outs[0][0].float()).all()
+
+
 def test_core_iteration_nebel_fp32_against_fp32_oracle(pkg):
     """One recurrence at the 3.5b shape in fp32, one row, 1024 cached positions per step slot, against the fp32 oracle at
     the fp32 bar (1e-4 / 1e-5): with rounding out of the picture this is a test of indexing at the real strides (5280-wide
