@@ -5,8 +5,10 @@
 The statistics over the vocabulary (entropy, KL divergence, min-p filtered KL) and over the latent
 state (relative change, cosine distance) are computed by HIP kernels (csrc/exit_stats.hip); only the
 comparison with the threshold and the bookkeeping of who has exited happen on the host, as they do in
-the reference.  `reduce=True` (the generate loop's setting) is the only mode built: statistics of the
-last position for the logit criteria, the mean over positions for the latent criteria.
+the reference.  `reduce=True` (the generate loop's setting): statistics of the last position for the logit
+criteria, the mean over positions for the latent criteria; `reduce=False`: one value per position, every
+position's logits going through the same kernels, with the reference's broadcasting of the initial state
+(a [B] or [B, V] start against [B, S] / [B, S, V] statistics: one sequence, or as many positions as sequences).
 """
 
 from __future__ import annotations
@@ -28,11 +30,6 @@ class PerIterationExitEvaluator:
         raise NotImplementedError()
 
 
-def _only_reduce(reduce: bool) -> None:
-    if not reduce:
-        raise NotImplementedError("per-position exit values (reduce=False) are not built; the generate loop uses reduce=True")
-
-
 class NoOpExitEvaluator(PerIterationExitEvaluator):
     """Never exits early (RMM:2117-2125)."""
 
@@ -42,24 +39,31 @@ class NoOpExitEvaluator(PerIterationExitEvaluator):
 
 
 class _LogitEvaluator(PerIterationExitEvaluator):
-    def _last_logits(self, model, latents, aux_inputs):
+    reduce = True
+
+    def _rows(self, model, latents, aux_inputs):
+        """(outputs, logits as rows [R, V], shape the per-row statistics take): the last position's logits, [B], under
+        `reduce`; every position's, [B, S], otherwise."""
         outputs = model.predict_from_latents(latents, **aux_inputs)
-        return outputs, outputs.logits[:, -1, :].contiguous()
+        logits = outputs.logits
+        if self.reduce:
+            return outputs, logits[:, -1, :].contiguous(), logits.shape[:1]
+        return outputs, logits.reshape(-1, logits.shape[-1]).contiguous(), logits.shape[:2]
 
 
 class EntropyDiffExitEvaluator(_LogitEvaluator):
     """Exit when the entropy of the next-token distribution stops changing (RMM:2128-2148)."""
 
     def __init__(self, exit_threshold: Union[str, float] = "auto", reduce: bool = True):
-        _only_reduce(reduce)
         self.exit_threshold = 1e-3 if exit_threshold == "auto" else float(exit_threshold)
+        self.reduce = reduce
 
     def init(self, initial_latents):
         self.prev_entropy = torch.ones(initial_latents.shape[0], device=initial_latents.device) * 100.0
 
     def check(self, model, latents, aux_inputs):
-        outputs, last = self._last_logits(model, latents, aux_inputs)
-        entropy = hip.exit_logit_stats(last, hip.EXIT_ENTROPY)
+        outputs, rows, shape = self._rows(model, latents, aux_inputs)
+        entropy = hip.exit_logit_stats(rows, hip.EXIT_ENTROPY).view(*shape)
         exit_values = (entropy - self.prev_entropy).abs()
         self.prev_entropy = entropy
         return exit_values < self.exit_threshold, outputs, exit_values
@@ -71,9 +75,9 @@ class KLExitEvaluator(_LogitEvaluator):
     _kind = hip.EXIT_KL
 
     def __init__(self, model, exit_threshold: Union[str, float] = "auto", reduce: bool = True):
-        _only_reduce(reduce)
         self.exit_threshold = self._auto if exit_threshold == "auto" else float(exit_threshold)
         self.V = model.config.padded_vocab_size
+        self.reduce = reduce
 
     _auto = 0.001
 
@@ -82,8 +86,10 @@ class KLExitEvaluator(_LogitEvaluator):
         self.prev_log_probs = ((1 / self.V) * torch.ones(B, self.V, device=initial_latents.device)).log()
 
     def check(self, model, latents, aux_inputs):
-        outputs, last = self._last_logits(model, latents, aux_inputs)
-        exit_values = hip.exit_logit_stats(last, self._kind, self.prev_log_probs)  # also stores the new log-probabilities
+        outputs, rows, shape = self._rows(model, latents, aux_inputs)
+        if self.prev_log_probs.shape != rows.shape:  # per position: the [B, V] start against [B, S, V], as torch broadcasts it
+            self.prev_log_probs = torch.broadcast_to(self.prev_log_probs, (*shape, rows.shape[-1])).reshape(rows.shape).contiguous()
+        exit_values = hip.exit_logit_stats(rows, self._kind, self.prev_log_probs).view(*shape)  # also stores the new log-probabilities
         return exit_values < self.exit_threshold, outputs, exit_values
 
 
@@ -98,8 +104,8 @@ class ArgmaxStabilityExitEvaluator(_LogitEvaluator):
     """Exit once the arg-max token has not changed for a number of checks (RMM:2219-2241)."""
 
     def __init__(self, exit_threshold: Union[str, int] = "auto", reduce: bool = True):
-        _only_reduce(reduce)
         self.exit_threshold = 5 if exit_threshold == "auto" else int(exit_threshold)
+        self.reduce = reduce
 
     def init(self, initial_latents):
         B, dev = initial_latents.shape[0], initial_latents.device
@@ -107,8 +113,8 @@ class ArgmaxStabilityExitEvaluator(_LogitEvaluator):
         self.stable_for_n_steps = torch.zeros(B, dtype=torch.long, device=dev)
 
     def check(self, model, latents, aux_inputs):
-        outputs, last = self._last_logits(model, latents, aux_inputs)
-        current = hip.argmax(last)
+        outputs, rows, shape = self._rows(model, latents, aux_inputs)
+        current = hip.argmax(rows).view(*shape)
         self.stable_for_n_steps = torch.where(current == self.prev_argmax, self.stable_for_n_steps + 1,
                                               torch.zeros_like(self.stable_for_n_steps))
         self.prev_argmax = current
@@ -131,11 +137,13 @@ class LatentDiffExitEvaluator(_LatentEvaluator):
     """Exit on a small relative change of the latent state (RMM:2151-2167)."""
 
     def __init__(self, exit_threshold: Union[str, float] = "auto", reduce: bool = True):
-        _only_reduce(reduce)
         self.exit_threshold = 0.03 if exit_threshold == "auto" else float(exit_threshold)
+        self.reduce = reduce
 
     def check(self, model, latents, aux_inputs):
-        exit_values = self._stats(latents, want_cos=False).mean(dim=-1)
+        exit_values = self._stats(latents, want_cos=False)
+        if self.reduce:
+            exit_values = exit_values.mean(dim=-1)
         return exit_values < self.exit_threshold, None, exit_values
 
 
@@ -143,11 +151,12 @@ class CosineExitEvaluator(_LatentEvaluator):
     """Exit when successive latent states point the same way (RMM:2244-2260)."""
 
     def __init__(self, exit_threshold: Union[str, float] = "auto", reduce: bool = True):
-        _only_reduce(reduce)
         self.exit_threshold = 1e-3 if exit_threshold == "auto" else float(exit_threshold)
+        self.reduce = reduce
 
     def check(self, model, latents, aux_inputs):
-        exit_values = 1 - self._stats(latents, want_cos=True).mean(dim=1)
+        cosine = self._stats(latents, want_cos=True)
+        exit_values = 1 - (cosine.mean(dim=1) if self.reduce else cosine)
         return exit_values < self.exit_threshold, None, exit_values
 
 

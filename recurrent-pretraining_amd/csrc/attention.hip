@@ -14,6 +14,8 @@
 
 #include <math.h>
 
+#include <atomic>
+
 #include "raven_common.h"
 
 namespace raven {
@@ -811,7 +813,9 @@ constexpr size_t kScratchBytes = ((kScratchMaxPairs * raven::kAttnMaxSplits * 2 
                                  ((kScratchMaxPairs * raven::kAttnMaxSplits * kScratchMaxHeadDim * 4 + 255) / 256 * 256);
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 constexpr int kScratchMaxDevices = 64;
-static void* g_scratch_ptr[kScratchMaxDevices];  // per device: each GPU holds its own copy of the array at its own address
+// per device: each GPU holds its own copy of the array at its own address.  Published atomically: two threads that race on
+// a device's first call both look the address up and store the same value
+static std::atomic<void*> g_scratch_ptr[kScratchMaxDevices];
 
 extern "C" size_t raven_qkv_attention_decode_static_scratch_bytes(void) { return kScratchBytes; }
 
@@ -826,14 +830,14 @@ extern "C" int raven_qkv_attention_decode_static(const void* qkv, const void* qk
                               hipGetErrorString(e), dev, kScratchMaxDevices);
         return e != hipSuccess ? (int)e : -1;
     }
-    if (g_scratch_ptr[dev] == nullptr) {
-        void* ptr = nullptr;
-        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-        if (e != hipSuccess || ptr == nullptr) {
+    void* scratch_dev = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (scratch_dev == nullptr) {  // the first call on this device (make it outside a stream capture)
+        e = hipGetSymbolAddress(&scratch_dev, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || scratch_dev == nullptr) {
             raven_host::set_error("qkv_attention_decode_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
             return e != hipSuccess ? (int)e : -1;
         }
-        g_scratch_ptr[dev] = ptr;
+        g_scratch_ptr[dev].store(scratch_dev, std::memory_order_release);
     }
     // the same size rule as raven_decode_attention_workspace_bytes; what would not fit the array is refused
     const size_t need = raven_decode_attention_workspace_bytes(B, n_heads, head_dim);
@@ -842,7 +846,7 @@ extern "C" int raven_qkv_attention_decode_static(const void* qkv, const void* qk
                   "(at most %zu (head, row) pairs in a split launch, head_dim up to %zu)",
                   B, n_heads, head_dim, need, kScratchBytes, kScratchMaxPairs, kScratchMaxHeadDim);
     return attention_common("qkv_attention_decode_static", true, qkv, qk_bias, freqs, y, cache, slot, B, 1, pos0, pos_dev, n_heads,
-                            head_dim, dtype, g_scratch_ptr[dev], kScratchBytes, stream);
+                            head_dim, dtype, scratch_dev, kScratchBytes, stream);
 }
 
 

@@ -211,6 +211,7 @@ class RavenForCausalLM(RavenPreTrainedModel, GenerationMixin):
         self._native_key = None
         self._native: dict = {}
         self._rope_override: Optional[torch.Tensor] = None  # a forward with positions that are not the cache's (see _rope_table_for)
+        self._rope_memo = None                               # the last such table and what it was built for
         self._scratch: dict = {}
         self.eval()
 
@@ -444,8 +445,12 @@ class RavenForCausalLM(RavenPreTrainedModel, GenerationMixin):
         if all(p == cache_pos0 + i for i, p in enumerate(rope_pos)):
             return None
         full = self._natives()["freqs"]
+        key = (cache_pos0, tuple(rope_pos), full.data_ptr())
+        if self._rope_memo is not None and self._rope_memo[0] == key:   # a batch that stays out of step asks for the same table again
+            return self._rope_memo[1]
         table = torch.zeros(cache_pos0 + len(rope_pos), full.shape[1], 2, dtype=full.dtype, device=full.device)
         table[cache_pos0:] = full[torch.as_tensor(rope_pos, device=full.device)]
+        self._rope_memo = (key, table)
         return table
 
     def _freqs(self) -> torch.Tensor:

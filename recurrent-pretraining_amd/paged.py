@@ -112,7 +112,7 @@ class PagedDecoder:
     @torch.no_grad()
     def forward_tokens(self, input_ids: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor, block_table: torch.Tensor,
                        seq_lens: torch.Tensor, query_start_loc: torch.Tensor, max_query_len: int,
-                       input_states: Optional[torch.Tensor] = None, init_scale: float = 1.0, check_bounds: bool = True):
+                       input_states: Optional[torch.Tensor] = None, init_scale: float = 1.0, check_bounds: Optional[bool] = None):
         """What the plugin's model computes for one scheduler step (RavenModel.forward, vllm/raven_vllm.py:374-411), straight on
         the pages: input_ids [T] are the new rows of B sequences, flattened (prompt chunks of any length and decode rows
         together); positions [T] and slot_mapping [T] (int64) say where each row sits; sequence b owns rows
@@ -125,7 +125,7 @@ class PagedDecoder:
         B = seq_lens.shape[0]
         if positions.shape != (T,) or slot_mapping.shape != (T,) or query_start_loc.shape != (B + 1,) or block_table.shape[0] != B:
             raise ValueError("positions [T], slot_mapping [T], block_table [B, max_blocks], seq_lens [B], query_start_loc [B + 1]")
-        if check_bounds:
+        if self._wants_check(check_bounds, block_table, seq_lens, positions, slot_mapping):
             self._check_pages(block_table, seq_lens, positions, slot_mapping)
         dev = m.device
         meta = (positions.to(dev, torch.int64), slot_mapping.to(dev, torch.int64), block_table.to(dev, torch.int32).contiguous(),
@@ -213,6 +213,12 @@ class PagedDecoder:
                                    cfg.padded_vocab_size, cfg.n_embd, hip.dtype_code(m.dtype), 1, hip._stream())
         hip._check(rc, "raven_gemm")
 
+    @staticmethod
+    def _wants_check(check_bounds: Optional[bool], *tensors) -> bool:
+        if check_bounds is not None:
+            return check_bounds
+        return all(t is None or t.device.type == "cpu" for t in tensors)
+
     def _check_pages(self, block_table: torch.Tensor, seq_lens: torch.Tensor, positions: Optional[torch.Tensor] = None,
                      slot_mapping: Optional[torch.Tensor] = None) -> None:
         """The kernels index the RoPE table by position and the pages through the block table without looking: whatever
@@ -241,17 +247,18 @@ class PagedDecoder:
                 raise ValueError(f"slot_mapping names slot {int(slots.max())}; the caches have {self.num_blocks * self.block_size}")
 
     def step(self, ids: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor, input_states: Optional[torch.Tensor] = None,
-             init_scale: float = 1.0, check_bounds: bool = True):
+             init_scale: float = 1.0, check_bounds: Optional[bool] = None):
         """One new token per sequence.  ids [B]; block_table [B, max_blocks] int32; seq_lens [B] int32 = each sequence's
         length INCLUDING the new token (its position is seq_lens - 1; the page for it must be in the table).
         Returns (logits [B, V] float32, latents [B, h]); both are buffers reused by the next step of the same batch size.
-        check_bounds=False skips the host-side validation of seq_lens / block_table (a caller that builds them itself and
-        keeps them on the GPU saves one device-to-host read per step)."""
+        check_bounds: None (default) validates seq_lens / block_table when they arrive as CPU tensors, where looking costs
+        nothing, and trusts tensors that already live on the GPU (validating those is a device-to-host read and a
+        synchronisation per scheduler step); True validates either way, False never."""
         m = self.model
         B = ids.shape[0]
         if block_table.dim() != 2 or block_table.shape[0] != B or seq_lens.shape != (B,):
             raise ValueError("block_table [B, max_blocks] and seq_lens [B] must match ids [B]")
-        if check_bounds:
+        if self._wants_check(check_bounds, block_table, seq_lens):
             self._check_pages(block_table, seq_lens)
         buf = self._buffers(B, block_table.shape[1])
         buf["ids"].copy_(ids.view(-1))

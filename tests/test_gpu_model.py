@@ -561,8 +561,57 @@ def test_adaptive_compute_options(pkg, small242):
     assert stopped.shape[1] == 5 and int(stopped[0, 4]) == first
     with pytest.raises(ValueError, match="Invalid adaptive compute strategy"):
         model.generate(ids.cuda(), gc, criterion="no-such-criterion")
-    with pytest.raises(NotImplementedError):
-        pkg.EntropyDiffExitEvaluator(reduce=False)
+
+
+def test_exit_evaluators_per_position(pkg, small242):
+    """reduce=False (RMM:2128-2260): one exit value per position instead of the last position's / the mean.  One
+    sequence of five positions, two checks in a row (the second compares with what the first stored), every criterion,
+    against the reference's formulas in torch over all positions."""
+    import torch.nn.functional as F
+    s, w, model = small242
+    g = torch.Generator().manual_seed(44)
+    B, S, V = 1, 5, s.vocab_size
+    lat = [O.initialize_state(torch.empty(B, S, s.n_embd), s, 1.0, g).cuda() for _ in range(3)]
+    aux = {}
+    logits = [model.predict_from_latents(x, **aux).logits.float().cpu() for x in lat]
+    evs = {name: pkg.get_adaptive_exit_evaluator(model, name, "auto", reduce=False)
+           for name in ("entropy-diff", "latent-diff", "cosine", "kl", "minp-kl", "argmax-stability")}
+    for ev in evs.values():
+        ev.init(lat[0])
+    prev_entropy = torch.ones(B) * 100.0
+    prev_lp = {k: ((1 / V) * torch.ones(B, V)).log() for k in ("kl", "minp-kl")}
+    prev_arg, stable = torch.ones(B, dtype=torch.long) * -1, torch.zeros(B, dtype=torch.long)
+
+    def minp(lg):
+        probs = F.softmax(lg, dim=-1)
+        probs[probs < 0.1 * probs.max(dim=-1, keepdim=True)[0]] = 1 / V
+        return (probs / probs.sum(dim=-1, keepdim=True)).log()
+
+    for step in (1, 2):
+        lg, x, x_prev = logits[step], lat[step].cpu(), lat[step - 1].cpu()
+        got = {name: ev.check(model, lat[step], aux) for name, ev in evs.items()}
+        probs = F.softmax(lg, dim=-1)
+        entropy = -torch.sum(probs * torch.log(probs + 1e-10), dim=-1)
+        want = {"entropy-diff": (entropy - prev_entropy).abs(),
+                "latent-diff": (x - x_prev).norm(dim=-1) / x.norm(dim=-1),
+                "cosine": 1 - (x * x_prev).sum(dim=-1) / x.norm(dim=-1) / x_prev.norm(dim=-1)}
+        prev_entropy = entropy
+        for name, fn in (("kl", lambda t: F.log_softmax(t, dim=-1)), ("minp-kl", minp)):
+            lp = fn(lg.clone())
+            want[name] = F.kl_div(lp, prev_lp[name], reduction="none", log_target=True).sum(dim=-1)
+            prev_lp[name] = lp
+        cur = lg.argmax(dim=-1)
+        stable = torch.where(cur == prev_arg, stable + 1, torch.zeros_like(stable))
+        prev_arg = cur
+        want["argmax-stability"] = stable
+        for name, (should_exit, outputs, values) in got.items():
+            assert values.shape == (B, S) and should_exit.shape == (B, S), name
+            if name == "argmax-stability":
+                assert torch.equal(values.cpu(), want[name]), name
+                assert torch.equal(should_exit.cpu(), want[name] >= 5)
+            else:
+                assert torch.allclose(values.float().cpu(), want[name], rtol=2e-4, atol=2e-6), (name, step, values, want[name])
+                assert torch.equal(should_exit.cpu(), values.cpu() < evs[name].exit_threshold)
 
 
 def test_forward_with_adaptive_compute_token_by_token(pkg, small242):
@@ -1210,12 +1259,12 @@ def test_positions_and_pages_are_bounded_on_the_host(pkg, small242):
     table = torch.arange(8, dtype=torch.int32).view(2, 4)
     ids = torch.zeros(2, dtype=torch.int64, device="cuda")
     with pytest.raises(ValueError, match="does not fit"):
-        dec.step(ids, table.cuda(), torch.tensor([65, 3], dtype=torch.int32).cuda())
+        dec.step(ids, table, torch.tensor([65, 3], dtype=torch.int32))              # CPU tensors: validated by default
     with pytest.raises(ValueError, match="block_table names block"):
-        dec.step(ids, (table + 5).cuda(), torch.tensor([40, 3], dtype=torch.int32).cuda())
+        dec.step(ids, (table + 5).cuda(), torch.tensor([40, 3], dtype=torch.int32).cuda(), check_bounds=True)   # GPU tensors: on request
     with pytest.raises(ValueError, match="RoPE table"):
         big = pkg.PagedDecoder(model, num_blocks=2, block_size=model.config.block_size + 16, num_steps=2)
-        big.step(ids[:1], torch.zeros(1, 1, dtype=torch.int32).cuda(), torch.tensor([model.config.block_size + 1], dtype=torch.int32).cuda())
+        big.step(ids[:1], torch.zeros(1, 1, dtype=torch.int32), torch.tensor([model.config.block_size + 1], dtype=torch.int32))
     T = 3
     args = (torch.zeros(T, dtype=torch.int64), torch.tensor([0, 1, model.config.block_size]), torch.tensor([0, 1, 2]), table[:1],
             torch.tensor([3], dtype=torch.int32), torch.tensor([0, 3], dtype=torch.int32), 3)

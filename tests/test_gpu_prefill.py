@@ -87,6 +87,31 @@ def test_tiled_gemm_nebel_shapes_m16384(pkg, name):
     assert torch.isfinite(got.float()).all()
 
 
+@pytest.mark.parametrize("M", [33, 64, 65, 96, 128, 129, 160, 161])
+def test_products_around_the_switch_between_skinny_passes_and_tiles(pkg, M):
+    """33 to 161 token rows with the default dispatch: which kernel takes a product changes with the row count here
+    (passes of the 32-row kernels up to 64 rows at K = 5280, 128 at 10560, 160 at 17920; 128 x 128 tiles beyond).  The five
+    products of the 3.5b shape, each with its epilogue, on either side of every switch, against fp32 F.linear."""
+    dt = torch.bfloat16
+    x, e, res = _gpu_randn((M, H), 20 + M), _gpu_randn((M, H), 21 + M), _gpu_randn((M, H), 22 + M)
+    g = _gpu_randn((M, INTER), 23 + M)
+    rows = torch.arange(M).cuda()
+    w = _gpu_randn((3 * H, H), 30, 0.02)
+    check(pkg.hip.linear(x, w), _ref_rows(x, w, rows).to(dt), dt, f"Wqkv at {M} rows")
+    w = _gpu_randn((H, H), 31, 0.02)
+    p = _ref_rows(x, w, rows)
+    check(pkg.hip.linear(x, w, residual=res), (p.to(dt).float() + res.float()).to(dt), dt, f"attn.proj at {M} rows", mag=p, ulps=ULPS_RESIDUAL)
+    w = _gpu_randn((2 * INTER, H), 32, 0.02)
+    z = _ref_rows(x, w, rows).to(dt).float()
+    check(pkg.hip.linear(x, w, swiglu=True), (F.silu(z[:, :INTER]).to(dt).float() * z[:, INTER:]).to(dt), dt, f"mlp.fc at {M} rows",
+          ulps=ULPS_SWIGLU)
+    w = _gpu_randn((H, INTER), 33, 0.02)
+    p = _ref_rows(g, w, rows)
+    check(pkg.hip.linear(g, w, residual=res), (p.to(dt).float() + res.float()).to(dt), dt, f"mlp.proj at {M} rows", mag=p, ulps=ULPS_RESIDUAL)
+    w = _gpu_randn((H, 2 * H), 34, 0.02)
+    check(pkg.hip.linear(x, w, x1=e), _ref_rows(torch.cat([x, e], -1), w, rows).to(dt), dt, f"adapter at {M} rows")
+
+
 @pytest.mark.parametrize("variant", [1, 2])
 @pytest.mark.parametrize("M,N,K", [(33, 64, 64), (64, 256, 256), (100, 264, 320), (257, 520, 96), (300, 5280, 5280), (513, 776, 1096)])
 def test_tiled_gemm_edges_against_oracle(pkg, tuned, variant, M, N, K):

@@ -54,3 +54,36 @@ def test_static_scratch_decode_attention_equals_workspace_version(pkg, dt, nh, h
                                         workspace=pkg.hip.attention_workspace(32, nh, hd, "cuda"))
     got = pkg.hip.qkv_attention_decode_static(qkv, bias, freqs, pkg.hip.make_cache(kb, vb), 0, 32, 300, nh, hd, pos_dev=pos_dev)
     assert torch.equal(got, want) and torch.equal(ka, kb)
+
+
+def test_static_scratch_entry_allocates_nothing_and_replays_from_a_captured_graph(pkg):
+    """What the entry point is for: after one eager call on the device (which looks the array's address up), a call
+    leaves the allocator's counters where they were, and the call can be captured into a HIP graph -- position on the
+    device, output buffer given -- and replayed: every replay gives the bits of the version with a workspace at that
+    position, with eager work and synchronisations of the program between the replays."""
+    dt, nh, hd, B, T = torch.bfloat16, 55, 96, 2, 900
+    qkv, bias, freqs, k, v = _case(pkg, B, T, nh, hd, dt, 70)
+    ka, va, kb, vb = k.cuda(), v.cuda(), k.cuda(), v.cuda()
+    ca, cb = pkg.hip.make_cache(ka, va), pkg.hip.make_cache(kb, vb)
+    pos_dev = torch.tensor([T - 3], dtype=torch.int32, device="cuda")
+    out = torch.empty(B, nh * hd, dtype=dt, device="cuda")
+    ws = pkg.hip.attention_workspace(B, nh, hd, "cuda")
+    pkg.hip.qkv_attention_decode_static(qkv, bias, freqs, cb, 1, B, T, nh, hd, pos_dev=pos_dev, out=out)   # the warm call
+    torch.cuda.synchronize()
+    before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.memory_stats()["allocation.all.allocated"])
+    pkg.hip.qkv_attention_decode_static(qkv, bias, freqs, cb, 1, B, T, nh, hd, pos_dev=pos_dev, out=out)
+    torch.cuda.synchronize()
+    assert before == (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.memory_stats()["allocation.all.allocated"])
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        pkg.hip.qkv_attention_decode_static(qkv, bias, freqs, cb, 1, B, T, nh, hd, pos_dev=pos_dev, out=out)
+    for step in range(3):   # positions T - 3, T - 2, T - 1: the same graph, the position read from the device
+        out.zero_()
+        graph.replay()
+        want = pkg.hip.qkv_attention_decode(qkv, bias, freqs, ca, 1, B, T, nh, hd, pos_dev=pos_dev, workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {step}"
+        assert torch.equal(ka, kb) and torch.equal(va, vb), f"replay {step}: appended rows"
+        busy = (qkv.float() * 0.5 + 0.25).sum().item()   # eager work and a synchronisation between the replays
+        assert busy == busy
+        pkg.hip.advance_pos(pos_dev, 1)
