@@ -571,7 +571,7 @@ def main():
 
 # HBM bytes per launch of the mlp.fc kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy: profiler
 # figures, so constants here, with the file that holds the readings
-FC_TRAFFIC = {1: 386113760, 32: 385933770}
+FC_TRAFFIC = {1: 385924535, 8: 382192138, 32: 386341464}
 FC_TRAFFIC_SOURCE = "profiles/mlp_fc_decode_hbm_traffic.txt"
 
 
