@@ -342,23 +342,50 @@ __global__ __launch_bounds__(16 * G) void decode_attention_kernel(
     }
 }
 
-// y[m, head] = sum_s w_s O_s / sum_s w_s L_s with w_s = 2^(M_s - max M); grid (heads, rows), hd threads
-template <typename T>
+// y[m, head] = sum_s w_s O_s / sum_s w_s L_s with w_s = 2^(M_s - max M); grid (heads, rows), 128 threads (hd <= 128).
+// The launch is all latency, so every load is requested at once: thread t < n_splits fetches split t's (M, L) pair while
+// every thread fetches its column of all partial outputs (32 loads in flight; splits past n_splits repeat the last one and
+// get weight 0).  The sums then run over the splits in order, out of LDS and registers.
+constexpr int kCombineSplits = 32;  // = kAttnMaxSplits, the most a launch is split into
+// NS: the splits a thread holds in registers, 8 / 16 / 32 >= n_splits
+template <typename T, int NS>
 __global__ __launch_bounds__(128) void attention_combine_kernel(const float* __restrict__ ws_ml, const float* __restrict__ ws_o,
                                                                 T* __restrict__ y, int nh, int hd, int n_splits) {
+    __shared__ float sm_m[kCombineSplits], sm_l[kCombineSplits];
     const int head = blockIdx.x, m = blockIdx.y, t = threadIdx.x;
-    if (t >= hd) return;
     const int64_t mh = (int64_t)m * nh + head;
+    if (t < n_splits) {
+        const float2 ml = *reinterpret_cast<const float2*>(ws_ml + (mh * n_splits + t) * 2);
+        sm_m[t] = ml.x;
+        sm_l[t] = ml.y;
+    }
+    float o[NS];
+    const int col = t < hd ? t : hd - 1;
+#pragma unroll
+    for (int sp = 0; sp < NS; ++sp) o[sp] = ws_o[(mh * n_splits + min(sp, n_splits - 1)) * hd + col];
+    __syncthreads();
+    if (t >= hd) return;
     float Mg = -INFINITY;
-    for (int sp = 0; sp < n_splits; ++sp) Mg = fmaxf(Mg, ws_ml[(mh * n_splits + sp) * 2]);
+    for (int sp = 0; sp < n_splits; ++sp) Mg = fmaxf(Mg, sm_m[sp]);
     float Lg = 0.f, Og = 0.f;
-    for (int sp = 0; sp < n_splits; ++sp) {
-        const float ms = ws_ml[(mh * n_splits + sp) * 2];
-        const float wgt = (ms == -INFINITY) ? 0.f : exp2f(ms - Mg);
-        Lg += ws_ml[(mh * n_splits + sp) * 2 + 1] * wgt;
-        Og += ws_o[(mh * n_splits + sp) * hd + t] * wgt;
+#pragma unroll
+    for (int sp = 0; sp < NS; ++sp) {
+        if (sp < n_splits) {
+            const float ms = sm_m[sp];
+            const float wgt = (ms == -INFINITY) ? 0.f : exp2f(ms - Mg);
+            Lg += sm_l[sp] * wgt;
+            Og += o[sp] * wgt;
+        }
     }
     y[(int64_t)m * nh * hd + head * hd + t] = from_f32<T>(Lg > 0.f ? Og / Lg : 0.f);  // no position at all (an empty paged sequence): zeros
+}
+
+template <typename T>
+static void launch_combine(const float* ws_ml, const float* ws_o, T* y, int nh, int hd, int rows, int n_splits, hipStream_t s) {
+    const dim3 grid(nh, rows), block(128);
+    if (n_splits <= 8) attention_combine_kernel<T, 8><<<grid, block, 0, s>>>(ws_ml, ws_o, y, nh, hd, n_splits);
+    else if (n_splits <= 16) attention_combine_kernel<T, 16><<<grid, block, 0, s>>>(ws_ml, ws_o, y, nh, hd, n_splits);
+    else attention_combine_kernel<T, kCombineSplits><<<grid, block, 0, s>>>(ws_ml, ws_o, y, nh, hd, n_splits);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -566,6 +593,7 @@ __global__ __launch_bounds__(256) void paged_qkv_rope_append_kernel(const T* __r
 }
 
 constexpr int kAttnMaxSplits = 32;
+static_assert(kAttnMaxSplits == kCombineSplits, "the merge kernel holds one partial output per split in registers");
 int g_rope_tiled_rows = 16;       // chunk length from which the append kernel works on (head, 16 positions) tiles ("rope_tiled_rows")
 int g_attn_nosplit_pairs = 1024;  // (head, row) pairs from which a launch is never split ("attn_nosplit_pairs", at most 1024)
 int g_attn_split_target = 1536;  // workgroups a split launch aims for (raven_set_tuning "attn_split_target"); 1536 beats 2048 by 2-6 us at 3..9 sequences
@@ -742,7 +770,7 @@ static void launch_attention(bool fused, const void* q, const void* bias, const 
         else RAVEN_ATTN_LAUNCH(false, 4, false);
     }
 #undef RAVEN_ATTN_LAUNCH
-    if (ns > 1) attention_combine_kernel<T><<<dim3(cv.nh, M), dim3(128), 0, s>>>(ws_ml, ws_o, (T*)y, cv.nh, cv.hd, ns);
+    if (ns > 1) launch_combine<T>(ws_ml, ws_o, (T*)y, cv.nh, cv.hd, M, ns, s);
 }
 
 static int attention_common(const char* who, bool fused, const void* q, const void* bias, const float* freqs, void* y,
@@ -939,11 +967,11 @@ static int paged_attention_common(const char* who, bool fused, const void* q, co
     } while (0)
     if (dtype == RAVEN_BF16) {
         RAVEN_PAGED_LAUNCH(bf16, 1);
-        if (ns > 1) attention_combine_kernel<bf16><<<dim3(n_heads, B), dim3(128), 0, s>>>(ws_ml, ws_o, (bf16*)y, n_heads, head_dim, ns);
+        if (ns > 1) launch_combine<bf16>(ws_ml, ws_o, (bf16*)y, n_heads, head_dim, B, ns, s);
     } else {
         if (head_dim / 4 > 16) RAVEN_PAGED_LAUNCH(float, 2);
         else RAVEN_PAGED_LAUNCH(float, 1);
-        if (ns > 1) attention_combine_kernel<float><<<dim3(n_heads, B), dim3(128), 0, s>>>(ws_ml, ws_o, (float*)y, n_heads, head_dim, ns);
+        if (ns > 1) launch_combine<float>(ws_ml, ws_o, (float*)y, n_heads, head_dim, B, ns, s);
     }
 #undef RAVEN_PAGED_LAUNCH
     return raven_host::check_launch(who);
