@@ -96,7 +96,11 @@ const char* raven_last_error(void);
  * non-zero also makes raven_linear use that kernel for every shape it accepts), gemm_tiled_min_rows (fewest rows, 33 or
  * more, that the tiled MFMA kernel takes), gemm_tiled_variant (0 = tile size by shape, 1 = 256 x 256, 2 = 128 x 128 and
  * no tile-count rule), gemm_tiled_split_tail (1 = the tile columns of a last round that fills at most half the chip go to
- * 128 x 128 tiles, 0 = never), prefill_waves (waves per workgroup of the chunk attention at head_dim 96: 0 = by shape, 4 or 6).
+ * 128 x 128 tiles, 0 = never), prefill_waves (waves per workgroup of the chunk attention at head_dim 96: 0 = by shape, 4 or 6),
+ * gemm_ragged (1 = a 5..32-row product whose output columns divide into about two workgroups per compute unit runs as one
+ * round of workgroups with a partly empty last tile, 0 = whole tiles only), norm_early (1 / 0 = the RMSNorm kernel requests
+ * its weights before / after the row reduction, -1 = by row count), fuse_sums_norm (1 = a K-split product that feeds a
+ * norm leaves its slices to that norm's launch, which adds them in the same order; 0 = a launch of its own adds them).
  * Not needed in normal use: the defaults are the tuned values.  The knobs are process-global
  * state read at every launch: changing them while another thread or stream is inside a call of this library is a race. */
 int raven_set_tuning(const char* key, int32_t value);
