@@ -24,7 +24,7 @@ How each function is pinned (tests/test_oracle_pins.py), without running the ref
   block/iterate/forward/greedy   composition laws (r=0, cache vs no-cache,
                      prefill-then-decode vs token-by-token)                       -> pinned
   initialize_state   bounds, std, scale=0, generator determinism                  -> pinned
-  DictCache lookups  (latest-m4, available-m4, always-last-m4, skip) closed form on
+  DictCache lookups  (latest-m4, available-m4, always-last-m4, skip, randomized) closed form on
                      step-tagged entries                                          -> pinned
   ExitCriterion      entropy of uniform / one-hot rows, KL(p, p) = 0 and two-point closed
                      form, fp64 brute force, min-p floor by hand, latent ratios of scaled /
@@ -271,6 +271,13 @@ class DictCache:
                 if pos not in self.key_cache[step]:
                     continue
                 src = step
+            elif lookup.startswith("randomized"):       # RMM:255-271: one CPU draw per position, in position order
+                if step < 2:
+                    src = step if pos in self.key_cache[step] else 0
+                else:
+                    block = (step - 2) % 4 + 2
+                    have = [s for s in range(2, step + 1) if (s - 2) % 4 + 2 == block and pos in self.key_cache[s]]
+                    src = have[torch.randint(len(have), (1,))]
             else:
                 raise ValueError(f"Unknown lookup strategy: {lookup}")
             ks.append(self.key_cache[src][pos])

@@ -114,7 +114,9 @@ def lookup_mode(strategy: str) -> int:
     if strategy.startswith("always-last-m4"):
         return hip.LOOKUP_ALWAYS_LAST    # RMM:233-246
     if strategy.startswith("randomized"):
-        raise NotImplementedError("the 'randomized' lookup (a sanity check in the reference, RMM:255-271) is not built")
+        # a sanity check in the reference (RMM:255-271): HuginnDynamicCache.update serves it on the host, one CPU draw
+        # per position as there; the attention kernels, which resolve lookups in place, do not
+        raise NotImplementedError("the 'randomized' lookup is served by HuginnDynamicCache.update only, not by the attention kernels")
     raise ValueError(f"Unknown lookup strategy: {strategy}")  # RMM:272-273
 
 
@@ -351,6 +353,8 @@ class HuginnDynamicCache:
             return self._k[slot, :, :, :self._seen_tokens], self._v[slot, :, :, :self._seen_tokens]
         # some positions were never computed at this step: gather per position, as RMM:199-253 does
         lookup = self.lookup_strategy if lookup_strategy is None else lookup_strategy
+        if self.lookup_strategy != "full" and lookup.startswith("randomized"):
+            return self._gather_randomized(mapped)
         mode = hip.LOOKUP_SKIP if self.lookup_strategy == "full" else lookup_mode(lookup)
         if mode == hip.LOOKUP_ALWAYS_LAST and "compress-" in self.lookup_strategy:
             raise NotImplementedError("always-last-m4 lookups over shared (compress-*) entries with missing positions are not built")
@@ -360,6 +364,20 @@ class HuginnDynamicCache:
         src = [self._source_step(mapped, depths[p], mode) if p < len(depths) else mapped for p in range(self._seen_tokens)]
         pos = torch.tensor([p for p, st in enumerate(src) if st is not None], device=self._k.device)
         slots = torch.tensor([self._slot(st) for st in src if st is not None], device=self._k.device)
+        return self._k[slots, :, :, pos].permute(1, 2, 0, 3), self._v[slots, :, :, pos].permute(1, 2, 0, 3)
+
+    def _gather_randomized(self, step: int):
+        """RMM:255-271: every position, the new ones included, is read at a step drawn among those of the same block
+        that it holds up to `step` -- one `torch.randint` on the CPU's default generator per position, in position
+        order, as the reference draws them (an empty choice raises there and here)."""
+        if self._core.holes(self._seen_tokens):
+            raise NotImplementedError("lookups need positions that hold the core steps 2, 3, ... without holes")
+        src = []
+        for depth in self._core.depths(self._seen_tokens):
+            valid = [s for s in range(2, step + 1) if (s - step) % 4 == 0 and s - 2 < depth]
+            src.append(valid[int(torch.randint(len(valid), (1,)))])
+        pos = torch.arange(self._seen_tokens, device=self._k.device)
+        slots = torch.tensor([self._slot(st) for st in src], device=self._k.device)
         return self._k[slots, :, :, pos].permute(1, 2, 0, 3), self._v[slots, :, :, pos].permute(1, 2, 0, 3)
 
     @staticmethod

@@ -190,6 +190,24 @@ def test_cache_lookups_with_partially_filled_steps_match_dict_model(pkg, strateg
         assert torch.equal(got[0], want[0]), (strategy, step)
 
 
+@pytest.mark.parametrize("strategy", ["randomized", "randomized-compress-s4"])
+def test_randomized_lookup_matches_dict_model_draw_for_draw(pkg, strategy):
+    """RMM:255-271: with the CPU generator seeded alike, the contiguous cache returns the entries the dict model of the
+    reference draws, and leaves the generator in the same state (one draw per position and lookup, in position order)."""
+    g = torch.Generator().manual_seed(11)
+    ours, ref = pkg.HuginnDynamicCache(strategy), O.DictCache(strategy)
+    for i, (n_new, r) in enumerate(((4, 3), (1, 1), (1, 4), (2, 2), (1, 6), (1, 3))):
+        for step in [0, 1] + list(range(2, 2 + 4 * r)) + [-1, -2]:
+            k, v = torch.randn(2, 3, n_new, 8, generator=g), torch.randn(2, 3, n_new, 8, generator=g)
+            torch.manual_seed(100 * i + step + 7)
+            want = ref.update(k, v, step)
+            state = torch.get_rng_state()
+            torch.manual_seed(100 * i + step + 7)
+            got = ours.update(k, v, step)
+            assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]), (strategy, i, step)
+            assert torch.equal(torch.get_rng_state(), state), (strategy, i, step)
+
+
 def test_cache_lookup_errors(pkg):
     c = pkg.HuginnDynamicCache("latest-m4")
     k = torch.zeros(1, 1, 1, 4)
@@ -197,13 +215,13 @@ def test_cache_lookup_errors(pkg):
         c.update(k, k, step)
     for step in (0, 1, 2, 3, 4, 5, 6):
         c.update(k, k, step)
-    c2 = pkg.HuginnDynamicCache("randomized")
+    c2 = pkg.HuginnDynamicCache("randomized")  # update() serves it; the kernels' descriptor does not
     for step in (0, 1, 2, 3, 4, 5):
         c2.update(k, k, step)
-    for step in (0, 1, 2, 3, 4, 5):
+    for step in (0, 1, 2, 3, 4, 5, 6):
         c2.update(k, k, step)
     with pytest.raises(NotImplementedError, match="randomized"):
-        c2.update(k, k, 6)
+        pkg.cache.lookup_mode(c2.lookup_strategy)
     c3 = pkg.HuginnDynamicCache("no-such-strategy")
     for step in (0, 1, 2, 3, 4, 5, 0, 1, 2, 3, 4, 5):
         c3.update(k, k, step)

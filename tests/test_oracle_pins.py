@@ -380,6 +380,38 @@ def test_partial_fill_lookups_closed_form():
                 assert got == want, (strategy, pos, step, got, want)
 
 
+def test_randomized_lookup_draws_one_step_per_position():
+    """RMM:255-271: once a step has a gap, every position (the querying one too) is read at a step of the same block,
+    not deeper than the current step, drawn among those it holds -- one draw of `torch.randint(n_valid, (1,))` per
+    position, in position order, from the CPU's default generator.  Entries are tagged with (step, position); the draws
+    are replayed from the same seed, and the generator must stand where the replay leaves it."""
+    depths = [3, 1, 4, 2, 5]
+    seen_choices = set()
+    for seed in range(6):
+        c = O.DictCache("randomized")
+        for pos, d in enumerate(depths):
+            for step in [0, 1] + list(range(2, 2 + 4 * d)):
+                tag = torch.full((1, 1, 1, 1), float(step * 100 + pos))
+                torch.manual_seed(1000 * seed + 10 * pos + step)
+                k, _ = c.update(tag, tag, step)
+                after = int(torch.randint(1 << 30, (1,)))
+                got = [(int(t) // 100, int(t) % 100) for t in k.flatten().tolist()]
+                if step < 2 or all(dd > (step - 2) // 4 for dd in depths[:pos]):
+                    assert got == [(step, p) for p in range(pos + 1)]  # no gap: no draw
+                    continue
+                i, j = divmod(step - 2, 4)
+                torch.manual_seed(1000 * seed + 10 * pos + step)
+                want = []
+                for p, dd in enumerate(depths[:pos] + [i + 1]):
+                    n_valid = min(i + 1, dd)
+                    want.append((2 + 4 * int(torch.randint(n_valid, (1,))) + j, p))
+                assert got == want, (seed, pos, step, got, want)
+                assert after == int(torch.randint(1 << 30, (1,)))
+                seen_choices.update((pos, step, src) for src, p in got if p == 2)
+    # position 2 holds 4 recurrences: queried at recurrence 4 (step 18..21, token 4) each of its four is drawn at some seed
+    assert {src for pos, step, src in seen_choices if step == 18} == {2, 6, 10, 14}
+
+
 def test_step_remap_strategies():
     assert [O.remap_step(i, "full") for i in (0, 1, 2, 129, -1)] == [0, 1, 2, 129, -1]
     assert [O.remap_step(i, "latest-m4-compress-s4") for i in (0, 1, 2, 5, 6, 9, 129, -1, -2)] == [0, 1, 2, 5, 2, 5, 5, -1, -2]
