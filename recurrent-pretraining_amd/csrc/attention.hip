@@ -156,6 +156,10 @@ __device__ __forceinline__ float dot_piece(const Piece<T, CPL>& a, const Piece<T
     return acc;
 }
 
+// 2^x as the hardware instruction computes it (results below the smallest normal number come out as 0, which is what
+// a softmax weight that small amounts to); exp2f() wraps the same instruction in a range reduction for denormal results
+__device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
+
 // Online-softmax state (running maximum, sum, unnormalised output) of a wave's four 16-lane rows merged into one, in
 // registers; afterwards every row of the wave holds the merged state.
 template <int E>
@@ -188,8 +192,10 @@ __device__ __forceinline__ void merge_wave_rows(float& m_run, float& l_run, floa
 // G = 16-lane rows per workgroup (16 x G threads): 16, or 64 for the variant that gives a whole (head, row) to one
 // workgroup of 1024 threads whose every load is in flight at once -- what the split launch achieves with several
 // workgroups and a second launch, without that launch.
-template <typename T, bool FUSED, int kAttnU, bool LOOKUP = false, int CPL = 1, int G = 16>
-__global__ __launch_bounds__(16 * G) void decode_attention_kernel(
+// Waves per SIMD the register budget is held to: with a second tile in flight the 2-position variant must still hold the
+// 1760 workgroups of 32 rows x 55 heads at once (7 waves = 72 registers).
+template <typename T, bool FUSED, int kAttnU, bool LOOKUP = false, int CPL = 1, int G = 16, bool PF = false>
+__global__ __launch_bounds__(16 * G, (G == 16 && kAttnU == 2 && CPL == 1 && PF) ? 7 : 4) void decode_attention_kernel(
     const T* __restrict__ q_or_qkv, const T* __restrict__ qk_bias, const float* __restrict__ freqs, T* __restrict__ y,
     CacheView cv, int S, int pos0, const int* __restrict__ pos_dev, float scale_log2, int n_splits,
     float* __restrict__ ws_ml, float* __restrict__ ws_o) {
@@ -233,27 +239,48 @@ __global__ __launch_bounds__(16 * G) void decode_attention_kernel(
             qraw = load_piece<T, CPL>(q_or_qkv + (int64_t)m * h + col);
         }
     }
-    // first K/V tile, requested before q is touched
-    P kc[kAttnU], vc[kAttnU];
-    bool left_out[kAttnU];  // LOOKUP: the position takes no part
-    auto load_tile = [&](int base) {
+    // K/V tiles: kAttnU positions per 16-lane row.  Without lookups every load of a tile is unconditional, so that all
+    // of them are in flight before the first is waited for (a load under a per-lane condition makes the compiler wait for
+    // it inside the conditional block, one position after the other): positions past the range read the last position
+    // that is certainly cached instead, lanes past the head row's chunks repeat its last chunk (their q is zero), and the
+    // scores of such positions are masked below.  FUSED: the row's own position, the last one, is not read at all; it is
+    // added from registers behind the loop.
+    struct Tile {
+        P k[kAttnU], v[kAttnU];
+        bool left_out[kAttnU];  // LOOKUP: the position takes no part
+    };
+    const int end_c = FUSED ? min(end, pos) : end;       // end of the cached positions of this range
+    const int last_ok = max((FUSED ? pos : len) - 1, 0);  // initialised whenever a tile is consumed at all (then end_c >= 1)
+    const T* Kh = static_cast<const T*>(cv.k) + head_off;
+    const T* Vh = static_cast<const T*>(cv.v) + head_off;
+    const unsigned lane_off = (unsigned)(min(ci, cp - 1) * E);
+    auto load_tile = [&](int base, Tile& t) {
 #pragma unroll
         for (int j = 0; j < kAttnU; ++j) {
             const int p = base + j * G + group;
-            int64_t delta = 0;
-            left_out[j] = false;
-            if (LOOKUP && cv.steps_present != nullptr && p < end && p < first_new) left_out[j] = !lookup_source(cv, p, &delta);
-            if (active && p < end && !(FUSED && p == pos) && !left_out[j]) {
-                // large grids (the 2-position variant) stream K/V past the caches: +8 % at batch 32; small ones do not gain
-                kc[j] = load_piece<T, CPL, kAttnU == 2>(Kb + delta + (int64_t)p * hd);
-                vc[j] = load_piece<T, CPL, kAttnU == 2>(Vb + delta + (int64_t)p * hd);
+            if constexpr (LOOKUP) {
+                int64_t delta = 0;
+                t.left_out[j] = false;
+                if (cv.steps_present != nullptr && p < end_c && p < first_new) t.left_out[j] = !lookup_source(cv, p, &delta);
+                if (active && p < end_c && !t.left_out[j]) {
+                    t.k[j] = load_piece<T, CPL, kAttnU == 2>(Kb + delta + (int64_t)p * hd);
+                    t.v[j] = load_piece<T, CPL, kAttnU == 2>(Vb + delta + (int64_t)p * hd);
+                } else {
+                    t.k[j] = zero_piece<T, CPL>();
+                    t.v[j] = zero_piece<T, CPL>();
+                }
             } else {
-                kc[j] = zero_piece<T, CPL>();
-                vc[j] = zero_piece<T, CPL>();
+                // large grids (the 2-position variant) stream K/V past the caches: +8 % at batch 32; small ones do not gain
+                // a 32-bit byte offset from the workgroup's (uniform) head row: scalar base + vector offset addressing
+                const unsigned off = ((unsigned)min(p, last_ok) * (unsigned)hd + lane_off) * (unsigned)sizeof(T);
+                t.k[j] = load_piece<T, CPL, kAttnU == 2>(reinterpret_cast<const T*>(reinterpret_cast<const char*>(Kh) + off));
+                t.v[j] = load_piece<T, CPL, kAttnU == 2>(reinterpret_cast<const T*>(reinterpret_cast<const char*>(Vh) + off));
+                t.left_out[j] = false;
             }
         }
     };
-    load_tile(start);
+    Tile ta, tb;
+    load_tile(start, ta);  // requested before q is touched
 
     P qc = qraw, knew = kraw;
     if (FUSED && active) {
@@ -272,26 +299,21 @@ __global__ __launch_bounds__(16 * G) void decode_attention_kernel(
 #pragma unroll
     for (int e = 0; e < E; ++e) o[e] = 0.f;
 
-    for (int base = start; base < end; base += G * kAttnU) {  // trip count is uniform over the workgroup
-        if (base != start) load_tile(base);
+    auto consume = [&](int base, const Tile& t) {
         float sc[kAttnU], m_new = m_run;
 #pragma unroll
         for (int j = 0; j < kAttnU; ++j) {
             const int p = base + j * G + group;
-            if (FUSED && p == pos) {
-                kc[j] = knew;
-                vc[j] = vnew;
-            }
-            sc[j] = row16_sum(dot_piece<T, CPL>(qc, kc[j])) * scale_log2;
-            if (p >= end || (LOOKUP && left_out[j])) sc[j] = -INFINITY;
+            sc[j] = row16_sum(dot_piece<T, CPL>(qc, t.k[j])) * scale_log2;
+            if (p >= end_c || (LOOKUP && t.left_out[j])) sc[j] = -INFINITY;
             m_new = fmaxf(m_new, sc[j]);
         }
-        if (m_new == -INFINITY) continue;  // this row has not seen a valid position yet
-        const float corr = exp2f(m_run - m_new);
+        if (m_new == -INFINITY) return;  // this row has not seen a valid position yet
+        const float corr = exp2_raw(m_run - m_new);
         float pe[kAttnU], psum = 0.f;
 #pragma unroll
         for (int j = 0; j < kAttnU; ++j) {
-            pe[j] = exp2f(sc[j] - m_new);
+            pe[j] = exp2_raw(sc[j] - m_new);
             psum += pe[j];
         }
         l_run = l_run * corr + psum;
@@ -299,9 +321,36 @@ __global__ __launch_bounds__(16 * G) void decode_attention_kernel(
         for (int e = 0; e < E; ++e) {
             float acc = o[e] * corr;
 #pragma unroll
-            for (int j = 0; j < kAttnU; ++j) acc = __builtin_fmaf(pe[j], to_f32(vc[j].c[e / EC].v[e % EC]), acc);
+            for (int j = 0; j < kAttnU; ++j) acc = __builtin_fmaf(pe[j], to_f32(t.v[j].c[e / EC].v[e % EC]), acc);
             o[e] = acc;
         }
+        m_run = m_new;
+    };
+    constexpr int STEP = G * kAttnU;
+    if constexpr (PF && !LOOKUP) {
+        // two tiles in turn, the next one requested before the current one is used; always whole pairs (a tile past the
+        // range re-reads cached lines and adds nothing), so that the number of loads in flight is the same on every path
+        // and the waits can leave the younger tile's loads outstanding
+        for (int base = start; base < end_c; base += 2 * STEP) {  // trip count is uniform over the workgroup
+            load_tile(base + STEP, tb);
+            consume(base, ta);
+            load_tile(base + 2 * STEP, ta);
+            consume(base + STEP, tb);
+        }
+    } else {
+        for (int base = start; base < end_c;) {
+            consume(base, ta);
+            base += STEP;
+            if (base < end_c) load_tile(base, ta);
+        }
+    }
+    if (FUSED && group == 0 && pos >= start && pos < end) {  // the row's own position, from registers
+        const float sc = row16_sum(dot_piece<T, CPL>(qc, knew)) * scale_log2;
+        const float m_new = fmaxf(m_run, sc);
+        const float corr = exp2_raw(m_run - m_new), pe = exp2_raw(sc - m_new);
+        l_run = l_run * corr + pe;
+#pragma unroll
+        for (int e = 0; e < E; ++e) o[e] = __builtin_fmaf(pe, to_f32(vnew.c[e / EC].v[e % EC]), o[e] * corr);
         m_run = m_new;
     }
 
@@ -603,6 +652,7 @@ int g_attn_big_grid = 1280;      // workgroups from which the 2-positions-per-ro
 // about 2000 positions and from 8 sequences on), inside a decoded token the gain does not show (bs=1: 18.9-19.1 ms per
 // token either way; bs=4: -0.4 %), so it is off unless asked for.  "attn_wide" = longest cache it is used for, 0 = never.
 int g_attn_wide = 0;
+int g_attn_prefetch = 1;  // raven_set_tuning("attn_prefetch"): 0 = a decode-attention workgroup requests a tile only when it needs it
 
 // Splits are worth their extra launch only while heads x rows cannot fill the chip.
 static int splits_for(int M, int nh, int len_hint) {
@@ -751,23 +801,32 @@ static void launch_attention(bool fused, const void* q, const void* bias, const 
     // the launch is not split (512 or more (head, row) pairs), and for split launches from g_attn_big_grid workgroups on
     const bool big = ns == 1 ? (int64_t)cv.nh * M >= 512 : (int64_t)cv.nh * M * ns >= g_attn_big_grid;
     const T* bias_t = (const T*)bias;
-#define RAVEN_ATTN_LAUNCH(FUSED_, U_, LOOKUP_)                                                                            \
-    decode_attention_kernel<T, FUSED_, U_, LOOKUP_><<<grid, dim3(256), 0, s>>>((const T*)q, FUSED_ ? bias_t : nullptr,     \
+#define RAVEN_ATTN_LAUNCH(FUSED_, U_, LOOKUP_, PF_)                                                                       \
+    decode_attention_kernel<T, FUSED_, U_, LOOKUP_, 1, 16, PF_><<<grid, dim3(256), 0, s>>>((const T*)q, FUSED_ ? bias_t : nullptr, \
         FUSED_ ? freqs : nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o)
+    // a workgroup that walks many tiles requests the next tile before it uses the current one (unsplit launches of 512
+    // or more (head, row) pairs: 117.5 -> 114 us at 32 rows and 1024 positions; split launches, whose workgroups
+    // walk a few tiles each, lose 8 % to the tile of the last pair that lies past the range)
+    const int per = (pos0 + S + ns - 1) / ns;
+    const bool pf = g_attn_prefetch && (ns == 1 || g_attn_prefetch == 2) && per >= 8 * 16 * (big ? 2 : 4);
     if (cv.hd / Chunk<T>::N > 16) {  // fp32 heads wider than 64 elements: two chunks per lane, one variant per entry point
         if constexpr (sizeof(T) == 4) {
             if (fused) decode_attention_kernel<T, true, 2, true, 2><<<grid, dim3(256), 0, s>>>((const T*)q, bias_t, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
             else decode_attention_kernel<T, false, 2, true, 2><<<grid, dim3(256), 0, s>>>((const T*)q, nullptr, nullptr, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
         }
     } else if (cv.steps_present) {  // partial fill: rare, one variant per entry point
-        if (fused) RAVEN_ATTN_LAUNCH(true, 2, true);
-        else RAVEN_ATTN_LAUNCH(false, 2, true);
+        if (fused) RAVEN_ATTN_LAUNCH(true, 2, true, false);
+        else RAVEN_ATTN_LAUNCH(false, 2, true, false);
     } else if (fused) {
-        if (big) RAVEN_ATTN_LAUNCH(true, 2, false);
-        else RAVEN_ATTN_LAUNCH(true, 4, false);
+        if (big && pf) RAVEN_ATTN_LAUNCH(true, 2, false, true);
+        else if (big) RAVEN_ATTN_LAUNCH(true, 2, false, false);
+        else if (pf) RAVEN_ATTN_LAUNCH(true, 4, false, true);
+        else RAVEN_ATTN_LAUNCH(true, 4, false, false);
     } else {
-        if (big) RAVEN_ATTN_LAUNCH(false, 2, false);
-        else RAVEN_ATTN_LAUNCH(false, 4, false);
+        if (big && pf) RAVEN_ATTN_LAUNCH(false, 2, false, true);
+        else if (big) RAVEN_ATTN_LAUNCH(false, 2, false, false);
+        else if (pf) RAVEN_ATTN_LAUNCH(false, 4, false, true);
+        else RAVEN_ATTN_LAUNCH(false, 4, false, false);
     }
 #undef RAVEN_ATTN_LAUNCH
     if (ns > 1) launch_combine<T>(ws_ml, ws_o, (T*)y, cv.nh, cv.hd, M, ns, s);
