@@ -58,6 +58,8 @@ def parse():
                     help="with --prefill: run only N launches of the chunk attention kernel at that shape (for rocprofv3 --pmc runs)")
     ap.add_argument("--gemm-only", type=int, default=0, metavar="N",
                     help="with --prefill: launch each of the five products of a core iteration N times at the prefill shape and time it")
+    ap.add_argument("--library-gemm", action="store_true",
+                    help="with --prefill --gemm-only: also time torch.matmul (the vendor library) on each product's operands, as a yardstick")
     ap.add_argument("--kernel-only", type=int, default=0, metavar="N",
                     help="run only N launches of the dominant kernel plus one 256 MiB device copy (for rocprofv3 --pmc runs)")
     return ap.parse_args()
@@ -359,6 +361,15 @@ def gemm_only(args):
         total_flops += n_iter * flops
         out["products"][name] = {"N": ws[0].shape[0], "K": ws[0].shape[1], "ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
                                  "frac_of_mfma_peak": round(flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4)}
+        if args.library_gemm and "x1" not in kw:
+            # the same product without its epilogue through torch.matmul (the vendor library), same process and operands:
+            # a yardstick beside the figure above, never part of it
+            def lib_launch(i=[0]):
+                i[0] += 1
+                torch.matmul(xin, ws[i[0] % 4].t())
+
+            lib_ms = event_time_ms(lib_launch, args.gemm_only, warm=2)
+            out["products"][name]["library_matmul_no_epilogue"] = {"ms": round(lib_ms, 4), "TFLOP/s": round(flops / lib_ms / 1e9, 1)}
     out["per_iteration"] = {"ms": round(total_ms, 3), "TFLOP/s": round(total_flops / total_ms / 1e9, 1)}
     print(json.dumps(out))
 

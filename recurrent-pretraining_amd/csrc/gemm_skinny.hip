@@ -597,7 +597,7 @@ extern "C" int raven_set_tuning(const char* key, int32_t value) {
     else if (k == "norm_early" && value >= -1 && value <= 1) g_norm_early = value;
     else if (k == "fuse_sums_norm" && (value == 0 || value == 1)) g_fuse_sums_norm = value;
     else if (k == "gemm_tiled_min_rows" && value >= 33) g_tiled_min_rows = value;
-    else if (k == "gemm_tiled_variant" && value >= 0 && value <= 2) g_tiled_variant = value;
+    else if (k == "gemm_tiled_variant" && value >= 0 && value <= 3) g_tiled_variant = value;
     else if (k == "gemm_tiled_split_tail" && (value == 0 || value == 1)) g_tiled_split_tail = value;
     else RAVEN_REQUIRE(set_gemv1_tuning(key, value) == 0, "set_tuning: unknown key %s", key);
     return 0;

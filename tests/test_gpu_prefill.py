@@ -112,11 +112,13 @@ def test_products_around_the_switch_between_skinny_passes_and_tiles(pkg, M):
     check(pkg.hip.linear(x, w, x1=e), _ref_rows(torch.cat([x, e], -1), w, rows).to(dt), dt, f"adapter at {M} rows")
 
 
-@pytest.mark.parametrize("variant", [1, 2])
-@pytest.mark.parametrize("M,N,K", [(33, 64, 64), (64, 256, 256), (100, 264, 320), (257, 520, 96), (300, 5280, 5280), (513, 776, 1096)])
+@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("M,N,K", [(33, 64, 64), (64, 256, 256), (100, 264, 320), (257, 520, 96), (300, 5280, 5280), (513, 776, 1096), (700, 1032, 136)])
 def test_tiled_gemm_edges_against_oracle(pkg, tuned, variant, M, N, K):
-    """Both tile sizes (256 x 256 and 128 x 128) on shapes with partial tiles in M and N, K that is not a multiple of
-    the 64-wide step, every epilogue and the two-operand form, against the oracle's linear / SwiGLU / residual."""
+    """The three tile kernels (256 x 256 by four waves with an LDS ring, 128 x 128, 256 x 256 by eight waves with staging
+    registers) on shapes with partial tiles in M and N, K that is not a multiple of the 64-wide step (down to one and
+    two steps, fewer than the ring holds), every epilogue and the two-operand form, against the oracle's linear /
+    SwiGLU / residual."""
     dt = torch.bfloat16
     tuned(gemm_tiled_variant=variant)
     x, w, res = rnd((M, K), dt, 500 + M), rnd((N, K), dt, 501 + N, 0.05), rnd((M, N), dt, 502)
@@ -137,8 +139,9 @@ def test_tiled_gemm_edges_against_oracle(pkg, tuned, variant, M, N, K):
         check(pkg.hip.linear(dev(x), dev(w)), O.linear(x, w), dt, "oracle linear")
     # the same call twice: the same bits; and the tile size does not change a bit either (one accumulation order)
     a = pkg.hip.linear(dev(x), dev(w))
-    tuned(gemm_tiled_variant=3 - variant)
-    assert torch.equal(a, pkg.hip.linear(dev(x), dev(w)))
+    for other in {1, 2, 3} - {variant}:
+        tuned(gemm_tiled_variant=other)
+        assert torch.equal(a, pkg.hip.linear(dev(x), dev(w))), (variant, other)
 
 
 @pytest.mark.parametrize("N", [16640, 16544])
