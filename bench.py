@@ -91,10 +91,10 @@ def adapter_once_bytes(cfg, batch, elt=2):
     return h * h * elt + batch * h * 4
 
 
-# HBM-side bytes per launch of the tiled mlp.fc GEMM at M = 16384 from rocprofv3 --pmc (FETCH_SIZE 4,445,529 KiB x 1.99974 +
-# WRITE_SIZE 573,440 KiB x 1.0, both scaled by a 256 MiB copy): 8 x the 1.14 GB of operands + output, the panel re-reads
+# HBM-side bytes per launch of the tiled mlp.fc GEMM at M = 16384 from rocprofv3 --pmc (FETCH_SIZE 4,454,542 KiB x 1.99974 +
+# WRITE_SIZE 600,320 KiB x 1.0, both scaled by a 256 MiB copy): 8 x the 1.14 GB of operands + output, the panel re-reads
 # of 256 x 256 tiles in 8 x 4 groups per XCD.  Profiler figures, so constants, with the file that holds the readings.
-TILED_FC_TRAFFIC = int(4445529 * 1024 * 1.99974 + 573440 * 1024)
+TILED_FC_TRAFFIC = int(4454542 * 1024 * 1.99974 + 600320 * 1024)
 TILED_FC_TRAFFIC_SOURCE = "profiles/gemm_tiled_bs4x4096_counters.txt"
 
 
@@ -155,9 +155,9 @@ def prefill_record(pkg, model, B, S, r):
         "value": round(M * r / (ms * 1e-3), 1), "unit": "tokens*iterations/s", "steps": r, "warmup": 1, "ms_per_step": round(ms / r, 3),
         "config": {"workload": f"recurrent-core prefill, nebel-raven-3.5b shape, bs={B} x {S} tokens, {r} timed iterations "
                                f"(BASELINE.json configs[4])",
-                   "batch": B, "seq_len": S, "iterations": r, "gemm": "gemm_tiled_kernel (hand-written MFMA, 256 x 256 tiles)",
+                   "batch": B, "seq_len": S, "iterations": r, "gemm": "gemm_ring_kernel (hand-written MFMA, 256 x 256 tiles, four waves, operands global -> LDS ring)",
                    "attention": "attention_prefill_kernel"},
-        "roofline": {"bound": "mfma", "kernel": f"gemm_tiled_kernel<SwiGLU, 256x256> (mlp.fc {2 * inter}x{h}, M={M})",
+        "roofline": {"bound": "mfma", "kernel": f"gemm_ring_kernel<SwiGLU> 256x256 (mlp.fc {2 * inter}x{h}, M={M})",
                      "achieved": round(fc_tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(fc_tflops / MFMA_PEAK_TFLOPS, 4), "flops_per_launch": fc_flops, "avg_us": round(fc_ms * 1e3, 1),
                      "traffic": TILED_FC_TRAFFIC, "traffic_source": TILED_FC_TRAFFIC_SOURCE},
@@ -345,7 +345,7 @@ def gemm_only(args):
     cases = [("mlp.fc + SwiGLU", mats(2 * inter, h), dict(x=x, swiglu=True)), ("attn.Wqkv", mats(3 * h, h), dict(x=x)),
              ("attn.proj + residual", mats(h, h), dict(x=x, residual=res)), ("mlp.proj + residual", mats(h, inter), dict(x=g, residual=res)),
              ("adapter (two K segments)", mats(h, 2 * h), dict(x=x, x1=e))]
-    out = {"gemm_only": args.gemm_only, "kernel": "gemm_tiled_kernel", "rows": M, "products": {}}
+    out = {"gemm_only": args.gemm_only, "kernel": "gemm_ring_kernel / gemm_tiled_kernel", "rows": M, "products": {}}
     total_ms, total_flops = 0.0, 0.0
     for name, ws, kw in cases:
         xin = kw.pop("x")

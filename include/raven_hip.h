@@ -95,8 +95,10 @@ const char* raven_last_error(void);
  * without a workspace), linear_ks (K slices of the split-K kernel behind raven_linear;
  * non-zero also makes raven_linear use that kernel for every shape it accepts), gemm_tiled_min_rows (fewest rows, 33 or
  * more, that the tiled MFMA kernel takes), gemm_tiled_variant (0 = tile size by shape, 1 = 256 x 256, 2 = 128 x 128 and
- * no tile-count rule), gemm_tiled_split_tail (1 = the tile columns of a last round that fills at most half the chip go to
+ * no tile-count rule, 3 = 256 x 256 by the eight-wave kernel instead of the four-wave ring kernel), gemm_tiled_split_tail
+ * (1 = the tile columns of a last round that fills at most half the chip go to
  * 128 x 128 tiles, 0 = never), prefill_waves (waves per workgroup of the chunk attention at head_dim 96: 0 = by shape, 4 or 6),
+ * attn_prefetch (1 = an unsplit decode-attention launch requests a tile before it uses the one before, 0 = never),
  * gemm_ragged (1 = a 5..32-row product whose output columns divide into about two workgroups per compute unit runs as one
  * round of workgroups with a partly empty last tile, 0 = whole tiles only), norm_early (1 / 0 = the RMSNorm kernel requests
  * its weights before / after the row reduction, -1 = by row count), fuse_sums_norm (1 = a K-split product that feeds a

@@ -4,7 +4,12 @@
 // cat([x, input_embeds]), 711 lm_head), with the epilogues of the skinny kernels: plain, + residual (RMM:534-535),
 // float store (RMM:711), SwiGLU (RMM:507-508).  The concat of RMM:776 is two K segments of the X operand.
 //
-// Shape of the kernel (gfx950):
+// Two kernels: gemm_ring_kernel (further down) multiplies the 256 x 256 tiles; gemm_tiled_kernel, described here, the
+// 128 x 128 tiles (few tiles, and the last tile columns of a launch whose last round would be nearly empty), and the
+// 256 x 256 tiles too when asked to (tuning key gemm_tiled_variant = 3).  Both issue the same products in the same order
+// per accumulator: a result does not depend on which of them computed it.
+//
+// Shape of gemm_tiled_kernel (gfx950):
 //   * a workgroup of 8 waves (2 along the token rows x 4 along the weight rows, two waves per SIMD) owns a BN x BM tile
 //     of Y^T (256 weight rows x 256 token rows in the main variant); a wave owns 2 TN x 2 TM MFMA tiles of 16 x 16
 //     (v_mfma_f32_16x16x32_bf16, W rows as the A operand, X rows as B, so that a lane ends up with 4 neighbouring output
