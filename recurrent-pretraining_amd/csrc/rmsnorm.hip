@@ -26,9 +26,11 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
 // each weight chunk is fetched where it is used, which keeps 32 registers free and more rows in flight per CU: from
 // 1024 rows on the early form is 3-20 % slower (4096 rows: 25.7 against 23.7 us, two norms 31.9 against 26.7).
 //
-// SPLIT: the row is not read from x but formed from the fp32 partial sums a K-split product left behind (gemm_splitk.hip):
-// extra + slice 0 + slice 1 + ... in this order, rounded to T, plus the residual, rounded again -- the arithmetic of that
-// file's second launch, which this launch then replaces.
+// KS > 0: the row is not read from x but formed from the fp32 partial sums of KS slices that a K-split product left behind
+// (gemm_splitk.hip): extra + slice 0 + slice 1 + ... in this order, rounded to T, plus the residual, rounded again -- the
+// arithmetic of that file's second launch, which this launch then replaces.  The slice count is a template argument so
+// that every load of the row (slices, extra, residual) is requested before the first sum: with a run-time loop over the
+// slices each one was a memory round trip of its own, KS + 2 in a row per chunk.
 struct SplitSums {
     const float* partial;  // [ks][rows][dim]
     const float* extra;    // [rows][dim] or null
@@ -36,7 +38,7 @@ struct SplitSums {
     int64_t slice_stride;  // rows * dim
 };
 
-template <typename T, int MC, bool EARLY, bool SPLIT>
+template <typename T, int MC, bool EARLY, int KS>
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
     const T* __restrict__ x, const T* __restrict__ residual, const T* __restrict__ weight, T* __restrict__ y,
     T* __restrict__ sum_out, const T* __restrict__ weight2, T* __restrict__ y2, int dim, float eps, SplitSums sp) {
@@ -61,37 +63,48 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
 
     float v[MC][E];
     float ss = 0.f;
+    constexpr bool SPLIT = KS > 0;
+    constexpr int Q = E / 4;
+    Chunk<T> cxs[MC], crs[MC];
+    f32x4 pv[SPLIT ? MC : 1][SPLIT ? KS + 1 : 1][Q];  // [.][0]: extra, [.][1 + sl]: slice sl
+#pragma unroll
+    for (int i = 0; i < MC; ++i) {
+        const int c = threadIdx.x + i * kNormThreads;
+        if (c < n_chunks) {
+            if constexpr (SPLIT) {
+                const int64_t at = row * dim + c * E;
+#pragma unroll
+                for (int q = 0; q < Q; ++q) {
+                    pv[i][0][q] = sp.extra ? *reinterpret_cast<const f32x4*>(sp.extra + at + 4 * q) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int sl = 0; sl < KS; ++sl) pv[i][1 + sl][q] = *reinterpret_cast<const f32x4*>(sp.partial + sl * sp.slice_stride + at + 4 * q);
+                }
+            } else {
+                cxs[i] = load_chunk(xr + c * E);
+            }
+            if (rr) crs[i] = load_chunk(rr + c * E);
+        }
+    }
 #pragma unroll
     for (int i = 0; i < MC; ++i) {
         const int c = threadIdx.x + i * kNormThreads;
         if (c < n_chunks) {
             Chunk<T> cx;
             if constexpr (SPLIT) {
-                float acc[E];
-                const int64_t at = row * dim + c * E;
 #pragma unroll
-                for (int q = 0; q < E / 4; ++q) {
-                    const f32x4 ex = sp.extra ? *reinterpret_cast<const f32x4*>(sp.extra + at + 4 * q) : f32x4{0.f, 0.f, 0.f, 0.f};
+                for (int q = 0; q < Q; ++q) {
+                    f32x4 acc = pv[i][0][q];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[4 * q + e] = ex[e];
+                    for (int sl = 0; sl < KS; ++sl) acc += pv[i][1 + sl][q];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) cx.v[4 * q + e] = from_f32<T>(acc[e]);
                 }
-                for (int sl = 0; sl < sp.ks; ++sl) {
-#pragma unroll
-                    for (int q = 0; q < E / 4; ++q) {
-                        const f32x4 pv = *reinterpret_cast<const f32x4*>(sp.partial + sl * sp.slice_stride + at + 4 * q);
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[4 * q + e] += pv[e];
-                    }
-                }
-#pragma unroll
-                for (int e = 0; e < E; ++e) cx.v[e] = from_f32<T>(acc[e]);
             } else {
-                cx = load_chunk(xr + c * E);
+                cx = cxs[i];
             }
             if (rr) {
-                Chunk<T> cr = load_chunk(rr + c * E);
 #pragma unroll
-                for (int e = 0; e < E; ++e) cx.v[e] = from_f32<T>(to_f32(cx.v[e]) + to_f32(cr.v[e]));
+                for (int e = 0; e < E; ++e) cx.v[e] = from_f32<T>(to_f32(cx.v[e]) + to_f32(crs[i].v[e]));
             }
             if (sum_out && (rr || SPLIT)) store_chunk(sum_out + row * dim + c * E, cx);
 #pragma unroll
@@ -145,8 +158,17 @@ int splitk_sums_then_norm(const float* partial, int ks, const float* extra, cons
     RAVEN_REQUIRE(partial && ks >= 1 && weight && (y || y2) && (weight2 == nullptr) == (y2 == nullptr), "splitk_sums_then_norm: bad arguments");
     RAVEN_REQUIRE(rows >= 1 && dim % 8 == 0 && dim / 8 <= kNormThreads * 4, "splitk_sums_then_norm: unsupported shape %d x %d", rows, dim);
     SplitSums sp{partial, extra, ks, (int64_t)rows * dim};
-    rmsnorm_kernel<bf16, 4, true, true><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(
-        nullptr, (const bf16*)residual, (const bf16*)weight, (bf16*)y, (bf16*)sum_out, (const bf16*)weight2, (bf16*)y2, dim, eps, sp);
+#define RAVEN_SPLIT_NORM(KS_)                                                                                            \
+    case KS_:                                                                                                           \
+        rmsnorm_kernel<bf16, 4, true, KS_><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                          \
+            nullptr, (const bf16*)residual, (const bf16*)weight, (bf16*)y, (bf16*)sum_out, (const bf16*)weight2, (bf16*)y2, dim, eps, sp); \
+        break;
+    switch (ks) {
+        RAVEN_SPLIT_NORM(1) RAVEN_SPLIT_NORM(2) RAVEN_SPLIT_NORM(3) RAVEN_SPLIT_NORM(4)
+        RAVEN_SPLIT_NORM(5) RAVEN_SPLIT_NORM(6) RAVEN_SPLIT_NORM(7) RAVEN_SPLIT_NORM(8)
+        default: RAVEN_REQUIRE(false, "splitk_sums_then_norm: %d slices (at most 8)", ks);
+    }
+#undef RAVEN_SPLIT_NORM
     return raven_host::check_launch("split-K sums + rmsnorm");
 }
 
@@ -173,10 +195,10 @@ extern "C" int raven_rmsnorm_residual(const void* x, const void* residual, const
 #define RAVEN_NORM_LAUNCH(T_, MC_)                                                                                           \
     do {                                                                                                                     \
         if (early)                                                                                                           \
-            rmsnorm_kernel<T_, MC_, true, false><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                        \
+            rmsnorm_kernel<T_, MC_, true, 0><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                        \
                 (const T_*)x, (const T_*)residual, (const T_*)weight, (T_*)y, (T_*)sum_out, (const T_*)weight2, (T_*)y2, dim, eps, none); \
         else                                                                                                                 \
-            rmsnorm_kernel<T_, MC_, false, false><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                       \
+            rmsnorm_kernel<T_, MC_, false, 0><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                       \
                 (const T_*)x, (const T_*)residual, (const T_*)weight, (T_*)y, (T_*)sum_out, (const T_*)weight2, (T_*)y2, dim, eps, none); \
     } while (0)
     if (dtype == RAVEN_BF16) {
