@@ -102,7 +102,10 @@ const char* raven_last_error(void);
  * gemm_ragged (1 = a 5..32-row product whose output columns divide into about two workgroups per compute unit runs as one
  * round of workgroups with a partly empty last tile, 0 = whole tiles only), norm_early (1 / 0 = the RMSNorm kernel requests
  * its weights before / after the row reduction, -1 = by row count), fuse_sums_norm (1 = a K-split product that feeds a
- * norm leaves its slices to that norm's launch, which adds them in the same order; 0 = a launch of its own adds them).
+ * norm leaves its slices to that norm's launch, which adds them in the same order; 0 = a launch of its own adds them),
+ * fuse_qkv_rope (1 = inside raven_sandwich_block / raven_core_iteration(s) a chunk's q | k | v product on the tiled GEMM
+ * applies bias, RoPE and the cache append in its epilogue; 0 = the product is stored and raven_qkv_bias_rope_cache_append's
+ * kernel follows; same bits either way).
  * Not needed in normal use: the defaults are the tuned values.  The knobs are process-global
  * state read at every launch: changing them while another thread or stream is inside a call of this library is a race. */
 int raven_set_tuning(const char* key, int32_t value);

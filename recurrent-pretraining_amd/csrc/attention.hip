@@ -20,19 +20,6 @@
 
 namespace raven {
 
-// One RoPE pair, adjacent elements (recpre/raven_modeling_minimal.py:118-131): products and sums rounded one by one in
-// fp32, as the reference's separate elementwise kernels do; every kernel that rotates uses this one function, so that
-// the fused and the two-launch paths write the same bits.
-template <typename T>
-__device__ __forceinline__ void rope_pair(T& a, T& b, float cs, float sn) {
-#pragma clang fp contract(off)
-    const float x0 = to_f32(a), x1 = to_f32(b);
-    const float r0 = x0 * cs - x1 * sn;
-    const float r1 = x1 * cs + x0 * sn;
-    a = from_f32<T>(r0);
-    b = from_f32<T>(r1);
-}
-
 struct CacheView {
     void* k;
     void* v;
@@ -783,6 +770,32 @@ extern "C" int raven_qkv_bias_rope_cache_append(const void* qkv, const void* qk_
     return raven_host::check_launch("qkv_append");
 }
 
+namespace raven {
+extern int g_tiled_min_rows;
+bool tiled_gemm_fits(int M, int N, int K0, int K1, int dtype);
+int tiled_gemm_qkv_rope(const void* x, const void* wqkv, const void* qk_bias, const float* freqs, void* q_out, void* k_cache,
+                        void* v_cache, int64_t slot_off, int nh, int hd, int t_max, int M, int S, int K, int pos0, const int* pos_dev,
+                        hipStream_t s);
+int g_fuse_qkv_rope = 1;  // raven_set_tuning("fuse_qkv_rope"): 0 = a chunk's q | k | v product is stored and rotated by a launch of its own
+
+// A chunk's Wqkv product with raven_qkv_bias_rope_cache_append as its epilogue (bf16 shapes that take the tiled GEMM):
+// *done = 0 and nothing launched when the shape does not take that path.
+int qkv_linear_rope_append(const void* x, const void* wqkv, const void* qk_bias, const float* freqs, void* q_out,
+                           const raven_kv_cache* cache, int slot, int B, int S, int pos0, const int32_t* pos_dev, int n_heads,
+                           int head_dim, int dtype, hipStream_t s, int* done) {
+    *done = 0;
+    const int M = B * S, h = n_heads * head_dim;
+    if (!g_fuse_qkv_rope || dtype != RAVEN_BF16 || M < g_tiled_min_rows || head_dim % 8 != 0 || !tiled_gemm_fits(M, 3 * h, h, 0, dtype)) return 0;
+    if (int rc = check_heads("qkv_append", n_heads, head_dim, dtype)) return rc;
+    RAVEN_REQUIRE(x && wqkv && freqs && q_out, "qkv_append: null pointer");
+    RAVEN_REQUIRE(B > 0 && S > 0 && pos0 >= 0, "qkv_append: bad B=%d S=%d pos0=%d", B, S, pos0);
+    CacheView cv;
+    if (int rc = make_view("qkv_append", cache, slot, B, n_heads, head_dim, &cv)) return rc;
+    RAVEN_REQUIRE(pos0 + S <= cv.t_max, "qkv_append: positions %d..%d exceed the cache length %d", pos0, pos0 + S - 1, cv.t_max);
+    *done = 1;
+    return tiled_gemm_qkv_rope(x, wqkv, qk_bias, freqs, q_out, cv.k, cv.v, cv.slot_off, cv.nh, cv.hd, cv.t_max, M, S, h, pos0, pos_dev, s);
+}
+}  // namespace raven
 
 template <typename T>
 static void launch_attention(bool fused, const void* q, const void* bias, const float* freqs, void* y, const raven::CacheView& cv,

@@ -33,6 +33,10 @@ int linear_leave_sums(const void* x0, const void* x1, const void* w, int ldw, co
 int splitk_sums_then_norm(const float* partial, int ks, const float* extra, const void* residual, void* sum_out, const void* weight,
                           void* y, const void* weight2, void* y2, int rows, int dim, float eps, hipStream_t s);
 
+int qkv_linear_rope_append(const void* x, const void* wqkv, const void* qk_bias, const float* freqs, void* q_out,
+                           const raven_kv_cache* cache, int slot, int B, int S, int pos0, const int32_t* pos_dev, int n_heads,
+                           int head_dim, int dtype, hipStream_t s, int* done);
+
 // y = round(round(x W^T) + residual), then RMSNorm(weight) -> out1 and RMSNorm(weight2) of that -> out2 (either may be
 // null): two launches where the product is K-split (the norm launch adds the slices), three otherwise
 static int linear_then_norm(const void* x, const void* w, const void* residual, void* y, const void* weight, void* out1,
@@ -116,7 +120,13 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
     int rc;
     if (!n1_ready)
         if ((rc = raven_rmsnorm_residual(x_in, nullptr, w->norm_1, s.n1, nullptr, nullptr, nullptr, M, h, d->eps, dt, stream))) return rc;
-    if ((rc = raven_linear(s.n1, nullptr, w->wqkv, nullptr, s.qkv, M, 3 * h, h, 0, 0, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
+    // a chunk of tokens on the tiled GEMM: bias, RoPE and the cache append are that product's epilogue
+    int qkv_done = 0;
+    if (!paged && S > 1)
+        if ((rc = qkv_linear_rope_append(s.n1, w->wqkv, w->qk_bias, freqs, s.q, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim,
+                                         dt, static_cast<hipStream_t>(stream), &qkv_done))) return rc;
+    if (!qkv_done)
+        if ((rc = raven_linear(s.n1, nullptr, w->wqkv, nullptr, s.qkv, M, 3 * h, h, 0, 0, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
     if (paged) {   // decode over block-paged caches, every sequence at its own position
         if ((rc = raven_paged_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, paged->k_caches[layer], paged->v_caches[layer],
                                                    paged->block_table, paged->seq_lens, B, paged->max_blocks, paged->block_size,
@@ -125,8 +135,9 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
         if ((rc = raven_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, cache, slot, B, pos0, pos_dev, d->n_heads,
                                              d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream))) return rc;
     } else {       // a chunk of S tokens: every row's keys must be in the cache before any row attends
-        if ((rc = raven_qkv_bias_rope_cache_append(s.qkv, w->qk_bias, freqs, s.q, cache, slot, B, S, pos0, pos_dev, d->n_heads,
-                                                   d->head_dim, dt, stream))) return rc;
+        if (!qkv_done)
+            if ((rc = raven_qkv_bias_rope_cache_append(s.qkv, w->qk_bias, freqs, s.q, cache, slot, B, S, pos0, pos_dev, d->n_heads,
+                                                       d->head_dim, dt, stream))) return rc;
         // chunks of 16 or more rows per sequence: 64 or 128 query rows of a head per workgroup on the matrix cores; a few
         // rows per sequence (or a partially filled cache, which only that kernel looks up): one row at a time
         const bool mfma = dt == RAVEN_BF16 && S >= 16 && (d->head_dim == 64 || d->head_dim == 96 || d->head_dim == 128) &&

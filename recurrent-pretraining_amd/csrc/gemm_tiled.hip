@@ -58,6 +58,20 @@ struct TiledArgs {
     int up_off;            // SwiGLU: weight rows between a gate row and its up row (the whole matrix's I)
     int out_f32;
     int tiles_m, tiles_n;
+    int rope_on;           // the epilogue below instead of y
+    // The product is a chunk's fused q | k | v rows (3 * nh * hd columns): instead of y, the epilogue adds the q / k bias,
+    // rotates q and k (RoPE on adjacent pairs) and writes q to q_out and k, v to their cache rows -- what
+    // qkv_rope_append_tiled_kernel (attention.hip) does to a stored product, with the same functions in the same order.
+    struct RopeAppend {
+        const float* freqs;
+        const bf16* qk_bias;   // [2, nh * hd] or null
+        bf16* q_out;           // [M, nh * hd]
+        bf16 *k, *v;           // cache tensors, [.., batch, nh, t_max, hd] from slot_off on
+        int64_t slot_off;
+        const int* pos_dev;    // position of a sequence's first row, on the device (or null: pos0)
+        int nh, hd, t_max, S, pos0;
+        int col0;              // column of the whole product that this launch's column 0 is
+    } rope;
 };
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -121,31 +135,14 @@ __device__ __forceinline__ void store_tiles(const TiledArgs& a, const f32x4 (&ac
     }
 }
 
-// Epilogue through LDS for the bf16 outputs: the accumulators (a lane: 4 columns of one token row per store, a wave
-// instruction 16 token rows) are laid down as the output tile, rows of BN_OUT columns, and read back so that a wave
-// instruction stores two whole tile rows, 16 bytes per lane: full 128-byte lines instead of pieces of 8 bytes.  The
-// residual is fetched the same way, before the tile is laid down, so that its latency hides behind the transposition.
-// 16-byte unit u of tile row r sits at position u ^ (r mod units per row): the 16 rows a store instruction spreads over
-// then fall on different banks.
-template <bool SWIGLU, int TM, int TN, int WM = 2, int WN = 4>
-__device__ __forceinline__ void store_tiles_lds(const TiledArgs& a, const f32x4 (&acc)[2 * TN][2 * TM], int tile_m, int tile_n, int wave,
-                                                int lane, unsigned lds_base) {
-    constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
+// The accumulators of a workgroup laid down in LDS as the output tile (rows of BN_OUT columns, 16-byte unit u of row r at
+// position u ^ (r mod units per row)), between two workgroup barriers: the first because the K loop's stages are reused.
+template <bool SWIGLU, int TM, int TN, int WM, int WN>
+__device__ __forceinline__ void lay_tiles_lds(const f32x4 (&acc)[2 * TN][2 * TM], int wave, int lane, unsigned lds_base) {
+    constexpr int BN = WN * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
     constexpr int NA = 2 * TN, NB = 2 * TM, NT = SWIGLU ? TN : NA;
-    constexpr int RB = BN_OUT * 2, U = RB / 16;      // bytes and 16-byte units per tile row
-    constexpr int ITERS = BM * U / (64 * WM * WN);    // 16-byte units per lane
+    constexpr int RB = BN_OUT * 2, U = RB / 16;
     const int wn = wave % WN, wm = wave / WN, l16 = lane & 15, q4 = lane >> 4;
-    bf16* const y = static_cast<bf16*>(a.y);
-    int64_t goff[ITERS];                             // element offset of this lane's unit in y / residual, -1: outside
-    u32x4 res[ITERS];
-#pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-        const int idx = (wave * ITERS + it) * 64 + lane;
-        const int m = tile_m * BM + idx / U, n = tile_n * BN_OUT + (idx % U) * 8;
-        goff[it] = (m < a.M && n < a.N) ? (int64_t)m * a.ldy + n : -1;
-        res[it] = u32x4{0, 0, 0, 0};
-        if (!SWIGLU && a.residual && goff[it] >= 0) res[it] = *reinterpret_cast<const u32x4*>(a.residual + goff[it]);
-    }
     // every wave has its last fragments; the stages are free
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
@@ -174,6 +171,34 @@ __device__ __forceinline__ void store_tiles_lds(const TiledArgs& a, const f32x4 
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+}
+
+// Epilogue through LDS for the bf16 outputs: the accumulators (a lane: 4 columns of one token row per store, a wave
+// instruction 16 token rows) are laid down as the output tile, rows of BN_OUT columns, and read back so that a wave
+// instruction stores two whole tile rows, 16 bytes per lane: full 128-byte lines instead of pieces of 8 bytes.  The
+// residual is fetched the same way, before the tile is laid down, so that its latency hides behind the transposition.
+// 16-byte unit u of tile row r sits at position u ^ (r mod units per row): the 16 rows a store instruction spreads over
+// then fall on different banks.
+template <bool SWIGLU, int TM, int TN, int WM = 2, int WN = 4>
+__device__ __forceinline__ void store_tiles_lds(const TiledArgs& a, const f32x4 (&acc)[2 * TN][2 * TM], int tile_m, int tile_n, int wave,
+                                                int lane, unsigned lds_base) {
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BN_OUT = SWIGLU ? BN / 2 : BN;
+    constexpr int NA = 2 * TN, NB = 2 * TM, NT = SWIGLU ? TN : NA;
+    constexpr int RB = BN_OUT * 2, U = RB / 16;      // bytes and 16-byte units per tile row
+    constexpr int ITERS = BM * U / (64 * WM * WN);    // 16-byte units per lane
+    const int wn = wave % WN, wm = wave / WN, l16 = lane & 15, q4 = lane >> 4;
+    bf16* const y = static_cast<bf16*>(a.y);
+    int64_t goff[ITERS];                             // element offset of this lane's unit in y / residual, -1: outside
+    u32x4 res[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int idx = (wave * ITERS + it) * 64 + lane;
+        const int m = tile_m * BM + idx / U, n = tile_n * BN_OUT + (idx % U) * 8;
+        goff[it] = (m < a.M && n < a.N) ? (int64_t)m * a.ldy + n : -1;
+        res[it] = u32x4{0, 0, 0, 0};
+        if (!SWIGLU && a.residual && goff[it] >= 0) res[it] = *reinterpret_cast<const u32x4*>(a.residual + goff[it]);
+    }
+    lay_tiles_lds<SWIGLU, TM, TN, WM, WN>(acc, wave, lane, lds_base);
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
         const int idx = (wave * ITERS + it) * 64 + lane;
@@ -188,6 +213,79 @@ __device__ __forceinline__ void store_tiles_lds(const TiledArgs& a, const f32x4 
             v = *reinterpret_cast<const u32x4*>(o);
         }
         if (goff[it] >= 0) *reinterpret_cast<u32x4*>(y + goff[it]) = v;
+    }
+}
+
+// Epilogue of a chunk's q | k | v product (TiledArgs::rope): the tile goes through LDS as above; each 16-byte unit (8
+// columns of one head, of one token row) then gets the q / k bias and the rotation and goes to q_out or to its cache row.
+// A lane's units all lie in the same 8 columns, so section, head and bias are fixed per lane; the (cos, sin) pairs of a
+// unit's position are requested eight units ahead (the first eight before the tile is laid down).
+template <int TM, int TN, int WM, int WN>
+__device__ __forceinline__ void store_tiles_rope(const TiledArgs& a, const f32x4 (&acc)[2 * TN][2 * TM], int tile_m, int tile_n, int wave,
+                                                 int lane, unsigned lds_base) {
+    constexpr int BM = WM * TM * 32, BN_OUT = WN * TN * 32;
+    constexpr int RB = BN_OUT * 2, U = RB / 16, RS = 64 / U;  // rows a wave instruction covers
+    constexpr int ITERS = BM * U / (64 * WM * WN);
+    constexpr int PD = ITERS < 8 ? ITERS : 8;
+    // read from the kernel's argument block here, through a pointer the compiler cannot trace: as ordinary kernel
+    // arguments the fields are fetched at the top and held in scalar registers through the K loop
+    const char __attribute__((address_space(4)))* ka = (const char __attribute__((address_space(4)))*)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(ka));
+    TiledArgs::RopeAppend r;
+#define RAVEN_ROPE_FIELD(F_) r.F_ = *reinterpret_cast<const decltype(r.F_) __attribute__((address_space(4)))*>(ka + offsetof(TiledArgs, rope) + offsetof(TiledArgs::RopeAppend, F_))
+    RAVEN_ROPE_FIELD(freqs); RAVEN_ROPE_FIELD(qk_bias); RAVEN_ROPE_FIELD(q_out); RAVEN_ROPE_FIELD(k); RAVEN_ROPE_FIELD(v);
+    RAVEN_ROPE_FIELD(slot_off); RAVEN_ROPE_FIELD(pos_dev); RAVEN_ROPE_FIELD(nh); RAVEN_ROPE_FIELD(hd); RAVEN_ROPE_FIELD(t_max);
+    RAVEN_ROPE_FIELD(S); RAVEN_ROPE_FIELD(pos0); RAVEN_ROPE_FIELD(col0);
+#undef RAVEN_ROPE_FIELD
+    const int unit = lane % U, row0 = wave * ITERS * RS + lane / U;
+    const int n_local = tile_n * BN_OUT + unit * 8;
+    const bool col_ok = n_local < a.N;
+    const int h = r.nh * r.hd;
+    const int n = col_ok ? r.col0 + n_local : 0;
+    const int sec = n >= 2 * h ? 2 : (n >= h ? 1 : 0);   // q, k or v columns
+    const int col = n - sec * h, head = col / r.hd, d = col - head * r.hd;
+    const int first = r.pos_dev ? *r.pos_dev : r.pos0;
+    Chunk<bf16> bch = zero_chunk<bf16>();
+    if (sec < 2 && r.qk_bias) bch = load_chunk(r.qk_bias + sec * h + col);
+    auto where = [&](int it, int& m, int& b, int& pos) {
+        m = min(tile_m * BM + row0 + it * RS, a.M - 1);
+        b = m / r.S;
+        pos = first + (m - b * r.S);
+    };
+    f32x4 fq[PD][2];
+    auto request = [&](int it, f32x4 (&f)[2]) {
+        int m, b, pos;
+        where(it, m, b, pos);
+        const float* fp = r.freqs + ((int64_t)pos * (r.hd / 2) + d / 2) * 2;
+        f[0] = *reinterpret_cast<const f32x4*>(fp);
+        f[1] = *reinterpret_cast<const f32x4*>(fp + 4);
+    };
+#pragma unroll
+    for (int it = 0; it < PD; ++it) request(it, fq[it]);
+    lay_tiles_lds<false, TM, TN, WM, WN>(acc, wave, lane, lds_base);
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int row = row0 + it * RS;
+        const u32x4 v = *reinterpret_cast<const lds_u32x4*>(lds_base + row * RB + ((unit ^ (row & (U - 1))) * 16));
+        int m, b, pos;
+        where(it, m, b, pos);
+        Chunk<bf16> x;
+        *reinterpret_cast<u32x4*>(x.v) = v;
+        const f32x4 f0 = fq[it % PD][0], f1 = fq[it % PD][1];
+        if (it + PD < ITERS) request(it + PD, fq[it % PD]);
+        if (sec < 2) {
+            if (r.qk_bias) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x.v[e] = from_f32<bf16>(to_f32(x.v[e]) + to_f32(bch.v[e]));
+            }
+            rope_pair<bf16>(x.v[0], x.v[1], f0[0], f0[1]);
+            rope_pair<bf16>(x.v[2], x.v[3], f0[2], f0[3]);
+            rope_pair<bf16>(x.v[4], x.v[5], f1[0], f1[1]);
+            rope_pair<bf16>(x.v[6], x.v[7], f1[2], f1[3]);
+        }
+        if (!col_ok || tile_m * BM + row >= a.M) continue;
+        if (sec == 0) store_chunk(r.q_out + (int64_t)m * h + col, x);
+        else if (pos < r.t_max) store_chunk((sec == 1 ? r.k : r.v) + r.slot_off + (((int64_t)b * r.nh + head) * r.t_max + pos) * r.hd + d, x);
     }
 }
 
@@ -416,6 +514,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(TiledArgs a) {
     run(e1, e2, std::false_type{});
     run(e2, e3, std::true_type{});
     run(e3, nk, std::false_type{});
+    if constexpr (!SWIGLU) {
+        if (a.rope_on) {  // uniform over the launch
+            store_tiles_rope<TM, TN, WM, WN>(a, acc, tile_m, tile_n, wave, lane, lds_base);
+            return;
+        }
+    }
     if (a.out_f32) store_tiles<SWIGLU, TM, TN, WM, WN>(a, acc, tile_m, tile_n, wm, wn, l16, q4);
     else store_tiles_lds<SWIGLU, TM, TN, WM, WN>(a, acc, tile_m, tile_n, wave, lane, lds_base);
 }
@@ -616,6 +720,12 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(TiledArgs a) {
     run(e3, nk, std::false_type{});
     // requests past the last step still write into the ring, and the last products must land before their tiles are read
     asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    if constexpr (!SWIGLU) {
+        if (a.rope_on) {  // uniform over the launch
+            store_tiles_rope<TM, TN, WM, WN>(a, acc, tile_m, tile_n, wave, lane, lds_base);
+            return;
+        }
+    }
     if (a.out_f32) store_tiles<SWIGLU, TM, TN, WM, WN>(a, acc, tile_m, tile_n, wm, wn, l16, q4);
     else store_tiles_lds<SWIGLU, TM, TN, WM, WN>(a, acc, tile_m, tile_n, wave, lane, lds_base);
 }
@@ -681,8 +791,8 @@ bool tiled_gemm_fits(int M, int N, int K0, int K1, int dtype) {
            (int64_t)N * 2 * (K0 + K1) < (1ll << 31);
 }
 
-int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residual, void* y, int M, int N, int K0, int K1, int swiglu,
-               int out_f32, hipStream_t s) {
+static int tiled_gemm_impl(const void* x0, const void* x1, const void* w, const void* residual, void* y, int M, int N, int K0, int K1,
+                           int swiglu, int out_f32, const TiledArgs::RopeAppend* rope, hipStream_t s) {
     RAVEN_REQUIRE(tiled_gemm_fits(M, N, K0, K1, RAVEN_BF16), "gemm (tiled): unsupported shape M=%d N=%d K0=%d K1=%d", M, N, K0, K1);
     RAVEN_REQUIRE(!(swiglu && (residual || out_f32)), "gemm (tiled): the SwiGLU epilogue has no residual and stores bf16");
     RAVEN_REQUIRE(((uintptr_t)x0 & 15) == 0 && ((uintptr_t)x1 & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)y & 15) == 0 &&
@@ -696,6 +806,10 @@ int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residu
     a.M = M; a.N = N; a.K0 = K0; a.K1 = x1 ? K1 : 0; a.out_f32 = out_f32;
     a.ldy = N;
     a.up_off = N;
+    if (rope) {
+        a.rope = *rope;
+        a.rope_on = 1;
+    }
     // 256 x 256 tiles when they fill the chip at least once; 128 x 128 tiles otherwise
     const int bn_out = swiglu ? 128 : 256;
     const int64_t tiles_n = (N + bn_out - 1) / bn_out, tiles_m = (M + 255) / 256;
@@ -722,10 +836,35 @@ int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residu
         tail.w = a.w + (int64_t)n_big * (K0 + a.K1);
         tail.residual = a.residual ? a.residual + n_big : nullptr;
         tail.y = out_f32 ? static_cast<void*>(static_cast<float*>(y) + n_big) : static_cast<void*>(static_cast<bf16*>(y) + n_big);
+        tail.rope.col0 = n_big;
         const int rc = launch(head, true);
         return rc ? rc : launch(tail, false);
     }
     return launch(a, big);
+}
+
+int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residual, void* y, int M, int N, int K0, int K1, int swiglu,
+               int out_f32, hipStream_t s) {
+    return tiled_gemm_impl(x0, x1, w, residual, y, M, N, K0, K1, swiglu, out_f32, nullptr, s);
+}
+
+// A chunk's q | k | v product (wqkv: [3 * nh * hd, K]) whose epilogue adds the q / k bias, applies RoPE and writes q to
+// q_out [M, nh * hd] and k, v to the cache rows of positions pos0 (or *pos_dev) + 0 .. S - 1 of each of the M / S sequences:
+// the product itself is never stored.  k_cache / v_cache: the cache tensors, slot_off the slot's element offset.
+int tiled_gemm_qkv_rope(const void* x, const void* wqkv, const void* qk_bias, const float* freqs, void* q_out, void* k_cache,
+                        void* v_cache, int64_t slot_off, int nh, int hd, int t_max, int M, int S, int K, int pos0, const int* pos_dev,
+                        hipStream_t s) {
+    RAVEN_REQUIRE(freqs && q_out && k_cache && v_cache && hd % 8 == 0 && S > 0 && M % S == 0, "gemm (tiled, q/k/v epilogue): bad arguments");
+    TiledArgs::RopeAppend r{};
+    r.freqs = freqs;
+    r.qk_bias = static_cast<const bf16*>(qk_bias);
+    r.q_out = static_cast<bf16*>(q_out);
+    r.k = static_cast<bf16*>(k_cache);
+    r.v = static_cast<bf16*>(v_cache);
+    r.slot_off = slot_off;
+    r.pos_dev = pos_dev;
+    r.nh = nh; r.hd = hd; r.t_max = t_max; r.S = S; r.pos0 = pos0; r.col0 = 0;
+    return tiled_gemm_impl(x, nullptr, wqkv, nullptr, nullptr, M, 3 * nh * hd, K, 0, 0, 0, &r, s);
 }
 
 }  // namespace raven

@@ -114,6 +114,19 @@ __device__ __forceinline__ float wave_max(float v) {
 // inside the fp32 bar, and a true division costs five times the instructions in the SwiGLU epilogue of a 256 x 256 tile.
 __device__ __forceinline__ float silu_f32(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
+// One RoPE pair, adjacent elements (recpre/raven_modeling_minimal.py:118-131): products and sums rounded one by one in
+// fp32, as the reference's separate elementwise kernels do; every kernel that rotates uses this one function, so that
+// the fused and the two-launch paths write the same bits.
+template <typename T>
+__device__ __forceinline__ void rope_pair(T& a, T& b, float cs, float sn) {
+#pragma clang fp contract(off)
+    const float x0 = to_f32(a), x1 = to_f32(b);
+    const float r0 = x0 * cs - x1 * sn;
+    const float r1 = x1 * cs + x0 * sn;
+    a = from_f32<T>(r0);
+    b = from_f32<T>(r1);
+}
+
 }  // namespace raven
 
 // ---- host side ------------------------------------------------------------------------------

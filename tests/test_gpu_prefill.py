@@ -289,6 +289,47 @@ def test_sandwich_block_config4_rows(pkg):
     assert not torch.equal(out.view(B, S, H)[0], out.view(B, S, H)[b])
 
 
+@pytest.mark.parametrize("nh,hd,B,S,pos0,on_device", [(5, 96, 3, 50, 7, False), (55, 96, 2, 600, 0, True), (22, 128, 4, 512, 3, False),
+                                                       (3, 64, 1, 33, 0, False)])
+def test_chunk_qkv_epilogue_writes_the_bits_of_the_two_launch_path(pkg, tuned, nh, hd, B, S, pos0, on_device):
+    """A chunk's q | k | v product with bias, RoPE and the cache append as its epilogue (fuse_qkv_rope = 1, the default) against
+    the stored product followed by raven_qkv_bias_rope_cache_append (RMM:463-481): block output and the K / V rows the block
+    appended, bit for bit.  Shapes: 128 x 128 tiles with rows of three sequences in one tile and heads across tile edges;
+    256 x 256 tiles at the 3.5b head layout with the first position on the device; 256 x 256 tiles whose last tile column
+    goes to 128 x 128 tiles (2048 rows x 8448 columns: 264 tiles); a single small tile with rows and columns past the end."""
+    dt, h, inter = torch.bfloat16, nh * hd, 256
+    g = torch.Generator().manual_seed(nh * 1000 + S)
+    norms = [(torch.randn(h, generator=g) * 0.02 + 1).to(dt).cuda() for _ in range(4)]
+    wqkv = (torch.randn(3 * h, h, generator=g) * 0.02).to(dt).cuda()
+    bias = (torch.randn(2, 1, nh, hd, generator=g) * 0.02).to(dt).cuda()
+    proj = (torch.randn(h, h, generator=g) * 0.02).to(dt).cuda()
+    fc = (torch.randn(2 * inter, h, generator=g) * 0.02).to(dt).cuda()
+    mproj = (torch.randn(h, inter, generator=g) * 0.02).to(dt).cuda()
+    x = _gpu_randn((B * S, h), 5)
+    t_max = pos0 + S + 3
+    freqs = O.rope_table(hd, t_max, 50000).to(dt).float().reshape(t_max, hd // 2, 2).contiguous().cuda()
+    dims = pkg.hip.make_dims(h, nh, inter, 1e-6, dt)
+    blk = pkg.hip.make_block_weights(*norms, wqkv, bias, proj, fc, mproj)
+    ws = pkg.hip.block_workspace(dims, B * S, "cuda")
+    pos_dev = torch.tensor([pos0], dtype=torch.int32, device="cuda") if on_device else None
+    results = []
+    for fuse in (1, 0):
+        tuned(fuse_qkv_rope=fuse)
+        kd = _gpu_randn((2, B, nh, t_max, hd), 6)     # rows outside pos0 .. pos0 + S - 1 must stay as they are
+        vd = _gpu_randn((2, B, nh, t_max, hd), 7)
+        cache = pkg.hip.make_cache(kd, vd)
+        out = pkg.hip.sandwich_block(dims, blk, x, torch.empty_like(x), freqs, cache, 1, B, S, pos0, ws, pos_dev=pos_dev)
+        torch.cuda.synchronize()
+        results.append((out.clone(), kd, vd))
+    (o1, k1, v1), (o0, k0, v0) = results
+    assert torch.equal(k1, k0), "appended K differs between the epilogue and the two-launch path"
+    assert torch.equal(v1, v0), "appended V differs"
+    assert torch.equal(o1, o0), "block output differs"
+    fresh = _gpu_randn((2, B, nh, t_max, hd), 6)
+    assert torch.equal(k1[0], fresh[0]) and torch.equal(k1[1, :, :, :pos0], fresh[1, :, :, :pos0]) and torch.equal(k1[1, :, :, pos0 + S:], fresh[1, :, :, pos0 + S:])
+    assert not torch.equal(k1[1, :, :, pos0:pos0 + S], fresh[1, :, :, pos0:pos0 + S])
+
+
 def test_bench_prefill_iteration_runs_through_the_c_abi(pkg):
     """One recurrence over 4 x 512 rows through raven_core_iteration (adapter with two K segments, four blocks, chunk
     attention over a cache that already holds 512 positions): determinism, and the call equals adapter + four
