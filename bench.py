@@ -60,6 +60,8 @@ def parse():
                     help="with --prefill: launch each of the five products of a core iteration N times at the prefill shape and time it")
     ap.add_argument("--library-gemm", action="store_true",
                     help="with --prefill --gemm-only: also time torch.matmul (the vendor library) on each product's operands, as a yardstick")
+    ap.add_argument("--plain-weights", action="store_true",
+                    help="with --prefill: the tiled GEMMs read the weight matrices as given instead of line-aligned copies of them")
     ap.add_argument("--kernel-only", type=int, default=0, metavar="N",
                     help="run only N launches of the dominant kernel plus one 256 MiB device copy (for rocprofv3 --pmc runs)")
     return ap.parse_args()
@@ -174,7 +176,10 @@ def prefill(args):
     pkg.hip.load()
     model = pkg.RavenForCausalLM(pkg.RavenConfig(), device=torch.device("cuda:0"), dtype=torch.bfloat16)
     fill_synthetic(model, 0)
+    model.pack_chunk_weights = not args.plain_weights
     rec = prefill_record(pkg, model, args.prefill_batch, args.prefill_len, args.recurrence)
+    rec["config"]["weights"] = ("as loaded" if args.plain_weights else
+                                "Wqkv, attn.proj, mlp.fc read through line-aligned copies made once (raven_register_packed_weight)")
     line = {"metric": "core prefill tokens*iterations/s, raven-3.5b shape bf16; MFMA utilisation", "value": rec["value"],
             "unit": rec["unit"], "n_gpus": 1, "steps": rec["steps"], "warmup": rec["warmup"], "ms_per_step": rec["ms_per_step"],
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -345,10 +350,15 @@ def gemm_only(args):
     cases = [("mlp.fc + SwiGLU", mats(2 * inter, h), dict(x=x, swiglu=True)), ("attn.Wqkv", mats(3 * h, h), dict(x=x)),
              ("attn.proj + residual", mats(h, h), dict(x=x, residual=res)), ("mlp.proj + residual", mats(h, inter), dict(x=g, residual=res)),
              ("adapter (two K segments)", mats(h, 2 * h), dict(x=x, x1=e))]
-    out = {"gemm_only": args.gemm_only, "kernel": "gemm_ring_kernel / gemm_tiled_kernel", "rows": M, "products": {}}
+    out = {"gemm_only": args.gemm_only, "kernel": "gemm_ring_kernel / gemm_tiled_kernel", "rows": M, "products": {},
+           "weights": "as given ([N, K] rows K elements apart)" if args.plain_weights else
+                      "line-aligned copies (raven_register_packed_weight) of the matrices with K = 5280, as the model makes them for prompt chunks"}
     total_ms, total_flops = 0.0, 0.0
+    keep = []
     for name, ws, kw in cases:
         xin = kw.pop("x")
+        if not args.plain_weights and (ws[0].shape[1] * 2) % 128 != 0:
+            keep += [pkg.hip.register_packed_weight(w) for w in ws]
 
         def launch(i=[0]):
             i[0] += 1
@@ -370,7 +380,25 @@ def gemm_only(args):
 
             lib_ms = event_time_ms(lib_launch, args.gemm_only, warm=2)
             out["products"][name]["library_matmul_no_epilogue"] = {"ms": round(lib_ms, 4), "TFLOP/s": round(flops / lib_ms / 1e9, 1)}
+            if (ws[0].shape[1] * 2) % 128 != 0:  # and with the weight rows a whole number of lines apart, as the packed copies are
+                K, ld = ws[0].shape[1], (ws[0].shape[1] + 63) // 64 * 64
+                padded = []
+                for w in ws:
+                    wp = torch.zeros(w.shape[0], ld, device=dev, dtype=w.dtype)
+                    wp[:, :K] = w
+                    padded.append(wp[:, :K])
+
+                def lib_padded(i=[0]):
+                    i[0] += 1
+                    torch.matmul(xin, padded[i[0] % 4].t())
+
+                lib_ms = event_time_ms(lib_padded, args.gemm_only, warm=2)
+                out["products"][name]["library_matmul_padded_rows"] = {"ms": round(lib_ms, 4), "TFLOP/s": round(flops / lib_ms / 1e9, 1)}
+                del padded
     out["per_iteration"] = {"ms": round(total_ms, 3), "TFLOP/s": round(total_flops / total_ms / 1e9, 1)}
+    for _, ws, _ in cases:
+        for w in ws:
+            pkg.hip.unregister_packed_weight(w)
     print(json.dumps(out))
 
 

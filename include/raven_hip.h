@@ -150,6 +150,19 @@ int    raven_linear(const void* x0, const void* x1, const void* w, const void* r
                     int32_t M, int32_t N, int32_t K0, int32_t K1, int32_t swiglu, int32_t out_f32,
                     int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Line-aligned copies of bf16 weight matrices for products over 33 and more token rows.  No counterpart in the reference
+ * (its nn.Linear weights are [out, in] with rows K elements apart, RMM:463, 493, 507-509, and stay the layout every entry point
+ * takes).  Where K * 2 bytes is not a multiple of 128 (K = 5280: every second row starts 64 bytes into a cache line) the
+ * tiled MFMA kernels lose 5 to 7 % to half-line requests.  raven_register_packed_weight copies w [rows, K] (rows = out
+ * features; 2 * I for a GatedMLP fc matrix) into `packed` -- caller-allocated, raven_packed_weight_bytes(rows, K) bytes,
+ * 128-byte aligned, rows padded with zeros to a multiple of 64 elements -- on `stream`, and from then on every product
+ * whose weight pointer is `w`, with this K and these rows, that runs on the tiled kernels reads the copy: same values in
+ * the same order, same bits.  The caller registers again after changing w, and calls raven_unregister_packed_weight(w)
+ * before it frees either buffer.  Products of fewer rows (decode) always read w itself. */
+int64_t raven_packed_weight_bytes(int32_t rows, int32_t K);
+int     raven_register_packed_weight(const void* w, int32_t rows, int32_t K, void* packed, void* stream);
+int     raven_unregister_packed_weight(const void* w);
+
 /* Statistics behind the per-iteration exit criteria of adaptive compute (RMM:2128-2260), one value per row.
  * raven_exit_logit_stats on logits [rows, V] float:
  *   RAVEN_EXIT_ENTROPY  out = -sum p log(p + 1e-10), p = softmax(logits)                       (RMM:2142-2144)

@@ -43,6 +43,9 @@
 #include <type_traits>
 #include <utility>
 
+#include <mutex>
+#include <unordered_map>
+
 #include "raven_common.h"
 
 namespace raven {
@@ -55,6 +58,7 @@ struct TiledArgs {
     void* y;               // [M, N] bf16, or float when out_f32
     int M, N, K0, K1;      // N = output columns of this launch (I for SwiGLU)
     int ldy;               // row pitch of y and residual in elements (>= N: a launch may cover a range of columns)
+    int ldw, ldx;          // row pitch of w (K0 + K1, or more: a copy with rows padded to whole 128-byte lines) and of x0 / x1 (K0)
     int up_off;            // SwiGLU: weight rows between a gate row and its up row (the whole matrix's I)
     int out_f32;
     int tiles_m, tiles_n;
@@ -332,7 +336,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(TiledArgs a) {
     const int col8 = (lane & 7) * 8;           // this lane's column inside a step, in elements
     unsigned goff[LPW];                        // byte offset of this lane's row + column inside its operand (both segments
                                                // of the token rows have one row pitch)
-    const unsigned ld2 = 2u * (loads_w ? K : a.K0);
+    const unsigned ld2 = 2u * (loads_w ? a.ldw : a.ldx);
 #pragma unroll
     for (int p = 0; p < LPW; ++p) {
         const int r = (wave * LPW + p) * 8 + (lane >> 3);
@@ -578,8 +582,8 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(TiledArgs a) {
         int row_w;
         if (SWIGLU) row_w = min(tile_n * BN_OUT + (r >> 5) * 16 + (r & 15), a.N - 1) + ((r & 16) ? a.up_off : 0);
         else row_w = min(tile_n * BN + r, a.N - 1);
-        goff_w[p] = (unsigned)row_w * (2u * K) + 2u * colp[p & 1];
-        goff_x[p] = (unsigned)min(tile_m * BM + r, a.M - 1) * (2u * a.K0) + 2u * colp[p & 1];
+        goff_w[p] = (unsigned)row_w * (2u * a.ldw) + 2u * colp[p & 1];
+        goff_x[p] = (unsigned)min(tile_m * BM + r, a.M - 1) * (2u * a.ldx) + 2u * colp[p & 1];
     }
     const char* const zero = reinterpret_cast<const char*>(g_zero_piece);
     const char* const w0 = reinterpret_cast<const char*>(a.w);
@@ -791,8 +795,27 @@ bool tiled_gemm_fits(int M, int N, int K0, int K1, int dtype) {
            (int64_t)N * 2 * (K0 + K1) < (1ll << 31);
 }
 
-static int tiled_gemm_impl(const void* x0, const void* x1, const void* w, const void* residual, void* y, int M, int N, int K0, int K1,
-                           int swiglu, int out_f32, const TiledArgs::RopeAppend* rope, hipStream_t s) {
+// Copies of weight matrices with their rows padded to whole 128-byte lines (raven_register_packed_weight): at K = 5280 every
+// second row of [N, K] starts 64 bytes into a line, each 128-byte row piece of a K step is then two half lines, and the
+// tiled kernels lose 5 to 7 % to the extra requests.  Keyed by the address of the matrix as the caller passes it.
+struct PackedWeight {
+    const bf16* packed;
+    int rows, K, ld;
+};
+static std::mutex g_packed_mutex;
+static std::unordered_map<const void*, PackedWeight> g_packed;
+
+__global__ __launch_bounds__(256) void pack_rows_kernel(const bf16* __restrict__ w, bf16* __restrict__ out, int K, int ld) {
+    const int64_t row = blockIdx.x;
+    for (int c = threadIdx.x * 8; c < ld; c += 256 * 8) {
+        Chunk<bf16> v = zero_chunk<bf16>();
+        if (c < K) v = load_chunk(w + row * K + c);
+        store_chunk(out + row * ld + c, v);
+    }
+}
+
+static int tiled_gemm_impl(const void* x0, const void* x1, const void* w, const void* residual, void* y, int M, int N, int K0,
+                           int K1, int swiglu, int out_f32, const TiledArgs::RopeAppend* rope, hipStream_t s) {
     RAVEN_REQUIRE(tiled_gemm_fits(M, N, K0, K1, RAVEN_BF16), "gemm (tiled): unsupported shape M=%d N=%d K0=%d K1=%d", M, N, K0, K1);
     RAVEN_REQUIRE(!(swiglu && (residual || out_f32)), "gemm (tiled): the SwiGLU epilogue has no residual and stores bf16");
     RAVEN_REQUIRE(((uintptr_t)x0 & 15) == 0 && ((uintptr_t)x1 & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)y & 15) == 0 &&
@@ -806,6 +829,16 @@ static int tiled_gemm_impl(const void* x0, const void* x1, const void* w, const 
     a.M = M; a.N = N; a.K0 = K0; a.K1 = x1 ? K1 : 0; a.out_f32 = out_f32;
     a.ldy = N;
     a.up_off = N;
+    a.ldw = K0 + a.K1;
+    a.ldx = K0;
+    {
+        std::lock_guard<std::mutex> lock(g_packed_mutex);
+        const auto it = g_packed.find(w);
+        if (it != g_packed.end() && it->second.K == a.ldw && it->second.rows == (swiglu ? 2 * N : N) && (int64_t)it->second.rows * it->second.ld < (1ll << 31)) {
+            a.w = it->second.packed;
+            a.ldw = it->second.ld;
+        }
+    }
     if (rope) {
         a.rope = *rope;
         a.rope_on = 1;
@@ -833,7 +866,7 @@ static int tiled_gemm_impl(const void* x0, const void* x1, const void* w, const 
         TiledArgs head = a, tail = a;
         head.N = n_big;
         tail.N = N - n_big;
-        tail.w = a.w + (int64_t)n_big * (K0 + a.K1);
+        tail.w = a.w + (int64_t)n_big * a.ldw;
         tail.residual = a.residual ? a.residual + n_big : nullptr;
         tail.y = out_f32 ? static_cast<void*>(static_cast<float*>(y) + n_big) : static_cast<void*>(static_cast<bf16*>(y) + n_big);
         tail.rope.col0 = n_big;
@@ -868,3 +901,27 @@ int tiled_gemm_qkv_rope(const void* x, const void* wqkv, const void* qk_bias, co
 }
 
 }  // namespace raven
+
+extern "C" int64_t raven_packed_weight_bytes(int32_t rows, int32_t K) {
+    if (rows <= 0 || K <= 0) return 0;
+    return (int64_t)rows * ((K + 63) / 64 * 64) * (int64_t)sizeof(raven::bf16);
+}
+
+extern "C" int raven_register_packed_weight(const void* w, int32_t rows, int32_t K, void* packed, void* stream) {
+    using namespace raven;
+    RAVEN_REQUIRE(w && packed && rows > 0 && K > 0 && K % 8 == 0, "register_packed_weight: bad arguments (rows=%d K=%d)", rows, K);
+    RAVEN_REQUIRE(((uintptr_t)w & 15) == 0 && ((uintptr_t)packed & 127) == 0, "register_packed_weight: w must be 16-byte and packed 128-byte aligned");
+    const int ld = (K + 63) / 64 * 64;
+    pack_rows_kernel<<<dim3((unsigned)rows), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(static_cast<const bf16*>(w), static_cast<bf16*>(packed), K, ld);
+    if (int rc = raven_host::check_launch("register_packed_weight")) return rc;
+    std::lock_guard<std::mutex> lock(g_packed_mutex);
+    g_packed[w] = PackedWeight{static_cast<const bf16*>(packed), rows, K, ld};
+    return 0;
+}
+
+extern "C" int raven_unregister_packed_weight(const void* w) {
+    using namespace raven;
+    std::lock_guard<std::mutex> lock(g_packed_mutex);
+    g_packed.erase(w);
+    return 0;
+}

@@ -74,6 +74,9 @@ SIGNATURES = {
     "raven_gemm": (C.c_int, [_VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _VP]),
     "raven_adapter_gemm_concat": (C.c_int, [_VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _VP]),
     "raven_gemm_swiglu": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I32, _I32, _VP]),
+    "raven_packed_weight_bytes": (_I64, [_I32, _I32]),
+    "raven_register_packed_weight": (C.c_int, [_VP, _I32, _I32, _VP, _VP]),
+    "raven_unregister_packed_weight": (C.c_int, [_VP]),
     "raven_linear_workspace_bytes": (_SZ, [_I32, _I32]),
     "raven_linear": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _VP, _SZ, _VP]),
     "raven_exit_logit_stats": (C.c_int, [_VP, _VP, _VP, _I32, _I32, _I32, _VP]),
@@ -240,6 +243,22 @@ def gemm_swiglu(x, fc):
     rc = load().raven_gemm_swiglu(_ptr(x, "x"), _ptr(fc, "fc", dt), _ptr(y, "out"), M, inter, K, dtype_code(dt), _stream())
     _check(rc, "raven_gemm_swiglu")
     return y
+
+
+def register_packed_weight(w: torch.Tensor) -> torch.Tensor:
+    """Line-aligned copy of a bf16 weight matrix [rows, K] for the tiled GEMM; returns the copy, which the caller keeps
+    alive (together with w) until unregister_packed_weight(w)."""
+    assert w.dim() == 2 and w.dtype == torch.bfloat16 and w.is_contiguous()
+    rows, K = w.shape
+    n = load().raven_packed_weight_bytes(rows, K)
+    packed = torch.empty(n, dtype=torch.uint8, device=w.device)
+    rc = load().raven_register_packed_weight(_ptr(w, "w"), rows, K, _ptr(packed, "packed"), _stream())
+    _check(rc, "raven_register_packed_weight")
+    return packed
+
+
+def unregister_packed_weight(w: torch.Tensor) -> None:
+    _check(load().raven_unregister_packed_weight(_ptr(w, "w")), "raven_unregister_packed_weight")
 
 
 def linear_workspace(M, n_out_max, device):

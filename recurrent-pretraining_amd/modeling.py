@@ -19,6 +19,7 @@ What differs from the reference on purpose:
 from __future__ import annotations
 
 import math
+import weakref
 from dataclasses import dataclass
 from typing import Any, Callable, Optional, Union
 
@@ -118,6 +119,32 @@ class SandwichBlock(torch.nn.Module):
                                       a.Wqkv.weight, bias, a.proj.weight, m.fc.weight, m.proj.weight)
 
 
+class _PackedWeights:
+    """Line-aligned copies (hip.register_packed_weight) of the bf16 matrices whose rows are not whole 128-byte lines, read by
+    the tiled GEMM in place of the originals for products over 33 and more token rows.  A copy belongs to a weight tensor's
+    address and in-place version; `ensure` makes the copies again when either has changed (load_state_dict, .to()), `drop`
+    unregisters them (also when the model is collected: the library's table is keyed by address)."""
+
+    def __init__(self):
+        self.key = None
+        self.ptr_owner = []   # (weight tensor, packed buffer): both kept alive while registered
+
+    def ensure(self, mats) -> None:
+        mats = [w for w in mats if w.is_cuda and w.dtype == torch.bfloat16 and (w.shape[1] * 2) % 128 != 0 and w.shape[1] % 8 == 0]
+        key = tuple((w.data_ptr(), w._version) for w in mats)
+        if key == self.key:
+            return
+        self.drop()
+        self.ptr_owner = [(w.detach(), hip.register_packed_weight(w.detach())) for w in mats]
+        self.key = key
+
+    def drop(self) -> None:
+        for w, _ in self.ptr_owner:
+            hip.unregister_packed_weight(w)
+        self.ptr_owner = []
+        self.key = None
+
+
 def precompute_freqs_cis(dim: int, end: int, theta: float) -> torch.Tensor:
     """(cos, sin) table [1, end, 1, dim/2, 2] in fp32 (RMM:2076-2081)."""
     # always evaluated on the CPU, so the table does not depend on where the model lives
@@ -213,6 +240,9 @@ class RavenForCausalLM(RavenPreTrainedModel, GenerationMixin):
         self._rope_override: Optional[torch.Tensor] = None  # a forward with positions that are not the cache's (see _rope_table_for)
         self._rope_memo = None                               # the last such table and what it was built for
         self._scratch: dict = {}
+        self._packed = _PackedWeights()                      # line-aligned copies of weight matrices for prompt chunks
+        self.pack_chunk_weights = True                       # False: chunks read the matrices as they are (no copies are made)
+        self._packed_finalizer = weakref.finalize(self, self._packed.drop)
         self.eval()
 
     # ---- small helpers -------------------------------------------------------------------------
@@ -401,6 +431,10 @@ class RavenForCausalLM(RavenPreTrainedModel, GenerationMixin):
         return self._native
 
     def _workspace(self, M: int) -> torch.Tensor:
+        """Scratch for a block over M token rows; every block call fetches it, so this is also where a chunk of 33 rows or
+        more makes sure that the line-aligned weight copies are current."""
+        if M >= 33 and self.dtype == torch.bfloat16 and self.pack_chunk_weights:
+            self.pack_weights()
         ws = self._scratch.get(("ws", M))
         if ws is None:
             ws = hip.block_workspace(self._natives()["dims"], M, self.device)
@@ -606,6 +640,14 @@ class RavenForCausalLM(RavenPreTrainedModel, GenerationMixin):
                                       B, S, r)
         finally:
             self._rope_override = None
+
+    def pack_weights(self) -> None:
+        """Makes (or refreshes) the line-aligned copies of Wqkv, attn.proj and mlp.fc that products over 33 and more token rows
+        read (bf16 models whose n_embd * 2 bytes is not a multiple of 128: n_embd = 5280).  Every block call over such a
+        chunk calls this; call it by hand after changing a weight through `.data`, which leaves no trace a check could see."""
+        t = self.transformer
+        blocks = list(t.prelude) + list(t.core_block) + list(t.coda)
+        self._packed.ensure([w for b in blocks for w in (b.attn.Wqkv.weight, b.attn.proj.weight, b.mlp.fc.weight)])
 
     def _forward_rows(self, input_ids, input_embeds, input_states, labels, output_details, init_scale, cache, private, pos0, B, S, r):
         cfg, t = self.config, self.transformer

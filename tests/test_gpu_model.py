@@ -268,6 +268,46 @@ def test_forward_tiny_bf16_matches_oracle(tiny16):
     check(got.logits, want.logits, torch.bfloat16, "bf16 logits")
 
 
+def test_chunk_forward_reads_line_aligned_weight_copies_and_keeps_them_current(pkg):
+    """n_embd = 288 (rows of 576 bytes: every second one starts in the middle of a 128-byte line): a forward over 33 and more
+    token rows makes line-aligned copies of Wqkv, attn.proj and mlp.fc (RMM:463, 493, 507) for the tiled GEMM.  Same bits
+    as without them, against the oracle at the bf16 bar, and load_state_dict is followed by new copies."""
+    s = O.RavenShape(n_embd=288, n_heads=3, intermediate_size=704, vocab_size=1024, n_layers_in_prelude=1,
+                     n_layers_in_recurrent_block=2, n_layers_in_coda=1, mean_recurrence=3)
+    cfg = pkg.RavenConfig(n_embd=288, n_heads=3, n_layers=4, n_layers_in_prelude=1, n_layers_in_recurrent_block=2,
+                          n_layers_in_coda=1, intermediate_size=704, vocab_size=1024, mean_recurrence=3)
+    g = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, s.vocab_size, (2, 40), generator=g)
+    states = O.initialize_state(torch.empty(2, 40, s.n_embd), s, 1.0, g).to(torch.bfloat16)
+    outs = {}
+    model = pkg.RavenForCausalLM(cfg, device="cuda:0", dtype=torch.bfloat16)
+    for seed in (0, 1):
+        w = O.make_weights(s, seed=seed, dtype=torch.bfloat16)
+        w["freqs_cis"] = w["freqs_cis"].to(torch.bfloat16)
+        model.load_state_dict(w, strict=True)             # in place: the second round finds copies of the first round's weights
+        got = model(input_ids=ids.cuda(), input_states=states.cuda())
+        assert len(model._packed.ptr_owner) == 3 * 4      # three matrices of each of the four blocks
+        model.pack_chunk_weights = False
+        model._packed.drop()
+        plain = model(input_ids=ids.cuda(), input_states=states.cuda())
+        assert not model._packed.ptr_owner
+        model.pack_chunk_weights = True
+        assert torch.equal(got.logits, plain.logits) and torch.equal(got.latent_states, plain.latent_states)
+        want = O.forward(w, s, input_ids=ids, input_states=states)
+        check(got.latent_states, want.latent_states, torch.bfloat16, f"bf16 latents, weights of seed {seed}", ulps=ULPS_COMPOSED)
+        check(got.logits, want.logits, torch.bfloat16, f"bf16 logits, weights of seed {seed}")
+        outs[seed] = got.logits.clone()
+    assert not torch.equal(outs[0], outs[1])
+    finalizer = model._packed_finalizer
+    model(input_ids=ids.cuda(), input_states=states.cuda())
+    assert model._packed.ptr_owner and finalizer.alive
+    packed = model._packed
+    del model
+    import gc
+    gc.collect()
+    assert not finalizer.alive and not packed.ptr_owner   # collected model: its copies are unregistered
+
+
 @pytest.mark.parametrize("B,S", [(1, 64), (2, 70), (1, 200)])
 def test_wide_prefill_path_bf16(pkg, tiny16, tuned, B, S):
     """From 33 token rows on, the five products go to the tiled MFMA kernel and chunks of 16 or more rows to the matrix-core

@@ -330,6 +330,37 @@ def test_chunk_qkv_epilogue_writes_the_bits_of_the_two_launch_path(pkg, tuned, n
     assert not torch.equal(k1[1, :, :, pos0:pos0 + S], fresh[1, :, :, pos0:pos0 + S])
 
 
+@pytest.mark.parametrize("M,N,K,swiglu", [(300, 5280, 5280, False), (700, 1032, 136, False), (2048, 8448, 2816, False), (1100, 4096, 5280, True),
+                                          (40, 64, 72, False)])
+def test_packed_weight_copies_change_no_bit(pkg, M, N, K, swiglu):
+    """raven_register_packed_weight: a product over 33 and more rows reads the line-aligned copy and writes the bits it
+    writes from the matrix itself (both tile sizes, the last tile columns as small tiles, SwiGLU's gate / up rows, a
+    K with a partial last step); a matrix that changes must be registered again; after unregistering the matrix is read."""
+    hip = pkg.hip
+    x = _gpu_randn((M, K), 11)
+    w = _gpu_randn((2 * N if swiglu else N, K), 12, std=0.02)
+    res = None if swiglu else _gpu_randn((M, N), 13)
+    plain = hip.linear(x, w, residual=res, swiglu=swiglu).clone()
+    packed = hip.register_packed_weight(w)
+    try:
+        ld = (K + 63) // 64 * 64
+        assert packed.numel() == w.shape[0] * ld * 2
+        view = packed.view(torch.bfloat16).view(w.shape[0], ld)
+        assert torch.equal(view[:, :K], w) and not view[:, K:].any()
+        assert torch.equal(hip.linear(x, w, residual=res, swiglu=swiglu), plain)
+        w.mul_(2)                                          # exact in bf16; the copy still holds the old values ...
+        assert torch.equal(hip.linear(x, w, residual=res, swiglu=swiglu), plain), "the product did not read the registered copy"
+        few = hip.linear(x[:8], w, residual=None if res is None else res[:8], swiglu=swiglu).clone()   # ... which 8 rows never read
+        packed2 = hip.register_packed_weight(w)            # ... until the matrix is registered again
+        again = hip.linear(x, w, residual=res, swiglu=swiglu).clone()
+    finally:
+        hip.unregister_packed_weight(w)
+    want = hip.linear(x, w, residual=res, swiglu=swiglu)   # the matrix itself
+    assert torch.equal(again, want) and not torch.equal(again, plain)
+    check(few, want[:8].float(), torch.bfloat16, "8 rows against the first rows of the large product", ulps=ULPS_SWIGLU if swiglu else ULPS_RESIDUAL)
+    del packed, packed2
+
+
 def test_bench_prefill_iteration_runs_through_the_c_abi(pkg):
     """One recurrence over 4 x 512 rows through raven_core_iteration (adapter with two K segments, four blocks, chunk
     attention over a cache that already holds 512 positions): determinism, and the call equals adapter + four
