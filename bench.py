@@ -96,7 +96,7 @@ def adapter_once_bytes(cfg, batch, elt=2):
 # HBM-side bytes per launch of the tiled mlp.fc GEMM at M = 16384 from rocprofv3 --pmc (FETCH_SIZE 4,454,542 KiB x 1.99974 +
 # WRITE_SIZE 600,320 KiB x 1.0, both scaled by a 256 MiB copy): 8 x the 1.14 GB of operands + output, the panel re-reads
 # of 256 x 256 tiles in 8 x 4 groups per XCD.  Profiler figures, so constants, with the file that holds the readings.
-TILED_FC_TRAFFIC = int(4454542 * 1024 * 1.99974 + 600320 * 1024)
+TILED_FC_TRAFFIC = int(4457730 * 1024 * 1.99974 + 600320 * 1024)
 TILED_FC_TRAFFIC_SOURCE = "profiles/gemm_tiled_bs4x4096_counters.txt"
 
 
@@ -158,7 +158,9 @@ def prefill_record(pkg, model, B, S, r):
         "config": {"workload": f"recurrent-core prefill, nebel-raven-3.5b shape, bs={B} x {S} tokens, {r} timed iterations "
                                f"(BASELINE.json configs[4])",
                    "batch": B, "seq_len": S, "iterations": r, "gemm": "gemm_ring_kernel (hand-written MFMA, 256 x 256 tiles, four waves, operands global -> LDS ring)",
-                   "attention": "attention_prefill_kernel"},
+                   "attention": "attention_prefill_kernel",
+                   "weights": ("Wqkv, attn.proj, mlp.fc read through line-aligned copies made once (raven_register_packed_weight)"
+                               if model.pack_chunk_weights else "as loaded")},
         "roofline": {"bound": "mfma", "kernel": f"gemm_ring_kernel<SwiGLU> 256x256 (mlp.fc {2 * inter}x{h}, M={M})",
                      "achieved": round(fc_tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(fc_tflops / MFMA_PEAK_TFLOPS, 4), "flops_per_launch": fc_flops, "avg_us": round(fc_ms * 1e3, 1),
@@ -178,8 +180,6 @@ def prefill(args):
     fill_synthetic(model, 0)
     model.pack_chunk_weights = not args.plain_weights
     rec = prefill_record(pkg, model, args.prefill_batch, args.prefill_len, args.recurrence)
-    rec["config"]["weights"] = ("as loaded" if args.plain_weights else
-                                "Wqkv, attn.proj, mlp.fc read through line-aligned copies made once (raven_register_packed_weight)")
     line = {"metric": "core prefill tokens*iterations/s, raven-3.5b shape bf16; MFMA utilisation", "value": rec["value"],
             "unit": rec["unit"], "n_gpus": 1, "steps": rec["steps"], "warmup": rec["warmup"], "ms_per_step": rec["ms_per_step"],
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
