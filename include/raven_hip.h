@@ -105,7 +105,9 @@ const char* raven_last_error(void);
  * norm leaves its slices to that norm's launch, which adds them in the same order; 0 = a launch of its own adds them),
  * fuse_qkv_rope (1 = inside raven_sandwich_block / raven_core_iteration(s) a chunk's q | k | v product on the tiled GEMM
  * applies bias, RoPE and the cache append in its epilogue; 0 = the product is stored and raven_qkv_bias_rope_cache_append's
- * kernel follows; same bits either way).
+ * kernel follows; same bits either way), pad_chunk_rows (1 = inside the composed entry points the activations that the tiled
+ * GEMMs of a bf16 chunk read -- norm_1's and norm_3's output, the attention output -- are laid out in the workspace with rows
+ * padded to a multiple of 64 elements when n_embd is not one; 0 = rows n_embd elements apart; same bits either way).
  * Not needed in normal use: the defaults are the tuned values.  The knobs are process-global
  * state read at every launch: changing them while another thread or stream is inside a call of this library is a race. */
 int raven_set_tuning(const char* key, int32_t value);

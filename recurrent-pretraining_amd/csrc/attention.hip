@@ -774,13 +774,13 @@ namespace raven {
 extern int g_tiled_min_rows;
 bool tiled_gemm_fits(int M, int N, int K0, int K1, int dtype);
 int tiled_gemm_qkv_rope(const void* x, const void* wqkv, const void* qk_bias, const float* freqs, void* q_out, void* k_cache,
-                        void* v_cache, int64_t slot_off, int nh, int hd, int t_max, int M, int S, int K, int pos0, const int* pos_dev,
-                        hipStream_t s);
+                        void* v_cache, int64_t slot_off, int nh, int hd, int t_max, int M, int S, int K, int ldx, int pos0,
+                        const int* pos_dev, hipStream_t s);
 int g_fuse_qkv_rope = 1;  // raven_set_tuning("fuse_qkv_rope"): 0 = a chunk's q | k | v product is stored and rotated by a launch of its own
 
 // A chunk's Wqkv product with raven_qkv_bias_rope_cache_append as its epilogue (bf16 shapes that take the tiled GEMM):
-// *done = 0 and nothing launched when the shape does not take that path.
-int qkv_linear_rope_append(const void* x, const void* wqkv, const void* qk_bias, const float* freqs, void* q_out,
+// *done = 0 and nothing launched when the shape does not take that path.  ldx: elements between two rows of x (0 = n_embd).
+int qkv_linear_rope_append(const void* x, int ldx, const void* wqkv, const void* qk_bias, const float* freqs, void* q_out,
                            const raven_kv_cache* cache, int slot, int B, int S, int pos0, const int32_t* pos_dev, int n_heads,
                            int head_dim, int dtype, hipStream_t s, int* done) {
     *done = 0;
@@ -793,7 +793,7 @@ int qkv_linear_rope_append(const void* x, const void* wqkv, const void* qk_bias,
     if (int rc = make_view("qkv_append", cache, slot, B, n_heads, head_dim, &cv)) return rc;
     RAVEN_REQUIRE(pos0 + S <= cv.t_max, "qkv_append: positions %d..%d exceed the cache length %d", pos0, pos0 + S - 1, cv.t_max);
     *done = 1;
-    return tiled_gemm_qkv_rope(x, wqkv, qk_bias, freqs, q_out, cv.k, cv.v, cv.slot_off, cv.nh, cv.hd, cv.t_max, M, S, h, pos0, pos_dev, s);
+    return tiled_gemm_qkv_rope(x, wqkv, qk_bias, freqs, q_out, cv.k, cv.v, cv.slot_off, cv.nh, cv.hd, cv.t_max, M, S, h, ldx, pos0, pos_dev, s);
 }
 }  // namespace raven
 

@@ -34,7 +34,8 @@ constexpr int kPfKeys = 64;     // keys per tile
 
 struct PrefillArgs {
     const bf16* q;   // [B*S, h]
-    bf16* y;         // [B*S, h]
+    bf16* y;         // [B*S, h], rows ldy elements apart
+    int ldy;
     const bf16* k;   // cache tensors
     const bf16* v;
     int64_t slot_off;
@@ -396,7 +397,7 @@ __global__ __launch_bounds__(NW * 64, NW == 6 ? 3 : 2) void attention_prefill_ke
             const int r = c / CPR, dc = c - r * CPR;
             const int row = row0 + 16 * g0 + r;
             if (row < n_rows)
-                *reinterpret_cast<u32x4*>(a.y + (q_row0 + row) * h + head * HD + dc * 8) = *reinterpret_cast<const u32x4*>(ot + r * KP + dc * 8);
+                *reinterpret_cast<u32x4*>(a.y + (q_row0 + row) * a.ldy + head * HD + dc * 8) = *reinterpret_cast<const u32x4*>(ot + r * KP + dc * 8);
         }
     }
 }
@@ -407,10 +408,11 @@ namespace raven {
 int g_prefill_waves = 0;  // raven_set_tuning("prefill_waves"): 0 = by shape, 4 or 6 = waves per workgroup where the shape allows both
 }
 
-extern "C" int raven_prefill_attention(const void* q, void* y, const raven_kv_cache* cache, int32_t slot, int32_t B, int32_t S,
-                                       int32_t pos0, const int32_t* pos_dev, int32_t n_heads, int32_t head_dim, int32_t dtype,
-                                       void* stream) {
-    using namespace raven;
+namespace raven {
+// raven_prefill_attention with the rows of y ldy elements apart (>= n_heads * head_dim)
+int prefill_attention_pitched(const void* q, void* y, int ldy, const raven_kv_cache* cache, int32_t slot, int32_t B, int32_t S,
+                              int32_t pos0, const int32_t* pos_dev, int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream) {
+    RAVEN_REQUIRE(ldy >= n_heads * head_dim && ldy % 8 == 0, "prefill_attention: bad output row pitch %d", ldy);
     RAVEN_REQUIRE(dtype == RAVEN_BF16, "prefill_attention: bf16 only (dtype %d)", dtype);
     RAVEN_REQUIRE(head_dim == 64 || head_dim == 96 || head_dim == 128, "prefill_attention: head_dim %d not in {64, 96, 128}", head_dim);
     RAVEN_REQUIRE(q && y && cache && cache->k && cache->v, "prefill_attention: null pointer");
@@ -425,6 +427,7 @@ extern "C" int raven_prefill_attention(const void* q, void* y, const raven_kv_ca
     PrefillArgs a{};
     a.q = static_cast<const bf16*>(q);
     a.y = static_cast<bf16*>(y);
+    a.ldy = ldy;
     a.k = static_cast<const bf16*>(cache->k);
     a.v = static_cast<const bf16*>(cache->v);
     a.slot_off = (int64_t)sl * cache->batch * n_heads * cache->t_max * head_dim;
@@ -451,6 +454,13 @@ extern "C" int raven_prefill_attention(const void* q, void* y, const raven_kv_ca
 #undef RAVEN_PREFILL
     return raven_host::check_launch("prefill_attention");
 }
+}  // namespace raven
+
+extern "C" int raven_prefill_attention(const void* q, void* y, const raven_kv_cache* cache, int32_t slot, int32_t B, int32_t S,
+                                       int32_t pos0, const int32_t* pos_dev, int32_t n_heads, int32_t head_dim, int32_t dtype,
+                                       void* stream) {
+    return raven::prefill_attention_pitched(q, y, n_heads * head_dim, cache, slot, B, S, pos0, pos_dev, n_heads, head_dim, dtype, stream);
+}
 
 extern "C" int raven_paged_prefill_attention(const void* q, void* y, const void* k_cache, const void* v_cache,
                                              const int32_t* block_table, const int32_t* seq_lens, const int32_t* q_start, int32_t B,
@@ -467,6 +477,7 @@ extern "C" int raven_paged_prefill_attention(const void* q, void* y, const void*
     PrefillArgs a{};
     a.q = static_cast<const bf16*>(q);
     a.y = static_cast<bf16*>(y);
+    a.ldy = n_heads * head_dim;
     a.k = static_cast<const bf16*>(k_cache);
     a.v = static_cast<const bf16*>(v_cache);
     a.nh = n_heads; a.hd = head_dim;

@@ -33,23 +33,37 @@ int linear_leave_sums(const void* x0, const void* x1, const void* w, int ldw, co
 int splitk_sums_then_norm(const float* partial, int ks, const float* extra, const void* residual, void* sum_out, const void* weight,
                           void* y, const void* weight2, void* y2, int rows, int dim, float eps, hipStream_t s);
 
-int qkv_linear_rope_append(const void* x, const void* wqkv, const void* qk_bias, const float* freqs, void* q_out,
+int qkv_linear_rope_append(const void* x, int ldx, const void* wqkv, const void* qk_bias, const float* freqs, void* q_out,
                            const raven_kv_cache* cache, int slot, int B, int S, int pos0, const int32_t* pos_dev, int n_heads,
                            int head_dim, int dtype, hipStream_t s, int* done);
+
+extern int g_tiled_min_rows;
+bool tiled_gemm_fits(int M, int N, int K0, int K1, int dtype);
+int tiled_gemm_pitched(const void* x, int ldx, const void* w, const void* residual, void* y, int M, int N, int K, int swiglu, hipStream_t s);
+int rmsnorm_pitched(const void* x, const void* residual, const void* weight, void* y, int ldy, void* sum_out, const void* weight2,
+                    void* y2, int ldy2, int64_t rows, int32_t dim, float eps, int32_t dtype, void* stream);
+int prefill_attention_pitched(const void* q, void* y, int ldy, const raven_kv_cache* cache, int32_t slot, int32_t B, int32_t S,
+                              int32_t pos0, const int32_t* pos_dev, int32_t n_heads, int32_t head_dim, int32_t dtype, void* stream);
 
 // y = round(round(x W^T) + residual), then RMSNorm(weight) -> out1 and RMSNorm(weight2) of that -> out2 (either may be
 // null): two launches where the product is K-split (the norm launch adds the slices), three otherwise
 static int linear_then_norm(const void* x, const void* w, const void* residual, void* y, const void* weight, void* out1,
                             const void* weight2, void* out2, int M, int N, int K, float eps, int dtype, void* ws, size_t ws_bytes,
-                            hipStream_t s) {
+                            hipStream_t s, int ld_out2 = 0) {
     int ks = 0;
     if (int rc = linear_leave_sums(x, nullptr, w, 0, nullptr, residual, y, M, N, K, 0, dtype, ws, ws_bytes, s, &ks)) return rc;
-    if (ks) return splitk_sums_then_norm(static_cast<const float*>(ws), ks, nullptr, residual, nullptr, weight, out1, weight2, out2, M, N, eps, s);
-    return raven_rmsnorm_residual(y, nullptr, weight, out1, nullptr, weight2, out2, M, N, eps, dtype, s);
+    if (ks) {
+        RAVEN_REQUIRE(ld_out2 == 0 || ld_out2 == N, "linear_then_norm: padded rows behind a K-split product");
+        return splitk_sums_then_norm(static_cast<const float*>(ws), ks, nullptr, residual, nullptr, weight, out1, weight2, out2, M, N, eps, s);
+    }
+    return rmsnorm_pitched(y, nullptr, weight, out1, N, nullptr, weight2, out2, ld_out2 ? ld_out2 : N, M, N, eps, dtype, s);
 }
+
+int g_pad_chunk_rows = 1;  // raven_set_tuning("pad_chunk_rows"): 0 = the activations of a chunk keep rows n_embd elements apart
 
 struct BlockScratch {
     char *n1, *qkv, *q, *ya, *x1, *x2, *n3, *g, *x3, *xa, *xr;
+    int ld_pad;     // n1, ya and n3 have room for rows this many elements apart (n_embd, or the next multiple of 64 for chunks)
     float* e_sums;  // up to 32 rows: fp32 sums of the adapter's embedding half, computed once for all recurrences
     void* attn_ws;
     size_t attn_ws_bytes;
@@ -60,6 +74,10 @@ struct BlockScratch {
 static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
     const size_t es = raven_host::elt_size(d->dtype);
     const size_t row = raven_host::align_up((size_t)M * d->n_embd * es);
+    // chunks of bf16 rows that are not whole cache lines (n_embd = 5280: 82.5 lines): the three activations that a tiled GEMM
+    // reads (norm_1's and norm_3's output, the attention output) may be laid out with padded rows
+    const int ld_pad = (d->dtype == RAVEN_BF16 && M >= 33 && d->n_embd % 64 != 0) ? (d->n_embd + 63) / 64 * 64 : d->n_embd;
+    const size_t row_pad = raven_host::align_up((size_t)M * ld_pad * es);
     size_t off = 0;
     auto take = [&](size_t bytes) {
         char* p = base ? base + off : nullptr;
@@ -67,13 +85,14 @@ static size_t carve(const raven_dims* d, int M, char* base, BlockScratch* out) {
         return p;
     };
     BlockScratch s;
-    s.n1 = take(row);
+    s.ld_pad = ld_pad;
+    s.n1 = take(row_pad);
     s.qkv = take(3 * row);
     s.q = take(row);
-    s.ya = take(row);
+    s.ya = take(row_pad);
     s.x1 = take(row);
     s.x2 = take(row);
-    s.n3 = take(row);
+    s.n3 = take(row_pad);
     s.g = take((size_t)M * d->intermediate * es);
     s.x3 = take(row);
     s.xa = take(row);
@@ -117,16 +136,31 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
                      const raven_kv_cache* cache, int slot, int B, int S, int pos0, const int32_t* pos_dev, void* stream,
                      const raven_paged_kv* paged = nullptr, int layer = 0) {
     const int M = B * S, h = d->n_embd, I = d->intermediate, dt = d->dtype;
+    hipStream_t hs = static_cast<hipStream_t>(stream);
     int rc;
+    // chunks of 16 or more rows per sequence: 64 or 128 query rows of a head per workgroup on the matrix cores; a few
+    // rows per sequence (or a partially filled cache, which only that kernel looks up): one row at a time
+    const bool chunk = !paged && S > 1;
+    const bool mfma = chunk && dt == RAVEN_BF16 && S >= 16 && (d->head_dim == 64 || d->head_dim == 96 || d->head_dim == 128) &&
+                      (cache->steps_present == nullptr || cache->lookup_mode == RAVEN_LOOKUP_NONE);
+    // Rows of n_embd bf16 values that are not whole cache lines (5280: 82.5 lines): norm_1's and norm_3's output and the
+    // attention output, which the tiled GEMM reads as its token rows, are laid out with rows padded to whole lines (the pad
+    // is never read: the products' K stays n_embd).  Every block of a call decides this the same way.
+    const bool pad = g_pad_chunk_rows && mfma && s.ld_pad != h && M >= g_tiled_min_rows && tiled_gemm_fits(M, 3 * h, h, 0, dt) &&
+                     tiled_gemm_fits(M, h, h, 0, dt) && tiled_gemm_fits(M, I, h, 0, dt);
+    const int ld = pad ? s.ld_pad : h;
     if (!n1_ready)
-        if ((rc = raven_rmsnorm_residual(x_in, nullptr, w->norm_1, s.n1, nullptr, nullptr, nullptr, M, h, d->eps, dt, stream))) return rc;
+        if ((rc = rmsnorm_pitched(x_in, nullptr, w->norm_1, s.n1, ld, nullptr, nullptr, nullptr, ld, M, h, d->eps, dt, stream))) return rc;
     // a chunk of tokens on the tiled GEMM: bias, RoPE and the cache append are that product's epilogue
     int qkv_done = 0;
-    if (!paged && S > 1)
-        if ((rc = qkv_linear_rope_append(s.n1, w->wqkv, w->qk_bias, freqs, s.q, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim,
-                                         dt, static_cast<hipStream_t>(stream), &qkv_done))) return rc;
-    if (!qkv_done)
-        if ((rc = raven_linear(s.n1, nullptr, w->wqkv, nullptr, s.qkv, M, 3 * h, h, 0, 0, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
+    if (chunk)
+        if ((rc = qkv_linear_rope_append(s.n1, ld, w->wqkv, w->qk_bias, freqs, s.q, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim,
+                                         dt, hs, &qkv_done))) return rc;
+    if (!qkv_done) {
+        if (pad) rc = tiled_gemm_pitched(s.n1, ld, w->wqkv, nullptr, s.qkv, M, 3 * h, h, 0, hs);
+        else rc = raven_linear(s.n1, nullptr, w->wqkv, nullptr, s.qkv, M, 3 * h, h, 0, 0, 0, dt, s.lin_ws, s.lin_ws_bytes, stream);
+        if (rc) return rc;
+    }
     if (paged) {   // decode over block-paged caches, every sequence at its own position
         if ((rc = raven_paged_qkv_attention_decode(s.qkv, w->qk_bias, freqs, s.ya, paged->k_caches[layer], paged->v_caches[layer],
                                                    paged->block_table, paged->seq_lens, B, paged->max_blocks, paged->block_size,
@@ -138,18 +172,21 @@ static int run_block(const raven_dims* d, const raven_block_weights* w, const Bl
         if (!qkv_done)
             if ((rc = raven_qkv_bias_rope_cache_append(s.qkv, w->qk_bias, freqs, s.q, cache, slot, B, S, pos0, pos_dev, d->n_heads,
                                                        d->head_dim, dt, stream))) return rc;
-        // chunks of 16 or more rows per sequence: 64 or 128 query rows of a head per workgroup on the matrix cores; a few
-        // rows per sequence (or a partially filled cache, which only that kernel looks up): one row at a time
-        const bool mfma = dt == RAVEN_BF16 && S >= 16 && (d->head_dim == 64 || d->head_dim == 96 || d->head_dim == 128) &&
-                          (cache->steps_present == nullptr || cache->lookup_mode == RAVEN_LOOKUP_NONE);
-        if (mfma) rc = raven_prefill_attention(s.q, s.ya, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, stream);
+        if (mfma) rc = prefill_attention_pitched(s.q, s.ya, ld, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, stream);
         else rc = raven_decode_attention(s.q, s.ya, cache, slot, B, S, pos0, pos_dev, d->n_heads, d->head_dim, dt, s.attn_ws, s.attn_ws_bytes, stream);
         if (rc) return rc;
     }
-    hipStream_t hs = static_cast<hipStream_t>(stream);
-    if ((rc = linear_then_norm(s.ya, w->proj, x_in, s.x1, w->norm_2, s.x2, w->norm_3, s.n3, M, h, h, d->eps, dt, s.lin_ws, s.lin_ws_bytes, hs))) return rc;
-    if ((rc = raven_linear(s.n3, nullptr, w->fc, nullptr, s.g, M, I, h, 0, 1, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
-    return linear_then_norm(s.g, w->mlp_proj, s.x2, s.x3, w->norm_4, y_out, tail_w, tail_out, M, h, I, d->eps, dt, s.lin_ws, s.lin_ws_bytes, hs);
+    if (pad) {
+        if ((rc = tiled_gemm_pitched(s.ya, ld, w->proj, x_in, s.x1, M, h, h, 0, hs))) return rc;
+        if ((rc = rmsnorm_pitched(s.x1, nullptr, w->norm_2, s.x2, h, nullptr, w->norm_3, s.n3, ld, M, h, d->eps, dt, stream))) return rc;
+        if ((rc = tiled_gemm_pitched(s.n3, ld, w->fc, nullptr, s.g, M, I, h, 1, hs))) return rc;
+    } else {
+        if ((rc = linear_then_norm(s.ya, w->proj, x_in, s.x1, w->norm_2, s.x2, w->norm_3, s.n3, M, h, h, d->eps, dt, s.lin_ws, s.lin_ws_bytes, hs))) return rc;
+        if ((rc = raven_linear(s.n3, nullptr, w->fc, nullptr, s.g, M, I, h, 0, 1, 0, dt, s.lin_ws, s.lin_ws_bytes, stream))) return rc;
+    }
+    // the tail norm's output is the next block's norm_1 input when it goes to scratch.n1: rows as that block will read them
+    const int tail_ld = tail_out == static_cast<void*>(s.n1) ? ld : h;
+    return linear_then_norm(s.g, w->mlp_proj, s.x2, s.x3, w->norm_4, y_out, tail_w, tail_out, M, h, I, d->eps, dt, s.lin_ws, s.lin_ws_bytes, hs, tail_ld);
 }
 
 // One row.  x_raw is the block input before `pre_norm` (the previous block's norm_4, or null when x_raw is

@@ -58,7 +58,7 @@ struct TiledArgs {
     void* y;               // [M, N] bf16, or float when out_f32
     int M, N, K0, K1;      // N = output columns of this launch (I for SwiGLU)
     int ldy;               // row pitch of y and residual in elements (>= N: a launch may cover a range of columns)
-    int ldw, ldx;          // row pitch of w (K0 + K1, or more: a copy with rows padded to whole 128-byte lines) and of x0 / x1 (K0)
+    int ldw, ldx;          // row pitch of w and of x0 / x1 in elements: K0 + K1 and K0, or more where rows are padded to whole 128-byte lines
     int up_off;            // SwiGLU: weight rows between a gate row and its up row (the whole matrix's I)
     int out_f32;
     int tiles_m, tiles_n;
@@ -814,7 +814,7 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(const bf16* __restrict__
     }
 }
 
-static int tiled_gemm_impl(const void* x0, const void* x1, const void* w, const void* residual, void* y, int M, int N, int K0,
+static int tiled_gemm_impl(const void* x0, int ldx, const void* x1, const void* w, const void* residual, void* y, int M, int N, int K0,
                            int K1, int swiglu, int out_f32, const TiledArgs::RopeAppend* rope, hipStream_t s) {
     RAVEN_REQUIRE(tiled_gemm_fits(M, N, K0, K1, RAVEN_BF16), "gemm (tiled): unsupported shape M=%d N=%d K0=%d K1=%d", M, N, K0, K1);
     RAVEN_REQUIRE(!(swiglu && (residual || out_f32)), "gemm (tiled): the SwiGLU epilogue has no residual and stores bf16");
@@ -830,7 +830,8 @@ static int tiled_gemm_impl(const void* x0, const void* x1, const void* w, const 
     a.ldy = N;
     a.up_off = N;
     a.ldw = K0 + a.K1;
-    a.ldx = K0;
+    a.ldx = ldx > 0 ? ldx : K0;
+    RAVEN_REQUIRE(a.ldx >= K0 && a.ldx % 8 == 0 && (a.ldx == K0 || a.K1 == 0) && (int64_t)M * a.ldx < (1ll << 31), "gemm (tiled): bad row pitch %d of x", ldx);
     {
         std::lock_guard<std::mutex> lock(g_packed_mutex);
         const auto it = g_packed.find(w);
@@ -878,15 +879,20 @@ static int tiled_gemm_impl(const void* x0, const void* x1, const void* w, const 
 
 int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residual, void* y, int M, int N, int K0, int K1, int swiglu,
                int out_f32, hipStream_t s) {
-    return tiled_gemm_impl(x0, x1, w, residual, y, M, N, K0, K1, swiglu, out_f32, nullptr, s);
+    return tiled_gemm_impl(x0, 0, x1, w, residual, y, M, N, K0, K1, swiglu, out_f32, nullptr, s);
+}
+
+// The same with the rows of x `ldx` elements apart (>= K, one segment): activations whose rows are padded to whole cache lines
+int tiled_gemm_pitched(const void* x, int ldx, const void* w, const void* residual, void* y, int M, int N, int K, int swiglu, hipStream_t s) {
+    return tiled_gemm_impl(x, ldx, nullptr, w, residual, y, M, N, K, 0, swiglu, 0, nullptr, s);
 }
 
 // A chunk's q | k | v product (wqkv: [3 * nh * hd, K]) whose epilogue adds the q / k bias, applies RoPE and writes q to
 // q_out [M, nh * hd] and k, v to the cache rows of positions pos0 (or *pos_dev) + 0 .. S - 1 of each of the M / S sequences:
 // the product itself is never stored.  k_cache / v_cache: the cache tensors, slot_off the slot's element offset.
 int tiled_gemm_qkv_rope(const void* x, const void* wqkv, const void* qk_bias, const float* freqs, void* q_out, void* k_cache,
-                        void* v_cache, int64_t slot_off, int nh, int hd, int t_max, int M, int S, int K, int pos0, const int* pos_dev,
-                        hipStream_t s) {
+                        void* v_cache, int64_t slot_off, int nh, int hd, int t_max, int M, int S, int K, int ldx, int pos0,
+                        const int* pos_dev, hipStream_t s) {
     RAVEN_REQUIRE(freqs && q_out && k_cache && v_cache && hd % 8 == 0 && S > 0 && M % S == 0, "gemm (tiled, q/k/v epilogue): bad arguments");
     TiledArgs::RopeAppend r{};
     r.freqs = freqs;
@@ -897,7 +903,7 @@ int tiled_gemm_qkv_rope(const void* x, const void* wqkv, const void* qk_bias, co
     r.slot_off = slot_off;
     r.pos_dev = pos_dev;
     r.nh = nh; r.hd = hd; r.t_max = t_max; r.S = S; r.pos0 = pos0; r.col0 = 0;
-    return tiled_gemm_impl(x, nullptr, wqkv, nullptr, nullptr, M, 3 * nh * hd, K, 0, 0, 0, &r, s);
+    return tiled_gemm_impl(x, ldx, nullptr, wqkv, nullptr, nullptr, M, 3 * nh * hd, K, 0, 0, 0, &r, s);
 }
 
 }  // namespace raven

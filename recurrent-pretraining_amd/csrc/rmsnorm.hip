@@ -20,6 +20,8 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
     return red[0] + red[1] + red[2] + red[3];
 }
 
+// ldy, ldy2: elements between two rows of y and of y2 (dim, or more where the rows are padded to whole cache lines for
+// the tiled GEMM that reads them); x, residual and sum_out are dim apart.
 // MC = 16-byte chunks a thread keeps of its row (4 covers 5280 bf16 elements; fp32 rows of that length need 8)
 // EARLY: the weights are requested before the row, so that no load waits behind a reduction (taken for up to 64 rows;
 // measured at 5280 columns it is worth 0.1 us of a 3.6 us launch at best, the weights being cache hits).  Otherwise
@@ -41,7 +43,7 @@ struct SplitSums {
 template <typename T, int MC, bool EARLY, int KS>
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
     const T* __restrict__ x, const T* __restrict__ residual, const T* __restrict__ weight, T* __restrict__ y,
-    T* __restrict__ sum_out, const T* __restrict__ weight2, T* __restrict__ y2, int dim, float eps, SplitSums sp) {
+    T* __restrict__ sum_out, const T* __restrict__ weight2, T* __restrict__ y2, int dim, float eps, SplitSums sp, int ldy, int ldy2) {
     constexpr int E = Chunk<T>::N;
     __shared__ float red[4];
     const int64_t row = blockIdx.x;
@@ -129,7 +131,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
                 v[i][e] = to_f32(co.v[e]);
                 ss2 = __builtin_fmaf(v[i][e], v[i][e], ss2);
             }
-            if (y) store_chunk(y + row * dim + c * E, co);
+            if (y) store_chunk(y + row * ldy + c * E, co);
         }
     }
     if (weight2 == nullptr) return;
@@ -143,7 +145,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
             Chunk<T> co;
 #pragma unroll
             for (int e = 0; e < E; ++e) co.v[e] = from_f32<T>(round_to<T>(v[i][e] * inv) * to_f32(w2.v[e]));
-            store_chunk(y2 + row * dim + c * E, co);
+            store_chunk(y2 + row * ldy2 + c * E, co);
         }
     }
 }
@@ -161,7 +163,7 @@ int splitk_sums_then_norm(const float* partial, int ks, const float* extra, cons
 #define RAVEN_SPLIT_NORM(KS_)                                                                                            \
     case KS_:                                                                                                           \
         rmsnorm_kernel<bf16, 4, true, KS_><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                          \
-            nullptr, (const bf16*)residual, (const bf16*)weight, (bf16*)y, (bf16*)sum_out, (const bf16*)weight2, (bf16*)y2, dim, eps, sp); \
+            nullptr, (const bf16*)residual, (const bf16*)weight, (bf16*)y, (bf16*)sum_out, (const bf16*)weight2, (bf16*)y2, dim, eps, sp, dim, dim); \
         break;
     switch (ks) {
         RAVEN_SPLIT_NORM(1) RAVEN_SPLIT_NORM(2) RAVEN_SPLIT_NORM(3) RAVEN_SPLIT_NORM(4)
@@ -174,10 +176,10 @@ int splitk_sums_then_norm(const float* partial, int ks, const float* extra, cons
 
 }  // namespace raven
 
-extern "C" int raven_rmsnorm_residual(const void* x, const void* residual, const void* weight, void* y,
-                                      void* sum_out, const void* weight2, void* y2, int64_t rows, int32_t dim,
-                                      float eps, int32_t dtype, void* stream) {
-    using namespace raven;
+namespace raven {
+// raven_rmsnorm_residual with the rows of y and of y2 ldy and ldy2 elements apart (>= dim)
+int rmsnorm_pitched(const void* x, const void* residual, const void* weight, void* y, int ldy, void* sum_out, const void* weight2,
+                    void* y2, int ldy2, int64_t rows, int32_t dim, float eps, int32_t dtype, void* stream) {
     RAVEN_REQUIRE(dtype == RAVEN_F32 || dtype == RAVEN_BF16, "rmsnorm: unknown dtype %d", dtype);
     if (rows == 0) return 0;  // an empty tensor has no storage to point at
     RAVEN_REQUIRE(x && weight && (y || y2), "rmsnorm: null x / weight / output");
@@ -188,6 +190,7 @@ extern "C" int raven_rmsnorm_residual(const void* x, const void* residual, const
     RAVEN_REQUIRE(dim / elts <= kNormThreads * kNormMaxChunks, "rmsnorm: dim %d too large (max %d)", dim,
                   kNormThreads * kNormMaxChunks * elts);
     RAVEN_REQUIRE(rows > 0 && rows < (1ll << 31), "rmsnorm: bad row count %lld", (long long)rows);
+    RAVEN_REQUIRE(ldy >= dim && ldy2 >= dim && ldy % elts == 0 && ldy2 % elts == 0, "rmsnorm: bad output row pitch %d / %d", ldy, ldy2);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int per_thread = (dim / elts + kNormThreads - 1) / kNormThreads;
     const bool early = g_norm_early >= 0 ? g_norm_early != 0 : rows <= 64;
@@ -196,10 +199,10 @@ extern "C" int raven_rmsnorm_residual(const void* x, const void* residual, const
     do {                                                                                                                     \
         if (early)                                                                                                           \
             rmsnorm_kernel<T_, MC_, true, 0><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                        \
-                (const T_*)x, (const T_*)residual, (const T_*)weight, (T_*)y, (T_*)sum_out, (const T_*)weight2, (T_*)y2, dim, eps, none); \
+                (const T_*)x, (const T_*)residual, (const T_*)weight, (T_*)y, (T_*)sum_out, (const T_*)weight2, (T_*)y2, dim, eps, none, ldy, ldy2); \
         else                                                                                                                 \
             rmsnorm_kernel<T_, MC_, false, 0><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                       \
-                (const T_*)x, (const T_*)residual, (const T_*)weight, (T_*)y, (T_*)sum_out, (const T_*)weight2, (T_*)y2, dim, eps, none); \
+                (const T_*)x, (const T_*)residual, (const T_*)weight, (T_*)y, (T_*)sum_out, (const T_*)weight2, (T_*)y2, dim, eps, none, ldy, ldy2); \
     } while (0)
     if (dtype == RAVEN_BF16) {
         if (per_thread <= 4) RAVEN_NORM_LAUNCH(bf16, 4);
@@ -212,4 +215,11 @@ extern "C" int raven_rmsnorm_residual(const void* x, const void* residual, const
     }
 #undef RAVEN_NORM_LAUNCH
     return raven_host::check_launch("rmsnorm");
+}
+}  // namespace raven
+
+extern "C" int raven_rmsnorm_residual(const void* x, const void* residual, const void* weight, void* y,
+                                      void* sum_out, const void* weight2, void* y2, int64_t rows, int32_t dim,
+                                      float eps, int32_t dtype, void* stream) {
+    return raven::rmsnorm_pitched(x, residual, weight, y, dim, sum_out, weight2, y2, dim, rows, dim, eps, dtype, stream);
 }

@@ -294,7 +294,8 @@ def test_sandwich_block_config4_rows(pkg):
 def test_chunk_qkv_epilogue_writes_the_bits_of_the_two_launch_path(pkg, tuned, nh, hd, B, S, pos0, on_device):
     """A chunk's q | k | v product with bias, RoPE and the cache append as its epilogue (fuse_qkv_rope = 1, the default) against
     the stored product followed by raven_qkv_bias_rope_cache_append (RMM:463-481): block output and the K / V rows the block
-    appended, bit for bit.  Shapes: 128 x 128 tiles with rows of three sequences in one tile and heads across tile edges;
+    appended, bit for bit; likewise with and without padded rows for the activations the tiled GEMM reads (pad_chunk_rows;
+    n_embd 480 and 5280 are not multiples of 64).  Shapes: 128 x 128 tiles with rows of three sequences in one tile and heads across tile edges;
     256 x 256 tiles at the 3.5b head layout with the first position on the device; 256 x 256 tiles whose last tile column
     goes to 128 x 128 tiles (2048 rows x 8448 columns: 264 tiles); a single small tile with rows and columns past the end."""
     dt, h, inter = torch.bfloat16, nh * hd, 256
@@ -313,18 +314,20 @@ def test_chunk_qkv_epilogue_writes_the_bits_of_the_two_launch_path(pkg, tuned, n
     ws = pkg.hip.block_workspace(dims, B * S, "cuda")
     pos_dev = torch.tensor([pos0], dtype=torch.int32, device="cuda") if on_device else None
     results = []
-    for fuse in (1, 0):
-        tuned(fuse_qkv_rope=fuse)
+    for fuse, pad in ((1, 1), (0, 0), (0, 1), (1, 0)):
+        tuned(fuse_qkv_rope=fuse, pad_chunk_rows=pad)
         kd = _gpu_randn((2, B, nh, t_max, hd), 6)     # rows outside pos0 .. pos0 + S - 1 must stay as they are
         vd = _gpu_randn((2, B, nh, t_max, hd), 7)
         cache = pkg.hip.make_cache(kd, vd)
         out = pkg.hip.sandwich_block(dims, blk, x, torch.empty_like(x), freqs, cache, 1, B, S, pos0, ws, pos_dev=pos_dev)
         torch.cuda.synchronize()
         results.append((out.clone(), kd, vd))
-    (o1, k1, v1), (o0, k0, v0) = results
+    (o1, k1, v1), (o0, k0, v0) = results[:2]
     assert torch.equal(k1, k0), "appended K differs between the epilogue and the two-launch path"
     assert torch.equal(v1, v0), "appended V differs"
     assert torch.equal(o1, o0), "block output differs"
+    for o, k, v in results[2:]:   # rows of the activations padded to whole cache lines or not, with either q | k | v path
+        assert torch.equal(o, o0) and torch.equal(k, k0) and torch.equal(v, v0), "padded activation rows change the result"
     fresh = _gpu_randn((2, B, nh, t_max, hd), 6)
     assert torch.equal(k1[0], fresh[0]) and torch.equal(k1[1, :, :, :pos0], fresh[1, :, :, :pos0]) and torch.equal(k1[1, :, :, pos0 + S:], fresh[1, :, :, pos0 + S:])
     assert not torch.equal(k1[1, :, :, pos0:pos0 + S], fresh[1, :, :, pos0:pos0 + S])
