@@ -215,6 +215,10 @@ __global__ __launch_bounds__(16 * G, (G == 16 && kAttnU == 2 && CPL == 1 && PF) 
     // q (and the new k, v) first: these loads are the oldest, so their data is back before the K/V tiles
     typedef Piece<T, CPL> P;
     P qraw = zero_piece<T, CPL>(), kraw = zero_piece<T, CPL>(), vnew = zero_piece<T, CPL>();
+    // FUSED: the bias chunks and the (cos, sin) pairs of the row's position as well -- requested behind the tiles they would
+    // return behind them, and the rotation of q would wait for every tile load in flight
+    P bias_q = zero_piece<T, CPL>(), bias_k = zero_piece<T, CPL>();
+    alignas(16) float cs[FUSED ? E : 1];
     const int col = head * hd + ci * E;
     if (active) {
         if (FUSED) {
@@ -222,6 +226,13 @@ __global__ __launch_bounds__(16 * G, (G == 16 && kAttnU == 2 && CPL == 1 && PF) 
             qraw = load_piece<T, CPL>(row + col);
             kraw = load_piece<T, CPL>(row + h + col);
             vnew = load_piece<T, CPL>(row + 2 * h + col);
+            if (qk_bias) {
+                bias_q = load_piece<T, CPL>(qk_bias + col);
+                bias_k = load_piece<T, CPL>(qk_bias + h + col);
+            }
+            const float* f = freqs + ((int64_t)pos * (hd / 2) + ci * E / 2) * 2;
+#pragma unroll
+            for (int e = 0; e < E; e += 4) *reinterpret_cast<f32x4*>(&cs[FUSED ? e : 0]) = *reinterpret_cast<const f32x4*>(f + e);
         } else {
             qraw = load_piece<T, CPL>(q_or_qkv + (int64_t)m * h + col);
         }
@@ -268,13 +279,24 @@ __global__ __launch_bounds__(16 * G, (G == 16 && kAttnU == 2 && CPL == 1 && PF) 
     };
     Tile ta, tb;
     load_tile(start, ta);  // requested before q is touched
+    if constexpr (PF && !LOOKUP) load_tile(start + G * kAttnU, tb);  // and so is the second tile: bias and RoPE of q take a few memory latencies
 
     P qc = qraw, knew = kraw;
     if (FUSED && active) {
 #pragma unroll
-        for (int i = 0; i < CPL; ++i) {
-            qc.c[i] = bias_rope_chunk<T>(qraw.c[i], qk_bias, 0, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
-            knew.c[i] = bias_rope_chunk<T>(kraw.c[i], qk_bias, 1, h, col + i * EC, freqs, pos, hd, ci * E + i * EC);
+        for (int i = 0; i < CPL; ++i) {  // the arithmetic of bias_rope_chunk, on operands loaded above
+            if (qk_bias) {
+#pragma unroll
+                for (int e = 0; e < EC; ++e) {
+                    qc.c[i].v[e] = from_f32<T>(to_f32(qraw.c[i].v[e]) + to_f32(bias_q.c[i].v[e]));
+                    knew.c[i].v[e] = from_f32<T>(to_f32(kraw.c[i].v[e]) + to_f32(bias_k.c[i].v[e]));
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < EC; e += 2) {
+                rope_pair<T>(qc.c[i].v[e], qc.c[i].v[e + 1], cs[FUSED ? i * EC + e : 0], cs[FUSED ? i * EC + e + 1 : 0]);
+                rope_pair<T>(knew.c[i].v[e], knew.c[i].v[e + 1], cs[FUSED ? i * EC + e : 0], cs[FUSED ? i * EC + e + 1 : 0]);
+            }
         }
         if (group == 0 && pos >= start && pos < end) {
             store_piece<T, CPL>(static_cast<T*>(cv.k) + head_off + (int64_t)pos * hd + ci * E, knew);
@@ -315,14 +337,14 @@ __global__ __launch_bounds__(16 * G, (G == 16 && kAttnU == 2 && CPL == 1 && PF) 
     };
     constexpr int STEP = G * kAttnU;
     if constexpr (PF && !LOOKUP) {
-        // two tiles in turn, the next one requested before the current one is used; always whole pairs (a tile past the
-        // range re-reads cached lines and adds nothing), so that the number of loads in flight is the same on every path
-        // and the waits can leave the younger tile's loads outstanding
+        // two tiles in turn, each requested again as soon as it is used, the first two in front of everything else; always
+        // whole pairs (a tile past the range re-reads cached lines and adds nothing), so that the number of loads in flight
+        // is the same on every path and the waits can leave the younger tile's loads outstanding
         for (int base = start; base < end_c; base += 2 * STEP) {  // trip count is uniform over the workgroup
-            load_tile(base + STEP, tb);
             consume(base, ta);
             load_tile(base + 2 * STEP, ta);
             consume(base + STEP, tb);
+            load_tile(base + 3 * STEP, tb);
         }
     } else {
         for (int base = start; base < end_c;) {
@@ -480,7 +502,7 @@ __global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __
     }
     __syncthreads();
     const int64_t blk_stride = (int64_t)pv.block_size * pv.nh * hd;
-    const int64_t lane_off = head * pv.head_stride + ci * E;
+    const int64_t lane_off = head * pv.head_stride + min(ci, hd / E - 1) * E;  // lanes past the head row repeat its last chunk (their q is zero)
     auto elem_of = [&](int p) {  // this lane's first element of position p
         const int i = block_of(p) - blk0;
         const int blk = i < kTbl ? tbl[i] : table[blk0 + i];
@@ -508,36 +530,32 @@ __global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __
     float m_run = -INFINITY, l_run = 0.f, o[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) o[e] = 0.f;
-    for (int base = start; base < end; base += G * U) {  // trip count is uniform over the workgroup
+    // As in decode_attention_kernel: every load of a tile is unconditional (positions past the cached ones of this range
+    // re-read the range's last cached position, and their scores are masked), so that all of a tile's loads are in
+    // flight before the first is waited for; FUSED: the new token's own position is added from registers behind the loop.
+    const int end_c = FUSED ? min(end, pos) : end;
+    const int last_ok = end_c - 1;  // inside this workgroup's range, so that its page is among the staged table entries
+    for (int base = start; base < end_c; base += G * U) {  // trip count is uniform over the workgroup
         P kc[U], vc[U];
 #pragma unroll
         for (int j = 0; j < U; ++j) {
-            const int p = base + j * G + group;
-            if (FUSED && p == pos) {
-                kc[j] = knew;
-                vc[j] = vnew;
-            } else if (active && p < end) {
-                const int64_t off = elem_of(p);
-                kc[j] = load_piece<T, CPL, true>(K + off);
-                vc[j] = load_piece<T, CPL, true>(V + off);
-            } else {
-                kc[j] = zero_piece<T, CPL>();
-                vc[j] = zero_piece<T, CPL>();
-            }
+            const int64_t off = elem_of(min(base + j * G + group, last_ok));
+            kc[j] = load_piece<T, CPL, true>(K + off);
+            vc[j] = load_piece<T, CPL, true>(V + off);
         }
         float sc[U], m_new = m_run;
 #pragma unroll
         for (int j = 0; j < U; ++j) {
             sc[j] = row16_sum(dot_piece<T, CPL>(qc, kc[j])) * scale_log2;
-            if (base + j * G + group >= end) sc[j] = -INFINITY;
+            if (base + j * G + group >= end_c) sc[j] = -INFINITY;
             m_new = fmaxf(m_new, sc[j]);
         }
         if (m_new == -INFINITY) continue;
-        const float corr = exp2f(m_run - m_new);
+        const float corr = exp2_raw(m_run - m_new);
         float pe[U], psum = 0.f;
 #pragma unroll
         for (int j = 0; j < U; ++j) {
-            pe[j] = exp2f(sc[j] - m_new);
+            pe[j] = exp2_raw(sc[j] - m_new);
             psum += pe[j];
         }
         l_run = l_run * corr + psum;
@@ -548,6 +566,15 @@ __global__ __launch_bounds__(256) void paged_decode_attention_kernel(const T* __
             for (int j = 0; j < U; ++j) acc = __builtin_fmaf(pe[j], to_f32(vc[j].c[e / EC].v[e % EC]), acc);
             o[e] = acc;
         }
+        m_run = m_new;
+    }
+    if (FUSED && group == 0 && len > 0 && pos >= start && pos < end) {  // the new token's own position, from registers
+        const float sc = row16_sum(dot_piece<T, CPL>(qc, knew)) * scale_log2;
+        const float m_new = fmaxf(m_run, sc);
+        const float corr = exp2_raw(m_run - m_new), pe = exp2_raw(sc - m_new);
+        l_run = l_run * corr + pe;
+#pragma unroll
+        for (int e = 0; e < E; ++e) o[e] = __builtin_fmaf(pe, to_f32(vnew.c[e / EC].v[e % EC]), o[e] * corr);
         m_run = m_new;
     }
     merge_wave_rows<E>(m_run, l_run, o);
