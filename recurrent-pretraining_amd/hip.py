@@ -245,13 +245,15 @@ def gemm_swiglu(x, fc):
     return y
 
 
-def register_packed_weight(w: torch.Tensor) -> torch.Tensor:
+def register_packed_weight(w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Line-aligned copy of a bf16 weight matrix [rows, K] for the tiled GEMM; returns the copy, which the caller keeps
-    alive (together with w) until unregister_packed_weight(w)."""
+    alive (together with w) until unregister_packed_weight(w).  `out`: a buffer of an earlier registration of the same
+    shape to fill again (its address may be held by captured graphs)."""
     assert w.dim() == 2 and w.dtype == torch.bfloat16 and w.is_contiguous()
     rows, K = w.shape
     n = load().raven_packed_weight_bytes(rows, K)
-    packed = torch.empty(n, dtype=torch.uint8, device=w.device)
+    packed = out if out is not None else torch.empty(n, dtype=torch.uint8, device=w.device)
+    assert packed.numel() == n and packed.dtype == torch.uint8 and packed.device == w.device
     rc = load().raven_register_packed_weight(_ptr(w, "w"), rows, K, _ptr(packed, "packed"), _stream())
     _check(rc, "raven_register_packed_weight")
     return packed

@@ -134,8 +134,13 @@ class _PackedWeights:
         key = tuple((w.data_ptr(), w._version) for w in mats)
         if key == self.key:
             return
-        self.drop()
-        self.ptr_owner = [(w.detach(), hip.register_packed_weight(w.detach())) for w in mats]
+        # matrices that only changed in place keep their copy's buffer (a captured graph may hold its address)
+        old = {(w.data_ptr(), tuple(w.shape)): buf for w, buf in self.ptr_owner}
+        keep = {(w.data_ptr(), tuple(w.shape)) for w in mats}
+        for w, _ in self.ptr_owner:
+            if (w.data_ptr(), tuple(w.shape)) not in keep:
+                hip.unregister_packed_weight(w)
+        self.ptr_owner = [(w.detach(), hip.register_packed_weight(w.detach(), out=old.get((w.data_ptr(), tuple(w.shape))))) for w in mats]
         self.key = key
 
     def drop(self) -> None:

@@ -298,6 +298,15 @@ def test_chunk_forward_reads_line_aligned_weight_copies_and_keeps_them_current(p
         check(got.logits, want.logits, torch.bfloat16, f"bf16 logits, weights of seed {seed}")
         outs[seed] = got.logits.clone()
     assert not torch.equal(outs[0], outs[1])
+    # weights that change in place keep the buffers of their copies (a captured graph may hold their addresses)
+    model.pack_weights()
+    bufs = [buf.data_ptr() for _, buf in model._packed.ptr_owner]
+    w0 = O.make_weights(s, seed=0, dtype=torch.bfloat16)
+    w0["freqs_cis"] = w0["freqs_cis"].to(torch.bfloat16)
+    model.load_state_dict(w0, strict=True)
+    again = model(input_ids=ids.cuda(), input_states=states.cuda())
+    assert [buf.data_ptr() for _, buf in model._packed.ptr_owner] == bufs
+    assert torch.equal(again.logits, outs[0])
     finalizer = model._packed_finalizer
     model(input_ids=ids.cuda(), input_states=states.cuda())
     assert model._packed.ptr_owner and finalizer.alive
