@@ -1039,7 +1039,7 @@ def _block_weights(pkg, dev, prefix):
         dev[f"{prefix}.mlp.fc.weight"], dev[f"{prefix}.mlp.proj.weight"])
 
 
-@pytest.mark.parametrize("B", [1, 32])
+@pytest.mark.parametrize("B", [1, 8, 32])
 def test_core_iteration_nebel_bf16_config3(pkg, nebel_core, B):
     """One recurrence iteration at decode, 1024 cached positions per step slot filled with N(0,1)."""
     s, w, dev = nebel_core
@@ -1247,8 +1247,11 @@ def test_slice_sums_folded_into_the_norm_launch_change_no_bit(pkg, nebel_core, t
     slots = [[it * 4 + j for j in range(4)] for it in range(r)]
     lnf = rnd((h,), dt, 41, 0.02, 1.0).cuda()
     outs = []
-    for fold in (1, 0):
-        tuned(fuse_sums_norm=fold)
+    # (folding, K slices): the default, then folding on and off with three slices asked for (left to itself, a
+    # 5280 x 5280 product of up to 16 rows is K-split only where the norm launch adds the slices, so that folding on and
+    # off would compare two summation orders)
+    for fold, ks in ((1, 0), (1, 3), (0, 3)):
+        tuned(fuse_sums_norm=fold, linear_ks=ks)
         _, _, kd, vd, cache = _nebel_cache(pkg, 4 * r, B, T, dt, 930)
         out = torch.empty_like(state)
         pkg.hip.core_iterations(dims, dev["transformer.adapter.weight"], blocks, state, embeds, out, freqs, cache, slots, B, 1, T, ws, ln_f=lnf)
@@ -1256,9 +1259,9 @@ def test_slice_sums_folded_into_the_norm_launch_change_no_bit(pkg, nebel_core, t
         _, _, kd1, vd1, cache1 = _nebel_cache(pkg, 4, B, T, dt, 930)
         pkg.hip.core_iteration(dims, dev["transformer.adapter.weight"], blocks, state, embeds, one, freqs, cache1, 0, B, 1, T, ws)
         outs.append((out, kd[:, :, :, T].clone(), vd[:, :, :, T].clone(), one, kd1[:, :, :, T].clone()))
-    for a, b in zip(*outs):
-        assert torch.equal(a, b)
-    assert torch.isfinite(outs[0][0].float()).all()
+    for a, b, c in zip(*outs):
+        assert torch.equal(b, c)   # (a: asking for the slices also K-splits Wqkv and mlp.fc, so its bits are its own)
+        assert torch.isfinite(a.float()).all() and a.shape == b.shape
 
 
 def test_core_iteration_nebel_fp32_against_fp32_oracle(pkg):
