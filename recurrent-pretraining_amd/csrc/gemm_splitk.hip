@@ -346,7 +346,7 @@ int linear_leave_sums(const void* x0, const void* x1, const void* w, int ldw, co
     *ks_left = 0;
     bool split = g_fuse_sums_norm && dtype == RAVEN_BF16 && M >= 2 && M <= 32 && N % 16 == 0 && N <= 8192 && K0 % 32 == 0 && K1 % 32 == 0 &&
                  workspace != nullptr && ((uintptr_t)workspace & 255) == 0 && K0 / 128 + K1 / 128 >= 8 && M > g_linear_min_rows;
-    if (split && !ldw && g_linear_ks == 0) split = N / 16 < 2 * ns_cus() && M >= 5;  // every row count the K-split kernel takes: its second launch is saved, and the norm launch requests all slices of a row at once (5 / 8 / 12 rows: 228.7 / 350.7 / 501.5 tokens/s against 228.3 / 348.5 / 495.0 with the K split only from 13 rows or K >= 8192)
+    if (split && !ldw && g_linear_ks == 0) split = N / 16 < 2 * ns_cus() && (M >= 5 || K0 + K1 >= 8192);  // from 5 rows on, from 2 for long K: the product's second launch is saved, and the norm launch requests all slices of a row at once (5 / 8 / 12 rows: 228.7 / 350.7 / 501.5 tokens/s against 228.3 / 348.5 / 495.0 with the K split only from 13 rows or K >= 8192)
     if (!split) {
         if (ldw) return linear_column_block(x0, w, ldw, extra, y, 0, M, N, K0, workspace, workspace_bytes, s);
         return raven_linear(x0, x1, w, residual, y, M, N, K0, K1, 0, 0, dtype, workspace, workspace_bytes, s);
