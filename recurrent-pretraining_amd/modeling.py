@@ -248,6 +248,7 @@ class RavenForCausalLM(RavenPreTrainedModel, GenerationMixin):
         self._packed = _PackedWeights()                      # line-aligned copies of weight matrices for prompt chunks
         self.pack_chunk_weights = True                       # False: chunks read the matrices as they are (no copies are made)
         self._packed_finalizer = weakref.finalize(self, self._packed.drop)
+        self._packed_owner = id(self)
         self.eval()
 
     # ---- small helpers -------------------------------------------------------------------------
@@ -650,6 +651,11 @@ class RavenForCausalLM(RavenPreTrainedModel, GenerationMixin):
         """Makes (or refreshes) the line-aligned copies of Wqkv, attn.proj and mlp.fc that products over 33 and more token rows
         read (bf16 models whose n_embd * 2 bytes is not a multiple of 128: n_embd = 5280).  Every block call over such a
         chunk calls this; call it by hand after changing a weight through `.data`, which leaves no trace a check could see."""
+        if not self._packed_finalizer.alive or self._packed_owner != id(self):
+            # a copy of a model (copy.deepcopy) starts without registrations of its own
+            self._packed = _PackedWeights()
+            self._packed_finalizer = weakref.finalize(self, self._packed.drop)
+            self._packed_owner = id(self)
         t = self.transformer
         blocks = list(t.prelude) + list(t.core_block) + list(t.coda)
         self._packed.ensure([w for b in blocks for w in (b.attn.Wqkv.weight, b.attn.proj.weight, b.mlp.fc.weight)])
