@@ -251,32 +251,45 @@ __device__ __forceinline__ void store_tiles_rope(const TiledArgs& a, const f32x4
     const int first = r.pos_dev ? *r.pos_dev : r.pos0;
     Chunk<bf16> bch = zero_chunk<bf16>();
     if (sec < 2 && r.qk_bias) bch = load_chunk(r.qk_bias + sec * h + col);
-    auto where = [&](int it, int& m, int& b, int& pos) {
-        m = min(tile_m * BM + row0 + it * RS, a.M - 1);
-        b = m / r.S;
-        pos = first + (m - b * r.S);
+    // sequence and position inside it of this lane's row: one division for the first row, then RS rows further per unit
+    // (two walkers: the requests run PD units ahead of the units that are stored)
+    struct RowWalk {
+        int b, sq;
     };
+    const int m_first = tile_m * BM + row0;
+    RowWalk ahead{m_first / r.S, 0}, here;
+    ahead.sq = m_first - ahead.b * r.S;
+    here = ahead;
+    auto advance = [&](RowWalk& w) {
+        w.sq += RS;
+        while (w.sq >= r.S) {
+            w.sq -= r.S;
+            ++w.b;
+        }
+    };
+    // the table rows of positions pos0 + sq: sq < S whatever the row, so a row past M still names a valid table row
+    const float* const f_base = r.freqs + ((int64_t)first * (r.hd / 2) + d / 2) * 2;
+    const int f_step = (r.hd / 2) * 2;
     f32x4 fq[PD][2];
-    auto request = [&](int it, f32x4 (&f)[2]) {
-        int m, b, pos;
-        where(it, m, b, pos);
-        const float* fp = r.freqs + ((int64_t)pos * (r.hd / 2) + d / 2) * 2;
+    auto request = [&](f32x4 (&f)[2]) {
+        const float* fp = f_base + (int64_t)ahead.sq * f_step;
         f[0] = *reinterpret_cast<const f32x4*>(fp);
         f[1] = *reinterpret_cast<const f32x4*>(fp + 4);
+        advance(ahead);
     };
 #pragma unroll
-    for (int it = 0; it < PD; ++it) request(it, fq[it]);
+    for (int it = 0; it < PD; ++it) request(fq[it]);
     lay_tiles_lds<false, TM, TN, WM, WN>(acc, wave, lane, lds_base);
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
         const int row = row0 + it * RS;
         const u32x4 v = *reinterpret_cast<const lds_u32x4*>(lds_base + row * RB + ((unit ^ (row & (U - 1))) * 16));
-        int m, b, pos;
-        where(it, m, b, pos);
+        const int m = m_first + it * RS, b = here.b, pos = first + here.sq;
+        advance(here);
         Chunk<bf16> x;
         *reinterpret_cast<u32x4*>(x.v) = v;
         const f32x4 f0 = fq[it % PD][0], f1 = fq[it % PD][1];
-        if (it + PD < ITERS) request(it + PD, fq[it % PD]);
+        if (it + PD < ITERS) request(fq[it % PD]);
         if (sec < 2) {
             if (r.qk_bias) {
 #pragma unroll
