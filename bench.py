@@ -645,8 +645,9 @@ def decode_record(pkg, model, B, prompt_len, steps, warmup, r, use_graph):
     nat = model._natives()
     n_slots = 128 if B == 1 else 32
     n_it = n_slots // 4
-    kc = torch.empty(n_slots, B, nh, T + 1, hd, device=dev, dtype=torch.bfloat16).normal_()
-    vc = torch.empty(n_slots, B, nh, T + 1, hd, device=dev, dtype=torch.bfloat16).normal_()
+    t_cap = pkg.cache.line_aligned_positions(T + 1, hd, torch.bfloat16)   # the capacity HuginnDynamicCache allocates for T + 1 positions
+    kc = torch.empty(n_slots, B, nh, t_cap, hd, device=dev, dtype=torch.bfloat16).normal_()
+    vc = torch.empty(n_slots, B, nh, t_cap, hd, device=dev, dtype=torch.bfloat16).normal_()
     kv = pkg.hip.make_cache(kc, vc)
     ws = pkg.hip.block_workspace(nat["dims"], B, dev)
     state = torch.randn(B, h, device=dev, dtype=torch.bfloat16)

@@ -1143,8 +1143,8 @@ class DecodeRunner:
         if c.has_gap(last_step, pos0):
             raise NotImplementedError("the decode runner's fixed launch sequence needs a cache whose earlier tokens were all "
                                       f"computed with at least {self.r} recurrences; use forward() for partially filled caches")
-        if pos0 + 1 > c.t_max:
-            c.ensure(1, 0, self.B, m.config.n_heads, m.config.head_dim, pos0 + 1, m.dtype, m.device)  # grows; pointers move
+        if pos0 + 1 > c.t_max or (c.max_length is not None and pos0 + 1 > c.max_length):
+            c.ensure(1, 0, self.B, m.config.n_heads, m.config.head_dim, pos0 + 1, m.dtype, m.device)  # grows (pointers move), or refuses past max_length
             self.graph = None
         self.ids.copy_(ids.view(-1))
         self.pos.fill_(pos0)

@@ -123,6 +123,24 @@ def test_cache_growth_keeps_contents_and_slot_order(pkg):
         fixed.update(torch.zeros(1, 1, 1, 4), torch.zeros(1, 1, 1, 4), 0)
 
 
+def test_cache_capacity_keeps_head_regions_on_whole_cache_lines(pkg):
+    """The storage of a head ([t_max, head_dim], contiguous) is a whole number of 128-byte lines: 192-byte rows (head_dim 96,
+    bf16) get an even capacity, rows of 128 or 256 bytes any; max_length still bounds the sequence, not the storage."""
+    f = pkg.cache.line_aligned_positions
+    assert f(1025, 96, torch.bfloat16) == 1026 and f(1026, 96, torch.bfloat16) == 1026 and f(537, 96, torch.bfloat16) == 538
+    assert f(1025, 96, torch.float32) == 1025 and f(1025, 64, torch.bfloat16) == 1025 and f(1025, 128, torch.bfloat16) == 1025
+    assert f(5, 8, torch.bfloat16) == 8 and f(9, 8, torch.bfloat16) == 16          # 16-byte rows: eight to a line
+    for t in range(1, 40):
+        for hd, dt in ((96, torch.bfloat16), (8, torch.bfloat16), (24, torch.float32), (4, torch.float32)):
+            cap = f(t, hd, dt)
+            assert cap >= t and cap * hd * torch.empty((), dtype=dt).element_size() % 128 == 0 and cap - t < 128
+    c = pkg.HuginnDynamicCache(max_length=7)
+    c.update(torch.zeros(1, 2, 7, 96, dtype=torch.bfloat16), torch.zeros(1, 2, 7, 96, dtype=torch.bfloat16), 0)
+    assert c.t_max == 8 and c.get_seq_length() == 7
+    with pytest.raises(ValueError, match="max_length"):
+        c.update(torch.zeros(1, 2, 1, 96, dtype=torch.bfloat16), torch.zeros(1, 2, 1, 96, dtype=torch.bfloat16), 0)
+
+
 def test_cache_size_known_answers(pkg):
     """The reference notebooks' cache sizes (examples/inference_demo.ipynb:252, 373) from the
     contiguous cache's own accounting."""
