@@ -107,7 +107,10 @@ const char* raven_last_error(void);
  * applies bias, RoPE and the cache append in its epilogue; 0 = the product is stored and raven_qkv_bias_rope_cache_append's
  * kernel follows; same bits either way), pad_chunk_rows (1 = inside the composed entry points the activations that the tiled
  * GEMMs of a bf16 chunk read -- norm_1's and norm_3's output, the attention output -- are laid out in the workspace with rows
- * padded to a multiple of 64 elements when n_embd is not one; 0 = rows n_embd elements apart; same bits either way).
+ * padded to a multiple of 64 elements when n_embd is not one; 0 = rows n_embd elements apart; same bits either way),
+ * pad_decode_rows (1 = decode steps of 17..32 bf16 rows inside the composed entry points run Wqkv and mlp.fc over the padded
+ * length when line-aligned copies of both matrices of every block are registered -- zeros in the pads of the copies and of
+ * norm_1's / norm_3's output, another summation order than over the matrices themselves; 0 = never).
  * Not needed in normal use: the defaults are the tuned values.  The knobs are process-global
  * state read at every launch: changing them while another thread or stream is inside a call of this library is a race. */
 int raven_set_tuning(const char* key, int32_t value);
@@ -160,7 +163,9 @@ int    raven_linear(const void* x0, const void* x1, const void* w, const void* r
  * 128-byte aligned, rows padded with zeros to a multiple of 64 elements -- on `stream`, and from then on every product
  * whose weight pointer is `w`, with this K and these rows, that runs on the tiled kernels reads the copy: same values in
  * the same order, same bits.  The caller registers again after changing w, and calls raven_unregister_packed_weight(w)
- * before it frees either buffer.  Products of fewer rows (decode) always read w itself. */
+ * before it frees either buffer.  Products of fewer rows read w itself, with one exception: decode steps of 17..32 rows
+ * inside raven_sandwich_block / raven_core_iteration(s) / raven_paged_decode_blocks take Wqkv and mlp.fc from the copies
+ * when both are registered for every block of the call (5 % faster there; see pad_decode_rows under raven_set_tuning). */
 int64_t raven_packed_weight_bytes(int32_t rows, int32_t K);
 int     raven_register_packed_weight(const void* w, int32_t rows, int32_t K, void* packed, void* stream);
 int     raven_unregister_packed_weight(const void* w);

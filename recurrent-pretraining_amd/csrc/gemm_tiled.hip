@@ -818,6 +818,15 @@ struct PackedWeight {
 static std::mutex g_packed_mutex;
 static std::unordered_map<const void*, PackedWeight> g_packed;
 
+// The registered copy of w ([rows, K]) and its row pitch, or null
+const void* packed_weight_of(const void* w, int rows, int K, int* ld) {
+    std::lock_guard<std::mutex> lock(g_packed_mutex);
+    const auto it = g_packed.find(w);
+    if (it == g_packed.end() || it->second.K != K || it->second.rows != rows) return nullptr;
+    *ld = it->second.ld;
+    return it->second.packed;
+}
+
 __global__ __launch_bounds__(256) void pack_rows_kernel(const bf16* __restrict__ w, bf16* __restrict__ out, int K, int ld) {
     const int64_t row = blockIdx.x;
     for (int c = threadIdx.x * 8; c < ld; c += 256 * 8) {

@@ -134,6 +134,8 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
             if (y) store_chunk(y + row * ldy + c * E, co);
         }
     }
+    // padded rows: the pad is written as zeros, so that a product may also run over the padded length
+    if (y && ldy > dim && (int)threadIdx.x < (ldy - dim) / E) store_chunk(y + row * ldy + dim + threadIdx.x * E, zero_chunk<T>());
     if (weight2 == nullptr) return;
 
     inv = rsqrtf(block_sum_256(ss2, red) / (float)dim + eps);
@@ -148,6 +150,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
             store_chunk(y2 + row * ldy2 + c * E, co);
         }
     }
+    if (ldy2 > dim && (int)threadIdx.x < (ldy2 - dim) / E) store_chunk(y2 + row * ldy2 + dim + threadIdx.x * E, zero_chunk<T>());
 }
 
 int g_norm_early = -1;  // raven_set_tuning("norm_early"): -1 = by row count, 0 / 1 = weights fetched late / early
@@ -156,14 +159,18 @@ int g_norm_early = -1;  // raven_set_tuning("norm_early"): -1 = by row count, 0 
 // consume the result, as one launch: bf16, up to 32 rows of at most 8192 columns.  sum_out (may be null) receives the
 // product's value, y (may be null) the first norm's, y2 the second's when weight2 is given.
 int splitk_sums_then_norm(const float* partial, int ks, const float* extra, const void* residual, void* sum_out, const void* weight,
-                          void* y, const void* weight2, void* y2, int rows, int dim, float eps, hipStream_t s) {
+                          void* y, const void* weight2, void* y2, int rows, int dim, float eps, hipStream_t s, int ldy, int ldy2) {
     RAVEN_REQUIRE(partial && ks >= 1 && weight && (y || y2) && (weight2 == nullptr) == (y2 == nullptr), "splitk_sums_then_norm: bad arguments");
+    if (ldy <= 0) ldy = dim;
+    if (ldy2 <= 0) ldy2 = dim;
+    RAVEN_REQUIRE(ldy >= dim && ldy2 >= dim && ldy % 8 == 0 && ldy2 % 8 == 0 && ldy - dim <= 8 * kNormThreads && ldy2 - dim <= 8 * kNormThreads,
+                  "splitk_sums_then_norm: bad output row pitch %d / %d", ldy, ldy2);
     RAVEN_REQUIRE(rows >= 1 && dim % 8 == 0 && dim / 8 <= kNormThreads * 4, "splitk_sums_then_norm: unsupported shape %d x %d", rows, dim);
     SplitSums sp{partial, extra, ks, (int64_t)rows * dim};
 #define RAVEN_SPLIT_NORM(KS_)                                                                                            \
     case KS_:                                                                                                           \
         rmsnorm_kernel<bf16, 4, true, KS_><<<dim3((unsigned)rows), dim3(kNormThreads), 0, s>>>(                          \
-            nullptr, (const bf16*)residual, (const bf16*)weight, (bf16*)y, (bf16*)sum_out, (const bf16*)weight2, (bf16*)y2, dim, eps, sp, dim, dim); \
+            nullptr, (const bf16*)residual, (const bf16*)weight, (bf16*)y, (bf16*)sum_out, (const bf16*)weight2, (bf16*)y2, dim, eps, sp, ldy, ldy2); \
         break;
     switch (ks) {
         RAVEN_SPLIT_NORM(1) RAVEN_SPLIT_NORM(2) RAVEN_SPLIT_NORM(3) RAVEN_SPLIT_NORM(4)
@@ -190,7 +197,8 @@ int rmsnorm_pitched(const void* x, const void* residual, const void* weight, voi
     RAVEN_REQUIRE(dim / elts <= kNormThreads * kNormMaxChunks, "rmsnorm: dim %d too large (max %d)", dim,
                   kNormThreads * kNormMaxChunks * elts);
     RAVEN_REQUIRE(rows > 0 && rows < (1ll << 31), "rmsnorm: bad row count %lld", (long long)rows);
-    RAVEN_REQUIRE(ldy >= dim && ldy2 >= dim && ldy % elts == 0 && ldy2 % elts == 0, "rmsnorm: bad output row pitch %d / %d", ldy, ldy2);
+    RAVEN_REQUIRE(ldy >= dim && ldy2 >= dim && ldy % elts == 0 && ldy2 % elts == 0 && ldy - dim <= elts * kNormThreads &&
+                      ldy2 - dim <= elts * kNormThreads, "rmsnorm: bad output row pitch %d / %d", ldy, ldy2);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int per_thread = (dim / elts + kNormThreads - 1) / kNormThreads;
     const bool early = g_norm_early >= 0 ? g_norm_early != 0 : rows <= 64;

@@ -437,9 +437,10 @@ class RavenForCausalLM(RavenPreTrainedModel, GenerationMixin):
         return self._native
 
     def _workspace(self, M: int) -> torch.Tensor:
-        """Scratch for a block over M token rows; every block call fetches it, so this is also where a chunk of 33 rows or
-        more makes sure that the line-aligned weight copies are current."""
-        if M >= 33 and self.dtype == torch.bfloat16 and self.pack_chunk_weights:
+        """Scratch for a block over M token rows; every block call fetches it, so this is also where a call over 17 rows or
+        more (decode steps of 17..32 sequences read Wqkv and mlp.fc through them, chunks of 33 rows and more all three matrices)
+        makes sure that the line-aligned weight copies are current."""
+        if M >= 17 and self.dtype == torch.bfloat16 and self.pack_chunk_weights:
             self.pack_weights()
         ws = self._scratch.get(("ws", M))
         if ws is None:
@@ -1069,6 +1070,8 @@ class DecodeRunner:
         self.latents = torch.empty(batch, h, dtype=dt, device=dev)
         self.logits = torch.empty(batch, cfg.padded_vocab_size, dtype=torch.float32, device=dev)
         self.next_ids = torch.zeros(batch, dtype=torch.int64, device=dev)
+        if batch >= 17 and model.dtype == torch.bfloat16 and model.pack_chunk_weights:
+            model.pack_weights()  # decode steps of 17..32 rows read Wqkv and mlp.fc through their line-aligned copies
         self.ws = hip.block_workspace(model._natives()["dims"], batch, dev)
         self.use_graph = use_graph and cfg.test_time_noise <= 0  # the noise draws are not part of a replayable launch sequence
         self.graph: Optional[torch.cuda.CUDAGraph] = None

@@ -178,6 +178,8 @@ class PagedDecoder:
             m, cfg = self.model, self.cfg
             dev, dt, h = m.device, m.dtype, cfg.n_embd
             nat = m._natives()
+            if B >= 17 and dt == torch.bfloat16 and m.pack_chunk_weights:
+                m.pack_weights()  # decode steps of 17..32 rows read Wqkv and mlp.fc through their line-aligned copies
             mk = lambda: torch.empty(B, h, dtype=dt, device=dev)
             self._ws[key] = {
                 "ids": torch.zeros(B, dtype=torch.int64, device=dev),

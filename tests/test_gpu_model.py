@@ -1040,8 +1040,10 @@ def _block_weights(pkg, dev, prefix):
 
 
 @pytest.mark.parametrize("B", [1, 8, 32])
-def test_core_iteration_nebel_bf16_config3(pkg, nebel_core, B):
-    """One recurrence iteration at decode, 1024 cached positions per step slot filled with N(0,1)."""
+def test_core_iteration_nebel_bf16_config3(pkg, nebel_core, tuned, B):
+    """One recurrence iteration at decode, 1024 cached positions per step slot filled with N(0,1).  At 32 rows also with
+    line-aligned copies of Wqkv and mlp.fc registered: the step then runs those two products over operands with padded
+    rows (zeros in the pad), another summation order held to the same bar."""
     s, w, dev = nebel_core
     dt, h, nh, hd, T = torch.bfloat16, s.n_embd, s.n_heads, s.head_dim, 1024
     t_max = T + 1
@@ -1099,6 +1101,28 @@ def test_core_iteration_nebel_bf16_config3(pkg, nebel_core, B):
         assert close(kd[j, :, :, T], ref_cache.key_cache[2 + j][T])[1] <= 5e-2, f"appended K slot {j}"
         assert close(vd[j, :, :, T], ref_cache.value_cache[2 + j][T])[1] <= 5e-2, f"appended V slot {j}"
     assert torch.equal(kd[:, :, :, :T].cpu(), kc[:, :, :, :T]), "cached positions must be untouched"
+    if B == 32:
+        mats = [dev[f"transformer.core_block.{j}.{name}.weight"] for j in range(4) for name in ("attn.Wqkv", "mlp.fc")]
+        keep = [pkg.hip.register_packed_weight(m_) for m_ in mats]
+        try:
+            outs = {}
+            for on in (1, 0):
+                tuned(pad_decode_rows=on)
+                kd3, vd3 = kc.cuda(), vc.cuda()
+                o3 = torch.empty(B, h, dtype=dt, device="cuda")
+                pkg.hip.core_iteration(dims, dev["transformer.adapter.weight"], blocks, state.view(B, h).cuda(), embeds.view(B, h).cuda(), o3,
+                                       freqs, pkg.hip.make_cache(kd3, vd3), 0, B, 1, T, ws)
+                outs[on] = (o3, kd3[:, :, :, T].clone())
+            assert torch.equal(outs[0][0], out) and torch.equal(outs[0][1], kd[:, :, :, T])   # switched off: the bits of the run above
+            assert not torch.equal(outs[1][0], out)                                            # switched on: another summation order
+            e3, e3_alt = close(outs[1][0], want.view(B, h))[1], close(outs[1][0], alt.view(B, h))[1]
+            print(f"core iteration B={B}, padded rows: rel-L2 vs oracle {e3:.3e}, vs fp32-accumulate oracle {e3_alt:.3e}")
+            assert min(e3, e3_alt) <= max(1.5 * floor, 1e-2) and e3 <= 5e-2
+            check(outs[1][1][0], ref_cache.key_cache[2][T], dt, "appended K slot 0, padded rows", ulps=ULPS_COMPOSED)
+        finally:
+            for m_ in mats:
+                pkg.hip.unregister_packed_weight(m_)
+        del keep
     # a single SandwichBlock with the closing ln_f folded in
     x_in = rnd((B, h), dt, 77)
     lnw = rnd((h,), dt, 78, 0.02, 1.0)
