@@ -87,8 +87,9 @@ const char* raven_last_error(void);
  * results never depend on them.  Keys: gemv_units_per_wave, gemv_interleave, gemv_nontemporal,
  * gemv_wgs_per_cu, gemv1_pairs_norm, gemv1_pairs_plain, gemm_four_tiles (0 / 1 / 2 = never / by rule / always use
  * the four-tile MFMA variant), attn_split_target / attn_big_grid (workgroups a split decode-attention launch aims
- * for / from which its 2-positions-per-row variant is used), attn_nosplit_pairs ((head, row) pairs from which a launch is
- * never split, at most 1024), rope_tiled_rows (chunk length from which raven_qkv_bias_rope_cache_append works on tiles
+ * for / from which its 2-positions-per-row variant is used), attn_nosplit_pairs ((head, row) pairs from which a launch over the contiguous cache is
+ * never split, at most 1024; the paged entry point stops splitting at 1024), attn_nosplit_len (cache positions up to
+ * which two rows and more over the contiguous cache are not split either; 0 = off), rope_tiled_rows (chunk length from which raven_qkv_bias_rope_cache_append works on tiles
  * of one head and 64 positions), attn_wide (longest cache for which few (head, row) pairs get
  * one 1024-thread workgroup each instead of a split launch; 0 = never), gemm_mfma_min_rows (fewest rows the MFMA
  * kernels take; fewer go to the vector kernels), linear_min_rows (most rows raven_linear still hands to the kernels
@@ -98,7 +99,8 @@ const char* raven_last_error(void);
  * no tile-count rule, 3 = 256 x 256 by the eight-wave kernel instead of the four-wave ring kernel), gemm_tiled_split_tail
  * (1 = the tile columns of a last round that fills at most half the chip go to
  * 128 x 128 tiles, 0 = never), prefill_waves (waves per workgroup of the chunk attention at head_dim 96: 0 = by shape, 4 or 6),
- * attn_prefetch (1 = an unsplit decode-attention launch requests a tile before it uses the one before, 0 = never),
+ * attn_prefetch (1 = an unsplit decode-attention launch of fewer than 256 or of 1024 and more (head, row) pairs requests a
+ * tile before it uses the one before, 2 = every launch does, 0 = never),
  * gemm_ragged (1 = a 5..32-row product whose output columns divide into about two workgroups per compute unit runs as one
  * round of workgroups with a partly empty last tile, 0 = whole tiles only), norm_early (1 / 0 = the RMSNorm kernel requests
  * its weights before / after the row reduction, -1 = by row count), fuse_sums_norm (1 = a K-split product that feeds a

@@ -658,7 +658,8 @@ __global__ __launch_bounds__(256) void paged_qkv_rope_append_kernel(const T* __r
 constexpr int kAttnMaxSplits = 32;
 static_assert(kAttnMaxSplits == kCombineSplits, "the merge kernel holds one partial output per split in registers");
 int g_rope_tiled_rows = 16;       // chunk length from which the append kernel works on (head, 16 positions) tiles ("rope_tiled_rows")
-int g_attn_nosplit_pairs = 1024;  // (head, row) pairs from which a launch is never split ("attn_nosplit_pairs", at most 1024)
+int g_attn_nosplit_pairs = 165;   // (head, row) pairs from which a launch over the contiguous cache is never split ("attn_nosplit_pairs", at most 1024)
+int g_attn_nosplit_len = 1536;    // cache positions up to which two rows and more are not split either ("attn_nosplit_len", 0 = off)
 int g_attn_split_target = 1536;  // workgroups a split launch aims for (raven_set_tuning "attn_split_target"); 1536 beats 2048 by 2-6 us at 3..9 sequences
 int g_attn_big_grid = 1280;      // workgroups from which the 2-positions-per-row variant is used ("attn_big_grid")
 // Few (head, row) pairs and a short cache: one 1024-thread workgroup per pair instead of a split launch and its merge
@@ -669,8 +670,16 @@ int g_attn_wide = 0;
 int g_attn_prefetch = 1;  // raven_set_tuning("attn_prefetch"): 0 = a decode-attention workgroup requests a tile only when it needs it
 
 // Splits are worth their extra launch only while heads x rows cannot fill the chip.
-static int splits_for(int M, int nh, int len_hint) {
-    if ((int64_t)M * nh >= g_attn_nosplit_pairs) return 1;
+// The contiguous cache's kernel (contiguous = true) has variants that keep two tiles of four positions per 16-lane row in
+// flight, with which one workgroup per (head, row) beats a split launch and its merge launch (4.8 us) for two rows and
+// more over caches of up to about 1500 positions.  Core iteration at 1024 positions, split / unsplit, ms: 2 sequences
+// 0.682 / 0.679, 4: 0.710 / 0.699, 8: 0.770 / 0.768, 12: 0.824 / 0.810, 16: 0.900 / 0.881.  One sequence stays split:
+// measured alone (cache partly held by the memory-side cache) the unsplit launch is 3 us faster, inside the iteration,
+// whose slots stream from HBM, it is not (0.568 / 0.570 ms), and beyond 2000 positions the split wins clearly
+// (2048: 17.2 / 19.7 us, 4090: 23.5 / 35.8 us per step; 2 sequences: 23.1 / 22.5 and 37.9 / 40.2).
+static int splits_for(int M, int nh, int len_hint, bool contiguous = false) {
+    if ((int64_t)M * nh >= (contiguous ? g_attn_nosplit_pairs : 1024)) return 1;
+    if (contiguous && M >= 2 && len_hint <= g_attn_nosplit_len) return 1;
     int ns = (len_hint + 63) / 64;  // 64 positions per workgroup keeps every load in one round trip
     const int cap = (g_attn_split_target + M * nh - 1) / (M * nh);
     if (ns > cap) ns = cap;
@@ -848,7 +857,11 @@ static void launch_attention(bool fused, const void* q, const void* bias, const 
     // or more (head, row) pairs: 117.5 -> 114 us at 32 rows and 1024 positions; split launches, whose workgroups
     // walk a few tiles each, lose 8 % to the tile of the last pair that lies past the range)
     const int per = (pos0 + S + ns - 1) / ns;
-    const bool pf = g_attn_prefetch && (ns == 1 || g_attn_prefetch == 2) && per >= 8 * 16 * (big ? 2 : 4);
+    // ... and of fewer than 256 pairs; in between (256 .. 1023 pairs unsplit) requesting a tile only when it is needed is as
+    // fast or faster (10 sequences x 1024 positions: 37.1 us against 42.0; 5: 24.7 against 27.9; 8, 14, 16, 18: equal)
+    const int64_t pairs = (int64_t)cv.nh * M;
+    const bool pf = g_attn_prefetch && (ns == 1 || g_attn_prefetch == 2) && per >= 8 * 16 * (big ? 2 : 4) &&
+                    (g_attn_prefetch == 2 || ns > 1 || pairs < 256 || pairs >= 1024);
     if (cv.hd / Chunk<T>::N > 16) {  // fp32 heads wider than 64 elements: two chunks per lane, one variant per entry point
         if constexpr (sizeof(T) == 4) {
             if (fused) decode_attention_kernel<T, true, 2, true, 2><<<grid, dim3(256), 0, s>>>((const T*)q, bias_t, freqs, (T*)y, cv, S, pos0, pos_dev, scale_log2, ns, ws_ml, ws_o);
@@ -885,8 +898,9 @@ static int attention_common(const char* who, bool fused, const void* q, const vo
     RAVEN_REQUIRE(pos0 + S <= cv.t_max, "%s: positions up to %d exceed the cache length %d", who, pos0 + S - 1, cv.t_max);
     const int M = B * S;
     RAVEN_REQUIRE(M <= 65535, "%s: too many token rows (%d)", who, M);
-    int ns = splits_for(M, n_heads, pos0 + S);
     const int elts = 16 / (int)raven_host::elt_size(dtype);
+    // the variants for partially filled caches and for two chunks per lane keep one tile in flight: they split as before
+    int ns = splits_for(M, n_heads, pos0 + S, !cv.steps_present && head_dim / elts <= 16);
     const bool wide = fused && ns > 1 && pos0 + S <= g_attn_wide && M * n_heads <= 256 && !cv.steps_present && head_dim / elts <= 16;
     if (wide) ns = 1;
     float *ws_ml = nullptr, *ws_o = nullptr;

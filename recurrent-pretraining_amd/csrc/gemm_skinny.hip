@@ -29,7 +29,7 @@ extern int g_tiled_min_rows, g_tiled_variant, g_tiled_split_tail;
 bool tiled_gemm_fits(int M, int N, int K0, int K1, int dtype);
 int tiled_gemm(const void* x0, const void* x1, const void* w, const void* residual, void* y, int M, int N, int K0, int K1, int swiglu,
                int out_f32, hipStream_t s);
-extern int g_attn_split_target, g_attn_big_grid, g_attn_wide, g_linear_min_rows, g_attn_nosplit_pairs, g_rope_tiled_rows, g_prefill_waves, g_norm_early, g_fuse_sums_norm, g_attn_prefetch, g_fuse_qkv_rope, g_pad_chunk_rows, g_pad_decode_rows;
+extern int g_attn_split_target, g_attn_big_grid, g_attn_wide, g_linear_min_rows, g_attn_nosplit_pairs, g_attn_nosplit_len, g_rope_tiled_rows, g_prefill_waves, g_norm_early, g_fuse_sums_norm, g_attn_prefetch, g_fuse_qkv_rope, g_pad_chunk_rows, g_pad_decode_rows;
 
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
 
@@ -596,6 +596,7 @@ extern "C" int raven_set_tuning(const char* key, int32_t value) {
     else if (k == "pad_chunk_rows" && (value == 0 || value == 1)) g_pad_chunk_rows = value;
     else if (k == "pad_decode_rows" && (value == 0 || value == 1)) g_pad_decode_rows = value;
     else if (k == "attn_nosplit_pairs" && value > 0 && value <= 1024) g_attn_nosplit_pairs = value;
+    else if (k == "attn_nosplit_len" && value >= 0) g_attn_nosplit_len = value;
     else if (k == "linear_min_rows" && value >= 1) g_linear_min_rows = value;
     else if (k == "norm_early" && value >= -1 && value <= 1) g_norm_early = value;
     else if (k == "fuse_sums_norm" && (value == 0 || value == 1)) g_fuse_sums_norm = value;

@@ -46,7 +46,7 @@ def lib(pkg):
 
 
 # defaults of the launch-shape knobs the tests change (raven_set_tuning); results never depend on them
-TUNING_DEFAULTS = {"linear_ks": 0, "gemm_four_tiles": 1, "attn_wide": 0, "gemm_tiled_min_rows": 33, "gemm_tiled_variant": 0, "gemm_tiled_split_tail": 1, "prefill_waves": 0, "gemm_ragged": 1, "norm_early": -1, "fuse_sums_norm": 1, "attn_prefetch": 1, "fuse_qkv_rope": 1, "pad_chunk_rows": 1, "pad_decode_rows": 1}
+TUNING_DEFAULTS = {"linear_ks": 0, "gemm_four_tiles": 1, "attn_wide": 0, "gemm_tiled_min_rows": 33, "gemm_tiled_variant": 0, "gemm_tiled_split_tail": 1, "prefill_waves": 0, "gemm_ragged": 1, "norm_early": -1, "fuse_sums_norm": 1, "attn_prefetch": 1, "fuse_qkv_rope": 1, "pad_chunk_rows": 1, "pad_decode_rows": 1, "attn_nosplit_pairs": 165, "attn_nosplit_len": 1536}
 
 
 @pytest.fixture

@@ -420,6 +420,26 @@ def test_decode_attention(pkg, dt, nh, hd, B, S, pos0):
     check(y3, want, dt, "attention without workspace")
 
 
+@pytest.mark.parametrize("B,S,pos0,t_max,nosplit_len", [(3, 1, 1900, 2048, None), (2, 1, 70, 1024, 0), (1, 6, 200, 1024, 0),
+                                                        (4, 1, 1023, 1024, 0), (2, 1, 1023, 1024, None)])
+def test_decode_attention_of_several_rows_split_and_unsplit(pkg, tuned, B, S, pos0, t_max, nosplit_len):
+    """Two rows and more over the contiguous cache: split over positions by the library's rule (a long cache) or because
+    the length rule is switched off, and one workgroup per (head, row) otherwise; each against the oracle."""
+    dt, nh, hd = torch.bfloat16, 55, 96
+    k, v, kd, vd, cache = make_cache(pkg, 2, B, nh, t_max, hd, dt, fill_seed=95)
+    q = rnd((B * S, nh * hd), dt, 96)
+    T = pos0 + S
+    want = O.sdpa(q.view(B, S, nh, hd).transpose(1, 2), k[1, :, :, :T], v[1, :, :, :T]).transpose(1, 2).reshape(B * S, nh * hd)
+    ws = pkg.hip.attention_workspace(B * S, nh, hd, "cuda")
+    if nosplit_len is not None:
+        tuned(attn_nosplit_len=nosplit_len)
+    y = pkg.hip.decode_attention(q.cuda(), cache, 1, B, S, pos0, nh, hd, workspace=ws)
+    check(y, want, dt, f"attention B={B} S={S} T={T}, length rule {nosplit_len}")
+    tuned(attn_nosplit_len=1 << 20)   # never split two rows and more
+    y1 = pkg.hip.decode_attention(q.cuda(), cache, 1, B, S, pos0, nh, hd, workspace=ws)
+    check(y1, want, dt, f"attention B={B} S={S} T={T}, one workgroup per (head, row)")
+
+
 @pytest.mark.parametrize("dt,nh,hd,B,pos0", [(torch.bfloat16, 55, 96, 1, 1023), (torch.bfloat16, 55, 96, 32, 600),
                                              (torch.bfloat16, 55, 96, 1, 0), (torch.float32, 4, 64, 3, 17),
                                              (torch.bfloat16, 2, 128, 2, 130)])

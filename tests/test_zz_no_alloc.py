@@ -22,10 +22,10 @@ def _case(pkg, B, T, nh, hd, dt, seed):
 
 
 @pytest.mark.parametrize("dt,nh,hd", [(torch.bfloat16, 55, 96), (torch.float32, 4, 64)])
-def test_static_scratch_decode_attention_equals_workspace_version(pkg, dt, nh, hd):
+def test_static_scratch_decode_attention_equals_workspace_version(pkg, tuned, dt, nh, hd):
     lib = pkg.hip.load()
     assert lib.raven_qkv_attention_decode_static_scratch_bytes() >= lib.raven_decode_attention_workspace_bytes(18, 55, 128)
-    for call, (B, T) in enumerate([(3, 1500), (1, 700)]):  # both launches are split over positions
+    for call, (B, T) in enumerate([(3, 2100), (1, 700)]):  # both launches are split over positions by the library's rule
         qkv, bias, freqs, k, v = _case(pkg, B, T, nh, hd, dt, 40 + call)
         ka, va, kb, vb = k.cuda(), v.cuda(), k.cuda(), v.cuda()
         ws = pkg.hip.attention_workspace(B, nh, hd, "cuda")
@@ -36,6 +36,14 @@ def test_static_scratch_decode_attention_equals_workspace_version(pkg, dt, nh, h
         torch.cuda.synchronize()
         assert torch.equal(got, want), f"call {call}: output"
         assert torch.equal(ka, kb) and torch.equal(va, vb), f"call {call}: appended cache rows"
+        if dt == torch.float32:
+            # that the launch was split, seen from outside: one workgroup per (head, row) adds in another order
+            tuned(attn_nosplit_pairs=1)
+            kc, vc = k.cuda(), v.cuda()
+            unsplit = pkg.hip.qkv_attention_decode(qkv, bias, freqs, pkg.hip.make_cache(kc, vc), 1, B, T, nh, hd, workspace=ws)
+            tuned(attn_nosplit_pairs=165)
+            assert not torch.equal(unsplit, want), f"call {call}: the launch under test was not split"
+            check(unsplit, want, dt, f"call {call}: unsplit against split")
         # and both equal the oracle's attention over the T cached positions plus the new one
         h = nh * hd
         q_, k_, v_ = (t.view(B, 1, nh, hd) for t in qkv.cpu().split([h, h, h], dim=1))
@@ -61,7 +69,7 @@ def test_static_scratch_entry_allocates_nothing_and_replays_from_a_captured_grap
     leaves the allocator's counters where they were, and the call can be captured into a HIP graph -- position on the
     device, output buffer given -- and replayed: every replay gives the bits of the version with a workspace at that
     position, with eager work and synchronisations of the program between the replays."""
-    dt, nh, hd, B, T = torch.bfloat16, 55, 96, 2, 900
+    dt, nh, hd, B, T = torch.bfloat16, 55, 96, 2, 1800   # long enough for the launch to be split
     qkv, bias, freqs, k, v = _case(pkg, B, T, nh, hd, dt, 70)
     ka, va, kb, vb = k.cuda(), v.cuda(), k.cuda(), v.cuda()
     ca, cb = pkg.hip.make_cache(ka, va), pkg.hip.make_cache(kb, vb)
