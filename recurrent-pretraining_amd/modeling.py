@@ -1087,12 +1087,23 @@ class DecodeRunner:
         coda = [c._slot(-(i + 1)) for i in range(n_coda)]
         return pre, core, coda
 
-    def _enqueue(self):
-        """Launches one token's kernels; reads the position from self.pos."""
+    # positions (the new one included) up to which the library runs the decode attention of two rows and more as one
+    # workgroup per (head, row) instead of splitting the positions over workgroups (its "attn_nosplit_len" default)
+    SHORT_CACHE_POSITIONS = 1536
+
+    def _position_bound(self, pos0: int) -> int:
+        """The by-value position that sizes the grids of a step at position pos0; the kernels take the true position
+        from the device.  It is the cache's capacity, except while the sequence is short enough for the unsplit decode
+        attention: then it is that rule's limit, so that a cache sized for a long generation does not cost a short
+        sequence the split launch and its merge (the step's graph is captured again once, when the sequence crosses)."""
+        cap = self.cache.t_max - 1
+        return cap if pos0 + 1 > self.SHORT_CACHE_POSITIONS else min(cap, self.SHORT_CACHE_POSITIONS - 1)
+
+    def _enqueue(self, hint: int):
+        """Launches one token's kernels; reads the position from self.pos.  hint bounds the position for grid sizing."""
         m, t = self.model, self.model.transformer
         nat, cfg, B = m._natives(), m.config, self.B
         kv = self.cache.native()
-        hint = self.cache.t_max - 1  # sizes grids; the kernels take the true position from the device
         pre, core, coda = self._slots()
         hip.embed(t.wte.weight, self.ids, m.emb_scale, out=self.embeds)
         cur = self.embeds
@@ -1149,6 +1160,7 @@ class DecodeRunner:
         if pos0 + 1 > c.t_max or (c.max_length is not None and pos0 + 1 > c.max_length):
             c.ensure(1, 0, self.B, m.config.n_heads, m.config.head_dim, pos0 + 1, m.dtype, m.device)  # grows (pointers move), or refuses past max_length
             self.graph = None
+        hint = self._position_bound(pos0)
         self.ids.copy_(ids.view(-1))
         self.pos.fill_(pos0)
         if state is None:
@@ -1161,16 +1173,16 @@ class DecodeRunner:
         if self.use_graph and self._warm:
             # the captured launches hold the cache's pointers, slot numbers and capacity: any reallocation (more
             # positions, more step slots) makes them stale
-            key = (c._k.data_ptr(), c._v.data_ptr(), tuple(c._k.shape), c._neg_slots)
+            key = (c._k.data_ptr(), c._v.data_ptr(), tuple(c._k.shape), c._neg_slots, hint)
             if self.graph is None or self._graph_key != key:
                 self.graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(self.graph):
-                    self._enqueue()
+                    self._enqueue(hint)
                 self._graph_key = key
                 self.pos.fill_(pos0)  # capture does not execute; make sure the counter is what this step needs
             self.graph.replay()
         else:
-            self._enqueue()
+            self._enqueue(hint)
             self._warm = True
         # bookkeeping the reference does inside cache.update (RMM:188-196)
         cfg = m.config

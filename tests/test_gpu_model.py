@@ -375,6 +375,40 @@ def test_decode_runner_beyond_one_pass_of_rows_bf16(pkg, tiny16, use_graph):
     assert (runner.graph is not None) == use_graph
 
 
+def test_decode_runner_sizes_grids_for_a_short_sequence_in_a_long_cache(pkg, tiny16, tuned):
+    """A cache with room for a long generation: while the sequence is short the runner sizes its grids by the bound of
+    the library's rule for unsplit decode attention, not by the capacity, and captures the step again when the sequence
+    crosses that bound.  The bound is lowered to a few positions here (knob and runner alike); every step's logits against
+    the oracle and against forward() on the same cache contents, before, at and behind the crossing."""
+    s, w, model = tiny16
+    B, S, n_new, bound = 3, 6, 6, 9
+    g = torch.Generator().manual_seed(78)
+    ids = torch.randint(0, s.vocab_size, (B, S + n_new), generator=g)
+    states = O.initialize_state(torch.empty(B, S + n_new, s.n_embd), s, 1.0, g).to(torch.bfloat16)
+    ref_cache, cache, cache2 = O.DictCache(), pkg.HuginnDynamicCache(max_length=300), pkg.HuginnDynamicCache(max_length=300)
+    O.forward(w, s, input_ids=ids[:, :S], input_states=states[:, :S], past_key_values=ref_cache, use_cache=True)
+    for c in (cache, cache2):
+        model(input_ids=ids[:, :S].cuda(), input_states=states[:, :S].cuda(), past_key_values=c, use_cache=True)
+    tuned(attn_nosplit_len=bound)
+    runner = pkg.DecodeRunner(model, cache, B, s.mean_recurrence, use_graph=True)
+    runner.SHORT_CACHE_POSITIONS = bound
+    assert cache.t_max >= 300
+    bounds = []
+    for i in range(n_new):
+        pos = torch.arange(S + i, S + i + 1)
+        tok, st = ids[:, S + i:S + i + 1], states[:, S + i:S + i + 1]
+        want = O.forward(w, s, input_ids=tok, input_states=st, past_key_values=ref_cache, use_cache=True, cache_position=pos)
+        fwd = model(input_ids=tok.cuda(), input_states=st.cuda(), past_key_values=cache2, use_cache=True, cache_position=pos.cuda())
+        logits, nxt, lat = runner.step(tok.cuda(), st.cuda())
+        bounds.append(runner._position_bound(S + i))
+        check(logits, want.logits[:, 0], torch.bfloat16, f"runner logits, token {i}")
+        check(logits, fwd.logits[:, 0], torch.bfloat16, f"token {i}: runner against forward()")
+        if i > 0:
+            assert runner._graph_key[-1] == bounds[-1]
+    assert bounds == [bound - 1] * 3 + [cache.t_max - 1] * 3   # positions 6, 7, 8 fill up to 9 positions; from 9 on the capacity
+    assert cache.get_seq_length() == S + n_new
+
+
 class SharedDraws:
     """The random numbers of the test-time noise, drawn on the CPU from one seeded generator: the oracle and the model
     consume them in the same order (per recurrence: the amplitude for "chi", then the noise)."""
