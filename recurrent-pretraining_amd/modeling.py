@@ -1161,6 +1161,8 @@ class DecodeRunner:
             c.ensure(1, 0, self.B, m.config.n_heads, m.config.head_dim, pos0 + 1, m.dtype, m.device)  # grows (pointers move), or refuses past max_length
             self.graph = None
         hint = self._position_bound(pos0)
+        if self.B >= 17 and m.dtype == torch.bfloat16 and m.pack_chunk_weights:
+            m.pack_weights()  # no work unless a weight changed since the copies were made (in place: the copies keep their addresses)
         self.ids.copy_(ids.view(-1))
         self.pos.fill_(pos0)
         if state is None:
