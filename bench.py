@@ -38,7 +38,9 @@ def parse():
     ap.add_argument("--recurrence", type=int, default=32)
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-iters", type=int, default=3)
+    ap.add_argument("--cpu-iters", type=int, default=3, help="fewest timed recurrence iterations of the CPU baseline")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0,
+                    help="the CPU baseline keeps timing iterations until this much time has been spent on them (at most 400)")
     ap.add_argument("--also-batch", type=int, action="append", default=None, metavar="B",
                     help="further batch sizes reported as sub-records bs<B> (default 8 and 32; 0 = none)")
     ap.add_argument("--prefill-iters", type=int, default=8,
@@ -587,7 +589,7 @@ def main():
 
     cpu = None
     if not args.no_cpu_baseline:
-        cpu = cpu_baseline(model, args.cpu_iters, r)
+        cpu = cpu_baseline(model, args.cpu_iters, r, args.cpu_seconds)
 
     line = {
         "metric": "decode tokens/s at r=32, raven-3.5b shape bf16 bs=1/32; % HBM roofline",
@@ -748,10 +750,11 @@ def decode_record(pkg, model, B, prompt_len, steps, warmup, r, use_graph):
     }
 
 
-def cpu_baseline(model, n_iters, r):
-    """The CPU oracle (a port of the reference's CPU path) on the host cores: a few recurrence
-    iterations plus one LM-head product at the nebel shape, bs=1, 512 cached positions, scaled to
-    tokens/s as 1 / ((r + 1) * t_iteration + t_head) -- the 4 prelude/coda blocks cost one iteration.
+def cpu_baseline(model, n_iters, r, seconds=12.0):
+    """The CPU oracle (a port of the reference's CPU path) on the host cores: recurrence iterations
+    (at least n_iters, then on until `seconds` of CPU work are spent, at most 400) plus LM-head products
+    at the nebel shape, bs=1, 512 cached positions, scaled to tokens/s as
+    1 / ((r + 1) * t_iteration + t_head) -- the 4 prelude/coda blocks cost one iteration.
     The only part of this file that touches the oracle."""
     import torch
     from oracle import raven_oracle as O
@@ -770,20 +773,24 @@ def cpu_baseline(model, n_iters, r):
     emb = torch.randn(1, 1, shape.n_embd, generator=g).to(torch.bfloat16)
     n_threads = torch.get_num_threads()
     times = []
-    for it in range(n_iters + 1):  # first pass is warm-up
+    while len(times) < n_iters + 1 or (sum(times[1:]) < seconds and len(times) < 401):  # first pass is warm-up
         for j in range(4):
             cache.key_cache[2 + j] = {p: kv[0, :, :, p] for p in range(T - 1)}
             cache.value_cache[2 + j] = {p: kv[1, :, :, p] for p in range(T - 1)}
         t0 = time.perf_counter()
         O.core_block_forward(x, emb, w, table[:, T - 1:T], cache, 1, shape)
         times.append(time.perf_counter() - t0)
-    t_iter = sum(times[1:]) / max(1, len(times) - 1)
-    t0 = time.perf_counter()
-    torch.nn.functional.linear(x, w["transformer.wte.weight"]).float()
-    t_head = time.perf_counter() - t0
+    n_iters = len(times) - 1
+    t_iter = sum(times[1:]) / max(1, n_iters)
+    heads = []
+    for _ in range(4):  # the first product is warm-up
+        t0 = time.perf_counter()
+        torch.nn.functional.linear(x, w["transformer.wte.weight"]).float()
+        heads.append(time.perf_counter() - t0)
+    t_head = sum(heads[1:]) / 3
     tok_s = 1.0 / ((r + 1) * t_iter + t_head)
     return {"value": round(tok_s, 5), "unit": "tokens/s", "cores": n_threads, "kind": "port",
-            "sample": f"{n_iters} recurrence iterations (mean {t_iter * 1e3:.1f} ms) + 1 LM head ({t_head * 1e3:.1f} ms) at nebel shape, "
+            "sample": f"{n_iters} recurrence iterations ({sum(times[1:]):.1f} s, mean {t_iter * 1e3:.1f} ms) + 3 LM heads (mean {t_head * 1e3:.1f} ms) at nebel shape, "
                       f"bs=1, {T} cached positions, torch CPU bf16, {n_threads} threads of {os.cpu_count()} cpus; "
                       f"scaled to a token as ({r}+1) iterations + head"}
 
