@@ -697,7 +697,7 @@ def decode_record(pkg, model, B, prompt_len, steps, warmup, r, use_graph):
     lib = pkg.hip.load()
     stream = torch.cuda.current_stream().cuda_stream
     if B == 1:
-        kernel_name = "gemv1_kernel<bf16, C=3, SwiGLU, norm prologue, 4 row pairs per workgroup> (mlp.fc 35840x5280)"
+        kernel_name = "gemv1_kernel<bf16, C=3, SwiGLU, norm prologue, 7 row pairs per workgroup> (mlp.fc 35840x5280)"
 
         def fc_launch(i=[0]):
             blk = blocks[i[0] % len(blocks)]

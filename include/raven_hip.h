@@ -85,7 +85,8 @@ const char* raven_last_error(void);
 
 /* Launch-shape overrides for experiments (grid sizing and load hints of the skinny-GEMM kernels);
  * results never depend on them.  Keys: gemv_units_per_wave, gemv_interleave, gemv_nontemporal,
- * gemv_wgs_per_cu, gemv1_pairs_norm, gemv1_pairs_plain, gemm_four_tiles (0 / 1 / 2 = never / by rule / always use
+ * gemv_wgs_per_cu, gemv1_pairs_norm (weight-row pairs per workgroup of the one-row kernel with a norm prologue; 0 = by shape,
+ * about ten workgroups per compute unit), gemv1_pairs_plain, gemm_four_tiles (0 / 1 / 2 = never / by rule / always use
  * the four-tile MFMA variant), attn_split_target / attn_big_grid (workgroups a split decode-attention launch aims
  * for / from which its 2-positions-per-row variant is used), attn_nosplit_pairs ((head, row) pairs from which a launch over the contiguous cache is
  * never split, at most 1024; the paged entry point stops splitting at 1024), attn_nosplit_len (cache positions up to

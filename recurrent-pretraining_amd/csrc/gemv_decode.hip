@@ -223,10 +223,21 @@ __global__ __launch_bounds__(256) void gemv1_kernel(Gemv1Args a) {
 }
 
 struct Gemv1Tuning {
-    int pairs_norm = 4;    // pairs per workgroup when a norm prologue has to be amortised
+    int pairs_norm = 0;    // pairs per workgroup when a norm prologue has to be amortised; 0 = by shape (about ten workgroups per CU)
     int pairs_plain = 1;   // ... and when there is none
 };
 static Gemv1Tuning g_gemv1_tuning;
+
+static int gemv1_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t p;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;
+        if (cus <= 0) cus = 256;
+    }
+    return cus;
+}
 
 template <typename T, bool SWIGLU>
 static int launch_gemv1(Gemv1Args a, hipStream_t s) {
@@ -237,6 +248,9 @@ static int launch_gemv1(Gemv1Args a, hipStream_t s) {
     const int units = SWIGLU ? a.N : (a.N + 1) / 2;
     const bool norm = a.norm_a != nullptr;
     int ppw = norm ? g_gemv1_tuning.pairs_norm : g_gemv1_tuning.pairs_plain;
+    // with a norm prologue: as many pairs as leave about ten workgroups per CU -- 4 for Wqkv (7920 pairs, 1980 workgroups),
+    // 7 for mlp.fc (17920 gate / up pairs, 2560 workgroups: 57.6 us against 58.4 with 4, while Wqkv loses with more than 4)
+    if (norm && ppw <= 0) ppw = (units + 10 * gemv1_cus() - 1) / (10 * gemv1_cus());
     if (ppw < 1) ppw = 1;
     if (ppw > kMaxPairsPerWg) ppw = kMaxPairsPerWg;
     while (ppw > 1 && (units + ppw - 1) / ppw < 1024) --ppw;  // keep at least ~4 workgroups per CU
